@@ -1,0 +1,63 @@
+/*
+ * C ABI of the "HIP-MLA" ggml backend plugin (libggml-hip-mla.so).
+ *
+ * The plugin is loaded by the reference exactly like any other dynamic ggml backend:
+ *   ggml_backend_load(path)            ggml/src/ggml-backend-reg.cpp:401-403 -> load_backend :225-271
+ *   GGML_BACKEND_PATH=<path>           ggml/src/ggml-backend-reg.cpp:583-587
+ *   ggml_backend_load_all()            finds "libggml-hip-*.so" next to the executable, :488-558, :574
+ * After that the reference talks to it only through the vtables of ggml/src/ggml-backend-impl.h, whose layouts
+ * are mirrored in jittorinfer_amd/csrc/ggml_abi.h.  All handles are passed as void* here so that this header needs
+ * no ggml header; they are ggml_backend_reg_t / ggml_tensor* of the reference.
+ *
+ * Node contract of the one compute op it accepts, GGML_OP_FLASH_ATTN_EXT built by ggml_flash_attn_ext
+ * (ggml/src/ggml.c:3988-4022), with the operands llm_attn_mla defines (src/llama-graph-attn.cpp:259-315):
+ *   src[0] q     F32  [576, n_tok, n_head, n_seq]
+ *   src[1] k     F16 | BF16 | Q8_0  [576, n_kv, 1, n_seq or 1]   the latent KV rows
+ *   src[2] v     k itself (V := K, 576 wide) or a 512-wide view of k at offset 0 (the latent prefix)
+ *   src[3] mask  F16 [>= n_kv, >= n_tok] or NULL, additive, -inf removes a key (src/llama-context.cpp:364-404)
+ *   src[4], src[5]  optional, both or none: I32 block table [max_blocks, n_seq] of 128-token page ids into k
+ *                (k is then the page pool [576, n_pages*128, 1, 1]) and I32 [n_seq] sequence lengths -- the same
+ *                slot convention ggml_flash_attn_prompt uses for its length tensors (ggml/src/ggml.c:2707-2710)
+ *   op_params    {scale, max_bias, logit_softcap} f32, [3] = precision (ggml/src/ggml.c:4012-4013, :4024-4030)
+ *   dst          F32 [576, n_head, n_tok, n_seq]; the first v->ne[0] floats of every row are written
+ * Every other op except the no-op view ops (NONE, RESHAPE, VIEW, PERMUTE, TRANSPOSE) is reported unsupported, so
+ * the reference's scheduler keeps it on another backend (ggml/src/ggml-backend.cpp:820-846).
+ */
+#ifndef GGML_MLA_BACKEND_H
+#define GGML_MLA_BACKEND_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* replaces: the ggml_backend_init symbol every dynamic backend exports (GGML_BACKEND_DL_IMPL,
+ * ggml/src/ggml-backend-impl.h:227-243; CANN's is ggml_backend_cann_reg, ggml/src/ggml-cann/ggml-cann.cpp:2506-2550).
+ * Returns the process-lifetime ggml_backend_reg_t (api_version 1); one device per gfx950 GPU. */
+void * ggml_backend_init(void);
+
+/* replaces: the optional ggml_backend_score symbol (ggml/src/ggml-backend-impl.h:244-258, used at
+ * ggml/src/ggml-backend-reg.cpp:520-535).  100 when a gfx950 device is present, 0 otherwise. */
+int ggml_backend_score(void);
+
+/* replaces: the static-registration accessor each in-tree backend has (ggml_backend_cann_reg, ggml-cann.cpp:2506),
+ * for hosts that call ggml_backend_register(reg) (ggml/src/ggml-backend-reg.cpp:305-307) instead of dlopen. */
+void * ggml_backend_hip_mla_reg(void);
+
+/* no counterpart in the reference: entry i of the sizeof/offsetof/ordinal table this build assumes for the
+ * reference's structs; returns the table length.  Lets a maintainer (and tests/test_abi.py) check the mirror
+ * against the real headers without running anything on a GPU. */
+int mla_ggml_abi_table(int i, const char ** name, int64_t * value);
+
+/* no counterpart: supports_op's verdict for one FLASH_ATTN_EXT node plus the violated clause (for diagnostics). */
+int mla_ggml_supports_node(const void * ggml_tensor_node, const char ** why);
+
+/* no counterpart: frees a buffer obtained from this backend's buffer type when no ggml is present in the process
+ * to do it (what ggml_backend_buffer_free does, ggml/src/ggml-backend.cpp). */
+void mla_ggml_buffer_free(void * ggml_backend_buffer);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,128 @@
+/*
+ * Thin C ABI over the hand-written gfx950 kernels for absorbed-MLA attention
+ * (GGML_OP_FLASH_ATTN_EXT with 576-d Q.K, a 512- or 576-wide V that is a prefix of the same latent K row,
+ * one KV stream shared by all heads).
+ *
+ * Plain pointers and sizes only: no ggml, torch or HIP types.  All pointers are DEVICE pointers unless said
+ * otherwise; `stream` is a hipStream_t passed as void* (NULL = the default stream).  Every function returns 0 on
+ * success, a negative MLA_ERR_* code for a rejected argument, or a positive hipError_t value.
+ * Nothing here allocates device memory: scratch space comes from the caller (`workspace`).
+ *
+ * What each entry point replaces in the reference (paths relative to the JittorInfer tree):
+ *   mla_attn_launch            the per-node compute of GGML_OP_FLASH_ATTN_EXT,
+ *                              ggml/src/ggml-cpu/ggml-cpu.c:11914-12142 (dispatch :14267-14272), i.e. what
+ *                              iface.graph_compute (ggml/src/ggml-backend-impl.h:116) runs for that node; the
+ *                              operands are those llm_attn_mla defines, src/llama-graph-attn.cpp:259-315.
+ *   mla_attn_workspace_size    the per-thread scratch sizing of the same op, ggml-cpu.c:15175-15180.
+ *   mla_attn_plan              no counterpart: reports which kernel variant / split the launch will use.
+ *   mla_hbm_copy_launch        no counterpart: a plain 16-byte-per-lane copy kernel used to calibrate the
+ *                              rocprofv3 FETCH_SIZE / WRITE_SIZE counters against a known byte count.
+ */
+#ifndef MLA_ATTN_H
+#define MLA_ATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element types: the ggml_type ordinals of the reference (ggml/include/ggml.h:360-401) */
+#define MLA_TYPE_F32  0
+#define MLA_TYPE_F16  1
+#define MLA_TYPE_Q8_0 8
+#define MLA_TYPE_BF16 30
+
+/* flags */
+#define MLA_FLAG_F16_ACC_STRICT 1u /* F16 KV only: replay ggml-cpu's per-key f16 accumulator (ggml-cpu.c:12066-12080)
+                                      instead of accumulating in f32; sequential over keys, a correctness mode */
+
+/* errors */
+#define MLA_ERR_BAD_SHAPE     (-1)
+#define MLA_ERR_BAD_TYPE      (-2)
+#define MLA_ERR_BAD_ALIGNMENT (-3)
+#define MLA_ERR_WORKSPACE     (-4)
+#define MLA_ERR_NULL          (-5)
+#define MLA_ERR_UNSUPPORTED   (-6)
+
+#define MLA_PAGE_TOKENS 128
+
+typedef struct mla_attn_args {
+    /* ---- shapes (ggml names: q ne = {dk, n_tok, n_head, n_seq}) */
+    int32_t n_seq;   /* q->ne[3]: sequences in the batch */
+    int32_t n_head;  /* q->ne[2]: query heads; all of them read the same K/V rows (MQA broadcast, ggml-cpu.c:11955) */
+    int32_t n_tok;   /* q->ne[1]: query tokens per sequence (1 = decode) */
+    int32_t dk;      /* q->ne[0] = k->ne[0]: must be 576 */
+    int32_t dv;      /* v->ne[0]: 512 (latent prefix) or 576 (V := K, what ggml-cpu requires, ggml-cpu.c:11943) */
+    int32_t q_type;  /* MLA_TYPE_F32 (what ggml graphs carry); rounded to K's dot type as ggml-cpu does (:12034-12035) */
+    int32_t kv_type; /* MLA_TYPE_BF16 | MLA_TYPE_F16 | MLA_TYPE_Q8_0 */
+    uint32_t flags;
+
+    /* ---- op_params of the node (ggml/src/ggml.c:4012-4013) */
+    float scale;
+    float max_bias;
+    float logit_softcap;
+
+    /* ---- Q, byte strides as in ggml (nb0 == 4) */
+    const void * q;
+    int64_t q_nb1, q_nb2, q_nb3;
+
+    /* ---- latent KV.  V is the first dv columns of the same rows.
+     * Without a block table: row `ic` of sequence `b` is at kv + ic*kv_nb1 + b*kv_nb3 and every sequence has n_kv rows.
+     * With a block table: kv is the page pool; logical row ic of sequence b is pool row
+     *   block_table[b*bt_stride + ic/128]*128 + ic%128 (at kv + row*kv_nb1) and sequence b has seq_lens[b] rows. */
+    const void * kv;
+    int64_t kv_nb1; /* row stride in bytes: 1152 for f16/bf16, 612 for Q8_0 (18 x 34-byte blocks) when packed */
+    int64_t kv_nb3;
+    int64_t n_kv;   /* rows per sequence (no block table); with a block table: number of rows in the pool (bounds check) */
+
+    /* ---- optional additive mask, f16 [mask_ne0 >= keys, >= n_tok rows], shared by heads and sequences
+     * (src/llama-context.cpp:364-404; ggml-cpu.c:12024,12041-12044: -inf skips the key) */
+    const void * mask;
+    int64_t mask_nb1;
+    int64_t mask_ne0;
+
+    /* ---- optional paged extension (src[4]/src[5] of the node) */
+    const int32_t * block_table; /* [n_seq][bt_stride] page ids */
+    int64_t bt_stride;           /* ints per sequence (= max pages per sequence) */
+    const int32_t * seq_lens;    /* [n_seq] */
+
+    /* ---- output, f32: row (b*n_tok + t)*n_head + h starts at dst + row*dst_nb1 bytes (ggml-cpu.c:12122);
+     * dv floats of each row are written */
+    float * dst;
+    int64_t dst_nb1;
+
+    /* ---- scratch, at least mla_attn_workspace_size() bytes, 256-byte aligned */
+    void * workspace;
+    size_t workspace_size;
+
+    /* ---- tuning: 0 = choose; otherwise the number of KV splits per sequence */
+    int32_t n_splits;
+    int32_t reserved;
+} mla_attn_args;
+
+typedef struct mla_attn_plan_info {
+    int32_t variant;      /* 0 = tiled MFMA kernel, 1 = strict f16-accumulator replay */
+    int32_t rows_per_wg;  /* (token, head) rows one workgroup owns */
+    int32_t n_row_blocks; /* workgroups along rows, per sequence */
+    int32_t n_splits;     /* KV splits per sequence (1 = no combine pass) */
+    int32_t split_tokens; /* tokens per split */
+    int32_t n_passes;     /* passes over d (2 for dv = 576) */
+    int64_t lds_bytes;
+} mla_attn_plan_info;
+
+size_t mla_attn_workspace_size(const mla_attn_args * args);
+int    mla_attn_plan(const mla_attn_args * args, mla_attn_plan_info * out);
+int    mla_attn_launch(const mla_attn_args * args, void * stream);
+
+/* dst[i] = src[i] for n_bytes (multiple of 16) */
+int mla_hbm_copy_launch(const void * src, void * dst, size_t n_bytes, void * stream);
+
+/* library identification: "gfx950" and a build string; never NULL */
+const char * mla_attn_target_arch(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MLA_ATTN_H */

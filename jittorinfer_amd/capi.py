@@ -1,0 +1,153 @@
+"""ctypes binding of include/mla_attn.h.  PyTorch is used for device memory and streams only."""
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+MLA_TYPE_F32, MLA_TYPE_F16, MLA_TYPE_Q8_0, MLA_TYPE_BF16 = 0, 1, 8, 30
+MLA_FLAG_F16_ACC_STRICT = 1
+PAGE_TOKENS = 128
+ROW_BYTES = {MLA_TYPE_F16: 1152, MLA_TYPE_BF16: 1152, MLA_TYPE_Q8_0: 612}
+
+
+class MlaAttnArgs(C.Structure):
+    _fields_ = [
+        ("n_seq", C.c_int32), ("n_head", C.c_int32), ("n_tok", C.c_int32), ("dk", C.c_int32), ("dv", C.c_int32),
+        ("q_type", C.c_int32), ("kv_type", C.c_int32), ("flags", C.c_uint32),
+        ("scale", C.c_float), ("max_bias", C.c_float), ("logit_softcap", C.c_float),
+        ("q", C.c_void_p), ("q_nb1", C.c_int64), ("q_nb2", C.c_int64), ("q_nb3", C.c_int64),
+        ("kv", C.c_void_p), ("kv_nb1", C.c_int64), ("kv_nb3", C.c_int64), ("n_kv", C.c_int64),
+        ("mask", C.c_void_p), ("mask_nb1", C.c_int64), ("mask_ne0", C.c_int64),
+        ("block_table", C.c_void_p), ("bt_stride", C.c_int64), ("seq_lens", C.c_void_p),
+        ("dst", C.c_void_p), ("dst_nb1", C.c_int64),
+        ("workspace", C.c_void_p), ("workspace_size", C.c_size_t),
+        ("n_splits", C.c_int32), ("reserved", C.c_int32),
+    ]
+
+
+class MlaPlanInfo(C.Structure):
+    _fields_ = [("variant", C.c_int32), ("rows_per_wg", C.c_int32), ("n_row_blocks", C.c_int32), ("n_splits", C.c_int32),
+                ("split_tokens", C.c_int32), ("n_passes", C.c_int32), ("lds_bytes", C.c_int64)]
+
+
+def library_path():
+    return os.path.join(HERE, "libggml-hip-mla.so")
+
+
+_lib = None
+
+
+def library():
+    """The HIP library; raises if it has not been built (python -m jittorinfer_amd.build)."""
+    global _lib
+    if _lib is None:
+        path = library_path()
+        if not os.path.exists(path):
+            raise RuntimeError("%s is missing: build it with `python jittorinfer_amd/build.py` (there is no CPU fallback)" % path)
+        lib = C.CDLL(path)
+        lib.mla_attn_workspace_size.restype = C.c_size_t
+        lib.mla_attn_workspace_size.argtypes = [C.POINTER(MlaAttnArgs)]
+        lib.mla_attn_plan.restype = C.c_int
+        lib.mla_attn_plan.argtypes = [C.POINTER(MlaAttnArgs), C.POINTER(MlaPlanInfo)]
+        lib.mla_attn_launch.restype = C.c_int
+        lib.mla_attn_launch.argtypes = [C.POINTER(MlaAttnArgs), C.c_void_p]
+        lib.mla_hbm_copy_launch.restype = C.c_int
+        lib.mla_hbm_copy_launch.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
+        lib.mla_attn_target_arch.restype = C.c_char_p
+        lib.ggml_backend_init.restype = C.c_void_p
+        lib.ggml_backend_score.restype = C.c_int
+        lib.mla_ggml_abi_table.restype = C.c_int
+        lib.mla_ggml_abi_table.argtypes = [C.c_int, C.POINTER(C.c_char_p), C.POINTER(C.c_int64)]
+        _lib = lib
+    return _lib
+
+
+_workspaces = {}
+
+
+def _workspace(device, nbytes):
+    import torch
+    ws = _workspaces.get(device)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _workspaces[device] = ws
+    return ws
+
+
+def make_args(q, k, kv_type, dv=512, mask=None, scale=1.0, max_bias=0.0, logit_softcap=0.0, block_table=None,
+              seq_lens=None, out=None, n_splits=0, flags=0):
+    """Builds (args, out, keepalive) from torch tensors on one gfx950 device.
+
+    q     float32 [n_seq, n_head, n_tok, 576] (any strides with a contiguous last dim)
+    k     the latent KV rows: [n_seq, n_kv, row] (uint8/int16/bfloat16/float16 with `row` 1152/612 bytes) or,
+          with a block table, the page pool [n_rows, row] (n_rows a multiple of 128)
+    mask  float16 [>= n_tok, mask_ne0] or None;  block_table int32 [n_seq, max_blocks];  seq_lens int32 [n_seq]
+    out   float32 [n_seq, n_tok, n_head, 576] (ggml's dst layout); created if None.  dv columns of each row are written.
+    """
+    import torch
+    assert q.dtype == torch.float32 and q.dim() == 4 and q.shape[-1] == 576 and q.stride(-1) == 1
+    n_seq, n_head, n_tok, _ = q.shape
+    row = ROW_BYTES[kv_type]
+    a = MlaAttnArgs()
+    a.n_seq, a.n_head, a.n_tok, a.dk, a.dv = n_seq, n_head, n_tok, 576, dv
+    a.q_type, a.kv_type, a.flags = MLA_TYPE_F32, kv_type, flags
+    a.scale, a.max_bias, a.logit_softcap = scale, max_bias, logit_softcap
+    a.q = q.data_ptr()
+    a.q_nb1, a.q_nb2, a.q_nb3 = q.stride(2) * 4, q.stride(1) * 4, q.stride(0) * 4
+    es = k.element_size()
+    assert k.stride(-1) == 1 and k.shape[-1] * es == row, (k.shape, k.dtype)
+    a.kv = k.data_ptr()
+    if block_table is not None:
+        assert k.dim() == 2 and k.shape[0] % PAGE_TOKENS == 0
+        a.kv_nb1, a.kv_nb3, a.n_kv = k.stride(0) * es, 0, k.shape[0]
+        assert block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.shape[0] == n_seq and block_table.is_contiguous()
+        assert seq_lens.dtype == torch.int32 and seq_lens.numel() == n_seq and seq_lens.is_contiguous()
+        a.block_table, a.bt_stride, a.seq_lens = block_table.data_ptr(), block_table.shape[1], seq_lens.data_ptr()
+    else:
+        assert k.dim() == 3 and k.shape[0] in (1, n_seq)
+        a.kv_nb1, a.kv_nb3, a.n_kv = k.stride(1) * es, (k.stride(0) * es if k.shape[0] > 1 else 0), k.shape[1]
+    if mask is not None:
+        assert mask.dtype == torch.float16 and mask.dim() == 2 and mask.stride(1) == 1 and mask.shape[0] >= n_tok
+        a.mask, a.mask_nb1, a.mask_ne0 = mask.data_ptr(), mask.stride(0) * 2, mask.shape[1]
+    if out is None:
+        out = torch.empty((n_seq, n_tok, n_head, 576), dtype=torch.float32, device=q.device)
+    assert out.dtype == torch.float32 and out.is_contiguous() and out.shape[:3] == (n_seq, n_tok, n_head) and out.shape[3] >= dv
+    a.dst, a.dst_nb1 = out.data_ptr(), out.shape[3] * 4
+    a.n_splits = n_splits
+    need = library().mla_attn_workspace_size(C.byref(a))
+    ws = _workspace(q.device, need)
+    a.workspace, a.workspace_size = ws.data_ptr(), ws.numel()
+    return a, out, (q, k, mask, block_table, seq_lens, ws)
+
+
+def ggml_flash_attn_ext(q, k, kv_type, dv=512, mask=None, scale=1.0, max_bias=0.0, logit_softcap=0.0, *,
+                        block_table=None, seq_lens=None, out=None, n_splits=0, flags=0, stream=None):
+    """GGML_OP_FLASH_ATTN_EXT of the reference (ggml_flash_attn_ext(ctx, q, k, v, mask, scale, max_bias,
+    logit_softcap), ggml/src/ggml.c:3988) for the MLA shape, on the current torch stream.  v is the first `dv`
+    columns of k's rows.  Returns dst in ggml's layout: float32 [n_seq, n_tok, n_head, 576] with dv columns valid."""
+    import torch
+    if not q.is_cuda:
+        raise RuntimeError("jittorinfer_amd runs on a gfx950 GPU only (there is no CPU path)")
+    a, out, keep = make_args(q, k, kv_type, dv, mask, scale, max_bias, logit_softcap, block_table, seq_lens, out, n_splits, flags)
+    st = stream if stream is not None else torch.cuda.current_stream(q.device).cuda_stream
+    rc = library().mla_attn_launch(C.byref(a), C.c_void_p(st))
+    if rc != 0:
+        raise RuntimeError("mla_attn_launch failed with code %d" % rc)
+    return out
+
+
+def plan(q, k, kv_type, **kw):
+    a, _, keep = make_args(q, k, kv_type, **kw)
+    info = MlaPlanInfo()
+    rc = library().mla_attn_plan(C.byref(a), C.byref(info))
+    if rc != 0:
+        raise RuntimeError("mla_attn_plan failed with code %d" % rc)
+    return {f: getattr(info, f) for f, _ in MlaPlanInfo._fields_}
+
+
+def hbm_copy(src, dst, stream=None):
+    import torch
+    st = stream if stream is not None else torch.cuda.current_stream(src.device).cuda_stream
+    rc = library().mla_hbm_copy_launch(src.data_ptr(), dst.data_ptr(), src.numel() * src.element_size(), C.c_void_p(st))
+    if rc != 0:
+        raise RuntimeError("mla_hbm_copy_launch failed with code %d" % rc)

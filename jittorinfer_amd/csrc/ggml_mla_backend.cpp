@@ -1,0 +1,524 @@
+// ggml backend plugin "HIP-MLA": a drop-in for the reference's backend plugin interface that executes
+// GGML_OP_FLASH_ATTN_EXT nodes of the absorbed-MLA shape on an MI355X through the kernels of mla_kernels.hip.
+//
+// It answers the four vtables of ggml/src/ggml-backend-impl.h (buffer type :17-35, buffer :41-69, backend
+// :89-130, device :143-192, reg :198-214) and exports ggml_backend_init / ggml_backend_score, the symbols
+// load_backend looks up with dlsym (ggml/src/ggml-backend-reg.cpp:234-250).  The in-tree template for the wiring
+// is the CANN backend (ggml/src/ggml-cann/ggml-cann.cpp:2228-2432, :2487-2550); nothing of it is reused.
+//
+// The host's ggml is not linked: struct layouts come from ggml_abi.h.  ggml_backend_buffer_init is taken from the
+// host process with dlsym when it is there (so the host's ggml_backend_buffer_free pairs with its own allocation).
+//
+// Node contract (see include/ggml_mla_backend.h): src[0]=q F32 [576,n_tok,H,B]; src[1]=k F16|BF16|Q8_0
+// [576,n_kv,1,B|1]; src[2]=v: k itself or a 512/576-wide view of k at offset 0; src[3]=mask F16 or NULL;
+// optional src[4]=I32 block table [max_blocks,B] and src[5]=I32 [B] sequence lengths; dst F32 [576,H,n_tok,B].
+
+#include <hip/hip_runtime.h>
+#include <dlfcn.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "../../include/ggml_mla_backend.h"
+#include "../../include/mla_attn.h"
+#include "ggml_abi.h"
+
+using namespace ggml_abi;
+
+namespace {
+
+void log_error(const char * fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    fprintf(stderr, "ggml-hip-mla: ");
+    vfprintf(stderr, fmt, ap);
+    fprintf(stderr, "\n");
+    va_end(ap);
+}
+
+#define HIP_OK(expr) ((expr) == hipSuccess)
+
+// ---------------------------------------------------------------- per-device state
+
+struct device_ctx {
+    int         index;
+    std::string name;         // "HIPMLA0"
+    std::string description;  // hipDeviceProp_t::name
+    backend_buffer_type buft;
+};
+
+struct buffer_ctx {
+    int    device;
+    void * base;
+};
+
+struct backend_ctx {
+    int         device;
+    std::string name;
+    hipStream_t stream;
+    void *      workspace      = nullptr;
+    size_t      workspace_size = 0;
+};
+
+std::vector<device_ctx *>     g_device_ctx;
+std::vector<backend_device *> g_devices;
+backend_reg                   g_reg;
+std::once_flag                g_once;
+uint8_t                       g_guid[16] = { 0x6d, 0x6c, 0x61, 0x2d, 0x68, 0x69, 0x70, 0x2d, 0x67, 0x66, 0x78, 0x39, 0x35, 0x30, 0x00, 0x01 };
+
+int64_t nelements(const tensor * t) { return t->ne[0] * t->ne[1] * t->ne[2] * t->ne[3]; }
+bool    is_empty(const tensor * t) { return nelements(t) == 0; }
+
+// bytes spanned by a tensor with ggml strides (ggml_nbytes, ggml/src/ggml.c) for the types this backend sees
+size_t type_size(int type) {
+    switch (type) {
+        case TYPE_F32: case TYPE_I32: return 4;
+        case TYPE_F16: case TYPE_BF16: case TYPE_I16: return 2;
+        case TYPE_I8: return 1;
+        case TYPE_I64: case TYPE_F64: return 8;
+        case TYPE_Q8_0: return sizeof(block_q8_0);
+        default: return 0;
+    }
+}
+int64_t blck_size(int type) { return type == TYPE_Q8_0 ? 32 : 1; }
+size_t  tensor_nbytes(const tensor * t) {
+    if (is_empty(t)) return 0;
+    const int64_t blck = blck_size(t->type);
+    size_t nbytes;
+    if (blck == 1) {
+        nbytes = type_size(t->type);
+        for (int i = 0; i < MAX_DIMS; i++) nbytes += (t->ne[i] - 1) * t->nb[i];
+    } else {
+        nbytes = t->ne[0] * t->nb[0] / blck;
+        for (int i = 1; i < MAX_DIMS; i++) nbytes += (t->ne[i] - 1) * t->nb[i];
+    }
+    return nbytes;
+}
+bool is_contiguous(const tensor * t) {
+    size_t next = type_size(t->type);
+    if (t->ne[0] != blck_size(t->type) && t->nb[0] != next) return false;
+    next *= t->ne[0] / blck_size(t->type);
+    for (int i = 1; i < MAX_DIMS; i++) {
+        if (t->ne[i] != 1 && t->nb[i] != next) return false;
+        next *= t->ne[i];
+    }
+    return true;
+}
+
+// ---------------------------------------------------------------- buffer
+
+void buffer_free(backend_buffer * buffer) {
+    buffer_ctx * ctx = (buffer_ctx *) buffer->context;
+    (void) hipSetDevice(ctx->device);
+    (void) hipFree(ctx->base);
+    delete ctx;
+}
+void * buffer_get_base(backend_buffer * buffer) { return ((buffer_ctx *) buffer->context)->base; }
+
+void buffer_memset_tensor(backend_buffer * buffer, tensor * t, uint8_t value, size_t offset, size_t size) {
+    buffer_ctx * ctx = (buffer_ctx *) buffer->context;
+    (void) hipSetDevice(ctx->device);
+    if (!HIP_OK(hipMemset((char *) t->data + offset, value, size)) || !HIP_OK(hipDeviceSynchronize())) log_error("memset_tensor failed");
+}
+void buffer_set_tensor(backend_buffer * buffer, tensor * t, const void * data, size_t offset, size_t size) {
+    buffer_ctx * ctx = (buffer_ctx *) buffer->context;
+    (void) hipSetDevice(ctx->device);
+    if (!HIP_OK(hipMemcpy((char *) t->data + offset, data, size, hipMemcpyHostToDevice))) log_error("set_tensor failed");
+}
+void buffer_get_tensor(backend_buffer * buffer, const tensor * t, void * data, size_t offset, size_t size) {
+    buffer_ctx * ctx = (buffer_ctx *) buffer->context;
+    (void) hipSetDevice(ctx->device);
+    if (!HIP_OK(hipMemcpy(data, (const char *) t->data + offset, size, hipMemcpyDeviceToHost))) log_error("get_tensor failed");
+}
+const char * buft_get_name(backend_buffer_type * buft);
+bool buffer_cpy_tensor(backend_buffer * buffer, const tensor * src, tensor * dst) {
+    buffer_ctx * ctx = (buffer_ctx *) buffer->context;
+    if (!src->buffer || !src->buffer->buft) return false;
+    const size_t n = tensor_nbytes(src);
+    (void) hipSetDevice(ctx->device);
+    backend_buffer_type * sb = src->buffer->buft;
+    if (sb->iface.is_host && sb->iface.is_host(sb)) {
+        return HIP_OK(hipMemcpy(dst->data, src->data, n, hipMemcpyHostToDevice));
+    }
+    if (sb->iface.get_name == buft_get_name) {  // one of ours (any device)
+        return HIP_OK(hipMemcpy(dst->data, src->data, n, hipMemcpyDeviceToDevice));
+    }
+    return false;
+}
+void buffer_clear(backend_buffer * buffer, uint8_t value) {
+    buffer_ctx * ctx = (buffer_ctx *) buffer->context;
+    (void) hipSetDevice(ctx->device);
+    if (!HIP_OK(hipMemset(ctx->base, value, buffer->size)) || !HIP_OK(hipDeviceSynchronize())) log_error("clear failed");
+}
+
+const backend_buffer_i k_buffer_iface = {
+    /* free_buffer   */ buffer_free,
+    /* get_base      */ buffer_get_base,
+    /* init_tensor   */ nullptr,
+    /* memset_tensor */ buffer_memset_tensor,
+    /* set_tensor    */ buffer_set_tensor,
+    /* get_tensor    */ buffer_get_tensor,
+    /* cpy_tensor    */ buffer_cpy_tensor,
+    /* clear         */ buffer_clear,
+    /* reset         */ nullptr,
+};
+
+typedef backend_buffer * (*buffer_init_fn)(backend_buffer_type *, backend_buffer_i, void *, size_t);
+
+backend_buffer * make_buffer(backend_buffer_type * buft, void * context, size_t size) {
+    static buffer_init_fn host_init = (buffer_init_fn) dlsym(RTLD_DEFAULT, "ggml_backend_buffer_init");
+    if (host_init) return host_init(buft, k_buffer_iface, context, size);
+    // stand-alone use (no ggml in the process): same object the host would have built (ggml-backend.cpp buffer_init)
+    return new backend_buffer{ k_buffer_iface, buft, context, size, BUFFER_USAGE_ANY };
+}
+
+// ---------------------------------------------------------------- buffer type
+
+const char * buft_get_name(backend_buffer_type * buft) { return ((device_ctx *) buft->context)->name.c_str(); }
+
+backend_buffer * buft_alloc_buffer(backend_buffer_type * buft, size_t size) {
+    device_ctx * dc = (device_ctx *) buft->context;
+    if (!HIP_OK(hipSetDevice(dc->index))) return nullptr;
+    void * p = nullptr;
+    if (size == 0) size = 1;
+    const hipError_t e = hipMalloc(&p, size);
+    if (e != hipSuccess) {
+        log_error("allocating %.2f MiB on device %d failed: %s", size / 1048576.0, dc->index, hipGetErrorString(e));
+        return nullptr;
+    }
+    return make_buffer(buft, new buffer_ctx{ dc->index, p }, size);
+}
+size_t buft_get_alignment(backend_buffer_type *) { return 256; }
+bool   buft_is_host(backend_buffer_type *) { return false; }
+
+// ---------------------------------------------------------------- op support
+
+bool is_noop(int op) { return op == OP_NONE || op == OP_RESHAPE || op == OP_VIEW || op == OP_PERMUTE || op == OP_TRANSPOSE; }
+
+const tensor * view_root(const tensor * t, size_t * offs) {
+    *offs = 0;
+    while (t->view_src) { *offs += t->view_offs; t = t->view_src; }
+    return t;
+}
+
+// Fills `why` (if given) with the first violated clause of the node contract.
+bool mla_node_ok(const tensor * dst, const char ** why) {
+    const char * dummy;
+    if (!why) why = &dummy;
+    const tensor * q = dst->src[0], * k = dst->src[1], * v = dst->src[2], * mask = dst->src[3];
+    const tensor * bt = dst->src[4], * lens = dst->src[5];
+    if (!q || !k || !v) { *why = "missing q/k/v"; return false; }
+    if (q->type != TYPE_F32 || q->nb[0] != 4) { *why = "q must be F32 with contiguous rows"; return false; }
+    if (q->ne[0] != 576 || k->ne[0] != 576) { *why = "head size must be 576 (512 latent + 64 rope)"; return false; }
+    if (k->type != TYPE_F16 && k->type != TYPE_BF16 && k->type != TYPE_Q8_0) { *why = "k must be F16, BF16 or Q8_0"; return false; }
+    if (k->ne[2] != 1) { *why = "MLA has a single latent KV head"; return false; }
+    if (k->nb[0] != type_size(k->type)) { *why = "k rows must be contiguous"; return false; }
+    if (v->type != k->type) { *why = "v must have k's type"; return false; }
+    if (v->ne[0] != 512 && v->ne[0] != 576) { *why = "v must be 512 or 576 wide"; return false; }
+    if (v->ne[1] != k->ne[1] || v->ne[2] != 1 || v->ne[3] != k->ne[3]) { *why = "v must cover the same rows as k"; return false; }
+    if (v != k) {  // must alias k: the same latent row supplies both
+        size_t ko, vo;
+        const tensor * kr = view_root(k, &ko), * vr = view_root(v, &vo);
+        if (kr != vr || ko != vo || v->nb[1] != k->nb[1] || v->nb[3] != k->nb[3]) { *why = "v must be a view of k's rows at offset 0"; return false; }
+    }
+    if (dst->type != TYPE_F32 || dst->nb[0] != 4 || dst->ne[0] < v->ne[0]) { *why = "dst must be F32 rows of >= dv floats"; return false; }
+    if (dst->ne[1] != q->ne[2] || dst->ne[2] != q->ne[1] || dst->ne[3] != q->ne[3]) { *why = "dst must be [*, H, n_tok, B]"; return false; }
+    if (dst->nb[2] != dst->nb[1] * (size_t) dst->ne[1] || dst->nb[3] != dst->nb[2] * (size_t) dst->ne[2]) { *why = "dst rows must be evenly strided"; return false; }
+    if (mask) {
+        if (mask->type != TYPE_F16 || !is_contiguous(mask) || mask->ne[2] != 1 || mask->ne[3] != 1) { *why = "mask must be contiguous F16 2-D"; return false; }
+        if (mask->ne[1] < q->ne[1]) { *why = "mask has fewer rows than query tokens"; return false; }
+    }
+    float max_bias;
+    memcpy(&max_bias, (const char *) dst->op_params + 4, 4);
+    if (max_bias > 0.0f && !mask) { *why = "max_bias needs a mask"; return false; }
+    if ((bt != nullptr) != (lens != nullptr)) { *why = "block table and sequence lengths come together"; return false; }
+    if (bt) {
+        if (bt->type != TYPE_I32 || lens->type != TYPE_I32 || !is_contiguous(bt) || !is_contiguous(lens)) { *why = "block table / lengths must be contiguous I32"; return false; }
+        if (bt->ne[1] != q->ne[3] || nelements(lens) != q->ne[3]) { *why = "block table / lengths must have one row per sequence"; return false; }
+        if (k->ne[3] != 1) { *why = "with a block table k is the page pool [576, rows, 1, 1]"; return false; }
+        if (k->ne[1] % MLA_PAGE_TOKENS) { *why = "page pool must hold whole 128-token pages"; return false; }
+    } else {
+        if (k->ne[3] != q->ne[3] && k->ne[3] != 1) { *why = "k batch must equal q batch or be 1"; return false; }
+        if (mask && mask->ne[0] < k->ne[1]) { *why = "mask narrower than n_kv"; return false; }
+    }
+    return true;
+}
+
+bool device_supports_op(backend_device *, const tensor * op) {
+    if (is_noop(op->op)) return true;
+    if (op->op == OP_FLASH_ATTN_EXT) return mla_node_ok(op, nullptr);
+    return false;
+}
+
+// ---------------------------------------------------------------- backend (stream)
+
+const char * backend_get_name(backend * be) { return ((backend_ctx *) be->context)->name.c_str(); }
+
+void backend_free(backend * be) {
+    backend_ctx * ctx = (backend_ctx *) be->context;
+    (void) hipSetDevice(ctx->device);
+    (void) hipStreamSynchronize(ctx->stream);
+    if (ctx->workspace) (void) hipFree(ctx->workspace);
+    (void) hipStreamDestroy(ctx->stream);
+    delete ctx;
+    delete be;
+}
+
+void backend_set_tensor_async(backend * be, tensor * t, const void * data, size_t offset, size_t size) {
+    backend_ctx * ctx = (backend_ctx *) be->context;
+    (void) hipSetDevice(ctx->device);
+    if (!HIP_OK(hipMemcpyAsync((char *) t->data + offset, data, size, hipMemcpyHostToDevice, ctx->stream))) log_error("set_tensor_async failed");
+}
+void backend_get_tensor_async(backend * be, const tensor * t, void * data, size_t offset, size_t size) {
+    backend_ctx * ctx = (backend_ctx *) be->context;
+    (void) hipSetDevice(ctx->device);
+    if (!HIP_OK(hipMemcpyAsync(data, (const char *) t->data + offset, size, hipMemcpyDeviceToHost, ctx->stream))) log_error("get_tensor_async failed");
+}
+void backend_synchronize(backend * be) {
+    backend_ctx * ctx = (backend_ctx *) be->context;
+    (void) hipSetDevice(ctx->device);
+    if (!HIP_OK(hipStreamSynchronize(ctx->stream))) log_error("synchronize failed");
+}
+
+int compute_flash_attn(backend_ctx * ctx, const tensor * dst) {
+    const char * why = nullptr;
+    if (!mla_node_ok(dst, &why)) { log_error("FLASH_ATTN_EXT node '%s' rejected: %s", dst->name, why); return STATUS_FAILED; }
+    const tensor * q = dst->src[0], * k = dst->src[1], * v = dst->src[2], * mask = dst->src[3];
+    const tensor * bt = dst->src[4], * lens = dst->src[5];
+    if (!q->data || !k->data || !dst->data || v->data != k->data) { log_error("node '%s': operands not allocated, or v does not alias k", dst->name); return STATUS_FAILED; }
+
+    mla_attn_args a;
+    memset(&a, 0, sizeof(a));
+    a.n_seq = (int32_t) q->ne[3]; a.n_head = (int32_t) q->ne[2]; a.n_tok = (int32_t) q->ne[1];
+    a.dk = 576; a.dv = (int32_t) v->ne[0];
+    a.q_type = MLA_TYPE_F32; a.kv_type = k->type;
+    memcpy(&a.scale, (const char *) dst->op_params + 0, 4);
+    memcpy(&a.max_bias, (const char *) dst->op_params + 4, 4);
+    memcpy(&a.logit_softcap, (const char *) dst->op_params + 8, 4);
+    a.q = q->data; a.q_nb1 = (int64_t) q->nb[1]; a.q_nb2 = (int64_t) q->nb[2]; a.q_nb3 = (int64_t) q->nb[3];
+    a.kv = k->data; a.kv_nb1 = (int64_t) k->nb[1]; a.kv_nb3 = k->ne[3] == 1 ? 0 : (int64_t) k->nb[3]; a.n_kv = k->ne[1];
+    if (mask) { a.mask = mask->data; a.mask_nb1 = (int64_t) mask->nb[1]; a.mask_ne0 = mask->ne[0]; }
+    if (bt) { a.block_table = (const int32_t *) bt->data; a.bt_stride = bt->ne[0]; a.seq_lens = (const int32_t *) lens->data; }
+    a.dst = (float *) dst->data; a.dst_nb1 = (int64_t) dst->nb[1];
+
+    const size_t need = mla_attn_workspace_size(&a);
+    if (need > ctx->workspace_size) {
+        // grow the scratch area; work already queued on the stream may still be using the old one
+        if (!HIP_OK(hipStreamSynchronize(ctx->stream))) return STATUS_FAILED;
+        if (ctx->workspace) (void) hipFree(ctx->workspace);
+        ctx->workspace = nullptr; ctx->workspace_size = 0;
+        if (!HIP_OK(hipMalloc(&ctx->workspace, need))) { log_error("workspace of %zu bytes: out of memory", need); return STATUS_ALLOC_FAILED; }
+        ctx->workspace_size = need;
+    }
+    a.workspace = ctx->workspace; a.workspace_size = ctx->workspace_size;
+    const int rc = mla_attn_launch(&a, ctx->stream);
+    if (rc != 0) { log_error("mla_attn_launch failed for node '%s': %d", dst->name, rc); return STATUS_FAILED; }
+    return STATUS_SUCCESS;
+}
+
+int backend_graph_compute(backend * be, cgraph * g) {
+    backend_ctx * ctx = (backend_ctx *) be->context;
+    if (!HIP_OK(hipSetDevice(ctx->device))) return STATUS_FAILED;
+    for (int i = 0; i < g->n_nodes; i++) {
+        const tensor * node = g->nodes[i];
+        if (is_empty(node) || is_noop(node->op)) continue;
+        if (node->op != OP_FLASH_ATTN_EXT) { log_error("op %d of node '%s' is not supported", node->op, node->name); return STATUS_FAILED; }
+        const int st = compute_flash_attn(ctx, node);
+        if (st != STATUS_SUCCESS) return st;
+    }
+    return STATUS_SUCCESS;
+}
+
+const backend_i k_backend_iface = {
+    /* get_name           */ backend_get_name,
+    /* free               */ backend_free,
+    /* set_tensor_async   */ backend_set_tensor_async,
+    /* get_tensor_async   */ backend_get_tensor_async,
+    /* cpy_tensor_async   */ nullptr,
+    /* synchronize        */ backend_synchronize,
+    /* graph_plan_create  */ nullptr,
+    /* graph_plan_free    */ nullptr,
+    /* graph_plan_update  */ nullptr,
+    /* graph_plan_compute */ nullptr,
+    /* graph_compute      */ backend_graph_compute,
+    /* event_record       */ nullptr,
+    /* event_wait         */ nullptr,
+};
+
+// ---------------------------------------------------------------- device
+
+const char * device_get_name(backend_device * dev) { return ((device_ctx *) dev->context)->name.c_str(); }
+const char * device_get_description(backend_device * dev) { return ((device_ctx *) dev->context)->description.c_str(); }
+void device_get_memory(backend_device * dev, size_t * free, size_t * total) {
+    device_ctx * dc = (device_ctx *) dev->context;
+    *free = *total = 0;
+    if (HIP_OK(hipSetDevice(dc->index))) (void) hipMemGetInfo(free, total);
+}
+int  device_get_type(backend_device *) { return DEVICE_TYPE_GPU; }
+void device_get_props(backend_device * dev, dev_props * props) {
+    props->name        = device_get_name(dev);
+    props->description = device_get_description(dev);
+    props->type        = DEVICE_TYPE_GPU;
+    device_get_memory(dev, &props->memory_free, &props->memory_total);
+    props->caps = dev_caps{ /* async */ true, /* host_buffer */ false, /* buffer_from_host_ptr */ false, /* events */ false };
+}
+backend * device_init_backend(backend_device * dev, const char *) {
+    device_ctx * dc = (device_ctx *) dev->context;
+    if (!HIP_OK(hipSetDevice(dc->index))) return nullptr;
+    backend_ctx * ctx = new backend_ctx;
+    ctx->device = dc->index;
+    ctx->name   = dc->name;
+    if (!HIP_OK(hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking))) { delete ctx; return nullptr; }
+    return new backend{ &g_guid, k_backend_iface, dev, ctx };
+}
+backend_buffer_type * device_get_buffer_type(backend_device * dev) { return &((device_ctx *) dev->context)->buft; }
+bool device_supports_buft(backend_device * dev, backend_buffer_type * buft) { return buft == device_get_buffer_type(dev); }
+
+const backend_device_i k_device_iface = {
+    /* get_name             */ device_get_name,
+    /* get_description      */ device_get_description,
+    /* get_memory           */ device_get_memory,
+    /* get_type             */ device_get_type,
+    /* get_props            */ device_get_props,
+    /* init_backend         */ device_init_backend,
+    /* get_buffer_type      */ device_get_buffer_type,
+    /* get_host_buffer_type */ nullptr,
+    /* buffer_from_host_ptr */ nullptr,
+    /* supports_op          */ device_supports_op,
+    /* supports_buft        */ device_supports_buft,
+    /* offload_op           */ nullptr,
+    /* event_new            */ nullptr,
+    /* event_free           */ nullptr,
+    /* event_synchronize    */ nullptr,
+};
+
+// ---------------------------------------------------------------- registry
+
+const char * reg_get_name(backend_reg *) { return "HIP-MLA"; }
+size_t       reg_get_device_count(backend_reg *) { return g_devices.size(); }
+backend_device * reg_get_device(backend_reg *, size_t index) { return index < g_devices.size() ? g_devices[index] : nullptr; }
+// The reference probes for "ggml_backend_set_n_threads", "ggml_backend_set_abort_callback" and
+// "ggml_backend_comm_init*" (src/llama-context-load-utils.cpp:72-76, :360-385); none applies here.
+void * reg_get_proc_address(backend_reg *, const char *) { return nullptr; }
+
+int gfx950_device_count() {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) { (void) hipGetLastError(); return 0; }
+    int ok = 0;
+    for (int i = 0; i < n; i++) {
+        hipDeviceProp_t prop;
+        if (hipGetDeviceProperties(&prop, i) != hipSuccess) continue;
+        if (strncmp(prop.gcnArchName, "gfx950", 6) == 0) ok++;
+    }
+    return ok;
+}
+
+void init_registry() {
+    g_reg.api_version = BACKEND_API_VERSION;
+    g_reg.iface       = backend_reg_i{ reg_get_name, reg_get_device_count, reg_get_device, reg_get_proc_address };
+    g_reg.context     = nullptr;
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) { (void) hipGetLastError(); n = 0; }
+    for (int i = 0; i < n; i++) {
+        hipDeviceProp_t prop;
+        if (hipGetDeviceProperties(&prop, i) != hipSuccess) continue;
+        if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) continue;  // the kernels exist for gfx950 only
+        device_ctx * dc = new device_ctx;
+        dc->index       = i;
+        dc->name        = "HIPMLA" + std::to_string(i);
+        dc->description = prop.name;
+        backend_device * dev = new backend_device{ k_device_iface, &g_reg, dc };
+        dc->buft.iface   = backend_buffer_type_i{ buft_get_name, buft_alloc_buffer, buft_get_alignment, nullptr, nullptr, buft_is_host };
+        dc->buft.device  = dev;
+        dc->buft.context = dc;
+        g_device_ctx.push_back(dc);
+        g_devices.push_back(dev);
+    }
+}
+
+struct abi_entry { const char * name; int64_t value; };
+#define E(n, v) { n, (int64_t) (v) }
+const abi_entry k_abi_table[] = {
+    E("sizeof(ggml_tensor)", sizeof(tensor)),
+    E("offsetof(ggml_tensor,type)", offsetof(tensor, type)), E("offsetof(ggml_tensor,buffer)", offsetof(tensor, buffer)),
+    E("offsetof(ggml_tensor,ne)", offsetof(tensor, ne)), E("offsetof(ggml_tensor,nb)", offsetof(tensor, nb)),
+    E("offsetof(ggml_tensor,op)", offsetof(tensor, op)), E("offsetof(ggml_tensor,op_params)", offsetof(tensor, op_params)),
+    E("offsetof(ggml_tensor,flags)", offsetof(tensor, flags)), E("offsetof(ggml_tensor,src)", offsetof(tensor, src)),
+    E("offsetof(ggml_tensor,view_src)", offsetof(tensor, view_src)), E("offsetof(ggml_tensor,view_offs)", offsetof(tensor, view_offs)),
+    E("offsetof(ggml_tensor,data)", offsetof(tensor, data)), E("offsetof(ggml_tensor,name)", offsetof(tensor, name)),
+    E("offsetof(ggml_tensor,extra)", offsetof(tensor, extra)),
+    E("GGML_MAX_DIMS", MAX_DIMS), E("GGML_MAX_SRC", MAX_SRC), E("GGML_MAX_OP_PARAMS", MAX_OP_PARAMS), E("GGML_MAX_NAME", MAX_NAME),
+    E("GGML_KQ_MASK_PAD", KQ_MASK_PAD),
+    E("sizeof(ggml_cgraph)", sizeof(cgraph)), E("offsetof(ggml_cgraph,n_nodes)", offsetof(cgraph, n_nodes)), E("offsetof(ggml_cgraph,nodes)", offsetof(cgraph, nodes)),
+    E("sizeof(ggml_backend_buffer_type_i)", sizeof(backend_buffer_type_i)), E("sizeof(ggml_backend_buffer_type)", sizeof(backend_buffer_type)),
+    E("offsetof(ggml_backend_buffer_type,device)", offsetof(backend_buffer_type, device)), E("offsetof(ggml_backend_buffer_type,context)", offsetof(backend_buffer_type, context)),
+    E("sizeof(ggml_backend_buffer_i)", sizeof(backend_buffer_i)), E("sizeof(ggml_backend_buffer)", sizeof(backend_buffer)),
+    E("offsetof(ggml_backend_buffer,buft)", offsetof(backend_buffer, buft)), E("offsetof(ggml_backend_buffer,context)", offsetof(backend_buffer, context)),
+    E("offsetof(ggml_backend_buffer,size)", offsetof(backend_buffer, size)), E("offsetof(ggml_backend_buffer,usage)", offsetof(backend_buffer, usage)),
+    E("sizeof(ggml_backend_i)", sizeof(backend_i)), E("offsetof(ggml_backend_i,graph_compute)", offsetof(backend_i, graph_compute)),
+    E("offsetof(ggml_backend_i,synchronize)", offsetof(backend_i, synchronize)),
+    E("sizeof(ggml_backend)", sizeof(backend)), E("offsetof(ggml_backend,iface)", offsetof(backend, iface)),
+    E("offsetof(ggml_backend,device)", offsetof(backend, device)), E("offsetof(ggml_backend,context)", offsetof(backend, context)),
+    E("sizeof(ggml_backend_device_i)", sizeof(backend_device_i)), E("offsetof(ggml_backend_device_i,supports_op)", offsetof(backend_device_i, supports_op)),
+    E("sizeof(ggml_backend_device)", sizeof(backend_device)), E("offsetof(ggml_backend_device,reg)", offsetof(backend_device, reg)),
+    E("offsetof(ggml_backend_device,context)", offsetof(backend_device, context)),
+    E("sizeof(ggml_backend_reg_i)", sizeof(backend_reg_i)), E("sizeof(ggml_backend_reg)", sizeof(backend_reg)),
+    E("offsetof(ggml_backend_reg,iface)", offsetof(backend_reg, iface)), E("offsetof(ggml_backend_reg,context)", offsetof(backend_reg, context)),
+    E("sizeof(ggml_backend_dev_props)", sizeof(dev_props)), E("offsetof(ggml_backend_dev_props,type)", offsetof(dev_props, type)),
+    E("offsetof(ggml_backend_dev_props,caps)", offsetof(dev_props, caps)),
+    E("sizeof(ggml_backend_event)", sizeof(backend_event)),
+    E("GGML_BACKEND_API_VERSION", BACKEND_API_VERSION),
+    E("GGML_TYPE_F32", TYPE_F32), E("GGML_TYPE_F16", TYPE_F16), E("GGML_TYPE_Q8_0", TYPE_Q8_0), E("GGML_TYPE_I8", TYPE_I8),
+    E("GGML_TYPE_I32", TYPE_I32), E("GGML_TYPE_BF16", TYPE_BF16), E("GGML_TYPE_COUNT", TYPE_COUNT),
+    E("GGML_OP_NONE", OP_NONE), E("GGML_OP_CPY", OP_CPY), E("GGML_OP_CONT", OP_CONT), E("GGML_OP_RESHAPE", OP_RESHAPE),
+    E("GGML_OP_VIEW", OP_VIEW), E("GGML_OP_PERMUTE", OP_PERMUTE), E("GGML_OP_TRANSPOSE", OP_TRANSPOSE),
+    E("GGML_OP_FLASH_ATTN_EXT", OP_FLASH_ATTN_EXT), E("GGML_OP_SCATTER_UPDATE", OP_SCATTER_UPDATE), E("GGML_OP_COUNT", OP_COUNT),
+    E("GGML_STATUS_ALLOC_FAILED", STATUS_ALLOC_FAILED), E("GGML_STATUS_FAILED", STATUS_FAILED), E("GGML_STATUS_SUCCESS", STATUS_SUCCESS),
+    E("GGML_STATUS_ABORTED", STATUS_ABORTED),
+    E("GGML_BACKEND_DEVICE_TYPE_CPU", DEVICE_TYPE_CPU), E("GGML_BACKEND_DEVICE_TYPE_GPU", DEVICE_TYPE_GPU),
+    E("GGML_BACKEND_BUFFER_USAGE_ANY", BUFFER_USAGE_ANY), E("GGML_BACKEND_BUFFER_USAGE_COMPUTE", BUFFER_USAGE_COMPUTE),
+    E("GGML_PREC_DEFAULT", PREC_DEFAULT), E("GGML_PREC_F32", PREC_F32),
+    E("GGML_TENSOR_FLAG_INPUT", TENSOR_FLAG_INPUT), E("GGML_TENSOR_FLAG_OUTPUT", TENSOR_FLAG_OUTPUT),
+    E("sizeof(block_q8_0)", sizeof(block_q8_0)),
+};
+
+}  // namespace
+
+extern "C" {
+
+void * ggml_backend_init(void) {
+    std::call_once(g_once, init_registry);
+    return &g_reg;
+}
+
+int ggml_backend_score(void) { return gfx950_device_count() > 0 ? 100 : 0; }
+
+void * ggml_backend_hip_mla_reg(void) { return ggml_backend_init(); }
+
+int mla_ggml_abi_table(int i, const char ** name, int64_t * value) {
+    const int n = (int) (sizeof(k_abi_table) / sizeof(k_abi_table[0]));
+    if (i < 0 || i >= n) return n;
+    *name  = k_abi_table[i].name;
+    *value = k_abi_table[i].value;
+    return n;
+}
+
+void mla_ggml_buffer_free(void * buffer) {
+    backend_buffer * b = (backend_buffer *) buffer;
+    if (!b) return;
+    if (b->iface.free_buffer) b->iface.free_buffer(b);
+    delete b;
+}
+
+int mla_ggml_supports_node(const void * node, const char ** why) {
+    const tensor * t = (const tensor *) node;
+    if (t->op != OP_FLASH_ATTN_EXT) { if (why) *why = "not a FLASH_ATTN_EXT node"; return 0; }
+    return mla_node_ok(t, why) ? 1 : 0;
+}
+
+}  // extern "C"

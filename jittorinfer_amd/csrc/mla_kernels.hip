@@ -1,0 +1,767 @@
+// Absorbed-MLA attention for gfx950 (MI355X): hand-written HIP kernels behind the C ABI of include/mla_attn.h.
+//
+// The op is GGML_OP_FLASH_ATTN_EXT as ggml-cpu computes it (ggml/src/ggml-cpu/ggml-cpu.c:11914-12124 of the
+// reference) specialised to what llm_attn_mla feeds it (src/llama-graph-attn.cpp:259-315): Q rows of 576,
+// one latent K row of 576 per cached token shared by every head, V = the first 512 (or all 576) columns of
+// the same row.  A "row" below is one (query token, head) pair; all rows of a sequence read the same KV rows.
+//
+// Data flow of the tiled kernel (mla_attn_tile_kernel):
+//   HBM --16-byte coalesced loads (through the block table)--> registers --(dequant)--> LDS tile [32 tokens][576]
+//   S^T[token, row]  = K_tile . Q^T      v_mfma_f32_32x32x16_{bf16,f16}, K from LDS (ds_read_b128), Q in VGPRs
+//   online softmax on S^T in its accumulator layout (one row per lane pair, exchange across lanes 32 apart)
+//   O^T[d, row]     += V_tile^T . P^T    same MFMA; V^T fragments come from the SAME row-major LDS tile through
+//                                        ds_read_b64_tr_b16, P^T is the S^T accumulator re-packed in registers
+// so a KV tile is read from HBM once per workgroup and serves every head the workgroup owns.
+// Split-K partials (unnormalised O, running max, running sum) go to the workspace and are merged by
+// mla_attn_combine_kernel with the usual log-sum-exp rule.
+//
+// gfx950 only: v_mfma_f32_32x32x16_*, ds_read_b64_tr_b16, 160 KB LDS, 64-wide waves.
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <math.h>
+
+#include "../../include/mla_attn.h"
+
+namespace {
+
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
+typedef __attribute__((ext_vector_type(4))) short        s16x4;
+typedef __attribute__((ext_vector_type(16))) float       f32x16;
+typedef __attribute__((ext_vector_type(4))) float        f32x4;
+typedef __attribute__((ext_vector_type(8))) __bf16       bf16x8;
+typedef __attribute__((ext_vector_type(8))) _Float16     f16x8;
+
+#define LDS_PTR(T) T __attribute__((address_space(3))) *
+
+constexpr int DK          = 576;
+constexpr int KSTEPS      = DK / 16;  // 36 MFMA k-steps over the 576-d contraction
+constexpr int TILE_TOK    = 32;       // tokens per LDS tile (= MFMA M of S^T)
+constexpr int ROW_BYTES   = DK * 2;   // one latent row in LDS (bf16 / f16)
+constexpr int PITCH       = ROW_BYTES + 16;  // padded row pitch: 292 dwords, conflict-free for the b128 K reads
+constexpr int TILE_BYTES  = TILE_TOK * PITCH;
+constexpr int Q8_ROW      = 612;      // 18 blocks of (fp16 d, 32 x int8)
+constexpr int Q8_TILE_RAW = TILE_TOK * Q8_ROW;  // 19584 = 1224 x 16
+constexpr int NTHREADS    = 256;
+constexpr float LOG2E     = 1.4426950408889634f;
+
+enum { SRC_BF16 = 0, SRC_F16 = 1, SRC_Q8 = 2 };
+
+struct KParams {
+    const char *    q;
+    int64_t         q_nb1, q_nb2, q_nb3;
+    const char *    kv;
+    int64_t         kv_nb1, kv_nb3;
+    int64_t         n_kv;
+    const char *    mask;
+    int64_t         mask_nb1, mask_ne0;
+    const int32_t * block_table;
+    int64_t         bt_stride;
+    const int32_t * seq_lens;
+    float *         dst;
+    int64_t         dst_stride;  // floats
+    float *         part_o;      // [n_seq][n_splits][n_rows][dv_total]
+    float *         part_ml;     // [n_seq][n_splits][n_rows][2]  (max in log2 units, sum)
+    int             n_head, n_tok, n_rows;
+    int             n_splits, split_tokens;
+    int             dv_total, d_off;
+    float           scale, softcap, max_bias, m0, m1;
+    int             n_head_log2;
+    int             n_pool_pages;  // block-table mode: pages in the pool
+    int             rows_contig;  // kv rows are packed (kv_nb1 == row bytes): whole tiles are one contiguous run
+};
+
+template <typename T, typename U> __device__ __forceinline__ T bitcast(U u) { return __builtin_bit_cast(T, u); }
+
+template <bool F16> __device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
+    if constexpr (F16) return __builtin_amdgcn_mfma_f32_32x32x16_f16(bitcast<f16x8>(a), bitcast<f16x8>(b), c, 0, 0, 0);
+    else               return __builtin_amdgcn_mfma_f32_32x32x16_bf16(bitcast<bf16x8>(a), bitcast<bf16x8>(b), c, 0, 0, 0);
+}
+
+// f32 -> bf16 bits, round to nearest even, NaN quieted (ggml/src/ggml-impl.h:553-568)
+__device__ __forceinline__ unsigned int f32_to_bf16_bits(float f) {
+    unsigned int i = __float_as_uint(f);
+    if ((i & 0x7fffffffu) > 0x7f800000u) return (i >> 16) | 64u;
+    return (i + (0x7fffu + ((i >> 16) & 1u))) >> 16;
+}
+__device__ __forceinline__ unsigned int f32_to_f16_bits(float f) { return (unsigned int) bitcast<unsigned short>((_Float16) f); }
+__device__ __forceinline__ float        f16_bits_to_f32(unsigned int h) { return (float) bitcast<_Float16>((unsigned short) h); }
+
+template <bool F16> __device__ __forceinline__ unsigned int pack2(float a, float b) {
+    if constexpr (F16) return f32_to_f16_bits(a) | (f32_to_f16_bits(b) << 16);
+    else               return f32_to_bf16_bits(a) | (f32_to_bf16_bits(b) << 16);
+}
+template <bool F16> __device__ __forceinline__ float round_trip(float a) {
+    if constexpr (F16) return (float) (_Float16) a;
+    else               return __uint_as_float(f32_to_bf16_bits(a) << 16);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }  // v_exp_f32; exp2(-inf) = 0
+
+__device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); }
+
+// ---------------------------------------------------------------------------------------------------------------
+// Tiled MFMA kernel.
+//   SRC  : storage type of the KV rows
+//   NDB  : number of 32-wide d blocks of the output this launch produces (16 -> 512 columns, 9 -> 288 columns)
+//   WM   : waves along rows (each wave owns 32 rows); WD: waves along d (each owns NDB/WD blocks); WM*WD == 4
+// grid = (n_splits, n_row_blocks, n_seq), block = 256.
+// ---------------------------------------------------------------------------------------------------------------
+template <int SRC, int NDB, int WM, int WD>
+__global__ void __launch_bounds__(NTHREADS) mla_attn_tile_kernel(const KParams p) {
+    constexpr bool F16   = (SRC != SRC_BF16);  // LDS element type: f16 for f16 and Q8_0 sources, bf16 for bf16
+    constexpr bool SPLIT = !F16;               // bf16 P is split into hi + lo so that P.V keeps ~16 mantissa bits
+    constexpr int  NDBW  = NDB / WD;
+    constexpr int  RBLK  = 32 * WM;
+    static_assert(WM * WD == 4 && NDB % WD == 0, "wave layout");
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    // smem: [2][TILE_BYTES] tile double buffer, then (Q8 only) [Q8_TILE_RAW] raw staging
+
+    const int tid  = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm   = wave / WD;
+    const int wd   = wave % WD;
+    const int g    = lane >> 5;  // which half of the k-slots this lane feeds
+    const int rl   = lane & 31;  // MFMA column: the attention row this lane owns
+    const int b    = blockIdx.z;
+    const int split = blockIdx.x;
+
+    const int seq_len  = p.block_table ? min(p.seq_lens[b], (int) p.bt_stride * MLA_PAGE_TOKENS) : (int) p.n_kv;
+    const int kv_begin = split * p.split_tokens;
+    const int kv_end   = min(seq_len, kv_begin + p.split_tokens);
+    if (kv_begin >= kv_end && !(seq_len <= 0 && split == 0)) return;  // nothing to do; the combine pass knows
+
+    const int  row       = blockIdx.y * RBLK + wm * 32 + rl;
+    const bool row_valid = row < p.n_rows;
+    const int  rowc      = row_valid ? row : p.n_rows - 1;
+    const int  tq        = rowc / p.n_head;  // query token of this row
+    const int  head      = rowc - tq * p.n_head;
+
+    // ---- Q -> registers in MFMA B layout: k-step ks holds d = 16*ks + 8*g .. +7 of row `rl`
+    u32x4 qreg[KSTEPS];
+    {
+        const float * qrow = (const float *) (p.q + (int64_t) tq * p.q_nb1 + (int64_t) head * p.q_nb2 + (int64_t) b * p.q_nb3);
+        if constexpr (SRC == SRC_Q8) {
+            // ggml-cpu quantizes Q to Q8_0 when K is Q8_0 (ggml-cpu.c:313-322, :12034-12035): per 32-block
+            // d = amax/127 (stored as f16), id = 127/amax, q = round-half-even(x*id) (ggml-cpu-quants.c:855-900).
+            // The MFMA operand is the dequantized value q * f16(d), rounded to f16.
+#pragma unroll
+            for (int j = 0; j < KSTEPS / 2; j++) {
+                f32x4 x[4];
+                x[0] = *(const f32x4 *) (qrow + 32 * j + 8 * g);
+                x[1] = *(const f32x4 *) (qrow + 32 * j + 8 * g + 4);
+                x[2] = *(const f32x4 *) (qrow + 32 * j + 16 + 8 * g);
+                x[3] = *(const f32x4 *) (qrow + 32 * j + 16 + 8 * g + 4);
+                float amax = 0.f;
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+#pragma unroll
+                    for (int c = 0; c < 4; c++) amax = fmaxf(amax, fabsf(x[e][c]));
+                amax           = fmaxf(amax, xor32(amax));
+                const float d  = f16_bits_to_f32(f32_to_f16_bits(amax / 127.0f));
+                const float id = amax != 0.f ? 127.0f / amax : 0.f;
+                float y[16];
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+#pragma unroll
+                    for (int c = 0; c < 4; c++) y[e * 4 + c] = rintf(x[e][c] * id) * d;
+                u32x4 lo, hi;
+                lo.x = pack2<true>(y[0], y[1]);   lo.y = pack2<true>(y[2], y[3]);
+                lo.z = pack2<true>(y[4], y[5]);   lo.w = pack2<true>(y[6], y[7]);
+                hi.x = pack2<true>(y[8], y[9]);   hi.y = pack2<true>(y[10], y[11]);
+                hi.z = pack2<true>(y[12], y[13]); hi.w = pack2<true>(y[14], y[15]);
+                qreg[2 * j]     = lo;
+                qreg[2 * j + 1] = hi;
+            }
+        } else {
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS; ks++) {
+                const f32x4 x0 = *(const f32x4 *) (qrow + 16 * ks + 8 * g);
+                const f32x4 x1 = *(const f32x4 *) (qrow + 16 * ks + 8 * g + 4);
+                u32x4 v;
+                v.x = pack2<F16>(x0.x, x0.y); v.y = pack2<F16>(x0.z, x0.w);
+                v.z = pack2<F16>(x1.x, x1.y); v.w = pack2<F16>(x1.z, x1.w);
+                qreg[ks] = v;
+            }
+        }
+    }
+
+    // ALiBi slope of this row's head (ggml-cpu.c:11985-11989, :12006-12008); 1 when max_bias == 0
+    float slope = 1.0f;
+    if (p.max_bias > 0.0f) {
+        slope = head < p.n_head_log2 ? powf(p.m0, (float) (head + 1)) : powf(p.m1, (float) (2 * (head - p.n_head_log2) + 1));
+    }
+    const float scale_eff = p.softcap != 0.0f ? p.scale / p.softcap : p.scale;
+    const char * mask_row = p.mask ? p.mask + (int64_t) tq * p.mask_nb1 : nullptr;
+
+    f32x16 acc[NDBW];
+#pragma unroll
+    for (int i = 0; i < NDBW; i++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) acc[i][e] = 0.f;
+    float m_run = -INFINITY;  // running max, log2 units
+    float l_run = 0.f;        // running sum (this lane's 16 of the 32 tokens of each tile)
+
+    const int n_tiles = (kv_end - kv_begin + TILE_TOK - 1) / TILE_TOK;
+
+    // ---- staging: global -> registers -> LDS
+    constexpr int N_PRE = (SRC == SRC_Q8) ? (Q8_TILE_RAW / 16 + NTHREADS - 1) / NTHREADS : (TILE_TOK * (ROW_BYTES / 16)) / NTHREADS;  // 5 or 9
+    u32x4 pre[N_PRE];
+
+    auto tile_row_ptr = [&](int ic) -> const char * {  // address of logical KV row ic of this sequence
+        if (p.block_table) {
+            int page = p.block_table[(int64_t) b * p.bt_stride + (ic >> 7)];
+            page = max(0, min(page, p.n_pool_pages - 1));  // a corrupt table must not turn into a wild address
+            return p.kv + ((int64_t) page * MLA_PAGE_TOKENS + (ic & 127)) * p.kv_nb1;
+        }
+        return p.kv + (int64_t) ic * p.kv_nb1 + (int64_t) b * p.kv_nb3;
+    };
+
+    auto prefetch = [&](int it) {
+        const int t0   = kv_begin + it * TILE_TOK;
+        const int nrow = min(TILE_TOK, kv_end - t0);
+        if constexpr (SRC == SRC_Q8) {
+            if (p.rows_contig && nrow == TILE_TOK) {
+                const char * base = tile_row_ptr(t0);
+#pragma unroll
+                for (int j = 0; j < N_PRE; j++) {
+                    const int c = tid + j * NTHREADS;
+                    if (c < Q8_TILE_RAW / 16) pre[j] = *(const u32x4 *) (base + (int64_t) c * 16);
+                }
+            } else {
+                // generic: 2-byte granules, row by row (rows are only 2-byte aligned); zero past the end
+#pragma unroll
+                for (int j = 0; j < N_PRE; j++) {
+                    const int c = tid + j * NTHREADS;
+                    unsigned short h[8];
+#pragma unroll
+                    for (int e = 0; e < 8; e++) {
+                        const int off = c * 16 + e * 2;
+                        const int r   = off / Q8_ROW;
+                        unsigned short v = 0;
+                        if (c < Q8_TILE_RAW / 16 && r < nrow) v = *(const unsigned short *) (tile_row_ptr(t0 + r) + (off - r * Q8_ROW));
+                        h[e] = v;
+                    }
+                    u32x4 v;
+                    v.x = h[0] | ((unsigned) h[1] << 16); v.y = h[2] | ((unsigned) h[3] << 16);
+                    v.z = h[4] | ((unsigned) h[5] << 16); v.w = h[6] | ((unsigned) h[7] << 16);
+                    pre[j] = v;
+                }
+            }
+        } else {
+            if (p.rows_contig && nrow == TILE_TOK) {
+                const char * base = tile_row_ptr(t0);
+#pragma unroll
+                for (int j = 0; j < N_PRE; j++) pre[j] = *(const u32x4 *) (base + (int64_t) (tid + j * NTHREADS) * 16);
+            } else {
+#pragma unroll
+                for (int j = 0; j < N_PRE; j++) {
+                    const int c   = tid + j * NTHREADS;
+                    const int r   = c / (ROW_BYTES / 16);
+                    const int col = c - r * (ROW_BYTES / 16);
+                    u32x4 v = { 0u, 0u, 0u, 0u };
+                    if (r < nrow) v = *(const u32x4 *) (tile_row_ptr(t0 + r) + col * 16);
+                    pre[j] = v;
+                }
+            }
+        }
+    };
+
+    auto commit = [&](int buf) {  // registers -> LDS (for Q8: raw bytes into the staging area)
+        if constexpr (SRC == SRC_Q8) {
+            unsigned char * raw = smem + 2 * TILE_BYTES;
+#pragma unroll
+            for (int j = 0; j < N_PRE; j++) {
+                const int c = tid + j * NTHREADS;
+                if (c < Q8_TILE_RAW / 16) *(LDS_PTR(u32x4)) (raw + c * 16) = pre[j];
+            }
+        } else {
+            unsigned char * tile = smem + buf * TILE_BYTES;
+#pragma unroll
+            for (int j = 0; j < N_PRE; j++) {
+                const int c   = tid + j * NTHREADS;
+                const int r   = c / (ROW_BYTES / 16);
+                const int col = c - r * (ROW_BYTES / 16);
+                *(LDS_PTR(u32x4)) (tile + r * PITCH + col * 16) = pre[j];
+            }
+        }
+    };
+
+    // Q8_0 only: raw staging area -> f16 tile.  One (row, block) pair per work item: value = q * f32(d), rounded to
+    // f16 (the reference dequantizes to f32, ggml-quants.c:357-373; q*d has <= 19 significant bits, f16 keeps 11).
+    auto dequant = [&](int buf) {
+        if constexpr (SRC == SRC_Q8) {
+            const unsigned char * raw  = smem + 2 * TILE_BYTES;
+            unsigned char *       tile = smem + buf * TILE_BYTES;
+            for (int w = tid; w < TILE_TOK * 18; w += NTHREADS) {
+                const int r  = w / 18;
+                const int bk = w - r * 18;
+                const LDS_PTR(const unsigned short) src = (LDS_PTR(const unsigned short)) (raw + r * Q8_ROW + bk * 34);
+                const float d = f16_bits_to_f32(src[0]);
+                unsigned int o[16];
+#pragma unroll
+                for (int e = 0; e < 16; e++) {
+                    const unsigned int pr = src[1 + e];
+                    const float a = (float) (int) (signed char) (pr & 0xff) * d;
+                    const float c = (float) (int) (signed char) (pr >> 8) * d;
+                    o[e] = pack2<true>(a, c);
+                }
+                LDS_PTR(u32x4) dstp = (LDS_PTR(u32x4)) (tile + r * PITCH + bk * 64);
+                dstp[0] = u32x4{ o[0], o[1], o[2], o[3] };
+                dstp[1] = u32x4{ o[4], o[5], o[6], o[7] };
+                dstp[2] = u32x4{ o[8], o[9], o[10], o[11] };
+                dstp[3] = u32x4{ o[12], o[13], o[14], o[15] };
+            }
+        }
+    };
+
+    // per-lane LDS offsets
+    const int k_off = rl * PITCH + g * 16;  // K fragment of S^T = K.Q^T: token rl, d = 16*ks + 8*g..+7
+    // V^T fragment via ds_read_b64_tr_b16: within each 16-lane group, lane s supplies the address of token (s/4),
+    // columns 4*(s%4)..+3 of the group's 16 columns, and receives 4 tokens of column s.
+    const int v_off = (4 * g + ((lane & 15) >> 2)) * PITCH + (((lane >> 4) & 1) * 16 + (lane & 3) * 4) * 2;
+
+    if (n_tiles > 0) {
+        prefetch(0);
+        commit(0);
+        if constexpr (SRC == SRC_Q8) { __syncthreads(); dequant(0); }
+    }
+    __syncthreads();
+
+    for (int it = 0; it < n_tiles; it++) {
+        const int  buf      = it & 1;
+        const bool has_next = it + 1 < n_tiles;
+        if (has_next) prefetch(it + 1);
+
+        const unsigned char * tile = smem + buf * TILE_BYTES;
+        const int             t0   = kv_begin + it * TILE_TOK;
+
+        // ---- S^T = K . Q^T
+        f32x16 s;
+#pragma unroll
+        for (int e = 0; e < 16; e++) s[e] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ks++) {
+            const u32x4 a = *(LDS_PTR(const u32x4)) (tile + k_off + ks * 32);
+            s = mfma32<F16>(a, qreg[ks], s);
+        }
+
+        // ---- scores in log2 units; accumulator element e is token 8*(e/4) + 4*g + e%4 of the tile
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int e = 0; e < 16; e++) {
+            const int ic = t0 + 8 * (e >> 2) + 4 * g + (e & 3);
+            float v = s[e] * scale_eff;
+            if (p.softcap != 0.0f) v = p.softcap * tanhf(v);
+            if (mask_row) {
+                float mv = -INFINITY;
+                if (ic < p.mask_ne0) mv = f16_bits_to_f32(*(const unsigned short *) (mask_row + (int64_t) ic * 2));
+                v += slope * mv;
+            }
+            v *= LOG2E;
+            if (ic >= kv_end) v = -INFINITY;
+            s[e] = v;
+            tmax = fmaxf(tmax, v);
+        }
+        tmax = fmaxf(tmax, xor32(tmax));
+        const float m_new = fmaxf(m_run, tmax);
+        if (__any(m_new > m_run)) {
+            const float alpha = (m_run == -INFINITY) ? 0.f : fast_exp2(m_run - m_new);  // 1 where the max did not move
+#pragma unroll
+            for (int i = 0; i < NDBW; i++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) acc[i][e] *= alpha;
+            l_run *= alpha;
+            m_run = m_new;
+        }
+        const float m_use = (m_run == -INFINITY) ? 0.f : m_run;
+        float lsum = 0.f;
+#pragma unroll
+        for (int e = 0; e < 16; e++) {
+            const float pe = fast_exp2(s[e] - m_use);
+            s[e] = pe;
+            lsum += pe;
+        }
+        l_run += lsum;
+
+        // ---- P^T as MFMA B operand: k-step kk uses accumulator elements 8*kk .. 8*kk+7
+        u32x4 p_hi[2], p_lo[2];
+#pragma unroll
+        for (int kk = 0; kk < 2; kk++) {
+            u32x4 h;
+            h.x = pack2<F16>(s[8 * kk + 0], s[8 * kk + 1]); h.y = pack2<F16>(s[8 * kk + 2], s[8 * kk + 3]);
+            h.z = pack2<F16>(s[8 * kk + 4], s[8 * kk + 5]); h.w = pack2<F16>(s[8 * kk + 6], s[8 * kk + 7]);
+            p_hi[kk] = h;
+            if constexpr (SPLIT) {
+                float r[8];
+#pragma unroll
+                for (int e = 0; e < 8; e++) r[e] = s[8 * kk + e] - round_trip<F16>(s[8 * kk + e]);
+                u32x4 l;
+                l.x = pack2<F16>(r[0], r[1]); l.y = pack2<F16>(r[2], r[3]);
+                l.z = pack2<F16>(r[4], r[5]); l.w = pack2<F16>(r[6], r[7]);
+                p_lo[kk] = l;
+            }
+        }
+
+        // ---- O^T += V^T . P^T ; V^T fragments straight from the row-major tile via the transposing LDS read
+#pragma unroll
+        for (int i = 0; i < NDBW; i++) {
+            const int dcol = p.d_off + (wd * NDBW + i) * 32;  // first column of this 32-wide block
+#pragma unroll
+            for (int kk = 0; kk < 2; kk++) {
+                const unsigned char * vp = tile + v_off + (16 * kk) * PITCH + dcol * 2;
+                const s16x4 t0v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4)) (vp));
+                const s16x4 t1v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4)) (vp + 8 * PITCH));
+                const u32x2 a0 = bitcast<u32x2>(t0v), a1 = bitcast<u32x2>(t1v);
+                const u32x4 a  = { a0.x, a0.y, a1.x, a1.y };
+                acc[i] = mfma32<F16>(a, p_hi[kk], acc[i]);
+                if constexpr (SPLIT) acc[i] = mfma32<F16>(a, p_lo[kk], acc[i]);
+            }
+        }
+
+        if (has_next) {
+            commit(buf ^ 1);
+            if constexpr (SRC == SRC_Q8) { __syncthreads(); dequant(buf ^ 1); }
+        }
+        __syncthreads();
+    }
+
+    // ---- epilogue
+    const float l_tot = l_run + xor32(l_run);
+    if (!row_valid) return;
+    const int64_t orow = (int64_t) b * p.n_rows + row;
+    if (p.n_splits == 1) {
+        const float inv = 1.0f / l_tot;  // l == 0 (every key masked, or an empty sequence) gives NaN like the reference
+        float * o = p.dst + orow * p.dst_stride + p.d_off;
+#pragma unroll
+        for (int i = 0; i < NDBW; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                f32x4 v = { acc[i][4 * j] * inv, acc[i][4 * j + 1] * inv, acc[i][4 * j + 2] * inv, acc[i][4 * j + 3] * inv };
+                *(f32x4 *) (o + (wd * NDBW + i) * 32 + 8 * j + 4 * g) = v;
+            }
+    } else {
+        const int64_t prow = ((int64_t) b * p.n_splits + split) * p.n_rows + row;
+        float * o = p.part_o + prow * p.dv_total + p.d_off;
+#pragma unroll
+        for (int i = 0; i < NDBW; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                f32x4 v = { acc[i][4 * j], acc[i][4 * j + 1], acc[i][4 * j + 2], acc[i][4 * j + 3] };
+                *(f32x4 *) (o + (wd * NDBW + i) * 32 + 8 * j + 4 * g) = v;
+            }
+        if (wd == 0 && g == 0 && p.d_off == 0) {
+            p.part_ml[prow * 2]     = m_run;
+            p.part_ml[prow * 2 + 1] = l_tot;
+        }
+    }
+}
+
+// Log-sum-exp merge of the split-K partials: out = sum_c O_c 2^(m_c - M) / sum_c l_c 2^(m_c - M).
+// grid = (n_rows, n_seq), block = dv_total / 4 threads (one float4 column group each).
+__global__ void mla_attn_combine_kernel(const KParams p) {
+    const int row = blockIdx.x, b = blockIdx.y;
+    const int seq_len = p.block_table ? min(p.seq_lens[b], (int) p.bt_stride * MLA_PAGE_TOKENS) : (int) p.n_kv;
+    int nvalid = (seq_len + p.split_tokens - 1) / p.split_tokens;
+    nvalid = min(nvalid, p.n_splits);
+    const int d4 = threadIdx.x;
+    float M = -INFINITY;
+    for (int c = 0; c < nvalid; c++) M = fmaxf(M, p.part_ml[(((int64_t) b * p.n_splits + c) * p.n_rows + row) * 2]);
+    const float Mu = (M == -INFINITY) ? 0.f : M;
+    float L = 0.f;
+    f32x4 o = { 0.f, 0.f, 0.f, 0.f };
+    for (int c = 0; c < nvalid; c++) {
+        const int64_t prow = ((int64_t) b * p.n_splits + c) * p.n_rows + row;
+        const float mc = p.part_ml[prow * 2];
+        if (mc == -INFINITY) continue;  // that split saw only masked keys
+        const float w = fast_exp2(mc - Mu);
+        L += p.part_ml[prow * 2 + 1] * w;
+        const f32x4 v = *(const f32x4 *) (p.part_o + prow * p.dv_total + d4 * 4);
+        o.x += v.x * w; o.y += v.y * w; o.z += v.z * w; o.w += v.w * w;
+    }
+    const float inv = 1.0f / L;
+    f32x4 r = { o.x * inv, o.y * inv, o.z * inv, o.w * inv };
+    *(f32x4 *) (p.dst + ((int64_t) b * p.n_rows + row) * p.dst_stride + d4 * 4) = r;
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// Strict replay of ggml-cpu's f16 accumulator for F16 KV (ggml-cpu.c:12066-12080 with the x86 F16 vector forms
+// :621-659, :718-765: f32 FMA, result rounded to f16 after every scale and every multiply-add, keys in order).
+// Two small kernels: scores (f32 dot of f16-rounded Q with f16 K), then one wave per row walking the keys.
+// ---------------------------------------------------------------------------------------------------------------
+__global__ void mla_f16_scores_kernel(const KParams p, float * scores) {  // grid (ceil(n_kv/4), n_rows, n_seq), block 256
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int ic = blockIdx.x * 4 + wave, row = blockIdx.y, b = blockIdx.z;
+    if (ic >= p.n_kv) return;
+    const int tq = row / p.n_head, head = row - tq * p.n_head;
+    const float * qrow = (const float *) (p.q + (int64_t) tq * p.q_nb1 + (int64_t) head * p.q_nb2 + (int64_t) b * p.q_nb3);
+    const unsigned short * krow = (const unsigned short *) (p.kv + (int64_t) ic * p.kv_nb1 + (int64_t) b * p.kv_nb3);
+    float sum = 0.f;
+    for (int d = lane; d < DK; d += 64) sum += (float) (_Float16) qrow[d] * f16_bits_to_f32(krow[d]);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
+    if (lane == 0) scores[((int64_t) b * p.n_rows + row) * p.n_kv + ic] = sum;
+}
+
+__global__ void mla_f16_strict_kernel(const KParams p, const float * scores) {  // grid (n_rows, n_seq), block 64
+    const int lane = threadIdx.x, row = blockIdx.x, b = blockIdx.y;
+    const int tq = row / p.n_head, head = row - tq * p.n_head;
+    float slope = 1.0f;
+    if (p.max_bias > 0.0f) slope = head < p.n_head_log2 ? powf(p.m0, (float) (head + 1)) : powf(p.m1, (float) (2 * (head - p.n_head_log2) + 1));
+    const float scale_eff = p.softcap != 0.0f ? p.scale / p.softcap : p.scale;
+    const char * mask_row = p.mask ? p.mask + (int64_t) tq * p.mask_nb1 : nullptr;
+    const float * srow = scores + ((int64_t) b * p.n_rows + row) * p.n_kv;
+    float acc[9];
+#pragma unroll
+    for (int j = 0; j < 9; j++) acc[j] = 0.f;
+    float S = 0.f, M = -INFINITY;
+    for (int ic = 0; ic < (int) p.n_kv; ic++) {
+        const float mv = mask_row ? slope * f16_bits_to_f32(*(const unsigned short *) (mask_row + (int64_t) ic * 2)) : 0.0f;
+        if (mv == -INFINITY) continue;
+        float s = srow[ic] * scale_eff;
+        if (p.softcap != 0.0f) s = p.softcap * tanhf(s);
+        s += mv;
+        const float Mold = M;
+        float ms = 1.0f, vs = 1.0f;
+        const unsigned short * vrow = (const unsigned short *) (p.kv + (int64_t) ic * p.kv_nb1 + (int64_t) b * p.kv_nb3);
+        if (s > M) {
+            M  = s;
+            ms = expf(Mold - M);
+#pragma unroll
+            for (int j = 0; j < 9; j++) acc[j] = (float) (_Float16) (acc[j] * ms);
+        } else {
+            vs = expf(s - M);
+        }
+#pragma unroll
+        for (int j = 0; j < 9; j++) {
+            const int d = lane + 64 * j;
+            if (d < p.dv_total) acc[j] = (float) (_Float16) fmaf(f16_bits_to_f32(vrow[d]), vs, acc[j]);
+        }
+        S = S * ms + vs;
+    }
+    const float S_inv = 1.0f / S;
+    float * o = p.dst + ((int64_t) b * p.n_rows + row) * p.dst_stride;
+#pragma unroll
+    for (int j = 0; j < 9; j++) {
+        const int d = lane + 64 * j;
+        if (d < p.dv_total) o[d] = acc[j] * S_inv;
+    }
+}
+
+__global__ void __launch_bounds__(256) mla_hbm_copy_kernel(const u32x4 * __restrict__ src, u32x4 * __restrict__ dst, size_t n16) {
+    size_t       i      = (size_t) blockIdx.x * 256 + threadIdx.x;
+    const size_t stride = (size_t) gridDim.x * 256;
+    for (; i < n16; i += stride) dst[i] = src[i];
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------------------------------------------
+
+struct Plan {
+    int    variant;  // 0 tiled, 1 strict f16
+    int    wm, wd, rblk, n_row_blocks;
+    int    n_splits, split_tokens;
+    int    n_passes, ndb;
+    size_t lds_bytes;
+    size_t ws_part_o, ws_part_ml, ws_scores;
+};
+
+int validate(const mla_attn_args * a) {
+    if (!a) return MLA_ERR_NULL;
+    if (!a->q || !a->kv || !a->dst) return MLA_ERR_NULL;
+    if (a->n_seq < 1 || a->n_head < 1 || a->n_tok < 1) return MLA_ERR_BAD_SHAPE;
+    if (a->dk != DK || (a->dv != 512 && a->dv != 576)) return MLA_ERR_BAD_SHAPE;
+    if (a->q_type != MLA_TYPE_F32) return MLA_ERR_BAD_TYPE;
+    if (a->kv_type != MLA_TYPE_BF16 && a->kv_type != MLA_TYPE_F16 && a->kv_type != MLA_TYPE_Q8_0) return MLA_ERR_BAD_TYPE;
+    if ((a->flags & MLA_FLAG_F16_ACC_STRICT) && (a->kv_type != MLA_TYPE_F16 || a->block_table)) return MLA_ERR_UNSUPPORTED;
+    if (a->n_kv < 0 || a->n_kv > 0x7fffffff) return MLA_ERR_BAD_SHAPE;
+    if ((int64_t) a->n_tok * a->n_head > 0x7fffffff) return MLA_ERR_BAD_SHAPE;
+    if (((uintptr_t) a->q & 15) || (a->q_nb1 & 15) || (a->q_nb2 & 15) || (a->q_nb3 & 15)) return MLA_ERR_BAD_ALIGNMENT;
+    if (((uintptr_t) a->dst & 15) || (a->dst_nb1 & 15) || a->dst_nb1 < (int64_t) a->dv * 4) return MLA_ERR_BAD_ALIGNMENT;
+    if (a->kv_type == MLA_TYPE_Q8_0) {
+        if (((uintptr_t) a->kv & 1) || (a->kv_nb1 & 1) || (a->kv_nb3 & 1) || a->kv_nb1 < Q8_ROW) return MLA_ERR_BAD_ALIGNMENT;
+    } else {
+        if (((uintptr_t) a->kv & 15) || (a->kv_nb1 & 15) || (a->kv_nb3 & 15) || a->kv_nb1 < ROW_BYTES) return MLA_ERR_BAD_ALIGNMENT;
+    }
+    if (a->mask) {
+        if ((a->mask_nb1 & 1) || ((uintptr_t) a->mask & 1) || a->mask_ne0 < 0) return MLA_ERR_BAD_ALIGNMENT;
+    }
+    if (a->max_bias > 0.0f && !a->mask) return MLA_ERR_UNSUPPORTED;  // ggml.c:4005-4007
+    if (a->block_table) {
+        if (!a->seq_lens || a->bt_stride < 1) return MLA_ERR_NULL;
+        if (a->n_kv < MLA_PAGE_TOKENS || a->n_kv % MLA_PAGE_TOKENS) return MLA_ERR_BAD_SHAPE;  // pool of whole pages
+        if (a->bt_stride > (1 << 23)) return MLA_ERR_BAD_SHAPE;
+    }
+    if (a->n_splits < 0) return MLA_ERR_BAD_SHAPE;
+    return 0;
+}
+
+int make_plan(const mla_attn_args * a, Plan * pl) {
+    const int rc = validate(a);
+    if (rc) return rc;
+    const int64_t n_rows  = (int64_t) a->n_tok * a->n_head;
+    const int64_t max_len = a->block_table ? a->bt_stride * MLA_PAGE_TOKENS : a->n_kv;
+    *pl = Plan{};
+    if (a->flags & MLA_FLAG_F16_ACC_STRICT) {
+        pl->variant   = 1;
+        pl->n_splits  = 1;
+        pl->n_passes  = 1;
+        pl->ws_scores = (size_t) a->n_seq * n_rows * (size_t) (a->n_kv > 0 ? a->n_kv : 1) * sizeof(float);
+        pl->split_tokens = (int) max_len;
+        return 0;
+    }
+    if (a->dv == 576) { pl->n_passes = 2; pl->ndb = 9; pl->wm = 4; pl->wd = 1; }
+    else {
+        pl->n_passes = 1; pl->ndb = 16;
+        if (n_rows > 64)      { pl->wm = 4; pl->wd = 1; }
+        else if (n_rows > 32) { pl->wm = 2; pl->wd = 2; }
+        else                  { pl->wm = 1; pl->wd = 4; }
+    }
+    pl->rblk         = 32 * pl->wm;
+    pl->n_row_blocks = (int) ((n_rows + pl->rblk - 1) / pl->rblk);
+    // split the KV range so that about two workgroups per CU exist (256 CUs), in units of whole pages
+    int64_t n_pages = (max_len + MLA_PAGE_TOKENS - 1) / MLA_PAGE_TOKENS;
+    if (n_pages < 1) n_pages = 1;
+    int64_t splits = a->n_splits;
+    if (splits == 0) {
+        const int64_t wgs = (int64_t) a->n_seq * pl->n_row_blocks;
+        splits = (256 + wgs - 1) / wgs;
+        if (pl->wd > 1) splits *= 2;  // small-row shapes leave room for two workgroups per CU
+    }
+    if (splits > n_pages) splits = n_pages;
+    if (splits < 1) splits = 1;
+    const int64_t pages_per_split = (n_pages + splits - 1) / splits;
+    pl->split_tokens = (int) (pages_per_split * MLA_PAGE_TOKENS);
+    pl->n_splits     = (int) ((n_pages + pages_per_split - 1) / pages_per_split);
+    pl->lds_bytes    = 2 * TILE_BYTES + (a->kv_type == MLA_TYPE_Q8_0 ? Q8_TILE_RAW : 0);
+    if (pl->n_splits > 1) {
+        pl->ws_part_o  = (size_t) a->n_seq * pl->n_splits * n_rows * a->dv * sizeof(float);
+        pl->ws_part_ml = (size_t) a->n_seq * pl->n_splits * n_rows * 2 * sizeof(float);
+    }
+    return 0;
+}
+
+size_t align256(size_t x) { return (x + 255) & ~(size_t) 255; }
+size_t plan_ws(const Plan & pl) { return align256(pl.ws_part_o) + align256(pl.ws_part_ml) + align256(pl.ws_scores); }
+
+template <int SRC, int NDB, int WM, int WD>
+hipError_t launch_tile(const KParams & kp, dim3 grid, size_t lds, hipStream_t st) {
+    auto kern = mla_attn_tile_kernel<SRC, NDB, WM, WD>;
+    static bool attr_done = false;  // raising the dynamic LDS limit is a per-function, per-process setting
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute((const void *) kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int) (160 * 1024));
+        if (e != hipSuccess) return e;
+        attr_done = true;
+    }
+    hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), lds, st, kp);
+    return hipGetLastError();
+}
+
+template <int SRC>
+hipError_t launch_tile_src(const Plan & pl, const KParams & kp, dim3 grid, hipStream_t st) {
+    if (pl.ndb == 9) return launch_tile<SRC, 9, 4, 1>(kp, grid, pl.lds_bytes, st);
+    if (pl.wm == 4) return launch_tile<SRC, 16, 4, 1>(kp, grid, pl.lds_bytes, st);
+    if (pl.wm == 2) return launch_tile<SRC, 16, 2, 2>(kp, grid, pl.lds_bytes, st);
+    return launch_tile<SRC, 16, 1, 4>(kp, grid, pl.lds_bytes, st);
+}
+
+}  // namespace
+
+extern "C" {
+
+const char * mla_attn_target_arch(void) { return "gfx950 (mla_attn tiled MFMA kernels, " __DATE__ ")"; }
+
+size_t mla_attn_workspace_size(const mla_attn_args * args) {
+    Plan pl;
+    if (make_plan(args, &pl)) return 0;
+    return plan_ws(pl);
+}
+
+int mla_attn_plan(const mla_attn_args * args, mla_attn_plan_info * out) {
+    Plan pl;
+    const int rc = make_plan(args, &pl);
+    if (rc) return rc;
+    if (!out) return MLA_ERR_NULL;
+    out->variant      = pl.variant;
+    out->rows_per_wg  = pl.rblk;
+    out->n_row_blocks = pl.n_row_blocks;
+    out->n_splits     = pl.n_splits;
+    out->split_tokens = pl.split_tokens;
+    out->n_passes     = pl.n_passes;
+    out->lds_bytes    = (int64_t) pl.lds_bytes;
+    return 0;
+}
+
+int mla_attn_launch(const mla_attn_args * a, void * stream) {
+    Plan pl;
+    const int rc = make_plan(a, &pl);
+    if (rc) return rc;
+    const size_t need = plan_ws(pl);
+    if (need > 0 && (!a->workspace || a->workspace_size < need || ((uintptr_t) a->workspace & 255))) return MLA_ERR_WORKSPACE;
+    hipStream_t st = (hipStream_t) stream;
+
+    KParams kp{};
+    kp.q = (const char *) a->q; kp.q_nb1 = a->q_nb1; kp.q_nb2 = a->q_nb2; kp.q_nb3 = a->q_nb3;
+    kp.kv = (const char *) a->kv; kp.kv_nb1 = a->kv_nb1; kp.kv_nb3 = a->kv_nb3; kp.n_kv = a->n_kv;
+    kp.mask = (const char *) a->mask; kp.mask_nb1 = a->mask_nb1; kp.mask_ne0 = a->mask_ne0;
+    kp.block_table = a->block_table; kp.bt_stride = a->bt_stride; kp.seq_lens = a->seq_lens;
+    kp.dst = a->dst; kp.dst_stride = a->dst_nb1 / 4;
+    kp.n_head = a->n_head; kp.n_tok = a->n_tok; kp.n_rows = a->n_tok * a->n_head;
+    kp.n_splits = pl.n_splits; kp.split_tokens = pl.split_tokens;
+    kp.dv_total = a->dv;
+    kp.scale = a->scale; kp.softcap = a->logit_softcap; kp.max_bias = a->max_bias;
+    kp.n_head_log2 = 1 << (int) floor(log2((double) a->n_head));
+    kp.m0 = powf(2.0f, -(a->max_bias) / kp.n_head_log2);
+    kp.m1 = powf(2.0f, -(a->max_bias / 2.0f) / kp.n_head_log2);
+    kp.n_pool_pages = (int) (a->n_kv / MLA_PAGE_TOKENS);
+    kp.rows_contig = a->kv_nb1 == (a->kv_type == MLA_TYPE_Q8_0 ? Q8_ROW : ROW_BYTES) && (((uintptr_t) a->kv & 15) == 0) &&
+                     (a->block_table || (a->kv_nb3 & 15) == 0);
+    char * ws = (char *) a->workspace;
+    kp.part_o  = (float *) ws;
+    kp.part_ml = (float *) (ws + align256(pl.ws_part_o));
+    float * scores = (float *) (ws + align256(pl.ws_part_o) + align256(pl.ws_part_ml));
+
+    if (pl.variant == 1) {
+        if (a->n_kv > 0) {
+            dim3 g1((unsigned) ((a->n_kv + 3) / 4), (unsigned) kp.n_rows, (unsigned) a->n_seq);
+            hipLaunchKernelGGL(mla_f16_scores_kernel, g1, dim3(256), 0, st, kp, scores);
+            hipError_t e = hipGetLastError();
+            if (e != hipSuccess) return (int) e;
+        }
+        dim3 g2((unsigned) kp.n_rows, (unsigned) a->n_seq);
+        hipLaunchKernelGGL(mla_f16_strict_kernel, g2, dim3(64), 0, st, kp, (const float *) scores);
+        return (int) hipGetLastError();
+    }
+
+    dim3 grid((unsigned) pl.n_splits, (unsigned) pl.n_row_blocks, (unsigned) a->n_seq);
+    for (int pass = 0; pass < pl.n_passes; pass++) {
+        kp.d_off = pass * pl.ndb * 32;
+        hipError_t e;
+        switch (a->kv_type) {
+            case MLA_TYPE_BF16: e = launch_tile_src<SRC_BF16>(pl, kp, grid, st); break;
+            case MLA_TYPE_F16:  e = launch_tile_src<SRC_F16>(pl, kp, grid, st); break;
+            default:            e = launch_tile_src<SRC_Q8>(pl, kp, grid, st); break;
+        }
+        if (e != hipSuccess) return (int) e;
+    }
+    if (pl.n_splits > 1) {
+        dim3 g((unsigned) kp.n_rows, (unsigned) a->n_seq);
+        hipLaunchKernelGGL(mla_attn_combine_kernel, g, dim3(a->dv / 4), 0, st, kp);
+        return (int) hipGetLastError();
+    }
+    return 0;
+}
+
+int mla_hbm_copy_launch(const void * src, void * dst, size_t n_bytes, void * stream) {
+    if (!src || !dst) return MLA_ERR_NULL;
+    if ((n_bytes & 15) || ((uintptr_t) src & 15) || ((uintptr_t) dst & 15)) return MLA_ERR_BAD_ALIGNMENT;
+    if (n_bytes == 0) return 0;
+    hipLaunchKernelGGL(mla_hbm_copy_kernel, dim3(2048), dim3(256), 0, (hipStream_t) stream, (const u32x4 *) src, (u32x4 *) dst, n_bytes / 16);
+    return (int) hipGetLastError();
+}
+
+}  // extern "C"

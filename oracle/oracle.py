@@ -1,0 +1,261 @@
+"""ctypes front end of the CPU oracle (oracle/mla_oracle.c) and, when built, of the reference's own compiled
+ggml (oracle/_ref/).  TEST INFRASTRUCTURE ONLY -- see oracle/__init__.py.
+
+Array conventions (numpy, C order; ggml lists dimensions the other way round):
+  q     float32 [n_seq, n_head, n_tok, 576]          ggml ne = {576, n_tok, n_head, n_seq}
+  k     f16/bf16: uint16 [n_seq, n_kv, 576];  q8_0: uint8 [n_seq, n_kv, 612]
+  mask  uint16 (f16 bits) [n_tok, n_kv] or None
+  out   float32 [n_seq, n_tok, n_head, dv]
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+TYPE_F32, TYPE_F16, TYPE_Q8_0, TYPE_BF16 = 0, 1, 8, 30
+Q8_ROW = 612
+
+
+class _Tensor(C.Structure):
+    _fields_ = [("type", C.c_int32), ("_pad", C.c_int32), ("ne", C.c_int64 * 4), ("nb", C.c_int64 * 4), ("data", C.c_void_p)]
+
+
+def build(force=False):
+    """Compile liboracle.so (and oracle/_ref when the reference tree is present) with the Makefile beside this file."""
+    if force or not os.path.exists(os.path.join(HERE, "liboracle.so")) or (
+            os.path.isdir("/root/reference/ggml") and not os.path.exists(os.path.join(HERE, "_ref", "libref_driver.so"))):
+        subprocess.run(["make", "-C", HERE, "-j8"], check=True, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)
+
+
+_lib = None
+_ref = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        path = os.path.join(HERE, "liboracle.so")
+        if not os.path.exists(path):
+            build()
+        _lib = C.CDLL(path)
+        _lib.mla_oracle_flash_attn_ext.restype = C.c_int
+        _lib.mla_oracle_flash_attn_ext.argtypes = [C.POINTER(_Tensor)] * 4 + [C.c_void_p, C.c_int64, C.c_float, C.c_float, C.c_float, C.c_int, C.c_int]
+        _lib.mla_oracle_flash_attn_ext_f64.restype = C.c_int
+        _lib.mla_oracle_flash_attn_ext_f64.argtypes = [C.POINTER(_Tensor)] * 4 + [C.c_void_p, C.c_int64, C.c_float, C.c_int, C.c_int]
+        for name in ("mla_oracle_f32_to_bf16_row", "mla_oracle_f32_to_f16_row", "mla_oracle_bf16_to_f32_row", "mla_oracle_f16_to_f32_row"):
+            getattr(_lib, name).argtypes = [C.c_void_p, C.c_void_p, C.c_int64]
+            getattr(_lib, name).restype = None
+        _lib.mla_oracle_quantize_row_q8_0.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int]
+        _lib.mla_oracle_quantize_row_q8_0.restype = None
+        _lib.mla_oracle_dequantize_row_q8_0.argtypes = [C.c_void_p, C.c_void_p, C.c_int64]
+        _lib.mla_oracle_dequantize_row_q8_0.restype = None
+    return _lib
+
+
+def ref_available():
+    return os.path.exists(os.path.join(HERE, "_ref", "libref_driver.so"))
+
+
+def ref():
+    """The reference's compiled ggml behind oracle/ref_driver.c; None when oracle/_ref is not built."""
+    global _ref
+    if _ref is None and ref_available():
+        C.CDLL(os.path.join(HERE, "_ref", "libggml_ref.so"), mode=C.RTLD_GLOBAL)
+        _ref = C.CDLL(os.path.join(HERE, "_ref", "libref_driver.so"))
+        _ref.ref_flash_attn_ext.restype = C.c_int
+        _ref.ref_flash_attn_ext.argtypes = [C.c_int] + [C.c_int64] * 5 + [C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, C.c_float, C.c_float, C.c_void_p, C.c_int]
+        _ref.ref_backend_flash_attn_ext.restype = C.c_int
+        _ref.ref_backend_flash_attn_ext.argtypes = [C.c_char_p, C.c_int] + [C.c_int64] * 6 + [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64,
+                                                    C.c_void_p, C.c_int64, C.c_void_p, C.c_float, C.c_float, C.c_float, C.c_int,
+                                                    C.c_void_p, C.c_char_p, C.c_size_t]
+        for name in ("ref_quantize_q8_0_ref", "ref_quantize_q8_0_cpu", "ref_dequantize_q8_0", "ref_f32_to_f16_row", "ref_f32_to_bf16_row", "ref_f16_to_f32_row"):
+            getattr(_ref, name).argtypes = [C.c_void_p, C.c_void_p, C.c_int64]
+            getattr(_ref, name).restype = None
+        _ref.ref_abi_table.restype = C.c_int
+        _ref.ref_abi_table.argtypes = [C.c_int, C.POINTER(C.c_char_p), C.POINTER(C.c_int64)]
+    return _ref
+
+
+# ------------------------------------------------------------------ conversions
+
+def _conv(name, x, in_dtype, out_dtype):
+    x = np.ascontiguousarray(x, dtype=in_dtype)
+    y = np.empty(x.shape, dtype=out_dtype)
+    getattr(lib(), name)(x.ctypes.data, y.ctypes.data, x.size)
+    return y
+
+
+def f32_to_bf16(x): return _conv("mla_oracle_f32_to_bf16_row", x, np.float32, np.uint16)
+def f32_to_f16(x): return _conv("mla_oracle_f32_to_f16_row", x, np.float32, np.uint16)
+def bf16_to_f32(x): return _conv("mla_oracle_bf16_to_f32_row", x, np.uint16, np.float32)
+def f16_to_f32(x): return _conv("mla_oracle_f16_to_f32_row", x, np.uint16, np.float32)
+
+
+def quantize_q8_0(x, mode=0):
+    """x float32 [..., n] (n % 32 == 0) -> uint8 [..., n/32*34].  mode 0: reference quantizer, 1: x86 CPU-backend one."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    n = x.shape[-1]
+    assert n % 32 == 0
+    y = np.empty(x.shape[:-1] + (n // 32 * 34,), dtype=np.uint8)
+    lib().mla_oracle_quantize_row_q8_0(x.ctypes.data, y.ctypes.data, x.size, mode)
+    return y
+
+
+def dequantize_q8_0(y):
+    y = np.ascontiguousarray(y, dtype=np.uint8)
+    n = y.shape[-1] // 34 * 32
+    x = np.empty(y.shape[:-1] + (n,), dtype=np.float32)
+    lib().mla_oracle_dequantize_row_q8_0(y.ctypes.data, x.ctypes.data, x.size)
+    return x
+
+
+def make_q8_0(qs, d_f16_bits):
+    """Assemble Q8_0 rows from int8 quants [..., n] and f16 scale bits [..., n/32] -> uint8 [..., n/32*34]."""
+    qs = np.asarray(qs, dtype=np.int8)
+    d = np.asarray(d_f16_bits, dtype=np.uint16)
+    nb = qs.shape[-1] // 32
+    out = np.empty(qs.shape[:-1] + (nb, 34), dtype=np.uint8)
+    out[..., 0:2] = d.reshape(d.shape + (1,)).view(np.uint8).reshape(d.shape + (2,))
+    out[..., 2:] = qs.reshape(qs.shape[:-1] + (nb, 32)).view(np.uint8)
+    return out.reshape(qs.shape[:-1] + (nb * 34,))
+
+
+def to_f32(k, k_type):
+    if k_type == TYPE_BF16: return bf16_to_f32(k)
+    if k_type == TYPE_F16: return f16_to_f32(k)
+    if k_type == TYPE_Q8_0: return dequantize_q8_0(k)
+    raise ValueError(k_type)
+
+
+# ------------------------------------------------------------------ the op
+
+def _desc(arr, type_id, ne, nb):
+    t = _Tensor()
+    t.type = type_id
+    t.ne = (C.c_int64 * 4)(*ne)
+    t.nb = (C.c_int64 * 4)(*nb)
+    t.data = arr.ctypes.data
+    return t
+
+
+def _row_bytes(k_type, n=576):
+    return n * 2 if k_type in (TYPE_F16, TYPE_BF16) else n // 32 * 34
+
+
+def _prep(q, k, k_type, dv, mask):
+    q = np.ascontiguousarray(q, dtype=np.float32)
+    n3, H, N, DK = q.shape
+    k = np.ascontiguousarray(k)
+    n3k, n_kv = k.shape[0], k.shape[1]
+    rb = _row_bytes(k_type, DK)
+    assert k.dtype.itemsize * k.shape[2] == rb, (k.shape, k.dtype, rb)
+    tq = _desc(q, TYPE_F32, (DK, N, H, n3), (4, DK * 4, DK * 4 * N, DK * 4 * N * H))
+    tk = _desc(k, k_type, (DK, n_kv, 1, n3k), (2 if k_type != TYPE_Q8_0 else 34, rb, rb * n_kv, rb * n_kv))
+    tv = _desc(k, k_type, (dv, n_kv, 1, n3k), (2 if k_type != TYPE_Q8_0 else 34, rb, rb * n_kv, rb * n_kv))
+    tm = None
+    if mask is not None:
+        mask = np.ascontiguousarray(mask, dtype=np.uint16)
+        assert mask.shape[0] >= N and mask.shape[1] >= n_kv
+        tm = _desc(mask, TYPE_F16, (mask.shape[1], mask.shape[0], 1, 1), (2, mask.shape[1] * 2, 0, 0))
+    return q, k, mask, tq, tk, tv, tm, (n3, H, N, DK)
+
+
+def flash_attn_ext(q, k, k_type, dv=512, mask=None, scale=1.0, max_bias=0.0, softcap=0.0, q8_mode=1, n_threads=None):
+    """The oracle: ggml-cpu's flash_attn_ext restated (oracle/mla_oracle.c).  Returns float32 [n_seq, n_tok, n_head, dv]."""
+    q, k, mask, tq, tk, tv, tm, (n3, H, N, DK) = _prep(q, k, k_type, dv, mask)
+    out = np.empty((n3, N, H, dv), dtype=np.float32)
+    nt = n_threads or min(os.cpu_count() or 1, 16)
+    rc = lib().mla_oracle_flash_attn_ext(C.byref(tq), C.byref(tk), C.byref(tv), C.byref(tm) if tm is not None else None,
+                                         out.ctypes.data, dv, scale, max_bias, softcap, q8_mode, nt)
+    if rc != 0:
+        raise RuntimeError("mla_oracle_flash_attn_ext failed: %d" % rc)
+    return out
+
+
+def flash_attn_ext_f64(q, k, k_type, dv=512, mask=None, scale=1.0, q8_mode=1, n_threads=None):
+    """softmax(scale q.k + mask).v evaluated in float64 on the same rounded inputs (no ALiBi / softcap)."""
+    q, k, mask, tq, tk, tv, tm, (n3, H, N, DK) = _prep(q, k, k_type, dv, mask)
+    out = np.empty((n3, N, H, dv), dtype=np.float32)
+    nt = n_threads or min(os.cpu_count() or 1, 16)
+    rc = lib().mla_oracle_flash_attn_ext_f64(C.byref(tq), C.byref(tk), C.byref(tv), C.byref(tm) if tm is not None else None,
+                                             out.ctypes.data, dv, scale, q8_mode, nt)
+    if rc != 0:
+        raise RuntimeError("mla_oracle_flash_attn_ext_f64 failed: %d" % rc)
+    return out
+
+
+def ref_flash_attn_ext(q, k, k_type, mask=None, scale=1.0, max_bias=0.0, softcap=0.0, n_threads=None):
+    """The reference's own compiled ggml-cpu (V := K, all 576 output columns).  float32 [n_seq, n_tok, n_head, 576]."""
+    r = ref()
+    if r is None:
+        raise RuntimeError("oracle/_ref is not built")
+    q = np.ascontiguousarray(q, dtype=np.float32)
+    n3, H, N, DK = q.shape
+    k = np.ascontiguousarray(k)
+    assert k.shape[0] == n3
+    n_kv = k.shape[1]
+    if mask is not None:
+        mask = np.ascontiguousarray(mask, dtype=np.uint16)
+        assert mask.shape == (N, n_kv)
+    out = np.empty((n3, N, H, DK), dtype=np.float32)
+    nt = n_threads or min(os.cpu_count() or 1, 16)
+    rc = r.ref_flash_attn_ext(k_type, DK, N, H, n3, n_kv, q.ctypes.data, k.ctypes.data, mask.ctypes.data if mask is not None else None,
+                              scale, max_bias, softcap, out.ctypes.data, nt)
+    if rc != 0:
+        raise RuntimeError("ref_flash_attn_ext failed: %d" % rc)
+    return out
+
+
+def ref_backend_flash_attn_ext(so_path, q, k, k_type, dv=576, mask=None, block_table=None, seq_lens=None, scale=1.0,
+                               max_bias=0.0, softcap=0.0, use_sched=False):
+    """Run the node on a backend .so loaded by the reference's ggml_backend_load, through its ggml-backend API.
+    k: [n_seq, n_kv, row] or, with a block table, the pool [n_rows, row].  Returns (float32 [n_seq, n_tok, n_head, 576], info)."""
+    r = ref()
+    if r is None:
+        raise RuntimeError("oracle/_ref is not built")
+    q = np.ascontiguousarray(q, dtype=np.float32)
+    n3, H, N, DK = q.shape
+    k = np.ascontiguousarray(k)
+    n_kv = k.shape[-2]
+    mask_ne0 = 0
+    if mask is not None:
+        mask = np.ascontiguousarray(mask, dtype=np.uint16)
+        mask_ne0 = mask.shape[1]
+    max_blocks = 0
+    if block_table is not None:
+        block_table = np.ascontiguousarray(block_table, dtype=np.int32)
+        seq_lens = np.ascontiguousarray(seq_lens, dtype=np.int32)
+        max_blocks = block_table.shape[1]
+    out = np.full((n3, N, H, DK), np.nan, dtype=np.float32)
+    info = C.create_string_buffer(512)
+    rc = r.ref_backend_flash_attn_ext(so_path.encode(), k_type, DK, dv, N, H, n3, n_kv, q.ctypes.data, k.ctypes.data,
+                                      mask.ctypes.data if mask is not None else None, mask_ne0,
+                                      block_table.ctypes.data if block_table is not None else None, max_blocks,
+                                      seq_lens.ctypes.data if seq_lens is not None else None,
+                                      scale, max_bias, softcap, 1 if use_sched else 0, out.ctypes.data, info, 512)
+    if rc != 0:
+        raise RuntimeError("ref_backend_flash_attn_ext failed: %d (%s)" % (rc, info.value.decode()))
+    return out, info.value.decode()
+
+
+def ref_abi_table():
+    r = ref()
+    name, val = C.c_char_p(), C.c_int64()
+    n = r.ref_abi_table(-1, C.byref(name), C.byref(val))
+    out = {}
+    for i in range(n):
+        r.ref_abi_table(i, C.byref(name), C.byref(val))
+        out[name.value.decode()] = val.value
+    return out
+
+
+# ------------------------------------------------------------------ error metrics used by every parity test
+
+def errors(a, b):
+    """(max-abs error, relative L2 error) of a against b."""
+    a = np.asarray(a, dtype=np.float64)
+    b = np.asarray(b, dtype=np.float64)
+    return float(np.max(np.abs(a - b))), float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-300))

@@ -1,0 +1,259 @@
+/*
+ * Driver around the REFERENCE's own compiled ggml (oracle/_ref/libggml_ref.so).  TEST INFRASTRUCTURE ONLY.
+ *
+ * This file is ours; it includes the reference's public headers at build time (from /root/reference, never
+ * copied) and exports a few plain-C entry points for the Python tests:
+ *   ref_flash_attn_ext            run ggml_flash_attn_ext (ggml/src/ggml.c:3988-4022) on the ggml-cpu backend
+ *   ref_backend_flash_attn_ext    load a backend .so with ggml_backend_load (ggml-backend-reg.cpp:401-403) and
+ *                                 run the same node on it through the reference's ggml-backend API, i.e. the
+ *                                 way the reference's scheduler would drive a drop-in backend
+ *   ref_quantize_q8_0_ref / _cpu  the two Q8_0 quantizers (ggml-quants.c:202-226, ggml-cpu-quants.c:767-900)
+ *   ref_f32_to_f16_row / bf16     the reference's conversions
+ *   ref_abi_table                 sizeof/offsetof/enum facts of the structs a backend must mirror
+ */
+#include <stddef.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "ggml.h"
+#include "ggml-alloc.h"
+#include "ggml-backend.h"
+#include "ggml-cpu.h"
+#include "ggml-backend-impl.h"
+#include "ggml-impl.h"
+#define GGML_COMMON_DECL_C
+#include "ggml-common.h"
+#include "ggml-quants.h"
+
+void quantize_row_q8_0(const float * x, void * y, int64_t k); /* ggml-cpu-quants.c:767 */
+
+static size_t row_bytes(enum ggml_type t, int64_t n) { return ggml_row_size(t, n); }
+
+static struct ggml_tensor * make_mask(struct ggml_context * ctx, int64_t n_kv, int64_t n_tok) {
+    return ggml_new_tensor_2d(ctx, GGML_TYPE_F16, n_kv, GGML_PAD(n_tok, GGML_KQ_MASK_PAD));
+}
+
+/*
+ * q:    f32, contiguous [n3][n_head][n_tok][DK]        (ggml ne = {DK, n_tok, n_head, n3})
+ * k:    k_type rows, contiguous [n3][n_kv][row_bytes]  (ggml ne = {DK, n_kv, 1, n3});  V := K
+ * mask: f16 [n_tok][n_kv] or NULL (rows n_tok..pad64 are filled with -inf here)
+ * dst:  f32 [n3][n_tok][n_head][DK]
+ */
+int ref_flash_attn_ext(int k_type, int64_t DK, int64_t n_tok, int64_t n_head, int64_t n3, int64_t n_kv,
+                       const float * q, const void * k, const uint16_t * mask, float scale, float max_bias,
+                       float softcap, float * dst, int n_threads) {
+    const enum ggml_type kt = (enum ggml_type) k_type;
+    size_t mem = (size_t) DK * n_tok * n_head * n3 * 4 * 2 + row_bytes(kt, DK) * n_kv * n3 +
+                 (size_t) n_kv * GGML_PAD(n_tok, GGML_KQ_MASK_PAD) * 2 + (64u << 20);
+    mem += (size_t) n_threads * (3 * DK + 64) * 4 + (16u << 20);
+    struct ggml_init_params ip = { mem, NULL, false };
+    struct ggml_context *   ctx = ggml_init(ip);
+    if (!ctx) return -1;
+    struct ggml_tensor * tq = ggml_new_tensor_4d(ctx, GGML_TYPE_F32, DK, n_tok, n_head, n3);
+    struct ggml_tensor * tk = ggml_new_tensor_4d(ctx, kt, DK, n_kv, 1, n3);
+    memcpy(tq->data, q, ggml_nbytes(tq));
+    memcpy(tk->data, k, ggml_nbytes(tk));
+    struct ggml_tensor * tm = NULL;
+    if (mask) {
+        tm = make_mask(ctx, n_kv, n_tok);
+        uint16_t * md = (uint16_t *) tm->data;
+        for (int64_t i = 0; i < tm->ne[1]; i++)
+            for (int64_t j = 0; j < n_kv; j++) md[i * n_kv + j] = i < n_tok ? mask[i * n_kv + j] : 0xfc00; /* -inf */
+    }
+    struct ggml_tensor * o = ggml_flash_attn_ext(ctx, tq, tk, tk, tm, scale, max_bias, softcap);
+    ggml_flash_attn_ext_set_prec(o, GGML_PREC_F32);
+    struct ggml_cgraph * gf = ggml_new_graph(ctx);
+    ggml_build_forward_expand(gf, o);
+    enum ggml_status st = ggml_graph_compute_with_ctx(ctx, gf, n_threads);
+    if (st == GGML_STATUS_SUCCESS) memcpy(dst, o->data, ggml_nbytes(o));
+    ggml_free(ctx);
+    return (int) st;
+}
+
+/*
+ * Same node, computed by a backend loaded from `so_path`, driven only through the reference's ggml-backend API.
+ * Optional paged extension: block_table (i32 [n3][max_blocks]) and seq_lens (i32 [n3]) become src[4]/src[5] of
+ * the node; k is then the page pool, contiguous [n_kv][row_bytes] with n_kv = pool tokens (ggml ne = {DK, n_kv, 1, 1}).
+ * mask (optional) is f16 [n_tok][mask_ne0]; rows n_tok..pad64 are filled with -inf here.
+ * dv: DK passes V := K; 512 passes a 512-wide view of K as V (which ggml-cpu itself asserts on, ggml-cpu.c:11943).
+ * use_sched != 0 runs the graph through ggml_backend_sched with {loaded backend, CPU} the way llama_decode does
+ * (ggml-backend.cpp:1493-1587, :1727-1739) instead of calling ggml_backend_graph_compute directly.
+ * Returns 0 on success; negative for set-up failures; the ggml_status otherwise.
+ */
+int ref_backend_flash_attn_ext(const char * so_path, int k_type, int64_t DK, int64_t dv, int64_t n_tok, int64_t n_head,
+                               int64_t n3, int64_t n_kv, const float * q, const void * k, const uint16_t * mask,
+                               int64_t mask_ne0, const int32_t * block_table, int64_t max_blocks,
+                               const int32_t * seq_lens, float scale, float max_bias, float softcap, int use_sched,
+                               float * dst, char * info, size_t info_len) {
+    static ggml_backend_reg_t reg = NULL;
+    static char               loaded_path[4096];
+    if (!reg || strcmp(loaded_path, so_path) != 0) {
+        reg = ggml_backend_load(so_path);
+        if (!reg) return -10;
+        snprintf(loaded_path, sizeof(loaded_path), "%s", so_path);
+    }
+    if (ggml_backend_reg_dev_count(reg) < 1) return -11;
+    ggml_backend_dev_t dev = ggml_backend_reg_dev_get(reg, 0);
+    ggml_backend_t     be  = ggml_backend_dev_init(dev, NULL);
+    if (!be) return -12;
+    if (info) snprintf(info, info_len, "reg=%s dev=%s (%s) type=%d backend=%s buft=%s", ggml_backend_reg_name(reg),
+                       ggml_backend_dev_name(dev), ggml_backend_dev_description(dev), (int) ggml_backend_dev_type(dev),
+                       ggml_backend_name(be), ggml_backend_buft_name(ggml_backend_dev_buffer_type(dev)));
+
+    const enum ggml_type    kt    = (enum ggml_type) k_type;
+    const int               paged = block_table != NULL;
+    struct ggml_init_params ip    = { ggml_tensor_overhead() * 32 + ggml_graph_overhead() + 4096, NULL, true };
+    struct ggml_context *   ctx   = ggml_init(ip);
+    if (!ctx) { ggml_backend_free(be); return -13; }
+
+    struct ggml_tensor * tq = ggml_new_tensor_4d(ctx, GGML_TYPE_F32, DK, n_tok, n_head, n3);
+    struct ggml_tensor * tk = ggml_new_tensor_4d(ctx, kt, DK, n_kv, 1, paged ? 1 : n3);
+    struct ggml_tensor * tv = tk;
+    if (dv != DK) tv = ggml_view_4d(ctx, tk, dv, tk->ne[1], tk->ne[2], tk->ne[3], tk->nb[1], tk->nb[2], tk->nb[3], 0);
+    struct ggml_tensor * tm = mask ? make_mask(ctx, mask_ne0, n_tok) : NULL;
+    struct ggml_tensor * tb = paged ? ggml_new_tensor_2d(ctx, GGML_TYPE_I32, max_blocks, n3) : NULL;
+    struct ggml_tensor * tl = paged ? ggml_new_tensor_1d(ctx, GGML_TYPE_I32, n3) : NULL;
+    ggml_set_input(tq); ggml_set_input(tk);
+    if (tm) ggml_set_input(tm);
+    if (tb) { ggml_set_input(tb); ggml_set_input(tl); }
+    struct ggml_tensor * o = ggml_flash_attn_ext(ctx, tq, tk, tv, tm, scale, max_bias, softcap);
+    ggml_flash_attn_ext_set_prec(o, GGML_PREC_F32);
+    o->src[4] = tb; /* same slot convention as ggml_flash_attn_prompt's length tensors, ggml.c:2707-2710 */
+    o->src[5] = tl;
+    ggml_set_output(o);
+    struct ggml_cgraph * gf = ggml_new_graph(ctx);
+    ggml_build_forward_expand(gf, o);
+
+    int                   rc    = 0;
+    ggml_backend_buffer_t buf   = NULL;
+    ggml_backend_sched_t  sched = NULL;
+    ggml_backend_t        cpu   = NULL;
+    if (!ggml_backend_dev_supports_op(dev, o)) { rc = -14; goto done; }
+
+    if (use_sched) {
+        cpu = ggml_backend_init_by_type(GGML_BACKEND_DEVICE_TYPE_CPU, NULL);
+        if (!cpu) { rc = -15; goto done; }
+        ggml_backend_t backends[2] = { be, cpu };
+        sched = ggml_backend_sched_new(backends, NULL, 2, GGML_DEFAULT_GRAPH_SIZE, false);
+        if (!sched || !ggml_backend_sched_alloc_graph(sched, gf)) { rc = -16; goto done; }
+        if (ggml_backend_sched_get_tensor_backend(sched, o) != be) { rc = -17; goto done; }
+    } else {
+        buf = ggml_backend_alloc_ctx_tensors(ctx, be);
+        if (!buf) { rc = -18; goto done; }
+    }
+
+    ggml_backend_tensor_set(tq, q, 0, ggml_nbytes(tq));
+    ggml_backend_tensor_set(tk, k, 0, ggml_nbytes(tk));
+    if (tm) {
+        const size_t nrow = (size_t) tm->ne[1];
+        uint16_t *   md   = (uint16_t *) malloc(nrow * mask_ne0 * 2);
+        for (size_t i = 0; i < nrow; i++)
+            for (int64_t j = 0; j < mask_ne0; j++) md[i * mask_ne0 + j] = (int64_t) i < n_tok ? mask[i * mask_ne0 + j] : 0xfc00;
+        ggml_backend_tensor_set(tm, md, 0, ggml_nbytes(tm));
+        free(md);
+    }
+    if (tb) {
+        ggml_backend_tensor_set(tb, block_table, 0, ggml_nbytes(tb));
+        ggml_backend_tensor_set(tl, seq_lens, 0, ggml_nbytes(tl));
+    }
+    {
+        enum ggml_status st = use_sched ? ggml_backend_sched_graph_compute(sched, gf) : ggml_backend_graph_compute(be, gf);
+        if (st != GGML_STATUS_SUCCESS) { rc = (int) st ? (int) st : -19; goto done; }
+    }
+    ggml_backend_tensor_get(o, dst, 0, ggml_nbytes(o));
+done:
+    if (sched) ggml_backend_sched_free(sched);
+    if (buf) ggml_backend_buffer_free(buf);
+    if (cpu) ggml_backend_free(cpu);
+    ggml_free(ctx);
+    ggml_backend_free(be);
+    return rc;
+}
+
+/* ------------------------------------------------------------------ small pinning helpers */
+
+void ref_quantize_q8_0_ref(const float * x, void * y, int64_t k) { quantize_row_q8_0_ref(x, (block_q8_0 *) y, k); }
+void ref_quantize_q8_0_cpu(const float * x, void * y, int64_t k) { quantize_row_q8_0(x, y, k); }
+void ref_dequantize_q8_0(const void * x, float * y, int64_t k) { dequantize_row_q8_0((const block_q8_0 *) x, y, k); }
+void ref_f32_to_f16_row(const float * x, uint16_t * y, int64_t n) { ggml_fp32_to_fp16_row(x, y, n); }
+void ref_f32_to_bf16_row(const float * x, uint16_t * y, int64_t n) { ggml_fp32_to_bf16_row(x, (ggml_bf16_t *) y, n); }
+void ref_f16_to_f32_row(const uint16_t * x, float * y, int64_t n) { ggml_fp16_to_fp32_row(x, y, n); }
+
+/* sizeof / offsetof / ordinals a drop-in backend has to agree with (ggml.h:597-631, :360-401, :438-549,
+ * ggml-backend-impl.h, ggml-impl.h:287-304).  Names are matched by tests/test_abi.py against the mirror. */
+struct ref_abi_entry { const char * name; int64_t value; };
+#define E(n, v) { n, (int64_t) (v) }
+static const struct ref_abi_entry abi_table[] = {
+    E("sizeof(ggml_tensor)", sizeof(struct ggml_tensor)),
+    E("offsetof(ggml_tensor,type)", offsetof(struct ggml_tensor, type)),
+    E("offsetof(ggml_tensor,buffer)", offsetof(struct ggml_tensor, buffer)),
+    E("offsetof(ggml_tensor,ne)", offsetof(struct ggml_tensor, ne)),
+    E("offsetof(ggml_tensor,nb)", offsetof(struct ggml_tensor, nb)),
+    E("offsetof(ggml_tensor,op)", offsetof(struct ggml_tensor, op)),
+    E("offsetof(ggml_tensor,op_params)", offsetof(struct ggml_tensor, op_params)),
+    E("offsetof(ggml_tensor,flags)", offsetof(struct ggml_tensor, flags)),
+    E("offsetof(ggml_tensor,src)", offsetof(struct ggml_tensor, src)),
+    E("offsetof(ggml_tensor,view_src)", offsetof(struct ggml_tensor, view_src)),
+    E("offsetof(ggml_tensor,view_offs)", offsetof(struct ggml_tensor, view_offs)),
+    E("offsetof(ggml_tensor,data)", offsetof(struct ggml_tensor, data)),
+    E("offsetof(ggml_tensor,name)", offsetof(struct ggml_tensor, name)),
+    E("offsetof(ggml_tensor,extra)", offsetof(struct ggml_tensor, extra)),
+    E("GGML_MAX_DIMS", GGML_MAX_DIMS), E("GGML_MAX_SRC", GGML_MAX_SRC), E("GGML_MAX_OP_PARAMS", GGML_MAX_OP_PARAMS),
+    E("GGML_MAX_NAME", GGML_MAX_NAME), E("GGML_KQ_MASK_PAD", GGML_KQ_MASK_PAD),
+    E("sizeof(ggml_cgraph)", sizeof(struct ggml_cgraph)),
+    E("offsetof(ggml_cgraph,n_nodes)", offsetof(struct ggml_cgraph, n_nodes)),
+    E("offsetof(ggml_cgraph,nodes)", offsetof(struct ggml_cgraph, nodes)),
+    E("sizeof(ggml_backend_buffer_type_i)", sizeof(struct ggml_backend_buffer_type_i)),
+    E("sizeof(ggml_backend_buffer_type)", sizeof(struct ggml_backend_buffer_type)),
+    E("offsetof(ggml_backend_buffer_type,device)", offsetof(struct ggml_backend_buffer_type, device)),
+    E("offsetof(ggml_backend_buffer_type,context)", offsetof(struct ggml_backend_buffer_type, context)),
+    E("sizeof(ggml_backend_buffer_i)", sizeof(struct ggml_backend_buffer_i)),
+    E("sizeof(ggml_backend_buffer)", sizeof(struct ggml_backend_buffer)),
+    E("offsetof(ggml_backend_buffer,buft)", offsetof(struct ggml_backend_buffer, buft)),
+    E("offsetof(ggml_backend_buffer,context)", offsetof(struct ggml_backend_buffer, context)),
+    E("offsetof(ggml_backend_buffer,size)", offsetof(struct ggml_backend_buffer, size)),
+    E("offsetof(ggml_backend_buffer,usage)", offsetof(struct ggml_backend_buffer, usage)),
+    E("sizeof(ggml_backend_i)", sizeof(struct ggml_backend_i)),
+    E("offsetof(ggml_backend_i,graph_compute)", offsetof(struct ggml_backend_i, graph_compute)),
+    E("offsetof(ggml_backend_i,synchronize)", offsetof(struct ggml_backend_i, synchronize)),
+    E("sizeof(ggml_backend)", sizeof(struct ggml_backend)),
+    E("offsetof(ggml_backend,iface)", offsetof(struct ggml_backend, iface)),
+    E("offsetof(ggml_backend,device)", offsetof(struct ggml_backend, device)),
+    E("offsetof(ggml_backend,context)", offsetof(struct ggml_backend, context)),
+    E("sizeof(ggml_backend_device_i)", sizeof(struct ggml_backend_device_i)),
+    E("offsetof(ggml_backend_device_i,supports_op)", offsetof(struct ggml_backend_device_i, supports_op)),
+    E("sizeof(ggml_backend_device)", sizeof(struct ggml_backend_device)),
+    E("offsetof(ggml_backend_device,reg)", offsetof(struct ggml_backend_device, reg)),
+    E("offsetof(ggml_backend_device,context)", offsetof(struct ggml_backend_device, context)),
+    E("sizeof(ggml_backend_reg_i)", sizeof(struct ggml_backend_reg_i)),
+    E("sizeof(ggml_backend_reg)", sizeof(struct ggml_backend_reg)),
+    E("offsetof(ggml_backend_reg,iface)", offsetof(struct ggml_backend_reg, iface)),
+    E("offsetof(ggml_backend_reg,context)", offsetof(struct ggml_backend_reg, context)),
+    E("sizeof(ggml_backend_dev_props)", sizeof(struct ggml_backend_dev_props)),
+    E("offsetof(ggml_backend_dev_props,type)", offsetof(struct ggml_backend_dev_props, type)),
+    E("offsetof(ggml_backend_dev_props,caps)", offsetof(struct ggml_backend_dev_props, caps)),
+    E("sizeof(ggml_backend_event)", sizeof(struct ggml_backend_event)),
+    E("GGML_BACKEND_API_VERSION", GGML_BACKEND_API_VERSION),
+    E("GGML_TYPE_F32", GGML_TYPE_F32), E("GGML_TYPE_F16", GGML_TYPE_F16), E("GGML_TYPE_Q8_0", GGML_TYPE_Q8_0),
+    E("GGML_TYPE_I8", GGML_TYPE_I8), E("GGML_TYPE_I32", GGML_TYPE_I32), E("GGML_TYPE_BF16", GGML_TYPE_BF16),
+    E("GGML_TYPE_COUNT", GGML_TYPE_COUNT),
+    E("GGML_OP_NONE", GGML_OP_NONE), E("GGML_OP_CPY", GGML_OP_CPY), E("GGML_OP_CONT", GGML_OP_CONT),
+    E("GGML_OP_RESHAPE", GGML_OP_RESHAPE), E("GGML_OP_VIEW", GGML_OP_VIEW), E("GGML_OP_PERMUTE", GGML_OP_PERMUTE),
+    E("GGML_OP_TRANSPOSE", GGML_OP_TRANSPOSE), E("GGML_OP_FLASH_ATTN_EXT", GGML_OP_FLASH_ATTN_EXT),
+    E("GGML_OP_SCATTER_UPDATE", GGML_OP_SCATTER_UPDATE), E("GGML_OP_COUNT", GGML_OP_COUNT),
+    E("GGML_STATUS_ALLOC_FAILED", GGML_STATUS_ALLOC_FAILED), E("GGML_STATUS_FAILED", GGML_STATUS_FAILED),
+    E("GGML_STATUS_SUCCESS", GGML_STATUS_SUCCESS), E("GGML_STATUS_ABORTED", GGML_STATUS_ABORTED),
+    E("GGML_BACKEND_DEVICE_TYPE_CPU", GGML_BACKEND_DEVICE_TYPE_CPU), E("GGML_BACKEND_DEVICE_TYPE_GPU", GGML_BACKEND_DEVICE_TYPE_GPU),
+    E("GGML_BACKEND_BUFFER_USAGE_ANY", GGML_BACKEND_BUFFER_USAGE_ANY), E("GGML_BACKEND_BUFFER_USAGE_COMPUTE", GGML_BACKEND_BUFFER_USAGE_COMPUTE),
+    E("GGML_PREC_DEFAULT", GGML_PREC_DEFAULT), E("GGML_PREC_F32", GGML_PREC_F32),
+    E("GGML_TENSOR_FLAG_INPUT", GGML_TENSOR_FLAG_INPUT), E("GGML_TENSOR_FLAG_OUTPUT", GGML_TENSOR_FLAG_OUTPUT),
+    E("sizeof(block_q8_0)", sizeof(block_q8_0)),
+};
+int ref_abi_table(int i, const char ** name, int64_t * value) {
+    const int n = (int) (sizeof(abi_table) / sizeof(abi_table[0]));
+    if (i < 0 || i >= n) return n;
+    *name = abi_table[i].name; *value = abi_table[i].value;
+    return n;
+}

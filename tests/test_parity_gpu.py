@@ -1,0 +1,111 @@
+"""GPU parity: the HIP path (through the C ABI of include/mla_attn.h) against the oracle on the same seeded inputs.
+Tolerance (stated by the target): max-abs 2e-3 and relative L2 1e-3 on the fp32 output."""
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+from tests import util as U
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(gpu, q, k, k_type, dv=512, mask=None, bt=None, lens=None, **kw):
+    import torch
+    import jittorinfer_amd as J
+    tq = torch.from_numpy(q).to(gpu)
+    tk = torch.from_numpy(k.view(np.int16) if k.dtype == np.uint16 else k).to(gpu)
+    tm = None if mask is None else torch.from_numpy(mask.view(np.float16)).to(gpu)
+    tb = None if bt is None else torch.from_numpy(bt).to(gpu)
+    tl = None if lens is None else torch.from_numpy(np.asarray(lens, dtype=np.int32)).to(gpu)
+    out = torch.full((q.shape[0], q.shape[2], q.shape[1], 576), float("nan"), dtype=torch.float32, device=gpu)
+    J.ggml_flash_attn_ext(tq, tk, k_type, dv=dv, mask=tm, block_table=tb, seq_lens=tl, out=out, **kw)
+    torch.cuda.synchronize()
+    return out.cpu().numpy()
+
+
+@pytest.mark.parametrize("k_type", [O.TYPE_BF16, O.TYPE_F16, O.TYPE_Q8_0])
+@pytest.mark.parametrize("n_head,n_kv", [(16, 1024), (16, 77), (128, 384), (48, 200)])
+def test_contiguous_decode(gpu, k_type, n_head, n_kv):
+    rng = np.random.default_rng(1234 + n_head + n_kv)
+    q = rng.standard_normal((2, n_head, 1, 576)).astype(np.float32)
+    k = U.encode_kv(rng.standard_normal((2, n_kv, 576)).astype(np.float32), k_type)
+    got = _run(gpu, q, k, k_type, scale=U.SCALE)
+    if k_type == O.TYPE_F16:
+        # ggml-cpu accumulates V in f16 for F16 KV; the fast kernel accumulates in f32 and is held to the f64 value
+        want = O.flash_attn_ext_f64(q, k, k_type, dv=512, scale=U.SCALE)
+    else:
+        want = O.flash_attn_ext(q, k, k_type, dv=512, scale=U.SCALE)
+    print(U.check(got[..., :512], want, "contiguous decode"))
+    assert np.isnan(got[..., 512:]).all()  # columns >= dv are left untouched
+
+
+def test_config1_f16_strict(gpu):
+    """BASELINE config 1: one sequence, 16 heads, 1024 contiguous f16 keys, V = K[:, :512]; strict replay of the
+    reference's f16 accumulator."""
+    import jittorinfer_amd as J
+    rng = np.random.default_rng(1234)
+    q = rng.standard_normal((1, 16, 1, 576)).astype(np.float32)
+    k = O.f32_to_f16(rng.standard_normal((1, 1024, 576)).astype(np.float32))
+    want = O.flash_attn_ext(q, k, O.TYPE_F16, dv=512, scale=U.SCALE)
+    got = _run(gpu, q, k, O.TYPE_F16, scale=U.SCALE, flags=J.MLA_FLAG_F16_ACC_STRICT)
+    print(U.check(got[..., :512], want, "config 1 strict f16"))
+
+
+@pytest.mark.parametrize("k_type", [O.TYPE_BF16, O.TYPE_Q8_0])
+def test_config2_paged_decode(gpu, k_type):
+    """BASELINE config 2 shape: batch 8, 16 heads, lengths uniform in [512, 4096], 512-page pool, shuffled table."""
+    rng = np.random.default_rng(2)
+    lens = rng.integers(512, 4097, size=8)
+    pool, bt, seqs = U.make_paged(rng, lens, k_type, n_pool_pages=512)
+    q = rng.standard_normal((8, 16, 1, 576)).astype(np.float32)
+    got = _run(gpu, q, pool, k_type, bt=bt, lens=lens, scale=U.SCALE)
+    want = U.oracle_per_seq(q, seqs, k_type, 512)
+    print(U.check(got[..., :512], want, "config 2"))
+
+
+@pytest.mark.parametrize("n_splits", [0, 1, 3])
+def test_config3_reduced(gpu, n_splits):
+    """Config 3 at reduced size: 128 heads, bf16 pages, K ~ N(0, 0.5), split-K over the context."""
+    rng = np.random.default_rng(3)
+    lens = [1024, 1000, 129]
+    pool, bt, seqs = U.make_paged(rng, lens, O.TYPE_BF16, sigma=0.5)
+    q = rng.standard_normal((3, 128, 1, 576)).astype(np.float32)
+    got = _run(gpu, q, pool, O.TYPE_BF16, bt=bt, lens=lens, scale=U.SCALE, n_splits=n_splits)
+    want = U.oracle_per_seq(q, seqs, O.TYPE_BF16, 512)
+    print(U.check(got[..., :512], want, "config 3 reduced"))
+
+
+def test_config4_reduced_prefill(gpu):
+    """Config 4 at reduced size: causal chunked prefill, 40 new tokens on 200 cached ones, 16 heads, 2 sequences."""
+    rng = np.random.default_rng(4)
+    n_new, n_old = 40, 200
+    lens = [n_new + n_old] * 2
+    pool, bt, seqs = U.make_paged(rng, lens, O.TYPE_BF16)
+    q = rng.standard_normal((2, 16, n_new, 576)).astype(np.float32)
+    kv_pos = np.arange(n_new + n_old)[None, :]
+    mask = np.where(kv_pos > n_old + np.arange(n_new)[:, None], -np.inf, 0.0).astype(np.float16).view(np.uint16)
+    got = _run(gpu, q, pool, O.TYPE_BF16, mask=mask, bt=bt, lens=lens, scale=U.SCALE)
+    want = U.oracle_per_seq(q, seqs, O.TYPE_BF16, 512, mask=mask)
+    print(U.check(got[..., :512], want, "config 4 reduced"))
+
+
+def test_config5_reduced_q8(gpu):
+    """Config 5 at reduced size: Q8_0 pages built as int8 = clip(round(N(0,1)/scale)) with one fp16 scale."""
+    rng = np.random.default_rng(5)
+    lens = rng.integers(100, 700, size=4)
+    pool, bt, seqs = U.make_paged(rng, lens, O.TYPE_Q8_0, q8_scale=1.0 / 32)
+    q = rng.standard_normal((4, 128, 1, 576)).astype(np.float32)
+    got = _run(gpu, q, pool, O.TYPE_Q8_0, bt=bt, lens=lens, scale=U.SCALE)
+    want = U.oracle_per_seq(q, seqs, O.TYPE_Q8_0, 512)
+    print(U.check(got[..., :512], want, "config 5 reduced"))
+
+
+@pytest.mark.parametrize("k_type", [O.TYPE_BF16, O.TYPE_Q8_0])
+def test_dv576_matches_ggml_cpu_layout(gpu, k_type):
+    """V := K (576 wide), the only form the reference's CPU op accepts: all 576 output columns."""
+    rng = np.random.default_rng(6)
+    q = rng.standard_normal((2, 16, 3, 576)).astype(np.float32)
+    k = U.encode_kv(rng.standard_normal((2, 300, 576)).astype(np.float32), k_type)
+    got = _run(gpu, q, k, k_type, dv=576, scale=U.SCALE)
+    want = O.flash_attn_ext(q, k, k_type, dv=576, scale=U.SCALE)
+    print(U.check(got, want, "dv 576"))
