@@ -1,0 +1,186 @@
+#!/usr/bin/env python3
+"""Benchmark of the MLA paged-decode hot path on one MI355X.
+
+A step is one GGML_OP_FLASH_ATTN_EXT node of the DeepSeek-V2 shape through the C ABI (split-K decode kernel +
+combine pass): batch 32, 128 heads, every context 8192 tokens, bf16 latent KV (576-d QK, 512-d V) in 128-token
+pages behind a shuffled block table, Q ~ N(0,1), K ~ N(0,0.5).  Inputs are resident in HBM before the timed region.
+The KV pool is rotated between steps (several distinct pools) so that reads are HBM traffic, not Infinity-Cache hits.
+
+Prints ONE JSON line:  value = algorithmic KV bytes per step / step time, in GB/s (whole job, one GPU).
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
+KV_ROW_BYTES = 1152     # 576 bf16
+FLOP_PER_TOKEN_HEAD = 2 * 576 + 2 * 512
+
+
+def build_workload(dev, n_seq, n_head, ctx, n_pools, seed):
+    import torch
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed)
+    pages_per_seq = ctx // 128
+    n_pages = n_seq * pages_per_seq
+    pools = []
+    for _ in range(n_pools):
+        kf = torch.randn((n_pages * 128, 576), generator=g, device=dev, dtype=torch.float32) * 0.5
+        pools.append(kf.to(torch.bfloat16))
+        del kf
+    perm = torch.randperm(n_pages, generator=g, device=dev).to(torch.int32)
+    block_table = perm.reshape(n_seq, pages_per_seq).contiguous()
+    seq_lens = torch.full((n_seq,), ctx, dtype=torch.int32, device=dev)
+    q = torch.randn((n_seq, n_head, 1, 576), generator=g, device=dev, dtype=torch.float32)
+    return q, pools, block_table, seq_lens
+
+
+def cpu_baseline(q, pool, block_table, ctx, n_sample, scale, gpu_out):
+    """ggml-cpu's flash_attn_ext on the host cores for the first n_sample sequences of the same workload:
+    the reference's own compiled ggml when oracle/_ref is built (kind "reference"), else the C restatement ("port")."""
+    import numpy as np
+    import torch
+    from oracle import oracle as O
+    cores = min(os.cpu_count() or 1, 16)
+    qs = q[:n_sample].cpu().numpy()
+    ids = block_table[:n_sample].cpu().numpy().astype(np.int64)
+    pool_pages = pool.view(torch.int16).reshape(-1, 128, 576)
+    k = pool_pages[torch.from_numpy(ids).to(pool.device)].reshape(n_sample, ctx, 576).cpu().numpy().view(np.uint16)
+    kind = "reference" if O.ref_available() else "port"
+
+    def run():
+        if kind == "reference":
+            return O.ref_flash_attn_ext(qs, k, O.TYPE_BF16, scale=scale, n_threads=cores)[..., :512]
+        return O.flash_attn_ext(qs, k, O.TYPE_BF16, dv=512, scale=scale, n_threads=cores)
+
+    want = run()  # warm-up, also the parity check
+    best = float("inf")
+    for _ in range(3):
+        t0 = time.perf_counter()
+        run()
+        best = min(best, time.perf_counter() - t0)
+    kv_bytes = n_sample * ctx * KV_ROW_BYTES
+    got = gpu_out[:n_sample, :, :, :512].cpu().numpy()
+    max_abs, rel_l2 = O.errors(got, want)
+    return {
+        "value": kv_bytes / best / 1e9, "unit": "GB/s", "cores": cores, "kind": kind,
+        "sample": "%d of the workload's sequences (128 heads x %d keys each), OpenMP over rows, best of 3; %.1f ms" % (n_sample, ctx, best * 1e3),
+        "us_per_step_equiv": best * 1e6 * (q.shape[0] / n_sample),
+    }, {"max_abs": max_abs, "rel_l2": rel_l2, "vs": kind, "sequences": n_sample}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--batch", type=int, default=32)
+    ap.add_argument("--heads", type=int, default=128)
+    ap.add_argument("--ctx", type=int, default=8192)
+    ap.add_argument("--pools", type=int, default=4, help="distinct KV pools rotated between steps")
+    ap.add_argument("--splits", type=int, default=0)
+    ap.add_argument("--cpu-seqs", type=int, default=8, help="sequences of the workload timed on the host cores (0 = skip)")
+    ap.add_argument("--seed", type=int, default=1234)
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py: this build measures one GPU's share of the path; --gpus %d is not supported (use --gpus 1)" % a.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import jittorinfer_amd as J
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    lib = J.library()
+    dev = torch.device("cuda:0")
+    scale = 1.0 / (192.0 ** 0.5)
+
+    q, pools, block_table, seq_lens = build_workload(dev, a.batch, a.heads, a.ctx, a.pools, a.seed)
+    out = torch.empty((a.batch, 1, a.heads, 576), dtype=torch.float32, device=dev)
+    args = []
+    keep = []
+    for pool in pools:
+        ar, _, k = J.capi.make_args(q, pool.view(torch.int16), J.MLA_TYPE_BF16, dv=512, scale=scale, block_table=block_table,
+                                    seq_lens=seq_lens, out=out, n_splits=a.splits)
+        args.append(ar)
+        keep.append(k)
+    plan = J.plan(q, pools[0].view(torch.int16), J.MLA_TYPE_BF16, dv=512, scale=scale, block_table=block_table, seq_lens=seq_lens, out=out, n_splits=a.splits)
+    stream = torch.cuda.current_stream(dev)
+    st = C.c_void_p(stream.cuda_stream)
+
+    def step(i, fn=lib.mla_attn_launch):
+        rc = fn(C.byref(args[i % len(args)]), st)
+        if rc != 0:
+            raise RuntimeError("launch failed: %d" % rc)
+
+    for i in range(a.warmup):
+        step(i)
+    torch.cuda.synchronize()
+
+    # ---- timed region: exactly K steps, synchronised on both sides
+    t0 = time.perf_counter()
+    for i in range(a.steps):
+        step(i)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / a.steps
+
+    # ---- the dominant kernel alone (the split-K decode kernel), HIP events on the launch stream around each launch
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(a.steps)]
+    for i in range(a.steps):
+        evs[i][0].record(stream)
+        step(i, lib.mla_attn_launch_partials)
+        evs[i][1].record(stream)
+    torch.cuda.synchronize()
+    durs = sorted(e0.elapsed_time(e1) for e0, e1 in evs)
+    kern_ms = sum(durs) / len(durs)
+    # and whole steps with events (decode + combine)
+    for i in range(a.steps):
+        evs[i][0].record(stream)
+        step(i)
+        evs[i][1].record(stream)
+    torch.cuda.synchronize()
+    sdurs = sorted(e0.elapsed_time(e1) for e0, e1 in evs)
+
+    kv_bytes = a.batch * a.ctx * KV_ROW_BYTES
+    flops = a.batch * a.ctx * a.heads * FLOP_PER_TOKEN_HEAD
+    value = kv_bytes / (ms_per_step * 1e-3) / 1e9
+    achieved = kv_bytes / (kern_ms * 1e-3) / 1e9
+
+    # final output of the last step for the parity check
+    step(0)
+    torch.cuda.synchronize()
+    cpu, parity = (None, None)
+    if a.cpu_seqs > 0:
+        cpu, parity = cpu_baseline(q, pools[0], block_table, a.ctx, min(a.cpu_seqs, a.batch), scale, out)
+
+    res = {
+        "metric": "mla_paged_decode_kv_read_bandwidth", "value": value, "unit": "GB/s",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "BASELINE configs[2]: paged MLA decode B=%d H=%d ctx=%d, bf16 latent KV 576/512, 128-token pages, shuffled block table" % (a.batch, a.heads, a.ctx),
+                   "batch": a.batch, "heads": a.heads, "ctx": a.ctx, "kv_pools_rotated": a.pools, "plan": plan},
+        "us_per_step": ms_per_step * 1e3,
+        "us_per_step_events": {"median": sdurs[len(sdurs) // 2] * 1e3, "p10": sdurs[len(sdurs) // 10] * 1e3, "p90": sdurs[(len(sdurs) * 9) // 10] * 1e3},
+        "tokens_per_s": a.batch / (ms_per_step * 1e-3),
+        "pct_hbm_peak": 100.0 * value / HBM_PEAK_GBPS,
+        "tflops": flops / (ms_per_step * 1e-3) / 1e12,
+        "roofline": {"bound": "hbm", "kernel": "mla_attn_tile_kernel<bf16,16,4,1>", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+                     "algorithmic_bytes_per_launch": kv_bytes, "kernel_us": {"mean": kern_ms * 1e3, "median": durs[len(durs) // 2] * 1e3},
+                     "mfma_tflops": flops / (kern_ms * 1e-3) / 1e12},
+        "cpu_baseline": cpu,
+        "parity": parity,
+    }
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

@@ -116,6 +116,13 @@ size_t mla_attn_workspace_size(const mla_attn_args * args);
 int    mla_attn_plan(const mla_attn_args * args, mla_attn_plan_info * out);
 int    mla_attn_launch(const mla_attn_args * args, void * stream);
 
+/* The two halves of mla_attn_launch, for callers that time or schedule them separately: the attention kernel(s)
+ * that read the KV rows (writing split-K partials into the workspace, or the final output when the plan has one
+ * split), and the log-sum-exp combine pass over the partials (a no-op for one split).  No counterpart in the
+ * reference, whose CPU op has no split-K. */
+int    mla_attn_launch_partials(const mla_attn_args * args, void * stream);
+int    mla_attn_launch_combine(const mla_attn_args * args, void * stream);
+
 /* dst[i] = src[i] for n_bytes (multiple of 16) */
 int mla_hbm_copy_launch(const void * src, void * dst, size_t n_bytes, void * stream);
 

@@ -696,7 +696,8 @@ int mla_attn_plan(const mla_attn_args * args, mla_attn_plan_info * out) {
     return 0;
 }
 
-int mla_attn_launch(const mla_attn_args * a, void * stream) {
+// phases: bit 0 = the attention kernels (partials or final output), bit 1 = the combine pass
+static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
     Plan pl;
     const int rc = make_plan(a, &pl);
     if (rc) return rc;
@@ -726,6 +727,7 @@ int mla_attn_launch(const mla_attn_args * a, void * stream) {
     float * scores = (float *) (ws + align256(pl.ws_part_o) + align256(pl.ws_part_ml));
 
     if (pl.variant == 1) {
+        if (!(phases & 1)) return 0;
         if (a->n_kv > 0) {
             dim3 g1((unsigned) ((a->n_kv + 3) / 4), (unsigned) kp.n_rows, (unsigned) a->n_seq);
             hipLaunchKernelGGL(mla_f16_scores_kernel, g1, dim3(256), 0, st, kp, scores);
@@ -738,7 +740,7 @@ int mla_attn_launch(const mla_attn_args * a, void * stream) {
     }
 
     dim3 grid((unsigned) pl.n_splits, (unsigned) pl.n_row_blocks, (unsigned) a->n_seq);
-    for (int pass = 0; pass < pl.n_passes; pass++) {
+    for (int pass = 0; pass < pl.n_passes && (phases & 1); pass++) {
         kp.d_off = pass * pl.ndb * 32;
         hipError_t e;
         switch (a->kv_type) {
@@ -748,13 +750,17 @@ int mla_attn_launch(const mla_attn_args * a, void * stream) {
         }
         if (e != hipSuccess) return (int) e;
     }
-    if (pl.n_splits > 1) {
+    if (pl.n_splits > 1 && (phases & 2)) {
         dim3 g((unsigned) kp.n_rows, (unsigned) a->n_seq);
         hipLaunchKernelGGL(mla_attn_combine_kernel, g, dim3(a->dv / 4), 0, st, kp);
         return (int) hipGetLastError();
     }
     return 0;
 }
+
+int mla_attn_launch(const mla_attn_args * a, void * stream) { return launch_phases(a, stream, 3); }
+int mla_attn_launch_partials(const mla_attn_args * a, void * stream) { return launch_phases(a, stream, 1); }
+int mla_attn_launch_combine(const mla_attn_args * a, void * stream) { return launch_phases(a, stream, 2); }
 
 int mla_hbm_copy_launch(const void * src, void * dst, size_t n_bytes, void * stream) {
     if (!src || !dst) return MLA_ERR_NULL;
