@@ -85,6 +85,7 @@ def main():
     ap.add_argument("--ctx", type=int, default=8192)
     ap.add_argument("--pools", type=int, default=4, help="distinct KV pools rotated between steps")
     ap.add_argument("--splits", type=int, default=0)
+    ap.add_argument("--rows-per-wg", type=int, default=0)
     ap.add_argument("--cpu-seqs", type=int, default=8, help="sequences of the workload timed on the host cores (0 = skip)")
     ap.add_argument("--seed", type=int, default=1234)
     a = ap.parse_args()
@@ -107,10 +108,10 @@ def main():
     keep = []
     for pool in pools:
         ar, _, k = J.capi.make_args(q, pool.view(torch.int16), J.MLA_TYPE_BF16, dv=512, scale=scale, block_table=block_table,
-                                    seq_lens=seq_lens, out=out, n_splits=a.splits)
+                                    seq_lens=seq_lens, out=out, n_splits=a.splits, rows_per_wg=a.rows_per_wg)
         args.append(ar)
         keep.append(k)
-    plan = J.plan(q, pools[0].view(torch.int16), J.MLA_TYPE_BF16, dv=512, scale=scale, block_table=block_table, seq_lens=seq_lens, out=out, n_splits=a.splits)
+    plan = J.plan(q, pools[0].view(torch.int16), J.MLA_TYPE_BF16, dv=512, scale=scale, block_table=block_table, seq_lens=seq_lens, out=out, n_splits=a.splits, rows_per_wg=a.rows_per_wg)
     stream = torch.cuda.current_stream(dev)
     st = C.c_void_p(stream.cuda_stream)
 

@@ -97,13 +97,13 @@ typedef struct mla_attn_args {
     void * workspace;
     size_t workspace_size;
 
-    /* ---- tuning: 0 = choose; otherwise the number of KV splits per sequence */
+    /* ---- tuning: 0 = choose.  n_splits: KV splits per sequence; rows_per_wg: 32, 64 or 128 rows per workgroup */
     int32_t n_splits;
-    int32_t reserved;
+    int32_t rows_per_wg;
 } mla_attn_args;
 
 typedef struct mla_attn_plan_info {
-    int32_t variant;      /* 0 = tiled MFMA kernel, 1 = strict f16-accumulator replay */
+    int32_t variant;      /* 0 = general tiled MFMA kernel, 1 = strict f16-accumulator replay, 2 = pipelined decode kernel */
     int32_t rows_per_wg;  /* (token, head) rows one workgroup owns */
     int32_t n_row_blocks; /* workgroups along rows, per sequence */
     int32_t n_splits;     /* KV splits per sequence (1 = no combine pass) */

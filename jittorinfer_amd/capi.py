@@ -21,7 +21,7 @@ class MlaAttnArgs(C.Structure):
         ("block_table", C.c_void_p), ("bt_stride", C.c_int64), ("seq_lens", C.c_void_p),
         ("dst", C.c_void_p), ("dst_nb1", C.c_int64),
         ("workspace", C.c_void_p), ("workspace_size", C.c_size_t),
-        ("n_splits", C.c_int32), ("reserved", C.c_int32),
+        ("n_splits", C.c_int32), ("rows_per_wg", C.c_int32),
     ]
 
 
@@ -78,7 +78,7 @@ def _workspace(device, nbytes):
 
 
 def make_args(q, k, kv_type, dv=512, mask=None, scale=1.0, max_bias=0.0, logit_softcap=0.0, block_table=None,
-              seq_lens=None, out=None, n_splits=0, flags=0):
+              seq_lens=None, out=None, n_splits=0, flags=0, rows_per_wg=0):
     """Builds (args, out, keepalive) from torch tensors on one gfx950 device.
 
     q     float32 [n_seq, n_head, n_tok, 576] (any strides with a contiguous last dim)
@@ -117,6 +117,7 @@ def make_args(q, k, kv_type, dv=512, mask=None, scale=1.0, max_bias=0.0, logit_s
     assert out.dtype == torch.float32 and out.is_contiguous() and out.shape[:3] == (n_seq, n_tok, n_head) and out.shape[3] >= dv
     a.dst, a.dst_nb1 = out.data_ptr(), out.shape[3] * 4
     a.n_splits = n_splits
+    a.rows_per_wg = rows_per_wg
     need = library().mla_attn_workspace_size(C.byref(a))
     ws = _workspace(q.device, need)
     a.workspace, a.workspace_size = ws.data_ptr(), ws.numel()
@@ -124,14 +125,14 @@ def make_args(q, k, kv_type, dv=512, mask=None, scale=1.0, max_bias=0.0, logit_s
 
 
 def ggml_flash_attn_ext(q, k, kv_type, dv=512, mask=None, scale=1.0, max_bias=0.0, logit_softcap=0.0, *,
-                        block_table=None, seq_lens=None, out=None, n_splits=0, flags=0, stream=None):
+                        block_table=None, seq_lens=None, out=None, n_splits=0, flags=0, rows_per_wg=0, stream=None):
     """GGML_OP_FLASH_ATTN_EXT of the reference (ggml_flash_attn_ext(ctx, q, k, v, mask, scale, max_bias,
     logit_softcap), ggml/src/ggml.c:3988) for the MLA shape, on the current torch stream.  v is the first `dv`
     columns of k's rows.  Returns dst in ggml's layout: float32 [n_seq, n_tok, n_head, 576] with dv columns valid."""
     import torch
     if not q.is_cuda:
         raise RuntimeError("jittorinfer_amd runs on a gfx950 GPU only (there is no CPU path)")
-    a, out, keep = make_args(q, k, kv_type, dv, mask, scale, max_bias, logit_softcap, block_table, seq_lens, out, n_splits, flags)
+    a, out, keep = make_args(q, k, kv_type, dv, mask, scale, max_bias, logit_softcap, block_table, seq_lens, out, n_splits, flags, rows_per_wg)
     st = stream if stream is not None else torch.cuda.current_stream(q.device).cuda_stream
     rc = library().mla_attn_launch(C.byref(a), C.c_void_p(st))
     if rc != 0:

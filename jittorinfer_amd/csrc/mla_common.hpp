@@ -1,0 +1,95 @@
+// Shared definitions of the MLA attention kernels (gfx950).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <math.h>
+
+#include "../../include/mla_attn.h"
+
+namespace mla {
+
+
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
+typedef __attribute__((ext_vector_type(4))) short        s16x4;
+typedef __attribute__((ext_vector_type(16))) float       f32x16;
+typedef __attribute__((ext_vector_type(4))) float        f32x4;
+typedef __attribute__((ext_vector_type(8))) __bf16       bf16x8;
+typedef __attribute__((ext_vector_type(8))) _Float16     f16x8;
+
+#define LDS_PTR(T) T __attribute__((address_space(3))) *
+
+constexpr int DK          = 576;
+constexpr int KSTEPS      = DK / 16;  // 36 MFMA k-steps over the 576-d contraction
+constexpr int TILE_TOK    = 32;       // tokens per LDS tile (= MFMA M of S^T)
+constexpr int ROW_BYTES   = DK * 2;   // one latent row in LDS (bf16 / f16)
+constexpr int PITCH       = ROW_BYTES + 16;  // padded row pitch: 292 dwords, conflict-free for the b128 K reads
+constexpr int TILE_BYTES  = TILE_TOK * PITCH;
+constexpr int Q8_ROW      = 612;      // 18 blocks of (fp16 d, 32 x int8)
+constexpr int Q8_TILE_RAW = TILE_TOK * Q8_ROW;  // 19584 = 1224 x 16
+constexpr int NTHREADS    = 256;
+constexpr float LOG2E     = 1.4426950408889634f;
+
+enum { SRC_BF16 = 0, SRC_F16 = 1, SRC_Q8 = 2 };
+
+struct KParams {
+    const char *    q;
+    int64_t         q_nb1, q_nb2, q_nb3;
+    const char *    kv;
+    int64_t         kv_nb1, kv_nb3;
+    int64_t         n_kv;
+    const char *    mask;
+    int64_t         mask_nb1, mask_ne0;
+    const int32_t * block_table;
+    int64_t         bt_stride;
+    const int32_t * seq_lens;
+    float *         dst;
+    int64_t         dst_stride;  // floats
+    float *         part_o;      // [n_seq][n_splits][n_rows][dv_total]
+    float *         part_ml;     // [n_seq][n_splits][n_rows][2]  (max in log2 units, sum)
+    int             n_head, n_tok, n_rows;
+    int             n_splits, split_tokens;
+    int             dv_total, d_off;
+    float           scale, softcap, max_bias, m0, m1;
+    int             n_head_log2;
+    int             n_pool_pages;  // block-table mode: pages in the pool
+    int             rows_contig;  // kv rows are packed (kv_nb1 == row bytes): whole tiles are one contiguous run
+};
+
+template <typename T, typename U> __device__ __forceinline__ T bitcast(U u) { return __builtin_bit_cast(T, u); }
+
+template <bool F16> __device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
+    if constexpr (F16) return __builtin_amdgcn_mfma_f32_32x32x16_f16(bitcast<f16x8>(a), bitcast<f16x8>(b), c, 0, 0, 0);
+    else               return __builtin_amdgcn_mfma_f32_32x32x16_bf16(bitcast<bf16x8>(a), bitcast<bf16x8>(b), c, 0, 0, 0);
+}
+
+// f32 -> bf16 bits, round to nearest even, NaN quieted (ggml/src/ggml-impl.h:553-568)
+__device__ __forceinline__ unsigned int f32_to_bf16_bits(float f) {
+    unsigned int i = __float_as_uint(f);
+    if ((i & 0x7fffffffu) > 0x7f800000u) return (i >> 16) | 64u;
+    return (i + (0x7fffu + ((i >> 16) & 1u))) >> 16;
+}
+__device__ __forceinline__ unsigned int f32_to_f16_bits(float f) { return (unsigned int) bitcast<unsigned short>((_Float16) f); }
+__device__ __forceinline__ float        f16_bits_to_f32(unsigned int h) { return (float) bitcast<_Float16>((unsigned short) h); }
+
+template <bool F16> __device__ __forceinline__ unsigned int pack2(float a, float b) {
+    if constexpr (F16) return f32_to_f16_bits(a) | (f32_to_f16_bits(b) << 16);
+    else               return f32_to_bf16_bits(a) | (f32_to_bf16_bits(b) << 16);
+}
+template <bool F16> __device__ __forceinline__ float round_trip(float a) {
+    if constexpr (F16) return (float) (_Float16) a;
+    else               return __uint_as_float(f32_to_bf16_bits(a) << 16);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }  // v_exp_f32; exp2(-inf) = 0
+
+__device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); }
+
+
+// The pipelined decode kernel (mla_decode_kernel.hip); returns hipErrorInvalidValue for shapes it does not take.
+bool       decode_fast_applicable(const mla_attn_args * a);
+hipError_t launch_decode_fast(const KParams & kp, int kv_type, dim3 grid, hipStream_t st);
+size_t     decode_fast_lds_bytes();
+
+}  // namespace mla

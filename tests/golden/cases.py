@@ -1,0 +1,41 @@
+"""The golden cases: small seeded instances of each BASELINE config.  Inputs are regenerated from the seed
+(numpy default_rng); the fixture holds only a hash of the inputs and the reference's output."""
+import hashlib
+
+import numpy as np
+
+from oracle import oracle as O
+from tests import util as U
+
+CASES = {
+    # name: (k_type, n_seq, n_head, n_tok, n_kv, mask kind, seed)
+    "config1_f16_h16_kv1024": (O.TYPE_F16, 1, 16, 1, 1024, None, 1234),
+    "config2_bf16_h16_kv300": (O.TYPE_BF16, 2, 16, 1, 300, None, 2),
+    "config3_bf16_h128_kv256_sigma05": (O.TYPE_BF16, 1, 128, 1, 256, None, 3),
+    "config4_bf16_prefill_causal": (O.TYPE_BF16, 1, 16, 12, 76, "causal", 4),
+    "config5_q8_0_h128_kv200": (O.TYPE_Q8_0, 1, 128, 1, 200, None, 5),
+    "scattered_cells_mask": (O.TYPE_BF16, 1, 4, 3, 96, "random", 6),
+}
+
+
+def make_inputs(name):
+    k_type, n_seq, n_head, n_tok, n_kv, mask_kind, seed = CASES[name]
+    rng = np.random.default_rng(seed)
+    q = rng.standard_normal((n_seq, n_head, n_tok, 576)).astype(np.float32)
+    sigma = 0.5 if "sigma05" in name else 1.0
+    kf = (rng.standard_normal((n_seq, n_kv, 576)) * sigma).astype(np.float32)
+    k = U.encode_kv(kf, k_type, q8_scale=(1.0 / 32 if k_type == O.TYPE_Q8_0 else None))
+    mask = None
+    if mask_kind == "causal":
+        n_old = n_kv - n_tok
+        mask = np.where(np.arange(n_kv)[None, :] > n_old + np.arange(n_tok)[:, None], -np.inf, 0.0).astype(np.float16).view(np.uint16)
+    elif mask_kind == "random":
+        m = np.where(rng.random((n_tok, n_kv)) < 0.5, -np.inf, 0.0).astype(np.float16)
+        m[:, 0] = 0
+        mask = m.view(np.uint16)
+    h = hashlib.sha256()
+    h.update(q.tobytes())
+    h.update(k.tobytes())
+    if mask is not None:
+        h.update(mask.tobytes())
+    return dict(q=q, k=k, k_type=k_type, mask=mask, scale=U.SCALE, digest=h.hexdigest())

@@ -1,0 +1,105 @@
+"""The drop-in boundary without a GPU: the library loads, exports every symbol include/*.h declares, and its mirror
+of the reference's struct layouts / enum ordinals (jittorinfer_amd/csrc/ggml_abi.h) agrees with the real headers
+-- live against oracle/_ref when that is built, and always against the committed copy of the reference's table."""
+import ctypes as C
+import json
+import os
+import re
+
+import pytest
+
+from oracle import oracle as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+GOLDEN = os.path.join(ROOT, "tests", "golden", "ggml_abi_table.json")
+
+
+def _lib():
+    import jittorinfer_amd as J
+    return J.library()
+
+
+def _mirror_table():
+    lib = _lib()
+    name, val = C.c_char_p(), C.c_int64()
+    n = lib.mla_ggml_abi_table(-1, C.byref(name), C.byref(val))
+    out = {}
+    for i in range(n):
+        lib.mla_ggml_abi_table(i, C.byref(name), C.byref(val))
+        out[name.value.decode()] = val.value
+    return out
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib()
+    declared = set()
+    for hdr in ("mla_attn.h", "ggml_mla_backend.h"):
+        src = open(os.path.join(ROOT, "include", hdr)).read()
+        src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
+        declared |= set(re.findall(r"\b(mla_\w+|ggml_backend_\w+)\s*\(", src))
+    declared -= {"mla_attn_args", "mla_attn_plan_info"}
+    assert {"mla_attn_launch", "mla_attn_workspace_size", "ggml_backend_init", "ggml_backend_score"} <= declared
+    for sym in sorted(declared):
+        assert hasattr(lib, sym), "library does not export %s" % sym
+
+
+def test_mirror_matches_committed_reference_table():
+    golden = json.load(open(GOLDEN))
+    mirror = _mirror_table()
+    assert set(mirror) == set(golden)
+    bad = {k: (mirror[k], golden[k]) for k in golden if mirror[k] != golden[k]}
+    assert not bad, bad
+
+
+@pytest.mark.skipif(not O.ref_available(), reason="oracle/_ref is not built")
+def test_mirror_matches_live_reference_headers():
+    live = O.ref_abi_table()
+    mirror = _mirror_table()
+    assert live == mirror
+    assert live == json.load(open(GOLDEN))
+
+
+def test_args_struct_size_matches_header():
+    """ctypes mirror of mla_attn_args vs the C compiler's view of include/mla_attn.h."""
+    import subprocess
+    import tempfile
+    import jittorinfer_amd as J
+    src = '#include <stdio.h>\n#include <stddef.h>\n#include "mla_attn.h"\nint main(){printf("%zu %zu %zu %zu\\n", sizeof(mla_attn_args), offsetof(mla_attn_args, kv), offsetof(mla_attn_args, workspace), sizeof(mla_attn_plan_info));return 0;}\n'
+    with tempfile.TemporaryDirectory() as d:
+        c = os.path.join(d, "t.c")
+        open(c, "w").write(src)
+        exe = os.path.join(d, "t")
+        subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), c, "-o", exe], check=True)
+        out = subprocess.run([exe], check=True, stdout=subprocess.PIPE, text=True).stdout.split()
+    assert int(out[0]) == C.sizeof(J.MlaAttnArgs)
+    assert int(out[1]) == J.MlaAttnArgs.kv.offset
+    assert int(out[2]) == J.MlaAttnArgs.workspace.offset
+    assert int(out[3]) == C.sizeof(J.MlaPlanInfo)
+
+
+def test_argument_validation_without_gpu():
+    """Rejected arguments come back as negative codes before anything touches a device."""
+    import jittorinfer_amd as J
+    lib = _lib()
+    a = J.MlaAttnArgs()
+    assert lib.mla_attn_launch(C.byref(a), None) == -5          # null pointers
+    a.q, a.kv, a.dst = 4096, 8192, 16384
+    a.n_seq, a.n_head, a.n_tok, a.dk, a.dv = 1, 16, 1, 576, 512
+    a.kv_type, a.q_type = J.MLA_TYPE_BF16, J.MLA_TYPE_F32
+    a.q_nb1 = a.q_nb2 = a.q_nb3 = 2304
+    a.kv_nb1, a.n_kv, a.dst_nb1, a.scale = 1152, 256, 2304, 0.1
+    info = J.MlaPlanInfo()
+    assert lib.mla_attn_plan(C.byref(a), C.byref(info)) == 0 and info.n_splits >= 1
+    a.dk = 512
+    assert lib.mla_attn_plan(C.byref(a), C.byref(info)) == -1    # head size other than 576
+    a.dk, a.kv_type = 576, 2
+    assert lib.mla_attn_plan(C.byref(a), C.byref(info)) == -2    # unsupported KV type
+    a.kv_type, a.kv_nb1 = J.MLA_TYPE_BF16, 1150
+    assert lib.mla_attn_plan(C.byref(a), C.byref(info)) == -3    # misaligned rows
+    a.kv_nb1, a.max_bias = 1152, 1.0
+    assert lib.mla_attn_plan(C.byref(a), C.byref(info)) == -6    # ALiBi without a mask
+    a.max_bias = 0.0
+    a.n_splits = 4
+    assert lib.mla_attn_plan(C.byref(a), C.byref(info)) == 0
+    assert lib.mla_attn_launch(C.byref(a), None) == -4           # split-K needs a workspace
+    assert lib.ggml_backend_score() in (0, 100)
