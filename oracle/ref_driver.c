@@ -106,30 +106,43 @@ int ref_backend_flash_attn_ext(const char * so_path, int k_type, int64_t DK, int
     const int               paged = block_table != NULL;
     struct ggml_init_params ip    = { ggml_tensor_overhead() * 32 + ggml_graph_overhead() + 4096, NULL, true };
     struct ggml_context *   ctx   = ggml_init(ip);
-    if (!ctx) { ggml_backend_free(be); return -13; }
+    /* the KV rows live in their own context, allocated up front in the backend's buffer the way
+     * llama_kv_cache_init allocates k_l[il] (src/llama-kv-cache.cpp:82-90,153-158) */
+    struct ggml_init_params ipk    = { ggml_tensor_overhead() * 4, NULL, true };
+    struct ggml_context *   ctx_kv = ggml_init(ipk);
+    if (!ctx || !ctx_kv) { ggml_backend_free(be); return -13; }
 
     struct ggml_tensor * tq = ggml_new_tensor_4d(ctx, GGML_TYPE_F32, DK, n_tok, n_head, n3);
-    struct ggml_tensor * tk = ggml_new_tensor_4d(ctx, kt, DK, n_kv, 1, paged ? 1 : n3);
+    struct ggml_tensor * tk = ggml_new_tensor_4d(use_sched ? ctx_kv : ctx, kt, DK, n_kv, 1, paged ? 1 : n3);
     struct ggml_tensor * tv = tk;
     if (dv != DK) tv = ggml_view_4d(ctx, tk, dv, tk->ne[1], tk->ne[2], tk->ne[3], tk->nb[1], tk->nb[2], tk->nb[3], 0);
     struct ggml_tensor * tm = mask ? make_mask(ctx, mask_ne0, n_tok) : NULL;
     struct ggml_tensor * tb = paged ? ggml_new_tensor_2d(ctx, GGML_TYPE_I32, max_blocks, n3) : NULL;
     struct ggml_tensor * tl = paged ? ggml_new_tensor_1d(ctx, GGML_TYPE_I32, n3) : NULL;
-    ggml_set_input(tq); ggml_set_input(tk);
+    ggml_set_input(tq);
     if (tm) ggml_set_input(tm);
     if (tb) { ggml_set_input(tb); ggml_set_input(tl); }
-    struct ggml_tensor * o = ggml_flash_attn_ext(ctx, tq, tk, tv, tm, scale, max_bias, softcap);
+
+    int                   rc     = 0;
+    ggml_backend_buffer_t buf    = NULL;
+    ggml_backend_buffer_t buf_kv = NULL;
+    ggml_backend_sched_t  sched  = NULL;
+    ggml_backend_t        cpu    = NULL;
+    struct ggml_tensor *  o      = NULL;
+    struct ggml_cgraph *  gf     = NULL;
+
+    if (use_sched) {
+        buf_kv = ggml_backend_alloc_ctx_tensors(ctx_kv, be);
+        if (!buf_kv) { rc = -18; goto done; }
+        ggml_backend_buffer_clear(buf_kv, 0); /* src/llama-kv-cache.cpp:158 */
+    }
+    o = ggml_flash_attn_ext(ctx, tq, tk, tv, tm, scale, max_bias, softcap);
     ggml_flash_attn_ext_set_prec(o, GGML_PREC_F32);
     o->src[4] = tb; /* same slot convention as ggml_flash_attn_prompt's length tensors, ggml.c:2707-2710 */
     o->src[5] = tl;
     ggml_set_output(o);
-    struct ggml_cgraph * gf = ggml_new_graph(ctx);
+    gf = ggml_new_graph(ctx);
     ggml_build_forward_expand(gf, o);
-
-    int                   rc    = 0;
-    ggml_backend_buffer_t buf   = NULL;
-    ggml_backend_sched_t  sched = NULL;
-    ggml_backend_t        cpu   = NULL;
     if (!ggml_backend_dev_supports_op(dev, o)) { rc = -14; goto done; }
 
     if (use_sched) {
@@ -137,9 +150,13 @@ int ref_backend_flash_attn_ext(const char * so_path, int k_type, int64_t DK, int
         if (!cpu) { rc = -15; goto done; }
         ggml_backend_t backends[2] = { be, cpu };
         sched = ggml_backend_sched_new(backends, NULL, 2, GGML_DEFAULT_GRAPH_SIZE, false);
-        if (!sched || !ggml_backend_sched_alloc_graph(sched, gf)) { rc = -16; goto done; }
+        if (!sched) { rc = -16; goto done; }
+        /* llama's graph callback pins attention nodes to the layer's device the same way */
+        ggml_backend_sched_set_tensor_backend(sched, o, be);
+        if (!ggml_backend_sched_alloc_graph(sched, gf)) { rc = -16; goto done; }
         if (ggml_backend_sched_get_tensor_backend(sched, o) != be) { rc = -17; goto done; }
     } else {
+        ggml_set_input(tk);
         buf = ggml_backend_alloc_ctx_tensors(ctx, be);
         if (!buf) { rc = -18; goto done; }
     }
@@ -166,8 +183,10 @@ int ref_backend_flash_attn_ext(const char * so_path, int k_type, int64_t DK, int
 done:
     if (sched) ggml_backend_sched_free(sched);
     if (buf) ggml_backend_buffer_free(buf);
+    if (buf_kv) ggml_backend_buffer_free(buf_kv);
     if (cpu) ggml_backend_free(cpu);
     ggml_free(ctx);
+    ggml_free(ctx_kv);
     ggml_backend_free(be);
     return rc;
 }
