@@ -53,6 +53,9 @@ struct KParams {
     int             dv_total, d_off;
     float           scale, softcap, max_bias, m0, m1;
     int             n_head_log2;
+    int             c_log2_bits;   // bit pattern of scale * log2(e)
+    int             debug_flags;   // development builds of the decode kernel only
+    void *          debug_ptr;
     int             n_pool_pages;  // block-table mode: pages in the pool
     int             rows_contig;  // kv rows are packed (kv_nb1 == row bytes): whole tiles are one contiguous run
 };

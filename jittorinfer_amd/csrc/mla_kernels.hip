@@ -18,6 +18,8 @@
 // gfx950 only: v_mfma_f32_32x32x16_*, ds_read_b64_tr_b16, 160 KB LDS, 64-wide waves.
 
 #include "mla_common.hpp"
+#include <string.h>
+#include <stdlib.h>
 
 using namespace mla;
 
@@ -537,7 +539,7 @@ int make_plan(const mla_attn_args * a, Plan * pl) {
         pl->split_tokens = (int) max_len;
         return 0;
     }
-    if (decode_fast_applicable(a) && a->rows_per_wg == 0 && false) { pl->variant = 2; pl->n_passes = 1; pl->ndb = 16; pl->wm = 4; pl->wd = 1; }
+    if (decode_fast_applicable(a) && a->rows_per_wg == 0) { pl->variant = 2; pl->n_passes = 1; pl->ndb = 16; pl->wm = 4; pl->wd = 1; }
     else if (a->dv == 576) { pl->n_passes = 2; pl->ndb = 9; pl->wm = 4; pl->wd = 1; }
     else {
         pl->n_passes = 1; pl->ndb = 16;
@@ -558,6 +560,7 @@ int make_plan(const mla_attn_args * a, Plan * pl) {
         splits = (256 + wgs - 1) / wgs;
         if (pl->wd > 1) splits *= 2;  // small-row shapes leave room for two workgroups per CU
     }
+    if (pl->variant == 2 && splits * 64 < n_pages) splits = (n_pages + 63) / 64;  // that kernel indexes at most 64 pages per split
     if (splits > n_pages) splits = n_pages;
     if (splits < 1) splits = 1;
     const int64_t pages_per_split = (n_pages + splits - 1) / splits;
@@ -644,7 +647,9 @@ static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
     kp.n_head_log2 = 1 << (int) floor(log2((double) a->n_head));
     kp.m0 = powf(2.0f, -(a->max_bias) / kp.n_head_log2);
     kp.m1 = powf(2.0f, -(a->max_bias / 2.0f) / kp.n_head_log2);
+    { const float c = a->scale * LOG2E; memcpy(&kp.c_log2_bits, &c, 4); }
     kp.n_pool_pages = (int) (a->n_kv / MLA_PAGE_TOKENS);
+    if (const char * dbg = getenv("MLA_DEBUG")) { kp.debug_flags = atoi(dbg); kp.debug_ptr = a->dst; }
     kp.rows_contig = a->kv_nb1 == (a->kv_type == MLA_TYPE_Q8_0 ? Q8_ROW : ROW_BYTES) && (((uintptr_t) a->kv & 15) == 0) &&
                      (a->block_table || (a->kv_nb3 & 15) == 0);
     char * ws = (char *) a->workspace;
