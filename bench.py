@@ -132,22 +132,22 @@ def main():
     wall = time.perf_counter() - t0
     ms_per_step = wall * 1e3 / a.steps
 
-    # ---- the dominant kernel alone (the split-K decode kernel), HIP events on the launch stream around each launch
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(a.steps)]
+    # ---- the dominant kernel alone (the split-K decode kernel): HIP events on the launch stream around K back-to-back
+    # launches (the stream is in order, so this is K kernel durations plus the gaps between them)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
     for i in range(a.steps):
-        evs[i][0].record(stream)
         step(i, lib.mla_attn_launch_partials)
-        evs[i][1].record(stream)
+    e1.record(stream)
     torch.cuda.synchronize()
-    durs = sorted(e0.elapsed_time(e1) for e0, e1 in evs)
-    kern_ms = sum(durs) / len(durs)
+    kern_ms = e0.elapsed_time(e1) / a.steps
     # and whole steps with events (decode + combine)
+    e0.record(stream)
     for i in range(a.steps):
-        evs[i][0].record(stream)
         step(i)
-        evs[i][1].record(stream)
+    e1.record(stream)
     torch.cuda.synchronize()
-    sdurs = sorted(e0.elapsed_time(e1) for e0, e1 in evs)
+    step_ms_events = e0.elapsed_time(e1) / a.steps
 
     kv_bytes = a.batch * a.ctx * KV_ROW_BYTES
     flops = a.batch * a.ctx * a.heads * FLOP_PER_TOKEN_HEAD
@@ -169,13 +169,13 @@ def main():
         "config": {"workload": "BASELINE configs[2]: paged MLA decode B=%d H=%d ctx=%d, bf16 latent KV 576/512, 128-token pages, shuffled block table" % (a.batch, a.heads, a.ctx),
                    "batch": a.batch, "heads": a.heads, "ctx": a.ctx, "kv_pools_rotated": a.pools, "plan": plan},
         "us_per_step": ms_per_step * 1e3,
-        "us_per_step_events": {"median": sdurs[len(sdurs) // 2] * 1e3, "p10": sdurs[len(sdurs) // 10] * 1e3, "p90": sdurs[(len(sdurs) * 9) // 10] * 1e3},
+        "us_per_step_events": step_ms_events * 1e3,
         "tokens_per_s": a.batch / (ms_per_step * 1e-3),
         "pct_hbm_peak": 100.0 * value / HBM_PEAK_GBPS,
         "tflops": flops / (ms_per_step * 1e-3) / 1e12,
         "roofline": {"bound": "hbm", "kernel": "mla_attn_tile_kernel<bf16,16,4,1>", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
-                     "algorithmic_bytes_per_launch": kv_bytes, "kernel_us": {"mean": kern_ms * 1e3, "median": durs[len(durs) // 2] * 1e3},
+                     "algorithmic_bytes_per_launch": kv_bytes, "kernel_us": {"mean": kern_ms * 1e3},
                      "mfma_tflops": flops / (kern_ms * 1e-3) / 1e12},
         "cpu_baseline": cpu,
         "parity": parity,

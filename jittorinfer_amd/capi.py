@@ -31,7 +31,8 @@ class MlaPlanInfo(C.Structure):
 
 
 def library_path():
-    return os.path.join(HERE, "libggml-hip-mla.so")
+    # JITTORINFER_AMD_LIB: development override (an experimental build of the same library)
+    return os.environ.get("JITTORINFER_AMD_LIB") or os.path.join(HERE, "libggml-hip-mla.so")
 
 
 _lib = None

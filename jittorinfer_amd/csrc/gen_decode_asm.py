@@ -16,6 +16,12 @@ Register roles of S_cur/S_next swap every tile, so the loop body is emitted twic
 import sys
 
 DEBUG = "--debug" in sys.argv
+NO_LOOP_DMA = "--no-loop-dma" in sys.argv   # timing experiments only (wrong results)
+NO_PV = "--no-pv" in sys.argv
+NO_QK = "--no-qk" in sys.argv
+NO_SM = "--no-softmax" in sys.argv
+NO_STORE = "--no-store" in sys.argv
+NO_QLOAD = "--no-qload" in sys.argv
 F16 = "--f16" in sys.argv  # f16 KV: f16 MFMA, single P (no lo half)
 MF = "v_mfma_f32_32x32x16_f16" if F16 else "v_mfma_f32_32x32x16_bf16"
 CVT = "v_cvt_pk_f16_f32" if F16 else "v_cvt_pk_bf16_f32"
@@ -23,7 +29,9 @@ SPLIT = not F16
 
 PITCH = 1168
 TILE_BYTES = 32 * PITCH
-HOFF = 3 * TILE_BYTES          # hand-off area written by the C++ prologue: 32 bytes per thread
+NBUF = 4
+HOFF = NBUF * TILE_BYTES       # hand-off area written by the C++ prologue: 32 bytes per thread
+DMA_PER_TILE = 10              # LDS-DMA instructions each wave issues per tile
 CPR = 73                       # 16-byte chunks per padded row
 WAVE_CHUNKS = 8 * CPR          # 584: each wave moves rows 8w..8w+7 of a tile
 TAU = 8.0
@@ -45,7 +53,7 @@ DBG, TIDR = 230, 248   # debug builds only: T[6:7] holds the debug pointer until
 # ---- SGPR map (all inside the clobbered range s40..s79)
 KV, BT, KVB, KVE, CL2, NPP, NB1, FLG = 40, 42, 44, 45, 46, 47, 48, 49
 NT, IT, OFF0, OFF1, OFF2, WAVE, TB, TMP, NVM1 = 50, 51, 52, 53, 54, 55, 56, 58, 59
-EXS, S0, S1, S2, S3, DMAB, NVAL, THR, PG0, RSC, SPITCH, SCLS = 60, 62, 63, 64, 65, 66, 67, 68, 69, 70, 72, 73
+EXS, S0, S1, S2, S3, DMAB, NVAL, THR, PG0, RSC, SPITCH, SCLS, OFF3, VMW, OSTR = 60, 62, 63, 64, 65, 66, 67, 68, 69, 70, 72, 73, 74, 75, 76
 
 out = []
 uid = [0]
@@ -175,6 +183,8 @@ def dma_tile_lines(tile_sreg, off_sreg):
 
 def qk_slots(sreg, kaddr):
     """36 MFMA slots of S = K.Q^T into v[sreg:sreg+15]; K fragments come through a ring of 4."""
+    if NO_QK:
+        return [(lambda: None) for _ in range(36)]
     slots = []
     depth = 3
 
@@ -198,6 +208,8 @@ def qk_slots(sreg, kaddr):
 
 def softmax_part1(sreg):
     """tile max -> TMAX (log2 units), uniform test whether any row's max moved by more than TAU."""
+    if NO_SM:
+        return ["s_mov_b64 %s, 0" % s(RSC, 2)]
     L = []
     m = [T[0], T[1], T[2], T[3], T[4]]
     L.append("v_max3_f32 %s, %s, %s, %s" % (v(m[0]), v(sreg + 0), v(sreg + 1), v(sreg + 2)))
@@ -246,6 +258,8 @@ def rescale_block(ret_label):
 
 
 def softmax_part2(sreg):
+    if NO_SM:
+        return []
     L = []
     # p = 2^(s*c - m)
     for k in range(16):
@@ -337,12 +351,16 @@ def half_iteration(s_cur, s_next, tag):
     e("v_add_u32 %s, %s, %s" % (v(KADDR), s(OFF1), v(KADDR_LANE)))
     e("v_add_u32 %s, %s, %s" % (v(VADDR), s(OFF0), v(VADDR_LANE)))
     slots = qk_slots(s_next, KADDR)
-    # DMA of tile IT+2 (skipped when it does not exist)
-    e("s_add_u32 %s, %s, 2" % (s(TMP), s(IT)))
+    # DMA of tile IT+3 (skipped when it does not exist)
+    e("s_add_u32 %s, %s, 3" % (s(TMP), s(IT)))
+    e("s_mov_b32 %s, 0" % s(VMW))
     lab_nodma, lab_after = label("nodma"), label("afterdma")
     e("s_cmp_ge_u32 %s, %s" % (s(TMP), s(NT)))
     e("s_cbranch_scc1 %s" % lab_nodma)
-    dma = dma_tile_lines(TMP, OFF2)
+    if NO_LOOP_DMA:
+        e("s_branch %s" % lab_nodma)
+    e("s_mov_b32 %s, 1" % s(VMW))
+    dma = dma_tile_lines(TMP, OFF3)
     # part 1 of the softmax + DMA issue share the first MFMA slots
     p1 = softmax_part1(s_cur)
     n1 = 8
@@ -376,15 +394,25 @@ def half_iteration(s_cur, s_next, tag):
     e("%s:" % lab_after)
     assert not lds.pending and not saved
     # ---- PV of tile IT
-    pv_phase(VADDR)
+    if not NO_PV:
+        pv_phase(VADDR)
     lds.drain()
-    # ---- end of tile: all DMA of tile IT+2 landed, everyone done with tile IT
+    # ---- end of tile: the DMA of tile IT+2 has landed (the one of tile IT+3, issued in this iteration, may still be
+    # in flight: loads complete in order, so vmcnt(DMA_PER_TILE) is enough); everyone is done with tile IT
+    lab_w0, lab_wd = label("w0"), label("wd")
+    e("s_cmp_eq_u32 %s, 0" % s(VMW))
+    e("s_cbranch_scc1 %s" % lab_w0)
+    e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
+    e("s_branch %s" % lab_wd)
+    e("%s:" % lab_w0)
     e("s_waitcnt vmcnt(0)")
+    e("%s:" % lab_wd)
     e("s_barrier")
     e("s_mov_b32 %s, %s" % (s(TMP), s(OFF0)))
     e("s_mov_b32 %s, %s" % (s(OFF0), s(OFF1)))
     e("s_mov_b32 %s, %s" % (s(OFF1), s(OFF2)))
-    e("s_mov_b32 %s, %s" % (s(OFF2), s(TMP)))
+    e("s_mov_b32 %s, %s" % (s(OFF2), s(OFF3)))
+    e("s_mov_b32 %s, %s" % (s(OFF3), s(TMP)))
     e("s_add_u32 %s, %s, 1" % (s(IT), s(IT)))
     return (lab_resc, lab_back), (lab_resc2, lab_back2)
 
@@ -400,6 +428,7 @@ def main():
     e("s_mov_b32 %s, %%[nb1]" % s(NB1))
     e("s_mov_b32 %s, %%[flg]" % s(FLG))
     e("s_mov_b32 %s, %%[ntl]" % s(NT))
+    e("s_mov_b32 %s, %%[ostr]" % s(OSTR))
     e("v_mov_b32 %s, %%[tid]" % v(X0))
     if DEBUG:
         e("v_mov_b32 %s, %s" % (v(TIDR), v(X0)))
@@ -433,18 +462,6 @@ def main():
     e("v_lshlrev_b32 %s, 3, %s" % (v(X2), v(X2)))                      # *4 elements *2 bytes
     e("v_add_u32 %s, %s, %s" % (v(X1), v(X1), v(X2)))
     e("v_mad_u32_u24 %s, %s, %s, %s" % (v(VADDR_LANE), v(X0), s(SPITCH), v(X1)))
-    # ------------------------------------------------------------------ Q -> v[0:143] (q pointer already includes the 8*g float offset)
-    qp = T[0]  # T[0:1] still holds the q pointer
-    for grp in range(9):
-        for k in range(4):
-            ks = grp * 4 + k
-            e("global_load_dwordx4 %s, %s, off offset:%d" % (v(SA + 8 * k, 4), v(qp, 2), ks * 64))
-            e("global_load_dwordx4 %s, %s, off offset:%d" % (v(SA + 8 * k + 4, 4), v(qp, 2), ks * 64 + 16))
-        e("s_waitcnt vmcnt(0)")
-        for k in range(4):
-            ks = grp * 4 + k
-            for j in range(4):
-                e("%s %s, %s, %s" % (CVT, v(Q0 + 4 * ks + j), v(SA + 8 * k + 2 * j), v(SA + 8 * k + 2 * j + 1)))
     # ------------------------------------------------------------------ page ids of this split -> one lane each
     lab_nobt = label("nobt")
     e("s_lshr_b32 %s, %s, 7" % (s(PG0), s(KVB)))
@@ -467,32 +484,60 @@ def main():
     e("v_min_i32 %s, %s, %s" % (v(PAGES), s(NPP), v(PAGES)))
     e("%s:" % lab_nobt)
     # ------------------------------------------------------------------ state
-    for i in range(256):
-        e("v_accvgpr_write_b32 %s, 0" % a(i))
     e("v_mov_b32 %s, 0xff800000" % v(MRUN))
     e("v_mov_b32 %s, 0" % v(LRUN))
-    if "--swapbuf" in sys.argv:
-        e("s_mov_b32 %s, %d" % (s(OFF0), 2 * TILE_BYTES))
-        e("s_mov_b32 %s, %d" % (s(OFF1), TILE_BYTES))
-        e("s_mov_b32 %s, 0" % s(OFF2))
-    else:
-        e("s_mov_b32 %s, 0" % s(OFF0))
-        e("s_mov_b32 %s, %d" % (s(OFF1), TILE_BYTES))
-        e("s_mov_b32 %s, %d" % (s(OFF2), 2 * TILE_BYTES))
+    e("s_mov_b32 %s, 0" % s(OFF0))
+    e("s_mov_b32 %s, %d" % (s(OFF1), TILE_BYTES))
+    e("s_mov_b32 %s, %d" % (s(OFF2), 2 * TILE_BYTES))
+    e("s_mov_b32 %s, %d" % (s(OFF3), 3 * TILE_BYTES))
     e("s_mov_b32 %s, 0" % s(IT))
     # ------------------------------------------------------------------ prologue: tiles 0 and 1, S of tile 0
     e("s_mov_b32 %s, 0" % s(TMP))
     for ln in dma_tile_lines(TMP, OFF0):
         e(ln)
     lab_one = label("one")
+    lab_three, lab_pw = label("three"), label("pw")
     e("s_cmp_lt_u32 %s, 2" % s(NT))
     e("s_cbranch_scc1 %s" % lab_one)
     e("s_mov_b32 %s, 1" % s(TMP))
     for ln in dma_tile_lines(TMP, OFF1):
         e(ln)
+    e("s_cmp_lt_u32 %s, 3" % s(NT))
+    e("s_cbranch_scc1 %s" % lab_one)
+    e("s_mov_b32 %s, 2" % s(TMP))
+    for ln in dma_tile_lines(TMP, OFF2):
+        e(ln)
     e("%s:" % lab_one)
-    e("s_waitcnt vmcnt(0)")
+    # ------------------------------------------------------------------ Q -> v[0:143] (q pointer already includes the 8*g float offset)
+    # All 72 loads are issued back to back behind the tile DMAs (one latency instead of nine): k-steps 0..31 land in
+    # the 256 accumulator registers (not yet in use), k-steps 32..35 in v[144:175].
+    qp = T[0]  # T[0:1] still holds the q pointer
+    for ks in range(0 if NO_QLOAD else 36, 0):
+        pass
+    if not NO_QLOAD:
+        for ks in range(32):
+            e("global_load_dwordx4 %s, %s, off offset:%d" % (a(8 * ks, 4), v(qp, 2), ks * 64))
+            e("global_load_dwordx4 %s, %s, off offset:%d" % (a(8 * ks + 4, 4), v(qp, 2), ks * 64 + 16))
+        for k in range(4):
+            ks = 32 + k
+            e("global_load_dwordx4 %s, %s, off offset:%d" % (v(SA + 8 * k, 4), v(qp, 2), ks * 64))
+            e("global_load_dwordx4 %s, %s, off offset:%d" % (v(SA + 8 * k + 4, 4), v(qp, 2), ks * 64 + 16))
+        e("s_waitcnt vmcnt(0)")
+        for ks in range(32):
+            for j in range(4):
+                e("v_accvgpr_read_b32 %s, %s" % (v(T[2]), a(8 * ks + 2 * j)))
+                e("v_accvgpr_read_b32 %s, %s" % (v(T[3]), a(8 * ks + 2 * j + 1)))
+                e("s_nop 0")
+                e("%s %s, %s, %s" % (CVT, v(Q0 + 4 * ks + j), v(T[2]), v(T[3])))
+        for k in range(4):
+            ks = 32 + k
+            for j in range(4):
+                e("%s %s, %s, %s" % (CVT, v(Q0 + 4 * ks + j), v(SA + 8 * k + 2 * j), v(SA + 8 * k + 2 * j + 1)))
+    # the Q loads were issued after every tile DMA and are complete (vmcnt(0) above): all prologue tiles are in
     e("s_barrier")
+    # accumulators start at zero (they were the landing zone of the Q loads)
+    for i in range(256):
+        e("v_accvgpr_write_b32 %s, 0" % a(i))
     if DEBUG:
         # FLG bit 1: dump LDS tile 0 (2336 chunks) to the debug pointer and stop
         lab = label("nodump1")
@@ -564,10 +609,7 @@ def main():
     e("s_nop 1")
     e("v_add_f32 %s, %s, %s" % (v(LRUN), v(T[0]), v(T[1])))
     # scale: 1/l when this launch writes the final output, 1 otherwise
-    e("v_mov_b32 %s, 1.0" % v(T[2]))
     lab_part = label("part")
-    e("s_cmp_eq_u32 %s, 0" % s(FLG))
-    e("s_cbranch_scc1 %s" % lab_part)
     e("v_rcp_f32 %s, %s" % (v(T[2]), v(LRUN)))
     # one Newton step: r = r * (2 - l*r)   (keeps the quotient within 1 ulp; l = 0 still gives inf/NaN)
     e("s_nop 0")
@@ -583,7 +625,15 @@ def main():
     e("s_mov_b64 %s, exec" % s(EXS, 2))
     e("s_nop 1")
     e("s_and_b64 exec, exec, vcc")
-    # O^T block i, element 4j+c is column 32 i + 8 j + 4 g + c; the out pointer already includes the 4*g float offset
+    # O^T block i, element 4j+c is column 32 i + 8 j + 4 g + c.
+    # Final output (FLG bit 0): row-major rows of dst; the out pointer already includes the 4*g float offset.
+    # Split-K partial: layout [column/4][row][4 floats] so that the 32 lanes of a half-wave write 512 contiguous bytes;
+    # the out pointer already includes (g*n_rows + row)*16 bytes and every (i, j) step advances it by 2*n_rows*16 bytes.
+    lab_pstore, lab_sdone = label("pstore"), label("sdone")
+    if NO_STORE:
+        e("s_branch %s" % lab_sdone)
+    e("s_bitcmp1_b32 %s, 0" % s(FLG))
+    e("s_cbranch_scc0 %s" % lab_pstore)
     for i in range(16):
         for j in range(4):
             r = T[4] if (i * 4 + j) % 2 == 0 else SA  # alternate two 4-register staging groups
@@ -592,6 +642,24 @@ def main():
             for c in range(4):
                 e("v_mul_f32 %s, %s, %s" % (v(r + c), v(r + c), v(T[2])))
             e("global_store_dwordx4 %s, %s, off offset:%d" % (v(OPTR, 2), v(r, 4), (32 * i + 8 * j) * 4))
+    e("s_branch %s" % lab_sdone)
+    e("%s:" % lab_pstore)
+    # partial: O / l of this split as f16, layout [column/4][row][4 halves]; T[2] holds 1/l here as well
+    for i in range(16):
+        for j in range(4):
+            r = T[4] if (i * 4 + j) % 2 == 0 else SA
+            for c in range(4):
+                e("v_accvgpr_read_b32 %s, %s" % (v(r + c), a(16 * i + 4 * j + c)))
+            for c in range(4):
+                e("v_mul_f32 %s, %s, %s" % (v(r + c), v(r + c), v(T[2])))
+            e("v_cvt_pk_f16_f32 %s, %s, %s" % (v(r), v(r), v(r + 1)))
+            e("v_cvt_pk_f16_f32 %s, %s, %s" % (v(r + 1), v(r + 2), v(r + 3)))
+            e("s_nop 0")
+            e("global_store_dwordx2 %s, %s, off" % (v(OPTR, 2), v(r, 2)))
+            e("v_add_co_u32 %s, vcc, %s, %s" % (v(OPTR), s(OSTR), v(OPTR)))
+            e("s_nop 1")
+            e("v_addc_co_u32 %s, vcc, 0, %s, vcc" % (v(OPTR + 1), v(OPTR + 1)))
+    e("%s:" % lab_sdone)
     # (m, l) of this split, written by the g == 0 lane of each row when a pointer was handed over
     e("v_cmp_ne_u64 vcc, 0, %s" % v(MLPTR, 2))
     e("s_nop 1")

@@ -368,14 +368,18 @@ __global__ void __launch_bounds__(NTHREADS) mla_attn_tile_kernel(const KParams p
                 *(f32x4 *) (o + (wd * NDBW + i) * 32 + 8 * j + 4 * g) = v;
             }
     } else {
-        const int64_t prow = ((int64_t) b * p.n_splits + split) * p.n_rows + row;
-        float * o = p.part_o + prow * p.dv_total + p.d_off;
+        const int64_t prow   = ((int64_t) b * p.n_splits + split) * p.n_rows + row;
+        const int64_t pblock = ((int64_t) b * p.n_splits + split) * p.n_rows * p.dv_total;
+        // partial = O / l of this split, stored as f16 in layout [column/4][row][4]: coalesced for the writers here and
+        // for the combine pass, and half the bytes of f32 (the 2^-11 rounding is averaged over the splits)
+        const float pinv = 1.0f / l_tot;
 #pragma unroll
         for (int i = 0; i < NDBW; i++)
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                f32x4 v = { acc[i][4 * j], acc[i][4 * j + 1], acc[i][4 * j + 2], acc[i][4 * j + 3] };
-                *(f32x4 *) (o + (wd * NDBW + i) * 32 + 8 * j + 4 * g) = v;
+                const int d0 = p.d_off + (wd * NDBW + i) * 32 + 8 * j + 4 * g;
+                u32x2 v = { pack2<true>(acc[i][4 * j] * pinv, acc[i][4 * j + 1] * pinv), pack2<true>(acc[i][4 * j + 2] * pinv, acc[i][4 * j + 3] * pinv) };
+                *(u32x2 *) (p.part_o + pblock + ((int64_t) (d0 >> 2) * p.n_rows + row) * 4) = v;
             }
         if (wd == 0 && g == 0 && p.d_off == 0) {
             p.part_ml[prow * 2]     = m_run;
@@ -384,31 +388,40 @@ __global__ void __launch_bounds__(NTHREADS) mla_attn_tile_kernel(const KParams p
     }
 }
 
-// Log-sum-exp merge of the split-K partials: out = sum_c O_c 2^(m_c - M) / sum_c l_c 2^(m_c - M).
-// grid = (n_rows, n_seq), block = dv_total / 4 threads (one float4 column group each).
-__global__ void mla_attn_combine_kernel(const KParams p) {
-    const int row = blockIdx.x, b = blockIdx.y;
+// Log-sum-exp merge of the split-K partials: out = sum_c (O_c/l_c) l_c 2^(m_c - M) / sum_c l_c 2^(m_c - M).
+// Partials hold O_c/l_c as f16, laid out [seq][split][column/4][row][4].  One thread = one (row, group of 4 columns);
+// a block is 32 rows x 8 column groups, so each load instruction of a wave reads runs of 256 contiguous bytes and
+// each output row segment written by the block is 128 contiguous bytes.
+// grid = (ceil(n_rows/32), ceil(dv/32), n_seq), block = 256.
+__global__ void __launch_bounds__(256) mla_attn_combine_kernel(const KParams p) {
+    const int b = blockIdx.z;
+    const int row = blockIdx.x * 32 + (threadIdx.x & 31);
+    const int cg  = blockIdx.y * 8 + (threadIdx.x >> 5);
+    if (row >= p.n_rows || cg * 4 >= p.dv_total) return;
     const int seq_len = p.block_table ? min(p.seq_lens[b], (int) p.bt_stride * MLA_PAGE_TOKENS) : (int) p.n_kv;
     int nvalid = (seq_len + p.split_tokens - 1) / p.split_tokens;
     nvalid = min(nvalid, p.n_splits);
-    const int d4 = threadIdx.x;
+
+    const float *    ml = p.part_ml + ((int64_t) b * p.n_splits * p.n_rows + row) * 2;
+    const _Float16 * po = p.part_o + (int64_t) b * p.n_splits * p.n_rows * p.dv_total + ((int64_t) cg * p.n_rows + row) * 4;
+    const int64_t ml_step = (int64_t) p.n_rows * 2, po_step = (int64_t) p.n_rows * p.dv_total;
+
     float M = -INFINITY;
-    for (int c = 0; c < nvalid; c++) M = fmaxf(M, p.part_ml[(((int64_t) b * p.n_splits + c) * p.n_rows + row) * 2]);
+    for (int c = 0; c < nvalid; c++) M = fmaxf(M, ml[c * ml_step]);
     const float Mu = (M == -INFINITY) ? 0.f : M;
     float L = 0.f;
     f32x4 o = { 0.f, 0.f, 0.f, 0.f };
     for (int c = 0; c < nvalid; c++) {
-        const int64_t prow = ((int64_t) b * p.n_splits + c) * p.n_rows + row;
-        const float mc = p.part_ml[prow * 2];
+        const float mc = ml[c * ml_step];
         if (mc == -INFINITY) continue;  // that split saw only masked keys
-        const float w = fast_exp2(mc - Mu);
-        L += p.part_ml[prow * 2 + 1] * w;
-        const f32x4 v = *(const f32x4 *) (p.part_o + prow * p.dv_total + d4 * 4);
-        o.x += v.x * w; o.y += v.y * w; o.z += v.z * w; o.w += v.w * w;
+        const float w = ml[c * ml_step + 1] * fast_exp2(mc - Mu);  // l_c 2^(m_c - M)
+        L += w;
+        const u32x2 hv = *(const u32x2 *) (po + c * po_step);
+        o.x += f16_bits_to_f32(hv.x & 0xffff) * w; o.y += f16_bits_to_f32(hv.x >> 16) * w;
+        o.z += f16_bits_to_f32(hv.y & 0xffff) * w; o.w += f16_bits_to_f32(hv.y >> 16) * w;
     }
-    const float inv = 1.0f / L;
-    f32x4 r = { o.x * inv, o.y * inv, o.z * inv, o.w * inv };
-    *(f32x4 *) (p.dst + ((int64_t) b * p.n_rows + row) * p.dst_stride + d4 * 4) = r;
+    const float inv = 1.0f / L;  // no valid key at all: 0 * inf = NaN, like the reference
+    *(f32x4 *) (p.dst + ((int64_t) b * p.n_rows + row) * p.dst_stride + cg * 4) = f32x4{ o.x * inv, o.y * inv, o.z * inv, o.w * inv };
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -568,7 +581,7 @@ int make_plan(const mla_attn_args * a, Plan * pl) {
     pl->n_splits     = (int) ((n_pages + pages_per_split - 1) / pages_per_split);
     pl->lds_bytes    = pl->variant == 2 ? decode_fast_lds_bytes() : 2 * TILE_BYTES + (a->kv_type == MLA_TYPE_Q8_0 ? Q8_TILE_RAW : 0);
     if (pl->n_splits > 1) {
-        pl->ws_part_o  = (size_t) a->n_seq * pl->n_splits * n_rows * a->dv * sizeof(float);
+        pl->ws_part_o  = (size_t) a->n_seq * pl->n_splits * n_rows * a->dv * sizeof(_Float16);
         pl->ws_part_ml = (size_t) a->n_seq * pl->n_splits * n_rows * 2 * sizeof(float);
     }
     return 0;
@@ -653,7 +666,7 @@ static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
     kp.rows_contig = a->kv_nb1 == (a->kv_type == MLA_TYPE_Q8_0 ? Q8_ROW : ROW_BYTES) && (((uintptr_t) a->kv & 15) == 0) &&
                      (a->block_table || (a->kv_nb3 & 15) == 0);
     char * ws = (char *) a->workspace;
-    kp.part_o  = (float *) ws;
+    kp.part_o  = (_Float16 *) ws;
     kp.part_ml = (float *) (ws + align256(pl.ws_part_o));
     float * scores = (float *) (ws + align256(pl.ws_part_o) + align256(pl.ws_part_ml));
 
@@ -683,8 +696,8 @@ static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
         if (e != hipSuccess) return (int) e;
     }
     if (pl.n_splits > 1 && (phases & 2)) {
-        dim3 g((unsigned) kp.n_rows, (unsigned) a->n_seq);
-        hipLaunchKernelGGL(mla_attn_combine_kernel, g, dim3(a->dv / 4), 0, st, kp);
+        dim3 g((unsigned) ((kp.n_rows + 31) / 32), (unsigned) ((a->dv + 31) / 32), (unsigned) a->n_seq);
+        hipLaunchKernelGGL(mla_attn_combine_kernel, g, dim3(256), 0, st, kp);
         return (int) hipGetLastError();
     }
     return 0;
