@@ -23,7 +23,7 @@ KV_ROW_BYTES = 1152     # 576 bf16
 FLOP_PER_TOKEN_HEAD = 2 * 576 + 2 * 512
 
 
-def build_workload(dev, n_seq, n_head, ctx, n_pools, seed):
+def build_workload(dev, n_seq, n_head, ctx, n_pools, seed, kv="bf16"):
     import torch
     g = torch.Generator(device=dev)
     g.manual_seed(seed)
@@ -32,7 +32,7 @@ def build_workload(dev, n_seq, n_head, ctx, n_pools, seed):
     pools = []
     for _ in range(n_pools):
         kf = torch.randn((n_pages * 128, 576), generator=g, device=dev, dtype=torch.float32) * 0.5
-        pools.append(kf.to(torch.bfloat16))
+        pools.append(kf.to(torch.bfloat16 if kv == "bf16" else torch.float16))
         del kf
     perm = torch.randperm(n_pages, generator=g, device=dev).to(torch.int32)
     block_table = perm.reshape(n_seq, pages_per_seq).contiguous()
@@ -88,6 +88,7 @@ def main():
     ap.add_argument("--rows-per-wg", type=int, default=0)
     ap.add_argument("--cpu-seqs", type=int, default=8, help="sequences of the workload timed on the host cores (0 = skip)")
     ap.add_argument("--seed", type=int, default=1234)
+    ap.add_argument("--kv", default="bf16", choices=["bf16", "f16"], help="storage type of the latent KV pool (the headline config is bf16)")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this build measures one GPU's share of the path; --gpus %d is not supported (use --gpus 1)" % a.gpus, file=sys.stderr)
@@ -102,16 +103,17 @@ def main():
     dev = torch.device("cuda:0")
     scale = 1.0 / (192.0 ** 0.5)
 
-    q, pools, block_table, seq_lens = build_workload(dev, a.batch, a.heads, a.ctx, a.pools, a.seed)
+    q, pools, block_table, seq_lens = build_workload(dev, a.batch, a.heads, a.ctx, a.pools, a.seed, a.kv)
+    kv_type = J.MLA_TYPE_BF16 if a.kv == "bf16" else J.MLA_TYPE_F16
     out = torch.empty((a.batch, 1, a.heads, 576), dtype=torch.float32, device=dev)
     args = []
     keep = []
     for pool in pools:
-        ar, _, k = J.capi.make_args(q, pool.view(torch.int16), J.MLA_TYPE_BF16, dv=512, scale=scale, block_table=block_table,
+        ar, _, k = J.capi.make_args(q, pool.view(torch.int16), kv_type, dv=512, scale=scale, block_table=block_table,
                                     seq_lens=seq_lens, out=out, n_splits=a.splits, rows_per_wg=a.rows_per_wg)
         args.append(ar)
         keep.append(k)
-    plan = J.plan(q, pools[0].view(torch.int16), J.MLA_TYPE_BF16, dv=512, scale=scale, block_table=block_table, seq_lens=seq_lens, out=out, n_splits=a.splits, rows_per_wg=a.rows_per_wg)
+    plan = J.plan(q, pools[0].view(torch.int16), kv_type, dv=512, scale=scale, block_table=block_table, seq_lens=seq_lens, out=out, n_splits=a.splits, rows_per_wg=a.rows_per_wg)
     stream = torch.cuda.current_stream(dev)
     st = C.c_void_p(stream.cuda_stream)
 
@@ -165,7 +167,7 @@ def main():
         "metric": "mla_paged_decode_kv_read_bandwidth", "value": value, "unit": "GB/s",
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic",
+        "dtype": a.kv, "data": "synthetic",
         "config": {"workload": "BASELINE configs[2]: paged MLA decode B=%d H=%d ctx=%d, bf16 latent KV 576/512, 128-token pages, shuffled block table" % (a.batch, a.heads, a.ctx),
                    "batch": a.batch, "heads": a.heads, "ctx": a.ctx, "kv_pools_rotated": a.pools, "plan": plan},
         "us_per_step": ms_per_step * 1e3,
@@ -173,7 +175,7 @@ def main():
         "tokens_per_s": a.batch / (ms_per_step * 1e-3),
         "pct_hbm_peak": 100.0 * value / HBM_PEAK_GBPS,
         "tflops": flops / (ms_per_step * 1e-3) / 1e12,
-        "roofline": {"bound": "hbm", "kernel": "mla_attn_tile_kernel<bf16,16,4,1>", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+        "roofline": {"bound": "hbm", "kernel": "mla_decode_kernel<%s>" % a.kv, "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
                      "algorithmic_bytes_per_launch": kv_bytes, "kernel_us": {"mean": kern_ms * 1e3},
                      "mfma_tflops": flops / (kern_ms * 1e-3) / 1e12},

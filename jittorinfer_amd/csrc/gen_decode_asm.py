@@ -20,6 +20,7 @@ NO_LOOP_DMA = "--no-loop-dma" in sys.argv   # timing experiments only (wrong res
 NO_PV = "--no-pv" in sys.argv
 NO_QK = "--no-qk" in sys.argv
 NO_SM = "--no-softmax" in sys.argv
+DMA_PLACE = "pv" if "--dma-pv" in sys.argv else "bulk" if "--dma-bulk" in sys.argv else "a"
 NO_STORE = "--no-store" in sys.argv
 NO_QLOAD = "--no-qload" in sys.argv
 F16 = "--f16" in sys.argv  # f16 KV: f16 MFMA, single P (no lo half)
@@ -53,7 +54,7 @@ DBG, TIDR = 230, 248   # debug builds only: T[6:7] holds the debug pointer until
 # ---- SGPR map (all inside the clobbered range s40..s79)
 KV, BT, KVB, KVE, CL2, NPP, NB1, FLG = 40, 42, 44, 45, 46, 47, 48, 49
 NT, IT, OFF0, OFF1, OFF2, WAVE, TB, TMP, NVM1 = 50, 51, 52, 53, 54, 55, 56, 58, 59
-EXS, S0, S1, S2, S3, DMAB, NVAL, THR, PG0, RSC, SPITCH, SCLS, OFF3, VMW, OSTR = 60, 62, 63, 64, 65, 66, 67, 68, 69, 70, 72, 73, 74, 75, 76
+EXS, S0, S1, S2, S3, DMAB, NVAL, THR, PG0, RSC, SPITCH, SCLS, OFF3, VMW, OSTR, QP = 60, 62, 63, 64, 65, 66, 67, 68, 69, 70, 72, 73, 74, 75, 76, 78
 
 out = []
 uid = [0]
@@ -304,9 +305,12 @@ def mask_tail(sreg):
     e("%s:" % lab)
 
 
-def pv_phase(vaddr):
-    """O^T += V^T.P^T: 16 d-blocks x 2 k-steps; fragment ring of 4; d-blocks in pairs so dependent MFMAs alternate."""
+def pv_phase(vaddr, extra=None):
+    """O^T += V^T.P^T: 16 d-blocks x 2 k-steps; fragment ring of 4; d-blocks in pairs so dependent MFMAs alternate.
+    `extra`: instruction lines spread evenly between the MFMA pairs (whole-slot groups only)."""
     frags = [(kk, db) for kk in range(2) for db in range(16)]
+    extra = list(extra or [])
+    per_pair = -(-len(extra) // 16)
 
     def rd(idx):
         kk, db = frags[idx]
@@ -336,6 +340,11 @@ def pv_phase(vaddr):
         else:
             if i1 + depth < 32:
                 rd(i1 + depth)
+        for _ in range(per_pair):
+            if extra:
+                e(extra.pop(0))
+    for ln in extra:
+        e(ln)
 
 
 def half_iteration(s_cur, s_next, tag):
@@ -361,6 +370,12 @@ def half_iteration(s_cur, s_next, tag):
         e("s_branch %s" % lab_nodma)
     e("s_mov_b32 %s, 1" % s(VMW))
     dma = dma_tile_lines(TMP, OFF3)
+    if DMA_PLACE != "a":
+        if DMA_PLACE == "bulk":
+            for ln in dma:
+                e(ln)
+        e("s_branch %s" % lab_nodma)   # the compute part is the DMA-free code below
+        dma = []
     # part 1 of the softmax + DMA issue share the first MFMA slots
     p1 = softmax_part1(s_cur)
     n1 = 8
@@ -395,7 +410,20 @@ def half_iteration(s_cur, s_next, tag):
     assert not lds.pending and not saved
     # ---- PV of tile IT
     if not NO_PV:
-        pv_phase(VADDR)
+        if DMA_PLACE == "pv":
+            # DMA of tile IT+3 issued from inside the PV phase (VALU is otherwise idle there)
+            lab_pvnodma, lab_pvdone = label("pvnodma"), label("pvdone")
+            e("s_cmp_eq_u32 %s, 0" % s(VMW))
+            e("s_cbranch_scc1 %s" % lab_pvnodma)
+            pv_phase(VADDR, dma_tile_lines(TMP, OFF3))
+            lds.drain()
+            e("s_branch %s" % lab_pvdone)
+            e("%s:" % lab_pvnodma)
+            pv_phase(VADDR)
+            lds.drain()
+            e("%s:" % lab_pvdone)
+        else:
+            pv_phase(VADDR)
     lds.drain()
     # ---- end of tile: the DMA of tile IT+2 has landed (the one of tile IT+3, issued in this iteration, may still be
     # in flight: loads complete in order, so vmcnt(DMA_PER_TILE) is enough); everyone is done with tile IT
@@ -429,6 +457,7 @@ def main():
     e("s_mov_b32 %s, %%[flg]" % s(FLG))
     e("s_mov_b32 %s, %%[ntl]" % s(NT))
     e("s_mov_b32 %s, %%[ostr]" % s(OSTR))
+    e("s_mov_b64 %s, %%[qp]" % s(QP, 2))
     e("v_mov_b32 %s, %%[tid]" % v(X0))
     if DEBUG:
         e("v_mov_b32 %s, %s" % (v(TIDR), v(X0)))
@@ -491,7 +520,9 @@ def main():
     e("s_mov_b32 %s, %d" % (s(OFF2), 2 * TILE_BYTES))
     e("s_mov_b32 %s, %d" % (s(OFF3), 3 * TILE_BYTES))
     e("s_mov_b32 %s, 0" % s(IT))
-    # ------------------------------------------------------------------ prologue: tiles 0 and 1, S of tile 0
+    for i in range(256):
+        e("v_accvgpr_write_b32 %s, 0" % a(i))
+    # ------------------------------------------------------------------ prologue: tiles 0, 1, 2, S of tile 0
     e("s_mov_b32 %s, 0" % s(TMP))
     for ln in dma_tile_lines(TMP, OFF0):
         e(ln)
@@ -508,36 +539,19 @@ def main():
     for ln in dma_tile_lines(TMP, OFF2):
         e(ln)
     e("%s:" % lab_one)
-    # ------------------------------------------------------------------ Q -> v[0:143] (q pointer already includes the 8*g float offset)
-    # All 72 loads are issued back to back behind the tile DMAs (one latency instead of nine): k-steps 0..31 land in
-    # the 256 accumulator registers (not yet in use), k-steps 32..35 in v[144:175].
-    qp = T[0]  # T[0:1] still holds the q pointer
-    for ks in range(0 if NO_QLOAD else 36, 0):
-        pass
-    if not NO_QLOAD:
-        for ks in range(32):
-            e("global_load_dwordx4 %s, %s, off offset:%d" % (a(8 * ks, 4), v(qp, 2), ks * 64))
-            e("global_load_dwordx4 %s, %s, off offset:%d" % (a(8 * ks + 4, 4), v(qp, 2), ks * 64 + 16))
-        for k in range(4):
-            ks = 32 + k
-            e("global_load_dwordx4 %s, %s, off offset:%d" % (v(SA + 8 * k, 4), v(qp, 2), ks * 64))
-            e("global_load_dwordx4 %s, %s, off offset:%d" % (v(SA + 8 * k + 4, 4), v(qp, 2), ks * 64 + 16))
-        e("s_waitcnt vmcnt(0)")
-        for ks in range(32):
-            for j in range(4):
-                e("v_accvgpr_read_b32 %s, %s" % (v(T[2]), a(8 * ks + 2 * j)))
-                e("v_accvgpr_read_b32 %s, %s" % (v(T[3]), a(8 * ks + 2 * j + 1)))
-                e("s_nop 0")
-                e("%s %s, %s, %s" % (CVT, v(Q0 + 4 * ks + j), v(T[2]), v(T[3])))
-        for k in range(4):
-            ks = 32 + k
-            for j in range(4):
-                e("%s %s, %s, %s" % (CVT, v(Q0 + 4 * ks + j), v(SA + 8 * k + 2 * j), v(SA + 8 * k + 2 * j + 1)))
-    # the Q loads were issued after every tile DMA and are complete (vmcnt(0) above): all prologue tiles are in
+    # ------------------------------------------------------------------ Q operands: 36 coalesced 16-byte loads per lane from
+    # the packed image, issued behind the tile DMAs (one memory latency for everything)
+    e("v_lshlrev_b32 %s, 4, %s" % (v(X0), v(LANE)))
+    e("s_mul_i32 %s, %s, %d" % (s(S0), s(WAVE), 36 * 1024))
+    e("s_add_u32 %s, %s, %s" % (s(QP), s(QP), s(S0)))
+    e("s_addc_u32 %s, %s, 0" % (s(QP + 1), s(QP + 1)))
+    for ks in range(36):
+        if ks and ks % 4 == 0:
+            e("s_add_u32 %s, %s, 4096" % (s(QP), s(QP)))
+            e("s_addc_u32 %s, %s, 0" % (s(QP + 1), s(QP + 1)))
+        e("global_load_dwordx4 %s, %s, %s offset:%d" % (v(Q0 + 4 * ks, 4), v(X0), s(QP, 2), (ks % 4) * 1024))
+    e("s_waitcnt vmcnt(0)")
     e("s_barrier")
-    # accumulators start at zero (they were the landing zone of the Q loads)
-    for i in range(256):
-        e("v_accvgpr_write_b32 %s, 0" % a(i))
     if DEBUG:
         # FLG bit 1: dump LDS tile 0 (2336 chunks) to the debug pointer and stop
         lab = label("nodump1")

@@ -54,6 +54,7 @@ struct KParams {
     float           scale, softcap, max_bias, m0, m1;
     int             n_head_log2;
     int             c_log2_bits;   // bit pattern of scale * log2(e)
+    void *          q_pack;        // decode kernel: Q in MFMA operand layout (workspace)
     int             debug_flags;   // development builds of the decode kernel only
     void *          debug_ptr;
     int             n_pool_pages;  // block-table mode: pages in the pool
@@ -94,5 +95,6 @@ __device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); 
 bool       decode_fast_applicable(const mla_attn_args * a);
 hipError_t launch_decode_fast(const KParams & kp, int kv_type, dim3 grid, hipStream_t st);
 size_t     decode_fast_lds_bytes();
+size_t     decode_fast_qpack_bytes(int n_seq, int n_row_blocks);
 
 }  // namespace mla

@@ -504,7 +504,7 @@ struct Plan {
     int    n_splits, split_tokens;
     int    n_passes, ndb;
     size_t lds_bytes;
-    size_t ws_part_o, ws_part_ml, ws_scores;
+    size_t ws_part_o, ws_part_ml, ws_scores, ws_qpack;
 };
 
 int validate(const mla_attn_args * a) {
@@ -580,6 +580,7 @@ int make_plan(const mla_attn_args * a, Plan * pl) {
     pl->split_tokens = (int) (pages_per_split * MLA_PAGE_TOKENS);
     pl->n_splits     = (int) ((n_pages + pages_per_split - 1) / pages_per_split);
     pl->lds_bytes    = pl->variant == 2 ? decode_fast_lds_bytes() : 2 * TILE_BYTES + (a->kv_type == MLA_TYPE_Q8_0 ? Q8_TILE_RAW : 0);
+    if (pl->variant == 2) pl->ws_qpack = decode_fast_qpack_bytes(a->n_seq, pl->n_row_blocks);
     if (pl->n_splits > 1) {
         pl->ws_part_o  = (size_t) a->n_seq * pl->n_splits * n_rows * a->dv * sizeof(_Float16);
         pl->ws_part_ml = (size_t) a->n_seq * pl->n_splits * n_rows * 2 * sizeof(float);
@@ -588,7 +589,7 @@ int make_plan(const mla_attn_args * a, Plan * pl) {
 }
 
 size_t align256(size_t x) { return (x + 255) & ~(size_t) 255; }
-size_t plan_ws(const Plan & pl) { return align256(pl.ws_part_o) + align256(pl.ws_part_ml) + align256(pl.ws_scores); }
+size_t plan_ws(const Plan & pl) { return align256(pl.ws_part_o) + align256(pl.ws_part_ml) + align256(pl.ws_scores) + align256(pl.ws_qpack); }
 
 template <int SRC, int NDB, int WM, int WD>
 hipError_t launch_tile(const KParams & kp, dim3 grid, size_t lds, hipStream_t st) {
@@ -662,13 +663,13 @@ static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
     kp.m1 = powf(2.0f, -(a->max_bias / 2.0f) / kp.n_head_log2);
     { const float c = a->scale * LOG2E; memcpy(&kp.c_log2_bits, &c, 4); }
     kp.n_pool_pages = (int) (a->n_kv / MLA_PAGE_TOKENS);
-    if (const char * dbg = getenv("MLA_DEBUG")) { kp.debug_flags = atoi(dbg); kp.debug_ptr = a->dst; }
     kp.rows_contig = a->kv_nb1 == (a->kv_type == MLA_TYPE_Q8_0 ? Q8_ROW : ROW_BYTES) && (((uintptr_t) a->kv & 15) == 0) &&
                      (a->block_table || (a->kv_nb3 & 15) == 0);
     char * ws = (char *) a->workspace;
     kp.part_o  = (_Float16 *) ws;
     kp.part_ml = (float *) (ws + align256(pl.ws_part_o));
     float * scores = (float *) (ws + align256(pl.ws_part_o) + align256(pl.ws_part_ml));
+    kp.q_pack = ws + align256(pl.ws_part_o) + align256(pl.ws_part_ml) + align256(pl.ws_scores);
 
     if (pl.variant == 1) {
         if (!(phases & 1)) return 0;
