@@ -88,6 +88,9 @@ def main():
     ap.add_argument("--rows-per-wg", type=int, default=0)
     ap.add_argument("--cpu-seqs", type=int, default=8, help="sequences of the workload timed on the host cores (0 = skip)")
     ap.add_argument("--seed", type=int, default=1234)
+    ap.add_argument("--copy-calibration", type=int, default=0, metavar="N",
+                    help="also launch the library's plain copy kernel N times over one KV pool (known byte count) so that a "
+                         "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run can be scaled")
     ap.add_argument("--kv", default="bf16", choices=["bf16", "f16"], help="storage type of the latent KV pool (the headline config is bf16)")
     a = ap.parse_args()
     if a.gpus != 1:
@@ -156,6 +159,13 @@ def main():
     value = kv_bytes / (ms_per_step * 1e-3) / 1e9
     achieved = kv_bytes / (kern_ms * 1e-3) / 1e9
 
+    if a.copy_calibration > 0:
+        dst_copy = torch.empty_like(pools[0])
+        for _ in range(a.copy_calibration):
+            J.hbm_copy(pools[0], dst_copy)
+        torch.cuda.synchronize()
+        del dst_copy
+
     # final output of the last step for the parity check
     step(0)
     torch.cuda.synchronize()
@@ -163,6 +173,11 @@ def main():
     if a.cpu_seqs > 0:
         cpu, parity = cpu_baseline(q, pools[0], block_table, a.ctx, min(a.cpu_seqs, a.batch), scale, out)
 
+    # HBM bytes of one decode-kernel launch, from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by what the same
+    # counters read for the library's copy kernel; figures and commands in profiles/mla_decode_kernel_c3_pmc.md
+    traffic = None
+    if a.batch == 32 and a.heads == 128 and a.ctx == 8192 and a.kv == "bf16":
+        traffic = int(166156 * 1024 * (294912 / 147466.0) + 33024 * 1024)
     res = {
         "metric": "mla_paged_decode_kv_read_bandwidth", "value": value, "unit": "GB/s",
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms_per_step,
@@ -176,7 +191,7 @@ def main():
         "pct_hbm_peak": 100.0 * value / HBM_PEAK_GBPS,
         "tflops": flops / (ms_per_step * 1e-3) / 1e12,
         "roofline": {"bound": "hbm", "kernel": "mla_decode_kernel<%s>" % a.kv, "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic,
                      "algorithmic_bytes_per_launch": kv_bytes, "kernel_us": {"mean": kern_ms * 1e3},
                      "mfma_tflops": flops / (kern_ms * 1e-3) / 1e12},
         "cpu_baseline": cpu,
