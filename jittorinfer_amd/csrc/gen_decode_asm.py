@@ -7,11 +7,11 @@ registers for everything else; the instruction order (MFMA issue slots filled wi
 and the register map are fixed here instead of being left to a compiler that spills under that pressure.
 
 Work of one wave (32 attention rows, all 512 output columns), per 32-token tile `it`:
-    phase A   S_next = K[it+1] . Q^T      36 MFMA, interleaved with  softmax(S_cur) -> P (hi, lo)   (VALU)
-                                          and the address arithmetic + issue of the LDS-DMA loads of tile it+2
-    phase B   O^T += V[it]^T . P^T        32 V^T fragments (ds_read_b64_tr_b16 x2 each), 64 MFMA (hi and lo halves of P)
-    end       s_waitcnt vmcnt(0); s_barrier   (tile it+2 has landed for every wave)
-Register roles of S_cur/S_next swap every tile, so the loop body is emitted twice.
+    part 1   36 MFMA of S = K[it+1].Q^T alternating with the first 36 MFMA of O^T += V[it]^T.P[it]^T (independent
+             accumulators), with the address arithmetic + issue of the LDS-DMA loads of tile it+3 in their shadow
+    part 2   the remaining P.V MFMAs of tile it with softmax(S[it+1]) -> P[it+1] (in place) in their shadow
+    end      deferred accumulator rescale (rare), s_waitcnt vmcnt; s_barrier   (tile it+2 has landed for every wave)
+The two 16-register score/P groups swap roles every tile, so the loop body is emitted twice.
 """
 import sys
 
@@ -21,8 +21,12 @@ NO_PV = "--no-pv" in sys.argv
 NO_QK = "--no-qk" in sys.argv
 NO_SM = "--no-softmax" in sys.argv
 DMA_PLACE = "pv" if "--dma-pv" in sys.argv else "bulk" if "--dma-bulk" in sys.argv else "a"
+NO_VREAD = "--no-vread" in sys.argv
+NO_KREAD = "--no-kread" in sys.argv
 NO_STORE = "--no-store" in sys.argv
 NO_QLOAD = "--no-qload" in sys.argv
+CLKP = "--clk-parts" in sys.argv    # with --clk: accumulate the cycles of part 1 / part 2 of the iterations instead of the waits
+CLK = "--clk" in sys.argv or CLKP           # timing experiments only: s_memtime stamps, written to the hand-off area at the end
 F16 = "--f16" in sys.argv  # f16 KV: f16 MFMA, single P (no lo half)
 MF = "v_mfma_f32_32x32x16_f16" if F16 else "v_mfma_f32_32x32x16_bf16"
 CVT = "v_cvt_pk_f16_f32" if F16 else "v_cvt_pk_bf16_f32"
@@ -36,13 +40,19 @@ DMA_PER_TILE = 10              # LDS-DMA instructions each wave issues per tile
 CPR = 73                       # 16-byte chunks per padded row
 WAVE_CHUNKS = 8 * CPR          # 584: each wave moves rows 8w..8w+7 of a tile
 TAU = 8.0
+def _opt(name, default):
+    return int(sys.argv[sys.argv.index(name) + 1]) if name in sys.argv else default
+
+
+P1_PV = _opt("--p1pv", 24 if SPLIT else 12)   # P.V MFMAs issued among the 36 QK^T MFMAs; the rest cover the softmax
+P1_LEAD = _opt("--lead", 3)                   # P.V MFMAs at the head of an iteration (they cover the first K fragment reads)
 
 # ---- VGPR map
 Q0 = 0
-SA, SB = 144, 160
-PHI, PLO = 176, 184
-KF = 192   # 4 fragments x 4
-VF = 208   # 4 fragments x 4
+SA, SB = 144, 160   # two 16-register groups: scores of one tile, converted in place to its P^T operands
+KF, KRING = 176, 5  # K fragment ring (5 x 4 registers)
+ALPHA = 196
+VF, VRING = 200, 6  # V^T fragment ring (6 x 4 registers)
 T = list(range(224, 232))
 OPTR, MLPTR = 232, 234
 KADDR_LANE, VADDR_LANE, MRUN, LRUN, NEGM = 236, 237, 238, 239, 240
@@ -88,14 +98,16 @@ class Lds:
         self.pending = []
 
     def read(self, line, tag):
+        if (NO_VREAD and tag[0] == "v") or (NO_KREAD and tag[0] == "k"):
+            return
         e(line)
         self.pending.append(tag)
 
     def need(self, tag):
         if tag in self.pending:
-            after = len(self.pending) - 1 - self.pending.index(tag)
+            after = min(len(self.pending) - 1 - self.pending.index(tag), 15)   # the counter field has 4 bits
             e("s_waitcnt lgkmcnt(%d)" % after)
-            self.pending = self.pending[len(self.pending) - after:]
+            self.pending = self.pending[len(self.pending) - after:] if after else []
 
     def drain(self):
         if self.pending:
@@ -104,6 +116,13 @@ class Lds:
 
 
 lds = Lds()
+
+
+def stamp(k):
+    """--clk builds: shader-clock time stamp k into s[80+2k:81+2k]."""
+    if CLK:
+        e("s_memtime %s" % s(100 if k == 6 else 80 + 2 * k, 2))
+        e("s_waitcnt lgkmcnt(0)")
 
 
 def interleave(mfma_slots, valu, per_slot):
@@ -182,33 +201,93 @@ def dma_tile_lines(tile_sreg, off_sreg):
     return L
 
 
+def k_read(kaddr, p):
+    lds.read("ds_read_b128 %s, %s offset:%d" % (v(KF + 4 * (p % KRING), 4), v(kaddr), p * 32), ("k", p))
+
+
+def k_warm(kaddr):
+    """First K fragments of a tile into the ring."""
+    if not NO_QK:
+        for p in range(KRING - 1):
+            k_read(kaddr, p)
+
+
 def qk_slots(sreg, kaddr):
-    """36 MFMA slots of S = K.Q^T into v[sreg:sreg+15]; K fragments come through a ring of 4."""
+    """36 MFMA slots of S = K.Q^T into v[sreg:sreg+15]; K fragments come through a ring (k_warm first)."""
     if NO_QK:
         return [(lambda: None) for _ in range(36)]
-    slots = []
-    depth = 3
+    depth = KRING - 1
 
     def mk(ks):
         def slot():
-            # keep `depth` reads in flight
-            if ks == 0:
-                for p in range(depth):
-                    lds.read("ds_read_b128 %s, %s offset:%d" % (v(KF + 4 * (p % 4), 4), v(kaddr), p * 32), ("k", p))
             if ks + depth < 36:
-                p = ks + depth
-                lds.read("ds_read_b128 %s, %s offset:%d" % (v(KF + 4 * (p % 4), 4), v(kaddr), p * 32), ("k", p))
+                k_read(kaddr, ks + depth)
             lds.need(("k", ks))
             c = "0" if ks == 0 else v(sreg, 16)
-            e("%s %s, %s, %s, %s" % (MF, v(sreg, 16), v(KF + 4 * (ks % 4), 4), v(Q0 + 4 * ks, 4), c))
+            e("%s %s, %s, %s, %s" % (MF, v(sreg, 16), v(KF + 4 * (ks % KRING), 4), v(Q0 + 4 * ks, 4), c))
         return slot
-    for ks in range(36):
-        slots.append(mk(ks))
+    return [mk(ks) for ks in range(36)]
+
+
+V_FRAGS = [(kk, db) for kk in range(2) for db in range(16)]
+
+
+def v_read(vaddr, idx):
+    kk, db = V_FRAGS[idx]
+    r = VF + 4 * (idx % VRING)
+    base = 16 * kk * PITCH + db * 64
+    lds.read("ds_read_b64_tr_b16 %s, %s offset:%d" % (v(r, 2), v(vaddr), base), ("v", idx, 0))
+    lds.read("ds_read_b64_tr_b16 %s, %s offset:%d" % (v(r + 2, 2), v(vaddr), base + 8 * PITCH), ("v", idx, 1))
+
+
+def v_warm(vaddr):
+    """First V^T fragments of a tile into the ring (issued at the end of the previous tile)."""
+    if not NO_PV:
+        for idx in range(VRING - 1):
+            v_read(vaddr, idx)
+
+
+def v_warm_tags():
+    return [] if NO_PV or NO_VREAD else [("v", idx, h) for idx in range(VRING - 1) for h in range(2)]
+
+
+def pv_slots(vaddr, greg):
+    """MFMA slots of O^T += V^T.P^T for the tile whose P^T operands sit in group `greg`
+    (hi halves of k-step kk in greg+8kk .. +3, lo halves in greg+8kk+4 .. +7).  16 d-blocks x 2 k-steps, fragments
+    through a ring (v_warm first), d-blocks in pairs so that MFMAs on the same accumulator are never adjacent."""
+    if NO_PV:
+        return []
+    depth = VRING - 1
+
+    def mf(idx, lo, pre):
+        kk, db = V_FRAGS[idx]
+        def slot():
+            for p in pre:
+                v_read(vaddr, p)
+            lds.need(("v", idx, 1))
+            e("%s %s, %s, %s, %s" % (MF, a(16 * db, 16), v(VF + 4 * (idx % VRING), 4), v(greg + 8 * kk + (4 if lo else 0), 4), a(16 * db, 16)))
+        return slot
+    slots = []
+    for pair in range(16):
+        i0, i1 = 2 * pair, 2 * pair + 1
+        n0 = [i0 + depth] if i0 + depth < 32 else []
+        n1 = [i1 + depth] if i1 + depth < 32 else []
+        slots.append(mf(i0, False, n0))
+        if SPLIT:
+            slots.append(mf(i1, False, []))
+            slots.append(mf(i0, True, []))
+            slots.append(mf(i1, True, n1))   # fragment i0's ring slot is only reused by reads issued after its last MFMA
+        else:
+            slots.append(mf(i1, False, n1))
     return slots
 
 
-def softmax_part1(sreg):
-    """tile max -> TMAX (log2 units), uniform test whether any row's max moved by more than TAU."""
+def softmax_lines(sreg):
+    """Softmax of the scores in group sreg, as one list of VALU lines (no branches):
+    tile max -> lazy max update (new max only where it grew by more than TAU) -> ALPHA (rescale factor of O and l,
+    1 where the max stayed) and RSC (non-zero when some lane changed its max; the accumulators are rescaled by the
+    caller once the MFMAs of the current tile are done) -> p = 2^(s*c - m) -> l += sum p -> P^T operands in place:
+    k-step kk: hi halves in sreg+8kk..+3, lo halves in sreg+8kk+4..+7."""
     if NO_SM:
         return ["s_mov_b64 %s, 0" % s(RSC, 2)]
     L = []
@@ -228,40 +307,20 @@ def softmax_part1(sreg):
     L.append("v_max_f32 %s, %s, %s" % (v(TMAX), v(m[0]), v(m[1])))
     L.append("v_mul_f32 %s, %s, %s" % (v(TMAX), s(CL2), v(TMAX)))          # log2 units (c_log2 > 0)
     L.append("v_add_f32 %s, %s, %s" % (v(m[2]), s(THR), v(MRUN)))           # m_run + TAU  (-inf stays -inf)
-    L.append("v_cmp_gt_f32 %s, %s, %s" % (s(RSC, 2), v(TMAX), v(m[2])))
-    return L
-
-
-def rescale_block(ret_label):
-    """Rare path: m_new = max(m_run, tmax); alpha = 2^(m_run - m_new) (0 when m_run = -inf); acc *= alpha; l *= alpha."""
-    e("v_max_f32 %s, %s, %s" % (v(T[0]), v(MRUN), v(TMAX)))                 # m_new
-    e("v_sub_f32 %s, %s, %s" % (v(T[1]), v(MRUN), v(T[0])))                 # m_run - m_new (NaN when both -inf)
-    e("v_exp_f32 %s, %s" % (v(T[1]), v(T[1])))
-    e("v_mov_b32 %s, 0xff800000" % v(T[2]))
-    e("v_cmp_eq_f32 vcc, %s, %s" % (v(MRUN), v(T[2])))
-    e("s_nop 1")
-    e("v_cndmask_b32 %s, %s, 0, vcc" % (v(T[1]), v(T[1])))                  # alpha
-    e("v_mov_b32 %s, %s" % (v(MRUN), v(T[0])))
-    e("v_mul_f32 %s, %s, %s" % (v(LRUN), v(LRUN), v(T[1])))
-    e("s_nop 7")
-    e("s_nop 7")
-    e("s_nop 3")                                                            # last MFMA writes to acc are long done
-    for i in range(0, 256, 4):
-        for j in range(4):
-            e("v_accvgpr_read_b32 %s, %s" % (v(T[3 + j]), a(i + j)))
-        for j in range(4):
-            e("v_mul_f32 %s, %s, %s" % (v(T[3 + j]), v(T[3 + j]), v(T[1])))
-        for j in range(4):
-            e("v_accvgpr_write_b32 %s, %s" % (a(i + j), v(T[3 + j])))
-    e("s_nop 7")
-    e("s_nop 7")
-    e("s_branch %s" % ret_label)
-
-
-def softmax_part2(sreg):
-    if NO_SM:
-        return []
-    L = []
+    L.append("v_sub_f32 %s, %s, %s" % (v(m[3]), v(MRUN), v(TMAX)))          # m_run - tmax
+    L.append("v_exp_f32 %s, %s" % (v(m[3]), v(m[3])))                       # 2^(m_run - tmax); 0 when m_run = -inf
+    L.append("v_cmp_gt_f32 vcc, %s, %s" % (v(TMAX), v(m[2])))               # this lane's max moves
+    L.append("s_mov_b64 %s, vcc" % s(RSC, 2))
+    L.append("s_nop 1")
+    L.append("v_cndmask_b32 %s, 1.0, %s, vcc" % (v(ALPHA), v(m[3])))
+    L.append("v_cndmask_b32 %s, %s, %s, vcc" % (v(MRUN), v(MRUN), v(TMAX)))
+    L.append("v_mul_f32 %s, %s, %s" % (v(LRUN), v(LRUN), v(ALPHA)))
+    # -m (0 when still -inf)
+    L.append("v_mov_b32 %s, 0xff800000" % v(m[0]))
+    L.append("v_cmp_eq_f32 vcc, %s, %s" % (v(MRUN), v(m[0])))
+    L.append("v_sub_f32 %s, 0, %s" % (v(NEGM), v(MRUN)))
+    L.append("s_nop 0")
+    L.append("v_cndmask_b32 %s, %s, 0, vcc" % (v(NEGM), v(NEGM)))
     # p = 2^(s*c - m)
     for k in range(16):
         L.append("v_fma_f32 %s, %s, %s, %s" % (v(sreg + k), v(sreg + k), s(CL2), v(NEGM)))
@@ -275,18 +334,44 @@ def softmax_part2(sreg):
         L.append("v_add_f32 %s, %s, %s" % (v(T[1]), v(T[1]), v(sreg + k + 1)))
     L.append("v_add_f32 %s, %s, %s" % (v(T[0]), v(T[0]), v(T[1])))
     L.append("v_add_f32 %s, %s, %s" % (v(LRUN), v(LRUN), v(T[0])))
-    # P^T operands: k-step kk uses elements 8kk .. 8kk+7
-    for j in range(8):
-        L.append("%s %s, %s, %s" % (CVT, v(PHI + j), v(sreg + 2 * j), v(sreg + 2 * j + 1)))
-    if SPLIT:
-        for j in range(8):
-            t0, t1 = T[2 + (j % 3) * 2], T[3 + (j % 3) * 2]
-            L.append("v_lshlrev_b32 %s, 16, %s" % (v(t0), v(PHI + j)))
-            L.append("v_and_b32 %s, 0xffff0000, %s" % (v(t1), v(PHI + j)))
-            L.append("v_sub_f32 %s, %s, %s" % (v(t0), v(sreg + 2 * j), v(t0)))
-            L.append("v_sub_f32 %s, %s, %s" % (v(t1), v(sreg + 2 * j + 1), v(t1)))
-            L.append("%s %s, %s, %s" % (CVT, v(PLO + j), v(t0), v(t1)))
+    # P^T operands in place.  k-step kk owns registers b = sreg+8kk .. +7, holding p of tokens
+    # (8(2kk)+4g+0..3, 8(2kk+1)+4g+0..3); pairs (b0,b1) (b2,b3) (b4,b5) (b6,b7) become hi -> b0..b3, lo -> b4..b7.
+    for kk in range(2):
+        b = sreg + 8 * kk
+        if not SPLIT:
+            for j in range(4):
+                L.append("%s %s, %s, %s" % (CVT, v(b + j), v(b + 2 * j), v(b + 2 * j + 1)))
+            continue
+        H, X, Y = T[0], T[1], T[2]
+        Lo = [T[3], T[4], T[5], T[6]]
+        for j in range(4):
+            L.append("%s %s, %s, %s" % (CVT, v(H), v(b + 2 * j), v(b + 2 * j + 1)))
+            L.append("v_lshlrev_b32 %s, 16, %s" % (v(X), v(H)))
+            L.append("v_and_b32 %s, 0xffff0000, %s" % (v(Y), v(H)))
+            L.append("v_sub_f32 %s, %s, %s" % (v(X), v(b + 2 * j), v(X)))
+            L.append("v_sub_f32 %s, %s, %s" % (v(Y), v(b + 2 * j + 1), v(Y)))
+            L.append("%s %s, %s, %s" % (CVT, v(Lo[j]), v(X), v(Y)))
+            L.append("v_mov_b32 %s, %s" % (v(b + j), v(H)))       # b+j <= b+2j: already consumed
+        for j in range(4):
+            L.append("v_mov_b32 %s, %s" % (v(b + 4 + j), v(Lo[j])))
     return L
+
+
+def rescale_block(ret_label):
+    """Rare path, entered only when no MFMA is in flight on the accumulators: acc *= ALPHA (per lane = per row)."""
+    e("s_nop 7")
+    e("s_nop 7")
+    e("s_nop 3")
+    for i in range(0, 256, 4):
+        for j in range(4):
+            e("v_accvgpr_read_b32 %s, %s" % (v(T[3 + j]), a(i + j)))
+        for j in range(4):
+            e("v_mul_f32 %s, %s, %s" % (v(T[3 + j]), v(T[3 + j]), v(ALPHA)))
+        for j in range(4):
+            e("v_accvgpr_write_b32 %s, %s" % (a(i + j), v(T[3 + j])))
+    e("s_nop 7")
+    e("s_nop 7")
+    e("s_branch %s" % ret_label)
 
 
 def mask_tail(sreg):
@@ -305,129 +390,100 @@ def mask_tail(sreg):
     e("%s:" % lab)
 
 
-def pv_phase(vaddr, extra=None):
-    """O^T += V^T.P^T: 16 d-blocks x 2 k-steps; fragment ring of 4; d-blocks in pairs so dependent MFMAs alternate.
-    `extra`: instruction lines spread evenly between the MFMA pairs (whole-slot groups only)."""
-    frags = [(kk, db) for kk in range(2) for db in range(16)]
-    extra = list(extra or [])
-    per_pair = -(-len(extra) // 16)
-
-    def rd(idx):
-        kk, db = frags[idx]
-        r = VF + 4 * (idx % 4)
-        base = 16 * kk * PITCH + db * 64
-        lds.read("ds_read_b64_tr_b16 %s, %s offset:%d" % (v(r, 2), v(vaddr), base), ("v", idx, 0))
-        lds.read("ds_read_b64_tr_b16 %s, %s offset:%d" % (v(r + 2, 2), v(vaddr), base + 8 * PITCH), ("v", idx, 1))
-    depth = 3
-    for p in range(depth):
-        rd(p)
-    for pair in range(16):
-        i0, i1 = 2 * pair, 2 * pair + 1
-        # issue order: hi(i0), hi(i1), lo(i0), lo(i1) with prefetches in between
-        kk0, db0 = frags[i0]
-        kk1, db1 = frags[i1]
-        if i0 + depth < 32:
-            rd(i0 + depth)
-        lds.need(("v", i0, 1))
-        e("%s %s, %s, %s, %s" % (MF, a(16 * db0, 16), v(VF + 4 * (i0 % 4), 4), v(PHI + 4 * kk0, 4), a(16 * db0, 16)))
-        lds.need(("v", i1, 1))
-        e("%s %s, %s, %s, %s" % (MF, a(16 * db1, 16), v(VF + 4 * (i1 % 4), 4), v(PHI + 4 * kk1, 4), a(16 * db1, 16)))
-        if SPLIT:
-            e("%s %s, %s, %s, %s" % (MF, a(16 * db0, 16), v(VF + 4 * (i0 % 4), 4), v(PLO + 4 * kk0, 4), a(16 * db0, 16)))
-            if i1 + depth < 32:
-                rd(i1 + depth)
-            e("%s %s, %s, %s, %s" % (MF, a(16 * db1, 16), v(VF + 4 * (i1 % 4), 4), v(PLO + 4 * kk1, 4), a(16 * db1, 16)))
-        else:
-            if i1 + depth < 32:
-                rd(i1 + depth)
-        for _ in range(per_pair):
-            if extra:
-                e(extra.pop(0))
-    for ln in extra:
-        e(ln)
-
-
-def half_iteration(s_cur, s_next, tag):
-    """Tile IT: QK of tile IT+1 into s_next interleaved with softmax of s_cur; then PV of tile IT."""
-    e("; ---- half %s" % tag)
-    # n_valid of tile IT
-    e("s_lshl_b32 %s, %s, 5" % (s(S0), s(IT)))
+def iteration(g_cur, g_next, tag):
+    """Tile IT (its P^T operands are in g_cur): the 64 (32) P.V MFMAs, the first 36 of them alternating with the 36
+    MFMAs of S = K.Q^T of tile IT+1 (into g_next; independent accumulators, so the MFMA pipe never waits on a
+    dependency), the rest carrying the softmax of tile IT+1 in their shadow.  The LDS-DMA loads of tile IT+3 are
+    issued from the first part.  Returns the (label, return label) pairs of the out-of-line rescale blocks."""
+    e("; ---- iteration %s" % tag)
+    resc = []
+    if CLKP:
+        e("s_memtime s[94:95]")
+    # n_valid of tile IT+1
+    e("s_add_u32 %s, %s, 1" % (s(S0), s(IT)))
+    e("s_lshl_b32 %s, %s, 5" % (s(S0), s(S0)))
     e("s_add_u32 %s, %s, %s" % (s(S0), s(S0), s(KVB)))
     e("s_sub_u32 %s, %s, %s" % (s(NVAL), s(KVE), s(S0)))
     e("s_min_u32 %s, %s, 32" % (s(NVAL), s(NVAL)))
-    mask_tail(s_cur)
-    # addresses for this half
     e("v_add_u32 %s, %s, %s" % (v(KADDR), s(OFF1), v(KADDR_LANE)))
-    e("v_add_u32 %s, %s, %s" % (v(VADDR), s(OFF0), v(VADDR_LANE)))
-    slots = qk_slots(s_next, KADDR)
-    # DMA of tile IT+3 (skipped when it does not exist)
-    e("s_add_u32 %s, %s, 3" % (s(TMP), s(IT)))
     e("s_mov_b32 %s, 0" % s(VMW))
-    lab_nodma, lab_after = label("nodma"), label("afterdma")
+    e("s_mov_b64 %s, 0" % s(RSC, 2))
+    lab_last, lab_nodma, lab_p2, lab_end = label("last"), label("nodma"), label("p2"), label("iend")
+    e("s_add_u32 %s, %s, 1" % (s(TMP), s(IT)))
+    e("s_cmp_ge_u32 %s, %s" % (s(TMP), s(NT)))
+    e("s_cbranch_scc1 %s" % lab_last)
+    e("s_add_u32 %s, %s, 3" % (s(TMP), s(IT)))
     e("s_cmp_ge_u32 %s, %s" % (s(TMP), s(NT)))
     e("s_cbranch_scc1 %s" % lab_nodma)
     if NO_LOOP_DMA:
         e("s_branch %s" % lab_nodma)
+
+    def part1(dma):
+        lds.pending = v_warm_tags()
+        k_warm(KADDR)
+        qk = qk_slots(g_next, KADDR)
+        pv = pv_slots(VADDR, g_cur)
+        n1 = min(P1_PV, len(pv))
+        lead = min(P1_LEAD, n1)
+        merged = list(pv[:lead])
+        for n in range(36):
+            merged.append(qk[n])
+            merged.extend(pv[lead + n * (n1 - lead) // 36:lead + (n + 1) * (n1 - lead) // 36])
+        interleave(merged, dma, 2)
+        return pv[n1:]
+
+    # ---- part 1 with the DMA of tile IT+3
     e("s_mov_b32 %s, 1" % s(VMW))
-    dma = dma_tile_lines(TMP, OFF3)
-    if DMA_PLACE != "a":
-        if DMA_PLACE == "bulk":
-            for ln in dma:
-                e(ln)
-        e("s_branch %s" % lab_nodma)   # the compute part is the DMA-free code below
-        dma = []
-    # part 1 of the softmax + DMA issue share the first MFMA slots
-    p1 = softmax_part1(s_cur)
-    n1 = 8
-    interleave(slots[:n1], p1 + dma[:46], 8)  # 22 set-up lines + two whole DMA slots (vcc must not live across the cut)
-    rest_dma = dma[46:]
+    rest_a = part1(dma_tile_lines(TMP, OFF3))
+    state_a = list(lds.pending)
+    e("s_branch %s" % lab_p2)
+    # ---- part 1 without it (tiles IT+3.. do not exist)
+    e("%s:" % lab_nodma)
+    rest_b = part1([])
+    assert lds.pending == state_a and len(rest_a) == len(rest_b)
+    # ---- part 2: remaining P.V MFMAs of tile IT, softmax of tile IT+1 in their shadow
+    e("%s:" % lab_p2)
+    if CLKP:
+        e("s_memtime s[96:97]")
+    head = rest_b[:2]
+    for sl in head:
+        sl()
+    e("s_nop 7")                       # the last QK^T MFMA has written g_next
+    if len(head) < 2:
+        e("s_nop 7")
+    mask_tail(g_next)
+    interleave(rest_b[2:], softmax_lines(g_next), 4)
+    # first V^T fragments of tile IT+1 (next iteration's P.V starts without waiting for LDS)
+    e("v_add_u32 %s, %s, %s" % (v(VADDR), s(OFF1), v(VADDR_LANE)))
+    v_warm(VADDR)
+    assert lds.pending == v_warm_tags(), lds.pending
+    if CLKP:
+        e("s_memtime s[98:99]")
+        e("s_waitcnt lgkmcnt(0)")
+        e("s_sub_u32 s98, s98, s96")
+        e("s_sub_u32 s96, s96, s94")
+        e("s_add_u32 s92, s92, s96")       # part 1
+        e("s_add_u32 s93, s93, s98")       # part 2
+    e("s_branch %s" % lab_end)
+    # ---- last tile: P.V only
+    e("%s:" % lab_last)
+    lds.pending = v_warm_tags()
+    for sl in pv_slots(VADDR, g_cur):
+        sl()
+    lds.drain()
+    e("%s:" % lab_end)
+    # ---- the accumulators take the new row maxima now that no MFMA of tile IT is left to issue
     lab_resc, lab_back = label("resc"), label("back")
     e("s_cmp_lg_u64 %s, 0" % s(RSC, 2))
     e("s_cbranch_scc1 %s" % lab_resc)
     e("%s:" % lab_back)
-    # -m (0 when still -inf)
-    pre = ["v_mov_b32 %s, 0xff800000" % v(T[0]),
-           "v_cmp_eq_f32 vcc, %s, %s" % (v(MRUN), v(T[0])),
-           "v_sub_f32 %s, 0, %s" % (v(NEGM), v(MRUN)),
-           "s_nop 0",
-           "v_cndmask_b32 %s, %s, 0, vcc" % (v(NEGM), v(NEGM))]
-    p2 = softmax_part2(s_cur)
-    interleave(slots[n1:], pre + rest_dma + p2, 6)
-    e("s_branch %s" % lab_after)
-    # ---- same thing without the DMA (last two tiles)
-    e("%s:" % lab_nodma)
-    saved = list(lds.pending)
-    lds.pending = []
-    slots2 = qk_slots(s_next, KADDR)
-    p1b = softmax_part1(s_cur)
-    interleave(slots2[:n1], p1b, 4)
-    lab_resc2, lab_back2 = label("resc"), label("back")
-    e("s_cmp_lg_u64 %s, 0" % s(RSC, 2))
-    e("s_cbranch_scc1 %s" % lab_resc2)
-    e("%s:" % lab_back2)
-    interleave(slots2[n1:], list(pre) + softmax_part2(s_cur), 4)
-    e("%s:" % lab_after)
-    assert not lds.pending and not saved
-    # ---- PV of tile IT
-    if not NO_PV:
-        if DMA_PLACE == "pv":
-            # DMA of tile IT+3 issued from inside the PV phase (VALU is otherwise idle there)
-            lab_pvnodma, lab_pvdone = label("pvnodma"), label("pvdone")
-            e("s_cmp_eq_u32 %s, 0" % s(VMW))
-            e("s_cbranch_scc1 %s" % lab_pvnodma)
-            pv_phase(VADDR, dma_tile_lines(TMP, OFF3))
-            lds.drain()
-            e("s_branch %s" % lab_pvdone)
-            e("%s:" % lab_pvnodma)
-            pv_phase(VADDR)
-            lds.drain()
-            e("%s:" % lab_pvdone)
-        else:
-            pv_phase(VADDR)
-    lds.drain()
+    resc.append((lab_resc, lab_back))
     # ---- end of tile: the DMA of tile IT+2 has landed (the one of tile IT+3, issued in this iteration, may still be
     # in flight: loads complete in order, so vmcnt(DMA_PER_TILE) is enough); everyone is done with tile IT
     lab_w0, lab_wd = label("w0"), label("wd")
+    if CLK and not CLKP:
+        e("s_memtime s[94:95]")
+        e("s_waitcnt lgkmcnt(0)")
     e("s_cmp_eq_u32 %s, 0" % s(VMW))
     e("s_cbranch_scc1 %s" % lab_w0)
     e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
@@ -435,18 +491,35 @@ def half_iteration(s_cur, s_next, tag):
     e("%s:" % lab_w0)
     e("s_waitcnt vmcnt(0)")
     e("%s:" % lab_wd)
+    if CLK and not CLKP:
+        e("s_memtime s[96:97]")
+        e("s_waitcnt lgkmcnt(0)")
+        e("s_sub_u32 s96, s96, s94")
+        e("s_add_u32 s92, s92, s96")       # cycles spent waiting for the tile loads
+        e("s_mov_b32 s94, s96")
+        e("s_memtime s[96:97]")
+        e("s_waitcnt lgkmcnt(0)")
     e("s_barrier")
+    if CLK and not CLKP:
+        e("s_memtime s[98:99]")
+        e("s_waitcnt lgkmcnt(0)")
+        e("s_sub_u32 s98, s98, s96")
+        e("s_add_u32 s93, s93, s98")       # cycles spent in the barrier
     e("s_mov_b32 %s, %s" % (s(TMP), s(OFF0)))
     e("s_mov_b32 %s, %s" % (s(OFF0), s(OFF1)))
     e("s_mov_b32 %s, %s" % (s(OFF1), s(OFF2)))
     e("s_mov_b32 %s, %s" % (s(OFF2), s(OFF3)))
     e("s_mov_b32 %s, %s" % (s(OFF3), s(TMP)))
     e("s_add_u32 %s, %s, 1" % (s(IT), s(IT)))
-    return (lab_resc, lab_back), (lab_resc2, lab_back2)
+    return resc
 
 
 def main():
     # ------------------------------------------------------------------ entry: inputs -> fixed registers
+    stamp(0)
+    if CLK:
+        e("s_mov_b32 s92, 0")
+        e("s_mov_b32 s93, 0")
     e("s_mov_b64 %s, %%[kv]" % s(KV, 2))
     e("s_mov_b64 %s, %%[bt]" % s(BT, 2))
     e("s_mov_b32 %s, %%[kvb]" % s(KVB))
@@ -507,11 +580,20 @@ def main():
     e("v_add_u32 %s, %s, %s" % (v(X0), s(PG0), v(LANE)))
     e("v_lshlrev_b32 %s, 2, %s" % (v(X0), v(X0)))
     e("global_load_dword %s, %s, %s" % (v(PAGES), v(X0), s(BT, 2)))
-    e("s_waitcnt vmcnt(0)")
     e("s_mov_b64 exec, %s" % s(EXS, 2))
-    e("v_max_i32 %s, 0, %s" % (v(PAGES), v(PAGES)))
-    e("v_min_i32 %s, %s, %s" % (v(PAGES), s(NPP), v(PAGES)))
     e("%s:" % lab_nobt)
+    # ------------------------------------------------------------------ Q operands: 36 coalesced 16-byte loads per lane from
+    # the packed image, in flight together with the page ids
+    nq = 0 if NO_QLOAD else 36
+    e("v_lshlrev_b32 %s, 4, %s" % (v(X0), v(LANE)))
+    e("s_mul_i32 %s, %s, %d" % (s(S0), s(WAVE), 36 * 1024))
+    e("s_add_u32 %s, %s, %s" % (s(QP), s(QP), s(S0)))
+    e("s_addc_u32 %s, %s, 0" % (s(QP + 1), s(QP + 1)))
+    for ks in range(nq):
+        if ks and ks % 4 == 0:
+            e("s_add_u32 %s, %s, 4096" % (s(QP), s(QP)))
+            e("s_addc_u32 %s, %s, 0" % (s(QP + 1), s(QP + 1)))
+        e("global_load_dwordx4 %s, %s, %s offset:%d" % (v(Q0 + 4 * ks, 4), v(X0), s(QP, 2), (ks % 4) * 1024))
     # ------------------------------------------------------------------ state
     e("v_mov_b32 %s, 0xff800000" % v(MRUN))
     e("v_mov_b32 %s, 0" % v(LRUN))
@@ -522,36 +604,36 @@ def main():
     e("s_mov_b32 %s, 0" % s(IT))
     for i in range(256):
         e("v_accvgpr_write_b32 %s, 0" % a(i))
-    # ------------------------------------------------------------------ prologue: tiles 0, 1, 2, S of tile 0
+    # page ids have arrived (loads return in order: only the Q loads may still be in flight)
+    e("s_waitcnt vmcnt(%d)" % nq)
+    e("v_max_i32 %s, 0, %s" % (v(PAGES), v(PAGES)))
+    e("v_min_i32 %s, %s, %s" % (v(PAGES), s(NPP), v(PAGES)))
+    stamp(6)
+    # ------------------------------------------------------------------ tiles 0, 1, 2 -> LDS; go on as soon as Q and tile 0 are there
+    lab_w0, lab_w1, lab_wd = label("pw0"), label("pw1"), label("pwd")
     e("s_mov_b32 %s, 0" % s(TMP))
     for ln in dma_tile_lines(TMP, OFF0):
         e(ln)
-    lab_one = label("one")
-    lab_three, lab_pw = label("three"), label("pw")
     e("s_cmp_lt_u32 %s, 2" % s(NT))
-    e("s_cbranch_scc1 %s" % lab_one)
+    e("s_cbranch_scc1 %s" % lab_w0)
     e("s_mov_b32 %s, 1" % s(TMP))
     for ln in dma_tile_lines(TMP, OFF1):
         e(ln)
     e("s_cmp_lt_u32 %s, 3" % s(NT))
-    e("s_cbranch_scc1 %s" % lab_one)
+    e("s_cbranch_scc1 %s" % lab_w1)
     e("s_mov_b32 %s, 2" % s(TMP))
     for ln in dma_tile_lines(TMP, OFF2):
         e(ln)
-    e("%s:" % lab_one)
-    # ------------------------------------------------------------------ Q operands: 36 coalesced 16-byte loads per lane from
-    # the packed image, issued behind the tile DMAs (one memory latency for everything)
-    e("v_lshlrev_b32 %s, 4, %s" % (v(X0), v(LANE)))
-    e("s_mul_i32 %s, %s, %d" % (s(S0), s(WAVE), 36 * 1024))
-    e("s_add_u32 %s, %s, %s" % (s(QP), s(QP), s(S0)))
-    e("s_addc_u32 %s, %s, 0" % (s(QP + 1), s(QP + 1)))
-    for ks in range(36):
-        if ks and ks % 4 == 0:
-            e("s_add_u32 %s, %s, 4096" % (s(QP), s(QP)))
-            e("s_addc_u32 %s, %s, 0" % (s(QP + 1), s(QP + 1)))
-        e("global_load_dwordx4 %s, %s, %s offset:%d" % (v(Q0 + 4 * ks, 4), v(X0), s(QP, 2), (ks % 4) * 1024))
+    e("s_waitcnt vmcnt(%d)" % (2 * DMA_PER_TILE))
+    e("s_branch %s" % lab_wd)
+    e("%s:" % lab_w1)
+    e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
+    e("s_branch %s" % lab_wd)
+    e("%s:" % lab_w0)
     e("s_waitcnt vmcnt(0)")
+    e("%s:" % lab_wd)
     e("s_barrier")
+    stamp(1)
     if DEBUG:
         # FLG bit 1: dump LDS tile 0 (2336 chunks) to the debug pointer and stop
         lab = label("nodump1")
@@ -577,31 +659,38 @@ def main():
         e("s_endpgm")
         e("%s:" % lab)
     e("v_add_u32 %s, %s, %s" % (v(KADDR), s(OFF0), v(KADDR_LANE)))
+    k_warm(KADDR)
     for slot in qk_slots(SA, KADDR):
         slot()
-    if DEBUG:
-        lab = label("nodump2")
-        e("s_bitcmp1_b32 %s, 2" % s(FLG))
-        e("s_cbranch_scc0 %s" % lab)
-        e("s_nop 7")
-        e("s_nop 7")
-        e("s_nop 7")
-        e("v_lshlrev_b32 %s, 6, %s" % (v(X1), v(TIDR)))
-        e("v_add_co_u32 %s, vcc, %s, %s" % (v(DBG), v(DBG), v(X1)))
-        e("s_nop 1")
-        e("v_addc_co_u32 %s, vcc, 0, %s, vcc" % (v(DBG + 1), v(DBG + 1)))
-        for k in range(4):
-            e("global_store_dwordx4 %s, %s, off offset:%d" % (v(DBG, 2), v(SA + 4 * k, 4), 16 * k))
-        e("s_waitcnt vmcnt(0)")
-        e("s_endpgm")
-        e("%s:" % lab)
-    # ------------------------------------------------------------------ main loop (two halves: S roles swap)
+    # softmax of tile 0 (nothing to overlap it with); the accumulators are still zero, so no rescale
+    e("s_sub_u32 %s, %s, %s" % (s(NVAL), s(KVE), s(KVB)))
+    e("s_min_u32 %s, %s, 32" % (s(NVAL), s(NVAL)))
+    e("s_nop 7")
+    e("s_nop 7")
+    mask_tail(SA)
+    for ln in softmax_lines(SA):
+        e(ln)
+    # tile 1 has landed (tile 2 may still be in flight)
+    lab_t1, lab_t1d = label("t1"), label("t1d")
+    e("s_cmp_lt_u32 %s, 3" % s(NT))
+    e("s_cbranch_scc1 %s" % lab_t1)
+    e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
+    e("s_branch %s" % lab_t1d)
+    e("%s:" % lab_t1)
+    e("s_waitcnt vmcnt(0)")
+    e("%s:" % lab_t1d)
+    e("s_barrier")
+    # first V^T fragments of tile 0
+    e("v_add_u32 %s, %s, %s" % (v(VADDR), s(OFF0), v(VADDR_LANE)))
+    v_warm(VADDR)
+    # ------------------------------------------------------------------ main loop (two copies: the register groups swap roles)
     lab_loop, lab_end = label("loop"), label("end")
+    stamp(2)
     e("%s:" % lab_loop)
-    r1 = half_iteration(SA, SB, "A")
+    r1 = iteration(SA, SB, "A")
     e("s_cmp_ge_u32 %s, %s" % (s(IT), s(NT)))
     e("s_cbranch_scc1 %s" % lab_end)
-    r2 = half_iteration(SB, SA, "B")
+    r2 = iteration(SB, SA, "B")
     e("s_cmp_lt_u32 %s, %s" % (s(IT), s(NT)))
     e("s_cbranch_scc1 %s" % lab_loop)
     e("s_branch %s" % lab_end)
@@ -611,6 +700,7 @@ def main():
             e("%s:" % resc)
             rescale_block(back)
     e("%s:" % lab_end)
+    stamp(3)
     # ------------------------------------------------------------------ epilogue
     e("s_nop 7")
     e("s_nop 7")
@@ -674,6 +764,7 @@ def main():
             e("s_nop 1")
             e("v_addc_co_u32 %s, vcc, 0, %s, vcc" % (v(OPTR + 1), v(OPTR + 1)))
     e("%s:" % lab_sdone)
+    stamp(4)
     # (m, l) of this split, written by the g == 0 lane of each row when a pointer was handed over
     e("v_cmp_ne_u64 vcc, 0, %s" % v(MLPTR, 2))
     e("s_nop 1")
@@ -684,6 +775,17 @@ def main():
     e("global_store_dwordx2 %s, %s, off" % (v(MLPTR, 2), v(T[0], 2)))
     e("s_mov_b64 exec, %s" % s(EXS, 2))
     e("s_waitcnt vmcnt(0)")
+    stamp(5)
+    if CLK:
+        lab = label("noclk")
+        e("s_cmp_lg_u32 %s, 0" % s(WAVE))
+        e("s_cbranch_scc1 %s" % lab)
+        e("v_mov_b32 %s, %d" % (v(X0), HOFF))
+        for k, reg in enumerate([80, 82, 84, 86, 88, 90, 92, 93, 100]):
+            e("v_mov_b32 %s, %s" % (v(X1), s(reg)))
+            e("ds_write_b32 %s, %s offset:%d" % (v(X0), v(X1), 4 * k))
+        e("s_waitcnt lgkmcnt(0)")
+        e("%s:" % lab)
 
     print("// generated by gen_decode_asm.py%s -- do not edit" % (" --f16" if F16 else ""))
     for ln in out:
