@@ -247,8 +247,35 @@ def v_warm(vaddr):
             v_read(vaddr, idx)
 
 
-def v_warm_tags():
-    return [] if NO_PV or NO_VREAD else [("v", idx, h) for idx in range(VRING - 1) for h in range(2)]
+def canon_tags():
+    """LDS reads in flight at the top of every iteration, in issue order (see tile_handover)."""
+    vt = lambda idx: [] if NO_PV or NO_VREAD else [("v", idx, 0), ("v", idx, 1)]
+    kt = [] if NO_QK or NO_KREAD else [("k", p) for p in range(KRING - 1)]
+    t = []
+    for idx in range(2, VRING - 1):
+        t += vt(idx)
+    return t + kt + vt(0) + vt(1)
+
+
+def tile_handover(kaddr_off, vaddr_off, last_slots, sync):
+    """The hand-over from tile IT to tile IT+1, placed before the last two P.V MFMAs of tile IT so that it costs no
+    MFMA time: first fragment reads of the next iteration (V^T of tile IT+1 from the buffer at s[vaddr_off], K of tile
+    IT+2 from s[kaddr_off]) around the wait for the tile loads and the workgroup barrier (`sync` emits them).
+    Ring slots 0 and 1 of the V^T ring are still needed by the last two MFMAs, so fragments 0 and 1 follow them."""
+    if not NO_PV:
+        lds.need(("v", 31, 1))          # every read of tile IT's buffer has returned: the buffer may be overwritten
+        e("v_add_u32 %s, %s, %s" % (v(VADDR), s(vaddr_off), v(VADDR_LANE)))
+        for idx in range(2, VRING - 1):
+            v_read(VADDR, idx)
+    sync()
+    e("v_add_u32 %s, %s, %s" % (v(KADDR), s(kaddr_off), v(KADDR_LANE)))
+    k_warm(KADDR)
+    for n in range(2):
+        if n < len(last_slots):
+            last_slots[n]()
+        if not NO_PV:
+            v_read(VADDR, n)
+    assert lds.pending == canon_tags(), (lds.pending, canon_tags())
 
 
 def pv_slots(vaddr, greg):
@@ -405,7 +432,6 @@ def iteration(g_cur, g_next, tag):
     e("s_add_u32 %s, %s, %s" % (s(S0), s(S0), s(KVB)))
     e("s_sub_u32 %s, %s, %s" % (s(NVAL), s(KVE), s(S0)))
     e("s_min_u32 %s, %s, 32" % (s(NVAL), s(NVAL)))
-    e("v_add_u32 %s, %s, %s" % (v(KADDR), s(OFF1), v(KADDR_LANE)))
     e("s_mov_b32 %s, 0" % s(VMW))
     e("s_mov_b64 %s, 0" % s(RSC, 2))
     lab_last, lab_nodma, lab_p2, lab_end = label("last"), label("nodma"), label("p2"), label("iend")
@@ -419,8 +445,7 @@ def iteration(g_cur, g_next, tag):
         e("s_branch %s" % lab_nodma)
 
     def part1(dma):
-        lds.pending = v_warm_tags()
-        k_warm(KADDR)
+        lds.pending = canon_tags()
         qk = qk_slots(g_next, KADDR)
         pv = pv_slots(VADDR, g_cur)
         n1 = min(P1_PV, len(pv))
@@ -452,11 +477,23 @@ def iteration(g_cur, g_next, tag):
     if len(head) < 2:
         e("s_nop 7")
     mask_tail(g_next)
-    interleave(rest_b[2:], softmax_lines(g_next), 4)
-    # first V^T fragments of tile IT+1 (next iteration's P.V starts without waiting for LDS)
-    e("v_add_u32 %s, %s, %s" % (v(VADDR), s(OFF1), v(VADDR_LANE)))
-    v_warm(VADDR)
-    assert lds.pending == v_warm_tags(), lds.pending
+    body = rest_b[2:]
+    tail = body[-2:] if len(body) >= 2 else []
+    interleave(body[:len(body) - len(tail)], softmax_lines(g_next), 4)
+
+    def sync():
+        # the DMA of tile IT+2 has landed (the one of tile IT+3, issued in this iteration, may still be in flight:
+        # loads complete in order, so vmcnt(DMA_PER_TILE) is enough); every wave is done with tile IT's buffer
+        lab_w0, lab_wd = label("w0"), label("wd")
+        e("s_cmp_eq_u32 %s, 0" % s(VMW))
+        e("s_cbranch_scc1 %s" % lab_w0)
+        e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
+        e("s_branch %s" % lab_wd)
+        e("%s:" % lab_w0)
+        e("s_waitcnt vmcnt(0)")
+        e("%s:" % lab_wd)
+        e("s_barrier")
+    tile_handover(OFF2, OFF1, tail, sync)
     if CLKP:
         e("s_memtime s[98:99]")
         e("s_waitcnt lgkmcnt(0)")
@@ -467,7 +504,7 @@ def iteration(g_cur, g_next, tag):
     e("s_branch %s" % lab_end)
     # ---- last tile: P.V only
     e("%s:" % lab_last)
-    lds.pending = v_warm_tags()
+    lds.pending = canon_tags()
     for sl in pv_slots(VADDR, g_cur):
         sl()
     lds.drain()
@@ -478,33 +515,6 @@ def iteration(g_cur, g_next, tag):
     e("s_cbranch_scc1 %s" % lab_resc)
     e("%s:" % lab_back)
     resc.append((lab_resc, lab_back))
-    # ---- end of tile: the DMA of tile IT+2 has landed (the one of tile IT+3, issued in this iteration, may still be
-    # in flight: loads complete in order, so vmcnt(DMA_PER_TILE) is enough); everyone is done with tile IT
-    lab_w0, lab_wd = label("w0"), label("wd")
-    if CLK and not CLKP:
-        e("s_memtime s[94:95]")
-        e("s_waitcnt lgkmcnt(0)")
-    e("s_cmp_eq_u32 %s, 0" % s(VMW))
-    e("s_cbranch_scc1 %s" % lab_w0)
-    e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
-    e("s_branch %s" % lab_wd)
-    e("%s:" % lab_w0)
-    e("s_waitcnt vmcnt(0)")
-    e("%s:" % lab_wd)
-    if CLK and not CLKP:
-        e("s_memtime s[96:97]")
-        e("s_waitcnt lgkmcnt(0)")
-        e("s_sub_u32 s96, s96, s94")
-        e("s_add_u32 s92, s92, s96")       # cycles spent waiting for the tile loads
-        e("s_mov_b32 s94, s96")
-        e("s_memtime s[96:97]")
-        e("s_waitcnt lgkmcnt(0)")
-    e("s_barrier")
-    if CLK and not CLKP:
-        e("s_memtime s[98:99]")
-        e("s_waitcnt lgkmcnt(0)")
-        e("s_sub_u32 s98, s98, s96")
-        e("s_add_u32 s93, s93, s98")       # cycles spent in the barrier
     e("s_mov_b32 %s, %s" % (s(TMP), s(OFF0)))
     e("s_mov_b32 %s, %s" % (s(OFF0), s(OFF1)))
     e("s_mov_b32 %s, %s" % (s(OFF1), s(OFF2)))
@@ -670,19 +680,19 @@ def main():
     mask_tail(SA)
     for ln in softmax_lines(SA):
         e(ln)
-    # tile 1 has landed (tile 2 may still be in flight)
-    lab_t1, lab_t1d = label("t1"), label("t1d")
-    e("s_cmp_lt_u32 %s, 3" % s(NT))
-    e("s_cbranch_scc1 %s" % lab_t1)
-    e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
-    e("s_branch %s" % lab_t1d)
-    e("%s:" % lab_t1)
-    e("s_waitcnt vmcnt(0)")
-    e("%s:" % lab_t1d)
-    e("s_barrier")
-    # first V^T fragments of tile 0
-    e("v_add_u32 %s, %s, %s" % (v(VADDR), s(OFF0), v(VADDR_LANE)))
-    v_warm(VADDR)
+    # tile 1 has landed (tile 2 may still be in flight); first fragment reads of iteration 0
+    def sync0():
+        lab_t1, lab_t1d = label("t1"), label("t1d")
+        e("s_cmp_lt_u32 %s, 3" % s(NT))
+        e("s_cbranch_scc1 %s" % lab_t1)
+        e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
+        e("s_branch %s" % lab_t1d)
+        e("%s:" % lab_t1)
+        e("s_waitcnt vmcnt(0)")
+        e("%s:" % lab_t1d)
+        e("s_barrier")
+    assert not lds.pending
+    tile_handover(OFF1, OFF0, [], sync0)
     # ------------------------------------------------------------------ main loop (two copies: the register groups swap roles)
     lab_loop, lab_end = label("loop"), label("end")
     stamp(2)
