@@ -741,8 +741,8 @@ def main():
     e("s_and_b64 exec, exec, vcc")
     # O^T block i, element 4j+c is column 32 i + 8 j + 4 g + c.
     # Final output (FLG bit 0): row-major rows of dst; the out pointer already includes the 4*g float offset.
-    # Split-K partial: layout [column/4][row][4 floats] so that the 32 lanes of a half-wave write 512 contiguous bytes;
-    # the out pointer already includes (g*n_rows + row)*16 bytes and every (i, j) step advances it by 2*n_rows*16 bytes.
+    # Split-K partial: f16, layout [column/8][row][8] so that the 64 lanes of a wave write 512 contiguous bytes;
+    # the out pointer already includes row*16 + g*8 bytes and every (i, j) step advances it by n_rows*16 bytes.
     lab_pstore, lab_sdone = label("pstore"), label("sdone")
     if NO_STORE:
         e("s_branch %s" % lab_sdone)
@@ -758,7 +758,7 @@ def main():
             e("global_store_dwordx4 %s, %s, off offset:%d" % (v(OPTR, 2), v(r, 4), (32 * i + 8 * j) * 4))
     e("s_branch %s" % lab_sdone)
     e("%s:" % lab_pstore)
-    # partial: O / l of this split as f16, layout [column/4][row][4 halves]; T[2] holds 1/l here as well
+    # partial: O / l of this split as f16, layout [column/8][row][8 halves]; T[2] holds 1/l here as well
     for i in range(16):
         for j in range(4):
             r = T[4] if (i * 4 + j) % 2 == 0 else SA

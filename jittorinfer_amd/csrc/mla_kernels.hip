@@ -370,7 +370,7 @@ __global__ void __launch_bounds__(NTHREADS) mla_attn_tile_kernel(const KParams p
     } else {
         const int64_t prow   = ((int64_t) b * p.n_splits + split) * p.n_rows + row;
         const int64_t pblock = ((int64_t) b * p.n_splits + split) * p.n_rows * p.dv_total;
-        // partial = O / l of this split, stored as f16 in layout [column/4][row][4]: coalesced for the writers here and
+        // partial = O / l of this split, stored as f16 in layout [column/8][row][8]: coalesced for the writers here and
         // for the combine pass, and half the bytes of f32 (the 2^-11 rounding is averaged over the splits)
         const float pinv = 1.0f / l_tot;
 #pragma unroll
@@ -379,7 +379,7 @@ __global__ void __launch_bounds__(NTHREADS) mla_attn_tile_kernel(const KParams p
             for (int j = 0; j < 4; j++) {
                 const int d0 = p.d_off + (wd * NDBW + i) * 32 + 8 * j + 4 * g;
                 u32x2 v = { pack2<true>(acc[i][4 * j] * pinv, acc[i][4 * j + 1] * pinv), pack2<true>(acc[i][4 * j + 2] * pinv, acc[i][4 * j + 3] * pinv) };
-                *(u32x2 *) (p.part_o + pblock + ((int64_t) (d0 >> 2) * p.n_rows + row) * 4) = v;
+                *(u32x2 *) (p.part_o + pblock + ((int64_t) (d0 >> 3) * p.n_rows + row) * 8 + (d0 & 7)) = v;
             }
         if (wd == 0 && g == 0 && p.d_off == 0) {
             p.part_ml[prow * 2]     = m_run;
@@ -389,39 +389,59 @@ __global__ void __launch_bounds__(NTHREADS) mla_attn_tile_kernel(const KParams p
 }
 
 // Log-sum-exp merge of the split-K partials: out = sum_c (O_c/l_c) l_c 2^(m_c - M) / sum_c l_c 2^(m_c - M).
-// Partials hold O_c/l_c as f16, laid out [seq][split][column/4][row][4].  One thread = one (row, group of 4 columns);
-// a block is 32 rows x 8 column groups, so each load instruction of a wave reads runs of 256 contiguous bytes and
-// each output row segment written by the block is 128 contiguous bytes.
-// grid = (ceil(n_rows/32), ceil(dv/32), n_seq), block = 256.
+// Partials hold O_c/l_c as f16, laid out [seq][split][column/8][row][8].  One thread = one (row, group of 8 columns):
+// 16-byte loads, lanes along rows (contiguous in the partial layout), splits in groups of 8 so that all the loads of a
+// group are in flight together.  grid = (ceil(rows/32), ceil(dv/64), n_seq), block = 256 = 32 rows x 8 column groups.
 __global__ void __launch_bounds__(256) mla_attn_combine_kernel(const KParams p) {
     const int b = blockIdx.z;
     const int row = blockIdx.x * 32 + (threadIdx.x & 31);
     const int cg  = blockIdx.y * 8 + (threadIdx.x >> 5);
-    if (row >= p.n_rows || cg * 4 >= p.dv_total) return;
+    if (row >= p.n_rows || cg * 8 >= p.dv_total) return;
     const int seq_len = p.block_table ? min(p.seq_lens[b], (int) p.bt_stride * MLA_PAGE_TOKENS) : (int) p.n_kv;
     int nvalid = (seq_len + p.split_tokens - 1) / p.split_tokens;
     nvalid = min(nvalid, p.n_splits);
 
-    const float *    ml = p.part_ml + ((int64_t) b * p.n_splits * p.n_rows + row) * 2;
-    const _Float16 * po = p.part_o + (int64_t) b * p.n_splits * p.n_rows * p.dv_total + ((int64_t) cg * p.n_rows + row) * 4;
-    const int64_t ml_step = (int64_t) p.n_rows * 2, po_step = (int64_t) p.n_rows * p.dv_total;
+    const float2 *   ml = (const float2 *) p.part_ml + (int64_t) b * p.n_splits * p.n_rows + row;
+    const _Float16 * po = p.part_o + (int64_t) b * p.n_splits * p.n_rows * p.dv_total + ((int64_t) cg * p.n_rows + row) * 8;
+    const int64_t ml_step = p.n_rows, po_step = (int64_t) p.n_rows * p.dv_total;
 
-    float M = -INFINITY;
-    for (int c = 0; c < nvalid; c++) M = fmaxf(M, ml[c * ml_step]);
-    const float Mu = (M == -INFINITY) ? 0.f : M;
-    float L = 0.f;
-    f32x4 o = { 0.f, 0.f, 0.f, 0.f };
-    for (int c = 0; c < nvalid; c++) {
-        const float mc = ml[c * ml_step];
-        if (mc == -INFINITY) continue;  // that split saw only masked keys
-        const float w = ml[c * ml_step + 1] * fast_exp2(mc - Mu);  // l_c 2^(m_c - M)
-        L += w;
-        const u32x2 hv = *(const u32x2 *) (po + c * po_step);
-        o.x += f16_bits_to_f32(hv.x & 0xffff) * w; o.y += f16_bits_to_f32(hv.x >> 16) * w;
-        o.z += f16_bits_to_f32(hv.y & 0xffff) * w; o.w += f16_bits_to_f32(hv.y >> 16) * w;
+    float M = -INFINITY, L = 0.f;
+    float o[8] = { 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f };
+    for (int c0 = 0; c0 < nvalid; c0 += 8) {
+        float2 mlv[8];
+        u32x4  hv[8];
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const int c = min(c0 + k, nvalid - 1);  // past the end: a duplicate of the last split, given weight 0 below
+            mlv[k] = ml[c * ml_step];
+            hv[k]  = *(const u32x4 *) (po + c * po_step);
+        }
+        float Mg = M;
+#pragma unroll
+        for (int k = 0; k < 8; k++) if (c0 + k < nvalid) Mg = fmaxf(Mg, mlv[k].x);
+        if (Mg == -INFINITY) continue;  // every split so far saw only masked keys
+        const float r = fast_exp2(M - Mg);  // 0 when M was -inf
+        M = Mg;
+        L *= r;
+#pragma unroll
+        for (int k = 0; k < 8; k++) o[k] *= r;
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            // l_c 2^(m_c - M); a split that saw only masked keys (m_c = -inf) and the padding of the group get 0
+            const float w = (c0 + k < nvalid && mlv[k].x != -INFINITY) ? mlv[k].y * fast_exp2(mlv[k].x - M) : 0.f;
+            L += w;
+            const unsigned h[4] = { hv[k].x, hv[k].y, hv[k].z, hv[k].w };
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                o[2 * e]     += f16_bits_to_f32(h[e] & 0xffff) * w;
+                o[2 * e + 1] += f16_bits_to_f32(h[e] >> 16) * w;
+            }
+        }
     }
     const float inv = 1.0f / L;  // no valid key at all: 0 * inf = NaN, like the reference
-    *(f32x4 *) (p.dst + ((int64_t) b * p.n_rows + row) * p.dst_stride + cg * 4) = f32x4{ o.x * inv, o.y * inv, o.z * inv, o.w * inv };
+    float * out = p.dst + ((int64_t) b * p.n_rows + row) * p.dst_stride + cg * 8;
+    *(f32x4 *) out       = f32x4{ o[0] * inv, o[1] * inv, o[2] * inv, o[3] * inv };
+    *(f32x4 *) (out + 4) = f32x4{ o[4] * inv, o[5] * inv, o[6] * inv, o[7] * inv };
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -697,7 +717,7 @@ static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
         if (e != hipSuccess) return (int) e;
     }
     if (pl.n_splits > 1 && (phases & 2)) {
-        dim3 g((unsigned) ((kp.n_rows + 31) / 32), (unsigned) ((a->dv + 31) / 32), (unsigned) a->n_seq);
+        dim3 g((unsigned) ((kp.n_rows + 31) / 32), (unsigned) ((a->dv + 63) / 64), (unsigned) a->n_seq);
         hipLaunchKernelGGL(mla_attn_combine_kernel, g, dim3(256), 0, st, kp);
         return (int) hipGetLastError();
     }
