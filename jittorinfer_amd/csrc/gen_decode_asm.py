@@ -27,6 +27,7 @@ NO_STORE = "--no-store" in sys.argv
 NO_QLOAD = "--no-qload" in sys.argv
 CLKP = "--clk-parts" in sys.argv    # with --clk: accumulate the cycles of part 1 / part 2 of the iterations instead of the waits
 CLK = "--clk" in sys.argv or CLKP           # timing experiments only: s_memtime stamps, written to the hand-off area at the end
+MASK = "--mask" in sys.argv  # additive f16 mask rows (one per query token), added to the scaled scores
 F16 = "--f16" in sys.argv  # f16 KV: f16 MFMA, single P (no lo half)
 MF = "v_mfma_f32_32x32x16_f16" if F16 else "v_mfma_f32_32x32x16_bf16"
 CVT = "v_cvt_pk_f16_f32" if F16 else "v_cvt_pk_bf16_f32"
@@ -50,9 +51,11 @@ P1_LEAD = _opt("--lead", 3)                   # P.V MFMAs at the head of an iter
 # ---- VGPR map
 Q0 = 0
 SA, SB = 144, 160   # two 16-register groups: scores of one tile, converted in place to its P^T operands
-KF, KRING = 176, 5  # K fragment ring (5 x 4 registers)
+KF, KRING = 176, 4 if MASK else 5   # K fragment ring (x 4 registers)
 ALPHA = 196
-VF, VRING = 200, 6  # V^T fragment ring (6 x 4 registers)
+MOFF = 197                          # mask builds: byte offset of this lane's first mask element inside a tile's 64 mask bytes
+VF, VRING = 200, 5 if MASK else 6   # V^T fragment ring (x 4 registers)
+MKR = [192, 193, 194, 195, 220, 221, 222, 223]   # mask builds: the 16 f16 mask values of this lane's 16 tokens of a tile
 T = list(range(224, 232))
 OPTR, MLPTR = 232, 234
 KADDR_LANE, VADDR_LANE, MRUN, LRUN, NEGM = 236, 237, 238, 239, 240
@@ -64,6 +67,7 @@ DBG, TIDR = 230, 248   # debug builds only: T[6:7] holds the debug pointer until
 # ---- SGPR map (all inside the clobbered range s40..s79)
 KV, BT, KVB, KVE, CL2, NPP, NB1, FLG = 40, 42, 44, 45, 46, 47, 48, 49
 NT, IT, OFF0, OFF1, OFF2, WAVE, TB, TMP, NVM1 = 50, 51, 52, 53, 54, 55, 56, 58, 59
+SCL, L2E, MSK = 77, 73, 78   # mask builds: scale, log2(e) (the register of SCLS until the epilogue), mask base (QP's registers once Q is loaded)
 EXS, S0, S1, S2, S3, DMAB, NVAL, THR, PG0, RSC, SPITCH, SCLS, OFF3, VMW, OSTR, QP = 60, 62, 63, 64, 65, 66, 67, 68, 69, 70, 72, 73, 74, 75, 76, 78
 
 out = []
@@ -309,6 +313,15 @@ def pv_slots(vaddr, greg):
     return slots
 
 
+def mask_loads(tile_sreg):
+    """Mask builds: the 64 mask bytes of tile s[tile_sreg] for this lane's query token -> MKR (four 8-byte loads)."""
+    e("s_lshl_b32 %s, %s, 6" % (s(S0), s(tile_sreg)))
+    e("s_add_u32 %s, %s, %s" % (s(S0), s(MSK), s(S0)))
+    e("s_addc_u32 %s, %s, 0" % (s(S1), s(MSK + 1)))
+    for j in range(4):
+        e("global_load_dwordx2 %s, %s, %s offset:%d" % (v(MKR[2 * j], 2), v(MOFF), s(S0, 2), 16 * j))
+
+
 def softmax_lines(sreg):
     """Softmax of the scores in group sreg, as one list of VALU lines (no branches):
     tile max -> lazy max update (new max only where it grew by more than TAU) -> ALPHA (rescale factor of O and l,
@@ -319,6 +332,13 @@ def softmax_lines(sreg):
         return ["s_mov_b64 %s, 0" % s(RSC, 2)]
     L = []
     m = [T[0], T[1], T[2], T[3], T[4]]
+    if MASK:
+        # u = s * scale + mask (ggml-cpu.c:12048-12057 order), element k = token 8(k/4) + 4g + k%4
+        for k in range(16):
+            t = T[5 + (k & 1)]
+            L.append("v_cvt_f32_f16_sdwa %s, %s dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:WORD_%d" % (v(t), v(MKR[2 * (k // 4) + (k % 4) // 2]), k % 2))
+            L.append("v_fma_f32 %s, %s, %s, %s" % (v(sreg + k), v(sreg + k), s(SCL), v(t)))
+    CS = L2E if MASK else CL2           # factor from the values in sreg to log2 units
     L.append("v_max3_f32 %s, %s, %s, %s" % (v(m[0]), v(sreg + 0), v(sreg + 1), v(sreg + 2)))
     L.append("v_max3_f32 %s, %s, %s, %s" % (v(m[1]), v(sreg + 3), v(sreg + 4), v(sreg + 5)))
     L.append("v_max3_f32 %s, %s, %s, %s" % (v(m[2]), v(sreg + 6), v(sreg + 7), v(sreg + 8)))
@@ -332,7 +352,7 @@ def softmax_lines(sreg):
     L.append("v_permlane32_swap_b32 %s, %s" % (v(m[0]), v(m[1])))
     L.append("s_nop 1")
     L.append("v_max_f32 %s, %s, %s" % (v(TMAX), v(m[0]), v(m[1])))
-    L.append("v_mul_f32 %s, %s, %s" % (v(TMAX), s(CL2), v(TMAX)))          # log2 units (c_log2 > 0)
+    L.append("v_mul_f32 %s, %s, %s" % (v(TMAX), s(CS), v(TMAX)))           # log2 units (the factor is > 0)
     L.append("v_add_f32 %s, %s, %s" % (v(m[2]), s(THR), v(MRUN)))           # m_run + TAU  (-inf stays -inf)
     L.append("v_sub_f32 %s, %s, %s" % (v(m[3]), v(MRUN), v(TMAX)))          # m_run - tmax
     L.append("v_exp_f32 %s, %s" % (v(m[3]), v(m[3])))                       # 2^(m_run - tmax); 0 when m_run = -inf
@@ -350,7 +370,7 @@ def softmax_lines(sreg):
     L.append("v_cndmask_b32 %s, %s, 0, vcc" % (v(NEGM), v(NEGM)))
     # p = 2^(s*c - m)
     for k in range(16):
-        L.append("v_fma_f32 %s, %s, %s, %s" % (v(sreg + k), v(sreg + k), s(CL2), v(NEGM)))
+        L.append("v_fma_f32 %s, %s, %s, %s" % (v(sreg + k), v(sreg + k), s(CS), v(NEGM)))
     for k in range(16):
         L.append("v_exp_f32 %s, %s" % (v(sreg + k), v(sreg + k)))
     # running sum (this lane's 16 tokens)
@@ -438,6 +458,8 @@ def iteration(g_cur, g_next, tag):
     e("s_add_u32 %s, %s, 1" % (s(TMP), s(IT)))
     e("s_cmp_ge_u32 %s, %s" % (s(TMP), s(NT)))
     e("s_cbranch_scc1 %s" % lab_last)
+    if MASK:
+        mask_loads(TMP)              # mask of tile IT+1: behind the loads of tile IT+2, ahead of those of tile IT+3
     e("s_add_u32 %s, %s, 3" % (s(TMP), s(IT)))
     e("s_cmp_ge_u32 %s, %s" % (s(TMP), s(NT)))
     e("s_cbranch_scc1 %s" % lab_nodma)
@@ -477,6 +499,15 @@ def iteration(g_cur, g_next, tag):
     if len(head) < 2:
         e("s_nop 7")
     mask_tail(g_next)
+    if MASK:
+        lab_m0, lab_md = label("m0"), label("md")
+        e("s_cmp_eq_u32 %s, 0" % s(VMW))
+        e("s_cbranch_scc1 %s" % lab_m0)
+        e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
+        e("s_branch %s" % lab_md)
+        e("%s:" % lab_m0)
+        e("s_waitcnt vmcnt(0)")
+        e("%s:" % lab_md)
     body = rest_b[2:]
     tail = body[-2:] if len(body) >= 2 else []
     interleave(body[:len(body) - len(tail)], softmax_lines(g_next), 4)
@@ -545,6 +576,9 @@ def main():
     if DEBUG:
         e("v_mov_b32 %s, %s" % (v(TIDR), v(X0)))
     e("s_mov_b32 %s, 0x%08x" % (s(THR), 0x41000000))  # TAU = 8.0f
+    if MASK:
+        e("s_mov_b32 %s, %%[scl]" % s(SCL))
+        e("s_mov_b32 %s, 0x3fb8aa3b" % s(L2E))
     e("v_and_b32 %s, 63, %s" % (v(LANE), v(X0)))
     e("v_lshrrev_b32 %s, 6, %s" % (v(X1), v(X0)))
     e("s_nop 0")
@@ -559,6 +593,8 @@ def main():
     e("v_mov_b32 %s, %s" % (v(OPTR + 1), v(T[3])))
     e("v_mov_b32 %s, %s" % (v(MLPTR), v(T[4])))
     e("v_mov_b32 %s, %s" % (v(MLPTR + 1), v(T[5])))
+    if MASK:
+        e("v_mov_b32 %s, %s" % (v(MOFF), v(T[0])))
     # lane geometry
     e("v_and_b32 %s, 31, %s" % (v(X0), v(LANE)))                       # rl
     e("v_lshrrev_b32 %s, 5, %s" % (v(X1), v(LANE)))                    # g
@@ -604,6 +640,16 @@ def main():
             e("s_add_u32 %s, %s, 4096" % (s(QP), s(QP)))
             e("s_addc_u32 %s, %s, 0" % (s(QP + 1), s(QP + 1)))
         e("global_load_dwordx4 %s, %s, %s offset:%d" % (v(Q0 + 4 * ks, 4), v(X0), s(QP, 2), (ks % 4) * 1024))
+    n_early = nq
+    if MASK:
+        # mask rows start at key kv_begin of this split; QP's registers are free now
+        e("s_mov_b64 %s, %%[msk]" % s(MSK, 2))
+        e("s_lshl_b32 %s, %s, 1" % (s(S0), s(KVB)))
+        e("s_add_u32 %s, %s, %s" % (s(MSK), s(MSK), s(S0)))
+        e("s_addc_u32 %s, %s, 0" % (s(MSK + 1), s(MSK + 1)))
+        e("s_mov_b32 %s, 0" % s(TMP))
+        mask_loads(TMP)
+        n_early += 4
     # ------------------------------------------------------------------ state
     e("v_mov_b32 %s, 0xff800000" % v(MRUN))
     e("v_mov_b32 %s, 0" % v(LRUN))
@@ -614,8 +660,8 @@ def main():
     e("s_mov_b32 %s, 0" % s(IT))
     for i in range(256):
         e("v_accvgpr_write_b32 %s, 0" % a(i))
-    # page ids have arrived (loads return in order: only the Q loads may still be in flight)
-    e("s_waitcnt vmcnt(%d)" % nq)
+    # page ids have arrived (loads return in order: only the Q and mask loads may still be in flight)
+    e("s_waitcnt vmcnt(%d)" % n_early)
     e("v_max_i32 %s, 0, %s" % (v(PAGES), v(PAGES)))
     e("v_min_i32 %s, %s, %s" % (v(PAGES), s(NPP), v(PAGES)))
     stamp(6)
@@ -797,7 +843,7 @@ def main():
         e("s_waitcnt lgkmcnt(0)")
         e("%s:" % lab)
 
-    print("// generated by gen_decode_asm.py%s -- do not edit" % (" --f16" if F16 else ""))
+    print("// generated by gen_decode_asm.py%s%s -- do not edit" % (" --f16" if F16 else "", " --mask" if MASK else ""))
     for ln in out:
         print('"%s\\n\\t"' % ln)
 

@@ -524,7 +524,7 @@ struct Plan {
     int    n_splits, split_tokens;
     int    n_passes, ndb;
     size_t lds_bytes;
-    size_t ws_part_o, ws_part_ml, ws_scores, ws_qpack;
+    size_t ws_part_o, ws_part_ml, ws_scores, ws_qpack, ws_maskext;
 };
 
 int validate(const mla_attn_args * a) {
@@ -601,6 +601,7 @@ int make_plan(const mla_attn_args * a, Plan * pl) {
     pl->n_splits     = (int) ((n_pages + pages_per_split - 1) / pages_per_split);
     pl->lds_bytes    = pl->variant == 2 ? decode_fast_lds_bytes() : 2 * TILE_BYTES + (a->kv_type == MLA_TYPE_Q8_0 ? Q8_TILE_RAW : 0);
     if (pl->variant == 2) pl->ws_qpack = decode_fast_qpack_bytes(a->n_seq, pl->n_row_blocks);
+    if (pl->variant == 2 && a->mask) pl->ws_maskext = (size_t) pl->n_row_blocks * sizeof(int);
     if (pl->n_splits > 1) {
         pl->ws_part_o  = (size_t) a->n_seq * pl->n_splits * n_rows * a->dv * sizeof(_Float16);
         pl->ws_part_ml = (size_t) a->n_seq * pl->n_splits * n_rows * 2 * sizeof(float);
@@ -609,7 +610,9 @@ int make_plan(const mla_attn_args * a, Plan * pl) {
 }
 
 size_t align256(size_t x) { return (x + 255) & ~(size_t) 255; }
-size_t plan_ws(const Plan & pl) { return align256(pl.ws_part_o) + align256(pl.ws_part_ml) + align256(pl.ws_scores) + align256(pl.ws_qpack); }
+size_t plan_ws(const Plan & pl) {
+    return align256(pl.ws_part_o) + align256(pl.ws_part_ml) + align256(pl.ws_scores) + align256(pl.ws_qpack) + align256(pl.ws_maskext);
+}
 
 template <int SRC, int NDB, int WM, int WD>
 hipError_t launch_tile(const KParams & kp, dim3 grid, size_t lds, hipStream_t st) {
@@ -690,6 +693,7 @@ static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
     kp.part_ml = (float *) (ws + align256(pl.ws_part_o));
     float * scores = (float *) (ws + align256(pl.ws_part_o) + align256(pl.ws_part_ml));
     kp.q_pack = ws + align256(pl.ws_part_o) + align256(pl.ws_part_ml) + align256(pl.ws_scores);
+    kp.mask_ext = (int *) (ws + align256(pl.ws_part_o) + align256(pl.ws_part_ml) + align256(pl.ws_scores) + align256(pl.ws_qpack));
 
     if (pl.variant == 1) {
         if (!(phases & 1)) return 0;

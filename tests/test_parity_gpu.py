@@ -109,3 +109,58 @@ def test_dv576_matches_ggml_cpu_layout(gpu, k_type):
     got = _run(gpu, q, k, k_type, dv=576, scale=U.SCALE)
     want = O.flash_attn_ext(q, k, k_type, dv=576, scale=U.SCALE)
     print(U.check(got, want, "dv 576"))
+
+
+def _plan_variant(gpu, q, k, k_type, mask, bt, lens, **kw):
+    import torch
+    import jittorinfer_amd as J
+    tq = torch.from_numpy(q).to(gpu)
+    tk = torch.from_numpy(k.view(np.int16) if k.dtype == np.uint16 else k).to(gpu)
+    tm = torch.from_numpy(mask.view(np.float16)).to(gpu)
+    tb = None if bt is None else torch.from_numpy(bt).to(gpu)
+    tl = None if lens is None else torch.from_numpy(np.asarray(lens, dtype=np.int32)).to(gpu)
+    return J.plan(tq, tk, k_type, dv=512, mask=tm, block_table=tb, seq_lens=tl, **kw)["variant"]
+
+
+@pytest.mark.parametrize("k_type", [O.TYPE_BF16, O.TYPE_F16])
+@pytest.mark.parametrize("n_splits", [0, 1, 3])
+def test_masked_prefill_pipelined_kernel(gpu, k_type, n_splits):
+    """Causal chunked prefill through the pipelined kernel's mask path: 72 new tokens on 300 cached ones, 16 heads,
+    2 sequences sharing the mask (ggml-cpu.c:12024), mask rows as wide as the block table's pages (384 keys)."""
+    rng = np.random.default_rng(40 + n_splits)
+    n_new, n_old = 72, 300
+    lens = [n_new + n_old] * 2
+    pool, bt, seqs = U.make_paged(rng, lens, k_type)
+    q = rng.standard_normal((2, 16, n_new, 576)).astype(np.float32)
+    width = bt.shape[1] * 128
+    kv_pos = np.arange(width)[None, :]
+    mask = np.where((kv_pos > n_old + np.arange(n_new)[:, None]) | (kv_pos >= n_new + n_old), -np.inf, 0.0).astype(np.float16).view(np.uint16)
+    assert _plan_variant(gpu, q, pool, k_type, mask, bt, lens, scale=U.SCALE, n_splits=n_splits) == 2
+    got = _run(gpu, q, pool, k_type, mask=mask, bt=bt, lens=lens, scale=U.SCALE, n_splits=n_splits)
+    if k_type == O.TYPE_F16:
+        # f32 accumulation here against ggml-cpu's f16 accumulator: held to the f64 value, as in test_contiguous_decode
+        want = np.stack([O.flash_attn_ext_f64(q[b:b + 1], k[None], k_type, dv=512, mask=mask[:, :k.shape[0]], scale=U.SCALE)[0]
+                         for b, k in enumerate(seqs)])
+    else:
+        want = U.oracle_per_seq(q, seqs, k_type, 512, mask=mask)
+    print(U.check(got[..., :512], want, "masked prefill"))
+
+
+@pytest.mark.parametrize("n_splits", [0, 2, 4])
+def test_masked_decode_random_mask(gpu, n_splits):
+    """Contiguous KV, 128 heads, 3 query tokens: a mask of finite biases and -inf holes, one query token whose keys are
+    all masked (NaN rows, like the reference's 0 * (1/0)), one that sees only the first 40 keys (whole splits masked)."""
+    rng = np.random.default_rng(50 + n_splits)
+    n_kv, n_tok = 512, 3
+    q = rng.standard_normal((2, 128, n_tok, 576)).astype(np.float32)
+    k = U.encode_kv(rng.standard_normal((2, n_kv, 576)).astype(np.float32), O.TYPE_BF16)
+    m = (rng.standard_normal((n_tok, n_kv)) * 2).astype(np.float32)
+    m[rng.random((n_tok, n_kv)) < 0.3] = -np.inf
+    m[1, :] = -np.inf
+    m[2, 40:] = -np.inf
+    mask = m.astype(np.float16).view(np.uint16)
+    assert _plan_variant(gpu, q, k, O.TYPE_BF16, mask, None, None, scale=U.SCALE, n_splits=n_splits) == 2
+    got = _run(gpu, q, k, O.TYPE_BF16, mask=mask, scale=U.SCALE, n_splits=n_splits)
+    want = O.flash_attn_ext(q, k, O.TYPE_BF16, dv=512, mask=mask, scale=U.SCALE)
+    assert np.isnan(want[:, 1]).all()
+    print(U.check(got[..., :512], want, "masked decode"))
