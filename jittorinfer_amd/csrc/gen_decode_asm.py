@@ -28,16 +28,23 @@ NO_QLOAD = "--no-qload" in sys.argv
 CLKP = "--clk-parts" in sys.argv    # with --clk: accumulate the cycles of part 1 / part 2 of the iterations instead of the waits
 CLK = "--clk" in sys.argv or CLKP           # timing experiments only: s_memtime stamps, written to the hand-off area at the end
 MASK = "--mask" in sys.argv  # additive f16 mask rows (one per query token), added to the scaled scores
-F16 = "--f16" in sys.argv  # f16 KV: f16 MFMA, single P (no lo half)
+Q8 = "--q8" in sys.argv    # Q8_0 KV: raw tiles staged in LDS, dequantized to an f16 tile one tile ahead, then the f16 path
+F16 = "--f16" in sys.argv or Q8  # f16 KV: f16 MFMA, single P (no lo half)
+assert not (Q8 and MASK)
 MF = "v_mfma_f32_32x32x16_f16" if F16 else "v_mfma_f32_32x32x16_bf16"
 CVT = "v_cvt_pk_f16_f32" if F16 else "v_cvt_pk_bf16_f32"
 SPLIT = not F16
 
 PITCH = 1168
 TILE_BYTES = 32 * PITCH
-NBUF = 4
-HOFF = NBUF * TILE_BYTES       # hand-off area written by the C++ prologue: 32 bytes per thread
-DMA_PER_TILE = 10              # LDS-DMA instructions each wave issues per tile
+NBUF = 3 if Q8 else 4          # 16-bit tiles resident in LDS
+Q8_ROW = 612                   # 18 blocks of (f16 d, 32 x int8)
+RAW_TILE = 32 * Q8_ROW         # 19584 = 1224 x 16 bytes; Q8_0 builds keep two raw tiles behind the 16-bit tiles
+RAW0 = NBUF * TILE_BYTES
+RAW1 = RAW0 + RAW_TILE
+HOFF = RAW1 + RAW_TILE if Q8 else NBUF * TILE_BYTES   # hand-off area written by the C++ prologue: 32 bytes per thread
+DMA_PER_TILE = 5 if Q8 else 10 # LDS-DMA instructions each wave issues per tile
+Q8_WAVE_CHUNKS = 306           # a wave copies 306 of the 1224 16-byte chunks of a raw tile
 CPR = 73                       # 16-byte chunks per padded row
 WAVE_CHUNKS = 8 * CPR          # 584: each wave moves rows 8w..8w+7 of a tile
 TAU = 8.0
@@ -54,7 +61,7 @@ SA, SB = 144, 160   # two 16-register groups: scores of one tile, converted in p
 KF, KRING = 176, 4 if MASK else 5   # K fragment ring (x 4 registers)
 ALPHA = 196
 MOFF = 197                          # mask builds: byte offset of this lane's first mask element inside a tile's 64 mask bytes
-VF, VRING = 200, 5 if MASK else 6   # V^T fragment ring (x 4 registers)
+VF, VRING = 200, 5 if MASK or Q8 else 6   # V^T fragment ring (x 4 registers); 220..223 go to the mask values / the dequantizer
 MKR = [192, 193, 194, 195, 220, 221, 222, 223]   # mask builds: the 16 f16 mask values of this lane's 16 tokens of a tile
 T = list(range(224, 232))
 OPTR, MLPTR = 232, 234
@@ -67,6 +74,9 @@ DBG, TIDR = 230, 248   # debug builds only: T[6:7] holds the debug pointer until
 # ---- SGPR map (all inside the clobbered range s40..s79)
 KV, BT, KVB, KVE, CL2, NPP, NB1, FLG = 40, 42, 44, 45, 46, 47, 48, 49
 NT, IT, OFF0, OFF1, OFF2, WAVE, TB, TMP, NVM1 = 50, 51, 52, 53, 54, 55, 56, 58, 59
+RAWC, RAWN, SH, SHM2, PSEL = 74, 77, 78, 79, 72   # Q8_0 builds: raw buffer to dequantize / to load into (OFF3's and a free register), byte shifts and the
+                                                  # v_perm selector of the dequantizer (QP's and SPITCH's registers once the prologue is done with them)
+RAWB, DSTB, DZ = 197, 198, 199                    # Q8_0 builds: per-lane raw window / f16 destination offsets, all-ones where this lane's row is valid
 SCL, L2E, MSK = 77, 73, 78   # mask builds: scale, log2(e) (the register of SCLS until the epilogue), mask base (QP's registers once Q is loaded)
 EXS, S0, S1, S2, S3, DMAB, NVAL, THR, PG0, RSC, SPITCH, SCLS, OFF3, VMW, OSTR, QP = 60, 62, 63, 64, 65, 66, 67, 68, 69, 70, 72, 73, 74, 75, 76, 78
 
@@ -139,17 +149,24 @@ def interleave(mfma_slots, valu, per_slot):
         take = max(per_slot, -(-(len(valu) - vi) // remaining_slots)) if vi < len(valu) else 0
         for _ in range(take):
             if vi < len(valu):
-                e(valu[vi])
+                emit_item(valu[vi])
                 vi += 1
     while vi < len(valu):
-        e(valu[vi])
+        emit_item(valu[vi])
         vi += 1
 
 
+def emit_item(x):
+    """A shadow item is a line or a callable that emits lines (LDS accesses go through the tracker)."""
+    if callable(x):
+        x()
+    else:
+        e(x)
+
+
 # ---------------------------------------------------------------------------------------------------------------
-def dma_tile_lines(tile_sreg, off_sreg):
-    """Instruction list (to be interleaved) that issues the LDS-DMA loads of tile index s[tile_sreg] into the buffer
-    at LDS offset s[off_sreg].  Scalar part first (tile base address), then 10 slots."""
+def tile_base_lines(tile_sreg):
+    """Scalar lines: s[TB:TB+1] = address of the first row of tile s[tile_sreg]; s[NVM1] = its valid rows - 1."""
     L = []
     # t0 = kv_begin + 32*tile ; nvalid-1 = min(32, kv_end - t0) - 1
     L.append("s_lshl_b32 %s, %s, 5" % (s(S0), s(tile_sreg)))
@@ -171,6 +188,109 @@ def dma_tile_lines(tile_sreg, off_sreg):
     L.append("s_mul_i32 %s, %s, %s" % (s(S0), s(S0), s(NB1)))
     L.append("s_add_u32 %s, %s, %s" % (s(TB), s(KV), s(S0)))
     L.append("s_addc_u32 %s, %s, %s" % (s(TB + 1), s(KV + 1), s(S1)))
+    return L
+
+
+DQ_LOFF = 227   # lane * 16 for the flat raw-tile copy; as DQ_OUT + 3 the last register the dequantizer overwrites afterwards
+
+
+def q8_dma_lines(tile_sreg, raw_sreg):
+    """Q8_0 builds: the 19584 bytes of tile s[tile_sreg] (32 packed rows, contiguous in the pool) -> the raw buffer at
+    LDS offset s[raw_sreg], as a flat copy: 306 chunks per wave, 4 full LDS-DMA instructions and one of 50 lanes."""
+    L = tile_base_lines(tile_sreg)
+    L.append("s_mul_i32 %s, %s, %d" % (s(DMAB), s(WAVE), Q8_WAVE_CHUNKS * 16))
+    L.append("s_add_u32 %s, %s, %s" % (s(TB), s(TB), s(DMAB)))
+    L.append("s_addc_u32 %s, %s, 0" % (s(TB + 1), s(TB + 1)))
+    L.append("s_add_u32 %s, %s, %s" % (s(DMAB), s(DMAB), s(raw_sreg)))
+    L.append("v_lshlrev_b32 %s, 4, %s" % (v(DQ_LOFF), v(LANE)))
+    # no instruction offset on an LDS-DMA load: it would move the LDS address as well; the scalar base steps instead
+    for j in range(4):
+        L.append("\\n\\t".join(["s_add_u32 m0, %s, %d" % (s(DMAB), j * 1024),
+                                "s_nop 0",
+                                "global_load_lds_dwordx4 %s, %s" % (v(DQ_LOFF), s(TB, 2)),
+                                "s_add_u32 %s, %s, 1024" % (s(TB), s(TB)),
+                                "s_addc_u32 %s, %s, 0" % (s(TB + 1), s(TB + 1))]))
+    L.append("\\n\\t".join(["s_add_u32 m0, %s, %d" % (s(DMAB), 4 * 1024),
+                            "s_mov_b64 %s, exec" % s(EXS, 2),
+                            "s_mov_b32 exec_lo, -1",
+                            "s_mov_b32 exec_hi, 0x3ffff",                      # lanes 0..49
+                            "global_load_lds_dwordx4 %s, %s" % (v(DQ_LOFF), s(TB, 2)),
+                            "s_mov_b64 exec, %s" % s(EXS, 2)]))
+    return L
+
+
+DQ_OUT = 224                                  # T[0:3]: the 8 f16 values of a unit
+DQ_W = [(228, 229, 241), (230, 231, 251)]     # two 12-byte raw windows (the next unit's reads are in flight during a unit's arithmetic)
+DQ_D = [249, 221]                             # the block scales of the two units in flight
+RAWA, DSTA, RAWD = 242, 243, 220
+
+
+def q8_dequant_items(raw_sreg, dst_sreg, tile_plus):
+    """Q8_0 builds: raw tile at LDS offset s[raw_sreg] -> f16 tile at s[dst_sreg] (padded row layout).  A unit is
+    8 values (one 16-byte destination chunk); a wave does 576 units in 9 steps: waves 0/1 the even blocks of rows
+    0-15/16-31, waves 2/3 the odd blocks, lane = (row, quarter of the block).  The int8 values of an even block start
+    2 bytes past a 4-byte boundary, those of an odd block on one: a unit reads the 12-byte window from that boundary and
+    the same code shifts by s[SH] = 2 or 0 bytes; the block's f16 scale is read on its own (2-byte aligned).
+    value = f16(q) * d in packed f16: one rounding of an exact product, the same number as f16(q * f32(d)).
+    Rows past the end of the sequence become zeros (their bytes are not KV data).  tile_plus: the tile is IT + tile_plus."""
+    I = []
+    # valid rows of that tile: clamp(kv_end - kv_begin - 32*(IT + tile_plus), 0, 32), times the row pitch of the f16 tile
+    I.append("s_add_u32 %s, %s, %d" % (s(S0), s(IT), tile_plus))
+    I.append("s_lshl_b32 %s, %s, 5" % (s(S0), s(S0)))
+    I.append("s_add_u32 %s, %s, %s" % (s(S0), s(S0), s(KVB)))
+    I.append("s_sub_i32 %s, %s, %s" % (s(S0), s(KVE), s(S0)))
+    I.append("s_max_i32 %s, %s, 0" % (s(S0), s(S0)))
+    I.append("s_min_i32 %s, %s, 32" % (s(S0), s(S0)))
+    I.append("s_mul_i32 %s, %s, %d" % (s(S0), s(S0), PITCH))
+    I.append("v_cmp_gt_u32 vcc, %s, %s" % (s(S0), v(DSTB)))                      # row * PITCH + (< PITCH) < n_valid * PITCH
+    I.append("v_add_u32 %s, %s, %s" % (v(RAWA), s(raw_sreg), v(RAWB)))
+    I.append("v_add_u32 %s, %s, %s" % (v(DSTA), s(dst_sreg), v(DSTB)))
+    I.append("v_cndmask_b32_e64 %s, 0, -1, vcc" % v(DZ))
+    # the scale of (row, block 2u + parity) sits 8q (+ 2 for odd blocks) bytes before the window
+    I.append("v_and_b32 %s, 3, %s" % (v(RAWD), v(LANE)))
+    I.append("v_lshlrev_b32 %s, 3, %s" % (v(RAWD), v(RAWD)))
+    I.append("v_add_u32 %s, %s, %s" % (v(RAWD), s(SHM2), v(RAWD)))
+    I.append("v_sub_u32 %s, %s, %s" % (v(RAWD), v(RAWA), v(RAWD)))
+
+    def reads(u):
+        w = DQ_W[u & 1]
+        def f0():
+            lds.read("ds_read2_b32 %s, %s offset0:%d offset1:%d" % (v(w[0], 2), v(RAWA), 17 * u, 17 * u + 1), ("r", u, 0))
+        def f1():
+            lds.read("ds_read_b32 %s, %s offset:%d" % (v(w[2]), v(RAWA), 68 * u + 8), ("r", u, 1))
+        def f2():
+            lds.read("ds_read_u16 %s, %s offset:%d" % (v(DQ_D[u & 1]), v(RAWD), 68 * u), ("r", u, 2))
+        return [f0, f1, f2]
+
+    I += reads(0)
+    for u in range(9):
+        w, d = DQ_W[u & 1], DQ_D[u & 1]
+        if u + 1 < 9:
+            I += reads(u + 1)
+        def first(u=u, w=w):
+            lds.need(("r", u, 2))
+            e("v_alignbyte_b32 %s, %s, %s, %s" % (v(w[0]), v(w[1]), v(w[0]), s(SH)))      # values 0..3
+        I.append(first)
+        I.append("v_alignbyte_b32 %s, %s, %s, %s" % (v(w[1]), v(w[2]), v(w[1]), s(SH)))   # values 4..7
+        I.append("v_perm_b32 %s, %s, %s, %s" % (v(d), v(d), v(d), s(PSEL)))              # d in both halves
+        I.append("v_and_b32 %s, %s, %s" % (v(d), v(d), v(DZ)))
+        for h in range(2):
+            for j in range(4):
+                el = 2 * j + h
+                I.append("v_cvt_f16_i16_sdwa %s, sext(%s) dst_sel:WORD_%d dst_unused:%s src0_sel:BYTE_%d" % (
+                    v(DQ_OUT + j), v(w[el // 4]), h, "UNUSED_PAD" if h == 0 else "UNUSED_PRESERVE", el % 4))
+        for j in range(4):
+            I.append("v_pk_mul_f16 %s, %s, %s" % (v(DQ_OUT + j), v(DQ_OUT + j), v(d)))
+        def wr(u=u):
+            lds.read("ds_write_b128 %s, %s offset:%d" % (v(DSTA), v(DQ_OUT, 4), 128 * u), ("w", u))
+        I.append(wr)
+    return I
+
+
+def dma_tile_lines(tile_sreg, off_sreg):
+    """Instruction list (to be interleaved) that issues the LDS-DMA loads of tile index s[tile_sreg] into the buffer
+    at LDS offset s[off_sreg].  Scalar part first (tile base address), then 10 slots."""
+    L = tile_base_lines(tile_sreg)
     # LDS destination of this wave's first slot
     L.append("s_mul_i32 %s, %s, %d" % (s(DMAB), s(WAVE), WAVE_CHUNKS * 16))
     L.append("s_add_u32 %s, %s, %s" % (s(DMAB), s(DMAB), s(off_sreg)))
@@ -271,6 +391,8 @@ def tile_handover(kaddr_off, vaddr_off, last_slots, sync):
         e("v_add_u32 %s, %s, %s" % (v(VADDR), s(vaddr_off), v(VADDR_LANE)))
         for idx in range(2, VRING - 1):
             v_read(VADDR, idx)
+    if Q8:
+        lds.need(("w", 8))              # this wave's share of the next f16 tile is written
     sync()
     e("v_add_u32 %s, %s, %s" % (v(KADDR), s(kaddr_off), v(KADDR_LANE)))
     k_warm(KADDR)
@@ -481,13 +603,16 @@ def iteration(g_cur, g_next, tag):
 
     # ---- part 1 with the DMA of tile IT+3
     e("s_mov_b32 %s, 1" % s(VMW))
-    rest_a = part1(dma_tile_lines(TMP, OFF3))
+    if Q8:
+        rest_a = part1(q8_dma_lines(TMP, RAWN) + q8_dequant_items(RAWC, OFF2, 2))
+    else:
+        rest_a = part1(dma_tile_lines(TMP, OFF3))
     state_a = list(lds.pending)
     e("s_branch %s" % lab_p2)
     # ---- part 1 without it (tiles IT+3.. do not exist)
     e("%s:" % lab_nodma)
-    rest_b = part1([])
-    assert lds.pending == state_a and len(rest_a) == len(rest_b)
+    rest_b = part1(q8_dequant_items(RAWC, OFF2, 2) if Q8 else [])
+    assert lds.pending == state_a and len(rest_a) == len(rest_b), (lds.pending, state_a)
     # ---- part 2: remaining P.V MFMAs of tile IT, softmax of tile IT+1 in their shadow
     e("%s:" % lab_p2)
     if CLKP:
@@ -516,13 +641,16 @@ def iteration(g_cur, g_next, tag):
         # the DMA of tile IT+2 has landed (the one of tile IT+3, issued in this iteration, may still be in flight:
         # loads complete in order, so vmcnt(DMA_PER_TILE) is enough); every wave is done with tile IT's buffer
         lab_w0, lab_wd = label("w0"), label("wd")
-        e("s_cmp_eq_u32 %s, 0" % s(VMW))
-        e("s_cbranch_scc1 %s" % lab_w0)
-        e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
-        e("s_branch %s" % lab_wd)
-        e("%s:" % lab_w0)
-        e("s_waitcnt vmcnt(0)")
-        e("%s:" % lab_wd)
+        if Q8:
+            e("s_waitcnt vmcnt(0)")     # the raw tile loaded during this iteration is dequantized in the next one
+        else:
+            e("s_cmp_eq_u32 %s, 0" % s(VMW))
+            e("s_cbranch_scc1 %s" % lab_w0)
+            e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
+            e("s_branch %s" % lab_wd)
+            e("%s:" % lab_w0)
+            e("s_waitcnt vmcnt(0)")
+            e("%s:" % lab_wd)
         e("s_barrier")
     tile_handover(OFF2, OFF1, tail, sync)
     if CLKP:
@@ -549,8 +677,14 @@ def iteration(g_cur, g_next, tag):
     e("s_mov_b32 %s, %s" % (s(TMP), s(OFF0)))
     e("s_mov_b32 %s, %s" % (s(OFF0), s(OFF1)))
     e("s_mov_b32 %s, %s" % (s(OFF1), s(OFF2)))
-    e("s_mov_b32 %s, %s" % (s(OFF2), s(OFF3)))
-    e("s_mov_b32 %s, %s" % (s(OFF3), s(TMP)))
+    if Q8:
+        e("s_mov_b32 %s, %s" % (s(OFF2), s(TMP)))
+        e("s_mov_b32 %s, %s" % (s(TMP), s(RAWC)))
+        e("s_mov_b32 %s, %s" % (s(RAWC), s(RAWN)))
+        e("s_mov_b32 %s, %s" % (s(RAWN), s(TMP)))
+    else:
+        e("s_mov_b32 %s, %s" % (s(OFF2), s(OFF3)))
+        e("s_mov_b32 %s, %s" % (s(OFF3), s(TMP)))
     e("s_add_u32 %s, %s, 1" % (s(IT), s(IT)))
     return resc
 
@@ -665,30 +799,83 @@ def main():
     e("v_max_i32 %s, 0, %s" % (v(PAGES), v(PAGES)))
     e("v_min_i32 %s, %s, %s" % (v(PAGES), s(NPP), v(PAGES)))
     stamp(6)
-    # ------------------------------------------------------------------ tiles 0, 1, 2 -> LDS; go on as soon as Q and tile 0 are there
-    lab_w0, lab_w1, lab_wd = label("pw0"), label("pw1"), label("pwd")
-    e("s_mov_b32 %s, 0" % s(TMP))
-    for ln in dma_tile_lines(TMP, OFF0):
-        e(ln)
-    e("s_cmp_lt_u32 %s, 2" % s(NT))
-    e("s_cbranch_scc1 %s" % lab_w0)
-    e("s_mov_b32 %s, 1" % s(TMP))
-    for ln in dma_tile_lines(TMP, OFF1):
-        e(ln)
-    e("s_cmp_lt_u32 %s, 3" % s(NT))
-    e("s_cbranch_scc1 %s" % lab_w1)
-    e("s_mov_b32 %s, 2" % s(TMP))
-    for ln in dma_tile_lines(TMP, OFF2):
-        e(ln)
-    e("s_waitcnt vmcnt(%d)" % (2 * DMA_PER_TILE))
-    e("s_branch %s" % lab_wd)
-    e("%s:" % lab_w1)
-    e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
-    e("s_branch %s" % lab_wd)
-    e("%s:" % lab_w0)
-    e("s_waitcnt vmcnt(0)")
-    e("%s:" % lab_wd)
-    e("s_barrier")
+    if Q8:
+        # ------------------------------------------------------------------ Q8_0: per-lane offsets of the dequantizer
+        e("v_lshrrev_b32 %s, 2, %s" % (v(X0), v(LANE)))
+        e("s_and_b32 %s, %s, 1" % (s(S0), s(WAVE)))
+        e("s_lshl_b32 %s, %s, 4" % (s(S0), s(S0)))
+        e("v_add_u32 %s, %s, %s" % (v(X0), s(S0), v(X0)))                  # row = 16*(wave&1) + lane/4
+        e("v_and_b32 %s, 3, %s" % (v(X1), v(LANE)))                        # quarter of the block
+        e("s_lshr_b32 %s, %s, 1" % (s(S1), s(WAVE)))                       # 0: even blocks, 1: odd blocks
+        e("v_lshlrev_b32 %s, 3, %s" % (v(X2), v(X1)))
+        e("s_mov_b32 %s, %d" % (s(S2), Q8_ROW))
+        e("v_mad_u32_u24 %s, %s, %s, %s" % (v(RAWB), v(X0), s(S2), v(X2)))  # row*612 + 8q: window of (even block 0, quarter q)
+        e("s_mul_i32 %s, %s, 36" % (s(S2), s(S1)))
+        e("v_add_u32 %s, %s, %s" % (v(RAWB), s(S2), v(RAWB)))              # odd blocks: + 34 + 2: their values are 4-byte aligned
+        e("v_lshlrev_b32 %s, 4, %s" % (v(X2), v(X1)))
+        e("v_mad_u32_u24 %s, %s, %s, %s" % (v(DSTB), v(X0), s(SPITCH), v(X2)))
+        e("s_lshl_b32 %s, %s, 6" % (s(S2), s(S1)))
+        e("v_add_u32 %s, %s, %s" % (v(DSTB), s(S2), v(DSTB)))              # odd blocks: + 32 columns
+        e("s_lshl_b32 %s, %s, 1" % (s(SHM2), s(S1)))                       # 0 / 2
+        e("s_sub_u32 %s, 2, %s" % (s(SH), s(SHM2)))                        # 2 / 0
+        e("s_mov_b32 %s, 0x01000100" % s(PSEL))
+        e("s_mov_b32 %s, %d" % (s(RAWC), RAW0))
+        e("s_mov_b32 %s, %d" % (s(RAWN), RAW1))
+        # ------------------------------------------------------------------ raw tiles 0 and 1 -> LDS, tile 0 -> f16
+        lab_w0, lab_wd = label("pw0"), label("pwd")
+        e("s_mov_b32 %s, 0" % s(TMP))
+        for ln in q8_dma_lines(TMP, RAWC):
+            e(ln)
+        e("s_cmp_lt_u32 %s, 2" % s(NT))
+        e("s_cbranch_scc1 %s" % lab_w0)
+        e("s_mov_b32 %s, 1" % s(TMP))
+        for ln in q8_dma_lines(TMP, RAWN):
+            e(ln)
+        e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
+        e("s_branch %s" % lab_wd)
+        e("%s:" % lab_w0)
+        e("s_waitcnt vmcnt(0)")
+        e("%s:" % lab_wd)
+        e("s_barrier")
+        for it_ in q8_dequant_items(RAWC, OFF0, 0):
+            emit_item(it_)
+        lds.need(("w", 8))
+        e("s_waitcnt vmcnt(0)")
+        e("s_barrier")                      # f16 tile 0 complete, raw tile 1 landed, raw buffer 0 free
+        lab_n2 = label("pn2")
+        e("s_cmp_lt_u32 %s, 3" % s(NT))
+        e("s_cbranch_scc1 %s" % lab_n2)
+        e("s_mov_b32 %s, 2" % s(TMP))
+        for ln in q8_dma_lines(TMP, RAWC):
+            e(ln)
+        e("%s:" % lab_n2)
+        for it_ in q8_dequant_items(RAWN, OFF1, 1):
+            emit_item(it_)
+    else:
+        # ------------------------------------------------------------------ tiles 0, 1, 2 -> LDS; go on as soon as Q and tile 0 are there
+        lab_w0, lab_w1, lab_wd = label("pw0"), label("pw1"), label("pwd")
+        e("s_mov_b32 %s, 0" % s(TMP))
+        for ln in dma_tile_lines(TMP, OFF0):
+            e(ln)
+        e("s_cmp_lt_u32 %s, 2" % s(NT))
+        e("s_cbranch_scc1 %s" % lab_w0)
+        e("s_mov_b32 %s, 1" % s(TMP))
+        for ln in dma_tile_lines(TMP, OFF1):
+            e(ln)
+        e("s_cmp_lt_u32 %s, 3" % s(NT))
+        e("s_cbranch_scc1 %s" % lab_w1)
+        e("s_mov_b32 %s, 2" % s(TMP))
+        for ln in dma_tile_lines(TMP, OFF2):
+            e(ln)
+        e("s_waitcnt vmcnt(%d)" % (2 * DMA_PER_TILE))
+        e("s_branch %s" % lab_wd)
+        e("%s:" % lab_w1)
+        e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
+        e("s_branch %s" % lab_wd)
+        e("%s:" % lab_w0)
+        e("s_waitcnt vmcnt(0)")
+        e("%s:" % lab_wd)
+        e("s_barrier")
     stamp(1)
     if DEBUG:
         # FLG bit 1: dump LDS tile 0 (2336 chunks) to the debug pointer and stop
@@ -729,6 +916,10 @@ def main():
     # tile 1 has landed (tile 2 may still be in flight); first fragment reads of iteration 0
     def sync0():
         lab_t1, lab_t1d = label("t1"), label("t1d")
+        if Q8:
+            e("s_waitcnt vmcnt(0)")     # f16 tile 1 written (the hand-over waited for this wave's writes), raw tile 2 landed
+            e("s_barrier")
+            return
         e("s_cmp_lt_u32 %s, 3" % s(NT))
         e("s_cbranch_scc1 %s" % lab_t1)
         e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
@@ -737,7 +928,7 @@ def main():
         e("s_waitcnt vmcnt(0)")
         e("%s:" % lab_t1d)
         e("s_barrier")
-    assert not lds.pending
+    assert Q8 or not lds.pending
     tile_handover(OFF1, OFF0, [], sync0)
     # ------------------------------------------------------------------ main loop (two copies: the register groups swap roles)
     lab_loop, lab_end = label("loop"), label("end")
@@ -843,7 +1034,7 @@ def main():
         e("s_waitcnt lgkmcnt(0)")
         e("%s:" % lab)
 
-    print("// generated by gen_decode_asm.py%s%s -- do not edit" % (" --f16" if F16 else "", " --mask" if MASK else ""))
+    print("// generated by gen_decode_asm.py%s%s -- do not edit" % (" --q8" if Q8 else " --f16" if F16 else "", " --mask" if MASK else ""))
     for ln in out:
         print('"%s\\n\\t"' % ln)
 

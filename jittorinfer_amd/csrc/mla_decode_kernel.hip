@@ -18,9 +18,10 @@
 namespace mla {
 namespace {
 
-constexpr int NBUF        = 4;
-constexpr int HANDOFF_OFF = NBUF * TILE_BYTES;   // 32 bytes per thread: q pointer, out pointer, (m,l) pointer, row-valid flag
-constexpr int LDS_TOTAL   = HANDOFF_OFF + NTHREADS * 32;
+// LDS: 4 resident 16-bit tiles (bf16 / f16 KV), or 3 of them behind 2 raw Q8_0 tiles; then the hand-off area,
+// 32 bytes per thread: mask offset, out pointer, (m,l) pointer, debug pointer
+constexpr int handoff_off(int kvt) { return kvt == SRC_Q8 ? 3 * TILE_BYTES + 2 * Q8_TILE_RAW : 4 * TILE_BYTES; }
+constexpr int lds_total(int kvt) { return handoff_off(kvt) + NTHREADS * 32; }
 
 #define MLA_DECODE_CLOBBERS \
     "memory", "vcc", "scc", "s40", "s41", "s42", "s43", "s44", "s45", "s46", "s47", "s48", "s49", "s50", "s51", \
@@ -67,11 +68,14 @@ constexpr int LDS_TOTAL   = HANDOFF_OFF + NTHREADS * 32;
     [scl] "s"(s_scale), [tid] "v"(tid)
 
 // The wave-level program is generated by gen_decode_asm.py (register map, LDS-DMA issue, MFMA/VALU interleave).
-// F16 = false: bf16 KV rows, bf16 MFMA, P fed as hi + lo halves.   F16 = true: f16 KV rows, f16 MFMA, single P.
+// KVT = SRC_BF16: bf16 KV rows, bf16 MFMA, P fed as hi + lo halves.   SRC_F16: f16 KV rows, f16 MFMA, single P.
+// SRC_Q8: packed Q8_0 rows (612 bytes, contiguous), dequantized in LDS to f16 tiles one tile ahead, then as SRC_F16.
 // MASK: an f16 mask row per query token is added to the scaled scores (ggml-cpu.c:12041-12057); the keys past
 // p.mask_ext[row block] (the last key any row of the block may attend to, rounded up to a tile) are not visited.
-template <bool F16, bool MASK>
+template <int KVT, bool MASK>
 __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
+    constexpr int HANDOFF_OFF = handoff_off(KVT);
+    static_assert(!(KVT == SRC_Q8 && MASK), "no masked Q8_0 build of the wave program");
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -142,11 +146,15 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
     const int s_scale = __builtin_amdgcn_readfirstlane(__float_as_int(p.scale));
     const int s_ostr = __builtin_amdgcn_readfirstlane(p.n_rows * 16);  // bytes between the partial rows of column groups c and c+1
 
-    if constexpr (F16 && MASK) {
+    if constexpr (KVT == SRC_Q8) {
+        asm volatile(
+#include "mla_decode_asm_q8.inc"
+            : : MLA_DECODE_INPUTS : MLA_DECODE_CLOBBERS);
+    } else if constexpr (KVT == SRC_F16 && MASK) {
         asm volatile(
 #include "mla_decode_asm_f16_mask.inc"
             : : MLA_DECODE_INPUTS : MLA_DECODE_CLOBBERS);
-    } else if constexpr (F16) {
+    } else if constexpr (KVT == SRC_F16) {
         asm volatile(
 #include "mla_decode_asm_f16.inc"
             : : MLA_DECODE_INPUTS : MLA_DECODE_CLOBBERS);
@@ -214,15 +222,54 @@ __global__ void __launch_bounds__(NTHREADS) mla_mask_extent_kernel(const KParams
     if (tid == 0) p.mask_ext[blockIdx.x] = min(n_kv, (red[0] + TILE_TOK - 1) / TILE_TOK * TILE_TOK);
 }
 
+// The same image for Q8_0 KV: ggml-cpu quantizes Q to Q8_0 when K is Q8_0 (ggml-cpu.c:313-322, :12034-12035): per block of 32
+// d = amax/127 (stored as f16), id = 127/amax, q = round-half-even(x*id) (ggml-cpu-quants.c:855-900); the MFMA operand is the
+// dequantized value q * f16(d), rounded to f16.  grid = (n_row_blocks, n_seq, 18 blocks), block = 256: two k-steps per thread.
+__global__ void __launch_bounds__(NTHREADS) mla_q_pack_q8_kernel(const KParams p) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int g = lane >> 5, rl = lane & 31;
+    const int b = blockIdx.y, j = blockIdx.z;
+    const int row = min((int) blockIdx.x * 128 + wave * 32 + rl, p.n_rows - 1);
+    const int tq = row / p.n_head, head = row - tq * p.n_head;
+    const float * qrow = (const float *) (p.q + (int64_t) tq * p.q_nb1 + (int64_t) head * p.q_nb2 + (int64_t) b * p.q_nb3);
+    u32x4 * out = (u32x4 *) p.q_pack + ((((int64_t) b * gridDim.x + blockIdx.x) * 4 + wave) * KSTEPS) * 64 + lane;
+    f32x4 x[4];
+    x[0] = *(const f32x4 *) (qrow + 32 * j + 8 * g);
+    x[1] = *(const f32x4 *) (qrow + 32 * j + 8 * g + 4);
+    x[2] = *(const f32x4 *) (qrow + 32 * j + 16 + 8 * g);
+    x[3] = *(const f32x4 *) (qrow + 32 * j + 16 + 8 * g + 4);
+    float amax = 0.f;
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) amax = fmaxf(amax, fabsf(x[e][c]));
+    amax           = fmaxf(amax, xor32(amax));   // the other half of the block sits in lane ^ 32
+    const float d  = f16_bits_to_f32(f32_to_f16_bits(amax / 127.0f));
+    const float id = amax != 0.f ? 127.0f / amax : 0.f;
+    float y[16];
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) y[e * 4 + c] = rintf(x[e][c] * id) * d;
+    out[(2 * j) * 64]     = u32x4{ pack2<true>(y[0], y[1]), pack2<true>(y[2], y[3]), pack2<true>(y[4], y[5]), pack2<true>(y[6], y[7]) };
+    out[(2 * j + 1) * 64] = u32x4{ pack2<true>(y[8], y[9]), pack2<true>(y[10], y[11]), pack2<true>(y[12], y[13]), pack2<true>(y[14], y[15]) };
+}
+
 }  // namespace
 
-size_t decode_fast_lds_bytes() { return (size_t) LDS_TOTAL; }
+size_t decode_fast_lds_bytes(int kv_type) { return (size_t) lds_total(kv_type == MLA_TYPE_Q8_0 ? SRC_Q8 : SRC_BF16); }
 
 size_t decode_fast_qpack_bytes(int n_seq, int n_row_blocks) { return (size_t) n_seq * n_row_blocks * 4 * KSTEPS * 1024; }
 
 bool decode_fast_applicable(const mla_attn_args * a) {
-    if (a->kv_type != MLA_TYPE_BF16 && a->kv_type != MLA_TYPE_F16) return false;
+    if (a->kv_type != MLA_TYPE_BF16 && a->kv_type != MLA_TYPE_F16 && a->kv_type != MLA_TYPE_Q8_0) return false;
     if (a->dv != 512 || (a->flags & MLA_FLAG_F16_ACC_STRICT)) return false;
+    if (a->kv_type == MLA_TYPE_Q8_0) {
+        // raw tiles are copied as one run of 19584 bytes in 16-byte pieces: packed rows, 16-byte aligned tiles, whole tiles
+        // inside the allocation (always true for pages; a contiguous KV must end on a tile boundary); no masked build
+        if (a->mask || a->kv_nb1 != Q8_ROW || ((uintptr_t) a->kv & 15)) return false;
+        if (!a->block_table && ((a->kv_nb3 & 15) || a->n_kv % TILE_TOK)) return false;
+    }
     if (a->logit_softcap != 0.0f || a->max_bias > 0.0f) return false;
     if (a->mask) {
         // whole tiles only (no key past n_kv is touched in a mask row), 32-bit offsets into the mask, 8-byte aligned loads
@@ -235,29 +282,28 @@ bool decode_fast_applicable(const mla_attn_args * a) {
     return true;
 }
 
-hipError_t launch_decode_fast(const KParams & kp, int kv_type, dim3 grid, hipStream_t st) {
-    const size_t lds = decode_fast_lds_bytes();
-    static bool  attr_done[4] = { false, false, false, false };
-    const int    f = kv_type == MLA_TYPE_F16 ? 1 : 0, m = kp.mask ? 1 : 0, v = 2 * m + f;
-    const void * fns[4] = { (const void *) mla_decode_kernel<false, false>, (const void *) mla_decode_kernel<true, false>,
-                            (const void *) mla_decode_kernel<false, true>, (const void *) mla_decode_kernel<true, true> };
-    const void * fn = fns[v];
-    if (!attr_done[v]) {
+template <int KVT, bool MASK>
+static hipError_t launch_variant(const KParams & kp, dim3 grid, hipStream_t st) {
+    static bool attr_done = false;
+    const void * fn = (const void *) mla_decode_kernel<KVT, MASK>;
+    if (!attr_done) {
         hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
-        attr_done[v] = true;
+        attr_done = true;
     }
-    const dim3 pgrid(grid.y, grid.z, KSTEPS);
-    if (f) hipLaunchKernelGGL(mla_q_pack_kernel<true>, pgrid, dim3(NTHREADS), 0, st, kp);
-    else   hipLaunchKernelGGL(mla_q_pack_kernel<false>, pgrid, dim3(NTHREADS), 0, st, kp);
-    if (m) hipLaunchKernelGGL(mla_mask_extent_kernel, dim3(grid.y), dim3(NTHREADS), 0, st, kp);
-    switch (v) {
-        case 0: hipLaunchKernelGGL((mla_decode_kernel<false, false>), grid, dim3(NTHREADS), lds, st, kp); break;
-        case 1: hipLaunchKernelGGL((mla_decode_kernel<true, false>), grid, dim3(NTHREADS), lds, st, kp); break;
-        case 2: hipLaunchKernelGGL((mla_decode_kernel<false, true>), grid, dim3(NTHREADS), lds, st, kp); break;
-        default: hipLaunchKernelGGL((mla_decode_kernel<true, true>), grid, dim3(NTHREADS), lds, st, kp); break;
-    }
+    hipLaunchKernelGGL((mla_decode_kernel<KVT, MASK>), grid, dim3(NTHREADS), (size_t) lds_total(KVT), st, kp);
     return hipGetLastError();
+}
+
+hipError_t launch_decode_fast(const KParams & kp, int kv_type, dim3 grid, hipStream_t st) {
+    const bool m = kp.mask != nullptr;
+    if (kv_type == MLA_TYPE_Q8_0)     hipLaunchKernelGGL(mla_q_pack_q8_kernel, dim3(grid.y, grid.z, KSTEPS / 2), dim3(NTHREADS), 0, st, kp);
+    else if (kv_type == MLA_TYPE_F16) hipLaunchKernelGGL(mla_q_pack_kernel<true>, dim3(grid.y, grid.z, KSTEPS), dim3(NTHREADS), 0, st, kp);
+    else                              hipLaunchKernelGGL(mla_q_pack_kernel<false>, dim3(grid.y, grid.z, KSTEPS), dim3(NTHREADS), 0, st, kp);
+    if (m) hipLaunchKernelGGL(mla_mask_extent_kernel, dim3(grid.y), dim3(NTHREADS), 0, st, kp);
+    if (kv_type == MLA_TYPE_Q8_0) return launch_variant<SRC_Q8, false>(kp, grid, st);
+    if (kv_type == MLA_TYPE_F16)  return m ? launch_variant<SRC_F16, true>(kp, grid, st) : launch_variant<SRC_F16, false>(kp, grid, st);
+    return m ? launch_variant<SRC_BF16, true>(kp, grid, st) : launch_variant<SRC_BF16, false>(kp, grid, st);
 }
 
 }  // namespace mla

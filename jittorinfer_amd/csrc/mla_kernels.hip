@@ -599,7 +599,7 @@ int make_plan(const mla_attn_args * a, Plan * pl) {
     const int64_t pages_per_split = (n_pages + splits - 1) / splits;
     pl->split_tokens = (int) (pages_per_split * MLA_PAGE_TOKENS);
     pl->n_splits     = (int) ((n_pages + pages_per_split - 1) / pages_per_split);
-    pl->lds_bytes    = pl->variant == 2 ? decode_fast_lds_bytes() : 2 * TILE_BYTES + (a->kv_type == MLA_TYPE_Q8_0 ? Q8_TILE_RAW : 0);
+    pl->lds_bytes    = pl->variant == 2 ? decode_fast_lds_bytes(a->kv_type) : 2 * TILE_BYTES + (a->kv_type == MLA_TYPE_Q8_0 ? Q8_TILE_RAW : 0);
     if (pl->variant == 2) pl->ws_qpack = decode_fast_qpack_bytes(a->n_seq, pl->n_row_blocks);
     if (pl->variant == 2 && a->mask) pl->ws_maskext = (size_t) pl->n_row_blocks * sizeof(int);
     if (pl->n_splits > 1) {
