@@ -23,6 +23,8 @@ NO_SM = "--no-softmax" in sys.argv
 DMA_PLACE = "pv" if "--dma-pv" in sys.argv else "bulk" if "--dma-bulk" in sys.argv else "a"
 NO_VREAD = "--no-vread" in sys.argv
 NO_KREAD = "--no-kread" in sys.argv
+NO_DQ_VALU = "--no-dq-valu" in sys.argv   # timing experiments: Q8_0 dequantizer without its arithmetic / without its LDS traffic
+NO_DQ_LDS = "--no-dq-lds" in sys.argv
 NO_STORE = "--no-store" in sys.argv
 NO_QLOAD = "--no-qload" in sys.argv
 CLKP = "--clk-parts" in sys.argv    # with --clk: accumulate the cycles of part 1 / part 2 of the iterations instead of the waits
@@ -112,7 +114,7 @@ class Lds:
         self.pending = []
 
     def read(self, line, tag):
-        if (NO_VREAD and tag[0] == "v") or (NO_KREAD and tag[0] == "k"):
+        if (NO_VREAD and tag[0] == "v") or (NO_KREAD and tag[0] == "k") or (NO_DQ_LDS and tag[0] in "rw"):
             return
         e(line)
         self.pending.append(tag)
@@ -158,6 +160,8 @@ def interleave(mfma_slots, valu, per_slot):
 
 def emit_item(x):
     """A shadow item is a line or a callable that emits lines (LDS accesses go through the tracker)."""
+    if x is None:
+        return
     if callable(x):
         x()
     else:
@@ -271,6 +275,9 @@ def q8_dequant_items(raw_sreg, dst_sreg, tile_plus):
             lds.need(("r", u, 2))
             e("v_alignbyte_b32 %s, %s, %s, %s" % (v(w[0]), v(w[1]), v(w[0]), s(SH)))      # values 0..3
         I.append(first)
+        if NO_DQ_VALU:
+            I.append(lambda u=u: lds.read("ds_write_b128 %s, %s offset:%d" % (v(DSTA), v(DQ_OUT, 4), 128 * u), ("w", u)))
+            continue
         I.append("v_alignbyte_b32 %s, %s, %s, %s" % (v(w[1]), v(w[2]), v(w[1]), s(SH)))   # values 4..7
         I.append("v_perm_b32 %s, %s, %s, %s" % (v(d), v(d), v(d), s(PSEL)))              # d in both halves
         I.append("v_and_b32 %s, %s, %s" % (v(d), v(d), v(DZ)))
@@ -604,14 +611,16 @@ def iteration(g_cur, g_next, tag):
     # ---- part 1 with the DMA of tile IT+3
     e("s_mov_b32 %s, 1" % s(VMW))
     if Q8:
-        rest_a = part1(q8_dma_lines(TMP, RAWN) + q8_dequant_items(RAWC, OFF2, 2))
+        q8_dma = q8_dma_lines(TMP, RAWN)
+        rest_a = part1(q8_dma + q8_dequant_items(RAWC, OFF2, 2))
     else:
         rest_a = part1(dma_tile_lines(TMP, OFF3))
     state_a = list(lds.pending)
     e("s_branch %s" % lab_p2)
     # ---- part 1 without it (tiles IT+3.. do not exist)
     e("%s:" % lab_nodma)
-    rest_b = part1(q8_dequant_items(RAWC, OFF2, 2) if Q8 else [])
+    # (Q8_0: empty items in place of the loads, so that the dequantizer's LDS accesses fall into the same slots on both paths)
+    rest_b = part1([None] * len(q8_dma) + q8_dequant_items(RAWC, OFF2, 2) if Q8 else [])
     assert lds.pending == state_a and len(rest_a) == len(rest_b), (lds.pending, state_a)
     # ---- part 2: remaining P.V MFMAs of tile IT, softmax of tile IT+1 in their shadow
     e("%s:" % lab_p2)
@@ -641,6 +650,9 @@ def iteration(g_cur, g_next, tag):
         # the DMA of tile IT+2 has landed (the one of tile IT+3, issued in this iteration, may still be in flight:
         # loads complete in order, so vmcnt(DMA_PER_TILE) is enough); every wave is done with tile IT's buffer
         lab_w0, lab_wd = label("w0"), label("wd")
+        if CLK and not CLKP:
+            e("s_memtime s[94:95]")
+            e("s_waitcnt lgkmcnt(0)")
         if Q8:
             e("s_waitcnt vmcnt(0)")     # the raw tile loaded during this iteration is dequantized in the next one
         else:
@@ -651,7 +663,17 @@ def iteration(g_cur, g_next, tag):
             e("%s:" % lab_w0)
             e("s_waitcnt vmcnt(0)")
             e("%s:" % lab_wd)
+        if CLK and not CLKP:
+            e("s_memtime s[96:97]")
+            e("s_waitcnt lgkmcnt(0)")
+            e("s_sub_u32 s94, s96, s94")
+            e("s_add_u32 s92, s92, s94")       # cycles spent waiting for the tile loads
         e("s_barrier")
+        if CLK and not CLKP:
+            e("s_memtime s[98:99]")
+            e("s_waitcnt lgkmcnt(0)")
+            e("s_sub_u32 s98, s98, s96")
+            e("s_add_u32 s93, s93, s98")       # cycles spent in the barrier
     tile_handover(OFF2, OFF1, tail, sync)
     if CLKP:
         e("s_memtime s[98:99]")
@@ -1024,15 +1046,15 @@ def main():
     e("s_waitcnt vmcnt(0)")
     stamp(5)
     if CLK:
-        lab = label("noclk")
-        e("s_cmp_lg_u32 %s, 0" % s(WAVE))
-        e("s_cbranch_scc1 %s" % lab)
-        e("v_mov_b32 %s, %d" % (v(X0), HOFF))
+        # every wave leaves its stamps and accumulators in the hand-off area: 64 bytes per wave
+        e("s_lshl_b32 %s, %s, 6" % (s(S0), s(WAVE)))
+        e("s_add_u32 %s, %s, %d" % (s(S0), s(S0), HOFF))
+        e("v_mov_b32 %s, %s" % (v(X0), s(S0)))
         for k, reg in enumerate([80, 82, 84, 86, 88, 90, 92, 93, 100]):
             e("v_mov_b32 %s, %s" % (v(X1), s(reg)))
             e("ds_write_b32 %s, %s offset:%d" % (v(X0), v(X1), 4 * k))
         e("s_waitcnt lgkmcnt(0)")
-        e("%s:" % lab)
+        e("s_barrier")
 
     print("// generated by gen_decode_asm.py%s%s -- do not edit" % (" --q8" if Q8 else " --f16" if F16 else "", " --mask" if MASK else ""))
     for ln in out:
