@@ -41,6 +41,96 @@ def build_workload(dev, n_seq, n_head, ctx, n_pools, seed, kv="bf16"):
     return q, pools, block_table, seq_lens
 
 
+def build_paged(dev, lens, n_head, n_tok, kv, seed):
+    """Pages for sequences of the given lengths behind a shuffled block table (BASELINE configs 2, 4, 5)."""
+    import torch
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed)
+    nblk = [(l + 127) // 128 for l in lens]
+    n_pages = sum(nblk)
+    perm = torch.randperm(n_pages, generator=g, device=dev).to(torch.int32)
+    bt = torch.zeros((len(lens), max(nblk)), dtype=torch.int32, device=dev)
+    pos = 0
+    for b, n in enumerate(nblk):
+        bt[b, :n] = perm[pos:pos + n]
+        pos += n
+    if kv == "q8_0":
+        # int8 = clip(round(N(0,1) / scale)), one fp16 scale 1/32 per block (BASELINE config 5)
+        qs = torch.clamp(torch.round(torch.randn((n_pages * 128, 18, 32), generator=g, device=dev) * 32.0), -127, 127).to(torch.int8)
+        pool = torch.empty((n_pages * 128, 18, 34), dtype=torch.uint8, device=dev)
+        pool[:, :, 0] = 0x00
+        pool[:, :, 1] = 0x28   # fp16 0x2800 = 1/32
+        pool[:, :, 2:] = qs.view(torch.uint8)
+        pool = pool.reshape(n_pages * 128, 612)
+    else:
+        pool = torch.randn((n_pages * 128, 576), generator=g, device=dev).to(torch.bfloat16 if kv == "bf16" else torch.float16).view(torch.int16)
+    q = torch.randn((len(lens), n_head, n_tok, 576), generator=g, device=dev, dtype=torch.float32)
+    return q, pool, bt, torch.tensor(lens, dtype=torch.int32, device=dev)
+
+
+def other_config(a, dev, lib, J):
+    """BASELINE configs 2, 4 and 5 through the same C ABI: parity-test shapes, timed here for the profiles (not the
+    headline line).  One JSON line in the same format; the metric of the prefill config is its MFMA rate."""
+    import numpy as np
+    import torch
+    scale = 1.0 / (192.0 ** 0.5)
+    rng = np.random.default_rng(a.seed)
+    mask = None
+    if a.config == "c2":
+        lens, n_head, n_tok, kv, kvt = [int(x) for x in rng.integers(512, 4097, 8)], 16, 1, "bf16", J.MLA_TYPE_BF16
+        name = "BASELINE configs[1]: paged MLA decode B=8 H=16 L~U[512,4096], bf16"
+    elif a.config == "c4":
+        lens, n_head, n_tok, kv, kvt = [2560] * 4, 16, 512, "bf16", J.MLA_TYPE_BF16
+        mask = torch.where(torch.arange(2560, device=dev)[None, :] > 2048 + torch.arange(512, device=dev)[:, None], float("-inf"), 0.0).to(torch.float16)
+        name = "BASELINE configs[3]: chunked prefill B=4 H=16, 512 new on 2048 cached tokens, causal f16 mask, bf16 pages"
+    else:
+        lens, n_head, n_tok, kv, kvt = [int(x) for x in rng.integers(2048, 8193, 64)], 128, 1, "q8_0", J.MLA_TYPE_Q8_0
+        name = "BASELINE configs[4]: paged MLA decode B=64 H=128 L~U[2048,8192], Q8_0 pages"
+    q, pool, bt, sl = build_paged(dev, lens, n_head, n_tok, kv, a.seed)
+    out = torch.empty((len(lens), n_tok, n_head, 576), dtype=torch.float32, device=dev)
+    kw = dict(dv=512, scale=scale, mask=mask, block_table=bt, seq_lens=sl, out=out, n_splits=a.splits, rows_per_wg=a.rows_per_wg)
+    ar, _, keep = J.capi.make_args(q, pool, kvt, **kw)
+    plan = J.plan(q, pool, kvt, **kw)
+    stream = torch.cuda.current_stream(dev)
+    st = C.c_void_p(stream.cuda_stream)
+
+    def run(fn, n):
+        for _ in range(n):
+            rc = fn(C.byref(ar), st)
+            if rc != 0:
+                raise RuntimeError("launch failed: %d" % rc)
+
+    run(lib.mla_attn_launch, a.warmup)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    run(lib.mla_attn_launch, a.steps)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / a.steps
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    run(lib.mla_attn_launch_kernel, a.steps)
+    e1.record(stream)
+    torch.cuda.synchronize()
+    kern_ms = e0.elapsed_time(e1) / a.steps
+    if a.config == "c4":
+        n_old = 2048
+        kv_bytes = sum(lens) * KV_ROW_BYTES
+        flops = len(lens) * n_head * FLOP_PER_TOKEN_HEAD * (n_tok * n_old + n_tok * (n_tok + 1) // 2)
+        roof = {"bound": "mfma", "achieved": flops / (kern_ms * 1e-3) / 1e12, "peak": 2500.0, "unit": "TFLOP/s"}
+        metric, value, unit = "mla_prefill_attention_rate", flops / (ms * 1e-3) / 1e12, "TFLOP/s"
+    else:
+        kv_bytes = sum(lens) * (612 if kv == "q8_0" else KV_ROW_BYTES)
+        flops = sum(lens) * n_head * FLOP_PER_TOKEN_HEAD
+        roof = {"bound": "hbm", "achieved": kv_bytes / (kern_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s"}
+        metric, value, unit = "mla_paged_decode_kv_read_bandwidth", kv_bytes / (ms * 1e-3) / 1e9, "GB/s"
+    roof.update({"frac": roof["achieved"] / roof["peak"], "traffic": None, "kernel_us": {"mean": kern_ms * 1e3},
+                 "mfma_tflops": flops / (kern_ms * 1e-3) / 1e12, "algorithmic_bytes_per_launch": kv_bytes})
+    print(json.dumps({"metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+                      "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+                      "dtype": "f16" if kv == "q8_0" else kv, "data": "synthetic",
+                      "config": {"workload": name, "plan": plan}, "us_per_step": ms * 1e3, "roofline": roof, "cpu_baseline": None}))
+
+
 def cpu_baseline(q, pool, block_table, ctx, n_sample, scale, gpu_out):
     """ggml-cpu's flash_attn_ext on the host cores for the first n_sample sequences of the same workload:
     the reference's own compiled ggml when oracle/_ref is built (kind "reference"), else the C restatement ("port")."""
@@ -92,6 +182,8 @@ def main():
                     help="also launch the library's plain copy kernel N times over one KV pool (known byte count) so that a "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run can be scaled")
     ap.add_argument("--kv", default="bf16", choices=["bf16", "f16"], help="storage type of the latent KV pool (the headline config is bf16)")
+    ap.add_argument("--config", default="c3", choices=["c2", "c3", "c4", "c5"],
+                    help="c3 (default) is the headline workload; the others time BASELINE's remaining GPU configs for the profiles")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this build measures one GPU's share of the path; --gpus %d is not supported (use --gpus 1)" % a.gpus, file=sys.stderr)
@@ -105,6 +197,9 @@ def main():
     lib = J.library()
     dev = torch.device("cuda:0")
     scale = 1.0 / (192.0 ** 0.5)
+    if a.config != "c3":
+        other_config(a, dev, lib, J)
+        return
 
     q, pools, block_table, seq_lens = build_workload(dev, a.batch, a.heads, a.ctx, a.pools, a.seed, a.kv)
     kv_type = J.MLA_TYPE_BF16 if a.kv == "bf16" else J.MLA_TYPE_F16
@@ -137,12 +232,13 @@ def main():
     wall = time.perf_counter() - t0
     ms_per_step = wall * 1e3 / a.steps
 
-    # ---- the dominant kernel alone (the split-K decode kernel): HIP events on the launch stream around K back-to-back
-    # launches (the stream is in order, so this is K kernel durations plus the gaps between them)
+    # ---- the dominant kernel alone (the split-K decode kernel, without the Q pre-pack and the combine pass): HIP events
+    # on the launch stream around K back-to-back launches (the stream is in order, so this is K kernel durations plus the
+    # gaps between them)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record(stream)
     for i in range(a.steps):
-        step(i, lib.mla_attn_launch_partials)
+        step(i, lib.mla_attn_launch_kernel)   # the Q operand image in the workspace is the one the steps above wrote
     e1.record(stream)
     torch.cuda.synchronize()
     kern_ms = e0.elapsed_time(e1) / a.steps
@@ -177,7 +273,7 @@ def main():
     # counters read for the library's copy kernel; figures and commands in profiles/mla_decode_kernel_c3_pmc.md
     traffic = None
     if a.batch == 32 and a.heads == 128 and a.ctx == 8192 and a.kv == "bf16":
-        traffic = int(166156 * 1024 * (294912 / 147466.0) + 33024 * 1024)
+        traffic = int(166135 * 1024 * (294912 / 147466.0) + 33024 * 1024)
     res = {
         "metric": "mla_paged_decode_kv_read_bandwidth", "value": value, "unit": "GB/s",
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms_per_step,

@@ -52,7 +52,7 @@ def library():
         lib.mla_attn_plan.argtypes = [C.POINTER(MlaAttnArgs), C.POINTER(MlaPlanInfo)]
         lib.mla_attn_launch.restype = C.c_int
         lib.mla_attn_launch.argtypes = [C.POINTER(MlaAttnArgs), C.c_void_p]
-        for name in ("mla_attn_launch_partials", "mla_attn_launch_combine"):
+        for name in ("mla_attn_launch_partials", "mla_attn_launch_combine", "mla_attn_launch_kernel"):
             getattr(lib, name).restype = C.c_int
             getattr(lib, name).argtypes = [C.POINTER(MlaAttnArgs), C.c_void_p]
         lib.mla_hbm_copy_launch.restype = C.c_int

@@ -94,7 +94,7 @@ __device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); 
 
 // The pipelined decode kernel (mla_decode_kernel.hip); returns hipErrorInvalidValue for shapes it does not take.
 bool       decode_fast_applicable(const mla_attn_args * a);
-hipError_t launch_decode_fast(const KParams & kp, int kv_type, dim3 grid, hipStream_t st);
+hipError_t launch_decode_fast(const KParams & kp, int kv_type, dim3 grid, hipStream_t st, bool with_prepass);
 size_t     decode_fast_lds_bytes(int kv_type);
 size_t     decode_fast_qpack_bytes(int n_seq, int n_row_blocks);
 

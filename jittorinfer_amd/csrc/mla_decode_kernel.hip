@@ -295,12 +295,13 @@ static hipError_t launch_variant(const KParams & kp, dim3 grid, hipStream_t st) 
     return hipGetLastError();
 }
 
-hipError_t launch_decode_fast(const KParams & kp, int kv_type, dim3 grid, hipStream_t st) {
+hipError_t launch_decode_fast(const KParams & kp, int kv_type, dim3 grid, hipStream_t st, bool with_prepass) {
     const bool m = kp.mask != nullptr;
-    if (kv_type == MLA_TYPE_Q8_0)     hipLaunchKernelGGL(mla_q_pack_q8_kernel, dim3(grid.y, grid.z, KSTEPS / 2), dim3(NTHREADS), 0, st, kp);
+    if (!with_prepass) { /* the workspace still holds the Q image and the mask extents of an earlier launch of the same call */ }
+    else if (kv_type == MLA_TYPE_Q8_0)     hipLaunchKernelGGL(mla_q_pack_q8_kernel, dim3(grid.y, grid.z, KSTEPS / 2), dim3(NTHREADS), 0, st, kp);
     else if (kv_type == MLA_TYPE_F16) hipLaunchKernelGGL(mla_q_pack_kernel<true>, dim3(grid.y, grid.z, KSTEPS), dim3(NTHREADS), 0, st, kp);
     else                              hipLaunchKernelGGL(mla_q_pack_kernel<false>, dim3(grid.y, grid.z, KSTEPS), dim3(NTHREADS), 0, st, kp);
-    if (m) hipLaunchKernelGGL(mla_mask_extent_kernel, dim3(grid.y), dim3(NTHREADS), 0, st, kp);
+    if (m && with_prepass) hipLaunchKernelGGL(mla_mask_extent_kernel, dim3(grid.y), dim3(NTHREADS), 0, st, kp);
     if (kv_type == MLA_TYPE_Q8_0) return launch_variant<SRC_Q8, false>(kp, grid, st);
     if (kv_type == MLA_TYPE_F16)  return m ? launch_variant<SRC_F16, true>(kp, grid, st) : launch_variant<SRC_F16, false>(kp, grid, st);
     return m ? launch_variant<SRC_BF16, true>(kp, grid, st) : launch_variant<SRC_BF16, false>(kp, grid, st);

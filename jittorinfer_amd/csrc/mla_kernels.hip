@@ -662,7 +662,8 @@ int mla_attn_plan(const mla_attn_args * args, mla_attn_plan_info * out) {
     return 0;
 }
 
-// phases: bit 0 = the attention kernels (partials or final output), bit 1 = the combine pass
+// phases: bit 0 = the attention kernels (partials or final output), bit 1 = the combine pass,
+// bit 2 = the small passes ahead of the pipelined kernel (Q operand image, key extent of the mask)
 static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
     Plan pl;
     const int rc = make_plan(a, &pl);
@@ -712,7 +713,7 @@ static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
     for (int pass = 0; pass < pl.n_passes && (phases & 1); pass++) {
         kp.d_off = pass * pl.ndb * 32;
         hipError_t e;
-        if (pl.variant == 2) e = launch_decode_fast(kp, a->kv_type, grid, st);
+        if (pl.variant == 2) e = launch_decode_fast(kp, a->kv_type, grid, st, (phases & 4) != 0);
         else switch (a->kv_type) {
             case MLA_TYPE_BF16: e = launch_tile_src<SRC_BF16>(pl, kp, grid, st); break;
             case MLA_TYPE_F16:  e = launch_tile_src<SRC_F16>(pl, kp, grid, st); break;
@@ -728,8 +729,9 @@ static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
     return 0;
 }
 
-int mla_attn_launch(const mla_attn_args * a, void * stream) { return launch_phases(a, stream, 3); }
-int mla_attn_launch_partials(const mla_attn_args * a, void * stream) { return launch_phases(a, stream, 1); }
+int mla_attn_launch(const mla_attn_args * a, void * stream) { return launch_phases(a, stream, 7); }
+int mla_attn_launch_partials(const mla_attn_args * a, void * stream) { return launch_phases(a, stream, 5); }
+int mla_attn_launch_kernel(const mla_attn_args * a, void * stream) { return launch_phases(a, stream, 1); }
 int mla_attn_launch_combine(const mla_attn_args * a, void * stream) { return launch_phases(a, stream, 2); }
 
 int mla_hbm_copy_launch(const void * src, void * dst, size_t n_bytes, void * stream) {
