@@ -57,6 +57,8 @@ def library():
             getattr(lib, name).argtypes = [C.POINTER(MlaAttnArgs), C.c_void_p]
         lib.mla_hbm_copy_launch.restype = C.c_int
         lib.mla_hbm_copy_launch.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
+        lib.mla_kv_write_launch.restype = C.c_int
+        lib.mla_kv_write_launch.argtypes = [C.POINTER(MlaKvWriteArgs), C.c_void_p]
         lib.mla_attn_target_arch.restype = C.c_char_p
         lib.ggml_backend_init.restype = C.c_void_p
         lib.ggml_backend_score.restype = C.c_int
@@ -64,6 +66,14 @@ def library():
         lib.mla_ggml_abi_table.argtypes = [C.c_int, C.POINTER(C.c_char_p), C.POINTER(C.c_int64)]
         _lib = lib
     return _lib
+
+
+class MlaKvWriteArgs(C.Structure):
+    """mla_kv_write_args of include/mla_kv_write.h."""
+    _fields_ = [("n_tok", C.c_int32), ("src_type", C.c_int32), ("kv_type", C.c_int32), ("rows_type", C.c_int32),
+                ("src", C.c_void_p), ("src_nb1", C.c_int64), ("kv", C.c_void_p), ("kv_nb1", C.c_int64), ("n_kv_rows", C.c_int64),
+                ("row0", C.c_int64), ("rows", C.c_void_p), ("block_table", C.c_void_p), ("bt_stride", C.c_int64),
+                ("seq_ids", C.c_void_p), ("positions", C.c_void_p)]
 
 
 _workspaces = {}
@@ -156,3 +166,42 @@ def hbm_copy(src, dst, stream=None):
     rc = library().mla_hbm_copy_launch(src.data_ptr(), dst.data_ptr(), src.numel() * src.element_size(), C.c_void_p(st))
     if rc != 0:
         raise RuntimeError("mla_hbm_copy_launch failed with code %d" % rc)
+
+
+def kv_write(src, cache, kv_type, *, row0=None, rows=None, block_table=None, seq_ids=None, positions=None, stream=None):
+    """The KV cache write (ggml_cpy of src/llama-graph-attn.cpp:236-241 / ggml_scatter_update of :380-383) on the current
+    torch stream.  src: float32 [n_tok, 576] (converted to the cache type on write) or rows already in the cache type;
+    cache: [n_rows, row] in the storage type (row = 1152 or 612 bytes).  Exactly one addressing mode: row0 (consecutive
+    rows), rows (int32/int64 [n_tok] row indices), or block_table + seq_ids + positions (128-token pages)."""
+    import torch
+    if not src.is_cuda:
+        raise RuntimeError("jittorinfer_amd runs on a gfx950 GPU only (there is no CPU path)")
+    a = MlaKvWriteArgs()
+    a.n_tok = src.shape[0]
+    a.kv_type = kv_type
+    a.src_type = MLA_TYPE_F32 if src.dtype == torch.float32 else kv_type
+    assert src.dim() == 2 and src.stride(1) == 1 and cache.dim() == 2 and cache.stride(1) == 1
+    assert cache.shape[1] * cache.element_size() == ROW_BYTES[kv_type]
+    if a.src_type == MLA_TYPE_F32:
+        assert src.shape[1] == 576
+    else:
+        assert src.shape[1] * src.element_size() == ROW_BYTES[kv_type]
+    a.src, a.src_nb1 = src.data_ptr(), src.stride(0) * src.element_size()
+    a.kv, a.kv_nb1, a.n_kv_rows = cache.data_ptr(), cache.stride(0) * cache.element_size(), cache.shape[0]
+    assert (row0 is not None) + (rows is not None) + (block_table is not None) == 1
+    if row0 is not None:
+        a.row0 = row0
+    elif rows is not None:
+        assert rows.dtype in (torch.int32, torch.int64) and rows.is_contiguous() and rows.numel() == a.n_tok
+        a.rows, a.rows_type = rows.data_ptr(), 1 if rows.dtype == torch.int64 else 0
+    else:
+        for t in (block_table, seq_ids, positions):
+            assert t.dtype == torch.int32 and t.is_contiguous()
+        assert block_table.dim() == 2 and seq_ids.numel() == a.n_tok and positions.numel() == a.n_tok
+        a.block_table, a.bt_stride = block_table.data_ptr(), block_table.shape[1]
+        a.seq_ids, a.positions = seq_ids.data_ptr(), positions.data_ptr()
+    st = stream if stream is not None else torch.cuda.current_stream(src.device).cuda_stream
+    rc = library().mla_kv_write_launch(C.byref(a), C.c_void_p(st))
+    if rc != 0:
+        raise RuntimeError("mla_kv_write_launch failed with code %d" % rc)
+    return cache

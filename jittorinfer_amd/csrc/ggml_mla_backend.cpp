@@ -25,6 +25,7 @@
 #include <vector>
 
 #include "../../include/ggml_mla_backend.h"
+#include "../../include/mla_kv_write.h"
 #include "../../include/mla_attn.h"
 #include "ggml_abi.h"
 
@@ -249,9 +250,35 @@ bool mla_node_ok(const tensor * dst, const char ** why) {
     return true;
 }
 
+// The KV cache write of llm_attn_mla (src/llama-graph-attn.cpp:236-241): CPY of f32 rows [576, n_tok] into a contiguous
+// view of a BF16 / F16 / Q8_0 cache with the same number of elements; and SCATTER_UPDATE (ggml.c:3203-3223): rows of
+// `updates` (cache type or F32) into rows indices[i] of a [576, n_rows] cache.
+bool kv_cpy_ok(const tensor * op, const char ** why) {
+    const char * dummy; if (!why) why = &dummy;
+    const tensor * src = op->src[0];
+    if (!src || src->type != TYPE_F32 || src->ne[0] != 576 || src->ne[2] != 1 || src->ne[3] != 1) { *why = "source must be F32 [576, n_tok]"; return false; }
+    if (src->nb[0] != 4 || (src->nb[1] & 15)) { *why = "source rows must be dense and 16-byte aligned"; return false; }
+    if (op->type != TYPE_BF16 && op->type != TYPE_F16 && op->type != TYPE_Q8_0) { *why = "destination must be BF16, F16 or Q8_0"; return false; }
+    if (!is_contiguous(op) || nelements(op) != nelements(src)) { *why = "destination must be a contiguous view with as many elements"; return false; }
+    return true;
+}
+
+bool kv_scatter_ok(const tensor * op, const char ** why) {
+    const char * dummy; if (!why) why = &dummy;
+    const tensor * var = op->src[0], * idx = op->src[1], * upd = op->src[2];
+    if (!var || !idx || !upd) { *why = "missing operand"; return false; }
+    if (var->ne[0] != 576 || upd->ne[0] != 576 || var->ne[2] != 1 || var->ne[3] != 1 || upd->ne[2] != 1 || upd->ne[3] != 1) { *why = "cache and updates must be [576, rows]"; return false; }
+    if (var->type != TYPE_BF16 && var->type != TYPE_F16 && var->type != TYPE_Q8_0) { *why = "cache must be BF16, F16 or Q8_0"; return false; }
+    if (upd->type != var->type && upd->type != TYPE_F32) { *why = "updates must have the cache type or be F32"; return false; }
+    if ((idx->type != TYPE_I32 && idx->type != TYPE_I64) || !is_contiguous(idx) || idx->ne[0] != upd->ne[1]) { *why = "indices must be contiguous I32/I64, one per update row"; return false; }
+    return true;
+}
+
 bool device_supports_op(backend_device *, const tensor * op) {
     if (is_noop(op->op)) return true;
     if (op->op == OP_FLASH_ATTN_EXT) return mla_node_ok(op, nullptr);
+    if (op->op == OP_CPY) return kv_cpy_ok(op, nullptr);
+    if (op->op == OP_SCATTER_UPDATE) return kv_scatter_ok(op, nullptr);
     return false;
 }
 
@@ -321,14 +348,38 @@ int compute_flash_attn(backend_ctx * ctx, const tensor * dst) {
     return STATUS_SUCCESS;
 }
 
+int compute_kv_write(backend_ctx * ctx, const tensor * dst) {
+    const char * why = nullptr;
+    mla_kv_write_args a;
+    memset(&a, 0, sizeof(a));
+    if (dst->op == OP_CPY) {
+        if (!kv_cpy_ok(dst, &why)) { log_error("CPY node '%s' rejected: %s", dst->name, why); return STATUS_FAILED; }
+        const tensor * src = dst->src[0];
+        a.n_tok = (int32_t) src->ne[1]; a.src_type = MLA_TYPE_F32; a.kv_type = dst->type;
+        a.src = src->data; a.src_nb1 = (int64_t) src->nb[1];
+        a.kv = dst->data; a.kv_nb1 = dst->type == TYPE_Q8_0 ? 612 : 1152; a.n_kv_rows = src->ne[1]; a.row0 = 0;
+    } else {
+        if (!kv_scatter_ok(dst, &why)) { log_error("SCATTER_UPDATE node '%s' rejected: %s", dst->name, why); return STATUS_FAILED; }
+        const tensor * var = dst->src[0], * idx = dst->src[1], * upd = dst->src[2];
+        a.n_tok = (int32_t) upd->ne[1]; a.src_type = upd->type == TYPE_F32 ? MLA_TYPE_F32 : var->type; a.kv_type = var->type;
+        a.src = upd->data; a.src_nb1 = (int64_t) upd->nb[1];
+        a.kv = var->data; a.kv_nb1 = (int64_t) var->nb[1]; a.n_kv_rows = var->ne[1];
+        a.rows = idx->data; a.rows_type = idx->type == TYPE_I64 ? 1 : 0;
+    }
+    if (!a.src || !a.kv) { log_error("node '%s': operands not allocated", dst->name); return STATUS_FAILED; }
+    const int rc = mla_kv_write_launch(&a, ctx->stream);
+    if (rc != 0) { log_error("mla_kv_write_launch failed for node '%s': %d", dst->name, rc); return STATUS_FAILED; }
+    return STATUS_SUCCESS;
+}
+
 int backend_graph_compute(backend * be, cgraph * g) {
     backend_ctx * ctx = (backend_ctx *) be->context;
     if (!HIP_OK(hipSetDevice(ctx->device))) return STATUS_FAILED;
     for (int i = 0; i < g->n_nodes; i++) {
         const tensor * node = g->nodes[i];
         if (is_empty(node) || is_noop(node->op)) continue;
-        if (node->op != OP_FLASH_ATTN_EXT) { log_error("op %d of node '%s' is not supported", node->op, node->name); return STATUS_FAILED; }
-        const int st = compute_flash_attn(ctx, node);
+        if (node->op != OP_FLASH_ATTN_EXT && node->op != OP_CPY && node->op != OP_SCATTER_UPDATE) { log_error("op %d of node '%s' is not supported", node->op, node->name); return STATUS_FAILED; }
+        const int st = node->op == OP_FLASH_ATTN_EXT ? compute_flash_attn(ctx, node) : compute_kv_write(ctx, node);
         if (st != STATUS_SUCCESS) return st;
     }
     return STATUS_SUCCESS;

@@ -400,3 +400,31 @@ int mla_oracle_flash_attn_ext_f64(const mla_oracle_tensor *q, const mla_oracle_t
     }
     return 0;
 }
+
+/*
+ * KV cache write as ggml-cpu performs ggml_cpy(kv_cur f32 [576, n_tok] -> typed cache rows)
+ * (ggml/src/ggml-cpu/ggml-cpu.c:3965-4040 ggml_compute_forward_dup_f32: per source row, from_float of the destination
+ * type, table :269-434): F16 -> ggml_fp32_to_fp16_row, BF16 -> ggml_fp32_to_bf16_row, Q8_0 -> the CPU backend's
+ * quantize_row_q8_0 (q8_mode 1 = its x86 form, 0 = the reference form of ggml-quants.c:202-226).
+ * Destination rows are given explicitly (dest_rows[i], skipped when outside [0, n_kv_rows)), which also covers
+ * ggml_scatter_update's dst[indices[i]] = updates[i] (ggml/src/ggml.c:3203-3223, aclnn_ops.cpp:6052-6129) and a block table
+ * resolved by the caller.  src_type F32 converts; src_type == kv_type copies the row bytes.
+ * Pinned by tests/test_kv_write.py: conversions are the functions above (exhaustive tests), the row placement is checked
+ * against numpy indexing, and the whole against the reference's compiled ggml_cpy when oracle/_ref is built.
+ */
+int mla_oracle_kv_write(const void *src, int src_type, int64_t src_nb1, int64_t n_tok, void *kv, int kv_type, int64_t kv_nb1,
+                        int64_t n_kv_rows, const int64_t *dest_rows, int q8_mode) {
+    const size_t rs = type_row_size(kv_type, 576);
+    if (rs == 0 || (src_type != 0 && src_type != kv_type)) return -2;
+    for (int64_t t = 0; t < n_tok; t++) {
+        const int64_t r = dest_rows[t];
+        if (r < 0 || r >= n_kv_rows) continue;
+        const char *s = (const char *) src + t * src_nb1;
+        char *d = (char *) kv + r * kv_nb1;
+        if (src_type != 0) { memcpy(d, s, rs); continue; }
+        if (kv_type == 1)       mla_oracle_f32_to_f16_row((const float *) s, (uint16_t *) d, 576);
+        else if (kv_type == 30) mla_oracle_f32_to_bf16_row((const float *) s, (uint16_t *) d, 576);
+        else                    mla_oracle_quantize_row_q8_0((const float *) s, d, 576, q8_mode);
+    }
+    return 0;
+}

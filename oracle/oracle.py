@@ -45,6 +45,8 @@ def lib():
         _lib.mla_oracle_flash_attn_ext.argtypes = [C.POINTER(_Tensor)] * 4 + [C.c_void_p, C.c_int64, C.c_float, C.c_float, C.c_float, C.c_int, C.c_int]
         _lib.mla_oracle_flash_attn_ext_f64.restype = C.c_int
         _lib.mla_oracle_flash_attn_ext_f64.argtypes = [C.POINTER(_Tensor)] * 4 + [C.c_void_p, C.c_int64, C.c_float, C.c_int, C.c_int]
+        _lib.mla_oracle_kv_write.restype = C.c_int
+        _lib.mla_oracle_kv_write.argtypes = [C.c_void_p, C.c_int, C.c_int64, C.c_int64, C.c_void_p, C.c_int, C.c_int64, C.c_int64, C.c_void_p, C.c_int]
         for name in ("mla_oracle_f32_to_bf16_row", "mla_oracle_f32_to_f16_row", "mla_oracle_bf16_to_f32_row", "mla_oracle_f16_to_f32_row"):
             getattr(_lib, name).argtypes = [C.c_void_p, C.c_void_p, C.c_int64]
             getattr(_lib, name).restype = None
@@ -71,6 +73,10 @@ def ref():
         _ref.ref_backend_flash_attn_ext.argtypes = [C.c_char_p, C.c_int] + [C.c_int64] * 6 + [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64,
                                                     C.c_void_p, C.c_int64, C.c_void_p, C.c_float, C.c_float, C.c_float, C.c_int,
                                                     C.c_void_p, C.c_char_p, C.c_size_t]
+        _ref.ref_kv_cpy.restype = C.c_int
+        _ref.ref_kv_cpy.argtypes = [C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_int]
+        _ref.ref_backend_kv_cpy.restype = C.c_int
+        _ref.ref_backend_kv_cpy.argtypes = [C.c_char_p, C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_char_p, C.c_size_t]
         for name in ("ref_quantize_q8_0_ref", "ref_quantize_q8_0_cpu", "ref_dequantize_q8_0", "ref_f32_to_f16_row", "ref_f32_to_bf16_row", "ref_f16_to_f32_row"):
             getattr(_ref, name).argtypes = [C.c_void_p, C.c_void_p, C.c_int64]
             getattr(_ref, name).restype = None
@@ -259,3 +265,39 @@ def errors(a, b):
     a = np.asarray(a, dtype=np.float64)
     b = np.asarray(b, dtype=np.float64)
     return float(np.max(np.abs(a - b))), float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-300))
+
+
+def kv_write(src, cache, kv_type, dest_rows, src_type=TYPE_F32, q8_mode=1):
+    """The cache write as ggml-cpu's ggml_cpy does it per row: cache (uint16 [rows, 576] or uint8 [rows, 612]) is updated
+    in place and returned; src is float32 [n_tok, 576] (converted) or rows already in the cache type (copied)."""
+    src = np.ascontiguousarray(src)
+    assert cache.flags.c_contiguous
+    dest = np.ascontiguousarray(dest_rows, dtype=np.int64)
+    assert dest.shape == (src.shape[0],)
+    rc = lib().mla_oracle_kv_write(src.ctypes.data, src_type, src.strides[0], src.shape[0], cache.ctypes.data, kv_type,
+                                   cache.strides[0], cache.shape[0], dest.ctypes.data, q8_mode)
+    if rc != 0:
+        raise RuntimeError("mla_oracle_kv_write failed: %d" % rc)
+    return cache
+
+
+def ref_kv_cpy(kv_cur, cache, kv_type, kv_head, n_threads=4):
+    """ggml_cpy(kv_cur, view of the cache at row kv_head) on the reference's compiled ggml-cpu; cache updated in place."""
+    kv_cur = np.ascontiguousarray(kv_cur, dtype=np.float32)
+    assert cache.flags.c_contiguous
+    rc = ref().ref_kv_cpy(kv_type, cache.shape[0], kv_head, kv_cur.shape[0], kv_cur.ctypes.data, cache.ctypes.data, n_threads)
+    if rc != 0:
+        raise RuntimeError("ref_kv_cpy failed: %d" % rc)
+    return cache
+
+
+def ref_backend_kv_cpy(so_path, kv_cur, cache, kv_type, kv_head):
+    """The same node computed by a backend plugin loaded through the reference's ggml_backend_load."""
+    kv_cur = np.ascontiguousarray(kv_cur, dtype=np.float32)
+    assert cache.flags.c_contiguous
+    info = C.create_string_buffer(256)
+    rc = ref().ref_backend_kv_cpy(so_path.encode(), kv_type, cache.shape[0], kv_head, kv_cur.shape[0], kv_cur.ctypes.data,
+                                  cache.ctypes.data, info, 256)
+    if rc != 0:
+        raise RuntimeError("ref_backend_kv_cpy failed: %d (%s)" % (rc, info.value.decode()))
+    return cache, info.value.decode()

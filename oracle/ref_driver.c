@@ -193,6 +193,72 @@ done:
 
 /* ------------------------------------------------------------------ small pinning helpers */
 
+/*
+ * The KV cache write of llm_attn_mla (src/llama-graph-attn.cpp:236-241) on the reference's ggml-cpu:
+ * cache = typed tensor of n_cache rows of 576 (filled from `cache` first), kv_cur = f32 [576, n_tok],
+ * ggml_cpy(kv_cur, ggml_view_1d(cache, n_tok*576, row_size*kv_head)); the whole cache is copied back into `cache`.
+ */
+int ref_kv_cpy(int k_type, int64_t n_cache, int64_t kv_head, int64_t n_tok, const float * kv_cur, void * cache, int n_threads) {
+    const enum ggml_type kt = (enum ggml_type) k_type;
+    const int64_t D = 576;
+    size_t mem = row_bytes(kt, D) * n_cache + (size_t) D * n_tok * 4 + (32u << 20);
+    struct ggml_init_params ip = { mem, NULL, false };
+    struct ggml_context *   ctx = ggml_init(ip);
+    if (!ctx) return -1;
+    struct ggml_tensor * tc = ggml_new_tensor_1d(ctx, kt, D * n_cache);
+    struct ggml_tensor * tx = ggml_new_tensor_2d(ctx, GGML_TYPE_F32, D, n_tok);
+    memcpy(tc->data, cache, ggml_nbytes(tc));
+    memcpy(tx->data, kv_cur, ggml_nbytes(tx));
+    struct ggml_tensor * view = ggml_view_1d(ctx, tc, n_tok * D, ggml_row_size(kt, D) * kv_head);
+    struct ggml_tensor * o    = ggml_cpy(ctx, tx, view);
+    struct ggml_cgraph * gf   = ggml_new_graph(ctx);
+    ggml_build_forward_expand(gf, o);
+    enum ggml_status st = ggml_graph_compute_with_ctx(ctx, gf, n_threads);
+    if (st == GGML_STATUS_SUCCESS) memcpy(cache, tc->data, ggml_nbytes(tc));
+    ggml_free(ctx);
+    return (int) st;
+}
+
+/*
+ * The same write through a backend loaded from `so_path` (cache and kv_cur live in that backend's buffer, the node is
+ * computed by ggml_backend_graph_compute), followed by nothing else: the cache bytes come back in `cache`.
+ */
+int ref_backend_kv_cpy(const char * so_path, int k_type, int64_t n_cache, int64_t kv_head, int64_t n_tok, const float * kv_cur,
+                       void * cache, char * info, size_t info_len) {
+    const enum ggml_type kt = (enum ggml_type) k_type;
+    const int64_t D = 576;
+    ggml_backend_reg_t reg = ggml_backend_load(so_path);
+    if (!reg) return -10;
+    if (ggml_backend_reg_dev_count(reg) < 1) return -11;
+    ggml_backend_dev_t dev = ggml_backend_reg_dev_get(reg, 0);
+    ggml_backend_t     be  = ggml_backend_dev_init(dev, NULL);
+    if (!be) return -12;
+    if (info) snprintf(info, info_len, "%s / %s", ggml_backend_reg_name(reg), ggml_backend_dev_name(dev));
+    struct ggml_init_params ip = { ggml_tensor_overhead() * 16 + ggml_graph_overhead(), NULL, true };
+    struct ggml_context *   ctx = ggml_init(ip);
+    struct ggml_tensor * tc = ggml_new_tensor_1d(ctx, kt, D * n_cache);
+    struct ggml_tensor * tx = ggml_new_tensor_2d(ctx, GGML_TYPE_F32, D, n_tok);
+    struct ggml_tensor * view = ggml_view_1d(ctx, tc, n_tok * D, ggml_row_size(kt, D) * kv_head);
+    struct ggml_tensor * o    = ggml_cpy(ctx, tx, view);
+    struct ggml_cgraph * gf   = ggml_new_graph(ctx);
+    ggml_build_forward_expand(gf, o);
+    int rc = 0;
+    ggml_backend_buffer_t buf = ggml_backend_alloc_ctx_tensors(ctx, be);
+    if (!buf) rc = -13;
+    if (!rc && !ggml_backend_supports_op(be, o)) rc = -14;
+    if (!rc) {
+        ggml_backend_tensor_set(tc, cache, 0, ggml_nbytes(tc));
+        ggml_backend_tensor_set(tx, kv_cur, 0, ggml_nbytes(tx));
+        enum ggml_status st = ggml_backend_graph_compute(be, gf);
+        if (st != GGML_STATUS_SUCCESS) rc = (int) st ? (int) st : -15;
+        else ggml_backend_tensor_get(tc, cache, 0, ggml_nbytes(tc));
+    }
+    if (buf) ggml_backend_buffer_free(buf);
+    ggml_free(ctx);
+    ggml_backend_free(be);
+    return rc;
+}
+
 void ref_quantize_q8_0_ref(const float * x, void * y, int64_t k) { quantize_row_q8_0_ref(x, (block_q8_0 *) y, k); }
 void ref_quantize_q8_0_cpu(const float * x, void * y, int64_t k) { quantize_row_q8_0(x, y, k); }
 void ref_dequantize_q8_0(const void * x, float * y, int64_t k) { dequantize_row_q8_0((const block_q8_0 *) x, y, k); }
