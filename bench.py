@@ -68,6 +68,52 @@ def build_paged(dev, lens, n_head, n_tok, kv, seed):
     return q, pool, bt, torch.tensor(lens, dtype=torch.int32, device=dev)
 
 
+def kv_write_config(a, dev, lib, J):
+    """The latent-KV cache write (include/mla_kv_write.h) on 65536 new rows through a block table: f32 rows in, cache rows
+    out.  Algorithmic bytes per row: 2304 read + 1152 (bf16/f16) or 612 (Q8_0) written."""
+    import torch
+    n_tok, n_seq = 65536, 32
+    kvt = {"bf16": J.MLA_TYPE_BF16, "f16": J.MLA_TYPE_F16, "q8_0": J.MLA_TYPE_Q8_0}[a.kv]
+    row = 612 if a.kv == "q8_0" else 1152
+    g = torch.Generator(device=dev)
+    g.manual_seed(a.seed)
+    x = torch.randn((n_tok, 576), generator=g, device=dev, dtype=torch.float32)
+    pages = n_tok // 128
+    cache = torch.zeros((pages * 128, row), dtype=torch.uint8, device=dev)
+    bt = torch.randperm(pages, generator=g, device=dev).to(torch.int32).reshape(n_seq, pages // n_seq).contiguous()
+    order = torch.randperm(n_tok, generator=g, device=dev)
+    seq_ids = (order // (n_tok // n_seq)).to(torch.int32).contiguous()
+    positions = (order % (n_tok // n_seq)).to(torch.int32).contiguous()
+    stream = torch.cuda.current_stream(dev)
+
+    def run(n):
+        for _ in range(n):
+            J.kv_write(x, cache, kvt, block_table=bt, seq_ids=seq_ids, positions=positions)
+
+    run(a.warmup)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    run(a.steps)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / a.steps
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    run(a.steps)
+    e1.record(stream)
+    torch.cuda.synchronize()
+    kern_ms = e0.elapsed_time(e1) / a.steps
+    nbytes = n_tok * (2304 + row)
+    print(json.dumps({"metric": "mla_kv_cache_write_bandwidth", "value": nbytes / (ms * 1e-3) / 1e9, "unit": "GB/s", "n_gpus": 1,
+                      "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak",
+                      "vs_baseline": None, "dtype": a.kv, "data": "synthetic",
+                      "config": {"workload": "KV cache write: 65536 f32 rows of 576 -> %s cache rows through a block table (32 sequences, shuffled pages and arrival order)" % a.kv},
+                      "us_per_step": ms * 1e3,
+                      "roofline": {"bound": "hbm", "kernel": "mla_kv_write_kernel", "achieved": nbytes / (kern_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS,
+                                   "unit": "GB/s", "frac": nbytes / (kern_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, "traffic": None,
+                                   "algorithmic_bytes_per_launch": nbytes, "kernel_us": {"mean": kern_ms * 1e3}},
+                      "cpu_baseline": None}))
+
+
 def other_config(a, dev, lib, J):
     """BASELINE configs 2, 4 and 5 through the same C ABI: parity-test shapes, timed here for the profiles (not the
     headline line).  One JSON line in the same format; the metric of the prefill config is its MFMA rate."""
@@ -181,9 +227,9 @@ def main():
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="N",
                     help="also launch the library's plain copy kernel N times over one KV pool (known byte count) so that a "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run can be scaled")
-    ap.add_argument("--kv", default="bf16", choices=["bf16", "f16"], help="storage type of the latent KV pool (the headline config is bf16)")
-    ap.add_argument("--config", default="c3", choices=["c2", "c3", "c4", "c5"],
-                    help="c3 (default) is the headline workload; the others time BASELINE's remaining GPU configs for the profiles")
+    ap.add_argument("--kv", default="bf16", choices=["bf16", "f16", "q8_0"], help="storage type of the latent KV pool (the headline config is bf16; q8_0 only with --config kvwrite)")
+    ap.add_argument("--config", default="c3", choices=["c2", "c3", "c4", "c5", "kvwrite"],
+                    help="c3 (default) is the headline workload; the others time BASELINE's remaining GPU configs and the cache write for the profiles")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this build measures one GPU's share of the path; --gpus %d is not supported (use --gpus 1)" % a.gpus, file=sys.stderr)
@@ -197,9 +243,15 @@ def main():
     lib = J.library()
     dev = torch.device("cuda:0")
     scale = 1.0 / (192.0 ** 0.5)
+    if a.config == "kvwrite":
+        kv_write_config(a, dev, lib, J)
+        return
     if a.config != "c3":
         other_config(a, dev, lib, J)
         return
+    if a.kv == "q8_0":
+        print("bench.py: --kv q8_0 goes with --config kvwrite or --config c5", file=sys.stderr)
+        sys.exit(2)
 
     q, pools, block_table, seq_lens = build_workload(dev, a.batch, a.heads, a.ctx, a.pools, a.seed, a.kv)
     kv_type = J.MLA_TYPE_BF16 if a.kv == "bf16" else J.MLA_TYPE_F16

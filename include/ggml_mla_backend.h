@@ -9,7 +9,7 @@
  * are mirrored in jittorinfer_amd/csrc/ggml_abi.h.  All handles are passed as void* here so that this header needs
  * no ggml header; they are ggml_backend_reg_t / ggml_tensor* of the reference.
  *
- * Node contract of the one compute op it accepts, GGML_OP_FLASH_ATTN_EXT built by ggml_flash_attn_ext
+ * Node contract of the attention op it accepts, GGML_OP_FLASH_ATTN_EXT built by ggml_flash_attn_ext
  * (ggml/src/ggml.c:3988-4022), with the operands llm_attn_mla defines (src/llama-graph-attn.cpp:259-315):
  *   src[0] q     F32  [576, n_tok, n_head, n_seq]
  *   src[1] k     F16 | BF16 | Q8_0  [576, n_kv, 1, n_seq or 1]   the latent KV rows
@@ -20,6 +20,12 @@
  *                slot convention ggml_flash_attn_prompt uses for its length tensors (ggml/src/ggml.c:2707-2710)
  *   op_params    {scale, max_bias, logit_softcap} f32, [3] = precision (ggml/src/ggml.c:4012-4013, :4024-4030)
  *   dst          F32 [576, n_head, n_tok, n_seq]; the first v->ne[0] floats of every row are written
+ * The cache write that precedes it (kernels behind include/mla_kv_write.h):
+ *   GGML_OP_CPY             src[0] F32 [576, n_tok] with dense rows -> dst, a contiguous BF16 | F16 | Q8_0 view with as many
+ *                           elements (ggml_cpy(kv_cur, k_cache_view), src/llama-graph-attn.cpp:236-241)
+ *   GGML_OP_SCATTER_UPDATE  src[0] cache BF16 | F16 | Q8_0 [576, n_rows], src[1] I32 | I64 [n_tok] row indices,
+ *                           src[2] updates [576, n_tok] of the cache type (copied) or F32 (converted)
+ *                           (ggml_scatter_update, ggml/src/ggml.c:3203-3223; src/llama-graph-attn.cpp:380-383)
  * Every other op except the no-op view ops (NONE, RESHAPE, VIEW, PERMUTE, TRANSPOSE) is reported unsupported, so
  * the reference's scheduler keeps it on another backend (ggml/src/ggml-backend.cpp:820-846).
  */
