@@ -46,7 +46,9 @@ struct KParams {
     const int32_t * seq_lens;
     float *         dst;
     int64_t         dst_stride;  // floats
-    _Float16 *      part_o;      // split-K partials O_c / l_c as f16: [n_seq][n_splits][dv_total/8][n_rows][8]
+    _Float16 *      part_o;      // split-K partials O_c / l_c as f16: [n_seq][n_splits][dv_total/8][n_rows][8], or, when
+                                 // part_f32 is set (small problems: no second rounding), as f32 rows [n_seq][n_splits][n_rows][dv_total]
+    int             part_f32;
     float *         part_ml;     // [n_seq][n_splits][n_rows][2]  (max in log2 units, sum)
     int             n_head, n_tok, n_rows;
     int             n_splits, split_tokens;

@@ -119,7 +119,9 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
     // per-thread pointers for the wave program, handed over through LDS
     // final output: row-major dst rows.  split-K partial: [column/8][row][8] inside this (sequence, split) block.
     const int64_t pblock = ((int64_t) b * p.n_splits + split) * p.n_rows * p.dv_total;  // in f16 elements
+    // (f32 partials are rows of dv_total floats: the wave program stores them the way it stores final output rows)
     void * optr = row_valid ? (p.n_splits == 1 ? (void *) (p.dst + orow * p.dst_stride + 4 * g)
+                               : p.part_f32    ? (void *) ((float *) p.part_o + prow * p.dv_total + 4 * g)
                                                : (void *) (p.part_o + pblock + (int64_t) row * 8 + 4 * g)) : nullptr;
     float * mlptr = (p.n_splits > 1 && g == 0 && row_valid) ? p.part_ml + prow * 2 : nullptr;
     {
@@ -140,7 +142,7 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
     const int s_kve  = __builtin_amdgcn_readfirstlane(kv_end);
     const int s_npp  = __builtin_amdgcn_readfirstlane(p.n_pool_pages - 1);
     const int s_nb1  = __builtin_amdgcn_readfirstlane((int) p.kv_nb1);
-    const int s_flg  = __builtin_amdgcn_readfirstlane((p.n_splits == 1 ? 1 : 0) | p.debug_flags);
+    const int s_flg  = __builtin_amdgcn_readfirstlane((p.n_splits == 1 || p.part_f32 ? 1 : 0) | p.debug_flags);  // bit 0: f32 row store
     const int s_ntl  = __builtin_amdgcn_readfirstlane(n_tiles);
     const char * mask_base = p.mask;
     const int s_scale = __builtin_amdgcn_readfirstlane(__float_as_int(p.scale));

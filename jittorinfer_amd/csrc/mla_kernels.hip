@@ -373,6 +373,16 @@ __global__ void __launch_bounds__(NTHREADS) mla_attn_tile_kernel(const KParams p
         // partial = O / l of this split, stored as f16 in layout [column/8][row][8]: coalesced for the writers here and
         // for the combine pass, and half the bytes of f32 (the 2^-11 rounding is averaged over the splits)
         const float pinv = 1.0f / l_tot;
+        if (p.part_f32) {
+            float * o = (float *) p.part_o + prow * p.dv_total + p.d_off;
+#pragma unroll
+            for (int i = 0; i < NDBW; i++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    f32x4 v = { acc[i][4 * j] * pinv, acc[i][4 * j + 1] * pinv, acc[i][4 * j + 2] * pinv, acc[i][4 * j + 3] * pinv };
+                    *(f32x4 *) (o + (wd * NDBW + i) * 32 + 8 * j + 4 * g) = v;
+                }
+        } else
 #pragma unroll
         for (int i = 0; i < NDBW; i++)
 #pragma unroll
@@ -442,6 +452,37 @@ __global__ void __launch_bounds__(256) mla_attn_combine_kernel(const KParams p) 
     float * out = p.dst + ((int64_t) b * p.n_rows + row) * p.dst_stride + cg * 8;
     *(f32x4 *) out       = f32x4{ o[0] * inv, o[1] * inv, o[2] * inv, o[3] * inv };
     *(f32x4 *) (out + 4) = f32x4{ o[4] * inv, o[5] * inv, o[6] * inv, o[7] * inv };
+}
+
+// The same merge over f32 partials (rows of dv_total floats; small problems).  One thread = one (row, group of 4 columns),
+// lanes along the columns of a row.  grid = (ceil(rows/2), 1, n_seq), block = 256 = 2 rows x 128 column groups (dv <= 512)
+// or (rows, 1, n_seq) with 144 active threads for dv = 576: blockDim covers one or two rows, see the launch.
+__global__ void __launch_bounds__(256) mla_attn_combine_f32_kernel(const KParams p, int groups_per_row) {
+    const int b = blockIdx.z;
+    const int rows_per_block = 256 / groups_per_row;
+    const int row = blockIdx.x * rows_per_block + threadIdx.x / groups_per_row;
+    const int cg  = threadIdx.x % groups_per_row;
+    if (row >= p.n_rows || threadIdx.x >= rows_per_block * groups_per_row || cg * 4 >= p.dv_total) return;
+    const int seq_len = p.block_table ? min(p.seq_lens[b], (int) p.bt_stride * MLA_PAGE_TOKENS) : (int) p.n_kv;
+    int nvalid = (seq_len + p.split_tokens - 1) / p.split_tokens;
+    nvalid = min(nvalid, p.n_splits);
+    const float2 * ml = (const float2 *) p.part_ml + (int64_t) b * p.n_splits * p.n_rows + row;
+    const float *  po = (const float *) p.part_o + ((int64_t) b * p.n_splits * p.n_rows + row) * p.dv_total + cg * 4;
+    const int64_t ml_step = p.n_rows, po_step = (int64_t) p.n_rows * p.dv_total;
+    float M = -INFINITY;
+    for (int c = 0; c < nvalid; c++) M = fmaxf(M, ml[c * ml_step].x);
+    float L = 0.f;
+    f32x4 o = { 0.f, 0.f, 0.f, 0.f };
+    for (int c = 0; c < nvalid; c++) {
+        const float2 v = ml[c * ml_step];
+        if (v.x == -INFINITY) continue;   // that split saw only masked keys
+        const float w = v.y * fast_exp2(v.x - M);
+        const f32x4 x = *(const f32x4 *) (po + c * po_step);
+        L += w;
+        o.x += x.x * w; o.y += x.y * w; o.z += x.z * w; o.w += x.w * w;
+    }
+    const float inv = 1.0f / L;  // no valid key at all: 0 * inf = NaN, like the reference
+    *(f32x4 *) (p.dst + ((int64_t) b * p.n_rows + row) * p.dst_stride + cg * 4) = f32x4{ o.x * inv, o.y * inv, o.z * inv, o.w * inv };
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -525,6 +566,7 @@ struct Plan {
     int    n_passes, ndb;
     size_t lds_bytes;
     size_t ws_part_o, ws_part_ml, ws_scores, ws_qpack, ws_maskext;
+    int    part_f32;
 };
 
 int validate(const mla_attn_args * a) {
@@ -603,7 +645,11 @@ int make_plan(const mla_attn_args * a, Plan * pl) {
     if (pl->variant == 2) pl->ws_qpack = decode_fast_qpack_bytes(a->n_seq, pl->n_row_blocks);
     if (pl->variant == 2 && a->mask) pl->ws_maskext = (size_t) pl->n_row_blocks * sizeof(int);
     if (pl->n_splits > 1) {
-        pl->ws_part_o  = (size_t) a->n_seq * pl->n_splits * n_rows * a->dv * sizeof(_Float16);
+        // f32 partials while they are small (no second rounding of O on top of the MFMA operands' one), f16 beyond: there the
+        // partial traffic counts, and the rounding (2^-12 relative per split) is averaged over long contexts
+        const size_t n_part = (size_t) a->n_seq * pl->n_splits * n_rows * a->dv;
+        pl->part_f32   = n_part * sizeof(float) <= ((size_t) 32 << 20);
+        pl->ws_part_o  = n_part * (pl->part_f32 ? sizeof(float) : sizeof(_Float16));
         pl->ws_part_ml = (size_t) a->n_seq * pl->n_splits * n_rows * 2 * sizeof(float);
     }
     return 0;
@@ -691,6 +737,7 @@ static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
                      (a->block_table || (a->kv_nb3 & 15) == 0);
     char * ws = (char *) a->workspace;
     kp.part_o  = (_Float16 *) ws;
+    kp.part_f32 = pl.part_f32;
     kp.part_ml = (float *) (ws + align256(pl.ws_part_o));
     float * scores = (float *) (ws + align256(pl.ws_part_o) + align256(pl.ws_part_ml));
     kp.q_pack = ws + align256(pl.ws_part_o) + align256(pl.ws_part_ml) + align256(pl.ws_scores);
@@ -722,6 +769,12 @@ static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
         if (e != hipSuccess) return (int) e;
     }
     if (pl.n_splits > 1 && (phases & 2)) {
+        if (pl.part_f32) {
+            const int groups = a->dv / 4, rows_per_block = 256 / groups;   // 128 -> 2 rows, 144 -> 1 row
+            dim3 g((unsigned) ((kp.n_rows + rows_per_block - 1) / rows_per_block), 1, (unsigned) a->n_seq);
+            hipLaunchKernelGGL(mla_attn_combine_f32_kernel, g, dim3(256), 0, st, kp, groups);
+            return (int) hipGetLastError();
+        }
         dim3 g((unsigned) ((kp.n_rows + 31) / 32), (unsigned) ((a->dv + 63) / 64), (unsigned) a->n_seq);
         hipLaunchKernelGGL(mla_attn_combine_kernel, g, dim3(256), 0, st, kp);
         return (int) hipGetLastError();

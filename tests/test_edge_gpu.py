@@ -1,0 +1,146 @@
+"""Edge cases of the attention paths on the GPU (ragged, empty and boundary-length sequences, partial row blocks,
+strided Q, garbage in unused table entries) against the oracle, and size-independent properties at BASELINE's full
+sizes (page-permutation invariance, split invariance, causal independence)."""
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+from tests import util as U
+from tests.test_parity_gpu import _run
+
+pytestmark = pytest.mark.gpu
+
+
+def _want(q, seqs, k_type, mask=None):
+    if k_type == O.TYPE_F16:   # f32 accumulation against ggml-cpu's f16 accumulator: held to the f64 value
+        return np.stack([O.flash_attn_ext_f64(q[b:b + 1], k[None], k_type, dv=512, scale=U.SCALE,
+                                              mask=None if mask is None else mask[:, :k.shape[0]])[0] if len(k) else
+                         np.full((q.shape[2], q.shape[1], 512), np.nan, np.float32) for b, k in enumerate(seqs)])
+    outs = []
+    for b, k in enumerate(seqs):
+        if len(k) == 0:        # no key at all: 0 * (1/0), the reference's NaN row
+            outs.append(np.full((q.shape[2], q.shape[1], 512), np.nan, np.float32))
+        else:
+            outs.append(O.flash_attn_ext(q[b:b + 1], k[None], k_type, dv=512, scale=U.SCALE,
+                                         mask=None if mask is None else mask[:, :k.shape[0]])[0])
+    return np.stack(outs)
+
+
+@pytest.mark.parametrize("k_type", [O.TYPE_BF16, O.TYPE_F16, O.TYPE_Q8_0])
+@pytest.mark.parametrize("n_splits", [0, 3])
+def test_boundary_lengths_and_an_empty_sequence(gpu, k_type, n_splits):
+    rng = np.random.default_rng(11)
+    lens = [0, 1, 31, 32, 33, 127, 128, 129, 300]
+    pool, bt, seqs = U.make_paged(rng, np.maximum(lens, 1), k_type, n_pool_pages=16)
+    seqs = [s[:l] for s, l in zip(seqs, lens)]
+    bt = np.concatenate([bt, np.full((len(lens), 2), 2 ** 30, np.int32)], axis=1)   # table entries past every sequence: never read
+    q = rng.standard_normal((len(lens), 128, 1, 576)).astype(np.float32)
+    got = _run(gpu, q, pool, k_type, bt=bt, lens=lens, scale=U.SCALE, n_splits=n_splits)
+    print(U.check(got[..., :512], _want(q, seqs, k_type), "boundary lengths"))
+
+
+@pytest.mark.parametrize("k_type", [O.TYPE_BF16, O.TYPE_Q8_0])
+def test_partial_row_blocks(gpu, k_type):
+    """48 heads x 5 query tokens = 240 rows: one full block of 128 and one of 112, rows of one token split over blocks."""
+    rng = np.random.default_rng(12)
+    lens = [260, 200]
+    pool, bt, seqs = U.make_paged(rng, lens, k_type)
+    q = rng.standard_normal((2, 48, 5, 576)).astype(np.float32)
+    got = _run(gpu, q, pool, k_type, bt=bt, lens=lens, scale=U.SCALE)
+    print(U.check(got[..., :512], _want(q, seqs, k_type), "partial row blocks"))
+
+
+def test_partial_row_blocks_masked(gpu):
+    rng = np.random.default_rng(13)
+    n_tok, n_kv = 5, 384
+    q = rng.standard_normal((2, 48, n_tok, 576)).astype(np.float32)
+    k = U.encode_kv(rng.standard_normal((2, n_kv, 576)).astype(np.float32), O.TYPE_BF16)
+    m = np.where(np.arange(n_kv)[None, :] > 300 + 17 * np.arange(n_tok)[:, None], -np.inf, 0.0).astype(np.float32)
+    m[:, ::7] += 0.5
+    mask = m.astype(np.float16).view(np.uint16)
+    got = _run(gpu, q, k, O.TYPE_BF16, mask=mask, scale=U.SCALE)
+    want = O.flash_attn_ext(q, k, O.TYPE_BF16, dv=512, mask=mask, scale=U.SCALE)
+    print(U.check(got[..., :512], want, "partial row blocks, masked"))
+
+
+def test_strided_q(gpu):
+    """Q handed over as a permuted view ([seq, tok, head, 576] storage), the layout a fused Q projection would leave."""
+    import torch
+    import jittorinfer_amd as J
+    rng = np.random.default_rng(14)
+    q_store = rng.standard_normal((2, 3, 128, 576)).astype(np.float32)
+    k = U.encode_kv(rng.standard_normal((2, 256, 576)).astype(np.float32), O.TYPE_BF16)
+    tq = torch.from_numpy(q_store).to(gpu).permute(0, 2, 1, 3)   # [seq, head, tok, 576], non-contiguous
+    out = J.ggml_flash_attn_ext(tq, torch.from_numpy(k.view(np.int16)).to(gpu), O.TYPE_BF16, dv=512, scale=U.SCALE)
+    torch.cuda.synchronize()
+    want = O.flash_attn_ext(np.ascontiguousarray(q_store.transpose(0, 2, 1, 3)), k, O.TYPE_BF16, dv=512, scale=U.SCALE)
+    print(U.check(out.cpu().numpy()[..., :512], want, "strided q"))
+
+
+def test_full_size_config3_properties(gpu):
+    """BASELINE configs[2] at full size (B=32, H=128, ctx 8192, bf16 pages): the output does not depend on where the
+    pages sit in the pool (bit-exact under a permutation of pages + table), nor on the number of KV splits (within the
+    f16-partial rounding), and one sequence equals the oracle."""
+    import torch
+    import jittorinfer_amd as J
+    g = torch.Generator(device=gpu)
+    g.manual_seed(5)
+    B, H, L = 32, 128, 8192
+    pages = B * L // 128
+    pool = (torch.randn((pages * 128, 576), generator=g, device=gpu) * 0.5).to(torch.bfloat16).view(torch.int16)
+    bt = torch.randperm(pages, generator=g, device=gpu).to(torch.int32).reshape(B, L // 128).contiguous()
+    sl = torch.full((B,), L, dtype=torch.int32, device=gpu)
+    q = torch.randn((B, H, 1, 576), generator=g, device=gpu)
+    base = J.ggml_flash_attn_ext(q, pool, J.MLA_TYPE_BF16, dv=512, scale=U.SCALE, block_table=bt, seq_lens=sl)[..., :512].clone()
+    # (a) move every page: new_pool[perm[p]] = pool[p], table entries mapped through perm
+    perm = torch.randperm(pages, generator=g, device=gpu)
+    pool2 = torch.empty_like(pool)
+    pool2.view(pages, 128, 576)[perm] = pool.view(pages, 128, 576)
+    bt2 = perm[bt.long()].to(torch.int32).contiguous()
+    moved = J.ggml_flash_attn_ext(q, pool2, J.MLA_TYPE_BF16, dv=512, scale=U.SCALE, block_table=bt2, seq_lens=sl)[..., :512]
+    assert torch.equal(base, moved)
+    # (b) 16 splits instead of the planned 8
+    s16 = J.ggml_flash_attn_ext(q, pool, J.MLA_TYPE_BF16, dv=512, scale=U.SCALE, block_table=bt, seq_lens=sl, n_splits=16)[..., :512]
+    ma, rl = O.errors(s16.cpu().numpy(), base.cpu().numpy())
+    assert ma <= 5e-4 and rl <= 3e-4, (ma, rl)
+    # (c) sequence 7 against the oracle
+    b = 7
+    rows = (bt[b].long()[:, None] * 128 + torch.arange(128, device=gpu)[None, :]).reshape(-1)
+    k7 = pool[rows].cpu().numpy().view(np.uint16)[None]
+    want = O.flash_attn_ext(q[b:b + 1].cpu().numpy(), k7, O.TYPE_BF16, dv=512, scale=U.SCALE)
+    print(U.check(base[b:b + 1].cpu().numpy(), want, "config 3 full size, sequence 7"))
+
+
+def test_full_size_config4_causal_independence(gpu):
+    """BASELINE configs[3] at full size (B=4, H=16, 512 new tokens on 2048 cached, causal mask): query token t must not
+    depend on keys after position 2048 + t.  Keys after 2048 + 255 are replaced by other values: the outputs of tokens
+    0..255 stay bit-identical, later ones change; the last token's row equals the oracle."""
+    import torch
+    import jittorinfer_amd as J
+    g = torch.Generator(device=gpu)
+    g.manual_seed(6)
+    B, H, n_new, n_old = 4, 16, 512, 2048
+    L = n_new + n_old
+    pages = B * L // 128
+    pool = torch.randn((pages * 128, 576), generator=g, device=gpu).to(torch.bfloat16).view(torch.int16)
+    bt = torch.randperm(pages, generator=g, device=gpu).to(torch.int32).reshape(B, L // 128).contiguous()
+    sl = torch.full((B,), L, dtype=torch.int32, device=gpu)
+    q = torch.randn((B, H, n_new, 576), generator=g, device=gpu)
+    mask = torch.where(torch.arange(L, device=gpu)[None, :] > n_old + torch.arange(n_new, device=gpu)[:, None], float("-inf"), 0.0).to(torch.float16)
+    kw = dict(dv=512, scale=U.SCALE, mask=mask, block_table=bt, seq_lens=sl)
+    assert J.plan(q, pool, J.MLA_TYPE_BF16, **kw)["variant"] == 2
+    base = J.ggml_flash_attn_ext(q, pool, J.MLA_TYPE_BF16, **kw)[..., :512].clone()
+    pool2 = pool.clone()
+    for b in range(B):
+        pos = torch.arange(n_old + 256, L, device=gpu)
+        rows = bt[b].long()[pos // 128] * 128 + pos % 128
+        pool2[rows] = (torch.randn((len(pos), 576), generator=g, device=gpu) * 3).to(torch.bfloat16).view(torch.int16)
+    other = J.ggml_flash_attn_ext(q, pool2, J.MLA_TYPE_BF16, **kw)[..., :512]
+    assert torch.equal(base[:, :256], other[:, :256])
+    assert not torch.equal(base[:, 256:], other[:, 256:])
+    b = 2
+    rows = (bt[b].long()[:, None] * 128 + torch.arange(128, device=gpu)[None, :]).reshape(-1)
+    kb = pool[rows].cpu().numpy().view(np.uint16)[None]
+    mh = mask[-1:].cpu().numpy().view(np.uint16)
+    want = O.flash_attn_ext(q[b:b + 1, :, -1:].cpu().numpy(), kb, O.TYPE_BF16, dv=512, mask=mh, scale=U.SCALE)
+    print(U.check(base[b:b + 1, -1:].cpu().numpy(), want, "config 4 full size, last token"))
