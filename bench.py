@@ -228,6 +228,7 @@ def main():
                     help="also launch the library's plain copy kernel N times over one KV pool (known byte count) so that a "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run can be scaled")
     ap.add_argument("--kv", default="bf16", choices=["bf16", "f16", "q8_0"], help="storage type of the latent KV pool (the headline config is bf16; q8_0 only with --config kvwrite)")
+    ap.add_argument("--eager", action="store_true", help="time the K steps as K eager launch sequences instead of one replay of a HIP graph that holds them")
     ap.add_argument("--config", default="c3", choices=["c2", "c3", "c4", "c5", "kvwrite"],
                     help="c3 (default) is the headline workload; the others time BASELINE's remaining GPU configs and the cache write for the profiles")
     a = ap.parse_args()
@@ -276,13 +277,33 @@ def main():
         step(i)
     torch.cuda.synchronize()
 
-    # ---- timed region: exactly K steps, synchronised on both sides
+    # ---- timed region: exactly K steps, synchronised on both sides.  Eager: K calls of mla_attn_launch (three kernel
+    # launches each).  Default: the same K calls captured once into a HIP graph (the library neither allocates nor
+    # clears memory, so its launches can be captured) and replayed: what a serving loop does with a launch-bound step.
     t0 = time.perf_counter()
     for i in range(a.steps):
         step(i)
     torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    ms_per_step = wall * 1e3 / a.steps
+    eager_ms_per_step = (time.perf_counter() - t0) * 1e3 / a.steps
+    ms_per_step = eager_ms_per_step
+    if not a.eager:
+        side = torch.cuda.Stream(dev)
+        graph = torch.cuda.CUDAGraph()
+        sst = C.c_void_p(side.cuda_stream)
+        with torch.cuda.stream(side):
+            graph.capture_begin()
+            for i in range(a.steps):
+                rc = lib.mla_attn_launch(C.byref(args[i % len(args)]), sst)
+                if rc != 0:
+                    raise RuntimeError("launch failed during capture: %d" % rc)
+            graph.capture_end()
+        torch.cuda.synchronize()
+        graph.replay()          # untimed: first replay uploads the graph
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        graph.replay()          # K steps
+        torch.cuda.synchronize()
+        ms_per_step = (time.perf_counter() - t0) * 1e3 / a.steps
 
     # ---- the dominant kernel alone (the split-K decode kernel, without the Q pre-pack and the combine pass): HIP events
     # on the launch stream around K back-to-back launches (the stream is in order, so this is K kernel durations plus the
@@ -334,6 +355,8 @@ def main():
         "config": {"workload": "BASELINE configs[2]: paged MLA decode B=%d H=%d ctx=%d, bf16 latent KV 576/512, 128-token pages, shuffled block table" % (a.batch, a.heads, a.ctx),
                    "batch": a.batch, "heads": a.heads, "ctx": a.ctx, "kv_pools_rotated": a.pools, "plan": plan},
         "us_per_step": ms_per_step * 1e3,
+        "launch": "eager" if a.eager else "hip graph replay of the K steps",
+        "us_per_step_eager": eager_ms_per_step * 1e3,
         "us_per_step_events": step_ms_events * 1e3,
         "tokens_per_s": a.batch / (ms_per_step * 1e-3),
         "pct_hbm_peak": 100.0 * value / HBM_PEAK_GBPS,

@@ -144,3 +144,42 @@ def test_full_size_config4_causal_independence(gpu):
     mh = mask[-1:].cpu().numpy().view(np.uint16)
     want = O.flash_attn_ext(q[b:b + 1, :, -1:].cpu().numpy(), kb, O.TYPE_BF16, dv=512, mask=mh, scale=U.SCALE)
     print(U.check(base[b:b + 1, -1:].cpu().numpy(), want, "config 4 full size, last token"))
+
+
+def test_step_replayed_from_a_hip_graph(gpu):
+    """mla_attn_launch (Q pre-pack, split-K kernel, combine) captured into a HIP graph: every replay, with eager work and
+    synchronisations of the program's own in between and fresh inputs each time, equals the eager result bit for bit."""
+    import ctypes as C
+    import torch
+    import jittorinfer_amd as J
+    rng = np.random.default_rng(21)
+    lens = [700, 513, 260]
+    pool, bt, seqs = U.make_paged(rng, lens, O.TYPE_BF16)
+    tq = torch.zeros((3, 128, 1, 576), dtype=torch.float32, device=gpu)
+    tk = torch.from_numpy(pool.view(np.int16)).to(gpu)
+    tb, tl = torch.from_numpy(bt).to(gpu), torch.tensor(lens, dtype=torch.int32, device=gpu)
+    out = torch.zeros((3, 1, 128, 576), dtype=torch.float32, device=gpu)
+    a, _, keep = J.capi.make_args(tq, tk, J.MLA_TYPE_BF16, dv=512, scale=U.SCALE, block_table=tb, seq_lens=tl, out=out)
+    assert J.plan(tq, tk, J.MLA_TYPE_BF16, dv=512, scale=U.SCALE, block_table=tb, seq_lens=tl, out=out)["n_splits"] > 1
+    lib = J.library()
+    side = torch.cuda.Stream(gpu)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        graph.capture_begin()
+        assert lib.mla_attn_launch(C.byref(a), C.c_void_p(side.cuda_stream)) == 0
+        graph.capture_end()
+    torch.cuda.synchronize()
+    for it in range(4):
+        q = rng.standard_normal((3, 128, 1, 576)).astype(np.float32)
+        tq.copy_(torch.from_numpy(q).to(gpu))
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        replayed = out.clone()
+        out.fill_(float("nan"))
+        J.ggml_flash_attn_ext(tq, tk, J.MLA_TYPE_BF16, dv=512, scale=U.SCALE, block_table=tb, seq_lens=tl, out=out)   # eager
+        torch.cuda.synchronize()
+        assert torch.equal(replayed[..., :512], out[..., :512]), "replay %d differs from the eager launch" % it
+        if it == 0:
+            print(U.check(out.cpu().numpy()[..., :512], U.oracle_per_seq(q, seqs, O.TYPE_BF16, 512), "graph replay"))
