@@ -224,7 +224,7 @@ def q8_dma_lines(tile_sreg, raw_sreg):
 
 
 DQ_OUT = 224                                  # T[0:3]: the 8 f16 values of a unit
-DQ_W = [(228, 229, 241), (230, 231, 251)]     # two 12-byte raw windows (the next unit's reads are in flight during a unit's arithmetic)
+DQ_W = [(228, 229, 241), (230, 231, 251), (222, 223, 250)]   # three 12-byte raw windows: the reads of the next two units are in flight during a unit's arithmetic
 DQ_D = [249, 221]                             # the block scales of the two units in flight
 RAWA, DSTA, RAWD = 242, 243, 220
 
@@ -256,23 +256,29 @@ def q8_dequant_items(raw_sreg, dst_sreg, tile_plus):
     I.append("v_add_u32 %s, %s, %s" % (v(RAWD), s(SHM2), v(RAWD)))
     I.append("v_sub_u32 %s, %s, %s" % (v(RAWD), v(RAWA), v(RAWD)))
 
-    def reads(u):
-        w = DQ_W[u & 1]
+    def reads_w(u):
+        w = DQ_W[u % 3]
         def f0():
             lds.read("ds_read2_b32 %s, %s offset0:%d offset1:%d" % (v(w[0], 2), v(RAWA), 17 * u, 17 * u + 1), ("r", u, 0))
         def f1():
             lds.read("ds_read_b32 %s, %s offset:%d" % (v(w[2]), v(RAWA), 68 * u + 8), ("r", u, 1))
+        return [f0, f1]
+
+    def reads_d(u):
         def f2():
             lds.read("ds_read_u16 %s, %s offset:%d" % (v(DQ_D[u & 1]), v(RAWD), 68 * u), ("r", u, 2))
-        return [f0, f1, f2]
+        return [f2]
 
-    I += reads(0)
+    I += reads_w(0) + reads_d(0) + reads_w(1)
     for u in range(9):
-        w, d = DQ_W[u & 1], DQ_D[u & 1]
+        w, d = DQ_W[u % 3], DQ_D[u & 1]
         if u + 1 < 9:
-            I += reads(u + 1)
+            I += reads_d(u + 1)
+        if u + 2 < 9:
+            I += reads_w(u + 2)
         def first(u=u, w=w):
             lds.need(("r", u, 2))
+            lds.need(("r", u, 1))
             e("v_alignbyte_b32 %s, %s, %s, %s" % (v(w[0]), v(w[1]), v(w[0]), s(SH)))      # values 0..3
         I.append(first)
         if NO_DQ_VALU:
