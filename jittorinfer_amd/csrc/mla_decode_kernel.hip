@@ -70,8 +70,10 @@ constexpr int lds_total(int kvt) { return handoff_off(kvt) + NTHREADS * 32; }
 // The wave-level program is generated by gen_decode_asm.py (register map, LDS-DMA issue, MFMA/VALU interleave).
 // KVT = SRC_BF16: bf16 KV rows, bf16 MFMA, P fed as hi + lo halves.   SRC_F16: f16 KV rows, f16 MFMA, single P.
 // SRC_Q8: packed Q8_0 rows (612 bytes, contiguous), dequantized in LDS to f16 tiles one tile ahead, then as SRC_F16.
-// MASK: an f16 mask row per query token is added to the scaled scores (ggml-cpu.c:12041-12057); the keys past
-// p.mask_ext[row block] (the last key any row of the block may attend to, rounded up to a tile) are not visited.
+// MASK: an f16 mask row per query token is added to the scaled scores (ggml-cpu.c:12041-12057).  Only the key range
+// p.mask_ext[2*row block .. +1] (first / one past the last key that any row of the block may attend to, rounded to
+// tiles) is visited, and the KV splits divide that range, not the whole cache: the reference's batched decode, where
+// every token sees only its own sequence's cells of one shared cache, costs what its own cells cost.
 template <int KVT, bool MASK>
 __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
     constexpr int HANDOFF_OFF = handoff_off(KVT);
@@ -83,8 +85,8 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
     const int b = blockIdx.z, split = blockIdx.x;
 
     const int seq_len  = p.block_table ? min(p.seq_lens[b], (int) p.bt_stride * MLA_PAGE_TOKENS) : (int) p.n_kv;
-    const int kv_begin = split * p.split_tokens;
-    int       kv_end   = min(seq_len, kv_begin + p.split_tokens);
+    int kv_begin = split * p.split_tokens;
+    int kv_end   = min(seq_len, kv_begin + p.split_tokens);
     const int row       = blockIdx.y * 128 + wave * 32 + rl;
     const bool row_valid = row < p.n_rows;
     const int64_t orow  = (int64_t) b * p.n_rows + row;
@@ -92,15 +94,18 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
 
     bool all_masked = false;  // this split holds keys, but none that a row of this block may attend to
     if constexpr (MASK) {
-        const int ext = min(kv_end, p.mask_ext[blockIdx.y]);
-        all_masked = kv_begin < kv_end && (ext <= kv_begin) && !(split == 0);  // split 0 always runs (an all-masked row must come out NaN)
-        if (!all_masked) kv_end = max(ext, min(kv_end, kv_begin + TILE_TOK));
+        const int hi = min(seq_len, p.mask_ext[2 * blockIdx.y + 1]), lo = min(p.mask_ext[2 * blockIdx.y], hi);
+        int chunk = ((hi - lo + p.n_splits - 1) / p.n_splits + TILE_TOK - 1) / TILE_TOK * TILE_TOK;
+        kv_begin = lo + split * chunk;
+        kv_end   = min(hi, kv_begin + chunk);
+        if (split == 0 && kv_end <= kv_begin) kv_end = min(seq_len, kv_begin + TILE_TOK);  // no key at all: one masked tile, so that the rows come out NaN
+        all_masked = seq_len > 0 && kv_begin >= kv_end;
     }
     if (kv_begin >= kv_end || all_masked) {
         // Nothing to read.  Only the first split of an empty sequence writes something: a NaN row, like the reference's
         // 0 * (1/0); other empty splits are skipped by the combine pass.  A split whose keys are all masked tells the
         // combine pass so (m = -inf).
-        if (all_masked && row_valid && g == 0) {
+        if ((all_masked || (MASK && split > 0)) && p.n_splits > 1 && row_valid && g == 0) {
             p.part_ml[prow * 2] = -INFINITY;
             p.part_ml[prow * 2 + 1] = 0.f;
         } else if (seq_len <= 0 && split == 0 && row_valid && g == 0) {
@@ -189,39 +194,50 @@ __global__ void __launch_bounds__(NTHREADS) mla_q_pack_kernel(const KParams p) {
     out[ks * 64] = u32x4{ pack2<F16>(x0.x, x0.y), pack2<F16>(x0.z, x0.w), pack2<F16>(x1.x, x1.y), pack2<F16>(x1.z, x1.w) };
 }
 
-// Per block of 128 rows: one past the last key that any of its query tokens may attend to (mask value != -inf),
-// rounded up to a whole tile.  grid = n_row_blocks, block = 256.  The mask is shared by all sequences (ggml-cpu.c:12024).
+// Per block of 128 rows: the first key and one past the last key that any of its query tokens may attend to (mask value
+// != -inf), rounded outwards to whole tiles; 0, 0 when there is none.  grid = n_row_blocks, block = 256.  The mask is
+// shared by all sequences (ggml-cpu.c:12024).
 __global__ void __launch_bounds__(NTHREADS) mla_mask_extent_kernel(const KParams p) {
-    __shared__ int red[NTHREADS];
+    __shared__ int red_hi[NTHREADS], red_lo[NTHREADS];
     const int tid = threadIdx.x;
     const int r0 = blockIdx.x * 128, r1 = min(r0 + 127, p.n_rows - 1);
     const int t0 = r0 / p.n_head, t1 = r1 / p.n_head;
     const int n_kv = (int) (p.block_table ? p.bt_stride * MLA_PAGE_TOKENS : p.n_kv);
     const int n8 = n_kv / 8;   // groups of 8 mask values (16 bytes); n_kv is a multiple of 32 on this path
-    int ext = 0;
-    for (int t = t0; t <= t1; t++) {
-        const u32x4 * mrow = (const u32x4 *) (p.mask + (int64_t) t * p.mask_nb1);   // 8-byte aligned rows: read as 2 x 8 bytes
-        for (int i = n8 - 1 - tid; i >= 0; i -= NTHREADS) {
-            if (8 * i + 8 <= ext) break;
-            const u32x2 lo = *(const u32x2 *) ((const char *) mrow + 16 * (int64_t) i);
-            const u32x2 hi = *(const u32x2 *) ((const char *) mrow + 16 * (int64_t) i + 8);
-            const unsigned w[4] = { lo.x, lo.y, hi.x, hi.y };
-            int last = -1;
+    int hi = 0, lo = n_kv;
+    auto group = [&](const char * mrow, int i, int & first, int & last) {   // rows are 8-byte aligned: 2 x 8 bytes
+        const u32x2 a = *(const u32x2 *) (mrow + 16 * (int64_t) i), b = *(const u32x2 *) (mrow + 16 * (int64_t) i + 8);
+        const unsigned w[4] = { a.x, a.y, b.x, b.y };
+        first = 8; last = -1;
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                if ((w[e] & 0xffff) != 0xfc00u) last = 2 * e;
-                if ((w[e] >> 16) != 0xfc00u) last = 2 * e + 1;
-            }
-            if (last >= 0) { ext = max(ext, 8 * i + last + 1); break; }   // this thread's groups further left are lower
+        for (int e = 7; e >= 0; e--) if (((w[e >> 1] >> (16 * (e & 1))) & 0xffff) != 0xfc00u) first = e;
+#pragma unroll
+        for (int e = 0; e < 8; e++) if (((w[e >> 1] >> (16 * (e & 1))) & 0xffff) != 0xfc00u) last = e;
+    };
+    for (int t = t0; t <= t1; t++) {
+        const char * mrow = p.mask + (int64_t) t * p.mask_nb1;
+        for (int i = n8 - 1 - tid; i >= 0 && 8 * i + 8 > hi; i -= NTHREADS) {      // from the right: this thread's groups further left are lower
+            int first, last;
+            group(mrow, i, first, last);
+            if (last >= 0) { hi = max(hi, 8 * i + last + 1); break; }
+        }
+        for (int i = tid; i < n8 && 8 * i < lo; i += NTHREADS) {                   // from the left
+            int first, last;
+            group(mrow, i, first, last);
+            if (first < 8) { lo = min(lo, 8 * i + first); break; }
         }
     }
-    red[tid] = ext;
+    red_hi[tid] = hi; red_lo[tid] = lo;
     __syncthreads();
     for (int o = NTHREADS / 2; o > 0; o >>= 1) {
-        if (tid < o) red[tid] = max(red[tid], red[tid + o]);
+        if (tid < o) { red_hi[tid] = max(red_hi[tid], red_hi[tid + o]); red_lo[tid] = min(red_lo[tid], red_lo[tid + o]); }
         __syncthreads();
     }
-    if (tid == 0) p.mask_ext[blockIdx.x] = min(n_kv, (red[0] + TILE_TOK - 1) / TILE_TOK * TILE_TOK);
+    if (tid == 0) {
+        const int h = min(n_kv, (red_hi[0] + TILE_TOK - 1) / TILE_TOK * TILE_TOK);
+        p.mask_ext[2 * blockIdx.x]     = h > 0 ? red_lo[0] / TILE_TOK * TILE_TOK : 0;
+        p.mask_ext[2 * blockIdx.x + 1] = h;
+    }
 }
 
 // The same image for Q8_0 KV: ggml-cpu quantizes Q to Q8_0 when K is Q8_0 (ggml-cpu.c:313-322, :12034-12035): per block of 32

@@ -409,7 +409,7 @@ __global__ void __launch_bounds__(256) mla_attn_combine_kernel(const KParams p) 
     if (row >= p.n_rows || cg * 8 >= p.dv_total) return;
     const int seq_len = p.block_table ? min(p.seq_lens[b], (int) p.bt_stride * MLA_PAGE_TOKENS) : (int) p.n_kv;
     int nvalid = (seq_len + p.split_tokens - 1) / p.split_tokens;
-    nvalid = min(nvalid, p.n_splits);
+    nvalid = p.rel_splits ? p.n_splits : min(nvalid, p.n_splits);
 
     const float2 *   ml = (const float2 *) p.part_ml + (int64_t) b * p.n_splits * p.n_rows + row;
     const _Float16 * po = p.part_o + (int64_t) b * p.n_splits * p.n_rows * p.dv_total + ((int64_t) cg * p.n_rows + row) * 8;
@@ -440,6 +440,7 @@ __global__ void __launch_bounds__(256) mla_attn_combine_kernel(const KParams p) 
             // l_c 2^(m_c - M); a split that saw only masked keys (m_c = -inf) and the padding of the group get 0
             const float w = (c0 + k < nvalid && mlv[k].x != -INFINITY) ? mlv[k].y * fast_exp2(mlv[k].x - M) : 0.f;
             L += w;
+            if (w == 0.f) continue;  // its partial may hold anything (0/0 of a split without a key), never multiply it in
             const unsigned h[4] = { hv[k].x, hv[k].y, hv[k].z, hv[k].w };
 #pragma unroll
             for (int e = 0; e < 4; e++) {
@@ -465,7 +466,7 @@ __global__ void __launch_bounds__(256) mla_attn_combine_f32_kernel(const KParams
     if (row >= p.n_rows || threadIdx.x >= rows_per_block * groups_per_row || cg * 4 >= p.dv_total) return;
     const int seq_len = p.block_table ? min(p.seq_lens[b], (int) p.bt_stride * MLA_PAGE_TOKENS) : (int) p.n_kv;
     int nvalid = (seq_len + p.split_tokens - 1) / p.split_tokens;
-    nvalid = min(nvalid, p.n_splits);
+    nvalid = p.rel_splits ? p.n_splits : min(nvalid, p.n_splits);
     const float2 * ml = (const float2 *) p.part_ml + (int64_t) b * p.n_splits * p.n_rows + row;
     const float *  po = (const float *) p.part_o + ((int64_t) b * p.n_splits * p.n_rows + row) * p.dv_total + cg * 4;
     const int64_t ml_step = p.n_rows, po_step = (int64_t) p.n_rows * p.dv_total;
@@ -635,7 +636,9 @@ int make_plan(const mla_attn_args * a, Plan * pl) {
         splits = (256 + wgs - 1) / wgs;
         if (pl->wd > 1) splits *= 2;  // small-row shapes leave room for two workgroups per CU
     }
-    if (pl->variant == 2 && splits * 64 < n_pages) splits = (n_pages + 63) / 64;  // that kernel indexes at most 64 pages per split
+    // that kernel indexes at most 64 pages per split (63 with a mask, whose splits need not start on a page boundary)
+    const int64_t max_pages = pl->variant == 2 && a->mask ? 63 : 64;
+    if (pl->variant == 2 && splits * max_pages < n_pages) splits = (n_pages + max_pages - 1) / max_pages;
     if (splits > n_pages) splits = n_pages;
     if (splits < 1) splits = 1;
     const int64_t pages_per_split = (n_pages + splits - 1) / splits;
@@ -643,7 +646,7 @@ int make_plan(const mla_attn_args * a, Plan * pl) {
     pl->n_splits     = (int) ((n_pages + pages_per_split - 1) / pages_per_split);
     pl->lds_bytes    = pl->variant == 2 ? decode_fast_lds_bytes(a->kv_type) : 2 * TILE_BYTES + (a->kv_type == MLA_TYPE_Q8_0 ? Q8_TILE_RAW : 0);
     if (pl->variant == 2) pl->ws_qpack = decode_fast_qpack_bytes(a->n_seq, pl->n_row_blocks);
-    if (pl->variant == 2 && a->mask) pl->ws_maskext = (size_t) pl->n_row_blocks * sizeof(int);
+    if (pl->variant == 2 && a->mask) pl->ws_maskext = (size_t) pl->n_row_blocks * 2 * sizeof(int);
     if (pl->n_splits > 1) {
         // f32 partials while they are small (no second rounding of O on top of the MFMA operands' one), f16 beyond: there the
         // partial traffic counts, and the rounding (2^-12 relative per split) is averaged over long contexts
@@ -738,6 +741,7 @@ static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
     char * ws = (char *) a->workspace;
     kp.part_o  = (_Float16 *) ws;
     kp.part_f32 = pl.part_f32;
+    kp.rel_splits = pl.variant == 2 && a->mask != nullptr;
     kp.part_ml = (float *) (ws + align256(pl.ws_part_o));
     float * scores = (float *) (ws + align256(pl.ws_part_o) + align256(pl.ws_part_ml));
     kp.q_pack = ws + align256(pl.ws_part_o) + align256(pl.ws_part_ml) + align256(pl.ws_scores);

@@ -183,3 +183,40 @@ def test_step_replayed_from_a_hip_graph(gpu):
         assert torch.equal(replayed[..., :512], out[..., :512]), "replay %d differs from the eager launch" % it
         if it == 0:
             print(U.check(out.cpu().numpy()[..., :512], U.oracle_per_seq(q, seqs, O.TYPE_BF16, 512), "graph replay"))
+
+
+@pytest.mark.parametrize("k_type", [O.TYPE_BF16, O.TYPE_F16])
+@pytest.mark.parametrize("n_splits", [0, 1, 5])
+def test_reference_style_batched_decode_through_the_mask(gpu, k_type, n_splits):
+    """The reference's own decode batch (no block table): one shared cache, one query token per sequence, and the f16 mask
+    (src/llama-context.cpp:364-404) selects every token's own cells.  The pipelined kernel visits only the key range a
+    token's mask leaves open and divides that range into the KV splits."""
+    import torch
+    import jittorinfer_amd as J
+    rng = np.random.default_rng(31 + n_splits)
+    lens = [300, 512, 77, 1024, 5, 640, 128, 900]
+    order = rng.permutation(len(lens))
+    n_kv, start = 4352, {}
+    pos = 17
+    for s in order:                       # sequences sit in the cache in shuffled order with gaps between them
+        start[s] = pos
+        pos += lens[s] + int(rng.integers(0, 40))
+    assert pos <= n_kv
+    k = U.encode_kv((rng.standard_normal((1, n_kv, 576)) * 30).astype(np.float32), k_type)   # other cells: wild values
+    m = np.full((len(lens), n_kv), -np.inf, dtype=np.float32)
+    for s, l in enumerate(lens):
+        k[0, start[s]:start[s] + l] = U.encode_kv(rng.standard_normal((l, 576)).astype(np.float32), k_type)
+        m[s, start[s]:start[s] + l] = 0.0
+    m[3, start[3] + 100:start[3] + 400] = -np.inf       # a hole inside a sequence (cells of a removed span)
+    mask = m.astype(np.float16).view(np.uint16)
+    q = rng.standard_normal((1, 128, len(lens), 576)).astype(np.float32)
+    tq = torch.from_numpy(q).to(gpu)
+    tk = torch.from_numpy(k.view(np.int16)).to(gpu)
+    tm = torch.from_numpy(mask.view(np.float16)).to(gpu)
+    assert J.plan(tq, tk, k_type, dv=512, scale=U.SCALE, mask=tm, n_splits=n_splits)["variant"] == 2
+    got = _run(gpu, q, k, k_type, mask=mask, scale=U.SCALE, n_splits=n_splits)
+    if k_type == O.TYPE_F16:
+        want = O.flash_attn_ext_f64(q, k, k_type, dv=512, mask=mask, scale=U.SCALE)
+    else:
+        want = O.flash_attn_ext(q, k, k_type, dv=512, mask=mask, scale=U.SCALE)
+    print(U.check(got[..., :512], want, "batched decode through the mask"))
