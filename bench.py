@@ -125,6 +125,20 @@ def other_config(a, dev, lib, J):
     if a.config == "c2":
         lens, n_head, n_tok, kv, kvt = [int(x) for x in rng.integers(512, 4097, 8)], 16, 1, "bf16", J.MLA_TYPE_BF16
         name = "BASELINE configs[1]: paged MLA decode B=8 H=16 L~U[512,4096], bf16"
+    elif a.config == "c3mask":
+        # the headline shape as the reference's unmodified graph presents it: no block table, one cache shared by the 32
+        # sequences, one query token per sequence, membership through the f16 mask (src/llama-context.cpp:364-404)
+        B, L = 32, 8192
+        g = torch.Generator(device=dev)
+        g.manual_seed(a.seed)
+        pool = (torch.randn((1, B * L, 576), generator=g, device=dev) * 0.5).to(torch.bfloat16).view(torch.int16)
+        q = torch.randn((1, 128, B, 576), generator=g, device=dev)
+        mask = torch.full((64, B * L), float("-inf"), dtype=torch.float16, device=dev)
+        for b in range(B):
+            mask[b, b * L:(b + 1) * L] = 0
+        out = torch.empty((1, B, 128, 576), dtype=torch.float32, device=dev)
+        lens, n_head, n_tok, kv, kvt = [L] * B, 128, B, "bf16", J.MLA_TYPE_BF16
+        name = "BASELINE configs[2] without the block table: one shared cache of 262144 cells, 32 query tokens, f16 mask selects each token's 8192 cells"
     elif a.config == "c4":
         lens, n_head, n_tok, kv, kvt = [2560] * 4, 16, 512, "bf16", J.MLA_TYPE_BF16
         mask = torch.where(torch.arange(2560, device=dev)[None, :] > 2048 + torch.arange(512, device=dev)[:, None], float("-inf"), 0.0).to(torch.float16)
@@ -132,8 +146,11 @@ def other_config(a, dev, lib, J):
     else:
         lens, n_head, n_tok, kv, kvt = [int(x) for x in rng.integers(2048, 8193, 64)], 128, 1, "q8_0", J.MLA_TYPE_Q8_0
         name = "BASELINE configs[4]: paged MLA decode B=64 H=128 L~U[2048,8192], Q8_0 pages"
-    q, pool, bt, sl = build_paged(dev, lens, n_head, n_tok, kv, a.seed)
-    out = torch.empty((len(lens), n_tok, n_head, 576), dtype=torch.float32, device=dev)
+    if a.config == "c3mask":
+        bt = sl = None
+    else:
+        q, pool, bt, sl = build_paged(dev, lens, n_head, n_tok, kv, a.seed)
+        out = torch.empty((len(lens), n_tok, n_head, 576), dtype=torch.float32, device=dev)
     kw = dict(dv=512, scale=scale, mask=mask, block_table=bt, seq_lens=sl, out=out, n_splits=a.splits, rows_per_wg=a.rows_per_wg)
     ar, _, keep = J.capi.make_args(q, pool, kvt, **kw)
     plan = J.plan(q, pool, kvt, **kw)
@@ -229,7 +246,7 @@ def main():
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run can be scaled")
     ap.add_argument("--kv", default="bf16", choices=["bf16", "f16", "q8_0"], help="storage type of the latent KV pool (the headline config is bf16; q8_0 only with --config kvwrite)")
     ap.add_argument("--eager", action="store_true", help="time the K steps as K eager launch sequences instead of one replay of a HIP graph that holds them")
-    ap.add_argument("--config", default="c3", choices=["c2", "c3", "c4", "c5", "kvwrite"],
+    ap.add_argument("--config", default="c3", choices=["c2", "c3", "c3mask", "c4", "c5", "kvwrite"],
                     help="c3 (default) is the headline workload; the others time BASELINE's remaining GPU configs and the cache write for the profiles")
     a = ap.parse_args()
     if a.gpus != 1:

@@ -60,7 +60,7 @@ struct KParams {
     int             debug_flags;   // development builds of the decode kernel only
     void *          debug_ptr;
     int             n_pool_pages;  // block-table mode: pages in the pool
-    int *           mask_ext;      // pipelined kernel with a mask: per block of 128 rows, first / one past the last key that is not masked for all its rows (workspace)
+    int *           mask_ext;      // pipelined kernel with a mask: per block of 128 rows, 16 pairs (first, one past the last key that is not masked for all its rows) (workspace)
     int             rel_splits;    // the KV splits divide that key range (every split writes its (m, l), -inf when it has no key)
     int             rows_contig;  // kv rows are packed (kv_nb1 == row bytes): whole tiles are one contiguous run
 };

@@ -94,7 +94,12 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
 
     bool all_masked = false;  // this split holds keys, but none that a row of this block may attend to
     if constexpr (MASK) {
-        const int hi = min(seq_len, p.mask_ext[2 * blockIdx.y + 1]), lo = min(p.mask_ext[2 * blockIdx.y], hi);
+        int mlo = 0x7fffffff, mhi = 0;
+        for (int c = 0; c < 16; c++) {
+            mlo = min(mlo, p.mask_ext[(blockIdx.y * 16 + c) * 2]);
+            mhi = max(mhi, p.mask_ext[(blockIdx.y * 16 + c) * 2 + 1]);
+        }
+        const int hi = min(seq_len, (mhi + TILE_TOK - 1) / TILE_TOK * TILE_TOK), lo = min(mlo / TILE_TOK * TILE_TOK, hi);
         int chunk = ((hi - lo + p.n_splits - 1) / p.n_splits + TILE_TOK - 1) / TILE_TOK * TILE_TOK;
         kv_begin = lo + split * chunk;
         kv_end   = min(hi, kv_begin + chunk);
@@ -194,9 +199,11 @@ __global__ void __launch_bounds__(NTHREADS) mla_q_pack_kernel(const KParams p) {
     out[ks * 64] = u32x4{ pack2<F16>(x0.x, x0.y), pack2<F16>(x0.z, x0.w), pack2<F16>(x1.x, x1.y), pack2<F16>(x1.z, x1.w) };
 }
 
-// Per block of 128 rows: the first key and one past the last key that any of its query tokens may attend to (mask value
-// != -inf), rounded outwards to whole tiles; 0, 0 when there is none.  grid = n_row_blocks, block = 256.  The mask is
-// shared by all sequences (ggml-cpu.c:12024).
+// Per block of 128 rows and per sixteenth of the mask row: the first key and one past the last key that any of the
+// block's query tokens may attend to (mask value != -inf); n_kv, 0 when there is none.  The attention kernel merges the
+// 16 pairs and rounds outwards to tiles.  grid = (n_row_blocks, 16), block = 256.  The mask is shared by all sequences
+// (ggml-cpu.c:12024).
+constexpr int MASK_EXT_CHUNKS = 16;
 __global__ void __launch_bounds__(NTHREADS) mla_mask_extent_kernel(const KParams p) {
     __shared__ int red_hi[NTHREADS], red_lo[NTHREADS];
     const int tid = threadIdx.x;
@@ -204,27 +211,16 @@ __global__ void __launch_bounds__(NTHREADS) mla_mask_extent_kernel(const KParams
     const int t0 = r0 / p.n_head, t1 = r1 / p.n_head;
     const int n_kv = (int) (p.block_table ? p.bt_stride * MLA_PAGE_TOKENS : p.n_kv);
     const int n8 = n_kv / 8;   // groups of 8 mask values (16 bytes); n_kv is a multiple of 32 on this path
+    const int g0 = (int) ((int64_t) n8 * blockIdx.y / MASK_EXT_CHUNKS), g1 = (int) ((int64_t) n8 * (blockIdx.y + 1) / MASK_EXT_CHUNKS);
     int hi = 0, lo = n_kv;
-    auto group = [&](const char * mrow, int i, int & first, int & last) {   // rows are 8-byte aligned: 2 x 8 bytes
-        const u32x2 a = *(const u32x2 *) (mrow + 16 * (int64_t) i), b = *(const u32x2 *) (mrow + 16 * (int64_t) i + 8);
-        const unsigned w[4] = { a.x, a.y, b.x, b.y };
-        first = 8; last = -1;
-#pragma unroll
-        for (int e = 7; e >= 0; e--) if (((w[e >> 1] >> (16 * (e & 1))) & 0xffff) != 0xfc00u) first = e;
-#pragma unroll
-        for (int e = 0; e < 8; e++) if (((w[e >> 1] >> (16 * (e & 1))) & 0xffff) != 0xfc00u) last = e;
-    };
     for (int t = t0; t <= t1; t++) {
         const char * mrow = p.mask + (int64_t) t * p.mask_nb1;
-        for (int i = n8 - 1 - tid; i >= 0 && 8 * i + 8 > hi; i -= NTHREADS) {      // from the right: this thread's groups further left are lower
-            int first, last;
-            group(mrow, i, first, last);
-            if (last >= 0) { hi = max(hi, 8 * i + last + 1); break; }
-        }
-        for (int i = tid; i < n8 && 8 * i < lo; i += NTHREADS) {                   // from the left
-            int first, last;
-            group(mrow, i, first, last);
-            if (first < 8) { lo = min(lo, 8 * i + first); break; }
+        for (int i = g0 + tid; i < g1; i += NTHREADS) {
+            const u32x2 a = *(const u32x2 *) (mrow + 16 * (int64_t) i), b = *(const u32x2 *) (mrow + 16 * (int64_t) i + 8);   // rows are 8-byte aligned
+            const unsigned w[4] = { a.x, a.y, b.x, b.y };
+#pragma unroll
+            for (int e = 0; e < 8; e++)
+                if (((w[e >> 1] >> (16 * (e & 1))) & 0xffff) != 0xfc00u) { lo = min(lo, 8 * i + e); hi = max(hi, 8 * i + e + 1); }
         }
     }
     red_hi[tid] = hi; red_lo[tid] = lo;
@@ -234,9 +230,8 @@ __global__ void __launch_bounds__(NTHREADS) mla_mask_extent_kernel(const KParams
         __syncthreads();
     }
     if (tid == 0) {
-        const int h = min(n_kv, (red_hi[0] + TILE_TOK - 1) / TILE_TOK * TILE_TOK);
-        p.mask_ext[2 * blockIdx.x]     = h > 0 ? red_lo[0] / TILE_TOK * TILE_TOK : 0;
-        p.mask_ext[2 * blockIdx.x + 1] = h;
+        p.mask_ext[(blockIdx.x * MASK_EXT_CHUNKS + blockIdx.y) * 2]     = red_lo[0];
+        p.mask_ext[(blockIdx.x * MASK_EXT_CHUNKS + blockIdx.y) * 2 + 1] = red_hi[0];
     }
 }
 
@@ -319,7 +314,7 @@ hipError_t launch_decode_fast(const KParams & kp, int kv_type, dim3 grid, hipStr
     else if (kv_type == MLA_TYPE_Q8_0)     hipLaunchKernelGGL(mla_q_pack_q8_kernel, dim3(grid.y, grid.z, KSTEPS / 2), dim3(NTHREADS), 0, st, kp);
     else if (kv_type == MLA_TYPE_F16) hipLaunchKernelGGL(mla_q_pack_kernel<true>, dim3(grid.y, grid.z, KSTEPS), dim3(NTHREADS), 0, st, kp);
     else                              hipLaunchKernelGGL(mla_q_pack_kernel<false>, dim3(grid.y, grid.z, KSTEPS), dim3(NTHREADS), 0, st, kp);
-    if (m && with_prepass) hipLaunchKernelGGL(mla_mask_extent_kernel, dim3(grid.y), dim3(NTHREADS), 0, st, kp);
+    if (m && with_prepass) hipLaunchKernelGGL(mla_mask_extent_kernel, dim3(grid.y, MASK_EXT_CHUNKS), dim3(NTHREADS), 0, st, kp);
     if (kv_type == MLA_TYPE_Q8_0) return launch_variant<SRC_Q8, false>(kp, grid, st);
     if (kv_type == MLA_TYPE_F16)  return m ? launch_variant<SRC_F16, true>(kp, grid, st) : launch_variant<SRC_F16, false>(kp, grid, st);
     return m ? launch_variant<SRC_BF16, true>(kp, grid, st) : launch_variant<SRC_BF16, false>(kp, grid, st);

@@ -636,9 +636,9 @@ int make_plan(const mla_attn_args * a, Plan * pl) {
         splits = (256 + wgs - 1) / wgs;
         if (pl->wd > 1) splits *= 2;  // small-row shapes leave room for two workgroups per CU
     }
-    // that kernel indexes at most 64 pages per split (63 with a mask, whose splits need not start on a page boundary)
+    // with a block table that kernel indexes at most 64 pages per split (63 with a mask, whose splits need not start on a page boundary)
     const int64_t max_pages = pl->variant == 2 && a->mask ? 63 : 64;
-    if (pl->variant == 2 && splits * max_pages < n_pages) splits = (n_pages + max_pages - 1) / max_pages;
+    if (pl->variant == 2 && a->block_table && splits * max_pages < n_pages) splits = (n_pages + max_pages - 1) / max_pages;
     if (splits > n_pages) splits = n_pages;
     if (splits < 1) splits = 1;
     const int64_t pages_per_split = (n_pages + splits - 1) / splits;
@@ -646,7 +646,7 @@ int make_plan(const mla_attn_args * a, Plan * pl) {
     pl->n_splits     = (int) ((n_pages + pages_per_split - 1) / pages_per_split);
     pl->lds_bytes    = pl->variant == 2 ? decode_fast_lds_bytes(a->kv_type) : 2 * TILE_BYTES + (a->kv_type == MLA_TYPE_Q8_0 ? Q8_TILE_RAW : 0);
     if (pl->variant == 2) pl->ws_qpack = decode_fast_qpack_bytes(a->n_seq, pl->n_row_blocks);
-    if (pl->variant == 2 && a->mask) pl->ws_maskext = (size_t) pl->n_row_blocks * 2 * sizeof(int);
+    if (pl->variant == 2 && a->mask) pl->ws_maskext = (size_t) pl->n_row_blocks * 16 * 2 * sizeof(int);  // 16 (first, last) pairs per row block
     if (pl->n_splits > 1) {
         // f32 partials while they are small (no second rounding of O on top of the MFMA operands' one), f16 beyond: there the
         // partial traffic counts, and the rounding (2^-12 relative per split) is averaged over long contexts
