@@ -59,6 +59,20 @@ def library():
         lib.mla_hbm_copy_launch.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
         lib.mla_kv_write_launch.restype = C.c_int
         lib.mla_kv_write_launch.argtypes = [C.POINTER(MlaKvWriteArgs), C.c_void_p]
+        lib.mla_page_table_create.restype = C.c_void_p
+        lib.mla_page_table_create.argtypes = [C.c_int32] * 3
+        lib.mla_page_table_free.argtypes = [C.c_void_p]
+        lib.mla_page_table_clear.argtypes = [C.c_void_p]
+        lib.mla_page_table_find_slot.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p]
+        lib.mla_page_table_seq_rm.argtypes = [C.c_void_p, C.c_int32, C.c_int32, C.c_int32]
+        lib.mla_page_table_seq_cp.argtypes = [C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_int32] + [C.POINTER(C.c_int32)] * 3
+        lib.mla_page_table_seq_keep.argtypes = [C.c_void_p, C.c_int32]
+        for name in ("mla_page_table_seq_len", "mla_page_table_free_pages", "mla_page_table_used_cells"):
+            getattr(lib, name).restype = C.c_int32
+        lib.mla_page_table_seq_len.argtypes = [C.c_void_p, C.c_int32]
+        lib.mla_page_table_free_pages.argtypes = [C.c_void_p]
+        lib.mla_page_table_used_cells.argtypes = [C.c_void_p]
+        lib.mla_page_table_fill_inputs.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p]
         lib.mla_attn_target_arch.restype = C.c_char_p
         lib.ggml_backend_init.restype = C.c_void_p
         lib.ggml_backend_score.restype = C.c_int
@@ -205,3 +219,73 @@ def kv_write(src, cache, kv_type, *, row0=None, rows=None, block_table=None, seq
     if rc != 0:
         raise RuntimeError("mla_kv_write_launch failed with code %d" % rc)
     return cache
+
+
+class PageTable:
+    """Host-side page allocator / block-table builder (include/mla_page_table.h): the paged counterpart of the reference's
+    llama_kv_cache bookkeeping (src/llama-kv-cache.cpp) and of the mask builder of llama_set_inputs.  numpy in, numpy out."""
+
+    def __init__(self, n_pages, n_seq_max, max_blocks):
+        self._lib = library()
+        self.n_pages, self.n_seq_max, self.max_blocks = n_pages, n_seq_max, max_blocks
+        self._h = self._lib.mla_page_table_create(n_pages, n_seq_max, max_blocks)
+        if not self._h:
+            raise ValueError("mla_page_table_create rejected the sizes")
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            self._lib.mla_page_table_free(self._h)
+            self._h = None
+
+    def clear(self):
+        self._lib.mla_page_table_clear(self._h)
+
+    def find_slot(self, seq_id, pos):
+        """Cache rows (int32 [n_tokens]) of the batch's tokens, or None when the batch does not fit (nothing is changed);
+        other errors raise."""
+        import numpy as np
+        seq_id = np.ascontiguousarray(seq_id, dtype=np.int32)
+        pos = np.ascontiguousarray(pos, dtype=np.int32)
+        rows = np.empty(len(seq_id), dtype=np.int32)
+        rc = self._lib.mla_page_table_find_slot(self._h, len(seq_id), seq_id.ctypes.data, pos.ctypes.data, rows.ctypes.data)
+        if rc == -1:
+            return None
+        if rc != 0:
+            raise ValueError("mla_page_table_find_slot: %d" % rc)
+        return rows
+
+    def seq_rm(self, seq_id, p0=-1, p1=-1):
+        return self._lib.mla_page_table_seq_rm(self._h, seq_id, p0, p1) == 0
+
+    def seq_cp(self, src, dst, p0=-1, p1=-1):
+        """Returns (src_row, dst_row, n_rows): the row run the caller copies on the device (n_rows may be 0)."""
+        a, b, n = C.c_int32(0), C.c_int32(0), C.c_int32(0)
+        rc = self._lib.mla_page_table_seq_cp(self._h, src, dst, p0, p1, C.byref(a), C.byref(b), C.byref(n))
+        if rc != 0:
+            raise ValueError("mla_page_table_seq_cp: %d" % rc)
+        return a.value, b.value, n.value
+
+    def seq_keep(self, seq_id):
+        return self._lib.mla_page_table_seq_keep(self._h, seq_id) == 0
+
+    def seq_len(self, seq_id):
+        return self._lib.mla_page_table_seq_len(self._h, seq_id)
+
+    @property
+    def free_pages(self):
+        return self._lib.mla_page_table_free_pages(self._h)
+
+    @property
+    def used_cells(self):
+        return self._lib.mla_page_table_used_cells(self._h)
+
+    def fill_inputs(self, seq_ids):
+        """(block_table int32 [n_seqs, max_blocks], seq_lens int32 [n_seqs]): src[4] / src[5] of the attention node."""
+        import numpy as np
+        seq_ids = np.ascontiguousarray(seq_ids, dtype=np.int32)
+        bt = np.empty((len(seq_ids), self.max_blocks), dtype=np.int32)
+        sl = np.empty(len(seq_ids), dtype=np.int32)
+        rc = self._lib.mla_page_table_fill_inputs(self._h, len(seq_ids), seq_ids.ctypes.data, bt.ctypes.data, sl.ctypes.data)
+        if rc != 0:
+            raise ValueError("mla_page_table_fill_inputs: %d" % rc)
+        return bt, sl

@@ -33,11 +33,11 @@ def _mirror_table():
 def test_library_exports_every_declared_symbol():
     lib = _lib()
     declared = set()
-    for hdr in ("mla_attn.h", "mla_kv_write.h", "ggml_mla_backend.h"):
+    for hdr in ("mla_attn.h", "mla_kv_write.h", "mla_page_table.h", "ggml_mla_backend.h"):
         src = open(os.path.join(ROOT, "include", hdr)).read()
         src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
         declared |= set(re.findall(r"\b(mla_\w+|ggml_backend_\w+)\s*\(", src))
-    declared -= {"mla_attn_args", "mla_attn_plan_info"}
+    declared -= {"mla_attn_args", "mla_attn_plan_info", "mla_page_table", "mla_kv_write_args"}
     assert {"mla_attn_launch", "mla_attn_workspace_size", "ggml_backend_init", "ggml_backend_score"} <= declared
     for sym in sorted(declared):
         assert hasattr(lib, sym), "library does not export %s" % sym
