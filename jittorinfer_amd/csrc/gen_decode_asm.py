@@ -300,41 +300,69 @@ def q8_dequant_items(raw_sreg, dst_sreg, tile_plus):
     return I
 
 
+PT = [241, 242, 243, 249, 250]   # 16-bit tiles: per-lane byte offsets of the 10 LDS-DMA slots, two 16-bit values per register
+DT = [251, 199]                  # address temporaries of the slots
+
+
+def dma_table_lines():
+    """Once per kernel: where the 16 bytes that lane l of LDS-DMA slot j copies sit inside a tile.  The LDS side of a slot
+    is 64 consecutive 16-byte chunks of the padded tile (73 chunks per row, the 73rd is padding); the global side is
+    row * nb1 + min(column chunk, 71) * 16 -- at most 31 * 1152 + 1136, so two offsets share a register.  The walk
+    over (row, column chunk) is done here and never again: per tile a slot costs two VALU instructions."""
+    L = []
+    row, col, x0, x1, x2 = T[0], T[1], T[2], T[3], T[4]
+    L.append("v_mov_b32 %s, %s" % (v(col), v(LANE)))
+    L.append("s_lshl_b32 %s, %s, 3" % (s(S2), s(WAVE)))
+    L.append("v_mov_b32 %s, %s" % (v(row), s(S2)))                     # a wave copies rows 8w .. 8w+7
+    for j in range(10):
+        L.append("v_min_u32 %s, 71, %s" % (v(x1), v(col)))
+        L.append("v_lshlrev_b32 %s, 4, %s" % (v(x1), v(x1)))
+        L.append("v_mad_u32_u24 %s, %s, %s, %s" % (v(x0), v(row), s(NB1), v(x1)))
+        if j % 2 == 0:
+            L.append("v_mov_b32 %s, %s" % (v(PT[j // 2]), v(x0)))
+        else:
+            L.append("v_lshl_or_b32 %s, %s, 16, %s" % (v(PT[j // 2]), v(x0), v(PT[j // 2])))
+        if j < 9:
+            # advance 64 chunks: col += 64; if (col >= 73) { col -= 73; row += 1 }
+            L.append("v_add_u32 %s, 64, %s" % (v(col), v(col)))
+            L.append("v_cmp_le_u32 vcc, %d, %s" % (CPR, v(col)))
+            L.append("v_subrev_u32 %s, %d, %s" % (v(x2), CPR, v(col)))
+            L.append("v_add_u32 %s, 1, %s" % (v(x0), v(row)))
+            L.append("s_nop 0")
+            L.append("v_cndmask_b32 %s, %s, %s, vcc" % (v(col), v(col), v(x2)))
+            L.append("v_cndmask_b32 %s, %s, %s, vcc" % (v(row), v(row), v(x0)))
+    return L
+
+
 def dma_tile_lines(tile_sreg, off_sreg):
     """Instruction list (to be interleaved) that issues the LDS-DMA loads of tile index s[tile_sreg] into the buffer
-    at LDS offset s[off_sreg].  Scalar part first (tile base address), then 10 slots."""
+    at LDS offset s[off_sreg].  Scalar part first (tile base address), then 10 slots whose per-lane offsets come from
+    the table of dma_table_lines.  Rows past the end of the sequence are replaced by the last 16 bytes of the last valid
+    row (any finite data will do: their probabilities are exactly 0): one v_min against that offset."""
     L = tile_base_lines(tile_sreg)
+    L.append("s_mul_i32 %s, %s, %s" % (s(S3), s(NVM1), s(NB1)))
+    L.append("s_add_u32 %s, %s, %d" % (s(S3), s(S3), 71 * 16))
     # LDS destination of this wave's first slot
     L.append("s_mul_i32 %s, %s, %d" % (s(DMAB), s(WAVE), WAVE_CHUNKS * 16))
     L.append("s_add_u32 %s, %s, %s" % (s(DMAB), s(DMAB), s(off_sreg)))
-    # per-lane chunk walk: local chunk cl = 64*j + lane -> (row_l, col); row = 8*wave + row_l
-    L.append("v_mov_b32 %s, %s" % (v(DCOL), v(LANE)))
-    L.append("s_lshl_b32 %s, %s, 3" % (s(S2), s(WAVE)))
-    L.append("v_mov_b32 %s, %s" % (v(DROW), s(S2)))
     for j in range(10):
-        L.append("v_min_u32 %s, %s, %s" % (v(X0), s(NVM1), v(DROW)))
-        L.append("v_min_u32 %s, 71, %s" % (v(X1), v(DCOL)))
-        L.append("v_lshlrev_b32 %s, 4, %s" % (v(X1), v(X1)))
-        L.append("v_mad_u32_u24 %s, %s, %s, %s" % (v(VOFF), v(X0), s(NB1), v(X1)))
+        t = DT[j & 1]
+        if j % 2 == 0:
+            L.append("v_and_b32 %s, 0xffff, %s" % (v(t), v(PT[j // 2])))
+        else:
+            L.append("v_lshrrev_b32 %s, 16, %s" % (v(t), v(PT[j // 2])))
+        L.append("v_min_u32 %s, %s, %s" % (v(t), s(S3), v(t)))
         if j == 9:
             # 8 chunks left per wave: lanes 0..7 only.  One atomic group: nothing may be scheduled inside the exec window.
             L.append("\\n\\t".join(["s_add_u32 m0, %s, %d" % (s(DMAB), j * 1024),
                                     "s_mov_b64 %s, exec" % s(EXS, 2),
                                     "s_mov_b64 exec, 0xff",
-                                    "global_load_lds_dwordx4 %s, %s" % (v(VOFF), s(TB, 2)),
+                                    "global_load_lds_dwordx4 %s, %s" % (v(t), s(TB, 2)),
                                     "s_mov_b64 exec, %s" % s(EXS, 2)]))
         else:
             L.append("\\n\\t".join(["s_add_u32 m0, %s, %d" % (s(DMAB), j * 1024),
                                     "s_nop 0",
-                                    "global_load_lds_dwordx4 %s, %s" % (v(VOFF), s(TB, 2))]))
-            # advance 64 chunks: col += 64; if (col >= 73) { col -= 73; row += 1 }
-            L.append("v_add_u32 %s, 64, %s" % (v(DCOL), v(DCOL)))
-            L.append("v_cmp_le_u32 vcc, %d, %s" % (CPR, v(DCOL)))
-            L.append("v_subrev_u32 %s, %d, %s" % (v(X2), CPR, v(DCOL)))
-            L.append("v_add_u32 %s, 1, %s" % (v(X0), v(DROW)))
-            L.append("s_nop 0")
-            L.append("v_cndmask_b32 %s, %s, %s, vcc" % (v(DCOL), v(DCOL), v(X2)))
-            L.append("v_cndmask_b32 %s, %s, %s, vcc" % (v(DROW), v(DROW), v(X0)))
+                                    "global_load_lds_dwordx4 %s, %s" % (v(t), s(TB, 2))]))
     return L
 
 
@@ -822,6 +850,9 @@ def main():
     e("s_mov_b32 %s, 0" % s(IT))
     for i in range(256):
         e("v_accvgpr_write_b32 %s, 0" % a(i))
+    if not Q8:
+        for ln in dma_table_lines():
+            e(ln)
     # page ids have arrived (loads return in order: only the Q and mask loads may still be in flight)
     e("s_waitcnt vmcnt(%d)" % n_early)
     e("v_max_i32 %s, 0, %s" % (v(PAGES), v(PAGES)))

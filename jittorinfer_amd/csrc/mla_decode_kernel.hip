@@ -284,6 +284,8 @@ bool decode_fast_applicable(const mla_attn_args * a) {
         if (!a->block_table && ((a->kv_nb3 & 15) || a->n_kv % TILE_TOK)) return false;
     }
     if (a->logit_softcap != 0.0f || a->max_bias > 0.0f) return false;
+    // 16-bit rows must be packed: the per-lane offsets of the tile copy are kept as 16-bit values (31 * 1152 + 1136 < 65536)
+    if (a->kv_type != MLA_TYPE_Q8_0 && a->kv_nb1 != ROW_BYTES) return false;
     if (a->mask) {
         // whole tiles only (no key past n_kv is touched in a mask row), 32-bit offsets into the mask, 8-byte aligned loads
         const int64_t n_kv = a->block_table ? a->bt_stride * MLA_PAGE_TOKENS : a->n_kv;
