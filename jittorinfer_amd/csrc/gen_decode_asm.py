@@ -169,8 +169,13 @@ def emit_item(x):
 
 
 # ---------------------------------------------------------------------------------------------------------------
-def tile_base_lines(tile_sreg):
-    """Scalar lines: s[TB:TB+1] = address of the first row of tile s[tile_sreg]; s[NVM1] = its valid rows - 1."""
+PGZ = 75   # prologue only (VMW's register): id of the split's first page, handed over as a scalar
+
+
+def tile_base_lines(tile_sreg, first_page_scalar=False):
+    """Scalar lines: s[TB:TB+1] = address of the first row of tile s[tile_sreg]; s[NVM1] = its valid rows - 1.
+    first_page_scalar: a tile inside the split's first page takes the page id from s[PGZ] instead of the lane of PAGES
+    (the prologue's tiles, issued while the vector load of the page ids may still be in flight)."""
     L = []
     # t0 = kv_begin + 32*tile ; nvalid-1 = min(32, kv_end - t0) - 1
     L.append("s_lshl_b32 %s, %s, 5" % (s(S0), s(tile_sreg)))
@@ -182,6 +187,9 @@ def tile_base_lines(tile_sreg):
     L.append("s_lshr_b32 %s, %s, 7" % (s(S1), s(S0)))                             # logical page
     L.append("s_sub_u32 %s, %s, %s" % (s(S1), s(S1), s(PG0)))                     # index into the preloaded lanes
     L.append("v_readlane_b32 %s, %s, %s" % (s(S2), v(PAGES), s(S1)))
+    if first_page_scalar:
+        L.append("s_cmp_eq_u32 %s, 0" % s(S1))
+        L.append("s_cselect_b32 %s, %s, %s" % (s(S2), s(PGZ), s(S2)))
     L.append("s_lshl_b32 %s, %s, 7" % (s(S2), s(S2)))
     L.append("s_and_b32 %s, %s, 127" % (s(S3), s(S0)))
     L.append("s_add_u32 %s, %s, %s" % (s(S2), s(S2), s(S3)))                      # pool row when paged
@@ -198,10 +206,10 @@ def tile_base_lines(tile_sreg):
 DQ_LOFF = 227   # lane * 16 for the flat raw-tile copy; as DQ_OUT + 3 the last register the dequantizer overwrites afterwards
 
 
-def q8_dma_lines(tile_sreg, raw_sreg):
+def q8_dma_lines(tile_sreg, raw_sreg, first_page_scalar=False):
     """Q8_0 builds: the 19584 bytes of tile s[tile_sreg] (32 packed rows, contiguous in the pool) -> the raw buffer at
     LDS offset s[raw_sreg], as a flat copy: 306 chunks per wave, 4 full LDS-DMA instructions and one of 50 lanes."""
-    L = tile_base_lines(tile_sreg)
+    L = tile_base_lines(tile_sreg, first_page_scalar)
     L.append("s_mul_i32 %s, %s, %d" % (s(DMAB), s(WAVE), Q8_WAVE_CHUNKS * 16))
     L.append("s_add_u32 %s, %s, %s" % (s(TB), s(TB), s(DMAB)))
     L.append("s_addc_u32 %s, %s, 0" % (s(TB + 1), s(TB + 1)))
@@ -334,12 +342,12 @@ def dma_table_lines():
     return L
 
 
-def dma_tile_lines(tile_sreg, off_sreg):
+def dma_tile_lines(tile_sreg, off_sreg, first_page_scalar=False):
     """Instruction list (to be interleaved) that issues the LDS-DMA loads of tile index s[tile_sreg] into the buffer
     at LDS offset s[off_sreg].  Scalar part first (tile base address), then 10 slots whose per-lane offsets come from
     the table of dma_table_lines.  Rows past the end of the sequence are replaced by the last 16 bytes of the last valid
     row (any finite data will do: their probabilities are exactly 0): one v_min against that offset."""
-    L = tile_base_lines(tile_sreg)
+    L = tile_base_lines(tile_sreg, first_page_scalar)
     L.append("s_mul_i32 %s, %s, %s" % (s(S3), s(NVM1), s(NB1)))
     L.append("s_add_u32 %s, %s, %d" % (s(S3), s(S3), 71 * 16))
     # LDS destination of this wave's first slot
@@ -761,6 +769,7 @@ def main():
     e("s_mov_b32 %s, %%[flg]" % s(FLG))
     e("s_mov_b32 %s, %%[ntl]" % s(NT))
     e("s_mov_b32 %s, %%[ostr]" % s(OSTR))
+    e("s_mov_b32 %s, %%[pg0]" % s(PGZ))
     e("s_mov_b64 %s, %%[qp]" % s(QP, 2))
     e("v_mov_b32 %s, %%[tid]" % v(X0))
     if DEBUG:
@@ -848,15 +857,30 @@ def main():
     e("s_mov_b32 %s, %d" % (s(OFF2), 2 * TILE_BYTES))
     e("s_mov_b32 %s, %d" % (s(OFF3), 3 * TILE_BYTES))
     e("s_mov_b32 %s, 0" % s(IT))
-    for i in range(256):
-        e("v_accvgpr_write_b32 %s, 0" % a(i))
     if not Q8:
         for ln in dma_table_lines():
             e(ln)
-    # page ids have arrived (loads return in order: only the Q and mask loads may still be in flight)
+    # The first tiles can be requested before the page ids are there when the split starts on a page boundary (always,
+    # except for masked key ranges): they lie in the first page, whose id came as a scalar.  Otherwise wait for the ids
+    # (loads return in order: only the Q and mask loads may still be in flight).
+    lab_al = label("aligned")
+    e("s_and_b32 %s, %s, 127" % (s(S0), s(KVB)))
+    e("s_cmp_eq_u32 %s, 0" % s(S0))
+    e("s_cbranch_scc1 %s" % lab_al)
     e("s_waitcnt vmcnt(%d)" % n_early)
     e("v_max_i32 %s, 0, %s" % (v(PAGES), v(PAGES)))
     e("v_min_i32 %s, %s, %s" % (v(PAGES), s(NPP), v(PAGES)))
+    e("%s:" % lab_al)
+
+    def acc_init():
+        for i in range(256):
+            e("v_accvgpr_write_b32 %s, 0" % a(i))
+
+    def page_clamp():
+        # (again for the path that already waited: harmless) page ids outside the pool can only come from table entries
+        # that are never used; clamped so that no address leaves the pool
+        e("v_max_i32 %s, 0, %s" % (v(PAGES), v(PAGES)))
+        e("v_min_i32 %s, %s, %s" % (v(PAGES), s(NPP), v(PAGES)))
     stamp(6)
     if Q8:
         # ------------------------------------------------------------------ Q8_0: per-lane offsets of the dequantizer
@@ -883,18 +907,20 @@ def main():
         # ------------------------------------------------------------------ raw tiles 0 and 1 -> LDS, tile 0 -> f16
         lab_w0, lab_wd = label("pw0"), label("pwd")
         e("s_mov_b32 %s, 0" % s(TMP))
-        for ln in q8_dma_lines(TMP, RAWC):
+        for ln in q8_dma_lines(TMP, RAWC, True):
             e(ln)
+        acc_init()
         e("s_cmp_lt_u32 %s, 2" % s(NT))
         e("s_cbranch_scc1 %s" % lab_w0)
         e("s_mov_b32 %s, 1" % s(TMP))
-        for ln in q8_dma_lines(TMP, RAWN):
+        for ln in q8_dma_lines(TMP, RAWN, True):
             e(ln)
         e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
         e("s_branch %s" % lab_wd)
         e("%s:" % lab_w0)
         e("s_waitcnt vmcnt(0)")
         e("%s:" % lab_wd)
+        page_clamp()
         e("s_barrier")
         for it_ in q8_dequant_items(RAWC, OFF0, 0):
             emit_item(it_)
@@ -905,7 +931,7 @@ def main():
         e("s_cmp_lt_u32 %s, 3" % s(NT))
         e("s_cbranch_scc1 %s" % lab_n2)
         e("s_mov_b32 %s, 2" % s(TMP))
-        for ln in q8_dma_lines(TMP, RAWC):
+        for ln in q8_dma_lines(TMP, RAWC, True):
             e(ln)
         e("%s:" % lab_n2)
         for it_ in q8_dequant_items(RAWN, OFF1, 1):
@@ -914,17 +940,18 @@ def main():
         # ------------------------------------------------------------------ tiles 0, 1, 2 -> LDS; go on as soon as Q and tile 0 are there
         lab_w0, lab_w1, lab_wd = label("pw0"), label("pw1"), label("pwd")
         e("s_mov_b32 %s, 0" % s(TMP))
-        for ln in dma_tile_lines(TMP, OFF0):
+        for ln in dma_tile_lines(TMP, OFF0, True):
             e(ln)
+        acc_init()
         e("s_cmp_lt_u32 %s, 2" % s(NT))
         e("s_cbranch_scc1 %s" % lab_w0)
         e("s_mov_b32 %s, 1" % s(TMP))
-        for ln in dma_tile_lines(TMP, OFF1):
+        for ln in dma_tile_lines(TMP, OFF1, True):
             e(ln)
         e("s_cmp_lt_u32 %s, 3" % s(NT))
         e("s_cbranch_scc1 %s" % lab_w1)
         e("s_mov_b32 %s, 2" % s(TMP))
-        for ln in dma_tile_lines(TMP, OFF2):
+        for ln in dma_tile_lines(TMP, OFF2, True):
             e(ln)
         e("s_waitcnt vmcnt(%d)" % (2 * DMA_PER_TILE))
         e("s_branch %s" % lab_wd)
@@ -934,6 +961,7 @@ def main():
         e("%s:" % lab_w0)
         e("s_waitcnt vmcnt(0)")
         e("%s:" % lab_wd)
+        page_clamp()
         e("s_barrier")
     stamp(1)
     if DEBUG:

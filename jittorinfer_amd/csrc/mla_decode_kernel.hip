@@ -65,7 +65,7 @@ constexpr int lds_total(int kvt) { return handoff_off(kvt) + NTHREADS * 32; }
 #define MLA_DECODE_INPUTS                                                                                          \
     [kv] "s"(kv_base), [bt] "s"(bt_row), [kvb] "s"(s_kvb), [kve] "s"(s_kve), [cl2] "s"(c_log2_bits), [npp] "s"(s_npp), \
     [nb1] "s"(s_nb1), [flg] "s"(s_flg), [ntl] "s"(s_ntl), [ostr] "s"(s_ostr), [qp] "s"(qpack), [msk] "s"(mask_base),  \
-    [scl] "s"(s_scale), [tid] "v"(tid)
+    [scl] "s"(s_scale), [pg0] "s"(s_pg0), [tid] "v"(tid)
 
 // The wave-level program is generated by gen_decode_asm.py (register map, LDS-DMA issue, MFMA/VALU interleave).
 // KVT = SRC_BF16: bf16 KV rows, bf16 MFMA, P fed as hi + lo halves.   SRC_F16: f16 KV rows, f16 MFMA, single P.
@@ -154,6 +154,10 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
     const int s_nb1  = __builtin_amdgcn_readfirstlane((int) p.kv_nb1);
     const int s_flg  = __builtin_amdgcn_readfirstlane((p.n_splits == 1 || p.part_f32 ? 1 : 0) | p.debug_flags);  // bit 0: f32 row store
     const int s_ntl  = __builtin_amdgcn_readfirstlane(n_tiles);
+    // id of the split's first page as a scalar: the first tiles are requested before the vector load of all page ids is back
+    int pg0 = 0;
+    if (bt_row) pg0 = min(max(bt_row[min((int64_t) (kv_begin >> 7), p.bt_stride - 1)], 0), p.n_pool_pages - 1);
+    const int s_pg0 = __builtin_amdgcn_readfirstlane(pg0);
     const char * mask_base = p.mask;
     const int s_scale = __builtin_amdgcn_readfirstlane(__float_as_int(p.scale));
     const int s_ostr = __builtin_amdgcn_readfirstlane(p.n_rows * 16);  // bytes between the partial rows of column groups c and c+1
