@@ -24,7 +24,7 @@ def _run(cmd):
 
 def build(verbose=False):
     objs = []
-    for src in ("mla_kernels.hip", "mla_decode_kernel.hip", "mla_kv_write.hip", "ggml_mla_backend.cpp", "mla_page_table.cpp"):
+    for src in ("mla_kernels.hip", "mla_decode_kernel.hip", "mla_kv_write.hip", "mla_front.hip", "ggml_mla_backend.cpp", "mla_page_table.cpp"):
         obj = os.path.join(CSRC, os.path.splitext(src)[0] + ".o")
         cmd = [HIPCC] + COMMON + (["-x", "hip"] if src == "ggml_mla_backend.cpp" else []) + ["-c", os.path.join(CSRC, src), "-o", obj]
         out = _run(cmd)

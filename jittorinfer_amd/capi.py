@@ -59,6 +59,9 @@ def library():
         lib.mla_hbm_copy_launch.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
         lib.mla_kv_write_launch.restype = C.c_int
         lib.mla_kv_write_launch.argtypes = [C.POINTER(MlaKvWriteArgs), C.c_void_p]
+        for name, cls in (("mla_rope_launch", MlaRopeArgs), ("mla_mul_mat_launch", MlaMulMatArgs), ("mla_copy_f32_launch", MlaCopyArgs)):
+            getattr(lib, name).restype = C.c_int
+            getattr(lib, name).argtypes = [C.POINTER(cls), C.c_void_p]
         lib.mla_page_table_create.restype = C.c_void_p
         lib.mla_page_table_create.argtypes = [C.c_int32] * 3
         lib.mla_page_table_free.argtypes = [C.c_void_p]
@@ -219,6 +222,120 @@ def kv_write(src, cache, kv_type, *, row0=None, rows=None, block_table=None, seq
     if rc != 0:
         raise RuntimeError("mla_kv_write_launch failed with code %d" % rc)
     return cache
+
+
+class MlaRopeArgs(C.Structure):
+    """mla_rope_args of include/mla_front.h."""
+    _fields_ = [("src", C.c_void_p), ("ne", C.c_int64 * 4), ("src_nb", C.c_int64 * 4), ("dst", C.c_void_p), ("dst_nb", C.c_int64 * 4),
+                ("pos", C.c_void_p), ("freq_factors", C.c_void_p), ("n_dims", C.c_int32), ("mode", C.c_int32),
+                ("n_ctx_orig", C.c_int32), ("freq_base", C.c_float), ("freq_scale", C.c_float), ("ext_factor", C.c_float),
+                ("attn_factor", C.c_float), ("beta_fast", C.c_float), ("beta_slow", C.c_float)]
+
+
+class MlaMulMatArgs(C.Structure):
+    """mla_mul_mat_args of include/mla_front.h."""
+    _fields_ = [("w_type", C.c_int32), ("_pad", C.c_int32), ("w", C.c_void_p), ("K", C.c_int64), ("N", C.c_int64),
+                ("w_ne2", C.c_int64), ("w_ne3", C.c_int64), ("w_nb1", C.c_int64), ("w_nb2", C.c_int64), ("w_nb3", C.c_int64),
+                ("x", C.c_void_p), ("M", C.c_int64), ("ne2", C.c_int64), ("ne3", C.c_int64), ("x_nb1", C.c_int64),
+                ("x_nb2", C.c_int64), ("x_nb3", C.c_int64), ("dst", C.c_void_p), ("d_nb1", C.c_int64), ("d_nb2", C.c_int64),
+                ("d_nb3", C.c_int64)]
+
+
+class MlaCopyArgs(C.Structure):
+    """mla_copy_args of include/mla_front.h."""
+    _fields_ = [("src", C.c_void_p), ("dst", C.c_void_p), ("ne", C.c_int64 * 4), ("src_nb", C.c_int64 * 4), ("dst_nb", C.c_int64 * 4)]
+
+
+def _gpu_only(t):
+    if not t.is_cuda:
+        raise RuntimeError("jittorinfer_amd runs on a gfx950 GPU only (there is no CPU path)")
+
+
+def _stream(t, stream):
+    import torch
+    return stream if stream is not None else torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _nb4(t):
+    """ggml-order byte strides / sizes of a torch tensor of up to 4 dims (last torch dim = ggml dim 0)."""
+    es = t.element_size()
+    ne = list(reversed(t.shape)) + [1] * (4 - t.dim())
+    nb = [s * es for s in reversed(t.stride())]
+    while len(nb) < 4:
+        nb.append(nb[-1] * ne[len(nb) - 1])
+    return ne, nb
+
+
+def ggml_rope_ext(x, pos, *, n_dims, mode=0, n_ctx_orig=0, freq_base=10000.0, freq_scale=1.0, ext_factor=0.0, attn_factor=1.0,
+                  beta_fast=32.0, beta_slow=1.0, freq_factors=None, out=None, stream=None):
+    """ggml_rope_ext (ggml/src/ggml.c:3495-3501) on the current torch stream.  x: float32 [n_tok, n_head, ne0] (ggml ne =
+    {ne0, n_head, n_tok}), unit stride in the last dimension; pos: int32 [n_tok]; out: same shape (default: a new
+    contiguous tensor; pass out=x to rotate in place)."""
+    import torch
+    _gpu_only(x)
+    assert x.dtype == torch.float32 and x.dim() == 3 and x.stride(2) == 1
+    assert pos.dtype == torch.int32 and pos.is_contiguous() and pos.numel() == x.shape[0]
+    if out is None:
+        out = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+    assert out.shape == x.shape and out.dtype == torch.float32 and out.stride(2) == 1
+    a = MlaRopeArgs()
+    ne, nb = _nb4(x)
+    _, dnb = _nb4(out)
+    a.src, a.dst, a.pos = x.data_ptr(), out.data_ptr(), pos.data_ptr()
+    a.ne[:], a.src_nb[:], a.dst_nb[:] = ne, nb, dnb
+    if freq_factors is not None:
+        assert freq_factors.dtype == torch.float32 and freq_factors.is_contiguous() and freq_factors.numel() >= n_dims // 2
+        a.freq_factors = freq_factors.data_ptr()
+    a.n_dims, a.mode, a.n_ctx_orig = n_dims, mode, n_ctx_orig
+    a.freq_base, a.freq_scale, a.ext_factor, a.attn_factor = freq_base, freq_scale, ext_factor, attn_factor
+    a.beta_fast, a.beta_slow = beta_fast, beta_slow
+    rc = library().mla_rope_launch(C.byref(a), C.c_void_p(_stream(x, stream)))
+    if rc != 0:
+        raise RuntimeError("mla_rope_launch failed with code %d" % rc)
+    return out
+
+
+def ggml_mul_mat(w, w_type, x, *, out=None, stream=None):
+    """ggml_mul_mat(src0 = w, src1 = x) for the absorb products (src/llama-graph-attn.cpp:264-275, :303-317).
+    w: [w_ne2, N, K] 16-bit storage (bf16 / f16 bits, any 2-byte dtype), x: float32 [ne2, M, K], unit stride in the
+    last dimension of both, ne2 % w_ne2 == 0; returns float32 [ne2, M, N]."""
+    import torch
+    _gpu_only(x)
+    assert w.dim() == 3 and x.dim() == 3 and w.element_size() == 2 and x.dtype == torch.float32
+    assert w.stride(2) == 1 and x.stride(2) == 1 and w.shape[2] == x.shape[2]
+    if out is None:
+        out = torch.empty((x.shape[0], x.shape[1], w.shape[1]), dtype=torch.float32, device=x.device)
+    assert out.shape == (x.shape[0], x.shape[1], w.shape[1]) and out.dtype == torch.float32 and out.stride(2) == 1
+    a = MlaMulMatArgs()
+    a.w_type, a.w, a.x, a.dst = w_type, w.data_ptr(), x.data_ptr(), out.data_ptr()
+    a.K, a.N, a.w_ne2, a.w_ne3 = w.shape[2], w.shape[1], w.shape[0], 1
+    a.M, a.ne2, a.ne3 = x.shape[1], x.shape[0], 1
+    a.w_nb1, a.w_nb2 = w.stride(1) * 2, w.stride(0) * 2
+    a.x_nb1, a.x_nb2 = x.stride(1) * 4, x.stride(0) * 4
+    a.d_nb1, a.d_nb2 = out.stride(1) * 4, out.stride(0) * 4
+    a.w_nb3, a.x_nb3, a.d_nb3 = a.w_nb2 * a.w_ne2, a.x_nb2 * a.ne2, a.d_nb2 * a.ne2
+    rc = library().mla_mul_mat_launch(C.byref(a), C.c_void_p(_stream(x, stream)))
+    if rc != 0:
+        raise RuntimeError("mla_mul_mat_launch failed with code %d" % rc)
+    return out
+
+
+def copy_f32(src, dst, stream=None):
+    """Strided float32 copy (ggml_cont; each half of ggml_concat): dst[...] = src[...], same shape, any strides with a
+    unit last one."""
+    import torch
+    _gpu_only(src)
+    assert src.dtype == torch.float32 and dst.dtype == torch.float32 and src.shape == dst.shape and src.dim() <= 4
+    assert src.stride(-1) == 1 and dst.stride(-1) == 1
+    a = MlaCopyArgs()
+    ne, nb = _nb4(src)
+    _, dnb = _nb4(dst)
+    a.src, a.dst = src.data_ptr(), dst.data_ptr()
+    a.ne[:], a.src_nb[:], a.dst_nb[:] = ne, nb, dnb
+    rc = library().mla_copy_f32_launch(C.byref(a), C.c_void_p(_stream(src, stream)))
+    if rc != 0:
+        raise RuntimeError("mla_copy_f32_launch failed with code %d" % rc)
+    return dst
 
 
 class PageTable:

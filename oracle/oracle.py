@@ -301,3 +301,166 @@ def ref_backend_kv_cpy(so_path, kv_cur, cache, kv_type, kv_head):
     if rc != 0:
         raise RuntimeError("ref_backend_kv_cpy failed: %d (%s)" % (rc, info.value.decode()))
     return cache, info.value.decode()
+
+
+# ------------------------------------------------------------------ the nodes either side of the attention node
+
+class RopeParams(C.Structure):
+    """ggml_rope_ext's scalar arguments (ggml/src/ggml.c:3413-3449); mode 0 = adjacent pairs, 2 = NeoX halves."""
+    _fields_ = [("n_dims", C.c_int32), ("mode", C.c_int32), ("n_ctx_orig", C.c_int32), ("freq_base", C.c_float),
+                ("freq_scale", C.c_float), ("ext_factor", C.c_float), ("attn_factor", C.c_float), ("beta_fast", C.c_float),
+                ("beta_slow", C.c_float)]
+
+
+def rope_params(n_dims=64, mode=0, n_ctx_orig=4096, freq_base=10000.0, freq_scale=1.0, ext_factor=0.0, attn_factor=1.0,
+                beta_fast=32.0, beta_slow=1.0):
+    return RopeParams(n_dims, mode, n_ctx_orig, freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow)
+
+
+def _front():
+    l = lib()
+    if not hasattr(l, "_front_ready"):
+        l.mla_oracle_rope.restype = C.c_int
+        l.mla_oracle_rope.argtypes = [C.c_void_p, C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.c_void_p, C.POINTER(C.c_int64),
+                                      C.c_void_p, C.c_void_p, C.POINTER(RopeParams)]
+        l.mla_oracle_mul_mat.restype = C.c_int
+        l.mla_oracle_mul_mat.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.c_void_p,
+                                         C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.c_void_p, C.c_void_p]
+        l.mla_oracle_rope_corr_dims.restype = None
+        l.mla_oracle_rope_corr_dims.argtypes = [C.c_int, C.c_int, C.c_float, C.c_float, C.c_float, C.POINTER(C.c_float)]
+        l._front_ready = True
+    return l
+
+
+def _i64x4(v):
+    return (C.c_int64 * 4)(*[int(x) for x in v])
+
+
+def rope(x, pos, p, freq_factors=None):
+    """GGML_OP_ROPE as ggml-cpu computes it.  x float32 [n_tok, n_head, ne0] (ggml ne = {ne0, n_head, n_tok}), any
+    strides with a unit last one; pos int32 [n_tok]; returns a contiguous array of the same shape."""
+    assert x.dtype == np.float32 and x.ndim == 3 and x.strides[2] == 4
+    pos = np.ascontiguousarray(pos, dtype=np.int32)
+    out = np.empty(x.shape, dtype=np.float32)
+    ff = None if freq_factors is None else np.ascontiguousarray(freq_factors, dtype=np.float32)
+    ne = _i64x4([x.shape[2], x.shape[1], x.shape[0], 1])
+    nb = _i64x4([4, x.strides[1], x.strides[0], 0])
+    dnb = _i64x4([4, out.strides[1], out.strides[0], 0])
+    rc = _front().mla_oracle_rope(x.ctypes.data, ne, nb, out.ctypes.data, dnb, pos.ctypes.data,
+                                  None if ff is None else ff.ctypes.data, C.byref(p))
+    if rc != 0:
+        raise RuntimeError("mla_oracle_rope failed: %d" % rc)
+    return out
+
+
+def rope_corr_dims(p):
+    d = (C.c_float * 2)()
+    _front().mla_oracle_rope_corr_dims(p.n_dims, p.n_ctx_orig, p.freq_base, p.beta_fast, p.beta_slow, d)
+    return float(d[0]), float(d[1])
+
+
+def mul_mat(a, a_type, b, with_abs=False):
+    """GGML_OP_MUL_MAT: a = src0 [ne02, N, K] (uint16 bits for F16/BF16, float32 for F32), b = src1 float32 [ne12, M, K],
+    any strides with a unit last one; out float32 [ne12, M, N] (ne12 % ne02 == 0, src0 broadcast over the quotient)."""
+    assert a.ndim == 3 and b.ndim == 3 and b.dtype == np.float32 and a.strides[2] == a.itemsize and b.strides[2] == 4
+    ne0 = _i64x4([a.shape[2], a.shape[1], a.shape[0], 1])
+    nb0 = _i64x4([a.itemsize, a.strides[1], a.strides[0], 0])
+    ne1 = _i64x4([b.shape[2], b.shape[1], b.shape[0], 1])
+    nb1 = _i64x4([4, b.strides[1], b.strides[0], 0])
+    out = np.empty((b.shape[0], b.shape[1], a.shape[1]), dtype=np.float32)
+    ab = np.empty_like(out) if with_abs else None
+    rc = _front().mla_oracle_mul_mat(a.ctypes.data, a_type, ne0, nb0, b.ctypes.data, ne1, nb1, out.ctypes.data,
+                                     None if ab is None else ab.ctypes.data)
+    if rc != 0:
+        raise RuntimeError("mla_oracle_mul_mat failed: %d" % rc)
+    return (out, ab) if with_abs else out
+
+
+def mla_q_states(q, wkv_b, w_type, pos, p, n_head):
+    """The query side of llm_attn_mla (src/llama-graph-attn.cpp:264-277 after the rope of
+    src/llama-graph-deepseek2.cpp:216-222) from the oracle's own pieces: q float32 [n_tok, n_head*192], wkv_b
+    [n_head*256, 512] in w_type; returns q_states float32 [n_head, n_tok, 576]."""
+    n_tok = q.shape[0]
+    q3 = q.reshape(n_tok, n_head, 192)
+    q_pe = rope(np.ascontiguousarray(q3[:, :, 128:]), pos, p)                    # [n_tok, H, 64]
+    wk_b = wkv_b.reshape(-1)[:n_head * 512 * 128].reshape(n_head, 512, 128)       # ggml ne = {128, 512, H}
+    q_abs = mul_mat(wk_b, w_type, q3[:, :, :128].transpose(1, 0, 2))              # [H, n_tok, 512]
+    return np.concatenate([q_abs, q_pe.transpose(1, 0, 2)], axis=2)
+
+
+def mla_unabsorb(kqv, wkv_b, w_type, n_head):
+    """The output side (src/llama-graph-attn.cpp:303-323): kqv float32 [n_head, n_tok, 512] -> float32 [n_tok, n_head*128]."""
+    n_tok = kqv.shape[1]
+    wv_b = wkv_b.reshape(-1)[n_head * 512 * 128:].reshape(n_head, 128, 512)       # ggml ne = {512, 128, H}
+    o = mul_mat(wv_b, w_type, kqv)                                                # [H, n_tok, 128]
+    return np.ascontiguousarray(o.transpose(1, 0, 2)).reshape(n_tok, n_head * 128)
+
+
+def _ref_front():
+    r = ref()
+    if not hasattr(r, "_front_ready"):
+        r.ref_rope.restype = C.c_int
+        r.ref_rope.argtypes = [C.c_char_p, C.c_int64, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p,
+                               C.POINTER(RopeParams), C.c_void_p, C.c_int]
+        r.ref_mul_mat.restype = C.c_int
+        r.ref_mul_mat.argtypes = [C.c_char_p, C.c_int] + [C.c_int64] * 5 + [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]
+        r.ref_mla_q_states.restype = C.c_int
+        r.ref_mla_q_states.argtypes = [C.c_char_p, C.c_int, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p,
+                                       C.POINTER(RopeParams), C.c_void_p, C.c_int]
+        r.ref_mla_unabsorb.restype = C.c_int
+        r.ref_mla_unabsorb.argtypes = [C.c_char_p, C.c_int, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]
+        r._front_ready = True
+    return r
+
+
+def _so(so_path):
+    return None if so_path is None else so_path.encode()
+
+
+def ref_rope(x, pos, p, freq_factors=None, so_path=None, n_threads=4):
+    """One ROPE node on the reference's ggml-cpu (so_path None) or on the backend plugin loaded from so_path."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    pos = np.ascontiguousarray(pos, dtype=np.int32)
+    ff = None if freq_factors is None else np.ascontiguousarray(freq_factors, dtype=np.float32)
+    out = np.full(x.shape, np.nan, dtype=np.float32)
+    rc = _ref_front().ref_rope(_so(so_path), x.shape[2], x.shape[1], x.shape[0], x.ctypes.data, pos.ctypes.data,
+                               None if ff is None else ff.ctypes.data, C.byref(p), out.ctypes.data, n_threads)
+    if rc != 0:
+        raise RuntimeError("ref_rope failed: %d" % rc)
+    return out
+
+
+def ref_mul_mat(a, a_type, b, so_path=None, n_threads=4):
+    a = np.ascontiguousarray(a)
+    b = np.ascontiguousarray(b, dtype=np.float32)
+    out = np.full((b.shape[0], b.shape[1], a.shape[1]), np.nan, dtype=np.float32)
+    rc = _ref_front().ref_mul_mat(_so(so_path), a_type, a.shape[2], a.shape[1], a.shape[0], b.shape[1], b.shape[0],
+                                  a.ctypes.data, b.ctypes.data, out.ctypes.data, n_threads)
+    if rc != 0:
+        raise RuntimeError("ref_mul_mat failed: %d" % rc)
+    return out
+
+
+def ref_mla_q_states(q, wkv_b, w_type, pos, p, n_head, so_path=None, n_threads=4):
+    q = np.ascontiguousarray(q, dtype=np.float32)
+    wkv_b = np.ascontiguousarray(wkv_b)
+    pos = np.ascontiguousarray(pos, dtype=np.int32)
+    n_tok = q.shape[0]
+    out = np.full((n_head, n_tok, 576), np.nan, dtype=np.float32)
+    rc = _ref_front().ref_mla_q_states(_so(so_path), w_type, n_head, n_tok, q.ctypes.data, wkv_b.ctypes.data, pos.ctypes.data,
+                                       C.byref(p), out.ctypes.data, n_threads)
+    if rc != 0:
+        raise RuntimeError("ref_mla_q_states failed: %d" % rc)
+    return out
+
+
+def ref_mla_unabsorb(kqv, wkv_b, w_type, n_head, so_path=None, n_threads=4):
+    kqv = np.ascontiguousarray(kqv, dtype=np.float32)
+    wkv_b = np.ascontiguousarray(wkv_b)
+    n_tok = kqv.shape[1]
+    out = np.full((n_tok, n_head * 128), np.nan, dtype=np.float32)
+    rc = _ref_front().ref_mla_unabsorb(_so(so_path), w_type, n_head, n_tok, kqv.ctypes.data, wkv_b.ctypes.data, out.ctypes.data,
+                                       n_threads)
+    if rc != 0:
+        raise RuntimeError("ref_mla_unabsorb failed: %d" % rc)
+    return out

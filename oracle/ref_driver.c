@@ -9,6 +9,9 @@
  *                                 way the reference's scheduler would drive a drop-in backend
  *   ref_quantize_q8_0_ref / _cpu  the two Q8_0 quantizers (ggml-quants.c:202-226, ggml-cpu-quants.c:767-900)
  *   ref_f32_to_f16_row / bf16     the reference's conversions
+ *   ref_rope / ref_mul_mat        one ROPE / MUL_MAT node on ggml-cpu, or on a loaded backend
+ *   ref_mla_q_states / _unabsorb  the query side and the output side of llm_attn_mla around the attention node
+ *                                 (src/llama-graph-attn.cpp:264-277, :303-323), on ggml-cpu or on a loaded backend
  *   ref_abi_table                 sizeof/offsetof/enum facts of the structs a backend must mirror
  */
 #include <stddef.h>
@@ -259,6 +262,174 @@ int ref_backend_kv_cpy(const char * so_path, int k_type, int64_t n_cache, int64_
     return rc;
 }
 
+/* ------------------------------------------------------------------ the nodes either side of the attention node
+ * One code path for both executors: `so_path` == NULL runs the graph on the reference's ggml-cpu backend, otherwise on
+ * the backend loaded from that file; tensors live in the executor's buffer. */
+struct front_rt {
+    ggml_backend_t        be;
+    struct ggml_context * ctx;
+    struct ggml_cgraph *  gf;
+    ggml_backend_buffer_t buf;
+};
+
+static int front_open(struct front_rt * rt, const char * so_path, int n_threads) {
+    memset(rt, 0, sizeof(*rt));
+    if (so_path) {
+        ggml_backend_reg_t reg = ggml_backend_load(so_path);
+        if (!reg) return -10;
+        if (ggml_backend_reg_dev_count(reg) < 1) return -11;
+        rt->be = ggml_backend_dev_init(ggml_backend_reg_dev_get(reg, 0), NULL);
+    } else {
+        rt->be = ggml_backend_cpu_init();
+        if (rt->be) ggml_backend_cpu_set_n_threads(rt->be, n_threads);
+    }
+    if (!rt->be) return -12;
+    struct ggml_init_params ip = { ggml_tensor_overhead() * 64 + ggml_graph_overhead(), NULL, true };
+    rt->ctx = ggml_init(ip);
+    rt->gf  = ggml_new_graph(rt->ctx);
+    return 0;
+}
+/* allocate every tensor of the context, check that the executor takes every node */
+static int front_alloc(struct front_rt * rt) {
+    rt->buf = ggml_backend_alloc_ctx_tensors(rt->ctx, rt->be);
+    if (!rt->buf) return -13;
+    for (int i = 0; i < ggml_graph_n_nodes(rt->gf); i++)
+        if (!ggml_backend_supports_op(rt->be, ggml_graph_node(rt->gf, i))) return -100 - i;
+    return 0;
+}
+static int front_run(struct front_rt * rt) {
+    enum ggml_status st = ggml_backend_graph_compute(rt->be, rt->gf);
+    return st == GGML_STATUS_SUCCESS ? 0 : ((int) st ? (int) st : -15);
+}
+static void front_close(struct front_rt * rt) {
+    if (rt->buf) ggml_backend_buffer_free(rt->buf);
+    if (rt->ctx) ggml_free(rt->ctx);
+    if (rt->be) ggml_backend_free(rt->be);
+}
+
+struct ref_rope_params {
+    int32_t n_dims, mode, n_ctx_orig;
+    float   freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow;
+};
+
+/* ggml_rope_ext (ggml.c:3495-3501) of x = f32 [ne0, ne1, ne2] with pos[ne2] and optional freq_factors[n_dims/2] */
+int ref_rope(const char * so_path, int64_t ne0, int64_t ne1, int64_t ne2, const float * x, const int32_t * pos,
+             const float * freq_factors, const struct ref_rope_params * p, float * out, int n_threads) {
+    struct front_rt rt;
+    int rc = front_open(&rt, so_path, n_threads);
+    if (rc) return rc;
+    struct ggml_tensor * tx = ggml_new_tensor_3d(rt.ctx, GGML_TYPE_F32, ne0, ne1, ne2);
+    struct ggml_tensor * tp = ggml_new_tensor_1d(rt.ctx, GGML_TYPE_I32, ne2);
+    struct ggml_tensor * tf = freq_factors ? ggml_new_tensor_1d(rt.ctx, GGML_TYPE_F32, p->n_dims / 2) : NULL;
+    struct ggml_tensor * o  = ggml_rope_ext(rt.ctx, tx, tp, tf, p->n_dims, p->mode, p->n_ctx_orig, p->freq_base, p->freq_scale,
+                                            p->ext_factor, p->attn_factor, p->beta_fast, p->beta_slow);
+    ggml_build_forward_expand(rt.gf, o);
+    rc = front_alloc(&rt);
+    if (!rc) {
+        ggml_backend_tensor_set(tx, x, 0, ggml_nbytes(tx));
+        ggml_backend_tensor_set(tp, pos, 0, ggml_nbytes(tp));
+        if (tf) ggml_backend_tensor_set(tf, freq_factors, 0, ggml_nbytes(tf));
+        rc = front_run(&rt);
+        if (!rc) ggml_backend_tensor_get(o, out, 0, ggml_nbytes(o));
+    }
+    front_close(&rt);
+    return rc;
+}
+
+/* ggml_mul_mat of a contiguous src0 = type0 [K, N, ne02] and a contiguous f32 src1 = [K, M, ne12]; out f32 [N, M, ne12] */
+int ref_mul_mat(const char * so_path, int type0, int64_t K, int64_t N, int64_t ne02, int64_t M, int64_t ne12,
+                const void * a, const float * b, float * out, int n_threads) {
+    struct front_rt rt;
+    int rc = front_open(&rt, so_path, n_threads);
+    if (rc) return rc;
+    struct ggml_tensor * ta = ggml_new_tensor_3d(rt.ctx, (enum ggml_type) type0, K, N, ne02);
+    struct ggml_tensor * tb = ggml_new_tensor_3d(rt.ctx, GGML_TYPE_F32, K, M, ne12);
+    struct ggml_tensor * o  = ggml_mul_mat(rt.ctx, ta, tb);
+    ggml_build_forward_expand(rt.gf, o);
+    rc = front_alloc(&rt);
+    if (!rc) {
+        ggml_backend_tensor_set(ta, a, 0, ggml_nbytes(ta));
+        ggml_backend_tensor_set(tb, b, 0, ggml_nbytes(tb));
+        rc = front_run(&rt);
+        if (!rc) ggml_backend_tensor_get(o, out, 0, ggml_nbytes(o));
+    }
+    front_close(&rt);
+    return rc;
+}
+
+/*
+ * The query side of llm_attn_mla as the reference's graph builds it (src/llama-graph-deepseek2.cpp:183-194, :216-222,
+ * src/llama-graph-attn.cpp:264-277): q = f32 [192*H, n_tok]; q_nope / q_pe strided views; q_pe -> cont -> rope;
+ * q_nope permuted -> mul_mat with wk_b (view of wkv_b: [128, 512, H]); concat with the permuted q_pe along dim 0.
+ * out = q_states f32 [576, n_tok, H].  wkv_b = w_type [512, H*(128+128)] as the model stores it.
+ */
+int ref_mla_q_states(const char * so_path, int w_type, int64_t H, int64_t n_tok, const float * q, const void * wkv_b,
+                     const int32_t * pos, const struct ref_rope_params * p, float * out, int n_threads) {
+    const int64_t NOPE = 128, ROPE = 64, LORA = 512, DV = 128;
+    const enum ggml_type wt = (enum ggml_type) w_type;
+    struct front_rt rt;
+    int rc = front_open(&rt, so_path, n_threads);
+    if (rc) return rc;
+    struct ggml_context * c = rt.ctx;
+    struct ggml_tensor * tq = ggml_new_tensor_2d(c, GGML_TYPE_F32, (NOPE + ROPE) * H, n_tok);
+    struct ggml_tensor * tw = ggml_new_tensor_2d(c, wt, LORA, H * (NOPE + DV));
+    struct ggml_tensor * tp = ggml_new_tensor_1d(c, GGML_TYPE_I32, n_tok);
+    struct ggml_tensor * q_nope = ggml_view_3d(c, tq, NOPE, H, n_tok, ggml_row_size(tq->type, NOPE + ROPE),
+                                               ggml_row_size(tq->type, (NOPE + ROPE) * H), 0);
+    struct ggml_tensor * q_pe = ggml_view_3d(c, tq, ROPE, H, n_tok, ggml_row_size(tq->type, NOPE + ROPE),
+                                             ggml_row_size(tq->type, (NOPE + ROPE) * H), ggml_row_size(tq->type, NOPE));
+    q_pe = ggml_cont(c, q_pe);
+    q_pe = ggml_rope_ext(c, q_pe, tp, NULL, p->n_dims, p->mode, p->n_ctx_orig, p->freq_base, p->freq_scale, p->ext_factor,
+                         p->attn_factor, p->beta_fast, p->beta_slow);
+    struct ggml_tensor * wk_b = ggml_view_3d(c, tw, NOPE, LORA, H, ggml_row_size(wt, NOPE), ggml_row_size(wt, NOPE * LORA), 0);
+    q_nope = ggml_permute(c, q_nope, 0, 2, 1, 3);
+    q_nope = ggml_mul_mat(c, wk_b, q_nope);
+    q_pe   = ggml_permute(c, q_pe, 0, 2, 1, 3);
+    struct ggml_tensor * o = ggml_concat(c, q_nope, q_pe, 0);
+    ggml_build_forward_expand(rt.gf, o);
+    rc = front_alloc(&rt);
+    if (!rc) {
+        ggml_backend_tensor_set(tq, q, 0, ggml_nbytes(tq));
+        ggml_backend_tensor_set(tw, wkv_b, 0, ggml_nbytes(tw));
+        ggml_backend_tensor_set(tp, pos, 0, ggml_nbytes(tp));
+        rc = front_run(&rt);
+        if (!rc) ggml_backend_tensor_get(o, out, 0, ggml_nbytes(o));
+    }
+    front_close(&rt);
+    return rc;
+}
+
+/*
+ * The output side (src/llama-graph-attn.cpp:303-323): kqv = f32 [512, n_tok, H] (the attention result per head),
+ * wv_b = view of wkv_b [512, 128, H] behind the wk_b part; mul_mat, permute(0,2,1,3), cont_2d -> out f32 [128*H, n_tok].
+ */
+int ref_mla_unabsorb(const char * so_path, int w_type, int64_t H, int64_t n_tok, const float * kqv, const void * wkv_b,
+                     float * out, int n_threads) {
+    const int64_t NOPE = 128, LORA = 512, DV = 128;
+    const enum ggml_type wt = (enum ggml_type) w_type;
+    struct front_rt rt;
+    int rc = front_open(&rt, so_path, n_threads);
+    if (rc) return rc;
+    struct ggml_context * c = rt.ctx;
+    struct ggml_tensor * tk = ggml_new_tensor_3d(c, GGML_TYPE_F32, LORA, n_tok, H);
+    struct ggml_tensor * tw = ggml_new_tensor_2d(c, wt, LORA, H * (NOPE + DV));
+    struct ggml_tensor * wv_b = ggml_view_3d(c, tw, LORA, DV, H, ggml_row_size(wt, LORA), ggml_row_size(wt, LORA * DV),
+                                             ggml_row_size(wt, LORA * NOPE * H));
+    struct ggml_tensor * o = ggml_mul_mat(c, wv_b, tk);
+    o = ggml_permute(c, o, 0, 2, 1, 3);
+    o = ggml_cont_2d(c, o, DV * H, n_tok);
+    ggml_build_forward_expand(rt.gf, o);
+    rc = front_alloc(&rt);
+    if (!rc) {
+        ggml_backend_tensor_set(tk, kqv, 0, ggml_nbytes(tk));
+        ggml_backend_tensor_set(tw, wkv_b, 0, ggml_nbytes(tw));
+        rc = front_run(&rt);
+        if (!rc) ggml_backend_tensor_get(o, out, 0, ggml_nbytes(o));
+    }
+    front_close(&rt);
+    return rc;
+}
+
 void ref_quantize_q8_0_ref(const float * x, void * y, int64_t k) { quantize_row_q8_0_ref(x, (block_q8_0 *) y, k); }
 void ref_quantize_q8_0_cpu(const float * x, void * y, int64_t k) { quantize_row_q8_0(x, y, k); }
 void ref_dequantize_q8_0(const void * x, float * y, int64_t k) { dequantize_row_q8_0((const block_q8_0 *) x, y, k); }
@@ -327,7 +498,8 @@ static const struct ref_abi_entry abi_table[] = {
     E("GGML_OP_NONE", GGML_OP_NONE), E("GGML_OP_CPY", GGML_OP_CPY), E("GGML_OP_CONT", GGML_OP_CONT),
     E("GGML_OP_RESHAPE", GGML_OP_RESHAPE), E("GGML_OP_VIEW", GGML_OP_VIEW), E("GGML_OP_PERMUTE", GGML_OP_PERMUTE),
     E("GGML_OP_TRANSPOSE", GGML_OP_TRANSPOSE), E("GGML_OP_FLASH_ATTN_EXT", GGML_OP_FLASH_ATTN_EXT),
-    E("GGML_OP_SCATTER_UPDATE", GGML_OP_SCATTER_UPDATE), E("GGML_OP_COUNT", GGML_OP_COUNT),
+    E("GGML_OP_SCATTER_UPDATE", GGML_OP_SCATTER_UPDATE),
+    E("GGML_OP_ROPE", GGML_OP_ROPE), E("GGML_OP_MUL_MAT", GGML_OP_MUL_MAT), E("GGML_OP_CONCAT", GGML_OP_CONCAT), E("GGML_OP_COUNT", GGML_OP_COUNT),
     E("GGML_STATUS_ALLOC_FAILED", GGML_STATUS_ALLOC_FAILED), E("GGML_STATUS_FAILED", GGML_STATUS_FAILED),
     E("GGML_STATUS_SUCCESS", GGML_STATUS_SUCCESS), E("GGML_STATUS_ABORTED", GGML_STATUS_ABORTED),
     E("GGML_BACKEND_DEVICE_TYPE_CPU", GGML_BACKEND_DEVICE_TYPE_CPU), E("GGML_BACKEND_DEVICE_TYPE_GPU", GGML_BACKEND_DEVICE_TYPE_GPU),
