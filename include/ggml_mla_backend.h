@@ -26,6 +26,17 @@
  *   GGML_OP_SCATTER_UPDATE  src[0] cache BF16 | F16 | Q8_0 [576, n_rows], src[1] I32 | I64 [n_tok] row indices,
  *                           src[2] updates [576, n_tok] of the cache type (copied) or F32 (converted)
  *                           (ggml_scatter_update, ggml/src/ggml.c:3203-3223; src/llama-graph-attn.cpp:380-383)
+ * The nodes either side of it in llm_attn_mla and the DeepSeek-V2 graph (kernels behind include/mla_front.h):
+ *   GGML_OP_CONT            src[0] F32 with dense rows (any other strides) -> contiguous F32 dst with as many elements
+ *                           (ggml_cont of the q_pe / k_pe views, src/llama-graph-deepseek2.cpp:216-226; ggml_cont_2d of
+ *                           the permuted result, src/llama-graph-attn.cpp:322)
+ *   GGML_OP_ROPE            src[0] F32 [ne0, heads, n_tok, *], src[1] I32 [n_tok] positions, src[2] optional F32 frequency
+ *                           factors; op_params of ggml_rope_ext (ggml/src/ggml.c:3413-3449), mode 0 or 2
+ *   GGML_OP_MUL_MAT         src[0] F16 | BF16 [K, N, h, *] (K % 16 == 0, rows 16-byte aligned), src[1] F32 [K, M, H, *],
+ *                           dst F32 [N, M, H, *]: the absorb products q_nope x wk_b and wv_b x kqv
+ *                           (src/llama-graph-attn.cpp:264-275, :303-317)
+ *   GGML_OP_CONCAT          F32 operands with dense rows along any dimension (q_states = concat(q_nope_absorbed, q_pe),
+ *                           src/llama-graph-attn.cpp:277; kv_states, src/llama-graph-deepseek2.cpp:235)
  * Every other op except the no-op view ops (NONE, RESHAPE, VIEW, PERMUTE, TRANSPOSE) is reported unsupported, so
  * the reference's scheduler keeps it on another backend (ggml/src/ggml-backend.cpp:820-846).
  */

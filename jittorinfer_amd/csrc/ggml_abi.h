@@ -33,8 +33,8 @@ enum type : int {
 
 // only the ordinals the backend acts on; the fork appended 13 ops after upstream's list, so COUNT is 94
 enum op : int {
-    OP_NONE = 0, OP_CPY = 31, OP_CONT = 32, OP_RESHAPE = 33, OP_VIEW = 34, OP_PERMUTE = 35, OP_TRANSPOSE = 36,
-    OP_FLASH_ATTN_EXT = 61, OP_SCATTER_UPDATE = 92, OP_COUNT = 94,
+    OP_NONE = 0, OP_CONCAT = 20, OP_MUL_MAT = 26, OP_CPY = 31, OP_CONT = 32, OP_RESHAPE = 33, OP_VIEW = 34, OP_PERMUTE = 35, OP_TRANSPOSE = 36,
+    OP_ROPE = 44, OP_FLASH_ATTN_EXT = 61, OP_SCATTER_UPDATE = 92, OP_COUNT = 94,
 };
 
 enum prec : int { PREC_DEFAULT = 0, PREC_F32 = 1 };

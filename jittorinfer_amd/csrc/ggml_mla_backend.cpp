@@ -25,6 +25,7 @@
 #include <vector>
 
 #include "../../include/ggml_mla_backend.h"
+#include "../../include/mla_front.h"
 #include "../../include/mla_kv_write.h"
 #include "../../include/mla_attn.h"
 #include "ggml_abi.h"
@@ -274,11 +275,67 @@ bool kv_scatter_ok(const tensor * op, const char ** why) {
     return true;
 }
 
+// The nodes llm_attn_mla and the DeepSeek-V2 graph put either side of the attention node
+// (src/llama-graph-deepseek2.cpp:216-233, src/llama-graph-attn.cpp:264-277, :303-323): CONT and CONCAT of f32 tensors with
+// dense rows, ROPE (normal / NeoX pairing, f32), MUL_MAT of an F16 / BF16 src0 with an f32 src1.
+bool f32_rows(const tensor * t) { return t && t->type == TYPE_F32 && t->nb[0] == 4 && !(t->nb[1] & 3) && !(t->nb[2] & 3) && !(t->nb[3] & 3); }
+
+bool cont_ok(const tensor * op, const char ** why) {
+    const char * dummy; if (!why) why = &dummy;
+    const tensor * src = op->src[0];
+    if (!f32_rows(src)) { *why = "source must be F32 with dense rows"; return false; }
+    if (op->type != TYPE_F32 || !is_contiguous(op) || nelements(op) != nelements(src)) { *why = "destination must be contiguous F32 with as many elements"; return false; }
+    return true;
+}
+
+bool concat_ok(const tensor * op, const char ** why) {
+    const char * dummy; if (!why) why = &dummy;
+    const tensor * a = op->src[0], * b = op->src[1];
+    int32_t dim; memcpy(&dim, op->op_params, 4);
+    if (!f32_rows(a) || !f32_rows(b) || !f32_rows(op)) { *why = "operands must be F32 with dense rows"; return false; }
+    if (dim < 0 || dim > 3) { *why = "bad dimension"; return false; }
+    for (int i = 0; i < 4; i++)
+        if (i == dim ? op->ne[i] != a->ne[i] + b->ne[i] : (op->ne[i] != a->ne[i] || op->ne[i] != b->ne[i])) { *why = "shapes do not concatenate"; return false; }
+    return true;
+}
+
+bool rope_ok(const tensor * op, const char ** why) {
+    const char * dummy; if (!why) why = &dummy;
+    const tensor * x = op->src[0], * pos = op->src[1], * ff = op->src[2];
+    int32_t prm[5]; memcpy(prm, op->op_params, sizeof(prm));
+    if (!f32_rows(x) || !f32_rows(op)) { *why = "source and destination must be F32 with dense rows"; return false; }
+    for (int i = 0; i < 4; i++) if (op->ne[i] != x->ne[i]) { *why = "shape mismatch"; return false; }
+    if (!pos || pos->type != TYPE_I32 || !is_contiguous(pos) || nelements(pos) != x->ne[2]) { *why = "positions must be contiguous I32, one per token"; return false; }
+    if (prm[2] != MLA_ROPE_MODE_NORM && prm[2] != MLA_ROPE_MODE_NEOX) { *why = "only the normal and the NeoX pairing"; return false; }
+    if (prm[1] <= 0 || (prm[1] & 1) || prm[1] > x->ne[0] || prm[1] > 512) { *why = "n_dims must be even, <= ne0 and <= 512"; return false; }
+    if (ff && (ff->type != TYPE_F32 || !is_contiguous(ff) || ff->ne[0] < prm[1] / 2)) { *why = "frequency factors must be contiguous F32 [n_dims/2]"; return false; }
+    if (x->ne[2] > 65535 || x->ne[3] > 65535) { *why = "too many tokens for one launch"; return false; }
+    return true;
+}
+
+bool mul_mat_ok(const tensor * op, const char ** why) {
+    const char * dummy; if (!why) why = &dummy;
+    const tensor * w = op->src[0], * x = op->src[1];
+    if (!w || !x) { *why = "missing operand"; return false; }
+    if ((w->type != TYPE_F16 && w->type != TYPE_BF16) || w->nb[0] != 2) { *why = "src0 must be F16 or BF16 with dense rows"; return false; }
+    if (x->type != TYPE_F32 || x->nb[0] != 4 || op->type != TYPE_F32 || op->nb[0] != 4) { *why = "src1 and dst must be F32 with dense rows"; return false; }
+    if (w->ne[0] != x->ne[0] || w->ne[0] < 16 || w->ne[0] % 16) { *why = "K must be a multiple of 16"; return false; }
+    if (op->ne[0] != w->ne[1] || op->ne[1] != x->ne[1] || op->ne[2] != x->ne[2] || op->ne[3] != x->ne[3]) { *why = "dst must be [N, M, ne12, ne13]"; return false; }
+    if (w->ne[2] < 1 || w->ne[3] < 1 || x->ne[2] % w->ne[2] || x->ne[3] % w->ne[3]) { *why = "src0 does not broadcast over src1's batches"; return false; }
+    for (int i = 1; i < 4; i++) if ((w->nb[i] & 15) || (x->nb[i] & 15) || (op->nb[i] & 3)) { *why = "rows must be 16-byte aligned"; return false; }
+    if (x->ne[2] * x->ne[3] > 65535) { *why = "too many batches for one launch"; return false; }
+    return true;
+}
+
 bool device_supports_op(backend_device *, const tensor * op) {
     if (is_noop(op->op)) return true;
     if (op->op == OP_FLASH_ATTN_EXT) return mla_node_ok(op, nullptr);
     if (op->op == OP_CPY) return kv_cpy_ok(op, nullptr);
     if (op->op == OP_SCATTER_UPDATE) return kv_scatter_ok(op, nullptr);
+    if (op->op == OP_CONT) return cont_ok(op, nullptr);
+    if (op->op == OP_CONCAT) return concat_ok(op, nullptr);
+    if (op->op == OP_ROPE) return rope_ok(op, nullptr);
+    if (op->op == OP_MUL_MAT) return mul_mat_ok(op, nullptr);
     return false;
 }
 
@@ -372,14 +429,77 @@ int compute_kv_write(backend_ctx * ctx, const tensor * dst) {
     return STATUS_SUCCESS;
 }
 
+int launch_copy(backend_ctx * ctx, const tensor * node, const void * src, const size_t * src_nb, const int64_t * ne, void * dst, const size_t * dst_nb) {
+    mla_copy_args a;
+    a.src = src; a.dst = dst;
+    for (int i = 0; i < 4; i++) { a.ne[i] = ne[i]; a.src_nb[i] = (int64_t) src_nb[i]; a.dst_nb[i] = (int64_t) dst_nb[i]; }
+    const int rc = mla_copy_f32_launch(&a, ctx->stream);
+    if (rc != 0) { log_error("mla_copy_f32_launch failed for node '%s': %d", node->name, rc); return STATUS_FAILED; }
+    return STATUS_SUCCESS;
+}
+
+int compute_front(backend_ctx * ctx, const tensor * dst) {
+    const char * why = nullptr;
+    for (int i = 0; i < 3; i++) if (dst->src[i] && !dst->src[i]->data) { log_error("node '%s': operands not allocated", dst->name); return STATUS_FAILED; }
+    if (!dst->data) { log_error("node '%s': destination not allocated", dst->name); return STATUS_FAILED; }
+    if (dst->op == OP_CONT) {
+        if (!cont_ok(dst, &why)) { log_error("CONT node '%s' rejected: %s", dst->name, why); return STATUS_FAILED; }
+        const tensor * src = dst->src[0];   // the destination is walked in the source's shape: same element order (ggml_cont_2d)
+        const size_t dnb[4] = { 4, (size_t) src->ne[0] * 4, (size_t) (src->ne[0] * src->ne[1]) * 4, (size_t) (src->ne[0] * src->ne[1] * src->ne[2]) * 4 };
+        return launch_copy(ctx, dst, src->data, src->nb, src->ne, dst->data, dnb);
+    }
+    if (dst->op == OP_CONCAT) {
+        if (!concat_ok(dst, &why)) { log_error("CONCAT node '%s' rejected: %s", dst->name, why); return STATUS_FAILED; }
+        const tensor * a = dst->src[0], * b = dst->src[1];
+        int32_t dim; memcpy(&dim, dst->op_params, 4);
+        const int st = launch_copy(ctx, dst, a->data, a->nb, a->ne, dst->data, dst->nb);
+        if (st != STATUS_SUCCESS) return st;
+        return launch_copy(ctx, dst, b->data, b->nb, b->ne, (char *) dst->data + (size_t) a->ne[dim] * dst->nb[dim], dst->nb);
+    }
+    if (dst->op == OP_ROPE) {
+        if (!rope_ok(dst, &why)) { log_error("ROPE node '%s' rejected: %s", dst->name, why); return STATUS_FAILED; }
+        const tensor * x = dst->src[0];
+        mla_rope_args a;
+        memset(&a, 0, sizeof(a));
+        a.src = x->data; a.dst = dst->data; a.pos = (const int32_t *) dst->src[1]->data;
+        a.freq_factors = dst->src[2] ? (const float *) dst->src[2]->data : nullptr;
+        for (int i = 0; i < 4; i++) { a.ne[i] = x->ne[i]; a.src_nb[i] = (int64_t) x->nb[i]; a.dst_nb[i] = (int64_t) dst->nb[i]; }
+        int32_t prm[11]; memcpy(prm, dst->op_params, sizeof(prm));   // ggml.c:3431-3441
+        a.n_dims = prm[1]; a.mode = prm[2]; a.n_ctx_orig = prm[4];
+        memcpy(&a.freq_base, prm + 5, 4); memcpy(&a.freq_scale, prm + 6, 4); memcpy(&a.ext_factor, prm + 7, 4);
+        memcpy(&a.attn_factor, prm + 8, 4); memcpy(&a.beta_fast, prm + 9, 4); memcpy(&a.beta_slow, prm + 10, 4);
+        const int rc = mla_rope_launch(&a, ctx->stream);
+        if (rc != 0) { log_error("mla_rope_launch failed for node '%s': %d", dst->name, rc); return STATUS_FAILED; }
+        return STATUS_SUCCESS;
+    }
+    if (!mul_mat_ok(dst, &why)) { log_error("MUL_MAT node '%s' rejected: %s", dst->name, why); return STATUS_FAILED; }
+    const tensor * w = dst->src[0], * x = dst->src[1];
+    mla_mul_mat_args a;
+    memset(&a, 0, sizeof(a));
+    a.w_type = w->type; a.w = w->data; a.x = x->data; a.dst = dst->data;
+    a.K = w->ne[0]; a.N = w->ne[1]; a.w_ne2 = w->ne[2]; a.w_ne3 = w->ne[3];
+    a.M = x->ne[1]; a.ne2 = x->ne[2]; a.ne3 = x->ne[3];
+    a.w_nb1 = (int64_t) w->nb[1]; a.w_nb2 = (int64_t) w->nb[2]; a.w_nb3 = (int64_t) w->nb[3];
+    a.x_nb1 = (int64_t) x->nb[1]; a.x_nb2 = (int64_t) x->nb[2]; a.x_nb3 = (int64_t) x->nb[3];
+    a.d_nb1 = (int64_t) dst->nb[1]; a.d_nb2 = (int64_t) dst->nb[2]; a.d_nb3 = (int64_t) dst->nb[3];
+    const int rc = mla_mul_mat_launch(&a, ctx->stream);
+    if (rc != 0) { log_error("mla_mul_mat_launch failed for node '%s': %d", dst->name, rc); return STATUS_FAILED; }
+    return STATUS_SUCCESS;
+}
+
 int backend_graph_compute(backend * be, cgraph * g) {
     backend_ctx * ctx = (backend_ctx *) be->context;
     if (!HIP_OK(hipSetDevice(ctx->device))) return STATUS_FAILED;
     for (int i = 0; i < g->n_nodes; i++) {
         const tensor * node = g->nodes[i];
         if (is_empty(node) || is_noop(node->op)) continue;
-        if (node->op != OP_FLASH_ATTN_EXT && node->op != OP_CPY && node->op != OP_SCATTER_UPDATE) { log_error("op %d of node '%s' is not supported", node->op, node->name); return STATUS_FAILED; }
-        const int st = node->op == OP_FLASH_ATTN_EXT ? compute_flash_attn(ctx, node) : compute_kv_write(ctx, node);
+        int st;
+        switch (node->op) {
+            case OP_FLASH_ATTN_EXT: st = compute_flash_attn(ctx, node); break;
+            case OP_CPY: case OP_SCATTER_UPDATE: st = compute_kv_write(ctx, node); break;
+            case OP_CONT: case OP_CONCAT: case OP_ROPE: case OP_MUL_MAT: st = compute_front(ctx, node); break;
+            default: log_error("op %d of node '%s' is not supported", node->op, node->name); return STATUS_FAILED;
+        }
         if (st != STATUS_SUCCESS) return st;
     }
     return STATUS_SUCCESS;
@@ -529,6 +649,7 @@ const abi_entry k_abi_table[] = {
     E("GGML_OP_NONE", OP_NONE), E("GGML_OP_CPY", OP_CPY), E("GGML_OP_CONT", OP_CONT), E("GGML_OP_RESHAPE", OP_RESHAPE),
     E("GGML_OP_VIEW", OP_VIEW), E("GGML_OP_PERMUTE", OP_PERMUTE), E("GGML_OP_TRANSPOSE", OP_TRANSPOSE),
     E("GGML_OP_FLASH_ATTN_EXT", OP_FLASH_ATTN_EXT), E("GGML_OP_SCATTER_UPDATE", OP_SCATTER_UPDATE), E("GGML_OP_COUNT", OP_COUNT),
+    E("GGML_OP_ROPE", OP_ROPE), E("GGML_OP_MUL_MAT", OP_MUL_MAT), E("GGML_OP_CONCAT", OP_CONCAT),
     E("GGML_STATUS_ALLOC_FAILED", STATUS_ALLOC_FAILED), E("GGML_STATUS_FAILED", STATUS_FAILED), E("GGML_STATUS_SUCCESS", STATUS_SUCCESS),
     E("GGML_STATUS_ABORTED", STATUS_ABORTED),
     E("GGML_BACKEND_DEVICE_TYPE_CPU", DEVICE_TYPE_CPU), E("GGML_BACKEND_DEVICE_TYPE_GPU", DEVICE_TYPE_GPU),

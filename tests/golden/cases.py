@@ -39,3 +39,36 @@ def make_inputs(name):
     if mask is not None:
         h.update(mask.tobytes())
     return dict(q=q, k=k, k_type=k_type, mask=mask, scale=U.SCALE, digest=h.hexdigest())
+
+
+# The nodes either side of the attention node: (kind, weight type, n_head, n_tok, rope mode, freq_scale, ext_factor, attn_factor, seed)
+FRONT_CASES = {
+    "rope_norm_plain": ("rope", None, 3, 7, 0, 1.0, 0.0, 1.0, 11),
+    "rope_norm_yarn_deepseek": ("rope", None, 3, 7, 0, 0.025, 1.0, 0.8, 12),
+    "rope_neox_yarn_partial": ("rope", None, 2, 5, 2, 0.5, 0.25, 1.3, 13),
+    "q_states_bf16": ("q_states", O.TYPE_BF16, 4, 5, 0, 0.025, 1.0, 0.8, 14),
+    "q_states_f16": ("q_states", O.TYPE_F16, 4, 5, 0, 1.0, 0.0, 1.0, 15),
+    "unabsorb_bf16": ("unabsorb", O.TYPE_BF16, 4, 5, 0, 1.0, 0.0, 1.0, 16),
+    "unabsorb_f16": ("unabsorb", O.TYPE_F16, 4, 5, 0, 1.0, 0.0, 1.0, 17),
+}
+
+
+def make_front_inputs(name):
+    kind, w_type, H, n_tok, mode, fs, ext, af, seed = FRONT_CASES[name]
+    rng = np.random.default_rng(seed)
+    p = O.rope_params(n_dims=64, mode=mode, freq_scale=fs, ext_factor=ext, attn_factor=af, n_ctx_orig=4096)
+    pos = rng.integers(0, 160000, size=n_tok).astype(np.int32)
+    d = dict(kind=kind, w_type=w_type, n_head=H, p=p, pos=pos)
+    if kind == "rope":
+        d["x"] = rng.standard_normal((n_tok, H, 64)).astype(np.float32)
+        blobs = [d["x"], pos]
+    else:
+        w = (rng.standard_normal((H * 256, 512)) * 0.05).astype(np.float32)
+        d["wkv_b"] = O.f32_to_f16(w) if w_type == O.TYPE_F16 else O.f32_to_bf16(w)
+        d["x"] = rng.standard_normal((n_tok, H * 192) if kind == "q_states" else (H, n_tok, 512)).astype(np.float32)
+        blobs = [d["x"], pos, d["wkv_b"]]
+    h = hashlib.sha256()
+    for b in blobs:
+        h.update(b.tobytes())
+    d["digest"] = h.hexdigest()
+    return d

@@ -33,7 +33,7 @@ def _mirror_table():
 def test_library_exports_every_declared_symbol():
     lib = _lib()
     declared = set()
-    for hdr in ("mla_attn.h", "mla_kv_write.h", "mla_page_table.h", "ggml_mla_backend.h"):
+    for hdr in ("mla_attn.h", "mla_kv_write.h", "mla_front.h", "mla_page_table.h", "ggml_mla_backend.h"):
         src = open(os.path.join(ROOT, "include", hdr)).read()
         src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
         declared |= set(re.findall(r"\b(mla_\w+|ggml_backend_\w+)\s*\(", src))

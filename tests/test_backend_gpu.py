@@ -61,3 +61,52 @@ def test_batched_decode_through_the_mask_as_llama_builds_it(gpu, use_sched):
     got, info = O.ref_backend_flash_attn_ext(_so(), q, k, O.TYPE_BF16, dv=512, mask=mask, scale=U.SCALE, use_sched=use_sched)
     want = O.flash_attn_ext(q, k, O.TYPE_BF16, dv=512, mask=mask, scale=U.SCALE)
     print(U.check(got[..., :512], want, "masked batched decode through the reference's ggml"))
+
+
+@pytest.mark.parametrize("w_type", [O.TYPE_BF16, O.TYPE_F16])
+@pytest.mark.parametrize("n_tok", [1, 32, 150])
+def test_query_side_and_output_side_graphs_through_the_plugin(gpu, w_type, n_tok):
+    """The sub-graphs llm_attn_mla builds before and after the attention node (views of q, CONT, ROPE, PERMUTE, MUL_MAT
+    with the wk_b / wv_b views of wkv_b, CONCAT, CONT_2D), built by the reference's own ggml and computed node by node
+    by the plugin; the same graphs on the reference's ggml-cpu are the expected values.
+    Tolerances: the rope columns 4e-6 * max|x| * mscale, the products 2e-6 relative L2 (f32 accumulation order)."""
+    H = 16
+    rng = np.random.default_rng(500 + n_tok)
+    w = (rng.standard_normal((H * 256, 512)) * 0.05).astype(np.float32)
+    wkv_b = O.f32_to_f16(w) if w_type == O.TYPE_F16 else O.f32_to_bf16(w)
+    q = rng.standard_normal((n_tok, H * 192)).astype(np.float32)
+    pos = rng.integers(0, 100000, size=n_tok).astype(np.int32)
+    p = O.rope_params(freq_scale=0.025, ext_factor=1.0, attn_factor=0.8)
+    got = O.ref_mla_q_states(q, wkv_b, w_type, pos, p, H, so_path=_so())
+    cpu = O.ref_mla_q_states(q, wkv_b, w_type, pos, p, H)
+    assert not np.isnan(got).any()
+    assert float(np.max(np.abs(got[:, :, 512:] - cpu[:, :, 512:]))) <= 4e-6 * 6
+    assert O.errors(got[:, :, :512], cpu[:, :, :512])[1] < 2e-6
+    assert O.errors(got, O.mla_q_states(q, wkv_b, w_type, pos, p, H))[1] < 2e-6
+    kqv = rng.standard_normal((H, n_tok, 512)).astype(np.float32)
+    got = O.ref_mla_unabsorb(kqv, wkv_b, w_type, H, so_path=_so())
+    assert O.errors(got, O.ref_mla_unabsorb(kqv, wkv_b, w_type, H))[1] < 2e-6
+
+
+@pytest.mark.parametrize("mode", [0, 2])
+def test_rope_node_through_the_plugin(gpu, mode):
+    rng = np.random.default_rng(510)
+    p = O.rope_params(n_dims=32, mode=mode, freq_scale=0.25, ext_factor=1.0)
+    x = rng.standard_normal((9, 3, 80)).astype(np.float32)
+    pos = (np.arange(9) * 1000).astype(np.int32)
+    ff = (1 + rng.random(16)).astype(np.float32)
+    got = O.ref_rope(x, pos, p, ff, so_path=_so())
+    assert float(np.max(np.abs(got - O.ref_rope(x, pos, p, ff)))) <= 4e-6 * 6 * 1.2
+    np.testing.assert_array_equal(got[..., 32:], x[..., 32:])
+
+
+def test_mul_mat_node_the_plugin_leaves_to_other_backends(gpu):
+    """An F32 src0 is not taken (supports_op false -> the driver reports the node index), nothing is computed wrongly."""
+    rng = np.random.default_rng(520)
+    a = rng.standard_normal((2, 32, 64)).astype(np.float32)
+    b = rng.standard_normal((2, 5, 64)).astype(np.float32)
+    with pytest.raises(RuntimeError, match="-100"):
+        O.ref_mul_mat(a, O.TYPE_F32, b, so_path=_so())
+    w = O.f32_to_bf16(a)
+    got = O.ref_mul_mat(w, O.TYPE_BF16, b, so_path=_so())
+    assert O.errors(got, O.ref_mul_mat(w, O.TYPE_BF16, b))[1] < 2e-6

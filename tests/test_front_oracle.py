@@ -231,6 +231,23 @@ def test_mul_mat_and_absorb_graphs_against_compiled_reference(w_type):
     assert O.errors(O.mla_unabsorb(kqv, wkv_b, w_type, H), O.ref_mla_unabsorb(kqv, wkv_b, w_type, H))[1] < 1e-6
 
 
+def test_oracle_against_golden_vectors_of_the_compiled_reference():
+    """tests/golden/front_golden.npz: outputs of the reference's compiled ggml-cpu (made by tests/golden/gen_golden.py)."""
+    from tests.golden import cases
+    gold = np.load(os.path.join(ROOT, "tests", "golden", "front_golden.npz"))
+    for name in cases.FRONT_CASES:
+        inp = cases.make_front_inputs(name)
+        assert bytes(gold[name + "/digest"]).decode() == inp["digest"], "inputs of %s are not the ones the fixture was made from" % name
+        if inp["kind"] == "rope":
+            np.testing.assert_array_equal(O.rope(inp["x"], inp["pos"], inp["p"]), gold[name])
+        elif inp["kind"] == "q_states":
+            got = O.mla_q_states(inp["x"], inp["wkv_b"], inp["w_type"], inp["pos"], inp["p"], inp["n_head"])
+            np.testing.assert_array_equal(got[:, :, 512:], gold[name][:, :, 512:])
+            assert O.errors(got, gold[name])[1] < 1e-6
+        else:
+            assert O.errors(O.mla_unabsorb(inp["x"], inp["wkv_b"], inp["w_type"], inp["n_head"]), gold[name])[1] < 1e-6
+
+
 def _header_offsets(struct, fields):
     src = '#include <stdio.h>\n#include <stddef.h>\n#include "mla_front.h"\nint main(void){\n'
     src += 'printf("%%zu\\n", sizeof(%s));\n' % struct
