@@ -19,6 +19,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 / fp16 MFMA rate
 KV_ROW_BYTES = 1152     # 576 bf16
 FLOP_PER_TOKEN_HEAD = 2 * 576 + 2 * 512
 
@@ -112,6 +113,80 @@ def kv_write_config(a, dev, lib, J):
                                    "unit": "GB/s", "frac": nbytes / (kern_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, "traffic": None,
                                    "algorithmic_bytes_per_launch": nbytes, "kernel_us": {"mean": kern_ms * 1e3}},
                       "cpu_baseline": None}))
+
+
+def front_config(a, dev, lib, J):
+    """The nodes either side of the attention node (include/mla_front.h) at the headline model shape (128 heads):
+    absorb = q_nope [128] x wk_b [128 x 512] per head, unabsorb = wv_b [512 x 128] x kqv [512] per head, rope = q_pe
+    [64] per head.  --tokens 32 is a decode step of 32 sequences (bound by the 16.8 MB weight stream: wkv_b of 32
+    different layers is rotated so that it comes from HBM), --tokens 2048 a prefill chunk (bound by the matrix cores)."""
+    import torch
+    H, T, layers = a.heads, a.tokens, 32
+    g = torch.Generator(device=dev)
+    g.manual_seed(a.seed)
+    stream = torch.cuda.current_stream(dev)
+    if a.config == "rope":
+        x = torch.randn((T, H, 64), generator=g, device=dev, dtype=torch.float32)
+        pos = torch.randint(0, 163840, (T,), generator=g, device=dev, dtype=torch.int32)
+        out = torch.empty_like(x)
+        fn = lambda i: J.ggml_rope_ext(x, pos, n_dims=64, n_ctx_orig=4096, freq_scale=0.025, ext_factor=1.0, attn_factor=0.8, out=out)
+        nbytes, flops, kernel = x.numel() * 8, 0, "mla_rope_kernel"
+        what = "rotary embedding (YaRN) of q_pe: %d tokens x %d heads x 64" % (T, H)
+    else:
+        K, N = (128, 512) if a.config == "absorb" else (512, 128)
+        w = (torch.randn((layers, H, N, K), generator=g, device=dev, dtype=torch.float32) * 0.05).to(torch.bfloat16).view(torch.int16)
+        x = torch.randn((H, T, K), generator=g, device=dev, dtype=torch.float32)
+        out = torch.empty((H, T, N), device=dev, dtype=torch.float32)
+        fn = lambda i: J.ggml_mul_mat(w[i % layers], J.MLA_TYPE_BF16, x, out=out)
+        nbytes, flops = H * N * K * 2 + x.numel() * 4 + out.numel() * 4, 2 * H * T * N * K
+        kernel = "mla_mul_mat_kernel"
+        what = "%s product: %d heads x [%d tokens x %d] x [%d x %d] bf16 weights (one of %d layers per step)" % (a.config, H, T, K, K, N, layers)
+
+    def run(n):
+        for i in range(n):
+            fn(i)
+
+    run(a.warmup)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    run(a.steps)
+    torch.cuda.synchronize()
+    eager_ms = (time.perf_counter() - t0) * 1e3 / a.steps
+    # one launch per step: eager steps are bound by the host's launch rate, so the K steps are also replayed from a HIP graph
+    side = torch.cuda.Stream(dev)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        graph.capture_begin()
+        run(a.steps)
+        graph.capture_end()
+    torch.cuda.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    graph.replay()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / a.steps
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    graph.replay()
+    e1.record(stream)
+    torch.cuda.synchronize()
+    kern_ms = e0.elapsed_time(e1) / a.steps
+    hbm_time, mfma_time = nbytes / (HBM_PEAK_GBPS * 1e9), flops / (MFMA_BF16_PEAK_TFLOPS * 1e12)
+    if mfma_time > hbm_time:
+        ach = flops / (kern_ms * 1e-3) / 1e12
+        roof = {"bound": "mfma", "kernel": kernel, "achieved": ach, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": ach / MFMA_BF16_PEAK_TFLOPS}
+        metric, value, unit = "mla_%s_mfma_rate" % a.config, flops / (ms * 1e-3) / 1e12, "TFLOP/s"
+    else:
+        ach = nbytes / (kern_ms * 1e-3) / 1e9
+        roof = {"bound": "hbm", "kernel": kernel, "achieved": ach, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": ach / HBM_PEAK_GBPS}
+        metric, value, unit = "mla_%s_bandwidth" % a.config, nbytes / (ms * 1e-3) / 1e9, "GB/s"
+    roof.update({"traffic": None, "algorithmic_bytes_per_launch": nbytes, "flops_per_launch": flops, "kernel_us": {"mean": kern_ms * 1e3}})
+    print(json.dumps({"metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+                      "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+                      "dtype": "f32" if a.config == "rope" else "bf16", "data": "synthetic", "config": {"workload": what},
+                      "us_per_step": ms * 1e3, "eager_us_per_step": eager_ms * 1e3, "launch": "hip graph replay of the K steps",
+                      "roofline": roof, "cpu_baseline": None}))
 
 
 def other_config(a, dev, lib, J):
@@ -241,12 +316,13 @@ def main():
     ap.add_argument("--rows-per-wg", type=int, default=0)
     ap.add_argument("--cpu-seqs", type=int, default=8, help="sequences of the workload timed on the host cores (0 = skip)")
     ap.add_argument("--seed", type=int, default=1234)
+    ap.add_argument("--tokens", type=int, default=32, help="query tokens of --config rope / absorb / unabsorb (32 = a decode step, 2048 = a prefill chunk)")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="N",
                     help="also launch the library's plain copy kernel N times over one KV pool (known byte count) so that a "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run can be scaled")
     ap.add_argument("--kv", default="bf16", choices=["bf16", "f16", "q8_0"], help="storage type of the latent KV pool (the headline config is bf16; q8_0 only with --config kvwrite)")
     ap.add_argument("--eager", action="store_true", help="time the K steps as K eager launch sequences instead of one replay of a HIP graph that holds them")
-    ap.add_argument("--config", default="c3", choices=["c2", "c3", "c3mask", "c4", "c5", "kvwrite"],
+    ap.add_argument("--config", default="c3", choices=["c2", "c3", "c3mask", "c4", "c5", "kvwrite", "rope", "absorb", "unabsorb"],
                     help="c3 (default) is the headline workload; the others time BASELINE's remaining GPU configs and the cache write for the profiles")
     a = ap.parse_args()
     if a.gpus != 1:
@@ -263,6 +339,9 @@ def main():
     scale = 1.0 / (192.0 ** 0.5)
     if a.config == "kvwrite":
         kv_write_config(a, dev, lib, J)
+        return
+    if a.config in ("rope", "absorb", "unabsorb"):
+        front_config(a, dev, lib, J)
         return
     if a.config != "c3":
         other_config(a, dev, lib, J)

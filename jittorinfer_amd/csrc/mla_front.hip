@@ -162,10 +162,168 @@ __global__ void __launch_bounds__(256) mla_mul_mat_kernel(const MmP p) {
         }
 }
 
+// Few rows m (a decode step): nothing is shared between waves, so there is no staging and no barrier before the MFMAs.
+// A workgroup owns 32 outputs n and 32 rows m; its four waves take every fourth k-step of 16, load their weight and
+// activation fragments straight from global memory into the MFMA operand registers (up to 8 k-steps in flight per
+// wave), and the four partial accumulators meet in LDS.  The grid is (N / 32) x (M / 32) x batches workgroups, enough to
+// keep the weight stream of a 128-head layer in flight on every CU.
+template <bool F16>
+__global__ void __launch_bounds__(256) mla_mul_mat_skinny_kernel(const MmP p) {
+    __shared__ float red[4][16][64];
+    const int     lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t i2 = blockIdx.z % p.ne2, i3 = blockIdx.z / p.ne2;
+    const int64_t n0 = (int64_t) blockIdx.x * 32, m0 = (int64_t) blockIdx.y * 32;
+    const char *  wrow = p.w + (i2 / p.r2) * p.w_nb2 + (i3 / p.r3) * p.w_nb3 + min(n0 + (lane & 31), p.N - 1) * p.w_nb1 + (lane >> 5) * 16;
+    const char *  xrow = p.x + i2 * p.x_nb2 + i3 * p.x_nb3 + min(m0 + (lane & 31), p.M - 1) * p.x_nb1 + (lane >> 5) * 32;
+    const int     nks = (int) (p.K / 16);
+    constexpr int U = 8;
+    f32x16 acc;
+#pragma unroll
+    for (int j = 0; j < 16; j++) acc[j] = 0.f;
+    for (int base = wave; base < nks; base += 4 * U) {
+        u32x4  wf[U];
+        float4 xa[U], xb[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int ks = min(base + 4 * u, nks - 1);   // past the end: a valid address, the fragment is not used
+            wf[u] = *(const u32x4 *) (wrow + (int64_t) ks * 32);
+            xa[u] = *(const float4 *) (xrow + (int64_t) ks * 64);
+            xb[u] = *(const float4 *) (xrow + (int64_t) ks * 64 + 16);
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++)
+            if (base + 4 * u < nks) {
+                u32x4 af;
+                af[0] = pack2<F16>(xa[u].x, xa[u].y); af[1] = pack2<F16>(xa[u].z, xa[u].w);
+                af[2] = pack2<F16>(xb[u].x, xb[u].y); af[3] = pack2<F16>(xb[u].z, xb[u].w);
+                acc = mfma32<F16>(af, wf[u], acc);
+            }
+    }
+#pragma unroll
+    for (int j = 0; j < 16; j++) red[wave][j][lane] = acc[j];
+    __syncthreads();
+    const int64_t n = n0 + (lane & 31);
+    char * D = p.dst + i2 * p.d_nb2 + i3 * p.d_nb3;
+#pragma unroll
+    for (int jj = 0; jj < 4; jj++) {   // wave w finishes accumulator registers 4w .. 4w+3 (8 rows m)
+        const int     j = wave * 4 + jj;
+        const float   v = (red[0][j][lane] + red[1][j][lane]) + (red[2][j][lane] + red[3][j][lane]);
+        const int64_t m = m0 + (j >> 2) * 8 + (lane >> 5) * 4 + (j & 3);
+        if (m < p.M && n < p.N) ((float *) (D + m * p.d_nb1))[n] = v;
+    }
+}
+
+// Many rows m with K = 128, 256 or 512 (a prefill chunk through the absorb products): bound by the f32 activations
+// and results moving through HBM, not by the matrix cores, so the kernel is a software pipeline around the loads.  A
+// workgroup keeps its 128 weight rows (all of K) in MFMA operand registers and walks over tiles of 64 rows m; while the
+// MFMAs of one 64 x 128 activation chunk run out of LDS, the next chunk's global loads are in flight, and it is rounded
+// into the other LDS buffer at the end of the step: one barrier per chunk.
+template <bool F16, int KCH>
+__global__ void __launch_bounds__(256) mla_mul_mat_stream_kernel(const MmP p, const int tiles_per_wg) {
+    constexpr int TM = 64;
+    __shared__ __attribute__((aligned(16))) char lds[2][TM * MM_PITCH];
+    const int     lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t i2 = blockIdx.z % p.ne2, i3 = blockIdx.z / p.ne2;
+    const char *  X  = p.x + i2 * p.x_nb2 + i3 * p.x_nb3;
+    char *        D  = p.dst + i2 * p.d_nb2 + i3 * p.d_nb3;
+    const int64_t n0 = (int64_t) blockIdx.x * 128 + wave * 32;
+    const int64_t n  = n0 + (lane & 31);
+    const char *  wrow = p.w + (i2 / p.r2) * p.w_nb2 + (i3 / p.r3) * p.w_nb3 + min(n, p.N - 1) * p.w_nb1 + (lane >> 5) * 16;
+    const int64_t n_tiles = (p.M + TM - 1) / TM;
+    const int64_t t0 = (int64_t) blockIdx.y * tiles_per_wg, t1 = min(t0 + tiles_per_wg, n_tiles);
+    if (t0 >= t1) return;
+
+    u32x4 wf[KCH * 8];
+#pragma unroll
+    for (int i = 0; i < KCH * 8; i++) wf[i] = *(const u32x4 *) (wrow + i * 32);
+
+    // a chunk = 64 rows x 128 k of f32: thread t takes float4 number (t & 31) of rows (t >> 5) + 8 i
+    const int srow = threadIdx.x >> 5, sc4 = threadIdx.x & 31;
+    float4    st[8];
+    auto load_chunk = [&](int64_t tile, int kc) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int64_t m = tile * TM + srow + 8 * i;
+            st[i] = m < p.M ? *(const float4 *) (X + m * p.x_nb1 + (int64_t) (kc * MM_KC + sc4 * 4) * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    };
+    auto stage_chunk = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            u32x2 v;
+            v[0] = pack2<F16>(st[i].x, st[i].y); v[1] = pack2<F16>(st[i].z, st[i].w);
+            *(u32x2 *) (lds[buf] + (srow + 8 * i) * MM_PITCH + sc4 * 8) = v;
+        }
+    };
+
+    f32x16 acc[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 16; j++) acc[i][j] = 0.f;
+
+    load_chunk(t0, 0);
+    stage_chunk(0);
+    __syncthreads();
+    int buf = 0;
+    for (int64_t tile = t0; tile < t1; tile++) {
+#pragma unroll
+        for (int kc = 0; kc < KCH; kc++) {
+            const bool last_kc = kc == KCH - 1;
+            const bool more = !last_kc || tile + 1 < t1;
+            if (more) load_chunk(last_kc ? tile + 1 : tile, last_kc ? 0 : kc + 1);
+#pragma unroll
+            for (int ks = 0; ks < 8; ks++)
+#pragma unroll
+                for (int mb = 0; mb < 2; mb++) {
+                    const u32x4 af = *(const u32x4 *) (lds[buf] + (mb * 32 + (lane & 31)) * MM_PITCH + ks * 32 + (lane >> 5) * 16);
+                    acc[mb] = mfma32<F16>(af, wf[kc * 8 + ks], acc[mb]);
+                }
+            if (last_kc) {
+                if (n < p.N) {
+#pragma unroll
+                    for (int mb = 0; mb < 2; mb++)
+#pragma unroll
+                        for (int j = 0; j < 16; j++) {
+                            const int64_t m = tile * TM + mb * 32 + (j >> 2) * 8 + (lane >> 5) * 4 + (j & 3);
+                            if (m < p.M) ((float *) (D + m * p.d_nb1))[n] = acc[mb][j];
+                        }
+                }
+#pragma unroll
+                for (int mb = 0; mb < 2; mb++)
+#pragma unroll
+                    for (int j = 0; j < 16; j++) acc[mb][j] = 0.f;
+            }
+            if (more) stage_chunk(buf ^ 1);
+            __syncthreads();
+            buf ^= 1;
+        }
+    }
+}
+
+template <bool F16>
+hipError_t launch_mm_stream(const MmP & p, int64_t batches, hipStream_t st) {
+    const int64_t n_tiles = (p.M + 63) / 64, gx = (p.N + 127) / 128;
+    int64_t groups = (1024 + gx * batches - 1) / (gx * batches);   // about four workgroups per CU in total
+    if (groups > n_tiles) groups = n_tiles;
+    const int  tiles_per_wg = (int) ((n_tiles + groups - 1) / groups);
+    const dim3 grid((unsigned) gx, (unsigned) ((n_tiles + tiles_per_wg - 1) / tiles_per_wg), (unsigned) batches);
+    switch (p.K / MM_KC) {
+        case 1:  hipLaunchKernelGGL((mla_mul_mat_stream_kernel<F16, 1>), grid, dim3(256), 0, st, p, tiles_per_wg); break;
+        case 2:  hipLaunchKernelGGL((mla_mul_mat_stream_kernel<F16, 2>), grid, dim3(256), 0, st, p, tiles_per_wg); break;
+        default: hipLaunchKernelGGL((mla_mul_mat_stream_kernel<F16, 4>), grid, dim3(256), 0, st, p, tiles_per_wg); break;
+    }
+    return hipGetLastError();
+}
+
 template <bool F16>
 hipError_t launch_mm(const MmP & p, int64_t batches, hipStream_t st) {
+    if (p.M > 64 && (p.K == 128 || p.K == 256 || p.K == 512)) return launch_mm_stream<F16>(p, batches, st);
     const unsigned gx = (unsigned) ((p.N + 127) / 128);
-    if (p.M <= 32) {
+    if (p.M <= 64 && (int64_t) gx * ((p.M + 31) / 32) * batches < 512 && p.K >= 256) {
+        // few rows and fewer than two workgroups per CU with 128-wide tiles: split n finer and K over the waves
+        hipLaunchKernelGGL((mla_mul_mat_skinny_kernel<F16>), dim3((unsigned) ((p.N + 31) / 32), (unsigned) ((p.M + 31) / 32), (unsigned) batches), dim3(256), 0, st, p);
+    } else if (p.M <= 32) {
         hipLaunchKernelGGL((mla_mul_mat_kernel<F16, 1>), dim3(gx, (unsigned) ((p.M + 31) / 32), (unsigned) batches), dim3(256), 0, st, p);
     } else if (p.M <= 64) {
         hipLaunchKernelGGL((mla_mul_mat_kernel<F16, 2>), dim3(gx, (unsigned) ((p.M + 63) / 64), (unsigned) batches), dim3(256), 0, st, p);

@@ -99,7 +99,7 @@ def _check_mm(got, want, ab, what):
 
 @pytest.mark.parametrize("w_type", [O.TYPE_BF16, O.TYPE_F16])
 @pytest.mark.parametrize("K,N,M,H", [(128, 512, 32, 16), (512, 128, 32, 16), (128, 512, 1, 4), (512, 128, 33, 3),
-                                     (128, 512, 130, 2), (64, 100, 70, 5), (16, 32, 5, 1), (528, 40, 64, 2)])
+                                     (128, 512, 130, 2), (64, 100, 70, 5), (16, 32, 5, 1), (528, 40, 64, 2), (256, 96, 100, 3), (512, 128, 321, 2)])
 def test_mul_mat_shapes(gpu, w_type, K, N, M, H):
     import torch
     import jittorinfer_amd as J
