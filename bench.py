@@ -182,11 +182,36 @@ def front_config(a, dev, lib, J):
         roof = {"bound": "hbm", "kernel": kernel, "achieved": ach, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": ach / HBM_PEAK_GBPS}
         metric, value, unit = "mla_%s_bandwidth" % a.config, nbytes / (ms * 1e-3) / 1e9, "GB/s"
     roof.update({"traffic": None, "algorithmic_bytes_per_launch": nbytes, "flops_per_launch": flops, "kernel_us": {"mean": kern_ms * 1e3}})
+    cpu = None
+    if a.cpu_seqs > 0:
+        # the same node on the host cores: the reference's compiled ggml-cpu when oracle/_ref is built, else the C restatement
+        from oracle import oracle as O
+        cores = min(os.cpu_count() or 1, 16)
+        if a.config == "rope":
+            xs, ps = x.cpu().numpy(), pos.cpu().numpy()
+            prm = O.rope_params(freq_scale=0.025, ext_factor=1.0, attn_factor=0.8)
+            f = (lambda: O.ref_rope(xs, ps, prm, n_threads=cores)) if O.ref_available() else (lambda: O.rope(xs, ps, prm))
+            sample, frac = "the whole workload", 1.0
+        else:
+            hs = min(H, 8)
+            ws, xs = w[0, :hs].cpu().numpy().view("uint16"), x[:hs].cpu().numpy()
+            f = (lambda: O.ref_mul_mat(ws, O.TYPE_BF16, xs, n_threads=cores)) if O.ref_available() else (lambda: O.mul_mat(ws, O.TYPE_BF16, xs))
+            sample, frac = "%d of the %d heads" % (hs, H), hs / H
+        f()
+        best = min(_timed(f) for _ in range(3))
+        cpu = {"value": nbytes * frac / best / 1e9, "unit": "GB/s", "cores": cores if O.ref_available() else 1,
+               "kind": "reference" if O.ref_available() else "port", "sample": sample, "seconds": best}
     print(json.dumps({"metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
                       "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
                       "dtype": "f32" if a.config == "rope" else "bf16", "data": "synthetic", "config": {"workload": what},
                       "us_per_step": ms * 1e3, "eager_us_per_step": eager_ms * 1e3, "launch": "hip graph replay of the K steps",
-                      "roofline": roof, "cpu_baseline": None}))
+                      "roofline": roof, "cpu_baseline": cpu}))
+
+
+def _timed(f):
+    t0 = time.perf_counter()
+    f()
+    return time.perf_counter() - t0
 
 
 def other_config(a, dev, lib, J):
@@ -243,7 +268,25 @@ def other_config(a, dev, lib, J):
     t0 = time.perf_counter()
     run(lib.mla_attn_launch, a.steps)
     torch.cuda.synchronize()
-    ms = (time.perf_counter() - t0) * 1e3 / a.steps
+    eager_ms = ms = (time.perf_counter() - t0) * 1e3 / a.steps
+    if not a.eager:   # as for the headline config: the K steps replayed from one HIP graph
+        side = torch.cuda.Stream(dev)
+        graph = torch.cuda.CUDAGraph()
+        sst = C.c_void_p(side.cuda_stream)
+        with torch.cuda.stream(side):
+            graph.capture_begin()
+            for _ in range(a.steps):
+                rc = lib.mla_attn_launch(C.byref(ar), sst)
+                if rc != 0:
+                    raise RuntimeError("launch failed during capture: %d" % rc)
+            graph.capture_end()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        graph.replay()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / a.steps
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record(stream)
     run(lib.mla_attn_launch_kernel, a.steps)
@@ -266,7 +309,8 @@ def other_config(a, dev, lib, J):
     print(json.dumps({"metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
                       "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
                       "dtype": "f16" if kv == "q8_0" else kv, "data": "synthetic",
-                      "config": {"workload": name, "plan": plan}, "us_per_step": ms * 1e3, "roofline": roof, "cpu_baseline": None}))
+                      "config": {"workload": name, "plan": plan}, "us_per_step": ms * 1e3, "eager_us_per_step": eager_ms * 1e3,
+                      "launch": "eager" if a.eager else "hip graph replay of the K steps", "roofline": roof, "cpu_baseline": None}))
 
 
 def cpu_baseline(q, pool, block_table, ctx, n_sample, scale, gpu_out):

@@ -198,3 +198,27 @@ def test_rejected_arguments(gpu):
     with pytest.raises(RuntimeError):
         J.ggml_mul_mat(w, O.TYPE_BF16, torch.zeros((1, 4, 24), dtype=torch.float32, device=gpu))   # K % 16 != 0
     assert lib.mla_rope_launch(None, None) == -5 and lib.mla_mul_mat_launch(None, None) == -5 and lib.mla_copy_f32_launch(None, None) == -5
+
+
+def test_query_side_in_two_launches_through_the_strides(gpu):
+    """The byte strides of both entry points take the reference's views as they are: rope reads the q_pe view inside q and
+    writes the last 64 columns of q_states, the product reads the permuted q_nope view and writes the first 512: two
+    launches produce what cont + rope + permute + mul_mat + concat produce."""
+    import torch
+    import jittorinfer_amd as J
+    H, n_tok = 16, 40
+    rng = np.random.default_rng(600)
+    wkv_b = _w(rng, (H * 256, 512), O.TYPE_BF16)
+    q = rng.standard_normal((n_tok, H * 192)).astype(np.float32)
+    pos = rng.integers(0, 100000, size=n_tok).astype(np.int32)
+    p = O.rope_params(freq_scale=0.025, ext_factor=1.0, attn_factor=0.8)
+    tw, tq = _t(gpu, wkv_b).reshape(-1), _t(gpu, q).reshape(n_tok, H, 192)
+    q_states = torch.full((H, n_tok, 576), float("nan"), dtype=torch.float32, device=gpu)
+    J.ggml_rope_ext(tq[:, :, 128:], _t(gpu, pos), n_dims=64, n_ctx_orig=4096, freq_scale=0.025, ext_factor=1.0, attn_factor=0.8,
+                    out=q_states[:, :, 512:].permute(1, 0, 2))
+    J.ggml_mul_mat(tw[:H * 512 * 128].reshape(H, 512, 128), O.TYPE_BF16, tq[:, :, :128].permute(1, 0, 2), out=q_states[:, :, :512])
+    torch.cuda.synchronize()
+    want = O.mla_q_states(q, wkv_b, O.TYPE_BF16, pos, p, H)
+    got = q_states.cpu().numpy()
+    assert float(np.max(np.abs(got[:, :, 512:] - want[:, :, 512:]))) <= 4e-6 * 6
+    assert O.errors(got[:, :, :512], want[:, :, :512])[1] < 2e-6
