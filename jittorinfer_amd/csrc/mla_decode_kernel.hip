@@ -82,12 +82,24 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int g = lane >> 5, rl = lane & 31;
-    const int b = blockIdx.z, split = blockIdx.x;
+    // Workgroups are handed to the 8 XCDs round-robin in dispatch order, and each XCD has its own L2.  The splits of one
+    // (sequence, row block) all read the same 147 KB Q operand image, so the dispatch index is remapped to put them on one
+    // XCD: index i runs on XCD i % 8, and the i / 8-th workgroup of that XCD takes the tuple number (i % 8) * G / 8 + i / 8.
+    int bx = blockIdx.x, by = blockIdx.y, bz = blockIdx.z;
+    {
+        const unsigned G = gridDim.x * gridDim.y * gridDim.z;
+        if ((G & 7) == 0) {
+            const unsigned id = (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+            const unsigned v  = (id & 7) * (G >> 3) + (id >> 3);
+            bx = v % gridDim.x; by = (v / gridDim.x) % gridDim.y; bz = v / (gridDim.x * gridDim.y);
+        }
+    }
+    const int b = bz, split = bx;
 
     const int seq_len  = p.block_table ? min(p.seq_lens[b], (int) p.bt_stride * MLA_PAGE_TOKENS) : (int) p.n_kv;
     int kv_begin = split * p.split_tokens;
     int kv_end   = min(seq_len, kv_begin + p.split_tokens);
-    const int row       = blockIdx.y * 128 + wave * 32 + rl;
+    const int row       = by * 128 + wave * 32 + rl;
     const bool row_valid = row < p.n_rows;
     const int64_t orow  = (int64_t) b * p.n_rows + row;
     const int64_t prow  = ((int64_t) b * p.n_splits + split) * p.n_rows + row;
@@ -96,8 +108,8 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
     if constexpr (MASK) {
         int mlo = 0x7fffffff, mhi = 0;
         for (int c = 0; c < 16; c++) {
-            mlo = min(mlo, p.mask_ext[(blockIdx.y * 16 + c) * 2]);
-            mhi = max(mhi, p.mask_ext[(blockIdx.y * 16 + c) * 2 + 1]);
+            mlo = min(mlo, p.mask_ext[(by * 16 + c) * 2]);
+            mhi = max(mhi, p.mask_ext[(by * 16 + c) * 2 + 1]);
         }
         const int hi = min(seq_len, (mhi + TILE_TOK - 1) / TILE_TOK * TILE_TOK), lo = min(mlo / TILE_TOK * TILE_TOK, hi);
         int chunk = ((hi - lo + p.n_splits - 1) / p.n_splits + TILE_TOK - 1) / TILE_TOK * TILE_TOK;
@@ -143,7 +155,7 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
         h[3] = (unsigned long long) p.debug_ptr;
     }
     // this wave's packed Q operands: [seq][row block][wave][k-step][lane][16 bytes], written by mla_q_pack_kernel
-    const char * qpack = (const char *) p.q_pack + ((((int64_t) b * gridDim.y + blockIdx.y) * 4) * KSTEPS) * 1024;  // + wave*36 KB, added in the wave program
+    const char * qpack = (const char *) p.q_pack + ((((int64_t) b * gridDim.y + by) * 4) * KSTEPS) * 1024;  // + wave*36 KB, added in the wave program
     const char *    kv_base = p.kv + (p.block_table ? 0 : (int64_t) b * p.kv_nb3);
     const int32_t * bt_row  = p.block_table ? p.block_table + (int64_t) b * p.bt_stride : nullptr;
     // uniform scalars, forced into SGPRs
