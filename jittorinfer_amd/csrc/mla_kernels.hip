@@ -470,17 +470,32 @@ __global__ void __launch_bounds__(256) mla_attn_combine_f32_kernel(const KParams
     const float2 * ml = (const float2 *) p.part_ml + (int64_t) b * p.n_splits * p.n_rows + row;
     const float *  po = (const float *) p.part_o + ((int64_t) b * p.n_splits * p.n_rows + row) * p.dv_total + cg * 4;
     const int64_t ml_step = p.n_rows, po_step = (int64_t) p.n_rows * p.dv_total;
-    float M = -INFINITY;
-    for (int c = 0; c < nvalid; c++) M = fmaxf(M, ml[c * ml_step].x);
-    float L = 0.f;
+    float M = -INFINITY, L = 0.f;
     f32x4 o = { 0.f, 0.f, 0.f, 0.f };
-    for (int c = 0; c < nvalid; c++) {
-        const float2 v = ml[c * ml_step];
-        if (v.x == -INFINITY) continue;   // that split saw only masked keys
-        const float w = v.y * fast_exp2(v.x - M);
-        const f32x4 x = *(const f32x4 *) (po + c * po_step);
-        L += w;
-        o.x += x.x * w; o.y += x.y * w; o.z += x.z * w; o.w += x.w * w;
+    for (int c0 = 0; c0 < nvalid; c0 += 8) {   // groups of 8 splits: their loads are in flight together
+        float2 mlv[8];
+        f32x4  xv[8];
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const int c = min(c0 + k, nvalid - 1);  // past the end: a duplicate of the last split, given weight 0 below
+            mlv[k] = ml[c * ml_step];
+            xv[k]  = *(const f32x4 *) (po + c * po_step);
+        }
+        float Mg = M;
+#pragma unroll
+        for (int k = 0; k < 8; k++) if (c0 + k < nvalid) Mg = fmaxf(Mg, mlv[k].x);
+        if (Mg == -INFINITY) continue;  // every split so far saw only masked keys
+        const float r = fast_exp2(M - Mg);  // 0 when M was -inf
+        M = Mg;
+        L *= r;
+        o.x *= r; o.y *= r; o.z *= r; o.w *= r;
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const float w = (c0 + k < nvalid && mlv[k].x != -INFINITY) ? mlv[k].y * fast_exp2(mlv[k].x - M) : 0.f;
+            L += w;
+            if (w == 0.f) continue;  // that split saw only masked keys (or is padding): its partial may hold anything
+            o.x += xv[k].x * w; o.y += xv[k].y * w; o.z += xv[k].z * w; o.w += xv[k].w * w;
+        }
     }
     const float inv = 1.0f / L;  // no valid key at all: 0 * inf = NaN, like the reference
     *(f32x4 *) (p.dst + ((int64_t) b * p.n_rows + row) * p.dst_stride + cg * 4) = f32x4{ o.x * inv, o.y * inv, o.z * inv, o.w * inv };
