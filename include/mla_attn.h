@@ -37,6 +37,9 @@ extern "C" {
 /* flags */
 #define MLA_FLAG_F16_ACC_STRICT 1u /* F16 KV only: replay ggml-cpu's per-key f16 accumulator (ggml-cpu.c:12066-12080)
                                       instead of accumulating in f32; sequential over keys, a correctness mode */
+#define MLA_FLAG_UNIFORM_SPLITS 2u /* paged decode: give every sequence the same number of equal KV splits (sized for the longest
+                                      sequence the block table can hold) instead of the balanced schedule that deals equal
+                                      runs of the batch's whole page list to the workgroups; for comparing the two */
 
 /* errors */
 #define MLA_ERR_BAD_SHAPE     (-1)
@@ -110,6 +113,9 @@ typedef struct mla_attn_plan_info {
     int32_t split_tokens; /* tokens per split */
     int32_t n_passes;     /* passes over d (2 for dv = 576) */
     int64_t lds_bytes;
+    int32_t balanced;     /* 1 = paged decode with the balanced schedule: n_workgroups workgroups take equal runs of the batch's
+                             page list (n_splits / split_tokens then describe the uniform plan it replaces) */
+    int32_t n_workgroups;
 } mla_attn_plan_info;
 
 size_t mla_attn_workspace_size(const mla_attn_args * args);

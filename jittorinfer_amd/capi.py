@@ -6,6 +6,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 
 MLA_TYPE_F32, MLA_TYPE_F16, MLA_TYPE_Q8_0, MLA_TYPE_BF16 = 0, 1, 8, 30
 MLA_FLAG_F16_ACC_STRICT = 1
+MLA_FLAG_UNIFORM_SPLITS = 2
 PAGE_TOKENS = 128
 ROW_BYTES = {MLA_TYPE_F16: 1152, MLA_TYPE_BF16: 1152, MLA_TYPE_Q8_0: 612}
 
@@ -27,7 +28,8 @@ class MlaAttnArgs(C.Structure):
 
 class MlaPlanInfo(C.Structure):
     _fields_ = [("variant", C.c_int32), ("rows_per_wg", C.c_int32), ("n_row_blocks", C.c_int32), ("n_splits", C.c_int32),
-                ("split_tokens", C.c_int32), ("n_passes", C.c_int32), ("lds_bytes", C.c_int64)]
+                ("split_tokens", C.c_int32), ("n_passes", C.c_int32), ("lds_bytes", C.c_int64), ("balanced", C.c_int32),
+                ("n_workgroups", C.c_int32)]
 
 
 def library_path():

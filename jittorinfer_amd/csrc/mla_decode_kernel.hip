@@ -21,7 +21,9 @@ namespace {
 // LDS: 4 resident 16-bit tiles (bf16 / f16 KV), or 3 of them behind 2 raw Q8_0 tiles; then the hand-off area,
 // 32 bytes per thread: mask offset, out pointer, (m,l) pointer, debug pointer
 constexpr int handoff_off(int kvt) { return kvt == SRC_Q8 ? 3 * TILE_BYTES + 2 * Q8_TILE_RAW : 4 * TILE_BYTES; }
-constexpr int lds_total(int kvt) { return handoff_off(kvt) + NTHREADS * 32; }
+constexpr int SCHED_MAX_SEQ = 256;                   // balanced schedule: sequences per launch
+constexpr int sched_off(int kvt) { return handoff_off(kvt) + NTHREADS * 32; }   // prefix sums of the sequences' tile counts
+constexpr int lds_total(int kvt) { return sched_off(kvt) + (2 * SCHED_MAX_SEQ + 8) * 4; }   // prefix sums, then the lengths
 
 #define MLA_DECODE_CLOBBERS \
     "memory", "vcc", "scc", "s40", "s41", "s42", "s43", "s44", "s45", "s46", "s47", "s48", "s49", "s50", "s51", \
@@ -67,6 +69,50 @@ constexpr int lds_total(int kvt) { return handoff_off(kvt) + NTHREADS * 32; }
     [nb1] "s"(s_nb1), [flg] "s"(s_flg), [ntl] "s"(s_ntl), [ostr] "s"(s_ostr), [qp] "s"(qpack), [msk] "s"(mask_base),  \
     [scl] "s"(s_scale), [pg0] "s"(s_pg0), [tid] "v"(tid)
 
+// Balanced schedule: p.sched[b] = number of 128-token pages of the sequences before b, p.sched[n_seq] = all pages; and
+// p.wg_first[8 v ..] = the first piece of workgroup v, ready to run: {sequence, kv_begin, kv_end, id of its first page,
+// whole sequence?, page-list position after it, end of the run, sequence length}; kv_begin >= kv_end: no work.
+// Computed once per call by the first block of the Q pre-pack kernel (every thread of its 256 calls this); the decode
+// workgroups and the combine pass read it.  n_seq <= SCHED_MAX_SEQ, p.n_wg <= 256.
+__device__ __forceinline__ void sched_prefix(const KParams & p) {
+    __shared__ int wave_total[4];
+    __shared__ int pre[SCHED_MAX_SEQ + 1];
+    const int t = threadIdx.x, lane = t & 63;
+    int v = 0;
+    if (t < p.n_seq_sched) v = (max(min(p.seq_lens[t], (int) p.bt_stride * MLA_PAGE_TOKENS), 0) + MLA_PAGE_TOKENS - 1) / MLA_PAGE_TOKENS;
+    for (int d = 1; d < 64; d <<= 1) {   // inclusive scan inside the wave
+        const int up = __shfl_up(v, d, 64);
+        if (lane >= d) v += up;
+    }
+    if (lane == 63) wave_total[t >> 6] = v;
+    __syncthreads();
+    for (int w = 0; w < (t >> 6); w++) v += wave_total[w];
+    pre[t + 1] = v;
+    if (t == 0) pre[0] = 0;
+    if (t < p.n_seq_sched) p.sched[t + 1] = v;
+    if (t == 0) p.sched[0] = 0;
+    __syncthreads();
+    if (t >= p.n_wg) return;
+    const int total = pre[p.n_seq_sched], quota = (total + p.n_wg - 1) / p.n_wg;
+    int pos = min(t * quota, total);
+    const int end = min(pos + quota, total);
+    int hdr[8] = { 0, 0, 0, 0, 0, end, end, 0 };
+    if (pos < end) {
+        int lo = 0, hi = p.n_seq_sched - 1;   // the sequence that holds page `pos`: the last b with pre[b] <= pos that has pages
+        while (lo < hi) { const int mid = (lo + hi + 1) >> 1; if (pre[mid] <= pos) lo = mid; else hi = mid - 1; }
+        const int b = lo, first = pre[b], piece_end = min(pre[b + 1], end);
+        const int len = min(p.seq_lens[b], (int) p.bt_stride * MLA_PAGE_TOKENS);
+        hdr[0] = b;
+        hdr[1] = (pos - first) * MLA_PAGE_TOKENS;
+        hdr[2] = min(len, (piece_end - first) * MLA_PAGE_TOKENS);
+        hdr[3] = min(max(p.block_table[(int64_t) b * p.bt_stride + (pos - first)], 0), p.n_pool_pages - 1);
+        hdr[4] = pos == first && piece_end == pre[b + 1];
+        hdr[5] = piece_end;
+        hdr[7] = len;
+    }
+    for (int i = 0; i < 8; i++) p.wg_first[8 * t + i] = hdr[i];
+}
+
 // The wave-level program is generated by gen_decode_asm.py (register map, LDS-DMA issue, MFMA/VALU interleave).
 // KVT = SRC_BF16: bf16 KV rows, bf16 MFMA, P fed as hi + lo halves.   SRC_F16: f16 KV rows, f16 MFMA, single P.
 // SRC_Q8: packed Q8_0 rows (612 bytes, contiguous), dequantized in LDS to f16 tiles one tile ahead, then as SRC_F16.
@@ -80,8 +126,9 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
     static_assert(!(KVT == SRC_Q8 && MASK), "no masked Q8_0 build of the wave program");
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int g = lane >> 5, rl = lane & 31;
+    // (wave and lane are taken from a scalar and from the exec-mask count rather than kept in a vector register: the wave
+    // program clobbers every VGPR, and the balanced schedule runs it more than once)
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     // Workgroups are handed to the 8 XCDs round-robin in dispatch order, and each XCD has its own L2.  The splits of one
     // (sequence, row block) all read the same 147 KB Q operand image, so the dispatch index is remapped to put them on one
     // XCD: index i runs on XCD i % 8, and the i / 8-th workgroup of that XCD takes the tuple number (i % 8) * G / 8 + i / 8.
@@ -94,15 +141,63 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
             bx = v % gridDim.x; by = (v / gridDim.x) % gridDim.y; bz = v / (gridDim.x * gridDim.y);
         }
     }
-    const int b = bz, split = bx;
 
-    const int seq_len  = p.block_table ? min(p.seq_lens[b], (int) p.bt_stride * MLA_PAGE_TOKENS) : (int) p.n_kv;
-    int kv_begin = split * p.split_tokens;
-    int kv_end   = min(seq_len, kv_begin + p.split_tokens);
+    // Balanced schedule (p.balanced; a ragged decode batch): the pages of all sequences form one list, every workgroup
+    // takes an equal run of it (grid = (n_wg, 1, 1), bx = its place), and a run that crosses a sequence boundary is worked
+    // off piece by piece.  Piece of workgroup v in sequence b -> partial slot v + b: the slots of one sequence are
+    // consecutive, which is all the combine pass needs to know.
+    int * sched = (int *) (smem + sched_off(KVT));   // [0 .. n_seq]: pages before sequence b; [n_seq]: all pages; then the lengths
+    int run_pos = 0, run_end = 0, run_seq = 0;
+    int first_piece[8] = { 0, 0, 0, 0, 0, 0, 0, 0 };
+    if (p.balanced) {
+        // the first piece comes ready-made from the pre-pass; the page prefix sums and the lengths are only needed for
+        // what may follow it and are fetched into LDS meanwhile (made visible by the barrier between pieces)
+        for (int i = 0; i < 8; i++) first_piece[i] = __builtin_amdgcn_readfirstlane(p.wg_first[8 * bx + i]);
+        if (first_piece[1] >= first_piece[2]) return;
+        for (int i = threadIdx.x; i <= p.n_seq_sched; i += NTHREADS) {
+            sched[i] = p.sched[i];
+            if (i < p.n_seq_sched) sched[SCHED_MAX_SEQ + 8 + i] = p.seq_lens[i];
+        }
+        run_pos = first_piece[5]; run_end = first_piece[6]; run_seq = first_piece[0] + 1;
+    }
+
+  for (int piece = 0;; piece++) {
+    int lane;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane));
+    const int tid = wave * 64 + lane, g = lane >> 5, rl = lane & 31;
+    int b = bz, split = bx, slot = 0;
+    int seq_len, kv_begin, kv_end;
+    bool direct = p.n_splits == 1;   // this piece is the whole sequence: final rows go to dst, there is nothing to combine
+    int pg0_ready = -1;
+    if (p.balanced && piece == 0) {
+        b = first_piece[0]; kv_begin = first_piece[1]; kv_end = first_piece[2]; pg0_ready = first_piece[3];
+        direct = first_piece[4] != 0; seq_len = first_piece[7];
+        slot = bx + b; split = 1;
+    } else if (p.balanced) {
+        __syncthreads();   // every wave is through with the tile buffers and the hand-off records of the piece before
+        run_pos = __builtin_amdgcn_readfirstlane(run_pos); run_seq = __builtin_amdgcn_readfirstlane(run_seq);
+        while (run_pos < run_end && sched[run_seq + 1] <= run_pos) run_seq++;   // sequences without pages
+        if (run_pos >= run_end) return;
+        b = run_seq;
+        seq_len = min(sched[SCHED_MAX_SEQ + 8 + b], (int) p.bt_stride * MLA_PAGE_TOKENS);
+        const int first = sched[b], piece_end = min(sched[b + 1], run_end);
+        kv_begin = (run_pos - first) * MLA_PAGE_TOKENS;
+        kv_end   = min(seq_len, (piece_end - first) * MLA_PAGE_TOKENS);
+        slot     = bx + b;
+        direct   = run_pos == first && piece_end == sched[b + 1];
+        split    = 1;   // not the first split of anything: an empty piece writes nothing
+        run_pos  = piece_end;
+        run_seq  = b + 1;
+    } else {
+        seq_len  = p.block_table ? min(p.seq_lens[b], (int) p.bt_stride * MLA_PAGE_TOKENS) : (int) p.n_kv;
+        kv_begin = split * p.split_tokens;
+        kv_end   = min(seq_len, kv_begin + p.split_tokens);
+        slot     = b * p.n_splits + split;
+    }
     const int row       = by * 128 + wave * 32 + rl;
     const bool row_valid = row < p.n_rows;
     const int64_t orow  = (int64_t) b * p.n_rows + row;
-    const int64_t prow  = ((int64_t) b * p.n_splits + split) * p.n_rows + row;
+    const int64_t prow  = (int64_t) slot * p.n_rows + row;
 
     bool all_masked = false;  // this split holds keys, but none that a row of this block may attend to
     if constexpr (MASK) {
@@ -134,18 +229,19 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
                 p.part_ml[prow * 2 + 1] = 0.f;
             }
         }
+        if (p.balanced) continue;
         return;
     }
     const int n_tiles = (kv_end - kv_begin + TILE_TOK - 1) / TILE_TOK;
 
     // per-thread pointers for the wave program, handed over through LDS
     // final output: row-major dst rows.  split-K partial: [column/8][row][8] inside this (sequence, split) block.
-    const int64_t pblock = ((int64_t) b * p.n_splits + split) * p.n_rows * p.dv_total;  // in f16 elements
+    const int64_t pblock = (int64_t) slot * p.n_rows * p.dv_total;  // in f16 elements
     // (f32 partials are rows of dv_total floats: the wave program stores them the way it stores final output rows)
-    void * optr = row_valid ? (p.n_splits == 1 ? (void *) (p.dst + orow * p.dst_stride + 4 * g)
+    void * optr = row_valid ? (direct ? (void *) (p.dst + orow * p.dst_stride + 4 * g)
                                : p.part_f32    ? (void *) ((float *) p.part_o + prow * p.dv_total + 4 * g)
                                                : (void *) (p.part_o + pblock + (int64_t) row * 8 + 4 * g)) : nullptr;
-    float * mlptr = (p.n_splits > 1 && g == 0 && row_valid) ? p.part_ml + prow * 2 : nullptr;
+    float * mlptr = (!direct && g == 0 && row_valid) ? p.part_ml + prow * 2 : nullptr;
     {
         unsigned long long * h = (unsigned long long *) (smem + HANDOFF_OFF + tid * 32);
         // mask builds: byte offset of this lane's first mask element (its query token's row, tokens 4g.. of a tile)
@@ -164,11 +260,12 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
     const int s_kve  = __builtin_amdgcn_readfirstlane(kv_end);
     const int s_npp  = __builtin_amdgcn_readfirstlane(p.n_pool_pages - 1);
     const int s_nb1  = __builtin_amdgcn_readfirstlane((int) p.kv_nb1);
-    const int s_flg  = __builtin_amdgcn_readfirstlane((p.n_splits == 1 || p.part_f32 ? 1 : 0) | p.debug_flags);  // bit 0: f32 row store
+    const int s_flg  = __builtin_amdgcn_readfirstlane((direct || p.part_f32 ? 1 : 0) | p.debug_flags);  // bit 0: f32 row store
     const int s_ntl  = __builtin_amdgcn_readfirstlane(n_tiles);
     // id of the split's first page as a scalar: the first tiles are requested before the vector load of all page ids is back
     int pg0 = 0;
-    if (bt_row) pg0 = min(max(bt_row[min((int64_t) (kv_begin >> 7), p.bt_stride - 1)], 0), p.n_pool_pages - 1);
+    if (pg0_ready >= 0) pg0 = pg0_ready;
+    else if (bt_row) pg0 = min(max(bt_row[min((int64_t) (kv_begin >> 7), p.bt_stride - 1)], 0), p.n_pool_pages - 1);
     const int s_pg0 = __builtin_amdgcn_readfirstlane(pg0);
     const char * mask_base = p.mask;
     const int s_scale = __builtin_amdgcn_readfirstlane(__float_as_int(p.scale));
@@ -195,6 +292,8 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
 #include "mla_decode_asm.inc"
             : : MLA_DECODE_INPUTS : MLA_DECODE_CLOBBERS);
     }
+    if (!p.balanced) return;
+  }
 }
 
 // Q f32 -> the decode kernel's MFMA operand image, rounded to the KV type as ggml-cpu rounds it (ggml-cpu.c:12034-12035):
@@ -203,6 +302,10 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
 // grid = (n_row_blocks, n_seq, 36 k-steps), block = 256: one 16-byte output per thread.
 template <bool F16>
 __global__ void __launch_bounds__(NTHREADS) mla_q_pack_kernel(const KParams p) {
+    if (blockIdx.z == gridDim.z - 1 && p.balanced) {   // balanced schedule: one extra layer of blocks, the first of which builds it
+        if (blockIdx.x == 0 && blockIdx.y == 0) sched_prefix(p);
+        return;
+    }
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int g = lane >> 5, rl = lane & 31;
     const int b = blockIdx.y, ks = blockIdx.z;
@@ -255,6 +358,10 @@ __global__ void __launch_bounds__(NTHREADS) mla_mask_extent_kernel(const KParams
 // d = amax/127 (stored as f16), id = 127/amax, q = round-half-even(x*id) (ggml-cpu-quants.c:855-900); the MFMA operand is the
 // dequantized value q * f16(d), rounded to f16.  grid = (n_row_blocks, n_seq, 18 blocks), block = 256: two k-steps per thread.
 __global__ void __launch_bounds__(NTHREADS) mla_q_pack_q8_kernel(const KParams p) {
+    if (blockIdx.z == gridDim.z - 1 && p.balanced) {   // balanced schedule: one extra layer of blocks, the first of which builds it
+        if (blockIdx.x == 0 && blockIdx.y == 0) sched_prefix(p);
+        return;
+    }
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int g = lane >> 5, rl = lane & 31;
     const int b = blockIdx.y, j = blockIdx.z;
@@ -327,12 +434,14 @@ static hipError_t launch_variant(const KParams & kp, dim3 grid, hipStream_t st) 
 }
 
 hipError_t launch_decode_fast(const KParams & kp, int kv_type, dim3 grid, hipStream_t st, bool with_prepass) {
+    // the small passes ahead of the kernel run per (row block, sequence), whatever the kernel's own grid is
+    const unsigned n_rb = (unsigned) ((kp.n_rows + 127) / 128), n_seq = (unsigned) kp.n_seq_sched, extra = kp.balanced ? 1 : 0;
     const bool m = kp.mask != nullptr;
     if (!with_prepass) { /* the workspace still holds the Q image and the mask extents of an earlier launch of the same call */ }
-    else if (kv_type == MLA_TYPE_Q8_0)     hipLaunchKernelGGL(mla_q_pack_q8_kernel, dim3(grid.y, grid.z, KSTEPS / 2), dim3(NTHREADS), 0, st, kp);
-    else if (kv_type == MLA_TYPE_F16) hipLaunchKernelGGL(mla_q_pack_kernel<true>, dim3(grid.y, grid.z, KSTEPS), dim3(NTHREADS), 0, st, kp);
-    else                              hipLaunchKernelGGL(mla_q_pack_kernel<false>, dim3(grid.y, grid.z, KSTEPS), dim3(NTHREADS), 0, st, kp);
-    if (m && with_prepass) hipLaunchKernelGGL(mla_mask_extent_kernel, dim3(grid.y, MASK_EXT_CHUNKS), dim3(NTHREADS), 0, st, kp);
+    else if (kv_type == MLA_TYPE_Q8_0)     hipLaunchKernelGGL(mla_q_pack_q8_kernel, dim3(n_rb, n_seq, KSTEPS / 2 + extra), dim3(NTHREADS), 0, st, kp);
+    else if (kv_type == MLA_TYPE_F16) hipLaunchKernelGGL(mla_q_pack_kernel<true>, dim3(n_rb, n_seq, KSTEPS + extra), dim3(NTHREADS), 0, st, kp);
+    else                              hipLaunchKernelGGL(mla_q_pack_kernel<false>, dim3(n_rb, n_seq, KSTEPS + extra), dim3(NTHREADS), 0, st, kp);
+    if (m && with_prepass) hipLaunchKernelGGL(mla_mask_extent_kernel, dim3(n_rb, MASK_EXT_CHUNKS), dim3(NTHREADS), 0, st, kp);
     if (kv_type == MLA_TYPE_Q8_0) return launch_variant<SRC_Q8, false>(kp, grid, st);
     if (kv_type == MLA_TYPE_F16)  return m ? launch_variant<SRC_F16, true>(kp, grid, st) : launch_variant<SRC_F16, false>(kp, grid, st);
     return m ? launch_variant<SRC_BF16, true>(kp, grid, st) : launch_variant<SRC_BF16, false>(kp, grid, st);

@@ -398,6 +398,25 @@ __global__ void __launch_bounds__(NTHREADS) mla_attn_tile_kernel(const KParams p
     }
 }
 
+// Where the partials of sequence b sit: uniform splits -> slots b*n_splits .. +nvalid; balanced schedule -> the
+// workgroups whose runs of the page list touch the sequence, slot = workgroup + b (see mla_decode_kernel).
+__device__ __forceinline__ void partial_slots(const KParams & p, int b, int seq_len, int & slot0, int & nvalid) {
+    if (!p.balanced) {
+        nvalid = (seq_len + p.split_tokens - 1) / p.split_tokens;
+        nvalid = p.rel_splits ? p.n_splits : min(nvalid, p.n_splits);
+        slot0  = b * p.n_splits;
+        return;
+    }
+    const int before = p.sched[b], total = p.sched[p.n_seq_sched];   // pages of the sequences before b / of all sequences
+    const int mine  = (max(seq_len, 0) + MLA_PAGE_TOKENS - 1) / MLA_PAGE_TOKENS;
+    const int quota = (total + p.n_wg - 1) / p.n_wg;
+    if (mine == 0) { slot0 = 0; nvalid = 0; return; }
+    const int w0 = before / quota, w1 = (before + mine - 1) / quota;
+    slot0  = w0 + b;
+    nvalid = w1 - w0 + 1;
+    if (nvalid == 1) nvalid = -1;   // one workgroup had the whole sequence and wrote the final rows itself
+}
+
 // Log-sum-exp merge of the split-K partials: out = sum_c (O_c/l_c) l_c 2^(m_c - M) / sum_c l_c 2^(m_c - M).
 // Partials hold O_c/l_c as f16, laid out [seq][split][column/8][row][8].  One thread = one (row, group of 8 columns):
 // 16-byte loads, lanes along rows (contiguous in the partial layout), splits in groups of 8 so that all the loads of a
@@ -406,13 +425,13 @@ __global__ void __launch_bounds__(256) mla_attn_combine_kernel(const KParams p) 
     const int b = blockIdx.z;
     const int row = blockIdx.x * 32 + (threadIdx.x & 31);
     const int cg  = blockIdx.y * 8 + (threadIdx.x >> 5);
-    if (row >= p.n_rows || cg * 8 >= p.dv_total) return;
     const int seq_len = p.block_table ? min(p.seq_lens[b], (int) p.bt_stride * MLA_PAGE_TOKENS) : (int) p.n_kv;
-    int nvalid = (seq_len + p.split_tokens - 1) / p.split_tokens;
-    nvalid = p.rel_splits ? p.n_splits : min(nvalid, p.n_splits);
+    int slot0, nvalid;
+    partial_slots(p, b, seq_len, slot0, nvalid);
+    if (nvalid < 0 || row >= p.n_rows || cg * 8 >= p.dv_total) return;
 
-    const float2 *   ml = (const float2 *) p.part_ml + (int64_t) b * p.n_splits * p.n_rows + row;
-    const _Float16 * po = p.part_o + (int64_t) b * p.n_splits * p.n_rows * p.dv_total + ((int64_t) cg * p.n_rows + row) * 8;
+    const float2 *   ml = (const float2 *) p.part_ml + (int64_t) slot0 * p.n_rows + row;
+    const _Float16 * po = p.part_o + (int64_t) slot0 * p.n_rows * p.dv_total + ((int64_t) cg * p.n_rows + row) * 8;
     const int64_t ml_step = p.n_rows, po_step = (int64_t) p.n_rows * p.dv_total;
 
     float M = -INFINITY, L = 0.f;
@@ -463,12 +482,12 @@ __global__ void __launch_bounds__(256) mla_attn_combine_f32_kernel(const KParams
     const int rows_per_block = 256 / groups_per_row;
     const int row = blockIdx.x * rows_per_block + threadIdx.x / groups_per_row;
     const int cg  = threadIdx.x % groups_per_row;
-    if (row >= p.n_rows || threadIdx.x >= rows_per_block * groups_per_row || cg * 4 >= p.dv_total) return;
     const int seq_len = p.block_table ? min(p.seq_lens[b], (int) p.bt_stride * MLA_PAGE_TOKENS) : (int) p.n_kv;
-    int nvalid = (seq_len + p.split_tokens - 1) / p.split_tokens;
-    nvalid = p.rel_splits ? p.n_splits : min(nvalid, p.n_splits);
-    const float2 * ml = (const float2 *) p.part_ml + (int64_t) b * p.n_splits * p.n_rows + row;
-    const float *  po = (const float *) p.part_o + ((int64_t) b * p.n_splits * p.n_rows + row) * p.dv_total + cg * 4;
+    int slot0, nvalid;
+    partial_slots(p, b, seq_len, slot0, nvalid);
+    if (nvalid < 0 || row >= p.n_rows || threadIdx.x >= rows_per_block * groups_per_row || cg * 4 >= p.dv_total) return;
+    const float2 * ml = (const float2 *) p.part_ml + (int64_t) slot0 * p.n_rows + row;
+    const float *  po = (const float *) p.part_o + ((int64_t) slot0 * p.n_rows + row) * p.dv_total + cg * 4;
     const int64_t ml_step = p.n_rows, po_step = (int64_t) p.n_rows * p.dv_total;
     float M = -INFINITY, L = 0.f;
     f32x4 o = { 0.f, 0.f, 0.f, 0.f };
@@ -581,8 +600,9 @@ struct Plan {
     int    n_splits, split_tokens;
     int    n_passes, ndb;
     size_t lds_bytes;
-    size_t ws_part_o, ws_part_ml, ws_scores, ws_qpack, ws_maskext;
+    size_t ws_part_o, ws_part_ml, ws_scores, ws_qpack, ws_maskext, ws_sched;
     int    part_f32;
+    int    balanced, n_wg;   // balanced schedule of the pipelined kernel (ragged paged decode)
 };
 
 int validate(const mla_attn_args * a) {
@@ -662,20 +682,28 @@ int make_plan(const mla_attn_args * a, Plan * pl) {
     pl->lds_bytes    = pl->variant == 2 ? decode_fast_lds_bytes(a->kv_type) : 2 * TILE_BYTES + (a->kv_type == MLA_TYPE_Q8_0 ? Q8_TILE_RAW : 0);
     if (pl->variant == 2) pl->ws_qpack = decode_fast_qpack_bytes(a->n_seq, pl->n_row_blocks);
     if (pl->variant == 2 && a->mask) pl->ws_maskext = (size_t) pl->n_row_blocks * 16 * 2 * sizeof(int);  // 16 (first, last) pairs per row block
+    // A paged decode batch (one row block per sequence, no mask) that needs KV splits anyway: the pipelined kernel's
+    // workgroups take equal runs of the page list of all sequences instead of equal shares of the longest possible
+    // sequence, so a ragged batch keeps every CU busy.  One workgroup per CU; a run must fit the 64 page ids a wave holds.
+    if (pl->variant == 2 && a->block_table && !a->mask && pl->n_row_blocks == 1 && a->n_splits == 0 && pl->n_splits > 1 &&
+        a->n_seq <= 256 && !(a->flags & MLA_FLAG_UNIFORM_SPLITS)) {
+        if (((int64_t) a->n_seq * n_pages + 255) / 256 <= 64) { pl->balanced = 1; pl->n_wg = 256; pl->ws_sched = (size_t) (a->n_seq + 1 + 63) / 64 * 64 * sizeof(int) + (size_t) pl->n_wg * 8 * sizeof(int); }
+    }
     if (pl->n_splits > 1) {
         // f32 partials while they are small (no second rounding of O on top of the MFMA operands' one), f16 beyond: there the
         // partial traffic counts, and the rounding (2^-12 relative per split) is averaged over long contexts
-        const size_t n_part = (size_t) a->n_seq * pl->n_splits * n_rows * a->dv;
+        const size_t n_slots = pl->balanced ? (size_t) pl->n_wg + a->n_seq : (size_t) a->n_seq * pl->n_splits;
+        const size_t n_part = n_slots * n_rows * a->dv;
         pl->part_f32   = n_part * sizeof(float) <= ((size_t) 32 << 20);
         pl->ws_part_o  = n_part * (pl->part_f32 ? sizeof(float) : sizeof(_Float16));
-        pl->ws_part_ml = (size_t) a->n_seq * pl->n_splits * n_rows * 2 * sizeof(float);
+        pl->ws_part_ml = n_slots * n_rows * 2 * sizeof(float);
     }
     return 0;
 }
 
 size_t align256(size_t x) { return (x + 255) & ~(size_t) 255; }
 size_t plan_ws(const Plan & pl) {
-    return align256(pl.ws_part_o) + align256(pl.ws_part_ml) + align256(pl.ws_scores) + align256(pl.ws_qpack) + align256(pl.ws_maskext);
+    return align256(pl.ws_part_o) + align256(pl.ws_part_ml) + align256(pl.ws_scores) + align256(pl.ws_qpack) + align256(pl.ws_maskext) + align256(pl.ws_sched);
 }
 
 template <int SRC, int NDB, int WM, int WD>
@@ -716,6 +744,7 @@ int mla_attn_plan(const mla_attn_args * args, mla_attn_plan_info * out) {
     const int rc = make_plan(args, &pl);
     if (rc) return rc;
     if (!out) return MLA_ERR_NULL;
+    const int a_n_seq = args->n_seq;
     out->variant      = pl.variant;
     out->rows_per_wg  = pl.rblk;
     out->n_row_blocks = pl.n_row_blocks;
@@ -723,6 +752,8 @@ int mla_attn_plan(const mla_attn_args * args, mla_attn_plan_info * out) {
     out->split_tokens = pl.split_tokens;
     out->n_passes     = pl.n_passes;
     out->lds_bytes    = (int64_t) pl.lds_bytes;
+    out->balanced     = pl.balanced;
+    out->n_workgroups = pl.balanced ? pl.n_wg : pl.n_splits * pl.n_row_blocks * a_n_seq;
     return 0;
 }
 
@@ -757,10 +788,13 @@ static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
     kp.part_o  = (_Float16 *) ws;
     kp.part_f32 = pl.part_f32;
     kp.rel_splits = pl.variant == 2 && a->mask != nullptr;
+    kp.balanced = pl.balanced; kp.n_wg = pl.n_wg; kp.n_seq_sched = a->n_seq;
     kp.part_ml = (float *) (ws + align256(pl.ws_part_o));
     float * scores = (float *) (ws + align256(pl.ws_part_o) + align256(pl.ws_part_ml));
     kp.q_pack = ws + align256(pl.ws_part_o) + align256(pl.ws_part_ml) + align256(pl.ws_scores);
     kp.mask_ext = (int *) (ws + align256(pl.ws_part_o) + align256(pl.ws_part_ml) + align256(pl.ws_scores) + align256(pl.ws_qpack));
+    kp.sched = (int *) (ws + align256(pl.ws_part_o) + align256(pl.ws_part_ml) + align256(pl.ws_scores) + align256(pl.ws_qpack) + align256(pl.ws_maskext));
+    kp.wg_first = kp.sched + (a->n_seq + 1 + 63) / 64 * 64;
 
     if (pl.variant == 1) {
         if (!(phases & 1)) return 0;
@@ -776,6 +810,7 @@ static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
     }
 
     dim3 grid((unsigned) pl.n_splits, (unsigned) pl.n_row_blocks, (unsigned) a->n_seq);
+    if (pl.balanced) grid = dim3((unsigned) pl.n_wg, 1, 1);
     for (int pass = 0; pass < pl.n_passes && (phases & 1); pass++) {
         kp.d_off = pass * pl.ndb * 32;
         hipError_t e;

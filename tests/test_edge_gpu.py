@@ -220,3 +220,61 @@ def test_reference_style_batched_decode_through_the_mask(gpu, k_type, n_splits):
     else:
         want = O.flash_attn_ext(q, k, k_type, dv=512, mask=mask, scale=U.SCALE)
     print(U.check(got[..., :512], want, "batched decode through the mask"))
+
+
+def _run_flags(gpu, q, pool, k_type, bt, lens, flags):
+    import torch
+    import jittorinfer_amd as J
+    tq = torch.from_numpy(q).to(gpu)
+    tk = torch.from_numpy(pool.view(np.int16) if pool.dtype == np.uint16 else pool).to(gpu)
+    tb, tl = torch.from_numpy(bt).to(gpu), torch.from_numpy(np.asarray(lens, dtype=np.int32)).to(gpu)
+    out = torch.full((q.shape[0], q.shape[2], q.shape[1], 576), float("nan"), dtype=torch.float32, device=gpu)
+    info = J.plan(tq, tk, k_type, dv=512, scale=U.SCALE, block_table=tb, seq_lens=tl, out=out, flags=flags)
+    J.ggml_flash_attn_ext(tq, tk, k_type, dv=512, scale=U.SCALE, block_table=tb, seq_lens=tl, out=out, flags=flags)
+    torch.cuda.synchronize()
+    return out.cpu().numpy()[..., :512], info
+
+
+@pytest.mark.parametrize("k_type", [O.TYPE_BF16, O.TYPE_Q8_0])
+@pytest.mark.parametrize("shape", ["many_short", "few_long_many_short", "one_sequence", "with_empties"])
+def test_balanced_schedule_of_ragged_decode_batches(gpu, k_type, shape):
+    """The pipelined kernel's balanced schedule (equal runs of the batch's page list per workgroup, pieces of several
+    sequences inside one workgroup, whole-sequence pieces written without the combine pass) against the oracle and
+    against the uniform-split plan of the same call."""
+    import jittorinfer_amd as J
+    rng = np.random.default_rng({"many_short": 1, "few_long_many_short": 2, "one_sequence": 3, "with_empties": 4}[shape])
+    if shape == "many_short":
+        lens = [int(x) for x in rng.integers(1, 3 * 128, size=150)]          # ~300 pages: runs of 2 pages cross sequence ends
+    elif shape == "few_long_many_short":
+        lens = [4000, 3777] + [int(x) for x in rng.integers(1, 200, size=40)]
+    elif shape == "one_sequence":
+        lens = [5000]
+    else:
+        lens = [0, 0, 700, 0, 129, 0, 0, 1, 128, 0]
+    # Q8_0 pages as BASELINE's config 5 builds them (one power-of-two scale): with arbitrary block scales a lone key's
+    # V value rounded to the f16 MFMA operand alone costs up to 2^-11 |v| = 2.2e-3 at |v| = 4.5, whatever the schedule
+    pool, bt, seqs = U.make_paged(rng, np.maximum(lens, 1), k_type, q8_scale=1.0 / 32 if k_type == O.TYPE_Q8_0 else None)
+    seqs = [s[:l] for s, l in zip(seqs, lens)]
+    q = rng.standard_normal((len(lens), 32, 1, 576)).astype(np.float32)
+    got, info = _run_flags(gpu, q, pool, k_type, bt, lens, 0)
+    assert info["variant"] == 2 and info["balanced"] == 1 and info["n_workgroups"] == 256
+    uni, info_u = _run_flags(gpu, q, pool, k_type, bt, lens, J.MLA_FLAG_UNIFORM_SPLITS)
+    assert info_u["balanced"] == 0
+    want = _want(q, seqs, k_type)
+    print(U.check(got, want, "balanced schedule"), U.check(uni, want, "uniform splits"))
+
+
+def test_balanced_schedule_limits(gpu):
+    """A batch that already fills the GPU with one workgroup per sequence (nothing to split), or a block table so wide that
+    a workgroup's run could exceed the 64 pages a wave indexes, keeps the uniform plan."""
+    import torch
+    import jittorinfer_amd as J
+    q = torch.zeros((257, 16, 1, 576), device=gpu)
+    pool = torch.zeros((128 * 4, 576), dtype=torch.int16, device=gpu)
+    bt = torch.zeros((257, 4), dtype=torch.int32, device=gpu)
+    sl = torch.ones(257, dtype=torch.int32, device=gpu)
+    assert J.plan(q[:256], pool, J.MLA_TYPE_BF16, dv=512, scale=1.0, block_table=bt[:256], seq_lens=sl[:256])["balanced"] == 0   # one split: nothing to balance
+    q8 = torch.zeros((8, 16, 1, 576), device=gpu)
+    assert J.plan(q8, pool, J.MLA_TYPE_BF16, dv=512, scale=1.0, block_table=bt[:8], seq_lens=sl[:8])["balanced"] == 1
+    wide = torch.zeros((8, 4096), dtype=torch.int32, device=gpu)
+    assert J.plan(q8, pool, J.MLA_TYPE_BF16, dv=512, scale=1.0, block_table=wide, seq_lens=sl[:8])["balanced"] == 0
