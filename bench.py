@@ -208,6 +208,82 @@ def front_config(a, dev, lib, J):
                       "roofline": roof, "cpu_baseline": cpu}))
 
 
+def layer_config(a, dev, lib, J):
+    """One decode step of one attention layer between the q / kv projections and wo, every node through the C ABI:
+    rope(q_pe) and the absorb product written straight into the 576-wide Q rows, rope(k_pe) in place, the cache write
+    through the block table, paged attention, the un-absorb product written straight into the [token, head*128] rows.
+    Config 3's shape (32 sequences, 128 heads, 8191 cached tokens + the new one); wkv_b and the KV pool of 4 layers are
+    rotated between steps."""
+    import torch
+    B, H, ctx, layers = a.batch, a.heads, a.ctx, a.pools
+    scale = 1.0 / (192.0 ** 0.5)
+    _, pools, bt, sl = build_workload(dev, B, H, ctx, layers, a.seed, "bf16")
+    g = torch.Generator(device=dev)
+    g.manual_seed(a.seed + 1)
+    wkv_b = (torch.randn((layers, H * 256 * 512), generator=g, device=dev, dtype=torch.float32) * 0.05).to(torch.bfloat16).view(torch.int16)
+    q = torch.randn((B, H, 192), generator=g, device=dev, dtype=torch.float32)
+    kv_new = torch.randn((B, 576), generator=g, device=dev, dtype=torch.float32) * 0.5
+    pos = torch.full((B,), ctx - 1, dtype=torch.int32, device=dev)
+    seq_ids = torch.arange(B, dtype=torch.int32, device=dev)
+    q_states = torch.empty((H, B, 576), dtype=torch.float32, device=dev)
+    attn_out = torch.empty((B, 1, H, 576), dtype=torch.float32, device=dev)
+    cur = torch.empty((B, H, 128), dtype=torch.float32, device=dev)
+    rope_kw = dict(n_dims=64, n_ctx_orig=4096, freq_scale=0.025, ext_factor=1.0, attn_factor=0.8)
+    k_pe = kv_new[:, 512:].unsqueeze(1)                                  # [B, 1, 64] inside the rows of 576
+    attn_args = []
+    for pool in pools:
+        ar, _, keep = J.capi.make_args(q_states.permute(1, 0, 2).unsqueeze(2), pool.view(torch.int16), J.MLA_TYPE_BF16, dv=512,
+                                       scale=scale, block_table=bt, seq_lens=sl, out=attn_out)
+        attn_args.append((ar, keep))
+
+    def step(i, st):
+        w = wkv_b[i % layers]
+        pool = pools[i % layers].view(torch.int16)
+        J.ggml_rope_ext(q[:, :, 128:], pos, out=q_states[:, :, 512:].permute(1, 0, 2), **rope_kw)
+        J.ggml_rope_ext(k_pe, pos, out=k_pe, **rope_kw)
+        J.ggml_mul_mat(w[:H * 512 * 128].view(H, 512, 128), J.MLA_TYPE_BF16, q[:, :, :128].permute(1, 0, 2), out=q_states[:, :, :512])
+        J.kv_write(kv_new, pool, J.MLA_TYPE_BF16, block_table=bt, seq_ids=seq_ids, positions=pos)
+        rc = lib.mla_attn_launch(C.byref(attn_args[i % layers][0]), st)
+        if rc != 0:
+            raise RuntimeError("launch failed: %d" % rc)
+        J.ggml_mul_mat(w[H * 512 * 128:].view(H, 128, 512), J.MLA_TYPE_BF16, attn_out[:, 0].permute(1, 0, 2)[:, :, :512], out=cur.permute(1, 0, 2))
+
+    stream = torch.cuda.current_stream(dev)
+    for i in range(a.warmup):
+        step(i, C.c_void_p(stream.cuda_stream))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(a.steps):
+        step(i, C.c_void_p(stream.cuda_stream))
+    torch.cuda.synchronize()
+    eager_ms = (time.perf_counter() - t0) * 1e3 / a.steps
+    side = torch.cuda.Stream(dev)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        graph.capture_begin()
+        for i in range(a.steps):
+            step(i, C.c_void_p(side.cuda_stream))
+        graph.capture_end()
+    torch.cuda.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    graph.replay()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / a.steps
+    kv_bytes = B * ctx * KV_ROW_BYTES
+    nbytes = kv_bytes + 2 * H * 512 * 128 * 2 + q.numel() * 4 + cur.numel() * 4
+    print(json.dumps({"metric": "mla_decode_layer_step_bandwidth", "value": nbytes / (ms * 1e-3) / 1e9, "unit": "GB/s", "n_gpus": 1,
+                      "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak",
+                      "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+                      "config": {"workload": "decode step of one MLA layer, q projection output to wo input: rope x2, absorb, cache write, paged attention (B=%d H=%d ctx=%d bf16), un-absorb; 8 kernel launches" % (B, H, ctx)},
+                      "us_per_step": ms * 1e3, "eager_us_per_step": eager_ms * 1e3, "launch": "hip graph replay of the K steps",
+                      "tokens_per_s": B / (ms * 1e-3),
+                      "roofline": {"bound": "hbm", "kernel": "whole step", "achieved": nbytes / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                                   "frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, "traffic": None, "algorithmic_bytes_per_launch": nbytes},
+                      "cpu_baseline": None}))
+
+
 def _timed(f):
     t0 = time.perf_counter()
     f()
@@ -368,7 +444,7 @@ def main():
     ap.add_argument("--kv", default="bf16", choices=["bf16", "f16", "q8_0"], help="storage type of the latent KV pool (the headline config is bf16; q8_0 only with --config kvwrite)")
     ap.add_argument("--uniform-splits", action="store_true", help="paged decode: equal KV splits per sequence (MLA_FLAG_UNIFORM_SPLITS) instead of the balanced schedule")
     ap.add_argument("--eager", action="store_true", help="time the K steps as K eager launch sequences instead of one replay of a HIP graph that holds them")
-    ap.add_argument("--config", default="c3", choices=["c2", "c3", "c3mask", "c4", "c5", "kvwrite", "rope", "absorb", "unabsorb"],
+    ap.add_argument("--config", default="c3", choices=["c2", "c3", "c3mask", "c4", "c5", "kvwrite", "rope", "absorb", "unabsorb", "layer"],
                     help="c3 (default) is the headline workload; the others time BASELINE's remaining GPU configs and the cache write for the profiles")
     a = ap.parse_args()
     if a.gpus != 1:
@@ -388,6 +464,9 @@ def main():
         return
     if a.config in ("rope", "absorb", "unabsorb"):
         front_config(a, dev, lib, J)
+        return
+    if a.config == "layer":
+        layer_config(a, dev, lib, J)
         return
     if a.config != "c3":
         other_config(a, dev, lib, J)
