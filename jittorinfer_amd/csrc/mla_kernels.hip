@@ -655,7 +655,7 @@ int make_plan(const mla_attn_args * a, Plan * pl) {
     else {
         pl->n_passes = 1; pl->ndb = 16;
         int rpw = a->rows_per_wg;
-        if (rpw == 0) rpw = n_rows > 64 ? 128 : n_rows > 32 ? 64 : 32;
+        if (rpw == 0) rpw = n_rows > 32 ? 64 : 32;   // 128 rows per workgroup (4 x 1 waves) spills: 2.3 times slower than 64 (2 x 2) at 128 heads
         if (rpw == 128)     { pl->wm = 4; pl->wd = 1; }
         else if (rpw == 64) { pl->wm = 2; pl->wd = 2; }
         else                { pl->wm = 1; pl->wd = 4; }
