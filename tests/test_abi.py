@@ -103,3 +103,47 @@ def test_argument_validation_without_gpu():
     assert lib.mla_attn_plan(C.byref(a), C.byref(info)) == 0
     assert lib.mla_attn_launch(C.byref(a), None) == -4           # split-K needs a workspace
     assert lib.ggml_backend_score() in (0, 100)
+
+
+def _plan(**kw):
+    """mla_attn_plan on made-up (never dereferenced) device addresses: the planner is host logic."""
+    import jittorinfer_amd as J
+    a = J.MlaAttnArgs()
+    a.q, a.kv, a.dst = 4096, 8192, 16384
+    a.n_seq, a.n_head, a.n_tok, a.dk, a.dv = 32, 128, 1, 576, 512
+    a.kv_type, a.q_type = J.MLA_TYPE_BF16, J.MLA_TYPE_F32
+    a.q_nb1 = a.q_nb2 = 2304
+    a.q_nb3 = 2304 * 128
+    a.kv_nb1, a.n_kv, a.dst_nb1, a.scale = 1152, 2048 * 128, 2304, 0.1
+    a.block_table, a.bt_stride, a.seq_lens = 32768, 64, 65536
+    for k, v in kw.items():
+        setattr(a, k, v)
+    info = J.MlaPlanInfo()
+    rc = _lib().mla_attn_plan(C.byref(a), C.byref(info))
+    return rc, info, _lib().mla_attn_workspace_size(C.byref(a))
+
+
+def test_planner_schedules_without_gpu():
+    """Which kernel and which split schedule the planner picks for the BASELINE shapes, and what the workspace holds."""
+    import jittorinfer_amd as J
+    rc, info, ws = _plan()                                       # config 3: 32 sequences x 64 pages
+    assert rc == 0 and info.variant == 2 and info.balanced == 1 and info.n_workgroups == 256
+    assert info.n_splits == 8 and info.split_tokens == 1024     # the uniform plan the balanced schedule replaces
+    slots = 256 + 32                                            # f16 partials, (m, l), Q image, schedule
+    assert ws >= slots * 128 * 512 * 2 + slots * 128 * 8 + 32 * 4 * 36 * 1024 + 33 * 4 + 256 * 32
+    rc, info, _ = _plan(flags=J.MLA_FLAG_UNIFORM_SPLITS)
+    assert rc == 0 and info.variant == 2 and info.balanced == 0 and info.n_workgroups == 256
+    rc, info, _ = _plan(n_splits=4)                              # an explicit split count is honoured as it is
+    assert rc == 0 and info.balanced == 0 and info.n_splits == 4
+    rc, info, _ = _plan(n_seq=64, kv_type=J.MLA_TYPE_Q8_0, kv_nb1=612)   # config 5
+    assert rc == 0 and info.variant == 2 and info.balanced == 1
+    rc, info, _ = _plan(n_seq=256)                               # one workgroup per sequence fills the GPU: nothing to split
+    assert rc == 0 and info.n_splits == 1 and info.balanced == 0
+    rc, info, _ = _plan(n_seq=8, bt_stride=4096)                 # runs could exceed the 64 pages a wave indexes
+    assert rc == 0 and info.balanced == 0 and info.n_splits * 64 * 128 >= 4096 * 128
+    rc, info, _ = _plan(block_table=0, seq_lens=0, bt_stride=0, n_kv=8192, kv_nb3=8192 * 1152)   # contiguous KV: uniform splits
+    assert rc == 0 and info.variant == 2 and info.balanced == 0 and info.n_splits == 8
+    rc, info, _ = _plan(dv=576)                                  # V := K: the general kernel, two passes over the columns
+    assert rc == 0 and info.variant == 0 and info.n_passes == 2 and info.balanced == 0
+    rc, info, _ = _plan(logit_softcap=30.0)                      # softcap: general kernel, 64 rows per workgroup
+    assert rc == 0 and info.variant == 0 and info.rows_per_wg == 64
