@@ -310,11 +310,13 @@ def other_config(a, dev, lib, J):
         pool = (torch.randn((1, B * L, 576), generator=g, device=dev) * 0.5).to(torch.bfloat16).view(torch.int16)
         q = torch.randn((1, 128, B, 576), generator=g, device=dev)
         mask = torch.full((64, B * L), float("-inf"), dtype=torch.float16, device=dev)
+        # --ragged: every sequence owns a slot of 8192 cells of the shared cache but has filled only 2048 .. 8192 of them
+        lens = [int(x) for x in rng.integers(2048, 8193, B)] if a.ragged else [L] * B
         for b in range(B):
-            mask[b, b * L:(b + 1) * L] = 0
+            mask[b, b * L:b * L + lens[b]] = 0
         out = torch.empty((1, B, 128, 576), dtype=torch.float32, device=dev)
-        lens, n_head, n_tok, kv, kvt = [L] * B, 128, B, "bf16", J.MLA_TYPE_BF16
-        name = "BASELINE configs[2] without the block table: one shared cache of 262144 cells, 32 query tokens, f16 mask selects each token's 8192 cells"
+        n_head, n_tok, kv, kvt = 128, B, "bf16", J.MLA_TYPE_BF16
+        name = "BASELINE configs[2] without the block table: one shared cache of 262144 cells, 32 query tokens, f16 mask selects each token's %s cells" % ("2048..8192" if a.ragged else "8192")
     elif a.config == "c4":
         lens, n_head, n_tok, kv, kvt = [2560] * 4, 16, 512, "bf16", J.MLA_TYPE_BF16
         mask = torch.where(torch.arange(2560, device=dev)[None, :] > 2048 + torch.arange(512, device=dev)[:, None], float("-inf"), 0.0).to(torch.float16)
@@ -442,6 +444,7 @@ def main():
                     help="also launch the library's plain copy kernel N times over one KV pool (known byte count) so that a "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run can be scaled")
     ap.add_argument("--kv", default="bf16", choices=["bf16", "f16", "q8_0"], help="storage type of the latent KV pool (the headline config is bf16; q8_0 only with --config kvwrite)")
+    ap.add_argument("--ragged", action="store_true", help="--config c3mask: sequence lengths uniform in [2048, 8192] instead of 8192")
     ap.add_argument("--uniform-splits", action="store_true", help="paged decode: equal KV splits per sequence (MLA_FLAG_UNIFORM_SPLITS) instead of the balanced schedule")
     ap.add_argument("--eager", action="store_true", help="time the K steps as K eager launch sequences instead of one replay of a HIP graph that holds them")
     ap.add_argument("--config", default="c3", choices=["c2", "c3", "c3mask", "c4", "c5", "kvwrite", "rope", "absorb", "unabsorb", "layer"],

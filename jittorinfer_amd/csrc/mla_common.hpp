@@ -62,11 +62,15 @@ struct KParams {
     int             n_pool_pages;  // block-table mode: pages in the pool
     int *           mask_ext;      // pipelined kernel with a mask: per block of 128 rows, 16 pairs (first, one past the last key that is not masked for all its rows) (workspace)
     int             rel_splits;    // the KV splits divide that key range (every split writes its (m, l), -inf when it has no key)
-    int             balanced;      // pipelined kernel, ragged paged decode: workgroups take equal runs of the page list of all sequences;
-    int             n_wg;
-    int *           wg_first;      //   [n_wg][8] first piece of every workgroup (workspace; written by the Q pre-pack pass)
-    int *           sched;         //   [n_seq_sched + 1] pages before each sequence / in total (workspace; written by the Q pre-pack pass)
-    int             n_seq_sched;   //   partial slot of workgroup v's piece of sequence b = v + b, n_seq_sched sequences, grid = (n_wg, 1, 1)
+    int             balanced;      // pipelined kernel: 1 = ragged paged decode, workgroups take equal runs of the page list of all
+                                   // sequences; 2 = masked launch, equal runs of the tile list of the row blocks' key ranges
+    int             n_wg;          //   workgroups (grid = (n_wg, 1, 1)); partial slot of workgroup v's piece of item i = v + i
+    int             n_units;       //   items: sequences (1) / row blocks (2)
+    int             slot_rows;     // rows per partial slot: n_rows, or 128 with balanced == 2
+    int             n_seq_sched;   // sequences of the launch (grids of the pre-pack passes)
+    int *           wg_first;      //   [n_wg][8] first piece of every workgroup (balanced == 1; workspace, written by the pre-pass)
+    int *           sched;         //   [n_units + 1] units before each item / in total (workspace; written by the pre-pass (1) or by the
+                                   //   first workgroup of the kernel itself (2); the combine pass reads it)
     int             rows_contig;  // kv rows are packed (kv_nb1 == row bytes): whole tiles are one contiguous run
 };
 

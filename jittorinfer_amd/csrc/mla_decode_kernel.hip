@@ -69,47 +69,69 @@ constexpr int lds_total(int kvt) { return sched_off(kvt) + (2 * SCHED_MAX_SEQ + 
     [nb1] "s"(s_nb1), [flg] "s"(s_flg), [ntl] "s"(s_ntl), [ostr] "s"(s_ostr), [qp] "s"(qpack), [msk] "s"(mask_base),  \
     [scl] "s"(s_scale), [pg0] "s"(s_pg0), [tid] "v"(tid)
 
-// Balanced schedule: p.sched[b] = number of 128-token pages of the sequences before b, p.sched[n_seq] = all pages; and
-// p.wg_first[8 v ..] = the first piece of workgroup v, ready to run: {sequence, kv_begin, kv_end, id of its first page,
-// whole sequence?, page-list position after it, end of the run, sequence length}; kv_begin >= kv_end: no work.
-// Computed once per call by the first block of the Q pre-pack kernel (every thread of its 256 calls this); the decode
-// workgroups and the combine pass read it.  n_seq <= SCHED_MAX_SEQ, p.n_wg <= 256.
-__device__ __forceinline__ void sched_prefix(const KParams & p) {
-    __shared__ int wave_total[4];
-    __shared__ int pre[SCHED_MAX_SEQ + 1];
+// Balanced schedule.  The work of a launch is a list of units -- the 128-token pages of the sequences of a paged decode
+// batch (p.balanced == 1), or the 32-token tiles of the key ranges the row blocks of a masked launch may attend to
+// (p.balanced == 2) -- and each of p.n_wg workgroups takes an equal run of that list, piece by piece where the run
+// crosses from one item (sequence / row block) to the next.
+//
+// sched_scan: S (LDS, 2 * SCHED_MAX_SEQ + 8 ints) <- S[i] = units of the items before i (i <= n_units), and from
+// S[SCHED_MAX_SEQ + 8] the `base` of every item; `count`, `base` belong to item threadIdx.x.  All 256 threads call it.
+__device__ __forceinline__ void sched_scan(int * S, int count, int base, int n_units) {
     const int t = threadIdx.x, lane = t & 63;
-    int v = 0;
-    if (t < p.n_seq_sched) v = (max(min(p.seq_lens[t], (int) p.bt_stride * MLA_PAGE_TOKENS), 0) + MLA_PAGE_TOKENS - 1) / MLA_PAGE_TOKENS;
+    int v = t < n_units ? count : 0;
     for (int d = 1; d < 64; d <<= 1) {   // inclusive scan inside the wave
         const int up = __shfl_up(v, d, 64);
         if (lane >= d) v += up;
     }
-    if (lane == 63) wave_total[t >> 6] = v;
+    if (lane == 63) S[SCHED_MAX_SEQ + 1 + (t >> 6)] = v;   // wave totals
     __syncthreads();
-    for (int w = 0; w < (t >> 6); w++) v += wave_total[w];
-    pre[t + 1] = v;
-    if (t == 0) pre[0] = 0;
-    if (t < p.n_seq_sched) p.sched[t + 1] = v;
-    if (t == 0) p.sched[0] = 0;
+    for (int w = 0; w < (t >> 6); w++) v += S[SCHED_MAX_SEQ + 1 + w];
     __syncthreads();
-    if (t >= p.n_wg) return;
-    const int total = pre[p.n_seq_sched], quota = (total + p.n_wg - 1) / p.n_wg;
-    int pos = min(t * quota, total);
-    const int end = min(pos + quota, total);
-    int hdr[8] = { 0, 0, 0, 0, 0, end, end, 0 };
-    if (pos < end) {
-        int lo = 0, hi = p.n_seq_sched - 1;   // the sequence that holds page `pos`: the last b with pre[b] <= pos that has pages
-        while (lo < hi) { const int mid = (lo + hi + 1) >> 1; if (pre[mid] <= pos) lo = mid; else hi = mid - 1; }
-        const int b = lo, first = pre[b], piece_end = min(pre[b + 1], end);
-        const int len = min(p.seq_lens[b], (int) p.bt_stride * MLA_PAGE_TOKENS);
-        hdr[0] = b;
-        hdr[1] = (pos - first) * MLA_PAGE_TOKENS;
-        hdr[2] = min(len, (piece_end - first) * MLA_PAGE_TOKENS);
-        hdr[3] = min(max(p.block_table[(int64_t) b * p.bt_stride + (pos - first)], 0), p.n_pool_pages - 1);
-        hdr[4] = pos == first && piece_end == pre[b + 1];
-        hdr[5] = piece_end;
+    S[t + 1] = v;
+    S[SCHED_MAX_SEQ + 8 + t] = base;
+    if (t == 0) S[0] = 0;
+    __syncthreads();
+}
+
+// The first piece of workgroup v: {item, kv_begin, kv_end, id of its first page (paged), whole item?, list position after
+// the piece, end of the run, sequence length}; kv_begin >= kv_end: the workgroup has no work.
+__device__ __forceinline__ void sched_first_piece(const KParams & p, const int * S, int v, int unit_tokens, int hdr[8]) {
+    const int total = S[p.n_units], quota = (total + p.n_wg - 1) / p.n_wg;
+    const int pos = min(v * quota, total), end = min(pos + quota, total);
+    hdr[0] = hdr[1] = hdr[2] = hdr[3] = hdr[4] = hdr[7] = 0;
+    hdr[5] = hdr[6] = end;
+    if (pos >= end) return;
+    int lo = 0, hi = p.n_units - 1;   // the item that holds unit `pos`: the last i with S[i] <= pos (it has units)
+    while (lo < hi) { const int mid = (lo + hi + 1) >> 1; if (S[mid] <= pos) lo = mid; else hi = mid - 1; }
+    const int it = lo, first = S[it], piece_end = min(S[it + 1], end), base = S[SCHED_MAX_SEQ + 8 + it];
+    hdr[0] = it;
+    hdr[1] = base + (pos - first) * unit_tokens;
+    hdr[2] = base + (piece_end - first) * unit_tokens;
+    if (p.balanced == 1) {
+        const int len = min(p.seq_lens[it], (int) p.bt_stride * MLA_PAGE_TOKENS);
+        hdr[2] = min(len, hdr[2]);
+        hdr[3] = min(max(p.block_table[(int64_t) it * p.bt_stride + (pos - first)], 0), p.n_pool_pages - 1);
         hdr[7] = len;
+    } else {
+        hdr[7] = (int) p.n_kv;
     }
+    hdr[4] = pos == first && piece_end == S[it + 1];
+    hdr[5] = piece_end;
+}
+
+// Paged decode batch: one block of the Q pre-pack kernel builds p.sched[0 .. n_units] (pages before every sequence) and
+// p.wg_first[8 v ..] (every workgroup's first piece, so that it can start after one scalar load).
+__device__ __forceinline__ void sched_prefix(const KParams & p) {
+    __shared__ int S[2 * SCHED_MAX_SEQ + 8];
+    const int t = threadIdx.x;
+    int pages = 0;
+    if (t < p.n_units) pages = (max(min(p.seq_lens[t], (int) p.bt_stride * MLA_PAGE_TOKENS), 0) + MLA_PAGE_TOKENS - 1) / MLA_PAGE_TOKENS;
+    sched_scan(S, pages, 0, p.n_units);
+    if (t <= p.n_units) p.sched[t] = S[t];
+    if (t == 0 && p.n_units == SCHED_MAX_SEQ) p.sched[SCHED_MAX_SEQ] = S[SCHED_MAX_SEQ];
+    if (t >= p.n_wg) return;
+    int hdr[8];
+    sched_first_piece(p, S, t, MLA_PAGE_TOKENS, hdr);
     for (int i = 0; i < 8; i++) p.wg_first[8 * t + i] = hdr[i];
 }
 
@@ -146,19 +168,49 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
     // takes an equal run of it (grid = (n_wg, 1, 1), bx = its place), and a run that crosses a sequence boundary is worked
     // off piece by piece.  Piece of workgroup v in sequence b -> partial slot v + b: the slots of one sequence are
     // consecutive, which is all the combine pass needs to know.
-    int * sched = (int *) (smem + sched_off(KVT));   // [0 .. n_seq]: pages before sequence b; [n_seq]: all pages; then the lengths
-    int run_pos = 0, run_end = 0, run_seq = 0;
+    int * sched = (int *) (smem + sched_off(KVT));   // [0 .. n_units]: units before item i; then, from SCHED_MAX_SEQ + 8, the
+                                                     // sequence lengths (paged) / first keys of the key ranges (masked)
+    int run_pos = 0, run_end = 0, run_item = 0;
     int first_piece[8] = { 0, 0, 0, 0, 0, 0, 0, 0 };
-    if (p.balanced) {
-        // the first piece comes ready-made from the pre-pass; the page prefix sums and the lengths are only needed for
-        // what may follow it and are fetched into LDS meanwhile (made visible by the barrier between pieces)
+    if (MASK && p.balanced == 2) {
+        // masked launch: every workgroup merges the 16 (first, one past the last) key pairs of each row block, rounds
+        // outwards to tiles and scans the tile counts itself (one round of loads; no extra kernel); the first workgroup
+        // leaves the prefix sums for the combine pass
+        const int t = threadIdx.x;
+        int tiles = 0, base = 0;
+        if (t < p.n_units) {
+            int mlo = 0x7fffffff, mhi = 0;
+            const u32x4 * pr = (const u32x4 *) (p.mask_ext + t * 32);   // 16 pairs = 8 x 16 bytes
+#pragma unroll
+            for (int c = 0; c < 8; c++) {
+                const u32x4 q = pr[c];
+                mlo = min(mlo, min((int) q.x, (int) q.z));
+                mhi = max(mhi, max((int) q.y, (int) q.w));
+            }
+            const int hi = min((int) p.n_kv, (mhi + TILE_TOK - 1) / TILE_TOK * TILE_TOK), lo = min(mlo / TILE_TOK * TILE_TOK, hi);
+            base  = lo;
+            tiles = (hi - lo) / TILE_TOK;
+        }
+        sched_scan(sched, tiles, base, p.n_units);
+        if (bx == 0) {
+            if (t <= p.n_units) p.sched[t] = sched[t];
+            if (t == 0 && p.n_units == SCHED_MAX_SEQ) p.sched[SCHED_MAX_SEQ] = sched[SCHED_MAX_SEQ];
+        }
+        int hdr[8];
+        sched_first_piece(p, sched, bx, TILE_TOK, hdr);
+        for (int i = 0; i < 8; i++) first_piece[i] = __builtin_amdgcn_readfirstlane(hdr[i]);
+        if (first_piece[1] >= first_piece[2]) return;
+        run_pos = first_piece[5]; run_end = first_piece[6]; run_item = first_piece[0] + 1;
+    } else if (p.balanced) {
+        // paged batch: the first piece comes ready-made from the pre-pass; the prefix sums and the lengths are only needed
+        // for what may follow it and are fetched into LDS meanwhile (made visible by the barrier between pieces)
         for (int i = 0; i < 8; i++) first_piece[i] = __builtin_amdgcn_readfirstlane(p.wg_first[8 * bx + i]);
         if (first_piece[1] >= first_piece[2]) return;
-        for (int i = threadIdx.x; i <= p.n_seq_sched; i += NTHREADS) {
+        for (int i = threadIdx.x; i <= p.n_units; i += NTHREADS) {
             sched[i] = p.sched[i];
-            if (i < p.n_seq_sched) sched[SCHED_MAX_SEQ + 8 + i] = p.seq_lens[i];
+            if (i < p.n_units) sched[SCHED_MAX_SEQ + 8 + i] = p.seq_lens[i];
         }
-        run_pos = first_piece[5]; run_end = first_piece[6]; run_seq = first_piece[0] + 1;
+        run_pos = first_piece[5]; run_end = first_piece[6]; run_item = first_piece[0] + 1;
     }
 
   for (int piece = 0;; piece++) {
@@ -167,27 +219,38 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
     const int tid = wave * 64 + lane, g = lane >> 5, rl = lane & 31;
     int b = bz, split = bx, slot = 0;
     int seq_len, kv_begin, kv_end;
-    bool direct = p.n_splits == 1;   // this piece is the whole sequence: final rows go to dst, there is nothing to combine
+    bool direct = p.n_splits == 1;   // this piece is the whole sequence / key range: final rows go to dst, there is nothing to combine
     int pg0_ready = -1;
-    if (p.balanced && piece == 0) {
-        b = first_piece[0]; kv_begin = first_piece[1]; kv_end = first_piece[2]; pg0_ready = first_piece[3];
-        direct = first_piece[4] != 0; seq_len = first_piece[7];
-        slot = bx + b; split = 1;
-    } else if (p.balanced) {
-        __syncthreads();   // every wave is through with the tile buffers and the hand-off records of the piece before
-        run_pos = __builtin_amdgcn_readfirstlane(run_pos); run_seq = __builtin_amdgcn_readfirstlane(run_seq);
-        while (run_pos < run_end && sched[run_seq + 1] <= run_pos) run_seq++;   // sequences without pages
-        if (run_pos >= run_end) return;
-        b = run_seq;
-        seq_len = min(sched[SCHED_MAX_SEQ + 8 + b], (int) p.bt_stride * MLA_PAGE_TOKENS);
-        const int first = sched[b], piece_end = min(sched[b + 1], run_end);
-        kv_begin = (run_pos - first) * MLA_PAGE_TOKENS;
-        kv_end   = min(seq_len, (piece_end - first) * MLA_PAGE_TOKENS);
-        slot     = bx + b;
-        direct   = run_pos == first && piece_end == sched[b + 1];
-        split    = 1;   // not the first split of anything: an empty piece writes nothing
-        run_pos  = piece_end;
-        run_seq  = b + 1;
+    if (p.balanced) {
+        int item;
+        if (piece == 0) {
+            item = first_piece[0]; kv_begin = first_piece[1]; kv_end = first_piece[2];
+            if (!MASK) pg0_ready = first_piece[3];
+            direct = first_piece[4] != 0; seq_len = first_piece[7];
+        } else {
+            __syncthreads();   // every wave is through with the tile buffers and the hand-off records of the piece before
+            run_pos = __builtin_amdgcn_readfirstlane(run_pos); run_item = __builtin_amdgcn_readfirstlane(run_item);
+            while (run_pos < run_end && sched[run_item + 1] <= run_pos) run_item++;   // items without units
+            if (run_pos >= run_end) return;
+            item = run_item;
+            const int first = sched[item], piece_end = min(sched[item + 1], run_end);
+            if constexpr (MASK) {
+                const int base = sched[SCHED_MAX_SEQ + 8 + item];
+                seq_len  = (int) p.n_kv;
+                kv_begin = base + (run_pos - first) * TILE_TOK;
+                kv_end   = base + (piece_end - first) * TILE_TOK;
+            } else {
+                seq_len  = min(sched[SCHED_MAX_SEQ + 8 + item], (int) p.bt_stride * MLA_PAGE_TOKENS);
+                kv_begin = (run_pos - first) * MLA_PAGE_TOKENS;
+                kv_end   = min(seq_len, (piece_end - first) * MLA_PAGE_TOKENS);
+            }
+            direct   = run_pos == first && piece_end == sched[item + 1];
+            run_pos  = piece_end;
+            run_item = item + 1;
+        }
+        if constexpr (MASK) by = item; else b = item;   // an item is a row block of the one masked launch, or a sequence
+        slot  = bx + item;
+        split = 1;   // not the first split of anything: an empty piece writes nothing
     } else {
         seq_len  = p.block_table ? min(p.seq_lens[b], (int) p.bt_stride * MLA_PAGE_TOKENS) : (int) p.n_kv;
         kv_begin = split * p.split_tokens;
@@ -197,10 +260,12 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
     const int row       = by * 128 + wave * 32 + rl;
     const bool row_valid = row < p.n_rows;
     const int64_t orow  = (int64_t) b * p.n_rows + row;
-    const int64_t prow  = (int64_t) slot * p.n_rows + row;
+    // a partial slot holds p.slot_rows rows: all rows of the sequence (uniform splits), or the 128 of one row block
+    const int lrow      = p.balanced == 2 ? row - by * 128 : row;
+    const int64_t prow  = (int64_t) slot * p.slot_rows + lrow;
 
     bool all_masked = false;  // this split holds keys, but none that a row of this block may attend to
-    if constexpr (MASK) {
+    if (MASK && !p.balanced) {
         int mlo = 0x7fffffff, mhi = 0;
         for (int c = 0; c < 16; c++) {
             mlo = min(mlo, p.mask_ext[(by * 16 + c) * 2]);
@@ -236,11 +301,11 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
 
     // per-thread pointers for the wave program, handed over through LDS
     // final output: row-major dst rows.  split-K partial: [column/8][row][8] inside this (sequence, split) block.
-    const int64_t pblock = (int64_t) slot * p.n_rows * p.dv_total;  // in f16 elements
+    const int64_t pblock = (int64_t) slot * p.slot_rows * p.dv_total;  // in f16 elements
     // (f32 partials are rows of dv_total floats: the wave program stores them the way it stores final output rows)
     void * optr = row_valid ? (direct ? (void *) (p.dst + orow * p.dst_stride + 4 * g)
                                : p.part_f32    ? (void *) ((float *) p.part_o + prow * p.dv_total + 4 * g)
-                                               : (void *) (p.part_o + pblock + (int64_t) row * 8 + 4 * g)) : nullptr;
+                                               : (void *) (p.part_o + pblock + (int64_t) lrow * 8 + 4 * g)) : nullptr;
     float * mlptr = (!direct && g == 0 && row_valid) ? p.part_ml + prow * 2 : nullptr;
     {
         unsigned long long * h = (unsigned long long *) (smem + HANDOFF_OFF + tid * 32);
@@ -251,7 +316,7 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
         h[3] = (unsigned long long) p.debug_ptr;
     }
     // this wave's packed Q operands: [seq][row block][wave][k-step][lane][16 bytes], written by mla_q_pack_kernel
-    const char * qpack = (const char *) p.q_pack + ((((int64_t) b * gridDim.y + by) * 4) * KSTEPS) * 1024;  // + wave*36 KB, added in the wave program
+    const char * qpack = (const char *) p.q_pack + ((((int64_t) b * ((p.n_rows + 127) / 128) + by) * 4) * KSTEPS) * 1024;  // + wave*36 KB, added in the wave program
     const char *    kv_base = p.kv + (p.block_table ? 0 : (int64_t) b * p.kv_nb3);
     const int32_t * bt_row  = p.block_table ? p.block_table + (int64_t) b * p.bt_stride : nullptr;
     // uniform scalars, forced into SGPRs
@@ -269,7 +334,7 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
     const int s_pg0 = __builtin_amdgcn_readfirstlane(pg0);
     const char * mask_base = p.mask;
     const int s_scale = __builtin_amdgcn_readfirstlane(__float_as_int(p.scale));
-    const int s_ostr = __builtin_amdgcn_readfirstlane(p.n_rows * 16);  // bytes between the partial rows of column groups c and c+1
+    const int s_ostr = __builtin_amdgcn_readfirstlane(p.slot_rows * 16);  // bytes between the partial rows of column groups c and c+1
 
     if constexpr (KVT == SRC_Q8) {
         asm volatile(
@@ -302,7 +367,7 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
 // grid = (n_row_blocks, n_seq, 36 k-steps), block = 256: one 16-byte output per thread.
 template <bool F16>
 __global__ void __launch_bounds__(NTHREADS) mla_q_pack_kernel(const KParams p) {
-    if (blockIdx.z == gridDim.z - 1 && p.balanced) {   // balanced schedule: one extra layer of blocks, the first of which builds it
+    if (blockIdx.z == gridDim.z - 1 && p.balanced == 1) {   // balanced schedule: one extra layer of blocks, the first of which builds it
         if (blockIdx.x == 0 && blockIdx.y == 0) sched_prefix(p);
         return;
     }
@@ -354,11 +419,12 @@ __global__ void __launch_bounds__(NTHREADS) mla_mask_extent_kernel(const KParams
     }
 }
 
+
 // The same image for Q8_0 KV: ggml-cpu quantizes Q to Q8_0 when K is Q8_0 (ggml-cpu.c:313-322, :12034-12035): per block of 32
 // d = amax/127 (stored as f16), id = 127/amax, q = round-half-even(x*id) (ggml-cpu-quants.c:855-900); the MFMA operand is the
 // dequantized value q * f16(d), rounded to f16.  grid = (n_row_blocks, n_seq, 18 blocks), block = 256: two k-steps per thread.
 __global__ void __launch_bounds__(NTHREADS) mla_q_pack_q8_kernel(const KParams p) {
-    if (blockIdx.z == gridDim.z - 1 && p.balanced) {   // balanced schedule: one extra layer of blocks, the first of which builds it
+    if (blockIdx.z == gridDim.z - 1 && p.balanced == 1) {   // balanced schedule: one extra layer of blocks, the first of which builds it
         if (blockIdx.x == 0 && blockIdx.y == 0) sched_prefix(p);
         return;
     }
@@ -435,7 +501,7 @@ static hipError_t launch_variant(const KParams & kp, dim3 grid, hipStream_t st) 
 
 hipError_t launch_decode_fast(const KParams & kp, int kv_type, dim3 grid, hipStream_t st, bool with_prepass) {
     // the small passes ahead of the kernel run per (row block, sequence), whatever the kernel's own grid is
-    const unsigned n_rb = (unsigned) ((kp.n_rows + 127) / 128), n_seq = (unsigned) kp.n_seq_sched, extra = kp.balanced ? 1 : 0;
+    const unsigned n_rb = (unsigned) ((kp.n_rows + 127) / 128), n_seq = (unsigned) kp.n_seq_sched, extra = kp.balanced == 1 ? 1 : 0;
     const bool m = kp.mask != nullptr;
     if (!with_prepass) { /* the workspace still holds the Q image and the mask extents of an earlier launch of the same call */ }
     else if (kv_type == MLA_TYPE_Q8_0)     hipLaunchKernelGGL(mla_q_pack_q8_kernel, dim3(n_rb, n_seq, KSTEPS / 2 + extra), dim3(NTHREADS), 0, st, kp);

@@ -398,23 +398,27 @@ __global__ void __launch_bounds__(NTHREADS) mla_attn_tile_kernel(const KParams p
     }
 }
 
-// Where the partials of sequence b sit: uniform splits -> slots b*n_splits .. +nvalid; balanced schedule -> the
-// workgroups whose runs of the page list touch the sequence, slot = workgroup + b (see mla_decode_kernel).
-__device__ __forceinline__ void partial_slots(const KParams & p, int b, int seq_len, int & slot0, int & nvalid) {
+// Where the partials of a row sit.  Uniform splits: slots b*n_splits .. +nvalid, each holding all n_rows rows.  Balanced
+// schedule: the workgroups whose runs of the unit list touch the item (the sequence b, or with a mask the row block of
+// the row), slot = workgroup + item (see mla_decode_kernel), each holding p.slot_rows rows; lrow = the row inside a slot.
+// nvalid < 0: one workgroup had the whole item and wrote the final rows itself.
+__device__ __forceinline__ void partial_slots(const KParams & p, int b, int row, int seq_len, int & slot0, int & nvalid, int & lrow) {
+    lrow = row;
     if (!p.balanced) {
         nvalid = (seq_len + p.split_tokens - 1) / p.split_tokens;
         nvalid = p.rel_splits ? p.n_splits : min(nvalid, p.n_splits);
         slot0  = b * p.n_splits;
         return;
     }
-    const int before = p.sched[b], total = p.sched[p.n_seq_sched];   // pages of the sequences before b / of all sequences
-    const int mine  = (max(seq_len, 0) + MLA_PAGE_TOKENS - 1) / MLA_PAGE_TOKENS;
+    const int item = p.balanced == 2 ? row / 128 : b;
+    if (p.balanced == 2) lrow = row - item * 128;
+    const int before = p.sched[item], mine = p.sched[item + 1] - before, total = p.sched[p.n_units];
     const int quota = (total + p.n_wg - 1) / p.n_wg;
     if (mine == 0) { slot0 = 0; nvalid = 0; return; }
     const int w0 = before / quota, w1 = (before + mine - 1) / quota;
-    slot0  = w0 + b;
+    slot0  = w0 + item;
     nvalid = w1 - w0 + 1;
-    if (nvalid == 1) nvalid = -1;   // one workgroup had the whole sequence and wrote the final rows itself
+    if (nvalid == 1) nvalid = -1;
 }
 
 // Log-sum-exp merge of the split-K partials: out = sum_c (O_c/l_c) l_c 2^(m_c - M) / sum_c l_c 2^(m_c - M).
@@ -426,13 +430,14 @@ __global__ void __launch_bounds__(256) mla_attn_combine_kernel(const KParams p) 
     const int row = blockIdx.x * 32 + (threadIdx.x & 31);
     const int cg  = blockIdx.y * 8 + (threadIdx.x >> 5);
     const int seq_len = p.block_table ? min(p.seq_lens[b], (int) p.bt_stride * MLA_PAGE_TOKENS) : (int) p.n_kv;
-    int slot0, nvalid;
-    partial_slots(p, b, seq_len, slot0, nvalid);
-    if (nvalid < 0 || row >= p.n_rows || cg * 8 >= p.dv_total) return;
+    if (row >= p.n_rows || cg * 8 >= p.dv_total) return;
+    int slot0, nvalid, lrow;
+    partial_slots(p, b, row, seq_len, slot0, nvalid, lrow);
+    if (nvalid < 0) return;
 
-    const float2 *   ml = (const float2 *) p.part_ml + (int64_t) slot0 * p.n_rows + row;
-    const _Float16 * po = p.part_o + (int64_t) slot0 * p.n_rows * p.dv_total + ((int64_t) cg * p.n_rows + row) * 8;
-    const int64_t ml_step = p.n_rows, po_step = (int64_t) p.n_rows * p.dv_total;
+    const float2 *   ml = (const float2 *) p.part_ml + (int64_t) slot0 * p.slot_rows + lrow;
+    const _Float16 * po = p.part_o + (int64_t) slot0 * p.slot_rows * p.dv_total + ((int64_t) cg * p.slot_rows + lrow) * 8;
+    const int64_t ml_step = p.slot_rows, po_step = (int64_t) p.slot_rows * p.dv_total;
 
     float M = -INFINITY, L = 0.f;
     float o[8] = { 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f };
@@ -483,12 +488,13 @@ __global__ void __launch_bounds__(256) mla_attn_combine_f32_kernel(const KParams
     const int row = blockIdx.x * rows_per_block + threadIdx.x / groups_per_row;
     const int cg  = threadIdx.x % groups_per_row;
     const int seq_len = p.block_table ? min(p.seq_lens[b], (int) p.bt_stride * MLA_PAGE_TOKENS) : (int) p.n_kv;
-    int slot0, nvalid;
-    partial_slots(p, b, seq_len, slot0, nvalid);
-    if (nvalid < 0 || row >= p.n_rows || threadIdx.x >= rows_per_block * groups_per_row || cg * 4 >= p.dv_total) return;
-    const float2 * ml = (const float2 *) p.part_ml + (int64_t) slot0 * p.n_rows + row;
-    const float *  po = (const float *) p.part_o + ((int64_t) slot0 * p.n_rows + row) * p.dv_total + cg * 4;
-    const int64_t ml_step = p.n_rows, po_step = (int64_t) p.n_rows * p.dv_total;
+    if (row >= p.n_rows || threadIdx.x >= rows_per_block * groups_per_row || cg * 4 >= p.dv_total) return;
+    int slot0, nvalid, lrow;
+    partial_slots(p, b, row, seq_len, slot0, nvalid, lrow);
+    if (nvalid < 0) return;
+    const float2 * ml = (const float2 *) p.part_ml + (int64_t) slot0 * p.slot_rows + lrow;
+    const float *  po = (const float *) p.part_o + ((int64_t) slot0 * p.slot_rows + lrow) * p.dv_total + cg * 4;
+    const int64_t ml_step = p.slot_rows, po_step = (int64_t) p.slot_rows * p.dv_total;
     float M = -INFINITY, L = 0.f;
     f32x4 o = { 0.f, 0.f, 0.f, 0.f };
     for (int c0 = 0; c0 < nvalid; c0 += 8) {   // groups of 8 splits: their loads are in flight together
@@ -602,7 +608,7 @@ struct Plan {
     size_t lds_bytes;
     size_t ws_part_o, ws_part_ml, ws_scores, ws_qpack, ws_maskext, ws_sched;
     int    part_f32;
-    int    balanced, n_wg;   // balanced schedule of the pipelined kernel (ragged paged decode)
+    int    balanced, n_wg, n_units;   // balanced schedule of the pipelined kernel (1: ragged paged decode, 2: masked launch)
 };
 
 int validate(const mla_attn_args * a) {
@@ -685,18 +691,28 @@ int make_plan(const mla_attn_args * a, Plan * pl) {
     // A paged decode batch (one row block per sequence, no mask) that needs KV splits anyway: the pipelined kernel's
     // workgroups take equal runs of the page list of all sequences instead of equal shares of the longest possible
     // sequence, so a ragged batch keeps every CU busy.  One workgroup per CU; a run must fit the 64 page ids a wave holds.
-    if (pl->variant == 2 && a->block_table && !a->mask && pl->n_row_blocks == 1 && a->n_splits == 0 && pl->n_splits > 1 &&
-        a->n_seq <= 256 && !(a->flags & MLA_FLAG_UNIFORM_SPLITS)) {
-        if (((int64_t) a->n_seq * n_pages + 255) / 256 <= 64) { pl->balanced = 1; pl->n_wg = 256; pl->ws_sched = (size_t) (a->n_seq + 1 + 63) / 64 * 64 * sizeof(int) + (size_t) pl->n_wg * 8 * sizeof(int); }
+    // The same for a masked launch over one contiguous cache (the reference's batched decode): equal runs of the tiles of
+    // the key ranges the row blocks may attend to.
+    if (pl->variant == 2 && a->n_splits == 0 && pl->n_splits > 1 && !(a->flags & MLA_FLAG_UNIFORM_SPLITS)) {
+        if (a->block_table && !a->mask && pl->n_row_blocks == 1 && a->n_seq <= 256 && ((int64_t) a->n_seq * n_pages + 255) / 256 <= 64) {
+            pl->balanced = 1; pl->n_units = a->n_seq;
+        } else if (a->mask && !a->block_table && a->n_seq == 1 && pl->n_row_blocks <= 256) {
+            pl->balanced = 2; pl->n_units = pl->n_row_blocks;
+        }
+        if (pl->balanced) {
+            pl->n_wg = 256;
+            pl->ws_sched = (size_t) ((pl->n_units + 1 + 63) / 64 * 64 + pl->n_wg * 8) * sizeof(int);
+        }
     }
     if (pl->n_splits > 1) {
         // f32 partials while they are small (no second rounding of O on top of the MFMA operands' one), f16 beyond: there the
         // partial traffic counts, and the rounding (2^-12 relative per split) is averaged over long contexts
-        const size_t n_slots = pl->balanced ? (size_t) pl->n_wg + a->n_seq : (size_t) a->n_seq * pl->n_splits;
-        const size_t n_part = n_slots * n_rows * a->dv;
+        const size_t n_slots = pl->balanced ? (size_t) pl->n_wg + pl->n_units : (size_t) a->n_seq * pl->n_splits;
+        const size_t slot_rows = pl->balanced == 2 ? 128 : (size_t) n_rows;
+        const size_t n_part = n_slots * slot_rows * a->dv;
         pl->part_f32   = n_part * sizeof(float) <= ((size_t) 32 << 20);
         pl->ws_part_o  = n_part * (pl->part_f32 ? sizeof(float) : sizeof(_Float16));
-        pl->ws_part_ml = n_slots * n_rows * 2 * sizeof(float);
+        pl->ws_part_ml = n_slots * slot_rows * 2 * sizeof(float);
     }
     return 0;
 }
@@ -788,13 +804,14 @@ static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
     kp.part_o  = (_Float16 *) ws;
     kp.part_f32 = pl.part_f32;
     kp.rel_splits = pl.variant == 2 && a->mask != nullptr;
-    kp.balanced = pl.balanced; kp.n_wg = pl.n_wg; kp.n_seq_sched = a->n_seq;
+    kp.balanced = pl.balanced; kp.n_wg = pl.n_wg; kp.n_seq_sched = a->n_seq; kp.n_units = pl.n_units;
+    kp.slot_rows = pl.balanced == 2 ? 128 : kp.n_rows;
     kp.part_ml = (float *) (ws + align256(pl.ws_part_o));
     float * scores = (float *) (ws + align256(pl.ws_part_o) + align256(pl.ws_part_ml));
     kp.q_pack = ws + align256(pl.ws_part_o) + align256(pl.ws_part_ml) + align256(pl.ws_scores);
     kp.mask_ext = (int *) (ws + align256(pl.ws_part_o) + align256(pl.ws_part_ml) + align256(pl.ws_scores) + align256(pl.ws_qpack));
     kp.sched = (int *) (ws + align256(pl.ws_part_o) + align256(pl.ws_part_ml) + align256(pl.ws_scores) + align256(pl.ws_qpack) + align256(pl.ws_maskext));
-    kp.wg_first = kp.sched + (a->n_seq + 1 + 63) / 64 * 64;
+    kp.wg_first = kp.sched + (pl.n_units + 1 + 63) / 64 * 64;
 
     if (pl.variant == 1) {
         if (!(phases & 1)) return 0;
