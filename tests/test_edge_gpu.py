@@ -213,8 +213,12 @@ def test_reference_style_batched_decode_through_the_mask(gpu, k_type, n_splits):
     tq = torch.from_numpy(q).to(gpu)
     tk = torch.from_numpy(k.view(np.int16)).to(gpu)
     tm = torch.from_numpy(mask.view(np.float16)).to(gpu)
-    assert J.plan(tq, tk, k_type, dv=512, scale=U.SCALE, mask=tm, n_splits=n_splits)["variant"] == 2
+    info = J.plan(tq, tk, k_type, dv=512, scale=U.SCALE, mask=tm, n_splits=n_splits)
+    assert info["variant"] == 2 and info["balanced"] == (2 if n_splits == 0 else 0)   # 0: the tiles of the 8 key ranges dealt out evenly
     got = _run(gpu, q, k, k_type, mask=mask, scale=U.SCALE, n_splits=n_splits)
+    if n_splits == 0:
+        uni = _run(gpu, q, k, k_type, mask=mask, scale=U.SCALE, flags=J.MLA_FLAG_UNIFORM_SPLITS)
+        assert float(np.nanmax(np.abs(uni[..., :512] - got[..., :512]))) < 2e-3
     if k_type == O.TYPE_F16:
         want = O.flash_attn_ext_f64(q, k, k_type, dv=512, mask=mask, scale=U.SCALE)
     else:
@@ -278,3 +282,32 @@ def test_balanced_schedule_limits(gpu):
     assert J.plan(q8, pool, J.MLA_TYPE_BF16, dv=512, scale=1.0, block_table=bt[:8], seq_lens=sl[:8])["balanced"] == 1
     wide = torch.zeros((8, 4096), dtype=torch.int32, device=gpu)
     assert J.plan(q8, pool, J.MLA_TYPE_BF16, dv=512, scale=1.0, block_table=wide, seq_lens=sl[:8])["balanced"] == 0
+
+
+def test_balanced_schedule_of_a_masked_launch_with_many_row_blocks(gpu):
+    """320 query tokens x 16 heads = 40 row blocks over one cache of 2048 cells; every token sees its own window, some see
+    nothing (NaN rows, like the reference), the windows of a row block's 8 tokens overlap only partly.  The workgroups'
+    runs of the tile list cross row-block boundaries (40 key ranges of up to 64 tiles over 256 workgroups)."""
+    import torch
+    import jittorinfer_amd as J
+    rng = np.random.default_rng(77)
+    n_tok, n_kv = 320, 2048
+    k = U.encode_kv(rng.standard_normal((1, n_kv, 576)).astype(np.float32), O.TYPE_BF16)
+    m = np.full((n_tok, n_kv), -np.inf, dtype=np.float32)
+    for t in range(n_tok):
+        if t % 37 == 5:
+            continue                                   # a token with no visible key at all
+        centre = (t // 8) * 45 + int(rng.integers(0, 200))
+        lo, hi = max(0, centre - int(rng.integers(1, 300))), min(n_kv, centre + int(rng.integers(1, 300)))
+        m[t, lo:hi] = 0.0
+    m[8:16] = -np.inf                                  # a whole row block without keys
+    mask = m.astype(np.float16).view(np.uint16)
+    q = rng.standard_normal((1, 16, n_tok, 576)).astype(np.float32)
+    tq, tk = torch.from_numpy(q).to(gpu), torch.from_numpy(k.view(np.int16)).to(gpu)
+    tm = torch.from_numpy(mask.view(np.float16)).to(gpu)
+    info = J.plan(tq, tk, O.TYPE_BF16, dv=512, scale=U.SCALE, mask=tm)
+    assert info["variant"] == 2 and info["balanced"] == 2 and info["n_row_blocks"] == 40
+    got = _run(gpu, q, k, O.TYPE_BF16, mask=mask, scale=U.SCALE)
+    want = O.flash_attn_ext(q, k, O.TYPE_BF16, dv=512, mask=mask, scale=U.SCALE)
+    assert np.isnan(want[0, 5]).all() and np.isnan(want[0, 8:16]).all()
+    print(U.check(got[..., :512], want, "masked launch, balanced schedule"))
