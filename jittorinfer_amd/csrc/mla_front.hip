@@ -220,17 +220,31 @@ __global__ void __launch_bounds__(256) mla_mul_mat_skinny_kernel(const MmP p) {
 // into the other LDS buffer at the end of the step: one barrier per chunk.
 template <bool F16, int KCH>
 __global__ void __launch_bounds__(256) mla_mul_mat_stream_kernel(const MmP p, const int tiles_per_wg) {
-    constexpr int TM = 64;
+    constexpr int TM = 64, OB_PITCH = 128 + 4;
     __shared__ __attribute__((aligned(16))) char lds[2][TM * MM_PITCH];
+    __shared__ __attribute__((aligned(16))) float obuf[TM * OB_PITCH];
+    // whole 128-wide n tiles and 16-byte aligned result rows: results are written row-wise through LDS
+    const bool vec_store = p.N % 128 == 0 && !(p.d_nb1 & 15) && !(p.d_nb2 & 15) && !(p.d_nb3 & 15) && !((uintptr_t) p.dst & 15);
     const int     lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int64_t i2 = blockIdx.z % p.ne2, i3 = blockIdx.z / p.ne2;
+    // dispatch index i runs on XCD i % 8: remapped so that the workgroups that read the same activation rows (the n tiles
+    // of one run of m tiles) sit on one XCD and share its L2
+    unsigned bx = blockIdx.x, by = blockIdx.y, bz = blockIdx.z;
+    {
+        const unsigned G = gridDim.x * gridDim.y * gridDim.z;
+        if ((G & 7) == 0 && gridDim.x > 1) {   // (with one n tile nothing is shared, and the plain order measured 12 % faster)
+            const unsigned id = (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+            const unsigned v  = (id & 7) * (G >> 3) + (id >> 3);
+            bx = v % gridDim.x; by = (v / gridDim.x) % gridDim.y; bz = v / (gridDim.x * gridDim.y);
+        }
+    }
+    const int64_t i2 = bz % p.ne2, i3 = bz / p.ne2;
     const char *  X  = p.x + i2 * p.x_nb2 + i3 * p.x_nb3;
     char *        D  = p.dst + i2 * p.d_nb2 + i3 * p.d_nb3;
-    const int64_t n0 = (int64_t) blockIdx.x * 128 + wave * 32;
+    const int64_t n0 = (int64_t) bx * 128 + wave * 32;
     const int64_t n  = n0 + (lane & 31);
     const char *  wrow = p.w + (i2 / p.r2) * p.w_nb2 + (i3 / p.r3) * p.w_nb3 + min(n, p.N - 1) * p.w_nb1 + (lane >> 5) * 16;
     const int64_t n_tiles = (p.M + TM - 1) / TM;
-    const int64_t t0 = (int64_t) blockIdx.y * tiles_per_wg, t1 = min(t0 + tiles_per_wg, n_tiles);
+    const int64_t t0 = (int64_t) by * tiles_per_wg, t1 = min(t0 + tiles_per_wg, n_tiles);
     if (t0 >= t1) return;
 
     u32x4 wf[KCH * 8];
@@ -280,7 +294,22 @@ __global__ void __launch_bounds__(256) mla_mul_mat_stream_kernel(const MmP p, co
                     acc[mb] = mfma32<F16>(af, wf[kc * 8 + ks], acc[mb]);
                 }
             if (last_kc) {
-                if (n < p.N) {
+                if (vec_store) {
+                    // through LDS, so that a row's 128 results leave as one 512-byte run (32 lanes x 16 bytes) instead of
+                    // four 128-byte pieces written by four waves at different times
+#pragma unroll
+                    for (int mb = 0; mb < 2; mb++)
+#pragma unroll
+                        for (int j = 0; j < 16; j++)
+                            obuf[(mb * 32 + (j >> 2) * 8 + (lane >> 5) * 4 + (j & 3)) * OB_PITCH + wave * 32 + (lane & 31)] = acc[mb][j];
+                    __syncthreads();
+#pragma unroll
+                    for (int i = 0; i < 8; i++) {
+                        const int     r = srow + 8 * i;
+                        const int64_t m = tile * TM + r;
+                        if (m < p.M) *(float4 *) (D + m * p.d_nb1 + ((int64_t) bx * 128 + sc4 * 4) * 4) = *(const float4 *) (obuf + r * OB_PITCH + sc4 * 4);
+                    }
+                } else if (n < p.N) {
 #pragma unroll
                     for (int mb = 0; mb < 2; mb++)
 #pragma unroll
