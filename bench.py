@@ -307,7 +307,14 @@ def other_config(a, dev, lib, J):
         B, L = 32, 8192
         g = torch.Generator(device=dev)
         g.manual_seed(a.seed)
-        pool = (torch.randn((1, B * L, 576), generator=g, device=dev) * 0.5).to(torch.bfloat16).view(torch.int16)
+        if a.kv == "q8_0":   # --kv q8_0: the same cache as Q8_0 cells (int8 = round(N(0, 0.5) * 32), block scale 1/32)
+            qs = torch.clamp(torch.round(torch.randn((B * L, 18, 32), generator=g, device=dev) * 16), -127, 127).to(torch.int8)
+            pool = torch.empty((B * L, 18, 34), dtype=torch.uint8, device=dev)
+            pool[:, :, 0], pool[:, :, 1] = 0x00, 0x28
+            pool[:, :, 2:] = qs.view(torch.uint8)
+            pool = pool.reshape(1, B * L, 612)
+        else:
+            pool = (torch.randn((1, B * L, 576), generator=g, device=dev) * 0.5).to(torch.bfloat16).view(torch.int16)
         q = torch.randn((1, 128, B, 576), generator=g, device=dev)
         mask = torch.full((64, B * L), float("-inf"), dtype=torch.float16, device=dev)
         # --ragged: every sequence owns a slot of 8192 cells of the shared cache but has filled only 2048 .. 8192 of them
@@ -315,7 +322,7 @@ def other_config(a, dev, lib, J):
         for b in range(B):
             mask[b, b * L:b * L + lens[b]] = 0
         out = torch.empty((1, B, 128, 576), dtype=torch.float32, device=dev)
-        n_head, n_tok, kv, kvt = 128, B, "bf16", J.MLA_TYPE_BF16
+        n_head, n_tok, kv, kvt = 128, B, ("q8_0" if a.kv == "q8_0" else "bf16"), (J.MLA_TYPE_Q8_0 if a.kv == "q8_0" else J.MLA_TYPE_BF16)
         name = "BASELINE configs[2] without the block table: one shared cache of 262144 cells, 32 query tokens, f16 mask selects each token's %s cells" % ("2048..8192" if a.ragged else "8192")
     elif a.config == "c4":
         lens, n_head, n_tok, kv, kvt = [2560] * 4, 16, 512, "bf16", J.MLA_TYPE_BF16

@@ -71,6 +71,7 @@ struct KParams {
     int *           wg_first;      //   [n_wg][8] first piece of every workgroup (balanced == 1; workspace, written by the pre-pass)
     int *           sched;         //   [n_units + 1] units before each item / in total (workspace; written by the pre-pass (1) or by the
                                    //   first workgroup of the kernel itself (2); the combine pass reads it)
+    int             q_as_q8;       // the KV rows are the f16 expansion of a Q8_0 cache: Q is quantized the Q8_0 way
     int             rows_contig;  // kv rows are packed (kv_nb1 == row bytes): whole tiles are one contiguous run
 };
 
@@ -106,6 +107,8 @@ __device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); 
 
 // The pipelined decode kernel (mla_decode_kernel.hip); returns hipErrorInvalidValue for shapes it does not take.
 bool       decode_fast_applicable(const mla_attn_args * a);
+int64_t    decode_fast_q8_copy_rows(const mla_attn_args * a);   // > 0: Q8_0 + mask runs on an f16 copy of that many rows (workspace)
+hipError_t launch_q8_to_f16(const char * src, int64_t src_nb1, int64_t src_nb3, int64_t rows_per_batch, void * dst, int64_t n_rows, hipStream_t st);
 hipError_t launch_decode_fast(const KParams & kp, int kv_type, dim3 grid, hipStream_t st, bool with_prepass);
 size_t     decode_fast_lds_bytes(int kv_type);
 size_t     decode_fast_qpack_bytes(int n_seq, int n_row_blocks);

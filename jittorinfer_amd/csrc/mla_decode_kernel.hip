@@ -463,10 +463,20 @@ size_t decode_fast_lds_bytes(int kv_type) { return (size_t) lds_total(kv_type ==
 
 size_t decode_fast_qpack_bytes(int n_seq, int n_row_blocks) { return (size_t) n_seq * n_row_blocks * 4 * KSTEPS * 1024; }
 
+// Q8_0 rows with a mask: there is no masked build of the Q8_0 wave program.  The cache is expanded into f16 rows in the
+// workspace -- the very f16 values the Q8_0 build feeds its MFMAs -- and the masked f16 build runs on that copy, with Q
+// quantized the Q8_0 way.  Costs a pass over the whole cache (612 bytes read, 1152 written per row), so only up to 1 GiB.
+int64_t decode_fast_q8_copy_rows(const mla_attn_args * a) {
+    if (a->kv_type != MLA_TYPE_Q8_0 || !a->mask || a->kv_nb1 < Q8_ROW) return 0;
+    const int64_t rows = a->block_table ? a->n_kv : a->n_kv * (a->kv_nb3 ? a->n_seq : 1);
+    return rows > 0 && rows * ROW_BYTES <= ((int64_t) 1 << 30) ? rows : 0;
+}
+
 bool decode_fast_applicable(const mla_attn_args * a) {
     if (a->kv_type != MLA_TYPE_BF16 && a->kv_type != MLA_TYPE_F16 && a->kv_type != MLA_TYPE_Q8_0) return false;
     if (a->dv != 512 || (a->flags & MLA_FLAG_F16_ACC_STRICT)) return false;
-    if (a->kv_type == MLA_TYPE_Q8_0) {
+    const bool q8_copy = decode_fast_q8_copy_rows(a) > 0;
+    if (a->kv_type == MLA_TYPE_Q8_0 && !q8_copy) {
         // raw tiles are copied as one run of 19584 bytes in 16-byte pieces: packed rows, 16-byte aligned tiles, whole tiles
         // inside the allocation (always true for pages; a contiguous KV must end on a tile boundary); no masked build
         if (a->mask || a->kv_nb1 != Q8_ROW || ((uintptr_t) a->kv & 15)) return false;
@@ -474,7 +484,7 @@ bool decode_fast_applicable(const mla_attn_args * a) {
     }
     if (a->logit_softcap != 0.0f || a->max_bias > 0.0f) return false;
     // 16-bit rows must be packed: the per-lane offsets of the tile copy are kept as 16-bit values (31 * 1152 + 1136 < 65536)
-    if (a->kv_type != MLA_TYPE_Q8_0 && a->kv_nb1 != ROW_BYTES) return false;
+    if (a->kv_type != MLA_TYPE_Q8_0 && a->kv_nb1 != ROW_BYTES) return false;   // (the f16 copy of a Q8_0 cache is packed by construction)
     if (a->mask) {
         // whole tiles only (no key past n_kv is touched in a mask row), 32-bit offsets into the mask, 8-byte aligned loads
         const int64_t n_kv = a->block_table ? a->bt_stride * MLA_PAGE_TOKENS : a->n_kv;
@@ -484,6 +494,33 @@ bool decode_fast_applicable(const mla_attn_args * a) {
     if (!(a->scale > 0.0f) || !(a->scale < INFINITY)) return false;
     if ((int64_t) a->n_tok * a->n_head < 16) return false;
     return true;
+}
+
+// Q8_0 rows -> f16 rows: value = f16(q * f32(d)), one rounding of an exact product, the operand the Q8_0 wave program
+// builds in LDS.  One thread = 8 values (a quarter of a block): grid = ceil(rows * 72 / 256).
+__global__ void __launch_bounds__(NTHREADS) mla_q8_to_f16_kernel(const char * src, int64_t src_nb1, int64_t src_nb3, int64_t rows_per_batch,
+                                                                 _Float16 * dst, int64_t n_rows) {
+    const int64_t i = (int64_t) blockIdx.x * NTHREADS + threadIdx.x;
+    const int64_t r = i / 72;
+    if (r >= n_rows) return;
+    const int g = (int) (i - r * 72), blk = g >> 2, quarter = g & 3;
+    const char * row = src + (r / rows_per_batch) * src_nb3 + (r % rows_per_batch) * src_nb1 + blk * 34;   // 2-byte aligned
+    const float d = f16_bits_to_f32(*(const unsigned short *) row);
+    const unsigned short * qs = (const unsigned short *) (row + 2 + quarter * 8);
+    u32x4 out;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const unsigned short w = qs[k];
+        const float lo = (float) (signed char) (w & 0xff) * d, hi = (float) (signed char) (w >> 8) * d;
+        out[k] = f32_to_f16_bits(lo) | (f32_to_f16_bits(hi) << 16);
+    }
+    *(u32x4 *) ((char *) dst + r * ROW_BYTES + g * 16) = out;
+}
+
+hipError_t launch_q8_to_f16(const char * src, int64_t src_nb1, int64_t src_nb3, int64_t rows_per_batch, void * dst, int64_t n_rows, hipStream_t st) {
+    hipLaunchKernelGGL(mla_q8_to_f16_kernel, dim3((unsigned) ((n_rows * 72 + NTHREADS - 1) / NTHREADS)), dim3(NTHREADS), 0, st,
+                       src, src_nb1, src_nb3, rows_per_batch, (_Float16 *) dst, n_rows);
+    return hipGetLastError();
 }
 
 template <int KVT, bool MASK>
@@ -504,7 +541,7 @@ hipError_t launch_decode_fast(const KParams & kp, int kv_type, dim3 grid, hipStr
     const unsigned n_rb = (unsigned) ((kp.n_rows + 127) / 128), n_seq = (unsigned) kp.n_seq_sched, extra = kp.balanced == 1 ? 1 : 0;
     const bool m = kp.mask != nullptr;
     if (!with_prepass) { /* the workspace still holds the Q image and the mask extents of an earlier launch of the same call */ }
-    else if (kv_type == MLA_TYPE_Q8_0)     hipLaunchKernelGGL(mla_q_pack_q8_kernel, dim3(n_rb, n_seq, KSTEPS / 2 + extra), dim3(NTHREADS), 0, st, kp);
+    else if (kv_type == MLA_TYPE_Q8_0 || kp.q_as_q8) hipLaunchKernelGGL(mla_q_pack_q8_kernel, dim3(n_rb, n_seq, KSTEPS / 2 + extra), dim3(NTHREADS), 0, st, kp);
     else if (kv_type == MLA_TYPE_F16) hipLaunchKernelGGL(mla_q_pack_kernel<true>, dim3(n_rb, n_seq, KSTEPS + extra), dim3(NTHREADS), 0, st, kp);
     else                              hipLaunchKernelGGL(mla_q_pack_kernel<false>, dim3(n_rb, n_seq, KSTEPS + extra), dim3(NTHREADS), 0, st, kp);
     if (m && with_prepass) hipLaunchKernelGGL(mla_mask_extent_kernel, dim3(n_rb, MASK_EXT_CHUNKS), dim3(NTHREADS), 0, st, kp);

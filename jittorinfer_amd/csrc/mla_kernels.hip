@@ -606,7 +606,8 @@ struct Plan {
     int    n_splits, split_tokens;
     int    n_passes, ndb;
     size_t lds_bytes;
-    size_t ws_part_o, ws_part_ml, ws_scores, ws_qpack, ws_maskext, ws_sched;
+    size_t ws_part_o, ws_part_ml, ws_scores, ws_qpack, ws_maskext, ws_sched, ws_kvcopy;
+    int64_t kvcopy_rows;
     int    part_f32;
     int    balanced, n_wg, n_units;   // balanced schedule of the pipelined kernel (1: ragged paged decode, 2: masked launch)
 };
@@ -685,8 +686,9 @@ int make_plan(const mla_attn_args * a, Plan * pl) {
     const int64_t pages_per_split = (n_pages + splits - 1) / splits;
     pl->split_tokens = (int) (pages_per_split * MLA_PAGE_TOKENS);
     pl->n_splits     = (int) ((n_pages + pages_per_split - 1) / pages_per_split);
-    pl->lds_bytes    = pl->variant == 2 ? decode_fast_lds_bytes(a->kv_type) : 2 * TILE_BYTES + (a->kv_type == MLA_TYPE_Q8_0 ? Q8_TILE_RAW : 0);
+    pl->lds_bytes    = pl->variant == 2 ? decode_fast_lds_bytes(a->mask && a->kv_type == MLA_TYPE_Q8_0 ? MLA_TYPE_F16 : a->kv_type) : 2 * TILE_BYTES + (a->kv_type == MLA_TYPE_Q8_0 ? Q8_TILE_RAW : 0);
     if (pl->variant == 2) pl->ws_qpack = decode_fast_qpack_bytes(a->n_seq, pl->n_row_blocks);
+    if (pl->variant == 2) { pl->kvcopy_rows = decode_fast_q8_copy_rows(a); pl->ws_kvcopy = (size_t) pl->kvcopy_rows * ROW_BYTES; }
     if (pl->variant == 2 && a->mask) pl->ws_maskext = (size_t) pl->n_row_blocks * 16 * 2 * sizeof(int);  // 16 (first, last) pairs per row block
     // A paged decode batch (one row block per sequence, no mask) that needs KV splits anyway: the pipelined kernel's
     // workgroups take equal runs of the page list of all sequences instead of equal shares of the longest possible
@@ -719,7 +721,7 @@ int make_plan(const mla_attn_args * a, Plan * pl) {
 
 size_t align256(size_t x) { return (x + 255) & ~(size_t) 255; }
 size_t plan_ws(const Plan & pl) {
-    return align256(pl.ws_part_o) + align256(pl.ws_part_ml) + align256(pl.ws_scores) + align256(pl.ws_qpack) + align256(pl.ws_maskext) + align256(pl.ws_sched);
+    return align256(pl.ws_part_o) + align256(pl.ws_part_ml) + align256(pl.ws_scores) + align256(pl.ws_qpack) + align256(pl.ws_maskext) + align256(pl.ws_sched) + align256(pl.ws_kvcopy);
 }
 
 template <int SRC, int NDB, int WM, int WD>
@@ -828,10 +830,22 @@ static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
 
     dim3 grid((unsigned) pl.n_splits, (unsigned) pl.n_row_blocks, (unsigned) a->n_seq);
     if (pl.balanced) grid = dim3((unsigned) pl.n_wg, 1, 1);
+    int kv_type = a->kv_type;
+    if (pl.kvcopy_rows > 0) {
+        // Q8_0 cache + mask: expand the cache to f16 rows (a pre-pass like the Q image) and run the masked f16 build on them
+        char * copy = ws + align256(pl.ws_part_o) + align256(pl.ws_part_ml) + align256(pl.ws_scores) + align256(pl.ws_qpack) + align256(pl.ws_maskext) + align256(pl.ws_sched);
+        if (phases & 4) {
+            const hipError_t e = launch_q8_to_f16(kp.kv, kp.kv_nb1, kp.kv_nb3, a->n_kv, copy, pl.kvcopy_rows, st);
+            if (e != hipSuccess) return (int) e;
+        }
+        kp.kv = copy; kp.kv_nb1 = ROW_BYTES; kp.kv_nb3 = kp.kv_nb3 ? a->n_kv * ROW_BYTES : 0;
+        kp.rows_contig = 1; kp.q_as_q8 = 1;
+        kv_type = MLA_TYPE_F16;
+    }
     for (int pass = 0; pass < pl.n_passes && (phases & 1); pass++) {
         kp.d_off = pass * pl.ndb * 32;
         hipError_t e;
-        if (pl.variant == 2) e = launch_decode_fast(kp, a->kv_type, grid, st, (phases & 4) != 0);
+        if (pl.variant == 2) e = launch_decode_fast(kp, kv_type, grid, st, (phases & 4) != 0);
         else switch (a->kv_type) {
             case MLA_TYPE_BF16: e = launch_tile_src<SRC_BF16>(pl, kp, grid, st); break;
             case MLA_TYPE_F16:  e = launch_tile_src<SRC_F16>(pl, kp, grid, st); break;

@@ -185,7 +185,7 @@ def test_step_replayed_from_a_hip_graph(gpu):
             print(U.check(out.cpu().numpy()[..., :512], U.oracle_per_seq(q, seqs, O.TYPE_BF16, 512), "graph replay"))
 
 
-@pytest.mark.parametrize("k_type", [O.TYPE_BF16, O.TYPE_F16])
+@pytest.mark.parametrize("k_type", [O.TYPE_BF16, O.TYPE_F16, O.TYPE_Q8_0])
 @pytest.mark.parametrize("n_splits", [0, 1, 5])
 def test_reference_style_batched_decode_through_the_mask(gpu, k_type, n_splits):
     """The reference's own decode batch (no block table): one shared cache, one query token per sequence, and the f16 mask
@@ -202,16 +202,19 @@ def test_reference_style_batched_decode_through_the_mask(gpu, k_type, n_splits):
         start[s] = pos
         pos += lens[s] + int(rng.integers(0, 40))
     assert pos <= n_kv
-    k = U.encode_kv((rng.standard_normal((1, n_kv, 576)) * 30).astype(np.float32), k_type)   # other cells: wild values
+    # (Q8_0 cells with one power-of-two block scale, as BASELINE's config 5 builds them: with arbitrary scales the f16 MFMA
+    # operand alone costs a 5-key sequence up to 2^-11 |v| = 2.1e-3 in single elements)
+    q8s = 1.0 / 32 if k_type == O.TYPE_Q8_0 else None
+    k = U.encode_kv((rng.standard_normal((1, n_kv, 576)) * 30).astype(np.float32), k_type, q8_scale=q8s)   # other cells: wild values
     m = np.full((len(lens), n_kv), -np.inf, dtype=np.float32)
     for s, l in enumerate(lens):
-        k[0, start[s]:start[s] + l] = U.encode_kv(rng.standard_normal((l, 576)).astype(np.float32), k_type)
+        k[0, start[s]:start[s] + l] = U.encode_kv(rng.standard_normal((l, 576)).astype(np.float32), k_type, q8_scale=q8s)
         m[s, start[s]:start[s] + l] = 0.0
     m[3, start[3] + 100:start[3] + 400] = -np.inf       # a hole inside a sequence (cells of a removed span)
     mask = m.astype(np.float16).view(np.uint16)
     q = rng.standard_normal((1, 128, len(lens), 576)).astype(np.float32)
     tq = torch.from_numpy(q).to(gpu)
-    tk = torch.from_numpy(k.view(np.int16)).to(gpu)
+    tk = torch.from_numpy(k.view(np.int16) if k.dtype == np.uint16 else k).to(gpu)
     tm = torch.from_numpy(mask.view(np.float16)).to(gpu)
     info = J.plan(tq, tk, k_type, dv=512, scale=U.SCALE, mask=tm, n_splits=n_splits)
     assert info["variant"] == 2 and info["balanced"] == (2 if n_splits == 0 else 0)   # 0: the tiles of the 8 key ranges dealt out evenly
