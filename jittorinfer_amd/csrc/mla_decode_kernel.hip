@@ -517,6 +517,11 @@ __global__ void __launch_bounds__(NTHREADS) mla_q8_to_f16_kernel(const char * sr
     *(u32x4 *) ((char *) dst + r * ROW_BYTES + g * 16) = out;
 }
 
+hipError_t launch_mask_extent(const KParams & kp, hipStream_t st) {
+    hipLaunchKernelGGL(mla_mask_extent_kernel, dim3((unsigned) ((kp.n_rows + 127) / 128), MASK_EXT_CHUNKS), dim3(NTHREADS), 0, st, kp);
+    return hipGetLastError();
+}
+
 hipError_t launch_q8_to_f16(const char * src, int64_t src_nb1, int64_t src_nb3, int64_t rows_per_batch, void * dst, int64_t n_rows, hipStream_t st) {
     hipLaunchKernelGGL(mla_q8_to_f16_kernel, dim3((unsigned) ((n_rows * 72 + NTHREADS - 1) / NTHREADS)), dim3(NTHREADS), 0, st,
                        src, src_nb1, src_nb3, rows_per_batch, (_Float16 *) dst, n_rows);

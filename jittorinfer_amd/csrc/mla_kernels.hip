@@ -54,9 +54,24 @@ __global__ void __launch_bounds__(NTHREADS) mla_attn_tile_kernel(const KParams p
     const int split = blockIdx.x;
 
     const int seq_len  = p.block_table ? min(p.seq_lens[b], (int) p.bt_stride * MLA_PAGE_TOKENS) : (int) p.n_kv;
-    const int kv_begin = split * p.split_tokens;
-    const int kv_end   = min(seq_len, kv_begin + p.split_tokens);
-    if (kv_begin >= kv_end && !(seq_len <= 0 && split == 0)) return;  // nothing to do; the combine pass knows
+    int kv_begin = split * p.split_tokens;
+    int kv_end   = min(seq_len, kv_begin + p.split_tokens);
+    if (p.mask_ext) {
+        // only the keys that the mask leaves open for some row of this block (16 (first, one past the last) pairs per 128
+        // rows from mla_mask_extent_kernel, rounded outwards to tiles), and the KV splits divide that range, not the
+        // cache.  A split left without keys runs no tile and its (m, l) = (-inf, 0) tells the combine pass so; with one
+        // split the rows then come out NaN like the reference's.
+        int mlo = 0x7fffffff, mhi = 0;
+        const int eb = blockIdx.y * RBLK / 128;
+        for (int c = 0; c < 16; c++) {
+            mlo = min(mlo, p.mask_ext[(eb * 16 + c) * 2]);
+            mhi = max(mhi, p.mask_ext[(eb * 16 + c) * 2 + 1]);
+        }
+        const int hi = min(seq_len, (mhi + TILE_TOK - 1) / TILE_TOK * TILE_TOK), lo = min(mlo / TILE_TOK * TILE_TOK, hi);
+        const int chunk = ((hi - lo + p.n_splits - 1) / p.n_splits + TILE_TOK - 1) / TILE_TOK * TILE_TOK;
+        kv_begin = min(hi, lo + split * chunk);
+        kv_end   = min(hi, kv_begin + chunk);
+    } else if (kv_begin >= kv_end && !(seq_len <= 0 && split == 0)) return;  // nothing to do; the combine pass knows
 
     const int  row       = blockIdx.y * RBLK + wm * 32 + rl;
     const bool row_valid = row < p.n_rows;
@@ -690,6 +705,13 @@ int make_plan(const mla_attn_args * a, Plan * pl) {
     if (pl->variant == 2) pl->ws_qpack = decode_fast_qpack_bytes(a->n_seq, pl->n_row_blocks);
     if (pl->variant == 2) { pl->kvcopy_rows = decode_fast_q8_copy_rows(a); pl->ws_kvcopy = (size_t) pl->kvcopy_rows * ROW_BYTES; }
     if (pl->variant == 2 && a->mask) pl->ws_maskext = (size_t) pl->n_row_blocks * 16 * 2 * sizeof(int);  // 16 (first, last) pairs per row block
+    if (pl->variant == 0 && a->mask) {
+        // the general kernel visits only the key range the mask leaves open, when the extent pass can read the mask rows
+        // (8-byte loads over whole groups of 8 keys)
+        const int64_t nk = a->block_table ? a->bt_stride * MLA_PAGE_TOKENS : a->n_kv;
+        if (nk % 8 == 0 && a->mask_ne0 >= nk && !(a->mask_nb1 & 7) && !((uintptr_t) a->mask & 7))
+            pl->ws_maskext = (size_t) ((n_rows + 127) / 128) * 16 * 2 * sizeof(int);
+    }
     // A paged decode batch (one row block per sequence, no mask) that needs KV splits anyway: the pipelined kernel's
     // workgroups take equal runs of the page list of all sequences instead of equal shares of the longest possible
     // sequence, so a ragged batch keeps every CU busy.  One workgroup per CU; a run must fit the 64 page ids a wave holds.
@@ -805,13 +827,13 @@ static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
     char * ws = (char *) a->workspace;
     kp.part_o  = (_Float16 *) ws;
     kp.part_f32 = pl.part_f32;
-    kp.rel_splits = pl.variant == 2 && a->mask != nullptr;
+    kp.rel_splits = a->mask != nullptr && (pl.variant == 2 || pl.ws_maskext > 0);
     kp.balanced = pl.balanced; kp.n_wg = pl.n_wg; kp.n_seq_sched = a->n_seq; kp.n_units = pl.n_units;
     kp.slot_rows = pl.balanced == 2 ? 128 : kp.n_rows;
     kp.part_ml = (float *) (ws + align256(pl.ws_part_o));
     float * scores = (float *) (ws + align256(pl.ws_part_o) + align256(pl.ws_part_ml));
     kp.q_pack = ws + align256(pl.ws_part_o) + align256(pl.ws_part_ml) + align256(pl.ws_scores);
-    kp.mask_ext = (int *) (ws + align256(pl.ws_part_o) + align256(pl.ws_part_ml) + align256(pl.ws_scores) + align256(pl.ws_qpack));
+    kp.mask_ext = pl.ws_maskext ? (int *) (ws + align256(pl.ws_part_o) + align256(pl.ws_part_ml) + align256(pl.ws_scores) + align256(pl.ws_qpack)) : nullptr;
     kp.sched = (int *) (ws + align256(pl.ws_part_o) + align256(pl.ws_part_ml) + align256(pl.ws_scores) + align256(pl.ws_qpack) + align256(pl.ws_maskext));
     kp.wg_first = kp.sched + (pl.n_units + 1 + 63) / 64 * 64;
 
@@ -841,6 +863,10 @@ static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
         kp.kv = copy; kp.kv_nb1 = ROW_BYTES; kp.kv_nb3 = kp.kv_nb3 ? a->n_kv * ROW_BYTES : 0;
         kp.rows_contig = 1; kp.q_as_q8 = 1;
         kv_type = MLA_TYPE_F16;
+    }
+    if (pl.variant == 0 && kp.mask_ext && (phases & 4)) {
+        const hipError_t e = launch_mask_extent(kp, st);
+        if (e != hipSuccess) return (int) e;
     }
     for (int pass = 0; pass < pl.n_passes && (phases & 1); pass++) {
         kp.d_off = pass * pl.ndb * 32;
