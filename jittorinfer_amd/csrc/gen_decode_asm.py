@@ -809,6 +809,10 @@ def main():
     e("v_lshlrev_b32 %s, 3, %s" % (v(X2), v(X2)))                      # *4 elements *2 bytes
     e("v_add_u32 %s, %s, %s" % (v(X1), v(X1), v(X2)))
     e("v_mad_u32_u24 %s, %s, %s, %s" % (v(VADDR_LANE), v(X0), s(SPITCH), v(X1)))
+    # FLG bit 4: V is columns 64 .. 575 of the rows instead of 0 .. 511 (second pass of a 576-wide V)
+    e("s_bitcmp1_b32 %s, 4" % s(FLG))
+    e("s_cselect_b32 %s, 128, 0" % s(S0))
+    e("v_add_u32 %s, %s, %s" % (v(VADDR_LANE), s(S0), v(VADDR_LANE)))
     # ------------------------------------------------------------------ page ids of this split -> one lane each
     lab_nobt = label("nobt")
     e("s_lshr_b32 %s, %s, 7" % (s(PG0), s(KVB)))

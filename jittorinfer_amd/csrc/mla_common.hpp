@@ -71,6 +71,8 @@ struct KParams {
     int *           wg_first;      //   [n_wg][8] first piece of every workgroup (balanced == 1; workspace, written by the pre-pass)
     int *           sched;         //   [n_units + 1] units before each item / in total (workspace; written by the pre-pass (1) or by the
                                    //   first workgroup of the kernel itself (2); the combine pass reads it)
+    int             v_col0;        // pipelined kernel: V = columns v_col0 .. v_col0 + 511 of the rows (0, or 64 in the second pass of a
+                                   // 576-wide V), and the 512 results go to columns v_col0 .. of the dst rows
     int             q_as_q8;       // the KV rows are the f16 expansion of a Q8_0 cache: Q is quantized the Q8_0 way
     int             rows_contig;  // kv rows are packed (kv_nb1 == row bytes): whole tiles are one contiguous run
 };

@@ -288,7 +288,7 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
         } else if (seq_len <= 0 && split == 0 && row_valid && g == 0) {
             if (p.n_splits == 1) {
                 float * o = p.dst + orow * p.dst_stride;
-                for (int d = 0; d < 512; d++) o[d] = __builtin_nanf("");
+                for (int d = 0; d < 512; d++) o[p.v_col0 + d] = __builtin_nanf("");
             } else {
                 p.part_ml[prow * 2] = -INFINITY;
                 p.part_ml[prow * 2 + 1] = 0.f;
@@ -303,7 +303,7 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
     // final output: row-major dst rows.  split-K partial: [column/8][row][8] inside this (sequence, split) block.
     const int64_t pblock = (int64_t) slot * p.slot_rows * p.dv_total;  // in f16 elements
     // (f32 partials are rows of dv_total floats: the wave program stores them the way it stores final output rows)
-    void * optr = row_valid ? (direct ? (void *) (p.dst + orow * p.dst_stride + 4 * g)
+    void * optr = row_valid ? (direct ? (void *) (p.dst + orow * p.dst_stride + p.v_col0 + 4 * g)
                                : p.part_f32    ? (void *) ((float *) p.part_o + prow * p.dv_total + 4 * g)
                                                : (void *) (p.part_o + pblock + (int64_t) lrow * 8 + 4 * g)) : nullptr;
     float * mlptr = (!direct && g == 0 && row_valid) ? p.part_ml + prow * 2 : nullptr;
@@ -325,7 +325,7 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
     const int s_kve  = __builtin_amdgcn_readfirstlane(kv_end);
     const int s_npp  = __builtin_amdgcn_readfirstlane(p.n_pool_pages - 1);
     const int s_nb1  = __builtin_amdgcn_readfirstlane((int) p.kv_nb1);
-    const int s_flg  = __builtin_amdgcn_readfirstlane((direct || p.part_f32 ? 1 : 0) | p.debug_flags);  // bit 0: f32 row store
+    const int s_flg  = __builtin_amdgcn_readfirstlane((direct || p.part_f32 ? 1 : 0) | (p.v_col0 ? 16 : 0) | p.debug_flags);  // bit 0: f32 row store; bit 4: V starts at column 64
     const int s_ntl  = __builtin_amdgcn_readfirstlane(n_tiles);
     // id of the split's first page as a scalar: the first tiles are requested before the vector load of all page ids is back
     int pg0 = 0;
@@ -474,7 +474,7 @@ int64_t decode_fast_q8_copy_rows(const mla_attn_args * a) {
 
 bool decode_fast_applicable(const mla_attn_args * a) {
     if (a->kv_type != MLA_TYPE_BF16 && a->kv_type != MLA_TYPE_F16 && a->kv_type != MLA_TYPE_Q8_0) return false;
-    if (a->dv != 512 || (a->flags & MLA_FLAG_F16_ACC_STRICT)) return false;
+    if ((a->dv != 512 && a->dv != 576) || (a->flags & MLA_FLAG_F16_ACC_STRICT)) return false;   // 576: two passes, V = columns 0.. and 64..
     const bool q8_copy = decode_fast_q8_copy_rows(a) > 0;
     if (a->kv_type == MLA_TYPE_Q8_0 && !q8_copy) {
         // raw tiles are copied as one run of 19584 bytes in 16-byte pieces: packed rows, 16-byte aligned tiles, whole tiles

@@ -489,7 +489,7 @@ __global__ void __launch_bounds__(256) mla_attn_combine_kernel(const KParams p) 
         }
     }
     const float inv = 1.0f / L;  // no valid key at all: 0 * inf = NaN, like the reference
-    float * out = p.dst + ((int64_t) b * p.n_rows + row) * p.dst_stride + cg * 8;
+    float * out = p.dst + ((int64_t) b * p.n_rows + row) * p.dst_stride + p.v_col0 + cg * 8;
     *(f32x4 *) out       = f32x4{ o[0] * inv, o[1] * inv, o[2] * inv, o[3] * inv };
     *(f32x4 *) (out + 4) = f32x4{ o[4] * inv, o[5] * inv, o[6] * inv, o[7] * inv };
 }
@@ -538,7 +538,7 @@ __global__ void __launch_bounds__(256) mla_attn_combine_f32_kernel(const KParams
         }
     }
     const float inv = 1.0f / L;  // no valid key at all: 0 * inf = NaN, like the reference
-    *(f32x4 *) (p.dst + ((int64_t) b * p.n_rows + row) * p.dst_stride + cg * 4) = f32x4{ o.x * inv, o.y * inv, o.z * inv, o.w * inv };
+    *(f32x4 *) (p.dst + ((int64_t) b * p.n_rows + row) * p.dst_stride + p.v_col0 + cg * 4) = f32x4{ o.x * inv, o.y * inv, o.z * inv, o.w * inv };
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -672,7 +672,7 @@ int make_plan(const mla_attn_args * a, Plan * pl) {
         pl->split_tokens = (int) max_len;
         return 0;
     }
-    if (decode_fast_applicable(a) && a->rows_per_wg == 0) { pl->variant = 2; pl->n_passes = 1; pl->ndb = 16; pl->wm = 4; pl->wd = 1; }
+    if (decode_fast_applicable(a) && a->rows_per_wg == 0) { pl->variant = 2; pl->n_passes = a->dv == 576 ? 2 : 1; pl->ndb = 16; pl->wm = 4; pl->wd = 1; }
     else if (a->dv == 576) { pl->n_passes = 2; pl->ndb = 9; pl->wm = 4; pl->wd = 1; }
     else {
         pl->n_passes = 1; pl->ndb = 16;
@@ -733,7 +733,7 @@ int make_plan(const mla_attn_args * a, Plan * pl) {
         // partial traffic counts, and the rounding (2^-12 relative per split) is averaged over long contexts
         const size_t n_slots = pl->balanced ? (size_t) pl->n_wg + pl->n_units : (size_t) a->n_seq * pl->n_splits;
         const size_t slot_rows = pl->balanced == 2 ? 128 : (size_t) n_rows;
-        const size_t n_part = n_slots * slot_rows * a->dv;
+        const size_t n_part = n_slots * slot_rows * (pl->variant == 2 ? 512 : a->dv);
         pl->part_f32   = n_part * sizeof(float) <= ((size_t) 32 << 20);
         pl->ws_part_o  = n_part * (pl->part_f32 ? sizeof(float) : sizeof(_Float16));
         pl->ws_part_ml = n_slots * slot_rows * 2 * sizeof(float);
@@ -868,28 +868,48 @@ static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
         const hipError_t e = launch_mask_extent(kp, st);
         if (e != hipSuccess) return (int) e;
     }
+    auto combine = [&](int dv) -> int {
+        if (pl.part_f32) {
+            const int groups = dv / 4, rows_per_block = 256 / groups;   // 128 -> 2 rows, 144 -> 1 row
+            dim3 g((unsigned) ((kp.n_rows + rows_per_block - 1) / rows_per_block), 1, (unsigned) a->n_seq);
+            hipLaunchKernelGGL(mla_attn_combine_f32_kernel, g, dim3(256), 0, st, kp, groups);
+            return (int) hipGetLastError();
+        }
+        dim3 g((unsigned) ((kp.n_rows + 31) / 32), (unsigned) ((dv + 63) / 64), (unsigned) a->n_seq);
+        hipLaunchKernelGGL(mla_attn_combine_kernel, g, dim3(256), 0, st, kp);
+        return (int) hipGetLastError();
+    };
+    if (pl.variant == 2) {
+        // the pipelined kernel produces 512 columns per pass; a 576-wide V (V := K, the form ggml-cpu accepts) takes a second
+        // pass with V = columns 64 .. 575 of the rows, whose results land on columns 64 .. 575 of dst (64 .. 511 twice, with
+        // the same values: the same P and the same accumulation order).  Each pass has its own combine.
+        kp.dv_total = 512;
+        for (int pass = 0; pass < pl.n_passes; pass++) {
+            kp.v_col0 = pass * 64;
+            if (phases & 1) {
+                const hipError_t e = launch_decode_fast(kp, kv_type, grid, st, (phases & 4) != 0 && pass == 0);
+                if (e != hipSuccess) return (int) e;
+            }
+            // the partials of a pass are consumed before the next pass overwrites them; a combine-only call finishes the last pass
+            const bool last = pass + 1 == pl.n_passes;
+            if (pl.n_splits > 1 && ((phases & 1) ? (!last || (phases & 2)) : (last && (phases & 2)))) {
+                const int rc2 = combine(512);
+                if (rc2) return rc2;
+            }
+        }
+        return 0;
+    }
     for (int pass = 0; pass < pl.n_passes && (phases & 1); pass++) {
         kp.d_off = pass * pl.ndb * 32;
         hipError_t e;
-        if (pl.variant == 2) e = launch_decode_fast(kp, kv_type, grid, st, (phases & 4) != 0);
-        else switch (a->kv_type) {
+        switch (a->kv_type) {
             case MLA_TYPE_BF16: e = launch_tile_src<SRC_BF16>(pl, kp, grid, st); break;
             case MLA_TYPE_F16:  e = launch_tile_src<SRC_F16>(pl, kp, grid, st); break;
             default:            e = launch_tile_src<SRC_Q8>(pl, kp, grid, st); break;
         }
         if (e != hipSuccess) return (int) e;
     }
-    if (pl.n_splits > 1 && (phases & 2)) {
-        if (pl.part_f32) {
-            const int groups = a->dv / 4, rows_per_block = 256 / groups;   // 128 -> 2 rows, 144 -> 1 row
-            dim3 g((unsigned) ((kp.n_rows + rows_per_block - 1) / rows_per_block), 1, (unsigned) a->n_seq);
-            hipLaunchKernelGGL(mla_attn_combine_f32_kernel, g, dim3(256), 0, st, kp, groups);
-            return (int) hipGetLastError();
-        }
-        dim3 g((unsigned) ((kp.n_rows + 31) / 32), (unsigned) ((a->dv + 63) / 64), (unsigned) a->n_seq);
-        hipLaunchKernelGGL(mla_attn_combine_kernel, g, dim3(256), 0, st, kp);
-        return (int) hipGetLastError();
-    }
+    if (pl.n_splits > 1 && (phases & 2)) return combine(a->dv);
     return 0;
 }
 

@@ -143,7 +143,9 @@ def test_planner_schedules_without_gpu():
     assert rc == 0 and info.balanced == 0 and info.n_splits * 64 * 128 >= 4096 * 128
     rc, info, _ = _plan(block_table=0, seq_lens=0, bt_stride=0, n_kv=8192, kv_nb3=8192 * 1152)   # contiguous KV: uniform splits
     assert rc == 0 and info.variant == 2 and info.balanced == 0 and info.n_splits == 8
-    rc, info, _ = _plan(dv=576)                                  # V := K: the general kernel, two passes over the columns
-    assert rc == 0 and info.variant == 0 and info.n_passes == 2 and info.balanced == 0
+    rc, info, _ = _plan(dv=576)                                  # V := K: two passes of the pipelined kernel (columns 0.., 64..)
+    assert rc == 0 and info.variant == 2 and info.n_passes == 2 and info.balanced == 1
+    rc, info, _ = _plan(dv=576, max_bias=8.0, mask=131072, mask_nb1=16384, mask_ne0=8192)   # ALiBi: the general kernel, 2 x 288 columns
+    assert rc == 0 and info.variant == 0 and info.n_passes == 2
     rc, info, _ = _plan(logit_softcap=30.0)                      # softcap: general kernel, 64 rows per workgroup
     assert rc == 0 and info.variant == 0 and info.rows_per_wg == 64
