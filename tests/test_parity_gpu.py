@@ -168,3 +168,31 @@ def test_masked_decode_random_mask(gpu, n_splits, k_type):
     want = O.flash_attn_ext(q, k, k_type, dv=512, mask=mask, scale=U.SCALE)
     assert np.isnan(want[:, 1]).all()
     print(U.check(got[..., :512], want, "masked decode"))
+
+
+@pytest.mark.parametrize("k_type", [O.TYPE_BF16, O.TYPE_Q8_0])
+def test_dv576_paged_split_and_masked(gpu, k_type):
+    """V := K (all 576 columns) through the pipelined kernel's two passes (V = columns 0..511, then 64..575): a paged ragged
+    batch with KV splits (balanced schedule, a combine per pass), and a masked launch over one cache."""
+    import torch
+    import jittorinfer_amd as J
+    rng = np.random.default_rng(60)
+    lens = [700, 129, 33, 1500]
+    q8s = 1.0 / 32 if k_type == O.TYPE_Q8_0 else None
+    pool, bt, seqs = U.make_paged(rng, lens, k_type, q8_scale=q8s)
+    q = rng.standard_normal((4, 128, 1, 576)).astype(np.float32)
+    tq = torch.from_numpy(q).to(gpu)
+    tk = torch.from_numpy(pool.view(np.int16) if pool.dtype == np.uint16 else pool).to(gpu)
+    info = J.plan(tq, tk, k_type, dv=576, scale=U.SCALE, block_table=torch.from_numpy(bt).to(gpu),
+                  seq_lens=torch.tensor(lens, dtype=torch.int32, device=gpu))
+    assert info["variant"] == 2 and info["n_passes"] == 2 and info["n_splits"] > 1
+    got = _run(gpu, q, pool, k_type, dv=576, bt=bt, lens=lens, scale=U.SCALE)
+    want = U.oracle_per_seq(q, seqs, k_type, 576)
+    print(U.check(got, want, "dv 576 paged"))
+    n_kv, n_tok = 256, 5
+    q = rng.standard_normal((1, 16, n_tok, 576)).astype(np.float32)
+    k = U.encode_kv(rng.standard_normal((1, n_kv, 576)).astype(np.float32), k_type, q8_scale=q8s)
+    m = np.where(np.arange(n_kv)[None, :] > 100 + 30 * np.arange(n_tok)[:, None], -np.inf, 0.0).astype(np.float16)
+    got = _run(gpu, q, k, k_type, dv=576, mask=m.view(np.uint16), scale=U.SCALE)
+    want = O.flash_attn_ext(q, k, k_type, dv=576, mask=m.view(np.uint16), scale=U.SCALE)
+    print(U.check(got, want, "dv 576 masked"))
