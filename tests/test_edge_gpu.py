@@ -185,6 +185,53 @@ def test_step_replayed_from_a_hip_graph(gpu):
             print(U.check(out.cpu().numpy()[..., :512], U.oracle_per_seq(q, seqs, O.TYPE_BF16, 512), "graph replay"))
 
 
+def test_graph_replay_with_sequence_lengths_changed_on_the_device(gpu):
+    """The balanced page schedule is built on the device from seq_lens at every launch, so a captured launch follows
+    lengths that change between replays (a serving loop appends a token per step and swaps sequences in and out): every
+    replay equals the eager launch bit for bit and the oracle on the current prefixes, lengths of 0 included."""
+    import ctypes as C
+    import torch
+    import jittorinfer_amd as J
+    rng = np.random.default_rng(77)
+    n_seq, cap = 20, 1536
+    pool, bt, seqs = U.make_paged(rng, [cap] * n_seq, O.TYPE_BF16)
+    tq = torch.zeros((n_seq, 128, 1, 576), dtype=torch.float32, device=gpu)
+    tk = torch.from_numpy(pool.view(np.int16)).to(gpu)
+    tb = torch.from_numpy(bt).to(gpu)
+    tl = torch.full((n_seq,), cap, dtype=torch.int32, device=gpu)
+    out = torch.zeros((n_seq, 1, 128, 512), dtype=torch.float32, device=gpu)
+    kw = dict(dv=512, scale=U.SCALE, block_table=tb, seq_lens=tl, out=out)
+    a, _, keep = J.capi.make_args(tq, tk, J.MLA_TYPE_BF16, **kw)
+    assert J.plan(tq, tk, J.MLA_TYPE_BF16, **kw)["balanced"] == 1
+    lib = J.library()
+    side = torch.cuda.Stream(gpu)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        graph.capture_begin()
+        assert lib.mla_attn_launch(C.byref(a), C.c_void_p(side.cuda_stream)) == 0
+        graph.capture_end()
+    torch.cuda.synchronize()
+    steps = [rng.integers(1, cap + 1, n_seq), np.full(n_seq, cap), rng.integers(0, 260, n_seq),
+             np.where(np.arange(n_seq) % 3 == 0, 0, rng.integers(1, cap + 1, n_seq)), np.full(n_seq, 1)]
+    for it, lens in enumerate(steps):
+        q = rng.standard_normal((n_seq, 128, 1, 576)).astype(np.float32)
+        tq.copy_(torch.from_numpy(q).to(gpu))
+        tl.copy_(torch.from_numpy(lens.astype(np.int32)).to(gpu))
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        replayed = out.clone()
+        out.fill_(float("nan"))
+        J.ggml_flash_attn_ext(tq, tk, J.MLA_TYPE_BF16, **kw)
+        torch.cuda.synchronize()
+        assert torch.equal(replayed.view(torch.int32), out.view(torch.int32)), "replay %d differs from the eager launch" % it
+        got = replayed.cpu().numpy()
+        some = list(range(6))
+        want = U.oracle_per_seq(q[some], [seqs[b][:lens[b]] for b in some], O.TYPE_BF16, 512)
+        print(it, U.check(got[some], want, "replay %d" % it))
+
+
 @pytest.mark.parametrize("k_type", [O.TYPE_BF16, O.TYPE_F16, O.TYPE_Q8_0])
 @pytest.mark.parametrize("n_splits", [0, 1, 5])
 def test_reference_style_batched_decode_through_the_mask(gpu, k_type, n_splits):
