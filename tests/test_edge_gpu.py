@@ -111,6 +111,61 @@ def test_full_size_config3_properties(gpu):
     print(U.check(base[b:b + 1].cpu().numpy(), want, "config 3 full size, sequence 7"))
 
 
+def test_full_size_config5_properties(gpu):
+    """BASELINE configs[4] at full size (B=64, H=128, lengths uniform in [2048, 8192], Q8_0 pages with the block scale
+    1/32): bit-exact under a permutation of the pages, the balanced page schedule agrees with uniform splits, the
+    garbage after every sequence's last token is never read, and one sequence equals the oracle."""
+    import torch
+    import jittorinfer_amd as J
+    g = torch.Generator(device=gpu)
+    g.manual_seed(55)
+    B, H = 64, 128
+    lens = torch.randint(2048, 8193, (B,), generator=g, device=gpu).to(torch.int32)
+    nblk = (lens.long() + 127) // 128
+    pages, max_blocks = int(nblk.sum()), int(nblk.max())
+    qs = torch.clamp(torch.round(torch.randn((pages * 128, 18, 32), generator=g, device=gpu) * 16), -127, 127).to(torch.int8)
+    pool = torch.empty((pages * 128, 18, 34), dtype=torch.uint8, device=gpu)
+    pool[..., 0], pool[..., 1] = 0x00, 0x28          # f16 1/32, little endian
+    pool[..., 2:] = qs.view(torch.uint8)
+    pool = pool.reshape(pages * 128, 612)
+    ids = torch.randperm(pages, generator=g, device=gpu).to(torch.int32)
+    bt = torch.full((B, max_blocks), 2 ** 30, dtype=torch.int32, device=gpu)   # entries past a sequence: never read
+    start = torch.cumsum(nblk, 0) - nblk
+    for b in range(B):
+        bt[b, :int(nblk[b])] = ids[int(start[b]):int(start[b]) + int(nblk[b])]
+    q = torch.randn((B, H, 1, 576), generator=g, device=gpu)
+    kw = dict(dv=512, scale=U.SCALE)
+    info = J.plan(q, pool, J.MLA_TYPE_Q8_0, block_table=bt, seq_lens=lens, **kw)
+    assert info["variant"] == 2 and info["balanced"] == 1
+    base = J.ggml_flash_attn_ext(q, pool, J.MLA_TYPE_Q8_0, block_table=bt, seq_lens=lens, **kw)[..., :512].clone()
+    assert not torch.isnan(base).any()
+    # (a) move every page
+    perm = torch.randperm(pages, generator=g, device=gpu)
+    pool2 = torch.empty_like(pool)
+    pool2.view(pages, 128, 612)[perm] = pool.view(pages, 128, 612)
+    bt2 = torch.where(bt < pages, perm[bt.clamp(max=pages - 1).long()].to(torch.int32), bt).contiguous()
+    moved = J.ggml_flash_attn_ext(q, pool2, J.MLA_TYPE_Q8_0, block_table=bt2, seq_lens=lens, **kw)[..., :512]
+    assert torch.equal(base, moved)
+    # (b) the rows after every sequence's last token hold other values: same bits
+    pool3 = pool.clone().view(pages, 128, 612)
+    for b in range(B):
+        tail = int(lens[b]) % 128
+        if tail:
+            pool3[int(bt[b, int(nblk[b]) - 1]), tail:] = 0x7b
+    same = J.ggml_flash_attn_ext(q, pool3.view(pages * 128, 612), J.MLA_TYPE_Q8_0, block_table=bt, seq_lens=lens, **kw)[..., :512]
+    assert torch.equal(base, same)
+    # (c) uniform splits per sequence instead of the balanced page schedule
+    uni = J.ggml_flash_attn_ext(q, pool, J.MLA_TYPE_Q8_0, block_table=bt, seq_lens=lens, flags=J.MLA_FLAG_UNIFORM_SPLITS, **kw)[..., :512]
+    ma, rl = O.errors(uni.cpu().numpy(), base.cpu().numpy())
+    assert ma <= 5e-4 and rl <= 3e-4, (ma, rl)
+    # (d) the shortest sequence against the oracle
+    b = int(torch.argmin(lens))
+    rows = (bt[b, :int(nblk[b])].long()[:, None] * 128 + torch.arange(128, device=gpu)[None, :]).reshape(-1)[:int(lens[b])]
+    kb = pool[rows].cpu().numpy()[None]
+    want = O.flash_attn_ext(q[b:b + 1].cpu().numpy(), kb, O.TYPE_Q8_0, dv=512, scale=U.SCALE)
+    print(U.check(base[b:b + 1].cpu().numpy(), want, "config 5 full size, sequence %d (%d keys)" % (b, int(lens[b]))))
+
+
 def test_full_size_config4_causal_independence(gpu):
     """BASELINE configs[3] at full size (B=4, H=16, 512 new tokens on 2048 cached, causal mask): query token t must not
     depend on keys after position 2048 + t.  Keys after 2048 + 255 are replaced by other values: the outputs of tokens
