@@ -32,7 +32,6 @@ CLK = "--clk" in sys.argv or CLKP           # timing experiments only: s_memtime
 MASK = "--mask" in sys.argv  # additive f16 mask rows (one per query token), added to the scaled scores
 Q8 = "--q8" in sys.argv    # Q8_0 KV: raw tiles staged in LDS, dequantized to an f16 tile one tile ahead, then the f16 path
 F16 = "--f16" in sys.argv or Q8  # f16 KV: f16 MFMA, single P (no lo half)
-assert not (Q8 and MASK)
 MF = "v_mfma_f32_32x32x16_f16" if F16 else "v_mfma_f32_32x32x16_bf16"
 CVT = "v_cvt_pk_f16_f32" if F16 else "v_cvt_pk_bf16_f32"
 SPLIT = not F16
@@ -62,9 +61,10 @@ Q0 = 0
 SA, SB = 144, 160   # two 16-register groups: scores of one tile, converted in place to its P^T operands
 KF, KRING = 176, 4 if MASK else 5   # K fragment ring (x 4 registers)
 ALPHA = 196
-MOFF = 197                          # mask builds: byte offset of this lane's first mask element inside a tile's 64 mask bytes
+RELOAD_PTRS = Q8 and MASK           # the output pointers are read again from the hand-off record in the epilogue: their registers carry MOFF
+MOFF = 232 if RELOAD_PTRS else 197  # mask builds: byte offset of this lane's first mask element inside a tile's 64 mask bytes
 VF, VRING = 200, 5 if MASK or Q8 else 6   # V^T fragment ring (x 4 registers); 220..223 go to the mask values / the dequantizer
-MKR = [192, 193, 194, 195, 220, 221, 222, 223]   # mask builds: the 16 f16 mask values of this lane's 16 tokens of a tile
+MKR = [192, 193, 194, 195] + ([252, 253, 254, 255] if Q8 else [220, 221, 222, 223])   # mask builds: the 16 f16 mask values of this lane's 16 tokens of a tile
 T = list(range(224, 232))
 OPTR, MLPTR = 232, 234
 KADDR_LANE, VADDR_LANE, MRUN, LRUN, NEGM = 236, 237, 238, 239, 240
@@ -79,7 +79,8 @@ NT, IT, OFF0, OFF1, OFF2, WAVE, TB, TMP, NVM1 = 50, 51, 52, 53, 54, 55, 56, 58, 
 RAWC, RAWN, SH, SHM2, PSEL = 74, 77, 78, 79, 72   # Q8_0 builds: raw buffer to dequantize / to load into (OFF3's and a free register), byte shifts and the
                                                   # v_perm selector of the dequantizer (QP's and SPITCH's registers once the prologue is done with them)
 RAWB, DSTB, DZ = 197, 198, 199                    # Q8_0 builds: per-lane raw window / f16 destination offsets, all-ones where this lane's row is valid
-SCL, L2E, MSK = 77, 73, 78   # mask builds: scale, log2(e) (the register of SCLS until the epilogue), mask base (QP's registers once Q is loaded)
+SCL, L2E, MSK = (82, 73, 80) if Q8 else (77, 73, 78)   # mask builds: scale, log2(e) (the register of SCLS until the epilogue), mask base (QP's registers once Q is loaded;
+                                                        # Q8_0 builds keep the dequantizer's scalars there and take s80..s83)
 EXS, S0, S1, S2, S3, DMAB, NVAL, THR, PG0, RSC, SPITCH, SCLS, OFF3, VMW, OSTR, QP = 60, 62, 63, 64, 65, 66, 67, 68, 69, 70, 72, 73, 74, 75, 76, 78
 
 out = []
@@ -788,10 +789,11 @@ def main():
     e("ds_read_b128 %s, %s" % (v(T[0], 4), v(X0)))
     e("ds_read_b128 %s, %s offset:16" % (v(T[4], 4), v(X0)))
     e("s_waitcnt lgkmcnt(0)")
-    e("v_mov_b32 %s, %s" % (v(OPTR), v(T[2])))
-    e("v_mov_b32 %s, %s" % (v(OPTR + 1), v(T[3])))
-    e("v_mov_b32 %s, %s" % (v(MLPTR), v(T[4])))
-    e("v_mov_b32 %s, %s" % (v(MLPTR + 1), v(T[5])))
+    if not RELOAD_PTRS:
+        e("v_mov_b32 %s, %s" % (v(OPTR), v(T[2])))
+        e("v_mov_b32 %s, %s" % (v(OPTR + 1), v(T[3])))
+        e("v_mov_b32 %s, %s" % (v(MLPTR), v(T[4])))
+        e("v_mov_b32 %s, %s" % (v(MLPTR + 1), v(T[5])))
     if MASK:
         e("v_mov_b32 %s, %s" % (v(MOFF), v(T[0])))
     # lane geometry
@@ -1062,6 +1064,15 @@ def main():
     e("s_nop 1")
     e("v_cndmask_b32 %s, %s, %s, vcc" % (v(T[2]), v(T[2]), v(T[3])))
     e("%s:" % lab_part)
+    if RELOAD_PTRS:
+        # bytes 8..23 of this thread's hand-off record: the output pointer and the (m, l) pointer
+        e("s_lshl_b32 %s, %s, 11" % (s(S0), s(WAVE)))
+        e("v_lshlrev_b32 %s, 5, %s" % (v(X0), v(LANE)))
+        e("v_add_u32 %s, %s, %s" % (v(X0), s(S0), v(X0)))
+        e("v_add_u32 %s, %d, %s" % (v(X0), HOFF, v(X0)))
+        e("ds_read_b64 %s, %s offset:8" % (v(OPTR, 2), v(X0)))
+        e("ds_read_b64 %s, %s offset:16" % (v(MLPTR, 2), v(X0)))
+        e("s_waitcnt lgkmcnt(0)")
     # rows past n_rows store nothing
     e("v_cmp_ne_u64 vcc, 0, %s" % v(OPTR, 2))
     e("s_mov_b64 %s, exec" % s(EXS, 2))
@@ -1125,7 +1136,7 @@ def main():
         e("s_waitcnt lgkmcnt(0)")
         e("s_barrier")
 
-    print("// generated by gen_decode_asm.py%s%s -- do not edit" % (" --q8" if Q8 else " --f16" if F16 else "", " --mask" if MASK else ""))
+    print("// generated by gen_decode_asm.py%s%s -- do not edit" % (" --q8" if Q8 else " --f16" if "--f16" in sys.argv else "", " --mask" if MASK else ""))
     for ln in out:
         print('"%s\\n\\t"' % ln)
 

@@ -28,7 +28,7 @@ constexpr int lds_total(int kvt) { return sched_off(kvt) + (2 * SCHED_MAX_SEQ + 
 #define MLA_DECODE_CLOBBERS \
     "memory", "vcc", "scc", "s40", "s41", "s42", "s43", "s44", "s45", "s46", "s47", "s48", "s49", "s50", "s51", \
     "s52", "s53", "s54", "s55", "s56", "s57", "s58", "s59", "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", \
-    "s68", "s69", "s70", "s71", "s72", "s73", "s74", "s75", "s76", "s77", "s78", "s79", "v0", "v1", "v2", "v3", "v4", \
+    "s68", "s69", "s70", "s71", "s72", "s73", "s74", "s75", "s76", "s77", "s78", "s79", "s80", "s81", "s82", "s83", "v0", "v1", "v2", "v3", "v4", \
     "v5", "v6", "v7", "v8", "v9", "v10", "v11", "v12", "v13", "v14", "v15", "v16", "v17", "v18", "v19", "v20", "v21", \
     "v22", "v23", "v24", "v25", "v26", "v27", "v28", "v29", "v30", "v31", "v32", "v33", "v34", "v35", "v36", "v37", \
     "v38", "v39", "v40", "v41", "v42", "v43", "v44", "v45", "v46", "v47", "v48", "v49", "v50", "v51", "v52", "v53", \
@@ -145,7 +145,6 @@ __device__ __forceinline__ void sched_prefix(const KParams & p) {
 template <int KVT, bool MASK>
 __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
     constexpr int HANDOFF_OFF = handoff_off(KVT);
-    static_assert(!(KVT == SRC_Q8 && MASK), "no masked Q8_0 build of the wave program");
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
     // (wave and lane are taken from a scalar and from the exec-mask count rather than kept in a vector register: the wave
@@ -336,7 +335,11 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
     const int s_scale = __builtin_amdgcn_readfirstlane(__float_as_int(p.scale));
     const int s_ostr = __builtin_amdgcn_readfirstlane(p.slot_rows * 16);  // bytes between the partial rows of column groups c and c+1
 
-    if constexpr (KVT == SRC_Q8) {
+    if constexpr (KVT == SRC_Q8 && MASK) {
+        asm volatile(
+#include "mla_decode_asm_q8_mask.inc"
+            : : MLA_DECODE_INPUTS : MLA_DECODE_CLOBBERS);
+    } else if constexpr (KVT == SRC_Q8) {
         asm volatile(
 #include "mla_decode_asm_q8.inc"
             : : MLA_DECODE_INPUTS : MLA_DECODE_CLOBBERS);
@@ -463,11 +466,21 @@ size_t decode_fast_lds_bytes(int kv_type) { return (size_t) lds_total(kv_type ==
 
 size_t decode_fast_qpack_bytes(int n_seq, int n_row_blocks) { return (size_t) n_seq * n_row_blocks * 4 * KSTEPS * 1024; }
 
-// Q8_0 rows with a mask: there is no masked build of the Q8_0 wave program.  The cache is expanded into f16 rows in the
-// workspace -- the very f16 values the Q8_0 build feeds its MFMAs -- and the masked f16 build runs on that copy, with Q
-// quantized the Q8_0 way.  Costs a pass over the whole cache (612 bytes read, 1152 written per row), so only up to 1 GiB.
+// The Q8_0 wave program copies a raw tile as one run of 19584 bytes in 16-byte pieces: packed rows, 16-byte aligned tiles
+// (tiles start on multiples of 32 rows: 32 * 612 = 16 * 1224), whole tiles inside the allocation (always true for pages; a
+// contiguous KV must end on a tile boundary).
+static bool q8_raw_tiles_ok(const mla_attn_args * a) {
+    if (a->kv_nb1 != Q8_ROW || ((uintptr_t) a->kv & 15)) return false;
+    if (!a->block_table && ((a->kv_nb3 & 15) || a->n_kv % TILE_TOK)) return false;
+    return true;
+}
+
+// Q8_0 rows with a mask that the Q8_0 wave program cannot take as raw tiles (padded rows, a misaligned base, a contiguous
+// cache that does not end on a tile boundary): the cache is expanded into f16 rows in the workspace -- the very f16
+// values the Q8_0 build feeds its MFMAs -- and the masked f16 build runs on that copy, with Q quantized the Q8_0 way.
+// Costs a pass over the whole cache (612 bytes read, 1152 written per row), so only up to 1 GiB.
 int64_t decode_fast_q8_copy_rows(const mla_attn_args * a) {
-    if (a->kv_type != MLA_TYPE_Q8_0 || !a->mask || a->kv_nb1 < Q8_ROW) return 0;
+    if (a->kv_type != MLA_TYPE_Q8_0 || !a->mask || a->kv_nb1 < Q8_ROW || q8_raw_tiles_ok(a)) return 0;
     const int64_t rows = a->block_table ? a->n_kv : a->n_kv * (a->kv_nb3 ? a->n_seq : 1);
     return rows > 0 && rows * ROW_BYTES <= ((int64_t) 1 << 30) ? rows : 0;
 }
@@ -476,12 +489,7 @@ bool decode_fast_applicable(const mla_attn_args * a) {
     if (a->kv_type != MLA_TYPE_BF16 && a->kv_type != MLA_TYPE_F16 && a->kv_type != MLA_TYPE_Q8_0) return false;
     if ((a->dv != 512 && a->dv != 576) || (a->flags & MLA_FLAG_F16_ACC_STRICT)) return false;   // 576: two passes, V = columns 0.. and 64..
     const bool q8_copy = decode_fast_q8_copy_rows(a) > 0;
-    if (a->kv_type == MLA_TYPE_Q8_0 && !q8_copy) {
-        // raw tiles are copied as one run of 19584 bytes in 16-byte pieces: packed rows, 16-byte aligned tiles, whole tiles
-        // inside the allocation (always true for pages; a contiguous KV must end on a tile boundary); no masked build
-        if (a->mask || a->kv_nb1 != Q8_ROW || ((uintptr_t) a->kv & 15)) return false;
-        if (!a->block_table && ((a->kv_nb3 & 15) || a->n_kv % TILE_TOK)) return false;
-    }
+    if (a->kv_type == MLA_TYPE_Q8_0 && !q8_copy && !q8_raw_tiles_ok(a)) return false;
     if (a->logit_softcap != 0.0f || a->max_bias > 0.0f) return false;
     // 16-bit rows must be packed: the per-lane offsets of the tile copy are kept as 16-bit values (31 * 1152 + 1136 < 65536)
     if (a->kv_type != MLA_TYPE_Q8_0 && a->kv_nb1 != ROW_BYTES) return false;   // (the f16 copy of a Q8_0 cache is packed by construction)
@@ -550,7 +558,7 @@ hipError_t launch_decode_fast(const KParams & kp, int kv_type, dim3 grid, hipStr
     else if (kv_type == MLA_TYPE_F16) hipLaunchKernelGGL(mla_q_pack_kernel<true>, dim3(n_rb, n_seq, KSTEPS + extra), dim3(NTHREADS), 0, st, kp);
     else                              hipLaunchKernelGGL(mla_q_pack_kernel<false>, dim3(n_rb, n_seq, KSTEPS + extra), dim3(NTHREADS), 0, st, kp);
     if (m && with_prepass) hipLaunchKernelGGL(mla_mask_extent_kernel, dim3(n_rb, MASK_EXT_CHUNKS), dim3(NTHREADS), 0, st, kp);
-    if (kv_type == MLA_TYPE_Q8_0) return launch_variant<SRC_Q8, false>(kp, grid, st);
+    if (kv_type == MLA_TYPE_Q8_0) return m ? launch_variant<SRC_Q8, true>(kp, grid, st) : launch_variant<SRC_Q8, false>(kp, grid, st);
     if (kv_type == MLA_TYPE_F16)  return m ? launch_variant<SRC_F16, true>(kp, grid, st) : launch_variant<SRC_F16, false>(kp, grid, st);
     return m ? launch_variant<SRC_BF16, true>(kp, grid, st) : launch_variant<SRC_BF16, false>(kp, grid, st);
 }

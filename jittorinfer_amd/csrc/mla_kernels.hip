@@ -701,7 +701,7 @@ int make_plan(const mla_attn_args * a, Plan * pl) {
     const int64_t pages_per_split = (n_pages + splits - 1) / splits;
     pl->split_tokens = (int) (pages_per_split * MLA_PAGE_TOKENS);
     pl->n_splits     = (int) ((n_pages + pages_per_split - 1) / pages_per_split);
-    pl->lds_bytes    = pl->variant == 2 ? decode_fast_lds_bytes(a->mask && a->kv_type == MLA_TYPE_Q8_0 ? MLA_TYPE_F16 : a->kv_type) : 2 * TILE_BYTES + (a->kv_type == MLA_TYPE_Q8_0 ? Q8_TILE_RAW : 0);
+    pl->lds_bytes    = pl->variant == 2 ? decode_fast_lds_bytes(decode_fast_q8_copy_rows(a) > 0 ? MLA_TYPE_F16 : a->kv_type) : 2 * TILE_BYTES + (a->kv_type == MLA_TYPE_Q8_0 ? Q8_TILE_RAW : 0);
     if (pl->variant == 2) pl->ws_qpack = decode_fast_qpack_bytes(a->n_seq, pl->n_row_blocks);
     if (pl->variant == 2) { pl->kvcopy_rows = decode_fast_q8_copy_rows(a); pl->ws_kvcopy = (size_t) pl->kvcopy_rows * ROW_BYTES; }
     if (pl->variant == 2 && a->mask) pl->ws_maskext = (size_t) pl->n_row_blocks * 16 * 2 * sizeof(int);  // 16 (first, last) pairs per row block
@@ -854,7 +854,8 @@ static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
     if (pl.balanced) grid = dim3((unsigned) pl.n_wg, 1, 1);
     int kv_type = a->kv_type;
     if (pl.kvcopy_rows > 0) {
-        // Q8_0 cache + mask: expand the cache to f16 rows (a pre-pass like the Q image) and run the masked f16 build on them
+        // Q8_0 cache + mask that the Q8_0 wave program cannot copy as raw tiles: expand the cache to f16 rows (a pre-pass like
+        // the Q image) and run the masked f16 build on them
         char * copy = ws + align256(pl.ws_part_o) + align256(pl.ws_part_ml) + align256(pl.ws_scores) + align256(pl.ws_qpack) + align256(pl.ws_maskext) + align256(pl.ws_sched);
         if (phases & 4) {
             const hipError_t e = launch_q8_to_f16(kp.kv, kp.kv_nb1, kp.kv_nb3, a->n_kv, copy, pl.kvcopy_rows, st);

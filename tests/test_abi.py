@@ -149,3 +149,16 @@ def test_planner_schedules_without_gpu():
     assert rc == 0 and info.variant == 0 and info.n_passes == 2
     rc, info, _ = _plan(logit_softcap=30.0)                      # softcap: general kernel, 64 rows per workgroup
     assert rc == 0 and info.variant == 0 and info.rows_per_wg == 64
+
+
+@pytest.mark.parametrize("flags,name", [([], "mla_decode_asm.inc"), (["--f16"], "mla_decode_asm_f16.inc"), (["--mask"], "mla_decode_asm_mask.inc"),
+                                        (["--f16", "--mask"], "mla_decode_asm_f16_mask.inc"), (["--q8"], "mla_decode_asm_q8.inc"),
+                                        (["--q8", "--mask"], "mla_decode_asm_q8_mask.inc")])
+def test_committed_wave_programs_are_what_the_generator_emits(flags, name):
+    """The six instruction streams the decode kernel includes are generated files: each equals the generator's output."""
+    import subprocess
+    import sys
+    csrc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "jittorinfer_amd", "csrc")
+    got = subprocess.run([sys.executable, os.path.join(csrc, "gen_decode_asm.py")] + flags, capture_output=True, text=True, check=True).stdout
+    with open(os.path.join(csrc, name)) as f:
+        assert got == f.read(), "%s is stale: regenerate it with gen_decode_asm.py %s" % (name, " ".join(flags))

@@ -153,7 +153,7 @@ def test_masked_prefill_pipelined_kernel(gpu, k_type, n_splits):
 def test_masked_decode_random_mask(gpu, n_splits, k_type):
     """Contiguous KV, 128 heads, 3 query tokens: a mask of finite biases and -inf holes, one query token whose keys are
     all masked (NaN rows, like the reference's 0 * (1/0)), one that sees only the first 40 keys (whole splits masked).
-    Q8_0: the masked f16 build on the f16 expansion of the cache."""
+    Q8_0: the masked build of the Q8_0 wave program."""
     rng = np.random.default_rng(50 + n_splits)
     n_kv, n_tok = 512, 3
     q = rng.standard_normal((2, 128, n_tok, 576)).astype(np.float32)
@@ -168,6 +168,46 @@ def test_masked_decode_random_mask(gpu, n_splits, k_type):
     want = O.flash_attn_ext(q, k, k_type, dv=512, mask=mask, scale=U.SCALE)
     assert np.isnan(want[:, 1]).all()
     print(U.check(got[..., :512], want, "masked decode"))
+
+
+@pytest.mark.parametrize("how", ["padded_rows", "misaligned_base"])
+def test_masked_q8_cache_the_wave_program_cannot_tile(gpu, how):
+    """A masked launch over Q8_0 rows that are not packed (640-byte pitch) or whose base is not 16-byte aligned cannot be
+    copied as raw tiles: the cache is expanded to f16 rows in the workspace and the masked f16 build runs on the copy.
+    Same f16 operands, same order of operations: the result equals the packed, aligned launch bit for bit."""
+    import torch
+    import jittorinfer_amd as J
+    rng = np.random.default_rng(61)
+    n_kv, n_tok = 768, 2
+    q = rng.standard_normal((2, 128, n_tok, 576)).astype(np.float32)
+    k = U.encode_kv(rng.standard_normal((2, n_kv, 576)).astype(np.float32), O.TYPE_Q8_0, q8_scale=1.0 / 32)
+    m = (rng.standard_normal((n_tok, n_kv)) * 2).astype(np.float32)
+    m[rng.random((n_tok, n_kv)) < 0.3] = -np.inf
+    m[1, 500:] = -np.inf
+    mask = m.astype(np.float16).view(np.uint16)
+    want = O.flash_attn_ext(q, k, O.TYPE_Q8_0, dv=512, mask=mask, scale=U.SCALE)
+    tq, tm = torch.from_numpy(q).to(gpu), torch.from_numpy(mask.view(np.float16)).to(gpu)
+    tk = torch.from_numpy(k).to(gpu)
+    if how == "padded_rows":
+        wide = torch.full((2, n_kv, 640), 0x7b, dtype=torch.uint8, device=gpu)
+        wide[..., :612] = tk
+        tk2 = wide[..., :612]
+    else:
+        flat = torch.full((2 * n_kv * 612 + 16,), 0x7b, dtype=torch.uint8, device=gpu)
+        flat[4:4 + 2 * n_kv * 612] = tk.reshape(-1)
+        tk2 = flat[4:4 + 2 * n_kv * 612].view(2, n_kv, 612)
+        assert tk2.data_ptr() % 16 == 4
+    kw = dict(dv=512, mask=tm, scale=U.SCALE)
+    assert J.plan(tq, tk, J.MLA_TYPE_Q8_0, **kw)["variant"] == 2 and J.plan(tq, tk2, J.MLA_TYPE_Q8_0, **kw)["variant"] == 2
+    def workspace(k_):
+        import ctypes as C
+        a, _, keep = J.capi.make_args(tq, k_, J.MLA_TYPE_Q8_0, **kw)
+        return J.library().mla_attn_workspace_size(C.byref(a))
+    assert workspace(tk2) >= workspace(tk) + 2 * n_kv * 1152        # room for the f16 copy
+    packed = J.ggml_flash_attn_ext(tq, tk, J.MLA_TYPE_Q8_0, **kw)[..., :512].cpu().numpy()
+    copied = J.ggml_flash_attn_ext(tq, tk2, J.MLA_TYPE_Q8_0, **kw)[..., :512].cpu().numpy()
+    print(U.check(packed, want, "masked Q8_0, raw tiles"), U.check(copied, want, "masked Q8_0, f16 copy"))
+    assert np.array_equal(packed.view(np.uint32), copied.view(np.uint32))
 
 
 @pytest.mark.parametrize("k_type", [O.TYPE_BF16, O.TYPE_Q8_0])
