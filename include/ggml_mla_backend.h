@@ -39,6 +39,16 @@
  *                           src/llama-graph-attn.cpp:277; kv_states, src/llama-graph-deepseek2.cpp:235)
  * Every other op except the no-op view ops (NONE, RESHAPE, VIEW, PERMUTE, TRANSPOSE) is reported unsupported, so
  * the reference's scheduler keeps it on another backend (ggml/src/ggml-backend.cpp:820-846).
+ *
+ * Besides the device buffer type ("HIPMLA<i>") every device offers, like the reference's own accelerator backend
+ * (ggml/src/ggml-cann/ggml-cann.cpp:1252-1365, :2192-2219, :2365-2410):
+ *   get_host_buffer_type   "HIPMLA<i>_Host": pinned host memory, is_host, which the reference asks for to hold the CPU
+ *                          backend's compute buffer and the logits (src/llama-context-load-utils.cpp:116-123,
+ *                          src/llama-context.cpp:181); pageable memory when pinning fails
+ *   event_new / event_free / event_synchronize and the backend's event_record / event_wait: HIP events on the
+ *                          backend's stream, which ggml_backend_sched uses to keep several copies of a graph's inputs in
+ *                          flight (ggml/src/ggml-backend.cpp:1508-1530, :1576-1580, :1630-1634)
+ * and reports caps {async, host_buffer, events} (struct ggml_backend_dev_caps, ggml/include/ggml-backend.h:145-154).
  */
 #ifndef GGML_MLA_BACKEND_H
 #define GGML_MLA_BACKEND_H

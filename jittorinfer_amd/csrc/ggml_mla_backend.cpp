@@ -52,6 +52,8 @@ struct device_ctx {
     std::string name;         // "HIPMLA0"
     std::string description;  // hipDeviceProp_t::name
     backend_buffer_type buft;
+    backend_buffer_type host_buft;   // pinned host memory (the reference's "CANN_Host", ggml/src/ggml-cann/ggml-cann.cpp:1252-1365)
+    std::string         host_name;   // "HIPMLA0_Host"
 };
 
 struct buffer_ctx {
@@ -172,11 +174,11 @@ const backend_buffer_i k_buffer_iface = {
 
 typedef backend_buffer * (*buffer_init_fn)(backend_buffer_type *, backend_buffer_i, void *, size_t);
 
-backend_buffer * make_buffer(backend_buffer_type * buft, void * context, size_t size) {
+backend_buffer * make_buffer(backend_buffer_type * buft, const backend_buffer_i & iface, void * context, size_t size) {
     static buffer_init_fn host_init = (buffer_init_fn) dlsym(RTLD_DEFAULT, "ggml_backend_buffer_init");
-    if (host_init) return host_init(buft, k_buffer_iface, context, size);
+    if (host_init) return host_init(buft, iface, context, size);
     // stand-alone use (no ggml in the process): same object the host would have built (ggml-backend.cpp buffer_init)
-    return new backend_buffer{ k_buffer_iface, buft, context, size, BUFFER_USAGE_ANY };
+    return new backend_buffer{ iface, buft, context, size, BUFFER_USAGE_ANY };
 }
 
 // ---------------------------------------------------------------- buffer type
@@ -193,10 +195,70 @@ backend_buffer * buft_alloc_buffer(backend_buffer_type * buft, size_t size) {
         log_error("allocating %.2f MiB on device %d failed: %s", size / 1048576.0, dc->index, hipGetErrorString(e));
         return nullptr;
     }
-    return make_buffer(buft, new buffer_ctx{ dc->index, p }, size);
+    return make_buffer(buft, k_buffer_iface, new buffer_ctx{ dc->index, p }, size);
 }
 size_t buft_get_alignment(backend_buffer_type *) { return 256; }
 bool   buft_is_host(backend_buffer_type *) { return false; }
+
+// ---------------------------------------------------------------- pinned host buffer type
+// What the reference asks a GPU device for to hold the CPU backend's compute buffer and the logits, "for faster transfer
+// of the intermediate state" (src/llama-context-load-utils.cpp:116-123, src/llama-context.cpp:181): host memory that
+// the CPU backend computes in (is_host) and that copies to and from the device need no staging for.  Counterpart of
+// ggml_backend_cann_host_buffer_type (ggml/src/ggml-cann/ggml-cann.cpp:1323-1365); the buffer functions are the plain
+// memory operations of the CPU buffer (ggml/src/ggml-backend.cpp:2022-2085), which this library cannot borrow without
+// linking ggml.
+
+struct host_buffer_ctx {
+    void * base;
+    bool   pinned;   // false: the pinned allocation failed and the buffer is ordinary aligned memory
+};
+
+void host_buffer_free(backend_buffer * buffer) {
+    host_buffer_ctx * ctx = (host_buffer_ctx *) buffer->context;
+    if (ctx->pinned) (void) hipHostFree(ctx->base); else free(ctx->base);
+    delete ctx;
+}
+void * host_buffer_get_base(backend_buffer * buffer) { return ((host_buffer_ctx *) buffer->context)->base; }
+void host_buffer_memset_tensor(backend_buffer *, tensor * t, uint8_t value, size_t offset, size_t size) { memset((char *) t->data + offset, value, size); }
+void host_buffer_set_tensor(backend_buffer *, tensor * t, const void * data, size_t offset, size_t size) { memcpy((char *) t->data + offset, data, size); }
+void host_buffer_get_tensor(backend_buffer *, const tensor * t, void * data, size_t offset, size_t size) { memcpy(data, (const char *) t->data + offset, size); }
+bool host_buffer_cpy_tensor(backend_buffer *, const tensor * src, tensor * dst) {
+    if (!src->buffer || !src->buffer->buft) return false;
+    backend_buffer_type * sb = src->buffer->buft;
+    if (!(sb->iface.is_host && sb->iface.is_host(sb))) return false;
+    memcpy(dst->data, src->data, tensor_nbytes(src));
+    return true;
+}
+void host_buffer_clear(backend_buffer * buffer, uint8_t value) { memset(((host_buffer_ctx *) buffer->context)->base, value, buffer->size); }
+
+const backend_buffer_i k_host_buffer_iface = {
+    /* free_buffer   */ host_buffer_free,
+    /* get_base      */ host_buffer_get_base,
+    /* init_tensor   */ nullptr,
+    /* memset_tensor */ host_buffer_memset_tensor,
+    /* set_tensor    */ host_buffer_set_tensor,
+    /* get_tensor    */ host_buffer_get_tensor,
+    /* cpy_tensor    */ host_buffer_cpy_tensor,
+    /* clear         */ host_buffer_clear,
+    /* reset         */ nullptr,
+};
+
+const char * host_buft_get_name(backend_buffer_type * buft) { return ((device_ctx *) buft->context)->host_name.c_str(); }
+backend_buffer * host_buft_alloc_buffer(backend_buffer_type * buft, size_t size) {
+    device_ctx * dc = (device_ctx *) buft->context;
+    if (size == 0) size = 1;
+    void * p = nullptr;
+    bool pinned = HIP_OK(hipSetDevice(dc->index)) && hipHostMalloc(&p, size, hipHostMallocDefault) == hipSuccess && p;
+    if (!pinned) {
+        // like the reference's host buffer (ggml-cann.cpp:1327-1331): fall back to ordinary memory rather than fail
+        (void) hipGetLastError();
+        log_error("pinning %.2f MiB of host memory failed: using pageable memory", size / 1048576.0);
+        if (posix_memalign(&p, 64, size) != 0) return nullptr;
+    }
+    return make_buffer(buft, k_host_buffer_iface, new host_buffer_ctx{ p, pinned }, size);
+}
+size_t host_buft_get_alignment(backend_buffer_type *) { return 64; }
+bool   host_buft_is_host(backend_buffer_type *) { return true; }
 
 // ---------------------------------------------------------------- op support
 
@@ -371,7 +433,13 @@ void backend_synchronize(backend * be) {
 
 int compute_flash_attn(backend_ctx * ctx, const tensor * dst) {
     const char * why = nullptr;
-    if (!mla_node_ok(dst, &why)) { log_error("FLASH_ATTN_EXT node '%s' rejected: %s", dst->name, why); return STATUS_FAILED; }
+    if (!mla_node_ok(dst, &why)) {
+        const tensor * q = dst->src[0], * k = dst->src[1];
+        log_error("FLASH_ATTN_EXT node '%s' rejected: %s (q '%s' [%lld,%lld,%lld,%lld], k '%s' [%lld,%lld,%lld,%lld])", dst->name, why,
+                  q ? q->name : "-", q ? (long long) q->ne[0] : 0, q ? (long long) q->ne[1] : 0, q ? (long long) q->ne[2] : 0, q ? (long long) q->ne[3] : 0,
+                  k ? k->name : "-", k ? (long long) k->ne[0] : 0, k ? (long long) k->ne[1] : 0, k ? (long long) k->ne[2] : 0, k ? (long long) k->ne[3] : 0);
+        return STATUS_FAILED;
+    }
     const tensor * q = dst->src[0], * k = dst->src[1], * v = dst->src[2], * mask = dst->src[3];
     const tensor * bt = dst->src[4], * lens = dst->src[5];
     if (!q->data || !k->data || !dst->data || v->data != k->data) { log_error("node '%s': operands not allocated, or v does not alias k", dst->name); return STATUS_FAILED; }
@@ -505,6 +573,25 @@ int backend_graph_compute(backend * be, cgraph * g) {
     return STATUS_SUCCESS;
 }
 
+// Events (ggml-backend-impl.h:120-122, :132-135, :183-185; the reference's own: ggml-cann.cpp:2192-2219, :2365-2410): what
+// ggml_backend_sched uses instead of full synchronisations when
+// it keeps several copies of a graph's inputs in flight (ggml-backend.cpp:1508-1530, :1576-1580).
+bool event_is_ours(const backend_event * ev);
+void backend_event_record(backend * be, backend_event * ev) {
+    backend_ctx * ctx = (backend_ctx *) be->context;
+    (void) hipSetDevice(ctx->device);
+    if (!HIP_OK(hipEventRecord((hipEvent_t) ev->context, ctx->stream))) log_error("event_record failed");
+}
+void backend_event_wait(backend * be, backend_event * ev) {
+    backend_ctx * ctx = (backend_ctx *) be->context;
+    (void) hipSetDevice(ctx->device);
+    if (event_is_ours(ev)) {
+        if (!HIP_OK(hipStreamWaitEvent(ctx->stream, (hipEvent_t) ev->context, 0))) log_error("event_wait failed");
+    } else if (ev->device && ev->device->iface.event_synchronize) {
+        ev->device->iface.event_synchronize(ev->device, ev);   // another backend's event: wait for it on the host
+    }
+}
+
 const backend_i k_backend_iface = {
     /* get_name           */ backend_get_name,
     /* free               */ backend_free,
@@ -517,8 +604,8 @@ const backend_i k_backend_iface = {
     /* graph_plan_update  */ nullptr,
     /* graph_plan_compute */ nullptr,
     /* graph_compute      */ backend_graph_compute,
-    /* event_record       */ nullptr,
-    /* event_wait         */ nullptr,
+    /* event_record       */ backend_event_record,
+    /* event_wait         */ backend_event_wait,
 };
 
 // ---------------------------------------------------------------- device
@@ -536,7 +623,7 @@ void device_get_props(backend_device * dev, dev_props * props) {
     props->description = device_get_description(dev);
     props->type        = DEVICE_TYPE_GPU;
     device_get_memory(dev, &props->memory_free, &props->memory_total);
-    props->caps = dev_caps{ /* async */ true, /* host_buffer */ false, /* buffer_from_host_ptr */ false, /* events */ false };
+    props->caps = dev_caps{ /* async */ true, /* host_buffer */ true, /* buffer_from_host_ptr */ false, /* events */ true };
 }
 backend * device_init_backend(backend_device * dev, const char *) {
     device_ctx * dc = (device_ctx *) dev->context;
@@ -549,6 +636,23 @@ backend * device_init_backend(backend_device * dev, const char *) {
 }
 backend_buffer_type * device_get_buffer_type(backend_device * dev) { return &((device_ctx *) dev->context)->buft; }
 bool device_supports_buft(backend_device * dev, backend_buffer_type * buft) { return buft == device_get_buffer_type(dev); }
+backend_buffer_type * device_get_host_buffer_type(backend_device * dev) { return &((device_ctx *) dev->context)->host_buft; }
+
+backend_event * device_event_new(backend_device * dev) {
+    device_ctx * dc = (device_ctx *) dev->context;
+    hipEvent_t ev = nullptr;
+    if (!HIP_OK(hipSetDevice(dc->index)) || !HIP_OK(hipEventCreateWithFlags(&ev, hipEventDisableTiming))) return nullptr;
+    return new backend_event{ dev, ev };
+}
+void device_event_free(backend_device *, backend_event * ev) {
+    if (!ev) return;
+    (void) hipEventDestroy((hipEvent_t) ev->context);
+    delete ev;
+}
+void device_event_synchronize(backend_device *, backend_event * ev) {
+    if (!HIP_OK(hipEventSynchronize((hipEvent_t) ev->context))) log_error("event_synchronize failed");
+}
+bool event_is_ours(const backend_event * ev) { return ev && ev->device && ev->device->iface.event_new == device_event_new; }
 
 const backend_device_i k_device_iface = {
     /* get_name             */ device_get_name,
@@ -558,14 +662,14 @@ const backend_device_i k_device_iface = {
     /* get_props            */ device_get_props,
     /* init_backend         */ device_init_backend,
     /* get_buffer_type      */ device_get_buffer_type,
-    /* get_host_buffer_type */ nullptr,
+    /* get_host_buffer_type */ device_get_host_buffer_type,
     /* buffer_from_host_ptr */ nullptr,
     /* supports_op          */ device_supports_op,
     /* supports_buft        */ device_supports_buft,
     /* offload_op           */ nullptr,
-    /* event_new            */ nullptr,
-    /* event_free           */ nullptr,
-    /* event_synchronize    */ nullptr,
+    /* event_new            */ device_event_new,
+    /* event_free           */ device_event_free,
+    /* event_synchronize    */ device_event_synchronize,
 };
 
 // ---------------------------------------------------------------- registry
@@ -607,6 +711,10 @@ void init_registry() {
         dc->buft.iface   = backend_buffer_type_i{ buft_get_name, buft_alloc_buffer, buft_get_alignment, nullptr, nullptr, buft_is_host };
         dc->buft.device  = dev;
         dc->buft.context = dc;
+        dc->host_name         = dc->name + "_Host";
+        dc->host_buft.iface   = backend_buffer_type_i{ host_buft_get_name, host_buft_alloc_buffer, host_buft_get_alignment, nullptr, nullptr, host_buft_is_host };
+        dc->host_buft.device  = dev;
+        dc->host_buft.context = dc;
         g_device_ctx.push_back(dc);
         g_devices.push_back(dev);
     }

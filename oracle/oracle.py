@@ -241,7 +241,7 @@ def ref_backend_flash_attn_ext(so_path, q, k, k_type, dv=576, mask=None, block_t
                                       mask.ctypes.data if mask is not None else None, mask_ne0,
                                       block_table.ctypes.data if block_table is not None else None, max_blocks,
                                       seq_lens.ctypes.data if seq_lens is not None else None,
-                                      scale, max_bias, softcap, 1 if use_sched else 0, out.ctypes.data, info, 512)
+                                      scale, max_bias, softcap, int(use_sched), out.ctypes.data, info, 512)
     if rc != 0:
         raise RuntimeError("ref_backend_flash_attn_ext failed: %d (%s)" % (rc, info.value.decode()))
     return out, info.value.decode()

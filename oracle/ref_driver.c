@@ -83,8 +83,52 @@ int ref_flash_attn_ext(int k_type, int64_t DK, int64_t n_tok, int64_t n_head, in
  * dv: DK passes V := K; 512 passes a 512-wide view of K as V (which ggml-cpu itself asserts on, ggml-cpu.c:11943).
  * use_sched != 0 runs the graph through ggml_backend_sched with {loaded backend, CPU} the way llama_decode does
  * (ggml-backend.cpp:1493-1587, :1727-1739) instead of calling ggml_backend_graph_compute directly.
+ * use_sched == 2 sets the scheduler up the way llama's context does (src/llama-context-load-utils.cpp:108-131): the CPU
+ * backend's compute buffer comes from the device's host buffer type, pipeline parallelism is on (several copies of the
+ * inputs, ordered by the backends' events), Q reaches the node through an op the CPU backend runs (ggml_scale by 1) and
+ * the result leaves through another; the graph is computed three times with Q, 2Q (softmax scale halved) and Q again.
  * Returns 0 on success; negative for set-up failures; the ggml_status otherwise.
  */
+struct fa_graph {
+    struct ggml_context * ctx;
+    struct ggml_tensor *  tq, *tm, *tb, *tl, *q_in, *fa, *o;
+    struct ggml_cgraph *  gf;
+};
+
+/* The node and its operands in a fresh context (llama rebuilds its graph for every decode too: the scheduler rewires the
+ * sources of the nodes it splits, so a graph is computed once).  tk may be NULL: K is then part of this context. */
+static int fa_graph_build(struct fa_graph * g, struct ggml_tensor * tk_in, struct ggml_tensor ** tk_out, enum ggml_type kt,
+                          int64_t DK, int64_t dv, int64_t n_tok, int64_t n_head, int64_t n3, int64_t n_kv, int paged,
+                          int with_mask, int64_t mask_ne0, int64_t max_blocks, float scale, float max_bias, float softcap,
+                          int cpu_ops) {
+    struct ggml_init_params ip = { ggml_tensor_overhead() * 32 + ggml_graph_overhead() + 4096, NULL, true };
+    memset(g, 0, sizeof(*g));
+    g->ctx = ggml_init(ip);
+    if (!g->ctx) return -13;
+    struct ggml_context * ctx = g->ctx;
+    g->tq = ggml_new_tensor_4d(ctx, GGML_TYPE_F32, DK, n_tok, n_head, n3);
+    struct ggml_tensor * tk = tk_in ? tk_in : ggml_new_tensor_4d(ctx, kt, DK, n_kv, 1, paged ? 1 : n3);
+    struct ggml_tensor * tv = tk;
+    if (dv != DK) tv = ggml_view_4d(ctx, tk, dv, tk->ne[1], tk->ne[2], tk->ne[3], tk->nb[1], tk->nb[2], tk->nb[3], 0);
+    g->tm = with_mask ? make_mask(ctx, mask_ne0, n_tok) : NULL;
+    g->tb = paged ? ggml_new_tensor_2d(ctx, GGML_TYPE_I32, max_blocks, n3) : NULL;
+    g->tl = paged ? ggml_new_tensor_1d(ctx, GGML_TYPE_I32, n3) : NULL;
+    ggml_set_input(g->tq);
+    if (g->tm) ggml_set_input(g->tm);
+    if (g->tb) { ggml_set_input(g->tb); ggml_set_input(g->tl); }
+    g->q_in = cpu_ops ? ggml_scale(ctx, g->tq, 1.0f) : g->tq;
+    g->fa = g->o = ggml_flash_attn_ext(ctx, g->q_in, tk, tv, g->tm, scale, max_bias, softcap);
+    ggml_flash_attn_ext_set_prec(g->fa, GGML_PREC_F32);
+    g->fa->src[4] = g->tb; /* same slot convention as ggml_flash_attn_prompt's length tensors, ggml.c:2707-2710 */
+    g->fa->src[5] = g->tl;
+    if (cpu_ops) g->o = ggml_scale(ctx, g->fa, 1.0f);
+    ggml_set_output(g->o);
+    g->gf = ggml_new_graph(ctx);
+    ggml_build_forward_expand(g->gf, g->o);
+    if (tk_out) *tk_out = tk;
+    return 0;
+}
+
 int ref_backend_flash_attn_ext(const char * so_path, int k_type, int64_t DK, int64_t dv, int64_t n_tok, int64_t n_head,
                                int64_t n3, int64_t n_kv, const float * q, const void * k, const uint16_t * mask,
                                int64_t mask_ne0, const int32_t * block_table, int64_t max_blocks,
@@ -105,92 +149,115 @@ int ref_backend_flash_attn_ext(const char * so_path, int k_type, int64_t DK, int
                        ggml_backend_dev_name(dev), ggml_backend_dev_description(dev), (int) ggml_backend_dev_type(dev),
                        ggml_backend_name(be), ggml_backend_buft_name(ggml_backend_dev_buffer_type(dev)));
 
-    const enum ggml_type    kt    = (enum ggml_type) k_type;
-    const int               paged = block_table != NULL;
-    struct ggml_init_params ip    = { ggml_tensor_overhead() * 32 + ggml_graph_overhead() + 4096, NULL, true };
-    struct ggml_context *   ctx   = ggml_init(ip);
-    /* the KV rows live in their own context, allocated up front in the backend's buffer the way
-     * llama_kv_cache_init allocates k_l[il] (src/llama-kv-cache.cpp:82-90,153-158) */
-    struct ggml_init_params ipk    = { ggml_tensor_overhead() * 4, NULL, true };
-    struct ggml_context *   ctx_kv = ggml_init(ipk);
-    if (!ctx || !ctx_kv) { ggml_backend_free(be); return -13; }
-
-    struct ggml_tensor * tq = ggml_new_tensor_4d(ctx, GGML_TYPE_F32, DK, n_tok, n_head, n3);
-    struct ggml_tensor * tk = ggml_new_tensor_4d(use_sched ? ctx_kv : ctx, kt, DK, n_kv, 1, paged ? 1 : n3);
-    struct ggml_tensor * tv = tk;
-    if (dv != DK) tv = ggml_view_4d(ctx, tk, dv, tk->ne[1], tk->ne[2], tk->ne[3], tk->nb[1], tk->nb[2], tk->nb[3], 0);
-    struct ggml_tensor * tm = mask ? make_mask(ctx, mask_ne0, n_tok) : NULL;
-    struct ggml_tensor * tb = paged ? ggml_new_tensor_2d(ctx, GGML_TYPE_I32, max_blocks, n3) : NULL;
-    struct ggml_tensor * tl = paged ? ggml_new_tensor_1d(ctx, GGML_TYPE_I32, n3) : NULL;
-    ggml_set_input(tq);
-    if (tm) ggml_set_input(tm);
-    if (tb) { ggml_set_input(tb); ggml_set_input(tl); }
-
+    const enum ggml_type  kt     = (enum ggml_type) k_type;
+    const int             paged  = block_table != NULL;
+    const int             n_runs = use_sched == 2 ? 3 : 1;
     int                   rc     = 0;
     ggml_backend_buffer_t buf    = NULL;
     ggml_backend_buffer_t buf_kv = NULL;
     ggml_backend_sched_t  sched  = NULL;
     ggml_backend_t        cpu    = NULL;
-    struct ggml_tensor *  o      = NULL;
-    struct ggml_cgraph *  gf     = NULL;
+    struct ggml_tensor *  tk     = NULL;
+    struct fa_graph       g;
+    memset(&g, 0, sizeof(g));
+    /* with a scheduler the KV rows live in their own context, allocated up front in the backend's buffer the way
+     * llama_kv_cache_init allocates k_l[il] (src/llama-kv-cache.cpp:82-90,153-158) */
+    struct ggml_init_params ipk    = { ggml_tensor_overhead() * 4, NULL, true };
+    struct ggml_context *   ctx_kv = ggml_init(ipk);
+    if (!ctx_kv) { ggml_backend_free(be); return -13; }
+    const size_t nq = (size_t) (DK * n_tok * n_head * n3);
+    float *      q2 = (float *) malloc(nq * sizeof(float));
+    float *      d2 = NULL;
+    for (size_t i = 0; i < nq; i++) q2[i] = 2.0f * q[i];
 
     if (use_sched) {
+        tk     = ggml_new_tensor_4d(ctx_kv, kt, DK, n_kv, 1, paged ? 1 : n3);
         buf_kv = ggml_backend_alloc_ctx_tensors(ctx_kv, be);
         if (!buf_kv) { rc = -18; goto done; }
         ggml_backend_buffer_clear(buf_kv, 0); /* src/llama-kv-cache.cpp:158 */
-    }
-    o = ggml_flash_attn_ext(ctx, tq, tk, tv, tm, scale, max_bias, softcap);
-    ggml_flash_attn_ext_set_prec(o, GGML_PREC_F32);
-    o->src[4] = tb; /* same slot convention as ggml_flash_attn_prompt's length tensors, ggml.c:2707-2710 */
-    o->src[5] = tl;
-    ggml_set_output(o);
-    gf = ggml_new_graph(ctx);
-    ggml_build_forward_expand(gf, o);
-    if (!ggml_backend_dev_supports_op(dev, o)) { rc = -14; goto done; }
-
-    if (use_sched) {
+        ggml_backend_tensor_set(tk, k, 0, ggml_nbytes(tk));
         cpu = ggml_backend_init_by_type(GGML_BACKEND_DEVICE_TYPE_CPU, NULL);
         if (!cpu) { rc = -15; goto done; }
-        ggml_backend_t backends[2] = { be, cpu };
-        sched = ggml_backend_sched_new(backends, NULL, 2, GGML_DEFAULT_GRAPH_SIZE, false);
+        ggml_backend_t             backends[2] = { be, cpu };
+        ggml_backend_buffer_type_t bufts[2]    = { ggml_backend_get_default_buffer_type(be), ggml_backend_get_default_buffer_type(cpu) };
+        if (use_sched == 2) {
+            ggml_backend_buffer_type_t   host = ggml_backend_dev_host_buffer_type(dev);
+            struct ggml_backend_dev_props props;
+            ggml_backend_dev_get_props(dev, &props);
+            if (!host || !ggml_backend_buft_is_host(host) || !props.caps.host_buffer || !props.caps.events) { rc = -20; goto done; }
+            if (info) snprintf(info + strlen(info), info_len - strlen(info), " host_buft=%s", ggml_backend_buft_name(host));
+            bufts[1] = host;
+        }
+        sched = ggml_backend_sched_new(backends, bufts, 2, GGML_DEFAULT_GRAPH_SIZE, use_sched == 2);
         if (!sched) { rc = -16; goto done; }
-        /* llama's graph callback pins attention nodes to the layer's device the same way */
-        ggml_backend_sched_set_tensor_backend(sched, o, be);
-        if (!ggml_backend_sched_alloc_graph(sched, gf)) { rc = -16; goto done; }
-        if (ggml_backend_sched_get_tensor_backend(sched, o) != be) { rc = -17; goto done; }
-    } else {
-        ggml_set_input(tk);
-        buf = ggml_backend_alloc_ctx_tensors(ctx, be);
-        if (!buf) { rc = -18; goto done; }
     }
 
-    ggml_backend_tensor_set(tq, q, 0, ggml_nbytes(tq));
-    ggml_backend_tensor_set(tk, k, 0, ggml_nbytes(tk));
-    if (tm) {
-        const size_t nrow = (size_t) tm->ne[1];
-        uint16_t *   md   = (uint16_t *) malloc(nrow * mask_ne0 * 2);
-        for (size_t i = 0; i < nrow; i++)
-            for (int64_t j = 0; j < mask_ne0; j++) md[i * mask_ne0 + j] = (int64_t) i < n_tok ? mask[i * mask_ne0 + j] : 0xfc00;
-        ggml_backend_tensor_set(tm, md, 0, ggml_nbytes(tm));
-        free(md);
-    }
-    if (tb) {
-        ggml_backend_tensor_set(tb, block_table, 0, ggml_nbytes(tb));
-        ggml_backend_tensor_set(tl, seq_lens, 0, ggml_nbytes(tl));
-    }
-    {
-        enum ggml_status st = use_sched ? ggml_backend_sched_graph_compute(sched, gf) : ggml_backend_graph_compute(be, gf);
+    /* use_sched == 2: three asynchronous computes, as consecutive llama_decode calls issue them: every one takes the next
+     * copy of the inputs, and the events keep a copy from being overwritten while the device still reads it */
+    for (int run = 0; run < n_runs; run++) {
+        const float run_scale = run == 1 ? 0.5f * scale : scale;
+        rc = fa_graph_build(&g, tk, use_sched ? NULL : &tk, kt, DK, dv, n_tok, n_head, n3, n_kv, paged, mask != NULL, mask_ne0,
+                            max_blocks, run_scale, max_bias, softcap, use_sched == 2);
+        if (rc) goto done;
+        if (!ggml_backend_dev_supports_op(dev, g.fa)) { rc = -14; goto done; }
+        if (use_sched) {
+            if (run > 0) ggml_backend_sched_reset(sched);
+            /* llama's graph callback pins attention nodes to the layer's device the same way */
+            ggml_backend_sched_set_tensor_backend(sched, g.fa, be);
+            if (!ggml_backend_sched_alloc_graph(sched, g.gf)) { rc = -16; goto done; }
+            if (ggml_backend_sched_get_tensor_backend(sched, g.fa) != be) { rc = -17; goto done; }
+            if (use_sched == 2 && (ggml_backend_sched_get_tensor_backend(sched, g.q_in) != cpu || ggml_backend_sched_get_n_splits(sched) < 3)) { rc = -21; goto done; }
+        } else {
+            ggml_set_input(tk);
+            buf = ggml_backend_alloc_ctx_tensors(g.ctx, be);
+            if (!buf) { rc = -18; goto done; }
+            ggml_backend_tensor_set(tk, k, 0, ggml_nbytes(tk));
+        }
+        ggml_backend_tensor_set(g.tq, run == 1 ? q2 : q, 0, ggml_nbytes(g.tq));
+        if (g.tm) {
+            const size_t nrow = (size_t) g.tm->ne[1];
+            uint16_t *   md   = (uint16_t *) malloc(nrow * mask_ne0 * 2);
+            for (size_t i = 0; i < nrow; i++)
+                for (int64_t j = 0; j < mask_ne0; j++) md[i * mask_ne0 + j] = (int64_t) i < n_tok ? mask[i * mask_ne0 + j] : 0xfc00;
+            ggml_backend_tensor_set(g.tm, md, 0, ggml_nbytes(g.tm));
+            free(md);
+        }
+        if (g.tb) {
+            ggml_backend_tensor_set(g.tb, block_table, 0, ggml_nbytes(g.tb));
+            ggml_backend_tensor_set(g.tl, seq_lens, 0, ggml_nbytes(g.tl));
+        }
+        enum ggml_status st;
+        if (use_sched == 2) {
+            st = ggml_backend_sched_graph_compute_async(sched, g.gf);
+            ggml_backend_sched_synchronize(sched);
+        } else {
+            st = use_sched ? ggml_backend_sched_graph_compute(sched, g.gf) : ggml_backend_graph_compute(be, g.gf);
+        }
         if (st != GGML_STATUS_SUCCESS) { rc = (int) st ? (int) st : -19; goto done; }
+        const size_t nb = ggml_nbytes(g.o);
+        if (run == 1) {
+            /* softmax(0.5 * scale * (2Q).K) is softmax(scale * Q.K) bit for bit: doubling is exact in every rounding step */
+            d2 = (float *) malloc(nb);
+            ggml_backend_tensor_get(g.o, d2, 0, nb);
+            if (memcmp(d2, dst, nb) != 0) { rc = -22; goto done; }
+        } else {
+            if (run == 2) memset(dst, 0xff, nb);
+            ggml_backend_tensor_get(g.o, dst, 0, nb);
+            if (run == 2 && memcmp(d2, dst, nb) != 0) { rc = -23; goto done; }
+        }
+        ggml_free(g.ctx);
+        g.ctx = NULL;
     }
-    ggml_backend_tensor_get(o, dst, 0, ggml_nbytes(o));
 done:
     if (sched) ggml_backend_sched_free(sched);
     if (buf) ggml_backend_buffer_free(buf);
     if (buf_kv) ggml_backend_buffer_free(buf_kv);
     if (cpu) ggml_backend_free(cpu);
-    ggml_free(ctx);
+    if (g.ctx) ggml_free(g.ctx);
     ggml_free(ctx_kv);
     ggml_backend_free(be);
+    free(q2);
+    free(d2);
     return rc;
 }
 

@@ -43,6 +43,31 @@ def test_latent_prefix_view_and_block_table(gpu):
     print(U.check(got[..., :512], want, "paged node through the scheduler"))
 
 
+@pytest.mark.parametrize("paged", [False, True])
+def test_scheduler_set_up_as_llama_sets_it_up(gpu, paged):
+    """The scheduler as the reference's context builds it (src/llama-context-load-utils.cpp:108-131): the CPU backend's
+    compute buffer in the device's pinned host buffer type, pipeline parallelism on (four copies of the inputs ordered
+    by the plugin's events), Q produced by a CPU op and the result consumed by one.  Three asynchronous computes in a row
+    (Q, then 2Q with half the softmax scale, which the driver checks to be bit-identical, then Q again)."""
+    rng = np.random.default_rng(29)
+    if paged:
+        lens = [300, 1, 128, 515]
+        pool, bt, seqs = U.make_paged(rng, lens, O.TYPE_BF16, n_pool_pages=16)
+        q = rng.standard_normal((4, 128, 1, 576)).astype(np.float32)
+        got, info = O.ref_backend_flash_attn_ext(_so(), q, pool, O.TYPE_BF16, dv=512, block_table=bt, seq_lens=lens, scale=U.SCALE, use_sched=2)
+        want = U.oracle_per_seq(q, seqs, O.TYPE_BF16, 512)
+    else:
+        q = rng.standard_normal((2, 16, 2, 576)).astype(np.float32)
+        k = U.encode_kv(rng.standard_normal((2, 200, 576)).astype(np.float32), O.TYPE_BF16)
+        mask = np.where(rng.random((2, 200)) < 0.2, -np.inf, 0.0).astype(np.float16)
+        mask[:, 0] = 0
+        mask = mask.view(np.uint16)
+        got, info = O.ref_backend_flash_attn_ext(_so(), q, k, O.TYPE_BF16, dv=512, mask=mask, scale=U.SCALE, use_sched=2)
+        want = O.flash_attn_ext(q, k, O.TYPE_BF16, dv=512, mask=mask, scale=U.SCALE)
+    assert "host_buft=HIPMLA0_Host" in info
+    print(info, U.check(got[..., :512], want[..., :512], "llama-style scheduler"))
+
+
 @pytest.mark.parametrize("use_sched", [False, True])
 def test_batched_decode_through_the_mask_as_llama_builds_it(gpu, use_sched):
     """The reference's decode batch: one shared cache, one query token per sequence, the f16 mask padded to 64 rows selects
