@@ -536,6 +536,17 @@ def main():
         graph.replay()          # K steps
         torch.cuda.synchronize()
         ms_per_step = (time.perf_counter() - t0) * 1e3 / a.steps
+        # spread of the same measurement: nine more replays of the K steps, each bracketed the same way
+        replays = [ms_per_step * 1e3]
+        for _ in range(9):
+            t0 = time.perf_counter()
+            graph.replay()
+            torch.cuda.synchronize()
+            replays.append((time.perf_counter() - t0) * 1e6 / a.steps)
+        replays.sort()
+        step_stats = {"median": 0.5 * (replays[4] + replays[5]), "p10": replays[1], "p90": replays[8], "replays_of_k_steps": len(replays)}
+    else:
+        step_stats = None
 
     # ---- the dominant kernel alone (the split-K decode kernel, without the Q pre-pack and the combine pass): HIP events
     # on the launch stream around K back-to-back launches (the stream is in order, so this is K kernel durations plus the
@@ -547,6 +558,16 @@ def main():
     e1.record(stream)
     torch.cuda.synchronize()
     kern_ms = e0.elapsed_time(e1) / a.steps
+    # spread over single launches: an event between every two launches of the same loop
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(a.steps + 1)]
+    marks[0].record(stream)
+    for i in range(a.steps):
+        step(i, lib.mla_attn_launch_kernel)
+        marks[i + 1].record(stream)
+    torch.cuda.synchronize()
+    per_launch = sorted(marks[i].elapsed_time(marks[i + 1]) * 1e3 for i in range(a.steps))
+    pick = lambda f: per_launch[min(len(per_launch) - 1, int(f * len(per_launch)))]
+    kern_stats = {"mean": kern_ms * 1e3, "median": pick(0.5), "p10": pick(0.1), "p90": pick(0.9)}
     # and whole steps with events (decode + combine)
     e0.record(stream)
     for i in range(a.steps):
@@ -590,12 +611,13 @@ def main():
         "launch": "eager" if a.eager else "hip graph replay of the K steps",
         "us_per_step_eager": eager_ms_per_step * 1e3,
         "us_per_step_events": step_ms_events * 1e3,
+        "us_per_step_spread": step_stats,
         "tokens_per_s": a.batch / (ms_per_step * 1e-3),
         "pct_hbm_peak": 100.0 * value / HBM_PEAK_GBPS,
         "tflops": flops / (ms_per_step * 1e-3) / 1e12,
         "roofline": {"bound": "hbm", "kernel": "mla_decode_kernel<%s>" % a.kv, "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic,
-                     "algorithmic_bytes_per_launch": kv_bytes, "kernel_us": {"mean": kern_ms * 1e3},
+                     "algorithmic_bytes_per_launch": kv_bytes, "kernel_us": kern_stats,
                      "mfma_tflops": flops / (kern_ms * 1e-3) / 1e12},
         "cpu_baseline": cpu,
         "parity": parity,
