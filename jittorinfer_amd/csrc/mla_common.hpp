@@ -109,6 +109,21 @@ __device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); 
 
 // The pipelined decode kernel (mla_decode_kernel.hip); returns hipErrorInvalidValue for shapes it does not take.
 bool       decode_fast_applicable(const mla_attn_args * a);
+// Raises a kernel's dynamic-LDS limit to the 160 KB of a CU, once per device: the attribute belongs to the function on the
+// device that is current.  `done` is the caller's per-function table (zero-initialised static); a second thread that gets
+// here before the first has finished only repeats the same call.
+constexpr int MLA_MAX_DEVICES = 64;
+inline hipError_t raise_lds_limit(const void * fn, bool (&done)[MLA_MAX_DEVICES]) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= MLA_MAX_DEVICES) return hipErrorInvalidDevice;
+    if (done[dev]) return hipSuccess;
+    e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e == hipSuccess) done[dev] = true;
+    return e;
+}
+
 int64_t    decode_fast_q8_copy_rows(const mla_attn_args * a);   // > 0: Q8_0 + mask on rows the wave program cannot tile runs on an f16 copy of that many rows (workspace)
 hipError_t launch_mask_extent(const KParams & kp, hipStream_t st);   // fills kp.mask_ext: 16 key pairs per block of 128 rows
 hipError_t launch_q8_to_f16(const char * src, int64_t src_nb1, int64_t src_nb3, int64_t rows_per_batch, void * dst, int64_t n_rows, hipStream_t st);

@@ -538,13 +538,9 @@ hipError_t launch_q8_to_f16(const char * src, int64_t src_nb1, int64_t src_nb3, 
 
 template <int KVT, bool MASK>
 static hipError_t launch_variant(const KParams & kp, dim3 grid, hipStream_t st) {
-    static bool attr_done = false;
-    const void * fn = (const void *) mla_decode_kernel<KVT, MASK>;
-    if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        if (e != hipSuccess) return e;
-        attr_done = true;
-    }
+    static bool attr_done[MLA_MAX_DEVICES];
+    const hipError_t e = raise_lds_limit((const void *) mla_decode_kernel<KVT, MASK>, attr_done);
+    if (e != hipSuccess) return e;
     hipLaunchKernelGGL((mla_decode_kernel<KVT, MASK>), grid, dim3(NTHREADS), (size_t) lds_total(KVT), st, kp);
     return hipGetLastError();
 }

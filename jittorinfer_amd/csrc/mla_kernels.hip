@@ -749,12 +749,9 @@ size_t plan_ws(const Plan & pl) {
 template <int SRC, int NDB, int WM, int WD>
 hipError_t launch_tile(const KParams & kp, dim3 grid, size_t lds, hipStream_t st) {
     auto kern = mla_attn_tile_kernel<SRC, NDB, WM, WD>;
-    static bool attr_done = false;  // raising the dynamic LDS limit is a per-function, per-process setting
-    if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute((const void *) kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int) (160 * 1024));
-        if (e != hipSuccess) return e;
-        attr_done = true;
-    }
+    static bool attr_done[MLA_MAX_DEVICES];
+    const hipError_t e = raise_lds_limit((const void *) kern, attr_done);
+    if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), lds, st, kp);
     return hipGetLastError();
 }

@@ -166,6 +166,58 @@ def test_full_size_config5_properties(gpu):
     print(U.check(base[b:b + 1].cpu().numpy(), want, "config 5 full size, sequence %d (%d keys)" % (b, int(lens[b]))))
 
 
+@pytest.mark.parametrize("k_type", [O.TYPE_BF16, O.TYPE_Q8_0])
+def test_long_sequences_in_a_pool_beyond_4_gib(gpu, k_type):
+    """Sequences of up to 131 072 tokens (1024 pages: sixteen times what one workgroup's page list holds) whose pages lie
+    anywhere in a pool of more than 4 GiB, the top page included: byte offsets need 64 bits.  The result equals, bit for
+    bit, the same sequences gathered into a compact pool, and the short one equals the oracle."""
+    import torch
+    import jittorinfer_amd as J
+    g = torch.Generator(device=gpu)
+    g.manual_seed(97)
+    row = 1152 if k_type == O.TYPE_BF16 else 612
+    n_pages = (5 << 30) // (128 * row) + 1
+    lens = [131072, 70001, 5000]
+    nblk = [(l + 127) // 128 for l in lens]
+    used = torch.randperm(n_pages - 1, generator=g, device=gpu)[:sum(nblk) - 1]
+    used = torch.cat([used, torch.tensor([n_pages - 1], device=gpu)])[torch.randperm(sum(nblk), generator=g, device=gpu)]
+    pool = torch.empty((n_pages * 128, row), dtype=torch.uint8, device=gpu)     # pages no sequence owns stay uninitialised
+    if k_type == O.TYPE_BF16:
+        data = (torch.randn((sum(nblk) * 128, 576), generator=g, device=gpu) * 0.7).to(torch.bfloat16).view(torch.uint8)
+    else:
+        data = torch.empty((sum(nblk) * 128, 18, 34), dtype=torch.uint8, device=gpu)
+        data[..., 0], data[..., 1] = 0x00, 0x28          # f16 1/32, little endian
+        data[..., 2:] = torch.clamp(torch.round(torch.randn((sum(nblk) * 128, 18, 32), generator=g, device=gpu) * 16), -127, 127).to(torch.int8).view(torch.uint8)
+        data = data.reshape(-1, 612)
+    pool.view(n_pages, 128 * row)[used] = data.view(sum(nblk), 128 * row)
+    bt = torch.full((3, max(nblk)), -7, dtype=torch.int32, device=gpu)
+    bt_small = bt.clone()
+    pos = 0
+    for b in range(3):
+        bt[b, :nblk[b]] = used[pos:pos + nblk[b]].to(torch.int32)
+        bt_small[b, :nblk[b]] = torch.arange(pos, pos + nblk[b], dtype=torch.int32, device=gpu)
+        pos += nblk[b]
+    sl = torch.tensor(lens, dtype=torch.int32, device=gpu)
+    q = torch.randn((3, 128, 1, 576), generator=g, device=gpu)
+    kt = J.MLA_TYPE_BF16 if k_type == O.TYPE_BF16 else J.MLA_TYPE_Q8_0
+    tk = pool.view(torch.int16) if k_type == O.TYPE_BF16 else pool
+    td = data.view(torch.int16) if k_type == O.TYPE_BF16 else data
+    kw = dict(dv=512, scale=U.SCALE, seq_lens=sl)
+    info = J.plan(q, tk, kt, block_table=bt, **kw)
+    assert info["variant"] == 2 and info["balanced"] == 1
+    big = J.ggml_flash_attn_ext(q, tk, kt, block_table=bt, **kw)[..., :512].clone()
+    small = J.ggml_flash_attn_ext(q, td, kt, block_table=bt_small, **kw)[..., :512]
+    assert not torch.isnan(big).any() and torch.equal(big, small)
+    uni = J.ggml_flash_attn_ext(q, tk, kt, block_table=bt, flags=J.MLA_FLAG_UNIFORM_SPLITS, **kw)[..., :512]
+    ma, rl = O.errors(uni.cpu().numpy(), big.cpu().numpy())
+    assert ma <= 5e-4 and rl <= 5e-4, (ma, rl)
+    k2 = data.view(sum(nblk), 128, row)[nblk[0] + nblk[1]:].reshape(-1, row)[:lens[2]].cpu().numpy()
+    if k_type == O.TYPE_BF16:
+        k2 = k2.view(np.uint16)
+    want = O.flash_attn_ext(q[2:3].cpu().numpy(), k2[None], k_type, dv=512, scale=U.SCALE)
+    print(U.check(big[2:3].cpu().numpy(), want, "5000-token sequence in the 5 GiB pool"))
+
+
 def test_full_size_config4_causal_independence(gpu):
     """BASELINE configs[3] at full size (B=4, H=16, 512 new tokens on 2048 cached, causal mask): query token t must not
     depend on keys after position 2048 + t.  Keys after 2048 + 255 are replaced by other values: the outputs of tokens
