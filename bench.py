@@ -444,7 +444,7 @@ def main():
     ap.add_argument("--pools", type=int, default=4, help="distinct KV pools rotated between steps")
     ap.add_argument("--splits", type=int, default=0)
     ap.add_argument("--rows-per-wg", type=int, default=0)
-    ap.add_argument("--cpu-seqs", type=int, default=8, help="sequences of the workload timed on the host cores (0 = skip)")
+    ap.add_argument("--cpu-seqs", type=int, default=32, help="sequences of the workload timed on the host cores (default: the whole step; 0 = skip)")
     ap.add_argument("--seed", type=int, default=1234)
     ap.add_argument("--tokens", type=int, default=32, help="query tokens of --config rope / absorb / unabsorb (32 = a decode step, 2048 = a prefill chunk)")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="N",
