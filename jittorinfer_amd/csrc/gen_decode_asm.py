@@ -81,6 +81,7 @@ RAWC, RAWN, SH, SHM2, PSEL = 74, 77, 78, 79, 72   # Q8_0 builds: raw buffer to d
 RAWB, DSTB, DZ = 197, 198, 199                    # Q8_0 builds: per-lane raw window / f16 destination offsets, all-ones where this lane's row is valid
 SCL, L2E, MSK = (82, 73, 80) if Q8 else (77, 73, 78)   # mask builds: scale, log2(e) (the register of SCLS until the epilogue), mask base (QP's registers once Q is loaded;
                                                         # Q8_0 builds keep the dequantizer's scalars there and take s80..s83)
+ONES = 83   # f16 builds: packed (1.0, 1.0)
 EXS, S0, S1, S2, S3, DMAB, NVAL, THR, PG0, RSC, SPITCH, SCLS, OFF3, VMW, OSTR, QP = 60, 62, 63, 64, 65, 66, 67, 68, 69, 70, 72, 73, 74, 75, 76, 78
 
 out = []
@@ -545,14 +546,18 @@ def softmax_lines(sreg):
         L.append("v_fma_f32 %s, %s, %s, %s" % (v(sreg + k), v(sreg + k), s(CS), v(NEGM)))
     for k in range(16):
         L.append("v_exp_f32 %s, %s" % (v(sreg + k), v(sreg + k)))
-    # running sum (this lane's 16 tokens)
-    L.append("v_add_f32 %s, %s, %s" % (v(T[0]), v(sreg + 0), v(sreg + 1)))
-    L.append("v_add_f32 %s, %s, %s" % (v(T[1]), v(sreg + 2), v(sreg + 3)))
-    for k in range(4, 16, 2):
-        L.append("v_add_f32 %s, %s, %s" % (v(T[0]), v(T[0]), v(sreg + k)))
-        L.append("v_add_f32 %s, %s, %s" % (v(T[1]), v(T[1]), v(sreg + k + 1)))
-    L.append("v_add_f32 %s, %s, %s" % (v(T[0]), v(T[0]), v(T[1])))
-    L.append("v_add_f32 %s, %s, %s" % (v(LRUN), v(LRUN), v(T[0])))
+    # running sum (this lane's 16 tokens).  With a hi/lo pair the operands carry p to 2^-17 and the f32 values are summed;
+    # a single f16 operand is p rounded to 11 bits, and there the sum is taken over the rounded values further down: the
+    # output stays an exact weighted mean of V rows (with weights that moved by 2^-12), so a dominant key's V value is not
+    # scaled by the rounding of its own weight.
+    if SPLIT:
+        L.append("v_add_f32 %s, %s, %s" % (v(T[0]), v(sreg + 0), v(sreg + 1)))
+        L.append("v_add_f32 %s, %s, %s" % (v(T[1]), v(sreg + 2), v(sreg + 3)))
+        for k in range(4, 16, 2):
+            L.append("v_add_f32 %s, %s, %s" % (v(T[0]), v(T[0]), v(sreg + k)))
+            L.append("v_add_f32 %s, %s, %s" % (v(T[1]), v(T[1]), v(sreg + k + 1)))
+        L.append("v_add_f32 %s, %s, %s" % (v(T[0]), v(T[0]), v(T[1])))
+        L.append("v_add_f32 %s, %s, %s" % (v(LRUN), v(LRUN), v(T[0])))
     # P^T operands in place.  k-step kk owns registers b = sreg+8kk .. +7, holding p of tokens
     # (8(2kk)+4g+0..3, 8(2kk+1)+4g+0..3); pairs (b0,b1) (b2,b3) (b4,b5) (b6,b7) become hi -> b0..b3, lo -> b4..b7.
     for kk in range(2):
@@ -560,6 +565,15 @@ def softmax_lines(sreg):
         if not SPLIT:
             for j in range(4):
                 L.append("%s %s, %s, %s" % (CVT, v(b + j), v(b + 2 * j), v(b + 2 * j + 1)))
+            # l += the eight rounded values of this k-step: dot products with (1, 1), two chains
+            for j in range(4):
+                acc = T[j & 1]
+                c = "0" if kk == 0 and j < 2 else v(acc)
+                L.append("v_dot2_f32_f16 %s, %s, %s, %s" % (v(acc), v(b + j), s(ONES), c))
+            if kk == 1:
+                L.append("s_nop 2")   # a dot product's result may be read by another kind of VALU instruction three wait states later
+                L.append("v_add_f32 %s, %s, %s" % (v(T[0]), v(T[0]), v(T[1])))
+                L.append("v_add_f32 %s, %s, %s" % (v(LRUN), v(LRUN), v(T[0])))
             continue
         H, X, Y = T[0], T[1], T[2]
         Lo = [T[3], T[4], T[5], T[6]]
@@ -776,6 +790,8 @@ def main():
     if DEBUG:
         e("v_mov_b32 %s, %s" % (v(TIDR), v(X0)))
     e("s_mov_b32 %s, 0x%08x" % (s(THR), 0x41000000))  # TAU = 8.0f
+    if not SPLIT:
+        e("s_mov_b32 %s, 0x3c003c00" % s(ONES))
     if MASK:
         e("s_mov_b32 %s, %%[scl]" % s(SCL))
         e("s_mov_b32 %s, 0x3fb8aa3b" % s(L2E))

@@ -87,9 +87,7 @@ def test_random_shapes_against_the_oracle(gpu, seed0):
             fn = O.flash_attn_ext_f64 if f64 else O.flash_attn_ext
             want = fn(q, k, k_type, dv=dv, mask=mask, scale=U.SCALE, **okw)
         try:
-            # Q8_0: Q as d*q and P rounded to the f16 MFMA operands move an output of magnitude 2 by up to 2e-3 in the tail of
-            # a few thousand rows (2.03e-3 seen at rel-L2 4e-4); the sweep allows 3e-3 there, rel-L2 stays at 1e-3
-            U.check(got, want, desc, max_abs=3e-3 if k_type == O.TYPE_Q8_0 else U.MAX_ABS_TOL)
+            U.check(got, want, desc)
             seen.add((info["variant"], info["balanced"]))
         except AssertionError as ex:
             bad.append(str(ex)[:300])
