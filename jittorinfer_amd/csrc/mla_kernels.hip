@@ -544,7 +544,7 @@ __global__ void __launch_bounds__(256) mla_attn_combine_f32_kernel(const KParams
 // ---------------------------------------------------------------------------------------------------------------
 // Strict replay of ggml-cpu's f16 accumulator for F16 KV (ggml-cpu.c:12066-12080 with the x86 F16 vector forms
 // :621-659, :718-765: f32 FMA, result rounded to f16 after every scale and every multiply-add, keys in order).
-// Two small kernels: scores (f32 dot of f16-rounded Q with f16 K), then one wave per row walking the keys.
+// Two small kernels: scores (f32 dot of f16-rounded Q with f16 K), then one block per row walking the keys.
 // ---------------------------------------------------------------------------------------------------------------
 __global__ void mla_f16_scores_kernel(const KParams p, float * scores) {  // grid (ceil(n_kv/4), n_rows, n_seq), block 256
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -560,49 +560,93 @@ __global__ void mla_f16_scores_kernel(const KParams p, float * scores) {  // gri
     if (lane == 0) scores[((int64_t) b * p.n_rows + row) * p.n_kv + ic] = sum;
 }
 
-__global__ void mla_f16_strict_kernel(const KParams p, const float * scores) {  // grid (n_rows, n_seq), block 64
-    const int lane = threadIdx.x, row = blockIdx.x, b = blockIdx.y;
+// One block per output row, one thread per output column; the keys are walked in chunks of STRICT_CHUNK:
+//   (a) the logits of the chunk (scale, softcap, ALiBi slope x mask), one key per thread,
+//   (b) their running maximum by a prefix scan -- the maximum before key k decides which branch ggml-cpu takes at k
+//       and what it feeds expf -- which gives every key its (ms, vs) pair without walking the keys,
+//   (c) the walk itself, per column: acc = f16(acc * ms) where the maximum moved, acc = f16(fma(v, vs, acc)), S = S * ms + vs,
+//       exactly the operations of the reference, in its order; the V values of eight keys are in flight at a time.
+constexpr int STRICT_CHUNK = 1024;
+__global__ void __launch_bounds__(576) mla_f16_strict_kernel(const KParams p, const float * scores) {  // grid (n_rows, n_seq), block 512 | 576
+    __shared__ __attribute__((aligned(16))) float lg[STRICT_CHUNK], pa[STRICT_CHUNK], pb[STRICT_CHUNK];   // logits (-inf: skipped key); scan buffers, then ms / vs
+    const int tid = threadIdx.x, nth = blockDim.x, row = blockIdx.x, b = blockIdx.y;
     const int tq = row / p.n_head, head = row - tq * p.n_head;
     float slope = 1.0f;
     if (p.max_bias > 0.0f) slope = head < p.n_head_log2 ? powf(p.m0, (float) (head + 1)) : powf(p.m1, (float) (2 * (head - p.n_head_log2) + 1));
     const float scale_eff = p.softcap != 0.0f ? p.scale / p.softcap : p.scale;
     const char * mask_row = p.mask ? p.mask + (int64_t) tq * p.mask_nb1 : nullptr;
     const float * srow = scores + ((int64_t) b * p.n_rows + row) * p.n_kv;
-    float acc[9];
-#pragma unroll
-    for (int j = 0; j < 9; j++) acc[j] = 0.f;
-    float S = 0.f, M = -INFINITY;
-    for (int ic = 0; ic < (int) p.n_kv; ic++) {
-        const float mv = mask_row ? slope * f16_bits_to_f32(*(const unsigned short *) (mask_row + (int64_t) ic * 2)) : 0.0f;
-        if (mv == -INFINITY) continue;
-        float s = srow[ic] * scale_eff;
-        if (p.softcap != 0.0f) s = p.softcap * tanhf(s);
-        s += mv;
-        const float Mold = M;
-        float ms = 1.0f, vs = 1.0f;
-        const unsigned short * vrow = (const unsigned short *) (p.kv + (int64_t) ic * p.kv_nb1 + (int64_t) b * p.kv_nb3);
-        if (s > M) {
-            M  = s;
-            ms = expf(Mold - M);
-#pragma unroll
-            for (int j = 0; j < 9; j++) acc[j] = (float) (_Float16) (acc[j] * ms);
-        } else {
-            vs = expf(s - M);
+    const bool col = tid < p.dv_total;
+    const char * vcol = p.kv + (int64_t) b * p.kv_nb3 + 2 * (col ? tid : 0);
+    float acc = 0.f, S = 0.f, M = -INFINITY;   // M: the maximum over the chunks before this one (the same in every thread)
+    for (int c0 = 0; c0 < (int) p.n_kv; c0 += STRICT_CHUNK) {
+        const int n = min(STRICT_CHUNK, (int) p.n_kv - c0);
+        for (int k = tid; k < n; k += nth) {
+            const int ic = c0 + k;
+            const float mv = mask_row ? slope * f16_bits_to_f32(*(const unsigned short *) (mask_row + (int64_t) ic * 2)) : 0.0f;
+            float sv = -INFINITY;   // ggml-cpu skips a key whose mask value is -inf (ggml-cpu.c:12041-12044)
+            if (mv != -INFINITY) {
+                sv = srow[ic] * scale_eff;
+                if (p.softcap != 0.0f) sv = p.softcap * tanhf(sv);
+                sv += mv;
+            }
+            lg[k] = sv; pa[k] = sv;
         }
-#pragma unroll
-        for (int j = 0; j < 9; j++) {
-            const int d = lane + 64 * j;
-            if (d < p.dv_total) acc[j] = (float) (_Float16) fmaf(f16_bits_to_f32(vrow[d]), vs, acc[j]);
+        __syncthreads();
+        float * src = pa, * dst = pb;   // inclusive prefix maximum (Hillis-Steele, ping-pong)
+        for (int off = 1; off < n; off <<= 1) {
+            for (int k = tid; k < n; k += nth) dst[k] = k >= off ? fmaxf(src[k], src[k - off]) : src[k];
+            __syncthreads();
+            float * t = src; src = dst; dst = t;
         }
-        S = S * ms + vs;
-    }
-    const float S_inv = 1.0f / S;
-    float * o = p.dst + ((int64_t) b * p.n_rows + row) * p.dst_stride;
+        float ms2[2], vs2[2];   // n <= 1024 and nth >= 512: at most two keys per thread
+        int nk = 0;
+        for (int k = tid; k < n; k += nth, nk++) {
+            const float mprev = k > 0 ? fmaxf(M, src[k - 1]) : M;
+            const float sv = lg[k];
+            float ms = 1.0f, vs = -1.0f;   // vs < 0 marks a skipped key
+            if (sv != -INFINITY || mask_row == nullptr) {
+                if (sv > mprev) { ms = expf(mprev - sv); vs = 1.0f; }
+                else            { vs = expf(sv - mprev); }
+            }
+            ms2[nk] = ms; vs2[nk] = vs;
+        }
+        const float m_chunk = src[n - 1];
+        __syncthreads();
+        nk = 0;
+        for (int k = tid; k < n; k += nth, nk++) { pa[k] = ms2[nk]; pb[k] = vs2[nk]; }
+        if (tid < 8 && n + tid < ((n + 7) & ~7)) { pa[n + tid] = 1.0f; pb[n + tid] = -1.0f; }   // pad the last group of eight with skipped keys
+        __syncthreads();
+        M = fmaxf(M, m_chunk);
+        if (col) {
+            const char * vp = vcol + (int64_t) c0 * p.kv_nb1;
+            unsigned short vn[8];
 #pragma unroll
-    for (int j = 0; j < 9; j++) {
-        const int d = lane + 64 * j;
-        if (d < p.dv_total) o[d] = acc[j] * S_inv;
+            for (int j = 0; j < 8; j++) vn[j] = *(const unsigned short *) (vp + (int64_t) min(j, n - 1) * p.kv_nb1);
+            for (int k0 = 0; k0 < n; k0 += 8) {
+                unsigned short v8[8];
+#pragma unroll
+                for (int j = 0; j < 8; j++) v8[j] = vn[j];
+#pragma unroll
+                for (int j = 0; j < 8; j++) vn[j] = *(const unsigned short *) (vp + (int64_t) min(k0 + 8 + j, n - 1) * p.kv_nb1);   // the next eight, in flight during this group
+                const f32x4 m0 = *(const f32x4 *) (pa + k0), m1 = *(const f32x4 *) (pa + k0 + 4);
+                const f32x4 w0 = *(const f32x4 *) (pb + k0), w1 = *(const f32x4 *) (pb + k0 + 4);
+                const float ms8[8] = { m0.x, m0.y, m0.z, m0.w, m1.x, m1.y, m1.z, m1.w };
+                const float vs8[8] = { w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w };
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    // acc * ms is the identity where the maximum did not move (ms = 1 and acc is an f16 value), so no branch on it
+                    const float scaled = (float) (_Float16) (acc * ms8[j]);
+                    const float next   = (float) (_Float16) fmaf(f16_bits_to_f32(v8[j]), vs8[j], scaled);
+                    const bool  skip   = vs8[j] < 0.0f;
+                    acc = skip ? acc : next;
+                    S   = skip ? S : S * ms8[j] + vs8[j];
+                }
+            }
+        }
+        __syncthreads();
     }
+    if (col) p.dst[((int64_t) b * p.n_rows + row) * p.dst_stride + tid] = acc * (1.0f / S);
 }
 
 __global__ void __launch_bounds__(256) mla_hbm_copy_kernel(const u32x4 * __restrict__ src, u32x4 * __restrict__ dst, size_t n16) {
@@ -843,7 +887,7 @@ static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
             if (e != hipSuccess) return (int) e;
         }
         dim3 g2((unsigned) kp.n_rows, (unsigned) a->n_seq);
-        hipLaunchKernelGGL(mla_f16_strict_kernel, g2, dim3(64), 0, st, kp, (const float *) scores);
+        hipLaunchKernelGGL(mla_f16_strict_kernel, g2, dim3(a->dv == 576 ? 576 : 512), 0, st, kp, (const float *) scores);
         return (int) hipGetLastError();
     }
 

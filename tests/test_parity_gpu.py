@@ -51,6 +51,23 @@ def test_config1_f16_strict(gpu):
     print(U.check(got[..., :512], want, "config 1 strict f16"))
 
 
+@pytest.mark.parametrize("n_kv,n_tok,dv,softcap,max_bias", [(2500, 3, 576, 0.0, 0.0), (300, 2, 512, 30.0, 8.0), (1, 1, 512, 0.0, 0.0), (1031, 1, 512, 0.0, 0.0)])
+def test_f16_strict_beyond_one_chunk_with_mask_softcap_alibi(gpu, n_kv, n_tok, dv, softcap, max_bias):
+    """The strict replay walks the keys in chunks of 1024 (prefix maximum per chunk, carried across chunks): several
+    chunks and a ragged last one, -inf holes in the mask (keys the reference skips), softcap and ALiBi slopes."""
+    import jittorinfer_amd as J
+    rng = np.random.default_rng(700 + n_kv)
+    q = rng.standard_normal((2, 5, n_tok, 576)).astype(np.float32)
+    k = O.f32_to_f16(rng.standard_normal((2, n_kv, 576)).astype(np.float32))
+    m = (rng.standard_normal((n_tok, n_kv)) * 1.5).astype(np.float32)
+    m[rng.random((n_tok, n_kv)) < 0.3] = -np.inf
+    m[:, 0] = 0
+    mask = m.astype(np.float16).view(np.uint16)
+    want = O.flash_attn_ext(q, k, O.TYPE_F16, dv=dv, mask=mask, scale=U.SCALE, max_bias=max_bias, softcap=softcap)
+    got = _run(gpu, q, k, O.TYPE_F16, dv=dv, mask=mask, scale=U.SCALE, max_bias=max_bias, logit_softcap=softcap, flags=J.MLA_FLAG_F16_ACC_STRICT)
+    print(U.check(got[..., :dv], want, "strict f16, %d keys" % n_kv))
+
+
 @pytest.mark.parametrize("k_type", [O.TYPE_BF16, O.TYPE_Q8_0])
 def test_config2_paged_decode(gpu, k_type):
     """BASELINE config 2 shape: batch 8, 16 heads, lengths uniform in [512, 4096], 512-page pool, shuffled table."""
