@@ -48,6 +48,9 @@
  *   event_new / event_free / event_synchronize and the backend's event_record / event_wait: HIP events on the
  *                          backend's stream, which ggml_backend_sched uses to keep several copies of a graph's inputs in
  *                          flight (ggml/src/ggml-backend.cpp:1508-1530, :1576-1580, :1630-1634)
+ * F16 KV: the node accumulates V in f32 (closer to the exact value than ggml-cpu's f16 accumulator, which is 4e-3 away);
+ * a backend initialised with params containing "f16_acc=strict" (ggml_backend_dev_init(dev, params)), or with
+ * GGML_HIP_MLA_F16_ACC=strict in the environment, replays the reference's accumulator instead (ggml-cpu.c:12066-12080).
  * and reports caps {async, host_buffer, events} (struct ggml_backend_dev_caps, ggml/include/ggml-backend.h:145-154).
  */
 #ifndef GGML_MLA_BACKEND_H

@@ -67,6 +67,7 @@ struct backend_ctx {
     hipStream_t stream;
     void *      workspace      = nullptr;
     size_t      workspace_size = 0;
+    bool        f16_strict     = false;   // F16 KV: replay ggml-cpu's f16 accumulator instead of accumulating in f32
 };
 
 std::vector<device_ctx *>     g_device_ctx;
@@ -457,6 +458,7 @@ int compute_flash_attn(backend_ctx * ctx, const tensor * dst) {
     if (mask) { a.mask = mask->data; a.mask_nb1 = (int64_t) mask->nb[1]; a.mask_ne0 = mask->ne[0]; }
     if (bt) { a.block_table = (const int32_t *) bt->data; a.bt_stride = bt->ne[0]; a.seq_lens = (const int32_t *) lens->data; }
     a.dst = (float *) dst->data; a.dst_nb1 = (int64_t) dst->nb[1];
+    if (ctx->f16_strict && k->type == TYPE_F16 && !bt) a.flags |= MLA_FLAG_F16_ACC_STRICT;
 
     const size_t need = mla_attn_workspace_size(&a);
     if (need > ctx->workspace_size) {
@@ -625,12 +627,17 @@ void device_get_props(backend_device * dev, dev_props * props) {
     device_get_memory(dev, &props->memory_free, &props->memory_total);
     props->caps = dev_caps{ /* async */ true, /* host_buffer */ true, /* buffer_from_host_ptr */ false, /* events */ true };
 }
-backend * device_init_backend(backend_device * dev, const char *) {
+// params (the string ggml_backend_dev_init hands through, ggml-backend.cpp:505-508) or the environment may ask for
+// "f16_acc=strict": attention over an F16 cache then reproduces ggml-cpu's f16 accumulator (ggml-cpu.c:12066-12080)
+// instead of the f32 accumulation that is closer to the exact value.
+backend * device_init_backend(backend_device * dev, const char * params) {
     device_ctx * dc = (device_ctx *) dev->context;
     if (!HIP_OK(hipSetDevice(dc->index))) return nullptr;
     backend_ctx * ctx = new backend_ctx;
     ctx->device = dc->index;
     ctx->name   = dc->name;
+    const char * env = getenv("GGML_HIP_MLA_F16_ACC");
+    ctx->f16_strict = (params && strstr(params, "f16_acc=strict")) || (env && strcmp(env, "strict") == 0);
     if (!HIP_OK(hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking))) { delete ctx; return nullptr; }
     return new backend{ &g_guid, k_backend_iface, dev, ctx };
 }

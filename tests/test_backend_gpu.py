@@ -43,6 +43,23 @@ def test_latent_prefix_view_and_block_table(gpu):
     print(U.check(got[..., :512], want, "paged node through the scheduler"))
 
 
+def test_f16_cache_with_the_reference_accumulator_on_request(gpu, monkeypatch):
+    """F16 KV: ggml-cpu accumulates V in f16 and lands 4e-3 from the exact value; the plugin accumulates in f32 unless
+    the backend is initialised with f16_acc=strict (here through the environment), and then replays the reference's
+    accumulator: only that mode agrees with ggml-cpu to the tolerance."""
+    rng = np.random.default_rng(31)
+    q = rng.standard_normal((1, 16, 1, 576)).astype(np.float32)
+    k = U.encode_kv(rng.standard_normal((1, 1024, 576)).astype(np.float32), O.TYPE_F16)
+    cpu = O.ref_flash_attn_ext(q, k, O.TYPE_F16, scale=U.SCALE)
+    fast, _ = O.ref_backend_flash_attn_ext(_so(), q, k, O.TYPE_F16, dv=576, scale=U.SCALE)
+    monkeypatch.setenv("GGML_HIP_MLA_F16_ACC", "strict")
+    strict, _ = O.ref_backend_flash_attn_ext(_so(), q, k, O.TYPE_F16, dv=576, scale=U.SCALE)
+    e_fast, e_strict = O.errors(fast, cpu), O.errors(strict, cpu)
+    print("vs ggml-cpu: f32 accumulation", e_fast, "replay", e_strict)
+    U.check(strict, cpu, "strict replay vs ggml-cpu")
+    assert e_strict[1] < 0.5 * e_fast[1]
+
+
 @pytest.mark.parametrize("paged", [False, True])
 def test_scheduler_set_up_as_llama_sets_it_up(gpu, paged):
     """The scheduler as the reference's context builds it (src/llama-context-load-utils.cpp:108-131): the CPU backend's
