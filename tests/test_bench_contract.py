@@ -1,0 +1,36 @@
+"""bench.py's command-line contract, as far as it can be checked without a GPU: more than one GPU is refused with a
+message, the help text lists the measured configurations, and the product raises (no CPU path) when asked to compute
+on a CPU tensor."""
+import os
+import subprocess
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _bench(*args):
+    return subprocess.run([sys.executable, os.path.join(ROOT, "bench.py")] + list(args), capture_output=True, text=True, timeout=300)
+
+
+def test_more_than_one_gpu_is_refused_with_a_message():
+    r = _bench("--gpus", "2")
+    assert r.returncode != 0
+    assert "one GPU" in (r.stdout + r.stderr) and "--gpus 2" in (r.stdout + r.stderr)
+
+
+def test_help_names_the_configurations():
+    r = _bench("--help")
+    assert r.returncode == 0
+    for word in ("--steps", "--warmup", "--gpus", "--config", "c3mask", "kvwrite", "layer", "--cpu-seqs"):
+        assert word in r.stdout, word
+
+
+def test_no_cpu_path():
+    import torch
+    import jittorinfer_amd as J
+    q = torch.zeros((1, 16, 1, 576))
+    k = torch.zeros((1, 32, 576), dtype=torch.int16)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        J.ggml_flash_attn_ext(q, k, J.MLA_TYPE_BF16)
