@@ -395,11 +395,13 @@ def qk_slots(sreg, kaddr):
 
     def mk(ks):
         def slot():
-            if ks + depth < 36:
-                k_read(kaddr, ks + depth)
             lds.need(("k", ks))
             c = "0" if ks == 0 else v(sreg, 16)
             e("%s %s, %s, %s, %s" % (MF, v(sreg, 16), v(KF + 4 * (ks % KRING), 4), v(Q0 + 4 * ks, 4), c))
+            # the next fragment read goes right behind the MFMA, ahead of the VALU work of this slot: an LDS read that
+            # follows VALU instructions in the shadow of an MFMA delays the next MFMA by 8 cycles more than one that leads them
+            if ks + depth < 36:
+                k_read(kaddr, ks + depth)
         return slot
     return [mk(ks) for ks in range(36)]
 
@@ -466,10 +468,10 @@ def pv_slots(vaddr, greg):
     def mf(idx, lo, pre):
         kk, db = V_FRAGS[idx]
         def slot():
-            for p in pre:
-                v_read(vaddr, p)
             lds.need(("v", idx, 1))
             e("%s %s, %s, %s, %s" % (MF, a(16 * db, 16), v(VF + 4 * (idx % VRING), 4), v(greg + 8 * kk + (4 if lo else 0), 4), a(16 * db, 16)))
+            for p in pre:
+                v_read(vaddr, p)
         return slot
     slots = []
     for pair in range(16):
