@@ -510,27 +510,28 @@ __global__ void __launch_bounds__(256) mla_attn_combine_f32_kernel(const KParams
     const float2 * ml = (const float2 *) p.part_ml + (int64_t) slot0 * p.slot_rows + lrow;
     const float *  po = (const float *) p.part_o + ((int64_t) slot0 * p.slot_rows + lrow) * p.dv_total + cg * 4;
     const int64_t ml_step = p.slot_rows, po_step = (int64_t) p.slot_rows * p.dv_total;
+    constexpr int G = 16;   // small problems are latency-bound: a ragged batch has up to 32 one-page pieces per sequence
     float M = -INFINITY, L = 0.f;
     f32x4 o = { 0.f, 0.f, 0.f, 0.f };
-    for (int c0 = 0; c0 < nvalid; c0 += 8) {   // groups of 8 splits: their loads are in flight together
-        float2 mlv[8];
-        f32x4  xv[8];
+    for (int c0 = 0; c0 < nvalid; c0 += G) {   // groups of G splits: their loads are in flight together
+        float2 mlv[G];
+        f32x4  xv[G];
 #pragma unroll
-        for (int k = 0; k < 8; k++) {
+        for (int k = 0; k < G; k++) {
             const int c = min(c0 + k, nvalid - 1);  // past the end: a duplicate of the last split, given weight 0 below
             mlv[k] = ml[c * ml_step];
             xv[k]  = *(const f32x4 *) (po + c * po_step);
         }
         float Mg = M;
 #pragma unroll
-        for (int k = 0; k < 8; k++) if (c0 + k < nvalid) Mg = fmaxf(Mg, mlv[k].x);
+        for (int k = 0; k < G; k++) if (c0 + k < nvalid) Mg = fmaxf(Mg, mlv[k].x);
         if (Mg == -INFINITY) continue;  // every split so far saw only masked keys
         const float r = fast_exp2(M - Mg);  // 0 when M was -inf
         M = Mg;
         L *= r;
         o.x *= r; o.y *= r; o.z *= r; o.w *= r;
 #pragma unroll
-        for (int k = 0; k < 8; k++) {
+        for (int k = 0; k < G; k++) {
             const float w = (c0 + k < nvalid && mlv[k].x != -INFINITY) ? mlv[k].y * fast_exp2(mlv[k].x - M) : 0.f;
             L += w;
             if (w == 0.f) continue;  // that split saw only masked keys (or is padding): its partial may hold anything
