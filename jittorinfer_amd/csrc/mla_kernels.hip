@@ -763,7 +763,10 @@ int make_plan(const mla_attn_args * a, Plan * pl) {
     // The same for a masked launch over one contiguous cache (the reference's batched decode): equal runs of the tiles of
     // the key ranges the row blocks may attend to.
     if (pl->variant == 2 && a->n_splits == 0 && pl->n_splits > 1 && !(a->flags & MLA_FLAG_UNIFORM_SPLITS)) {
-        if (a->block_table && !a->mask && pl->n_row_blocks == 1 && a->n_seq <= 256 && ((int64_t) a->n_seq * n_pages + 255) / 256 <= 64) {
+        // (with at most one page per workgroup even when every sequence is full there is nothing to balance: the uniform
+        // plan already hands out single pages, and the schedule itself costs a small batch 1.6 us)
+        if (a->block_table && !a->mask && pl->n_row_blocks == 1 && a->n_seq <= 256 && (int64_t) a->n_seq * n_pages > 256 &&
+            ((int64_t) a->n_seq * n_pages + 255) / 256 <= 64) {
             pl->balanced = 1; pl->n_units = a->n_seq;
         } else if (a->mask && !a->block_table && a->n_seq == 1 && pl->n_row_blocks <= 256) {
             pl->balanced = 2; pl->n_units = pl->n_row_blocks;

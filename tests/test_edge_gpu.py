@@ -300,7 +300,7 @@ def test_graph_replay_with_sequence_lengths_changed_on_the_device(gpu):
     import torch
     import jittorinfer_amd as J
     rng = np.random.default_rng(77)
-    n_seq, cap = 20, 1536
+    n_seq, cap = 24, 1536   # 24 x 12 pages: more than one page per workgroup, so the balanced schedule is planned
     pool, bt, seqs = U.make_paged(rng, [cap] * n_seq, O.TYPE_BF16)
     tq = torch.zeros((n_seq, 128, 1, 576), dtype=torch.float32, device=gpu)
     tk = torch.from_numpy(pool.view(np.int16)).to(gpu)
@@ -416,6 +416,9 @@ def test_balanced_schedule_of_ragged_decode_batches(gpu, k_type, shape):
     # V value rounded to the f16 MFMA operand alone costs up to 2^-11 |v| = 2.2e-3 at |v| = 4.5, whatever the schedule
     pool, bt, seqs = U.make_paged(rng, np.maximum(lens, 1), k_type, q8_scale=1.0 / 32 if k_type == O.TYPE_Q8_0 else None)
     seqs = [s[:l] for s, l in zip(seqs, lens)]
+    if len(lens) * bt.shape[1] <= 256:
+        # the schedule is planned when the table allows more than one page per workgroup: columns no sequence reaches
+        bt = np.concatenate([bt, np.full((len(lens), 300 - bt.shape[1]), -5, np.int32)], axis=1)
     q = rng.standard_normal((len(lens), 32, 1, 576)).astype(np.float32)
     got, info = _run_flags(gpu, q, pool, k_type, bt, lens, 0)
     assert info["variant"] == 2 and info["balanced"] == 1 and info["n_workgroups"] == 256
@@ -426,8 +429,9 @@ def test_balanced_schedule_of_ragged_decode_batches(gpu, k_type, shape):
 
 
 def test_balanced_schedule_limits(gpu):
-    """A batch that already fills the GPU with one workgroup per sequence (nothing to split), or a block table so wide that
-    a workgroup's run could exceed the 64 pages a wave indexes, keeps the uniform plan."""
+    """A batch that already fills the GPU with one workgroup per sequence (nothing to split), one whose table holds no more
+    pages than there are workgroups, or a block table so wide that a workgroup's run could exceed the 64 pages a wave
+    indexes, keeps the uniform plan."""
     import torch
     import jittorinfer_amd as J
     q = torch.zeros((257, 16, 1, 576), device=gpu)
@@ -436,7 +440,9 @@ def test_balanced_schedule_limits(gpu):
     sl = torch.ones(257, dtype=torch.int32, device=gpu)
     assert J.plan(q[:256], pool, J.MLA_TYPE_BF16, dv=512, scale=1.0, block_table=bt[:256], seq_lens=sl[:256])["balanced"] == 0   # one split: nothing to balance
     q8 = torch.zeros((8, 16, 1, 576), device=gpu)
-    assert J.plan(q8, pool, J.MLA_TYPE_BF16, dv=512, scale=1.0, block_table=bt[:8], seq_lens=sl[:8])["balanced"] == 1
+    assert J.plan(q8, pool, J.MLA_TYPE_BF16, dv=512, scale=1.0, block_table=bt[:8], seq_lens=sl[:8])["balanced"] == 0   # 32 pages at most: one per workgroup anyway
+    bt40 = torch.zeros((8, 40), dtype=torch.int32, device=gpu)
+    assert J.plan(q8, pool, J.MLA_TYPE_BF16, dv=512, scale=1.0, block_table=bt40, seq_lens=sl[:8])["balanced"] == 1
     wide = torch.zeros((8, 4096), dtype=torch.int32, device=gpu)
     assert J.plan(q8, pool, J.MLA_TYPE_BF16, dv=512, scale=1.0, block_table=wide, seq_lens=sl[:8])["balanced"] == 0
 
