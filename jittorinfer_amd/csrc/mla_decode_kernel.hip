@@ -402,8 +402,27 @@ __global__ void __launch_bounds__(NTHREADS) mla_mask_extent_kernel(const KParams
     int hi = 0, lo = n_kv;
     for (int t = t0; t <= t1; t++) {
         const char * mrow = p.mask + (int64_t) t * p.mask_nb1;
-        for (int i = g0 + tid; i < g1; i += NTHREADS) {
-            const u32x2 a = *(const u32x2 *) (mrow + 16 * (int64_t) i), b = *(const u32x2 *) (mrow + 16 * (int64_t) i + 8);   // rows are 8-byte aligned
+        int i1 = g0 + tid;
+        for (; i1 + 3 * NTHREADS < g1; i1 += 4 * NTHREADS) {   // long rows: four groups per thread in flight, the scan is a chain of load latencies otherwise
+            const int i0 = i1;
+            u32x2 a[4], b[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int i = i0 + u * NTHREADS;
+                a[u] = *(const u32x2 *) (mrow + 16 * (int64_t) i);   // rows are 8-byte aligned
+                b[u] = *(const u32x2 *) (mrow + 16 * (int64_t) i + 8);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int i = i0 + u * NTHREADS;
+                const unsigned w[4] = { a[u].x, a[u].y, b[u].x, b[u].y };
+#pragma unroll
+                for (int e = 0; e < 8; e++)
+                    if (((w[e >> 1] >> (16 * (e & 1))) & 0xffff) != 0xfc00u) { lo = min(lo, 8 * i + e); hi = max(hi, 8 * i + e + 1); }
+            }
+        }
+        for (int i = i1; i < g1; i += NTHREADS) {
+            const u32x2 a = *(const u32x2 *) (mrow + 16 * (int64_t) i), b = *(const u32x2 *) (mrow + 16 * (int64_t) i + 8);
             const unsigned w[4] = { a.x, a.y, b.x, b.y };
 #pragma unroll
             for (int e = 0; e < 8; e++)
