@@ -770,6 +770,9 @@ def iteration(g_cur, g_next, tag):
     return resc
 
 
+LAB_EXIT = "Lexit_%="
+
+
 def main():
     # ------------------------------------------------------------------ entry: inputs -> fixed registers
     stamp(0)
@@ -987,6 +990,53 @@ def main():
         e("%s:" % lab_wd)
         page_clamp()
         e("s_barrier")
+        # ---------------------------------------------------------------- waves without a valid row (FLG bit 5; fewer than 97 rows in
+        # the block, e.g. a 16- or 32-head model's decode step): they keep moving their eight rows of every tile and meet the
+        # others at every barrier, and issue no MFMA, no fragment read and no softmax: a quarter of the matrix-core power for a
+        # 32-head model, which the chip-wide clock gives back to the wave that computes
+        lab_busy, lab_iloop, lab_inodma, lab_iw0, lab_iwd, lab_iend = (label(x) for x in ("busy", "iloop", "inodma", "iw0", "iwd", "iend"))
+        lab_it1, lab_it1d = label("it1"), label("it1d")
+        e("s_bitcmp1_b32 %s, 5" % s(FLG))
+        e("s_cbranch_scc0 %s" % lab_busy)
+        e("s_cmp_lt_u32 %s, 3" % s(NT))                 # as the first hand-over: tile 1 has landed
+        e("s_cbranch_scc1 %s" % lab_it1)
+        e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
+        e("s_branch %s" % lab_it1d)
+        e("%s:" % lab_it1)
+        e("s_waitcnt vmcnt(0)")
+        e("%s:" % lab_it1d)
+        e("s_barrier")
+        e("%s:" % lab_iloop)
+        e("s_add_u32 %s, %s, 1" % (s(TMP), s(IT)))
+        e("s_cmp_ge_u32 %s, %s" % (s(TMP), s(NT)))
+        e("s_cbranch_scc1 %s" % lab_iend)               # the last tile has no successor to wait for
+        e("s_mov_b32 %s, 0" % s(VMW))
+        e("s_add_u32 %s, %s, 3" % (s(TMP), s(IT)))
+        e("s_cmp_ge_u32 %s, %s" % (s(TMP), s(NT)))
+        e("s_cbranch_scc1 %s" % lab_inodma)
+        e("s_mov_b32 %s, 1" % s(VMW))
+        for ln in dma_tile_lines(TMP, OFF3):
+            e(ln)
+        e("%s:" % lab_inodma)
+        e("s_cmp_eq_u32 %s, 0" % s(VMW))
+        e("s_cbranch_scc1 %s" % lab_iw0)
+        e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
+        e("s_branch %s" % lab_iwd)
+        e("%s:" % lab_iw0)
+        e("s_waitcnt vmcnt(0)")
+        e("%s:" % lab_iwd)
+        e("s_barrier")
+        e("s_mov_b32 %s, %s" % (s(TMP), s(OFF0)))
+        e("s_mov_b32 %s, %s" % (s(OFF0), s(OFF1)))
+        e("s_mov_b32 %s, %s" % (s(OFF1), s(OFF2)))
+        e("s_mov_b32 %s, %s" % (s(OFF2), s(OFF3)))
+        e("s_mov_b32 %s, %s" % (s(OFF3), s(TMP)))
+        e("s_add_u32 %s, %s, 1" % (s(IT), s(IT)))
+        e("s_branch %s" % lab_iloop)
+        e("%s:" % lab_iend)
+        e("s_waitcnt vmcnt(0)")
+        e("s_branch %s" % LAB_EXIT)
+        e("%s:" % lab_busy)
     stamp(1)
     if DEBUG:
         # FLG bit 1: dump LDS tile 0 (2336 chunks) to the debug pointer and stop
@@ -1153,6 +1203,8 @@ def main():
             e("ds_write_b32 %s, %s offset:%d" % (v(X0), v(X1), 4 * k))
         e("s_waitcnt lgkmcnt(0)")
         e("s_barrier")
+
+    e("%s:" % LAB_EXIT)
 
     print("// generated by gen_decode_asm.py%s%s -- do not edit" % (" --q8" if Q8 else " --f16" if "--f16" in sys.argv else "", " --mask" if MASK else ""))
     for ln in out:

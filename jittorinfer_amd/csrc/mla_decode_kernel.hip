@@ -324,7 +324,10 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
     const int s_kve  = __builtin_amdgcn_readfirstlane(kv_end);
     const int s_npp  = __builtin_amdgcn_readfirstlane(p.n_pool_pages - 1);
     const int s_nb1  = __builtin_amdgcn_readfirstlane((int) p.kv_nb1);
-    const int s_flg  = __builtin_amdgcn_readfirstlane((direct || p.part_f32 ? 1 : 0) | (p.v_col0 ? 16 : 0) | p.debug_flags);  // bit 0: f32 row store; bit 4: V starts at column 64
+    // bit 0: f32 row store; bit 4: V starts at column 64; bit 5: none of this wave's 32 rows exists (it only moves tiles; the
+    // Q8_0 programs have no such path: their waves share the dequantisation)
+    const int s_flg  = __builtin_amdgcn_readfirstlane((direct || p.part_f32 ? 1 : 0) | (p.v_col0 ? 16 : 0) |
+                                                      (KVT != SRC_Q8 && by * 128 + wave * 32 >= p.n_rows ? 32 : 0) | p.debug_flags);
     const int s_ntl  = __builtin_amdgcn_readfirstlane(n_tiles);
     // id of the split's first page as a scalar: the first tiles are requested before the vector load of all page ids is back
     int pg0 = 0;
