@@ -380,6 +380,7 @@ __global__ void __launch_bounds__(NTHREADS) mla_q_pack_kernel(const KParams p) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int g = lane >> 5, rl = lane & 31;
     const int b = blockIdx.y, ks = blockIdx.z;
+    if ((int) blockIdx.x * 128 + wave * 32 >= p.n_rows) return;   // a wave of the decode kernel without a row: it computes nothing, its image is never used
     const int row = min((int) blockIdx.x * 128 + wave * 32 + rl, p.n_rows - 1);
     const int tq = row / p.n_head, head = row - tq * p.n_head;
     const float * qrow = (const float *) (p.q + (int64_t) tq * p.q_nb1 + (int64_t) head * p.q_nb2 + (int64_t) b * p.q_nb3) + 8 * g;
