@@ -861,11 +861,17 @@ def main():
     e("s_mul_i32 %s, %s, %d" % (s(S0), s(WAVE), 36 * 1024))
     e("s_add_u32 %s, %s, %s" % (s(QP), s(QP), s(S0)))
     e("s_addc_u32 %s, %s, 0" % (s(QP + 1), s(QP + 1)))
+    # a wave without a valid row (FLG bit 5) never uses Q: it skips the loads (its part of the image is not written either)
+    lab_noq = label("noq")
+    if nq and not Q8:
+        e("s_bitcmp1_b32 %s, 5" % s(FLG))
+        e("s_cbranch_scc1 %s" % lab_noq)
     for ks in range(nq):
         if ks and ks % 4 == 0:
             e("s_add_u32 %s, %s, 4096" % (s(QP), s(QP)))
             e("s_addc_u32 %s, %s, 0" % (s(QP + 1), s(QP + 1)))
         e("global_load_dwordx4 %s, %s, %s offset:%d" % (v(Q0 + 4 * ks, 4), v(X0), s(QP, 2), (ks % 4) * 1024))
+    e("%s:" % lab_noq)
     n_early = nq
     if MASK:
         # mask rows start at key kv_begin of this split; QP's registers are free now
@@ -894,7 +900,17 @@ def main():
     e("s_and_b32 %s, %s, 127" % (s(S0), s(KVB)))
     e("s_cmp_eq_u32 %s, 0" % s(S0))
     e("s_cbranch_scc1 %s" % lab_al)
-    e("s_waitcnt vmcnt(%d)" % n_early)
+    if nq and not Q8:
+        lab_wq, lab_wqd = label("wq"), label("wqd")
+        e("s_bitcmp1_b32 %s, 5" % s(FLG))
+        e("s_cbranch_scc0 %s" % lab_wq)
+        e("s_waitcnt vmcnt(%d)" % (n_early - nq))     # no Q loads behind the page ids
+        e("s_branch %s" % lab_wqd)
+        e("%s:" % lab_wq)
+        e("s_waitcnt vmcnt(%d)" % n_early)
+        e("%s:" % lab_wqd)
+    else:
+        e("s_waitcnt vmcnt(%d)" % n_early)
     e("v_max_i32 %s, 0, %s" % (v(PAGES), v(PAGES)))
     e("v_min_i32 %s, %s, %s" % (v(PAGES), s(NPP), v(PAGES)))
     e("%s:" % lab_al)
