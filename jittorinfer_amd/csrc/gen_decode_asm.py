@@ -979,6 +979,45 @@ def main():
         e("%s:" % lab_n2)
         for it_ in q8_dequant_items(RAWN, OFF1, 1):
             emit_item(it_)
+        # ---------------------------------------------------------------- waves without a valid row (FLG bit 5): they keep their share
+        # of the loads and of the dequantisation and meet the others at every barrier, and issue no MFMA, no fragment read
+        # and no softmax
+        lab_busy, lab_iloop, lab_inodma, lab_iend = (label(x) for x in ("busy", "iloop", "inodma", "iend"))
+        busy_pending = list(lds.pending)
+        e("s_bitcmp1_b32 %s, 5" % s(FLG))
+        e("s_cbranch_scc0 %s" % lab_busy)
+        lds.drain()                                     # this wave's share of f16 tile 1 is written
+        e("s_waitcnt vmcnt(0)")                         # raw tile 2 has landed
+        e("s_barrier")
+        e("%s:" % lab_iloop)
+        e("s_add_u32 %s, %s, 1" % (s(TMP), s(IT)))
+        e("s_cmp_ge_u32 %s, %s" % (s(TMP), s(NT)))
+        e("s_cbranch_scc1 %s" % lab_iend)               # the last tile has no successor to prepare
+        e("s_add_u32 %s, %s, 3" % (s(TMP), s(IT)))
+        e("s_cmp_ge_u32 %s, %s" % (s(TMP), s(NT)))
+        e("s_cbranch_scc1 %s" % lab_inodma)
+        for ln in q8_dma_lines(TMP, RAWN):
+            e(ln)
+        e("%s:" % lab_inodma)
+        for it_ in q8_dequant_items(RAWC, OFF2, 2):
+            emit_item(it_)
+        lds.drain()
+        e("s_waitcnt vmcnt(0)")
+        e("s_barrier")
+        e("s_mov_b32 %s, %s" % (s(TMP), s(OFF0)))
+        e("s_mov_b32 %s, %s" % (s(OFF0), s(OFF1)))
+        e("s_mov_b32 %s, %s" % (s(OFF1), s(OFF2)))
+        e("s_mov_b32 %s, %s" % (s(OFF2), s(TMP)))
+        e("s_mov_b32 %s, %s" % (s(TMP), s(RAWC)))
+        e("s_mov_b32 %s, %s" % (s(RAWC), s(RAWN)))
+        e("s_mov_b32 %s, %s" % (s(RAWN), s(TMP)))
+        e("s_add_u32 %s, %s, 1" % (s(IT), s(IT)))
+        e("s_branch %s" % lab_iloop)
+        e("%s:" % lab_iend)
+        e("s_waitcnt vmcnt(0)")
+        e("s_branch %s" % LAB_EXIT)
+        e("%s:" % lab_busy)
+        lds.pending = busy_pending
     else:
         # ------------------------------------------------------------------ tiles 0, 1, 2 -> LDS; go on as soon as Q and tile 0 are there
         lab_w0, lab_w1, lab_wd = label("pw0"), label("pw1"), label("pwd")

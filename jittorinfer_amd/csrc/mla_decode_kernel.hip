@@ -324,10 +324,10 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
     const int s_kve  = __builtin_amdgcn_readfirstlane(kv_end);
     const int s_npp  = __builtin_amdgcn_readfirstlane(p.n_pool_pages - 1);
     const int s_nb1  = __builtin_amdgcn_readfirstlane((int) p.kv_nb1);
-    // bit 0: f32 row store; bit 4: V starts at column 64; bit 5: none of this wave's 32 rows exists (it only moves tiles; the
-    // Q8_0 programs have no such path: their waves share the dequantisation)
+    // bit 0: f32 row store; bit 4: V starts at column 64; bit 5: none of this wave's 32 rows exists (it only moves tiles and,
+    // in the Q8_0 programs, dequantizes its share of them)
     const int s_flg  = __builtin_amdgcn_readfirstlane((direct || p.part_f32 ? 1 : 0) | (p.v_col0 ? 16 : 0) |
-                                                      (KVT != SRC_Q8 && by * 128 + wave * 32 >= p.n_rows ? 32 : 0) | p.debug_flags);
+                                                      (by * 128 + wave * 32 >= p.n_rows ? 32 : 0) | p.debug_flags);
     const int s_ntl  = __builtin_amdgcn_readfirstlane(n_tiles);
     // id of the split's first page as a scalar: the first tiles are requested before the vector load of all page ids is back
     int pg0 = 0;
@@ -369,7 +369,8 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
 
 // Q f32 -> the decode kernel's MFMA operand image, rounded to the KV type as ggml-cpu rounds it (ggml-cpu.c:12034-12035):
 // out[((seq*n_row_blocks + rb)*4 + wave)*36 + ks][lane] = 8 values of row rb*128 + wave*32 + lane%32,
-// columns 16*ks + 8*(lane/32) .. +7.  Rows past n_rows repeat the last row (their results are never stored).
+// columns 16*ks + 8*(lane/32) .. +7.  Rows past n_rows repeat the last row (their results are never stored);
+// a group of 32 rows that lies past n_rows entirely is left unwritten, its wave of the decode kernel neither loads nor computes.
 // grid = (n_row_blocks, n_seq, 36 k-steps), block = 256: one 16-byte output per thread.
 template <bool F16>
 __global__ void __launch_bounds__(NTHREADS) mla_q_pack_kernel(const KParams p) {
