@@ -31,7 +31,9 @@ CLKP = "--clk-parts" in sys.argv    # with --clk: accumulate the cycles of part 
 CLK = "--clk" in sys.argv or CLKP           # timing experiments only: s_memtime stamps, written to the hand-off area at the end
 MASK = "--mask" in sys.argv  # additive f16 mask rows (one per query token), added to the scaled scores
 Q8 = "--q8" in sys.argv    # Q8_0 KV: raw tiles staged in LDS, dequantized to an f16 tile one tile ahead, then the f16 path
-F16 = "--f16" in sys.argv or Q8  # f16 KV: f16 MFMA, single P (no lo half)
+CVTB = "--cvt" in sys.argv  # bf16 KV converted in place to f16 inside LDS one tile ahead (exact between 2^-14 and 65504, saturating
+                            # beyond), then the f16 path: 68 MFMAs per tile instead of the 100 the hi + lo halves of a bf16 P need
+F16 = "--f16" in sys.argv or Q8 or CVTB  # f16 KV: f16 MFMA, single P (no lo half)
 MF = "v_mfma_f32_32x32x16_f16" if F16 else "v_mfma_f32_32x32x16_bf16"
 CVT = "v_cvt_pk_f16_f32" if F16 else "v_cvt_pk_bf16_f32"
 SPLIT = not F16
@@ -59,12 +61,15 @@ P1_LEAD = _opt("--lead", 3)                   # P.V MFMAs at the head of an iter
 # ---- VGPR map
 Q0 = 0
 SA, SB = 144, 160   # two 16-register groups: scores of one tile, converted in place to its P^T operands
-KF, KRING = 176, 4 if MASK else 5   # K fragment ring (x 4 registers)
+KF, KRING = 176, (3 if Q8 or CVTB else 4) if MASK else 5   # K fragment ring (x 4 registers); what a masked build takes from it goes to the mask values / the converter
 ALPHA = 196
 RELOAD_PTRS = Q8 and MASK           # the output pointers are read again from the hand-off record in the epilogue: their registers carry MOFF
 MOFF = 232 if RELOAD_PTRS else 197  # mask builds: byte offset of this lane's first mask element inside a tile's 64 mask bytes
-VF, VRING = 200, 5 if MASK or Q8 else 6   # V^T fragment ring (x 4 registers); 220..223 go to the mask values / the dequantizer
-MKR = [192, 193, 194, 195] + ([252, 253, 254, 255] if Q8 else [220, 221, 222, 223])   # mask builds: the 16 f16 mask values of this lane's 16 tokens of a tile
+# V^T fragment ring (x 4 registers); 220..223 go to the mask values / the dequantizer / the converter.  v252..v255 are never used: the clobber list of the asm block ends at v251, and the compiler
+# keeps what lives across the block there (among it the lanes it spills scalar registers to).
+VF, VRING = 200, 5 if MASK or Q8 or CVTB else 6
+assert 30 % VRING == 0   # the hand-over between tiles relies on the last two fragments of a tile sitting in ring slots 0 and 1
+MKR = [192, 193, 194, 195] + ([188, 189, 190, 191] if Q8 else [220, 221, 222, 223])   # mask builds: the 16 f16 mask values of this lane's 16 tokens of a tile
 T = list(range(224, 232))
 OPTR, MLPTR = 232, 234
 KADDR_LANE, VADDR_LANE, MRUN, LRUN, NEGM = 236, 237, 238, 239, 240
@@ -98,6 +103,7 @@ def label(prefix):
 
 
 def v(i, n=1):
+    assert 0 <= i and i + n - 1 < N_VGPR, (i, n)   # v252..v255 belong to the compiler
     return "v%d" % i if n == 1 else "v[%d:%d]" % (i, i + n - 1)
 
 
@@ -310,6 +316,40 @@ def q8_dequant_items(raw_sreg, dst_sreg, tile_plus):
     return I
 
 
+CVL, CADDR, CT0, CT1 = (188, 189, 190, 191) if MASK else (220, 221, 222, 223)   # --cvt builds: this lane's byte offset inside a tile, the address, two temporaries
+
+
+def cvt_items(off_sreg):
+    """--cvt builds: the bf16 tile at LDS offset s[off_sreg] -> f16, in place.  A wave converts the eight rows it loaded
+    itself (so only its own loads have to be back, no barrier): lane = (row, 16-byte column chunk mod 8), nine units of
+    16 bytes 128 bytes apart.  Per 32-bit word: both halves widened to f32, v_cvt_pkrtz_f16_f32 (exact inside the f16
+    range; round-toward-zero makes larger magnitudes 65504 instead of infinity).  The data registers are T[0:7], free
+    in the part of the iteration that carries these items."""
+    I = ["v_add_u32 %s, %s, %s" % (v(CADDR), s(off_sreg), v(CVL))]
+    D = [T[0], T[4]]
+
+    def rd(u):
+        return lambda: lds.read("ds_read_b128 %s, %s offset:%d" % (v(D[u & 1], 4), v(CADDR), 128 * u), ("r", u))
+
+    I.append(rd(0))
+    for u in range(9):
+        d = D[u & 1]
+        if u + 1 < 9:
+            I.append(rd(u + 1))
+        def first(u=u, d=d):
+            lds.need(("r", u))
+            e("v_lshlrev_b32 %s, 16, %s" % (v(CT0), v(d)))
+        I.append(first)
+        for j in range(4):
+            if j:
+                I.append("v_lshlrev_b32 %s, 16, %s" % (v(CT0), v(d + j)))
+            I.append("v_and_b32 %s, 0xffff0000, %s" % (v(CT1), v(d + j)))
+            I.append("v_cvt_pkrtz_f16_f32 %s, %s, %s" % (v(d + j), v(CT0), v(CT1)))
+        I.append("s_nop 0")
+        I.append(lambda u=u, d=d: lds.read("ds_write_b128 %s, %s offset:%d" % (v(CADDR), v(d, 4), 128 * u), ("w", u)))
+    return I
+
+
 PT = [241, 242, 243, 249, 250]   # 16-bit tiles: per-lane byte offsets of the 10 LDS-DMA slots, two 16-bit values per register
 DT = [251, 199]                  # address temporaries of the slots
 
@@ -444,7 +484,7 @@ def tile_handover(kaddr_off, vaddr_off, last_slots, sync):
         e("v_add_u32 %s, %s, %s" % (v(VADDR), s(vaddr_off), v(VADDR_LANE)))
         for idx in range(2, VRING - 1):
             v_read(VADDR, idx)
-    if Q8:
+    if Q8 or CVTB:
         lds.need(("w", 8))              # this wave's share of the next f16 tile is written
     sync()
     e("v_add_u32 %s, %s, %s" % (v(KADDR), s(kaddr_off), v(KADDR_LANE)))
@@ -672,6 +712,9 @@ def iteration(g_cur, g_next, tag):
     if Q8:
         q8_dma = q8_dma_lines(TMP, RAWN)
         rest_a = part1(q8_dma + q8_dequant_items(RAWC, OFF2, 2))
+    elif CVTB:
+        cv_dma = dma_tile_lines(TMP, OFF3)
+        rest_a = part1(cv_dma + cvt_items(OFF2))
     else:
         rest_a = part1(dma_tile_lines(TMP, OFF3))
     state_a = list(lds.pending)
@@ -679,7 +722,7 @@ def iteration(g_cur, g_next, tag):
     # ---- part 1 without it (tiles IT+3.. do not exist)
     e("%s:" % lab_nodma)
     # (Q8_0: empty items in place of the loads, so that the dequantizer's LDS accesses fall into the same slots on both paths)
-    rest_b = part1([None] * len(q8_dma) + q8_dequant_items(RAWC, OFF2, 2) if Q8 else [])
+    rest_b = part1([None] * len(q8_dma) + q8_dequant_items(RAWC, OFF2, 2) if Q8 else [None] * len(cv_dma) + cvt_items(OFF2) if CVTB else [])
     assert lds.pending == state_a and len(rest_a) == len(rest_b), (lds.pending, state_a)
     # ---- part 2: remaining P.V MFMAs of tile IT, softmax of tile IT+1 in their shadow
     e("%s:" % lab_p2)
@@ -712,8 +755,8 @@ def iteration(g_cur, g_next, tag):
         if CLK and not CLKP:
             e("s_memtime s[94:95]")
             e("s_waitcnt lgkmcnt(0)")
-        if Q8:
-            e("s_waitcnt vmcnt(0)")     # the raw tile loaded during this iteration is dequantized in the next one
+        if Q8 or CVTB:
+            e("s_waitcnt vmcnt(0)")     # the raw tile loaded during this iteration is dequantized / converted in the next one
         else:
             e("s_cmp_eq_u32 %s, 0" % s(VMW))
             e("s_cbranch_scc1 %s" % lab_w0)
@@ -836,6 +879,14 @@ def main():
     e("s_bitcmp1_b32 %s, 4" % s(FLG))
     e("s_cselect_b32 %s, 128, 0" % s(S0))
     e("v_add_u32 %s, %s, %s" % (v(VADDR_LANE), s(S0), v(VADDR_LANE)))
+    if CVTB:
+        # in-place conversion: lane = (row 8 wave + lane / 8, column chunk lane % 8 of every group of eight chunks)
+        e("v_lshrrev_b32 %s, 3, %s" % (v(CVL), v(LANE)))
+        e("s_lshl_b32 %s, %s, 3" % (s(S0), s(WAVE)))
+        e("v_add_u32 %s, %s, %s" % (v(CVL), s(S0), v(CVL)))
+        e("v_and_b32 %s, 7, %s" % (v(CT0), v(LANE)))
+        e("v_lshlrev_b32 %s, 4, %s" % (v(CT0), v(CT0)))
+        e("v_mad_u32_u24 %s, %s, %s, %s" % (v(CVL), v(CVL), s(SPITCH), v(CT0)))
     # ------------------------------------------------------------------ page ids of this split -> one lane each
     lab_nobt = label("nobt")
     e("s_lshr_b32 %s, %s, 7" % (s(PG0), s(KVB)))
@@ -1044,54 +1095,107 @@ def main():
         e("s_waitcnt vmcnt(0)")
         e("%s:" % lab_wd)
         page_clamp()
+        if CVTB:
+            # this wave's rows of tile 0 -> f16; once every wave has done that, the same for tile 1 (its loads may still be in
+            # flight with those of tile 2 behind them); tile 2 is converted by iteration 0
+            for it_ in cvt_items(OFF0):
+                emit_item(it_)
+            lds.drain()
         e("s_barrier")
-        # ---------------------------------------------------------------- waves without a valid row (FLG bit 5; fewer than 97 rows in
-        # the block, e.g. a 16- or 32-head model's decode step): they keep moving their eight rows of every tile and meet the
-        # others at every barrier, and issue no MFMA, no fragment read and no softmax: a quarter of the matrix-core power for a
-        # 32-head model, which the chip-wide clock gives back to the wave that computes
-        lab_busy, lab_iloop, lab_inodma, lab_iw0, lab_iwd, lab_iend = (label(x) for x in ("busy", "iloop", "inodma", "iw0", "iwd", "iend"))
-        lab_it1, lab_it1d = label("it1"), label("it1d")
-        e("s_bitcmp1_b32 %s, 5" % s(FLG))
-        e("s_cbranch_scc0 %s" % lab_busy)
-        e("s_cmp_lt_u32 %s, 3" % s(NT))                 # as the first hand-over: tile 1 has landed
-        e("s_cbranch_scc1 %s" % lab_it1)
-        e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
-        e("s_branch %s" % lab_it1d)
-        e("%s:" % lab_it1)
-        e("s_waitcnt vmcnt(0)")
-        e("%s:" % lab_it1d)
-        e("s_barrier")
-        e("%s:" % lab_iloop)
-        e("s_add_u32 %s, %s, 1" % (s(TMP), s(IT)))
-        e("s_cmp_ge_u32 %s, %s" % (s(TMP), s(NT)))
-        e("s_cbranch_scc1 %s" % lab_iend)               # the last tile has no successor to wait for
-        e("s_mov_b32 %s, 0" % s(VMW))
-        e("s_add_u32 %s, %s, 3" % (s(TMP), s(IT)))
-        e("s_cmp_ge_u32 %s, %s" % (s(TMP), s(NT)))
-        e("s_cbranch_scc1 %s" % lab_inodma)
-        e("s_mov_b32 %s, 1" % s(VMW))
-        for ln in dma_tile_lines(TMP, OFF3):
-            e(ln)
-        e("%s:" % lab_inodma)
-        e("s_cmp_eq_u32 %s, 0" % s(VMW))
-        e("s_cbranch_scc1 %s" % lab_iw0)
-        e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
-        e("s_branch %s" % lab_iwd)
-        e("%s:" % lab_iw0)
-        e("s_waitcnt vmcnt(0)")
-        e("%s:" % lab_iwd)
-        e("s_barrier")
-        e("s_mov_b32 %s, %s" % (s(TMP), s(OFF0)))
-        e("s_mov_b32 %s, %s" % (s(OFF0), s(OFF1)))
-        e("s_mov_b32 %s, %s" % (s(OFF1), s(OFF2)))
-        e("s_mov_b32 %s, %s" % (s(OFF2), s(OFF3)))
-        e("s_mov_b32 %s, %s" % (s(OFF3), s(TMP)))
-        e("s_add_u32 %s, %s, 1" % (s(IT), s(IT)))
-        e("s_branch %s" % lab_iloop)
-        e("%s:" % lab_iend)
-        e("s_waitcnt vmcnt(0)")
-        e("s_branch %s" % LAB_EXIT)
-        e("%s:" % lab_busy)
+        if CVTB:
+            lab_c1, lab_c1d = label("c1"), label("c1d")
+            e("s_cmp_lt_u32 %s, 3" % s(NT))
+            e("s_cbranch_scc1 %s" % lab_c1)
+            e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
+            e("s_branch %s" % lab_c1d)
+            e("%s:" % lab_c1)
+            e("s_waitcnt vmcnt(0)")
+            e("%s:" % lab_c1d)
+            for it_ in cvt_items(OFF1):
+                emit_item(it_)
+            # waves without a valid row: their share of the loads and of the conversion, every barrier, nothing else
+            lab_busy, lab_iloop, lab_inodma, lab_iend = (label(x) for x in ("busy", "iloop", "inodma", "iend"))
+            busy_pending = list(lds.pending)
+            e("s_bitcmp1_b32 %s, 5" % s(FLG))
+            e("s_cbranch_scc0 %s" % lab_busy)
+            lds.drain()
+            e("s_waitcnt vmcnt(0)")
+            e("s_barrier")
+            e("%s:" % lab_iloop)
+            e("s_add_u32 %s, %s, 1" % (s(TMP), s(IT)))
+            e("s_cmp_ge_u32 %s, %s" % (s(TMP), s(NT)))
+            e("s_cbranch_scc1 %s" % lab_iend)
+            e("s_add_u32 %s, %s, 3" % (s(TMP), s(IT)))
+            e("s_cmp_ge_u32 %s, %s" % (s(TMP), s(NT)))
+            e("s_cbranch_scc1 %s" % lab_inodma)
+            for ln in dma_tile_lines(TMP, OFF3):
+                e(ln)
+            e("%s:" % lab_inodma)
+            for it_ in cvt_items(OFF2):
+                emit_item(it_)
+            lds.drain()
+            e("s_waitcnt vmcnt(0)")
+            e("s_barrier")
+            e("s_mov_b32 %s, %s" % (s(TMP), s(OFF0)))
+            e("s_mov_b32 %s, %s" % (s(OFF0), s(OFF1)))
+            e("s_mov_b32 %s, %s" % (s(OFF1), s(OFF2)))
+            e("s_mov_b32 %s, %s" % (s(OFF2), s(OFF3)))
+            e("s_mov_b32 %s, %s" % (s(OFF3), s(TMP)))
+            e("s_add_u32 %s, %s, 1" % (s(IT), s(IT)))
+            e("s_branch %s" % lab_iloop)
+            e("%s:" % lab_iend)
+            e("s_waitcnt vmcnt(0)")
+            e("s_branch %s" % LAB_EXIT)
+            e("%s:" % lab_busy)
+            lds.pending = busy_pending
+        if not CVTB:
+            # ---------------------------------------------------------------- waves without a valid row (FLG bit 5; fewer than 97 rows in
+            # the block, e.g. a 16- or 32-head model's decode step): they keep moving their eight rows of every tile and meet the
+            # others at every barrier, and issue no MFMA, no fragment read and no softmax: a quarter of the matrix-core power for a
+            # 32-head model, which the chip-wide clock gives back to the wave that computes
+            lab_busy, lab_iloop, lab_inodma, lab_iw0, lab_iwd, lab_iend = (label(x) for x in ("busy", "iloop", "inodma", "iw0", "iwd", "iend"))
+            lab_it1, lab_it1d = label("it1"), label("it1d")
+            e("s_bitcmp1_b32 %s, 5" % s(FLG))
+            e("s_cbranch_scc0 %s" % lab_busy)
+            e("s_cmp_lt_u32 %s, 3" % s(NT))                 # as the first hand-over: tile 1 has landed
+            e("s_cbranch_scc1 %s" % lab_it1)
+            e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
+            e("s_branch %s" % lab_it1d)
+            e("%s:" % lab_it1)
+            e("s_waitcnt vmcnt(0)")
+            e("%s:" % lab_it1d)
+            e("s_barrier")
+            e("%s:" % lab_iloop)
+            e("s_add_u32 %s, %s, 1" % (s(TMP), s(IT)))
+            e("s_cmp_ge_u32 %s, %s" % (s(TMP), s(NT)))
+            e("s_cbranch_scc1 %s" % lab_iend)               # the last tile has no successor to wait for
+            e("s_mov_b32 %s, 0" % s(VMW))
+            e("s_add_u32 %s, %s, 3" % (s(TMP), s(IT)))
+            e("s_cmp_ge_u32 %s, %s" % (s(TMP), s(NT)))
+            e("s_cbranch_scc1 %s" % lab_inodma)
+            e("s_mov_b32 %s, 1" % s(VMW))
+            for ln in dma_tile_lines(TMP, OFF3):
+                e(ln)
+            e("%s:" % lab_inodma)
+            e("s_cmp_eq_u32 %s, 0" % s(VMW))
+            e("s_cbranch_scc1 %s" % lab_iw0)
+            e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
+            e("s_branch %s" % lab_iwd)
+            e("%s:" % lab_iw0)
+            e("s_waitcnt vmcnt(0)")
+            e("%s:" % lab_iwd)
+            e("s_barrier")
+            e("s_mov_b32 %s, %s" % (s(TMP), s(OFF0)))
+            e("s_mov_b32 %s, %s" % (s(OFF0), s(OFF1)))
+            e("s_mov_b32 %s, %s" % (s(OFF1), s(OFF2)))
+            e("s_mov_b32 %s, %s" % (s(OFF2), s(OFF3)))
+            e("s_mov_b32 %s, %s" % (s(OFF3), s(TMP)))
+            e("s_add_u32 %s, %s, 1" % (s(IT), s(IT)))
+            e("s_branch %s" % lab_iloop)
+            e("%s:" % lab_iend)
+            e("s_waitcnt vmcnt(0)")
+            e("s_branch %s" % LAB_EXIT)
+            e("%s:" % lab_busy)
     stamp(1)
     if DEBUG:
         # FLG bit 1: dump LDS tile 0 (2336 chunks) to the debug pointer and stop
@@ -1132,7 +1236,7 @@ def main():
     # tile 1 has landed (tile 2 may still be in flight); first fragment reads of iteration 0
     def sync0():
         lab_t1, lab_t1d = label("t1"), label("t1d")
-        if Q8:
+        if Q8 or CVTB:
             e("s_waitcnt vmcnt(0)")     # f16 tile 1 written (the hand-over waited for this wave's writes), raw tile 2 landed
             e("s_barrier")
             return
@@ -1144,7 +1248,7 @@ def main():
         e("s_waitcnt vmcnt(0)")
         e("%s:" % lab_t1d)
         e("s_barrier")
-    assert Q8 or not lds.pending
+    assert Q8 or CVTB or not lds.pending
     tile_handover(OFF1, OFF0, [], sync0)
     # ------------------------------------------------------------------ main loop (two copies: the register groups swap roles)
     lab_loop, lab_end = label("loop"), label("end")

@@ -346,6 +346,14 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
         asm volatile(
 #include "mla_decode_asm_q8.inc"
             : : MLA_DECODE_INPUTS : MLA_DECODE_CLOBBERS);
+    } else if constexpr (KVT == SRC_BF16_CVT && MASK) {
+        asm volatile(
+#include "mla_decode_asm_cvt_mask.inc"
+            : : MLA_DECODE_INPUTS : MLA_DECODE_CLOBBERS);
+    } else if constexpr (KVT == SRC_BF16_CVT) {
+        asm volatile(
+#include "mla_decode_asm_cvt.inc"
+            : : MLA_DECODE_INPUTS : MLA_DECODE_CLOBBERS);
     } else if constexpr (KVT == SRC_F16 && MASK) {
         asm volatile(
 #include "mla_decode_asm_f16_mask.inc"
@@ -372,7 +380,15 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
 // columns 16*ks + 8*(lane/32) .. +7.  Rows past n_rows repeat the last row (their results are never stored);
 // a group of 32 rows that lies past n_rows entirely is left unwritten, its wave of the decode kernel neither loads nor computes.
 // grid = (n_row_blocks, n_seq, 36 k-steps), block = 256: one 16-byte output per thread.
-template <bool F16>
+// MODE 0: bf16 operands; 1: f16; 2: rounded to bf16 as for MODE 0, then written as f16 (exact inside the f16 range,
+// +-65504 beyond it) for the program that converts its bf16 tiles to f16.
+template <int MODE> __device__ __forceinline__ unsigned int pack_q2(float a, float b) {
+    if constexpr (MODE == 2) {
+        const auto h = __builtin_amdgcn_cvt_pkrtz(round_trip<false>(a), round_trip<false>(b));
+        return bitcast<unsigned int>(h);
+    } else return pack2<MODE == 1>(a, b);
+}
+template <int MODE>
 __global__ void __launch_bounds__(NTHREADS) mla_q_pack_kernel(const KParams p) {
     if (blockIdx.z == gridDim.z - 1 && p.balanced == 1) {   // balanced schedule: one extra layer of blocks, the first of which builds it
         if (blockIdx.x == 0 && blockIdx.y == 0) sched_prefix(p);
@@ -388,7 +404,7 @@ __global__ void __launch_bounds__(NTHREADS) mla_q_pack_kernel(const KParams p) {
     u32x4 * out = (u32x4 *) p.q_pack + ((((int64_t) b * gridDim.x + blockIdx.x) * 4 + wave) * KSTEPS) * 64 + lane;
     const f32x4 x0 = *(const f32x4 *) (qrow + 16 * ks);
     const f32x4 x1 = *(const f32x4 *) (qrow + 16 * ks + 4);
-    out[ks * 64] = u32x4{ pack2<F16>(x0.x, x0.y), pack2<F16>(x0.z, x0.w), pack2<F16>(x1.x, x1.y), pack2<F16>(x1.z, x1.w) };
+    out[ks * 64] = u32x4{ pack_q2<MODE>(x0.x, x0.y), pack_q2<MODE>(x0.z, x0.w), pack_q2<MODE>(x1.x, x1.y), pack_q2<MODE>(x1.z, x1.w) };
 }
 
 // Per block of 128 rows and per sixteenth of the mask row: the first key and one past the last key that any of the
@@ -573,13 +589,17 @@ hipError_t launch_decode_fast(const KParams & kp, int kv_type, dim3 grid, hipStr
     // the small passes ahead of the kernel run per (row block, sequence), whatever the kernel's own grid is
     const unsigned n_rb = (unsigned) ((kp.n_rows + 127) / 128), n_seq = (unsigned) kp.n_seq_sched, extra = kp.balanced == 1 ? 1 : 0;
     const bool m = kp.mask != nullptr;
+    static const bool bf16_cvt_env = [] { const char * v = getenv("MLA_BF16_PROGRAM"); return v && v[0] == 'c'; }();
+    const bool bf16_cvt = bf16_cvt_env;
     if (!with_prepass) { /* the workspace still holds the Q image and the mask extents of an earlier launch of the same call */ }
     else if (kv_type == MLA_TYPE_Q8_0 || kp.q_as_q8) hipLaunchKernelGGL(mla_q_pack_q8_kernel, dim3(n_rb, n_seq, KSTEPS / 2 + extra), dim3(NTHREADS), 0, st, kp);
-    else if (kv_type == MLA_TYPE_F16) hipLaunchKernelGGL(mla_q_pack_kernel<true>, dim3(n_rb, n_seq, KSTEPS + extra), dim3(NTHREADS), 0, st, kp);
-    else                              hipLaunchKernelGGL(mla_q_pack_kernel<false>, dim3(n_rb, n_seq, KSTEPS + extra), dim3(NTHREADS), 0, st, kp);
+    else if (kv_type == MLA_TYPE_F16) hipLaunchKernelGGL(mla_q_pack_kernel<1>, dim3(n_rb, n_seq, KSTEPS + extra), dim3(NTHREADS), 0, st, kp);
+    else if (bf16_cvt)                hipLaunchKernelGGL(mla_q_pack_kernel<2>, dim3(n_rb, n_seq, KSTEPS + extra), dim3(NTHREADS), 0, st, kp);
+    else                              hipLaunchKernelGGL(mla_q_pack_kernel<0>, dim3(n_rb, n_seq, KSTEPS + extra), dim3(NTHREADS), 0, st, kp);
     if (m && with_prepass) hipLaunchKernelGGL(mla_mask_extent_kernel, dim3(n_rb, MASK_EXT_CHUNKS), dim3(NTHREADS), 0, st, kp);
     if (kv_type == MLA_TYPE_Q8_0) return m ? launch_variant<SRC_Q8, true>(kp, grid, st) : launch_variant<SRC_Q8, false>(kp, grid, st);
     if (kv_type == MLA_TYPE_F16)  return m ? launch_variant<SRC_F16, true>(kp, grid, st) : launch_variant<SRC_F16, false>(kp, grid, st);
+    if (bf16_cvt)                 return m ? launch_variant<SRC_BF16_CVT, true>(kp, grid, st) : launch_variant<SRC_BF16_CVT, false>(kp, grid, st);
     return m ? launch_variant<SRC_BF16, true>(kp, grid, st) : launch_variant<SRC_BF16, false>(kp, grid, st);
 }
 
