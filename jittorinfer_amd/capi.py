@@ -7,6 +7,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 MLA_TYPE_F32, MLA_TYPE_F16, MLA_TYPE_Q8_0, MLA_TYPE_BF16 = 0, 1, 8, 30
 MLA_FLAG_F16_ACC_STRICT = 1
 MLA_FLAG_UNIFORM_SPLITS = 2
+MLA_FLAG_BF16_DIRECT = 4
 PAGE_TOKENS = 128
 ROW_BYTES = {MLA_TYPE_F16: 1152, MLA_TYPE_BF16: 1152, MLA_TYPE_Q8_0: 612}
 

@@ -68,6 +68,7 @@ struct backend_ctx {
     void *      workspace      = nullptr;
     size_t      workspace_size = 0;
     bool        f16_strict     = false;   // F16 KV: replay ggml-cpu's f16 accumulator instead of accumulating in f32
+    bool        bf16_direct    = false;   // BF16 KV: the hi + lo bf16 program instead of the one that converts the tiles to f16 (MLA_FLAG_BF16_DIRECT)
 };
 
 std::vector<device_ctx *>     g_device_ctx;
@@ -459,6 +460,7 @@ int compute_flash_attn(backend_ctx * ctx, const tensor * dst) {
     if (bt) { a.block_table = (const int32_t *) bt->data; a.bt_stride = bt->ne[0]; a.seq_lens = (const int32_t *) lens->data; }
     a.dst = (float *) dst->data; a.dst_nb1 = (int64_t) dst->nb[1];
     if (ctx->f16_strict && k->type == TYPE_F16 && !bt) a.flags |= MLA_FLAG_F16_ACC_STRICT;
+    if (ctx->bf16_direct) a.flags |= MLA_FLAG_BF16_DIRECT;
 
     const size_t need = mla_attn_workspace_size(&a);
     if (need > ctx->workspace_size) {
@@ -638,6 +640,8 @@ backend * device_init_backend(backend_device * dev, const char * params) {
     ctx->name   = dc->name;
     const char * env = getenv("GGML_HIP_MLA_F16_ACC");
     ctx->f16_strict = (params && strstr(params, "f16_acc=strict")) || (env && strcmp(env, "strict") == 0);
+    const char * env_bf = getenv("GGML_HIP_MLA_BF16");
+    ctx->bf16_direct = (params && strstr(params, "bf16=direct")) || (env_bf && strcmp(env_bf, "direct") == 0);
     if (!HIP_OK(hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking))) { delete ctx; return nullptr; }
     return new backend{ &g_guid, k_backend_iface, dev, ctx };
 }

@@ -74,6 +74,7 @@ struct KParams {
     int             v_col0;        // pipelined kernel: V = columns v_col0 .. v_col0 + 511 of the rows (0, or 64 in the second pass of a
                                    // 576-wide V), and the 512 results go to columns v_col0 .. of the dst rows
     int             q_as_q8;       // the KV rows are the f16 expansion of a Q8_0 cache: Q is quantized the Q8_0 way
+    int             bf16_direct;   // bf16 KV: the hi + lo program instead of the one that converts the tiles to f16 (MLA_FLAG_BF16_DIRECT)
     int             rows_contig;  // kv rows are packed (kv_nb1 == row bytes): whole tiles are one contiguous run
 };
 

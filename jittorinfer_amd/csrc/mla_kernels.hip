@@ -874,6 +874,7 @@ static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
     kp.part_f32 = pl.part_f32;
     kp.rel_splits = a->mask != nullptr && (pl.variant == 2 || pl.ws_maskext > 0);
     kp.balanced = pl.balanced; kp.n_wg = pl.n_wg; kp.n_seq_sched = a->n_seq; kp.n_units = pl.n_units;
+    kp.bf16_direct = (a->flags & MLA_FLAG_BF16_DIRECT) ? 1 : 0;
     kp.slot_rows = pl.balanced == 2 ? 128 : kp.n_rows;
     kp.part_ml = (float *) (ws + align256(pl.ws_part_o));
     float * scores = (float *) (ws + align256(pl.ws_part_o) + align256(pl.ws_part_ml));

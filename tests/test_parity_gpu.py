@@ -133,7 +133,7 @@ def _plan_variant(gpu, q, k, k_type, mask, bt, lens, **kw):
     import jittorinfer_amd as J
     tq = torch.from_numpy(q).to(gpu)
     tk = torch.from_numpy(k.view(np.int16) if k.dtype == np.uint16 else k).to(gpu)
-    tm = torch.from_numpy(mask.view(np.float16)).to(gpu)
+    tm = None if mask is None else torch.from_numpy(mask.view(np.float16)).to(gpu)
     tb = None if bt is None else torch.from_numpy(bt).to(gpu)
     tl = None if lens is None else torch.from_numpy(np.asarray(lens, dtype=np.int32)).to(gpu)
     return J.plan(tq, tk, k_type, dv=512, mask=tm, block_table=tb, seq_lens=tl, **kw)["variant"]
@@ -253,3 +253,45 @@ def test_dv576_paged_split_and_masked(gpu, k_type):
     got = _run(gpu, q, k, k_type, dv=576, mask=m.view(np.uint16), scale=U.SCALE)
     want = O.flash_attn_ext(q, k, k_type, dv=576, mask=m.view(np.uint16), scale=U.SCALE)
     print(U.check(got, want, "dv 576 masked"))
+
+
+@pytest.mark.parametrize("masked", [False, True])
+def test_bf16_direct_program_and_values_beyond_the_f16_range(gpu, masked):
+    """BF16 cache: by default the decode kernel converts its tiles to f16 inside LDS (bit-exact operands for magnitudes in
+    [2^-14, 65504], probabilities rounded to f16); MLA_FLAG_BF16_DIRECT keeps the tiles in bf16 and feeds the probabilities
+    as two bf16 halves.  Both are held to the oracle on ordinary values, the direct program more tightly; with 1e6 and
+    1e-30 in the cache only the direct program is (the converting one saturates at 65504, as documented)."""
+    import jittorinfer_amd as J
+    rng = np.random.default_rng(77 + masked)
+    n_kv, n_tok = 512, (3 if masked else 1)
+    q = rng.standard_normal((2, 128, n_tok, 576)).astype(np.float32)
+    kf = rng.standard_normal((2, n_kv, 576)).astype(np.float32)
+    mask = None
+    if masked:
+        m = (rng.standard_normal((n_tok, n_kv)) * 2).astype(np.float32)
+        m[rng.random((n_tok, n_kv)) < 0.3] = -np.inf
+        mask = m.astype(np.float16).view(np.uint16)
+    k = U.encode_kv(kf, O.TYPE_BF16)
+    kw = dict(mask=mask, scale=U.SCALE, n_splits=2)
+    assert _plan_variant(gpu, q, k, O.TYPE_BF16, mask, None, None, scale=U.SCALE, n_splits=2) == 2
+    want = O.flash_attn_ext(q, k, O.TYPE_BF16, dv=512, mask=mask, scale=U.SCALE)
+    conv = _run(gpu, q, k, O.TYPE_BF16, **kw)
+    direct = _run(gpu, q, k, O.TYPE_BF16, flags=J.MLA_FLAG_BF16_DIRECT, **kw)
+    print(U.check(conv[..., :512], want, "bf16 tiles converted to f16"))
+    print(U.check(direct[..., :512], want, "bf16 tiles as they are", max_abs=2e-5, rel_l2=2e-5))
+    assert not np.array_equal(conv, direct)            # two different programs ran
+    # values outside the f16 range, in V columns and in the rope columns
+    kf[0, 5, 17] = 1.0e6
+    kf[1, 200, 300] = -3.0e5
+    kf[:, 7, 100] = 1.0e-30
+    kf[0, 9, 530] = 2.0e5
+    k = U.encode_kv(kf, O.TYPE_BF16)
+    want = O.flash_attn_ext(q, k, O.TYPE_BF16, dv=512, mask=mask, scale=U.SCALE)
+    direct = _run(gpu, q, k, O.TYPE_BF16, flags=J.MLA_FLAG_BF16_DIRECT, **kw)
+    assert np.nanmax(np.abs(want)) > 1e3
+    big = np.where(np.isnan(want), 0, np.abs(want)).max(axis=(0, 1, 2)) > 100.0      # columns that carry the large values
+    print(U.check(direct[..., :512][..., ~big], want[..., ~big], "direct, ordinary columns", max_abs=1e-4, rel_l2=2e-5))
+    rel = np.nanmax(np.abs(direct[..., :512][..., big] - want[..., big]) / (np.abs(want[..., big]) + 1.0))
+    assert rel < 1e-5, rel
+    conv = _run(gpu, q, k, O.TYPE_BF16, **kw)
+    assert np.isfinite(conv[..., :512][~np.isnan(want)]).all()      # saturated, never infinite
