@@ -337,7 +337,7 @@ def other_config(a, dev, lib, J):
         q, pool, bt, sl = build_paged(dev, lens, n_head, n_tok, kv, a.seed)
         out = torch.empty((len(lens), n_tok, n_head, 576), dtype=torch.float32, device=dev)
     kw = dict(dv=512, scale=scale, mask=mask, block_table=bt, seq_lens=sl, out=out, n_splits=a.splits, rows_per_wg=a.rows_per_wg,
-              flags=J.MLA_FLAG_UNIFORM_SPLITS if a.uniform_splits else 0)
+              flags=(J.MLA_FLAG_UNIFORM_SPLITS if a.uniform_splits else 0) | (J.MLA_FLAG_BF16_DIRECT if a.bf16_direct else 0))
     ar, _, keep = J.capi.make_args(q, pool, kvt, **kw)
     plan = J.plan(q, pool, kvt, **kw)
     stream = torch.cuda.current_stream(dev)
@@ -453,6 +453,7 @@ def main():
     ap.add_argument("--kv", default="bf16", choices=["bf16", "f16", "q8_0"], help="storage type of the latent KV pool (the headline config is bf16; q8_0 only with --config kvwrite)")
     ap.add_argument("--ragged", action="store_true", help="--config c3mask: sequence lengths uniform in [2048, 8192] instead of 8192")
     ap.add_argument("--uniform-splits", action="store_true", help="paged decode: equal KV splits per sequence (MLA_FLAG_UNIFORM_SPLITS) instead of the balanced schedule")
+    ap.add_argument("--bf16-direct", action="store_true", help="bf16 KV: the hi + lo bf16 program (MLA_FLAG_BF16_DIRECT) instead of the default one that converts the tiles to f16 inside LDS")
     ap.add_argument("--eager", action="store_true", help="time the K steps as K eager launch sequences instead of one replay of a HIP graph that holds them")
     ap.add_argument("--config", default="c3", choices=["c2", "c3", "c3mask", "c4", "c5", "kvwrite", "rope", "absorb", "unabsorb", "layer"],
                     help="c3 (default) is the headline workload; the others time BASELINE's remaining GPU configs and the cache write for the profiles")
@@ -493,7 +494,7 @@ def main():
     for pool in pools:
         ar, _, k = J.capi.make_args(q, pool.view(torch.int16), kv_type, dv=512, scale=scale, block_table=block_table,
                                     seq_lens=seq_lens, out=out, n_splits=a.splits, rows_per_wg=a.rows_per_wg,
-                                    flags=J.MLA_FLAG_UNIFORM_SPLITS if a.uniform_splits else 0)
+                                    flags=(J.MLA_FLAG_UNIFORM_SPLITS if a.uniform_splits else 0) | (J.MLA_FLAG_BF16_DIRECT if a.bf16_direct else 0))
         args.append(ar)
         keep.append(k)
     plan = J.plan(q, pools[0].view(torch.int16), kv_type, dv=512, scale=scale, block_table=block_table, seq_lens=seq_lens, out=out, n_splits=a.splits, rows_per_wg=a.rows_per_wg)
