@@ -138,6 +138,9 @@ __device__ __forceinline__ void sched_prefix(const KParams & p) {
 // The wave-level program is generated by gen_decode_asm.py (register map, LDS-DMA issue, MFMA/VALU interleave).
 // KVT = SRC_BF16: bf16 KV rows, bf16 MFMA, P fed as hi + lo halves.   SRC_F16: f16 KV rows, f16 MFMA, single P.
 // SRC_Q8: packed Q8_0 rows (612 bytes, contiguous), dequantized in LDS to f16 tiles one tile ahead, then as SRC_F16.
+// SRC_BF16_CVT: bf16 KV rows converted in place to f16 inside LDS two tiles ahead (every wave the rows it loaded), then as
+// SRC_F16; exact for magnitudes in [2^-14, 65504], +-65504 beyond.  The default for a bf16 cache; MLA_FLAG_BF16_DIRECT
+// selects SRC_BF16.
 // MASK: an f16 mask row per query token is added to the scaled scores (ggml-cpu.c:12041-12057).  Only the key range
 // p.mask_ext[2*row block .. +1] (first / one past the last key that any row of the block may attend to, rounded to
 // tiles) is visited, and the KV splits divide that range, not the whole cache: the reference's batched decode, where
