@@ -169,3 +169,6 @@ def test_committed_wave_programs_are_what_the_generator_emits(flags, name):
     for m in re.finditer(r"\bv(\d+)\b|\bv\[(\d+):(\d+)\]", got):
         hi = int(m.group(1)) if m.group(1) else int(m.group(3))
         assert hi <= 251, "%s uses %s" % (name, m.group(0))
+    for m in re.finditer(r"\bs(\d+)\b|\bs\[(\d+):(\d+)\]", got):      # scalar registers: inside the clobbered range s40..s83
+        lo, hi = (int(m.group(1)),) * 2 if m.group(1) else (int(m.group(2)), int(m.group(3)))
+        assert 40 <= lo and hi <= 83, "%s uses %s" % (name, m.group(0))
