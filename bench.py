@@ -600,7 +600,8 @@ def main():
     # counters read for the library's copy kernel; figures and commands in profiles/mla_decode_kernel_c3_pmc.md
     traffic = None
     if a.batch == 32 and a.heads == 128 and a.ctx == 8192 and a.kv == "bf16":
-        traffic = int(150524 * 1024 * (294912 / 147466.0) + 34048 * 1024)
+        fetch_kib, write_kib = (150524, 34048) if a.bf16_direct else (150051, 35072)   # KiB per dispatch, mean
+        traffic = int(fetch_kib * 1024 * (294912 / 147466.0) + write_kib * 1024)
     res = {
         "metric": "mla_paged_decode_kv_read_bandwidth", "value": value, "unit": "GB/s",
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms_per_step,
