@@ -62,13 +62,13 @@ P1_LEAD = _opt("--lead", 3)                   # P.V MFMAs at the head of an iter
 # ---- VGPR map
 Q0 = 0
 SA, SB = 144, 160   # two 16-register groups: scores of one tile, converted in place to its P^T operands
-KF, KRING = 176, (3 if Q8 or CVTB else 4) if MASK else 5   # K fragment ring (x 4 registers); what a masked build takes from it goes to the mask values / the converter
+KF, KRING = 176, (3 if Q8 else 4) if MASK else 5   # K fragment ring (x 4 registers); what a masked build takes from it goes to the mask values
 ALPHA = 196
 RELOAD_PTRS = Q8 and MASK           # the output pointers are read again from the hand-off record in the epilogue: their registers carry MOFF
 MOFF = 232 if RELOAD_PTRS else 197  # mask builds: byte offset of this lane's first mask element inside a tile's 64 mask bytes
 # V^T fragment ring (x 4 registers); 220..223 go to the mask values / the dequantizer / the converter.  v252..v255 are never used: the clobber list of the asm block ends at v251, and the compiler
 # keeps what lives across the block there (among it the lanes it spills scalar registers to).
-VF, VRING = 200, 5 if MASK or Q8 or CVTB else 6
+VF, VRING = 200, 5 if MASK or Q8 else 6
 assert 30 % VRING == 0   # the hand-over between tiles relies on the last two fragments of a tile sitting in ring slots 0 and 1
 MKR = [192, 193, 194, 195] + ([188, 189, 190, 191] if Q8 else [220, 221, 222, 223])   # mask builds: the 16 f16 mask values of this lane's 16 tokens of a tile
 T = list(range(224, 232))
@@ -317,7 +317,10 @@ def q8_dequant_items(raw_sreg, dst_sreg, tile_plus):
     return I
 
 
-CVL, CADDR, CT0, CT1 = (188, 189, 190, 191) if MASK else (220, 221, 222, 223)   # --cvt builds: this lane's byte offset inside a tile, the address, two temporaries
+# --cvt builds: this lane's byte offset inside a tile (v198 is free in every build without a dequantizer), and for the address and
+# two temporaries the registers of NEGM, ALPHA and TMAX: those live from the softmax to the end of an iteration, the converter
+# runs in part 1 and in the prologue
+CVL, CADDR, CT0, CT1 = 198, 240, 196, 248
 
 
 def cvt_items(off_sreg):
