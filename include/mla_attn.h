@@ -41,7 +41,8 @@ extern "C" {
                                       sequence the block table can hold) instead of the balanced schedule that deals equal
                                       runs of the batch's whole page list to the workgroups; for comparing the two */
 #define MLA_FLAG_BF16_DIRECT 4u    /* BF16 KV, pipelined kernel: multiply the bf16 tiles as they are, with the probabilities fed as
-                                      hi + lo bf16 halves (100 MFMAs per 32 keys).  Without the flag the tiles are converted
+                                      hi + lo bf16 halves (100 MFMAs per 32 keys).  Without the flag, and with more than 32
+                                      attention rows (heads x query tokens) per sequence, the tiles are converted
                                       to f16 inside LDS and the f16 path runs (68 MFMAs): exact for values whose magnitude is
                                       0 or in [2^-14, 65504] (bf16 has fewer mantissa bits than f16), larger ones become
                                       +-65504, smaller ones lose bits below 2^-24; probabilities are rounded to f16.  Set it

@@ -592,7 +592,9 @@ hipError_t launch_decode_fast(const KParams & kp, int kv_type, dim3 grid, hipStr
     // the small passes ahead of the kernel run per (row block, sequence), whatever the kernel's own grid is
     const unsigned n_rb = (unsigned) ((kp.n_rows + 127) / 128), n_seq = (unsigned) kp.n_seq_sched, extra = kp.balanced == 1 ? 1 : 0;
     const bool m = kp.mask != nullptr;
-    const bool bf16_cvt = !kp.bf16_direct;   // bf16 tiles converted to f16 inside LDS unless the caller asks for the hi + lo program
+    // bf16 tiles are converted to f16 inside LDS unless the caller asks for the hi + lo program, or a single wave of a workgroup
+    // has rows (16- and 32-head decode): one computing wave is not bound by its MFMAs, and the hi + lo program is the more exact
+    const bool bf16_cvt = !kp.bf16_direct && kp.n_rows > 32;
     if (!with_prepass) { /* the workspace still holds the Q image and the mask extents of an earlier launch of the same call */ }
     else if (kv_type == MLA_TYPE_Q8_0 || kp.q_as_q8) hipLaunchKernelGGL(mla_q_pack_q8_kernel, dim3(n_rb, n_seq, KSTEPS / 2 + extra), dim3(NTHREADS), 0, st, kp);
     else if (kv_type == MLA_TYPE_F16) hipLaunchKernelGGL(mla_q_pack_kernel<1>, dim3(n_rb, n_seq, KSTEPS + extra), dim3(NTHREADS), 0, st, kp);
