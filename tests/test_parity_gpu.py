@@ -295,3 +295,19 @@ def test_bf16_direct_program_and_values_beyond_the_f16_range(gpu, masked):
     assert rel < 1e-5, rel
     conv = _run(gpu, q, k, O.TYPE_BF16, **kw)
     assert np.isfinite(conv[..., :512][~np.isnan(want)]).all()      # saturated, never infinite
+
+
+def test_bf16_few_rows_keep_the_direct_program(gpu):
+    """With at most 32 attention rows per sequence (a 16- or 32-head decode step) one wave of a workgroup computes and the
+    conversion of the tiles buys nothing: such launches run the hi + lo bf16 program whether the flag is set or not."""
+    import jittorinfer_amd as J
+    rng = np.random.default_rng(99)
+    lens = [700, 129, 300]
+    pool, bt, seqs = U.make_paged(rng, lens, O.TYPE_BF16)
+    for n_head in (16, 32):
+        q = rng.standard_normal((3, n_head, 1, 576)).astype(np.float32)
+        a = _run(gpu, q, pool, O.TYPE_BF16, bt=bt, lens=lens, scale=U.SCALE)
+        b = _run(gpu, q, pool, O.TYPE_BF16, bt=bt, lens=lens, scale=U.SCALE, flags=J.MLA_FLAG_BF16_DIRECT)
+        assert np.array_equal(a.view(np.int32), b.view(np.int32))
+        want = U.oracle_per_seq(q, seqs, O.TYPE_BF16, 512)
+        print(n_head, U.check(a[..., :512], want, "few rows", max_abs=2e-5, rel_l2=2e-5))
