@@ -51,7 +51,7 @@
  * F16 KV: the node accumulates V in f32 (closer to the exact value than ggml-cpu's f16 accumulator, which is 4e-3 away);
  * a backend initialised with params containing "f16_acc=strict" (ggml_backend_dev_init(dev, params)), or with
  * GGML_HIP_MLA_F16_ACC=strict in the environment, replays the reference's accumulator instead (ggml-cpu.c:12066-12080).
- * BF16 KV: the decode kernel converts the cache tiles to f16 on the way (exact for magnitudes in [2^-14, 65504], which a
+ * BF16 KV, more than 32 attention rows per sequence: the decode kernel converts the cache tiles to f16 on the way (exact for magnitudes in [2^-14, 65504], which a
  * latent cache holds; see MLA_FLAG_BF16_DIRECT in mla_attn.h); params containing "bf16=direct", or GGML_HIP_MLA_BF16=direct
  * in the environment, keep the tiles in bf16 for caches with values outside that range.
  * and reports caps {async, host_buffer, events} (struct ggml_backend_dev_caps, ggml/include/ggml-backend.h:145-154).
