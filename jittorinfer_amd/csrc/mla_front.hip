@@ -162,42 +162,57 @@ __global__ void __launch_bounds__(256) mla_mul_mat_kernel(const MmP p) {
         }
 }
 
-// Few rows m (a decode step): nothing is shared between waves, so there is no staging and no barrier before the MFMAs.
-// A workgroup owns 32 outputs n and 32 rows m; its four waves take every fourth k-step of 16, load their weight and
-// activation fragments straight from global memory into the MFMA operand registers (up to 8 k-steps in flight per
-// wave), and the four partial accumulators meet in LDS.  The grid is (N / 32) x (M / 32) x batches workgroups, enough to
-// keep the weight stream of a 128-head layer in flight on every CU.
+// Few rows m (a decode step) and too few 128-wide tiles to fill the chip: a workgroup owns 32 outputs n and 32 rows m, and
+// both operands come through LDS.  Loading MFMA fragments straight from global memory fetches 16 bytes per lane from 32
+// different rows per instruction, and the texture addresser takes those one row at a time (that form ran the un-absorb
+// product of a 128-head layer at 32 tokens in 12.5 us, this one in 11.2); here the workgroup copies its 32 weight rows and
+// its 32 activation rows chunk by chunk (256 k) with loads that run along the rows (a wave covers two whole 512-byte
+// weight rows, or one 1 KB piece of an f32 activation row, per instruction), rounds the activations on the way, and the
+// four waves take every fourth k-step of 16 out of LDS; their partial accumulators meet in LDS.  The grid is
+// (N / 32) x (M / 32) x batches workgroups, enough to keep the weight stream of a 128-head layer in flight on every CU.
+constexpr int MS_KC = 256, MS_PITCH = MS_KC * 2 + 16;
 template <bool F16>
-__global__ void __launch_bounds__(256) mla_mul_mat_skinny_kernel(const MmP p) {
+__global__ void __launch_bounds__(256) mla_mul_mat_small_kernel(const MmP p) {
+    __shared__ __attribute__((aligned(16))) char ws[32 * MS_PITCH];
+    __shared__ __attribute__((aligned(16))) char xs[32 * MS_PITCH];
     __shared__ float red[4][16][64];
     const int     lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int64_t i2 = blockIdx.z % p.ne2, i3 = blockIdx.z / p.ne2;
     const int64_t n0 = (int64_t) blockIdx.x * 32, m0 = (int64_t) blockIdx.y * 32;
-    const char *  wrow = p.w + (i2 / p.r2) * p.w_nb2 + (i3 / p.r3) * p.w_nb3 + min(n0 + (lane & 31), p.N - 1) * p.w_nb1 + (lane >> 5) * 16;
-    const char *  xrow = p.x + i2 * p.x_nb2 + i3 * p.x_nb3 + min(m0 + (lane & 31), p.M - 1) * p.x_nb1 + (lane >> 5) * 32;
-    const int     nks = (int) (p.K / 16);
-    constexpr int U = 8;
+    const char *  W = p.w + (i2 / p.r2) * p.w_nb2 + (i3 / p.r3) * p.w_nb3;
+    const char *  X = p.x + i2 * p.x_nb2 + i3 * p.x_nb3;
     f32x16 acc;
 #pragma unroll
     for (int j = 0; j < 16; j++) acc[j] = 0.f;
-    for (int base = wave; base < nks; base += 4 * U) {
-        u32x4  wf[U];
-        float4 xa[U], xb[U];
+    for (int64_t k0 = 0; k0 < p.K; k0 += MS_KC) {
+        const int kc = (int) min((int64_t) MS_KC, p.K - k0), groups = kc / 8, units = 32 * groups;   // a unit: 8 values of one row
+        u32x4  wv[4];
+        float4 xa[4], xb[4];
 #pragma unroll
-        for (int u = 0; u < U; u++) {
-            const int ks = min(base + 4 * u, nks - 1);   // past the end: a valid address, the fragment is not used
-            wf[u] = *(const u32x4 *) (wrow + (int64_t) ks * 32);
-            xa[u] = *(const float4 *) (xrow + (int64_t) ks * 64);
-            xb[u] = *(const float4 *) (xrow + (int64_t) ks * 64 + 16);
+        for (int i = 0; i < 4; i++) {
+            const int u = min((int) threadIdx.x + 256 * i, units - 1), row = u / groups, c = u - row * groups;
+            wv[i] = *(const u32x4 *) (W + min(n0 + row, p.N - 1) * p.w_nb1 + (k0 + c * 8) * 2);
+            const char * xr = X + min(m0 + row, p.M - 1) * p.x_nb1 + (k0 + c * 8) * 4;
+            xa[i] = *(const float4 *) xr;
+            xb[i] = *(const float4 *) (xr + 16);
         }
+        if (k0) __syncthreads();   // every wave is done with the previous chunk
 #pragma unroll
-        for (int u = 0; u < U; u++)
-            if (base + 4 * u < nks) {
-                u32x4 af;
-                af[0] = pack2<F16>(xa[u].x, xa[u].y); af[1] = pack2<F16>(xa[u].z, xa[u].w);
-                af[2] = pack2<F16>(xb[u].x, xb[u].y); af[3] = pack2<F16>(xb[u].z, xb[u].w);
-                acc = mfma32<F16>(af, wf[u], acc);
+        for (int i = 0; i < 4; i++) {
+            const int u = (int) threadIdx.x + 256 * i;
+            if (u < units) {
+                const int row = u / groups, c = u - row * groups;
+                *(u32x4 *) (ws + row * MS_PITCH + c * 16) = wv[i];
+                *(u32x4 *) (xs + row * MS_PITCH + c * 16) = u32x4{ pack2<F16>(xa[i].x, xa[i].y), pack2<F16>(xa[i].z, xa[i].w),
+                                                                    pack2<F16>(xb[i].x, xb[i].y), pack2<F16>(xb[i].z, xb[i].w) };
             }
+        }
+        __syncthreads();
+        for (int ks = wave; ks < kc / 16; ks += 4) {
+            const int    off = (lane & 31) * MS_PITCH + ks * 32 + (lane >> 5) * 16;
+            const u32x4 af = *(const u32x4 *) (xs + off), wf = *(const u32x4 *) (ws + off);
+            acc = mfma32<F16>(af, wf, acc);
+        }
     }
 #pragma unroll
     for (int j = 0; j < 16; j++) red[wave][j][lane] = acc[j];
@@ -351,7 +366,7 @@ hipError_t launch_mm(const MmP & p, int64_t batches, hipStream_t st) {
     const unsigned gx = (unsigned) ((p.N + 127) / 128);
     if (p.M <= 64 && (int64_t) gx * ((p.M + 31) / 32) * batches < 512 && p.K >= 256) {
         // few rows and fewer than two workgroups per CU with 128-wide tiles: split n finer and K over the waves
-        hipLaunchKernelGGL((mla_mul_mat_skinny_kernel<F16>), dim3((unsigned) ((p.N + 31) / 32), (unsigned) ((p.M + 31) / 32), (unsigned) batches), dim3(256), 0, st, p);
+        hipLaunchKernelGGL((mla_mul_mat_small_kernel<F16>), dim3((unsigned) ((p.N + 31) / 32), (unsigned) ((p.M + 31) / 32), (unsigned) batches), dim3(256), 0, st, p);
     } else if (p.M <= 32) {
         hipLaunchKernelGGL((mla_mul_mat_kernel<F16, 1>), dim3(gx, (unsigned) ((p.M + 31) / 32), (unsigned) batches), dim3(256), 0, st, p);
     } else if (p.M <= 64) {
