@@ -172,3 +172,20 @@ def test_committed_wave_programs_are_what_the_generator_emits(flags, name):
     for m in re.finditer(r"\bs(\d+)\b|\bs\[(\d+):(\d+)\]", got):      # scalar registers: inside the clobbered range s40..s83
         lo, hi = (int(m.group(1)),) * 2 if m.group(1) else (int(m.group(2)), int(m.group(3)))
         assert 40 <= lo and hi <= 83, "%s uses %s" % (name, m.group(0))
+
+
+def test_python_constants_match_the_header():
+    """The ctypes mirror restates the #defines of include/mla_attn.h (types, flags, errors): each one is compared with the header."""
+    import re
+    import jittorinfer_amd.capi as capi
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    with open(os.path.join(root, "include", "mla_attn.h")) as f:
+        text = f.read()
+    defs = {m.group(1): m.group(2) for m in re.finditer(r"#define\s+(MLA_(?:TYPE|FLAG|ERR)_\w+)\s+\(?(-?\d+)u?\)?", text)}
+    assert {"MLA_FLAG_F16_ACC_STRICT", "MLA_FLAG_UNIFORM_SPLITS", "MLA_FLAG_BF16_DIRECT", "MLA_TYPE_BF16", "MLA_TYPE_Q8_0"} <= set(defs)
+    checked = 0
+    for name, value in defs.items():
+        if hasattr(capi, name):
+            assert getattr(capi, name) == int(value), name
+            checked += 1
+    assert checked >= 6
