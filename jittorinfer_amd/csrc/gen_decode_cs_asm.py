@@ -1,0 +1,887 @@
+#!/usr/bin/env python3
+"""Generates mla_decode_cs_*.inc: the gfx950 instruction streams of the pipelined MLA decode kernel in its
+"column-split" form (one inline-asm block each inside mla_decode_kernel.hip).
+Usage: python gen_decode_cs_asm.py [--f16] > mla_decode_cs_[bf16|f16].inc
+
+Work of one wave w of a 4-wave workgroup (128 attention rows x one KV split), per 32-token tile `it`:
+    part 1   S = K[it+1].Q^T for the wave's own 32 rows (36 MFMA, Q resident in 144 VGPRs, K fragments from LDS);
+             in their shadow: the eight V^T fragments of tile `it` for the wave's own 128 output columns (transposing LDS
+             reads), bf16 fragments converted to f16 in registers, and the LDS-DMA loads of tile it+3
+    part 2   O^T[128 columns x 128 rows] += V[it]^T.P[it]^T (32 MFMA; the P^T fragments of all four waves come out of LDS),
+             with softmax(S[it+1]) -> P[it+1] in their shadow
+    end      barrier, P[it+1] -> LDS, barrier (tile it+2 has landed for every wave; P[it+1] is visible)
+A wave thus owns 128 columns of all 128 rows of O (16 accumulator blocks of 32 x 32 in 256 AGPRs): a V^T fragment feeds
+four MFMAs, so the transposing reads (the slow kind) drop to a quarter, and with 8 fragments per wave and tile the bf16 -> f16
+conversion fits in registers: no pass over the tile in LDS, no tile buffer held for it, two tiles of loads in flight.
+bf16 K is multiplied as bf16 (exact products either way); P and V meet as f16, which keeps 11 bits of P.
+"""
+import sys
+
+ARGS = sys.argv[1:]
+F16KV = "--f16" in ARGS                      # f16 KV rows: f16 MFMA for K.Q^T, V^T fragments used as they are
+CLK = "--clk" in ARGS                        # timing builds: s_memtime stamps left in LDS at the end
+NO_STORE = "--no-store" in ARGS              # timing experiments only (wrong results)
+MF_QK = "v_mfma_f32_32x32x16_f16" if F16KV else "v_mfma_f32_32x32x16_bf16"
+MF_PV = "v_mfma_f32_32x32x16_f16"
+
+
+def _opt(name, default):
+    return int(ARGS[ARGS.index(name) + 1]) if name in ARGS else default
+
+
+CONV_P1 = _opt("--conv-p1", 5)               # V^T fragments converted in part 1; the rest in the first half of part 2
+
+PITCH = 1168
+TILE_BYTES = 32 * PITCH
+NBUF = 4
+PBUF = NBUF * TILE_BYTES                     # P^T exchange: [row block hb][k-step kk][lane][16 bytes] = 8 KB
+HOFF = PBUF                                  # hand-off records of the C++ prologue (32 bytes per thread): read before P is first written
+AOFF = PBUF + 8192                           # rescale factors: [lane][hb] f32 (64 x 16 bytes; lanes 32.. hold copies)
+FOFF = AOFF + 1024                           # one word per wave: non-zero when its rows' running maxima moved
+CPR = 73                                     # 16-byte chunks per padded row
+WAVE_CHUNKS = 8 * CPR                        # each wave moves rows 8w .. 8w+7 of a tile
+DMA_PER_TILE = 10
+KRING, PRING = 5, 4
+
+# ---- VGPR map (v252..v255 are left to the compiler: the clobber list of the asm block ends at v251)
+Q0 = 0
+S = 144                 # scores of one tile; its P^T operands (f16 pairs) are built in place
+VF = 160                # the eight V^T fragments of a tile, fragment f = 4 kk + cb in VF + 4 f
+PR = 192                # ring of P^T fragments, fragment f = 4 kk + hb in slot f % 4
+KF = 208                # ring of K fragments
+T = list(range(228, 236))
+KADDR_LANE, VADDR_LANE, MRUN, LRUN, KADDR, VADDR, PAGES = 236, 237, 238, 239, 240, 241, 242
+PT = [243, 244, 245, 246, 247]   # per-lane byte offsets of the 10 LDS-DMA slots, two 16-bit values per register
+PADDR = 248             # PBUF + lane * 16
+X0 = 249
+DT = [250, 251]         # address temporaries of the LDS-DMA slots; conversion temporaries in part 2
+X1, X2 = 250, 251       # prologue / epilogue temporaries
+NEGM, ALPHA, TMAX = T[5], T[6], T[7]   # live inside the softmax only
+LANE = T[7]             # prologue only
+N_VGPR = 252
+# ---- SGPR map (all inside the clobbered range s40..s99)
+KV, BT, KVB, KVE, CL2, NPP, NB1, FLG = 40, 42, 44, 45, 46, 47, 48, 49
+NT, IT, OFF0, OFF1, OFF2, OFF3, WAVE, TMP = 50, 51, 52, 53, 54, 55, 56, 57
+TB, NVM1, VMW, EXS = 58, 60, 61, 62
+S0, S1, S2, S3, DMAB, NVAL, THR, PG0 = 64, 65, 66, 67, 68, 69, 70, 71
+RSC, ONES, OSTR, QP, OB, MLB, RSTR, NRV = 72, 74, 75, 76, 78, 80, 82, 83
+W4, WOFS, FADR, PGZ, SPITCH, SCLS = 84, 85, 86, 87, 88, 89
+VM = [90, 92, 94, 96]   # epilogue: lanes whose row of row block hb exists
+SB = 98                 # epilogue: running store base
+TAU_BITS = 0x41000000   # 8.0f
+
+out = []
+uid = [0]
+
+
+def e(s):
+    out.append(s)
+
+
+def label(prefix):
+    uid[0] += 1
+    return "L%s_%d_%%=" % (prefix, uid[0])
+
+
+def v(i, n=1):
+    assert 0 <= i and i + n - 1 < N_VGPR, (i, n)
+    return "v%d" % i if n == 1 else "v[%d:%d]" % (i, i + n - 1)
+
+
+def a(i, n=1):
+    return "a%d" % i if n == 1 else "a[%d:%d]" % (i, i + n - 1)
+
+
+def s(i, n=1):
+    return "s%d" % i if n == 1 else "s[%d:%d]" % (i, i + n - 1)
+
+
+class Lds:
+    """Tracks outstanding LDS accesses so that each use waits for exactly the accesses that precede it."""
+
+    def __init__(self):
+        self.pending = []
+        self.issued = set()      # since the last reset(): a use may only wait for an access that was issued
+
+    def op(self, line, tag):
+        e(line)
+        self.pending.append(tag)
+        self.issued.add(tag)
+
+    def reset(self, pending):
+        self.pending = list(pending)
+        self.issued = set(pending)
+
+    def need(self, tag):
+        assert tag in self.issued, tag
+        if tag in self.pending:
+            after = min(len(self.pending) - 1 - self.pending.index(tag), 15)   # the counter field has 4 bits
+            e("s_waitcnt lgkmcnt(%d)" % after)
+            self.pending = self.pending[len(self.pending) - after:] if after else []
+
+    def drain(self):
+        if self.pending:
+            e("s_waitcnt lgkmcnt(0)")
+            self.pending = []
+
+
+lds = Lds()
+
+
+def emit_item(x):
+    """A shadow item is a line, None, or a callable that emits lines (LDS accesses go through the tracker)."""
+    if x is None:
+        return
+    if callable(x):
+        x()
+    else:
+        e(x)
+
+
+def spread(items, first, last):
+    """Assigns the items of one stream to the MFMA slots first .. last, evenly and in order: [(slot, item)]."""
+    n = len(items)
+    span = last - first + 1
+    return [(first + (k * span) // n, it) for k, it in enumerate(items)]
+
+
+def run_slots(slots, first_index, streams, events=None):
+    """Emits the MFMA slots; behind slot i the items the streams assign to slot first_index + i, and ahead of it events[i]."""
+    by_slot = {}
+    for st in streams:
+        for idx, it in st:
+            by_slot.setdefault(idx, []).append(it)
+    for i, slot in enumerate(slots):
+        for ev in (events or {}).get(first_index + i, []):
+            emit_item(ev)
+        slot()
+        for it in by_slot.pop(first_index + i, []):
+            emit_item(it)
+    assert all(not (first_index <= k < first_index + len(slots)) for k in by_slot), sorted(by_slot)
+    return by_slot
+
+
+# ---------------------------------------------------------------------------------------------------------------
+def tile_base_lines(tile_sreg, first_page_scalar=False):
+    """Scalar lines: s[TB:TB+1] = address of the first row of tile s[tile_sreg]; s[NVM1] = its valid rows - 1.
+    first_page_scalar: a tile inside the split's first page takes the page id from s[PGZ] instead of the lane of PAGES
+    (the prologue's tiles, issued while the vector load of the page ids may still be in flight)."""
+    L = []
+    L.append("s_lshl_b32 %s, %s, 5" % (s(S0), s(tile_sreg)))
+    L.append("s_add_u32 %s, %s, %s" % (s(S0), s(S0), s(KVB)))                      # S0 = first token of the tile
+    L.append("s_sub_u32 %s, %s, %s" % (s(S1), s(KVE), s(S0)))
+    L.append("s_min_u32 %s, %s, 32" % (s(S1), s(S1)))
+    L.append("s_sub_u32 %s, %s, 1" % (s(NVM1), s(S1)))
+    L.append("s_lshr_b32 %s, %s, 7" % (s(S1), s(S0)))                             # logical page
+    L.append("s_sub_u32 %s, %s, %s" % (s(S1), s(S1), s(PG0)))                     # index into the preloaded lanes
+    L.append("v_readlane_b32 %s, %s, %s" % (s(S2), v(PAGES), s(S1)))
+    if first_page_scalar:
+        L.append("s_cmp_eq_u32 %s, 0" % s(S1))
+        L.append("s_cselect_b32 %s, %s, %s" % (s(S2), s(PGZ), s(S2)))
+    L.append("s_lshl_b32 %s, %s, 7" % (s(S2), s(S2)))
+    L.append("s_and_b32 %s, %s, 127" % (s(S3), s(S0)))
+    L.append("s_add_u32 %s, %s, %s" % (s(S2), s(S2), s(S3)))                      # pool row when paged
+    L.append("s_cmp_eq_u64 %s, 0" % s(BT, 2))
+    L.append("s_cselect_b32 %s, %s, %s" % (s(S0), s(S0), s(S2)))                  # no table: the logical row itself
+    L.append("s_mul_hi_u32 %s, %s, %s" % (s(S1), s(S0), s(NB1)))
+    L.append("s_mul_i32 %s, %s, %s" % (s(S0), s(S0), s(NB1)))
+    L.append("s_add_u32 %s, %s, %s" % (s(TB), s(KV), s(S0)))
+    L.append("s_addc_u32 %s, %s, %s" % (s(TB + 1), s(KV + 1), s(S1)))
+    return L
+
+
+def dma_table_lines(lane, tmp):
+    """Once per kernel: where the 16 bytes that lane l of LDS-DMA slot j copies sit inside a tile.  The LDS side of a slot
+    is 64 consecutive 16-byte chunks of the padded tile (73 chunks per row, the 73rd is padding); the global side is
+    row * nb1 + min(column chunk, 71) * 16 -- at most 31 * 1152 + 1136, so two offsets share a register."""
+    L = []
+    row, col, x0, x1, x2 = tmp
+    L.append("v_mov_b32 %s, %s" % (v(col), v(lane)))
+    L.append("s_lshl_b32 %s, %s, 3" % (s(S2), s(WAVE)))
+    L.append("v_mov_b32 %s, %s" % (v(row), s(S2)))                     # a wave copies rows 8w .. 8w+7
+    for j in range(10):
+        L.append("v_min_u32 %s, 71, %s" % (v(x1), v(col)))
+        L.append("v_lshlrev_b32 %s, 4, %s" % (v(x1), v(x1)))
+        L.append("v_mad_u32_u24 %s, %s, %s, %s" % (v(x0), v(row), s(NB1), v(x1)))
+        if j % 2 == 0:
+            L.append("v_mov_b32 %s, %s" % (v(PT[j // 2]), v(x0)))
+        else:
+            L.append("v_lshl_or_b32 %s, %s, 16, %s" % (v(PT[j // 2]), v(x0), v(PT[j // 2])))
+        if j < 9:
+            L.append("v_add_u32 %s, 64, %s" % (v(col), v(col)))
+            L.append("v_cmp_le_u32 vcc, %d, %s" % (CPR, v(col)))
+            L.append("v_subrev_u32 %s, %d, %s" % (v(x2), CPR, v(col)))
+            L.append("v_add_u32 %s, 1, %s" % (v(x0), v(row)))
+            L.append("s_nop 0")
+            L.append("v_cndmask_b32 %s, %s, %s, vcc" % (v(col), v(col), v(x2)))
+            L.append("v_cndmask_b32 %s, %s, %s, vcc" % (v(row), v(row), v(x0)))
+    return L
+
+
+def dma_tile_lines(tile_sreg, off_sreg, first_page_scalar=False):
+    """Instruction list (to be interleaved) that issues the LDS-DMA loads of tile s[tile_sreg] into the buffer at LDS
+    offset s[off_sreg].  Rows past the end of the sequence are replaced by the last 16 bytes of the last valid row (any
+    finite data will do: their probabilities are exactly 0): one v_min against that offset."""
+    L = tile_base_lines(tile_sreg, first_page_scalar)
+    L.append("s_mul_i32 %s, %s, %s" % (s(S3), s(NVM1), s(NB1)))
+    L.append("s_add_u32 %s, %s, %d" % (s(S3), s(S3), 71 * 16))
+    L.append("s_mul_i32 %s, %s, %d" % (s(DMAB), s(WAVE), WAVE_CHUNKS * 16))
+    L.append("s_add_u32 %s, %s, %s" % (s(DMAB), s(DMAB), s(off_sreg)))
+    for j in range(10):
+        t = DT[j & 1]
+        if j % 2 == 0:
+            L.append("v_and_b32 %s, 0xffff, %s" % (v(t), v(PT[j // 2])))
+        else:
+            L.append("v_lshrrev_b32 %s, 16, %s" % (v(t), v(PT[j // 2])))
+        L.append("v_min_u32 %s, %s, %s" % (v(t), s(S3), v(t)))
+        if j == 9:
+            # 8 chunks left per wave: lanes 0..7 only.  One atomic group: nothing may be scheduled inside the exec window.
+            L.append("\\n\\t".join(["s_add_u32 m0, %s, %d" % (s(DMAB), j * 1024),
+                                    "s_mov_b64 %s, exec" % s(EXS, 2),
+                                    "s_mov_b64 exec, 0xff",
+                                    "global_load_lds_dwordx4 %s, %s" % (v(t), s(TB, 2)),
+                                    "s_mov_b64 exec, %s" % s(EXS, 2)]))
+        else:
+            L.append("\\n\\t".join(["s_add_u32 m0, %s, %d" % (s(DMAB), j * 1024),
+                                    "s_nop 0",
+                                    "global_load_lds_dwordx4 %s, %s" % (v(t), s(TB, 2))]))
+    return L
+
+
+# ---------------------------------------------------------------------------------------------------------------
+def k_read(p):
+    lds.op("ds_read_b128 %s, %s offset:%d" % (v(KF + 4 * (p % KRING), 4), v(KADDR), p * 32), ("k", p))
+
+
+def k_warm():
+    for p in range(KRING - 1):
+        k_read(p)
+
+
+def qk_slots():
+    """36 MFMA slots of S = K.Q^T; K fragments come through a ring (k_warm first), one wait per two fragments."""
+    depth = KRING - 1
+
+    def mk(ks):
+        def slot():
+            lds.need(("k", ks + 1) if ks % 2 == 0 and ("k", ks + 1) in lds.pending else ("k", ks))   # fragments return in order
+            c = "0" if ks == 0 else v(S, 16)
+            e("%s %s, %s, %s, %s" % (MF_QK, v(S, 16), v(KF + 4 * (ks % KRING), 4), v(Q0 + 4 * ks, 4), c))
+            if ks + depth < 36:
+                k_read(ks + depth)
+        return slot
+    return [mk(ks) for ks in range(36)]
+
+
+def v_read_items(f):
+    """V^T fragment f = (kk, cb) of the tile at v[VADDR] -> VF + 4 f: two transposing reads."""
+    kk, cb = f // 4, f % 4
+    base = 16 * kk * PITCH + cb * 64
+    r = VF + 4 * f
+    return [lambda: lds.op("ds_read_b64_tr_b16 %s, %s offset:%d" % (v(r, 2), v(VADDR), base), ("v", f, 0)),
+            lambda: lds.op("ds_read_b64_tr_b16 %s, %s offset:%d" % (v(r + 2, 2), v(VADDR), base + 8 * PITCH), ("v", f, 1))]
+
+
+def v_conv_items(f, tmp):
+    """bf16 -> f16 of fragment f in place: per 32-bit word both halves widened to f32, then v_cvt_pkrtz_f16_f32 (exact inside
+    the f16 range; round-toward-zero turns larger magnitudes into 65504 instead of infinity)."""
+    if F16KV:
+        return []
+    r = VF + 4 * f
+    c0, c1 = tmp
+
+    def first():
+        lds.need(("v", f, 1))
+        e("v_lshlrev_b32 %s, 16, %s" % (v(c0), v(r)))
+    I = [first]
+    for j in range(4):
+        if j:
+            I.append("v_lshlrev_b32 %s, 16, %s" % (v(c0), v(r + j)))
+        I.append("v_and_b32 %s, 0xffff0000, %s" % (v(c1), v(r + j)))
+        I.append("v_cvt_pkrtz_f16_f32 %s, %s, %s" % (v(r + j), v(c0), v(c1)))
+    return I
+
+
+def p_read(f):
+    kk, hb = f // 4, f % 4
+    lds.op("ds_read_b128 %s, %s offset:%d" % (v(PR + 4 * (f % PRING), 4), v(PADDR), (hb * 2 + kk) * 1024), ("p", f))
+
+
+def pv_slots():
+    """32 MFMA slots of O^T += V^T.P^T in the order [kk][hb][cb]: a P^T fragment serves four consecutive MFMAs, and
+    MFMAs on the same accumulator block are 16 slots apart."""
+    def mk(n):
+        kk, hb, cb = n // 16, (n // 4) % 4, n % 4
+        f = 4 * kk + hb
+        acc = 16 * (4 * cb + hb)
+
+        def slot():
+            if cb == 0:
+                lds.need(("p", f))
+            lds.need(("v", 4 * kk + cb, 1))          # f16 KV: the fragment is used as read; bf16: converted long before (no-op)
+            e("%s %s, %s, %s, %s" % (MF_PV, a(acc, 16), v(VF + 4 * (4 * kk + cb), 4), v(PR + 4 * (f % PRING), 4), a(acc, 16)))
+            if cb == 0 and f + PRING - 1 < 8:
+                p_read(f + PRING - 1)                # into the slot of fragment f - 1 (for f = 0: the tile before's last), whose last MFMA has been issued
+        return slot
+    return [mk(n) for n in range(32)]
+
+
+def softmax_lines(first_tile=False):
+    """Softmax of the scores in S as one list of VALU lines (no branches): tile max -> lazy max update (a new max only where
+    it grew by more than TAU) -> ALPHA (rescale factor of O and l, 1 where the max stayed) and RSC (non-zero when some lane
+    changed its max) -> p = 2^(s*c - m) -> P^T operands (f16 pairs) in S+0..3 (k-step 0) and S+8..11 (k-step 1) ->
+    l += sum of the rounded p (the output stays an exact weighted mean of V rows)."""
+    L = []
+    m = [T[0], T[1], T[2], T[3], T[4]]
+    L.append("v_max3_f32 %s, %s, %s, %s" % (v(m[0]), v(S + 0), v(S + 1), v(S + 2)))
+    L.append("v_max3_f32 %s, %s, %s, %s" % (v(m[1]), v(S + 3), v(S + 4), v(S + 5)))
+    L.append("v_max3_f32 %s, %s, %s, %s" % (v(m[2]), v(S + 6), v(S + 7), v(S + 8)))
+    L.append("v_max3_f32 %s, %s, %s, %s" % (v(m[3]), v(S + 9), v(S + 10), v(S + 11)))
+    L.append("v_max3_f32 %s, %s, %s, %s" % (v(m[4]), v(S + 12), v(S + 13), v(S + 14)))
+    L.append("v_max3_f32 %s, %s, %s, %s" % (v(m[0]), v(m[0]), v(m[1]), v(S + 15)))
+    L.append("v_max3_f32 %s, %s, %s, %s" % (v(m[0]), v(m[0]), v(m[2]), v(m[3])))
+    L.append("v_max_f32 %s, %s, %s" % (v(m[0]), v(m[0]), v(m[4])))
+    L.append("v_mov_b32 %s, %s" % (v(m[1]), v(m[0])))
+    L.append("s_nop 1")
+    L.append("v_permlane32_swap_b32 %s, %s" % (v(m[0]), v(m[1])))
+    L.append("s_nop 1")
+    L.append("v_max_f32 %s, %s, %s" % (v(TMAX), v(m[0]), v(m[1])))
+    L.append("v_mul_f32 %s, %s, %s" % (v(TMAX), s(CL2), v(TMAX)))           # log2 units (the factor is > 0)
+    L.append("v_add_f32 %s, %s, %s" % (v(m[2]), s(THR), v(MRUN)))           # m_run + TAU  (-inf stays -inf)
+    L.append("v_sub_f32 %s, %s, %s" % (v(m[3]), v(MRUN), v(TMAX)))          # m_run - tmax
+    L.append("v_exp_f32 %s, %s" % (v(m[3]), v(m[3])))                       # 2^(m_run - tmax); 0 when m_run = -inf
+    L.append("v_cmp_gt_f32 vcc, %s, %s" % (v(TMAX), v(m[2])))               # this lane's max moves
+    L.append("s_mov_b64 %s, vcc" % s(RSC, 2))
+    L.append("s_nop 1")
+    L.append("v_cndmask_b32 %s, 1.0, %s, vcc" % (v(ALPHA), v(m[3])))
+    L.append("v_cndmask_b32 %s, %s, %s, vcc" % (v(MRUN), v(MRUN), v(TMAX)))
+    L.append("v_mul_f32 %s, %s, %s" % (v(LRUN), v(LRUN), v(ALPHA)))
+    # -m (0 when still -inf)
+    L.append("v_mov_b32 %s, 0xff800000" % v(m[0]))
+    L.append("v_cmp_eq_f32 vcc, %s, %s" % (v(MRUN), v(m[0])))
+    L.append("v_sub_f32 %s, 0, %s" % (v(NEGM), v(MRUN)))
+    L.append("s_nop 0")
+    L.append("v_cndmask_b32 %s, %s, 0, vcc" % (v(NEGM), v(NEGM)))
+    for k in range(16):
+        L.append("v_fma_f32 %s, %s, %s, %s" % (v(S + k), v(S + k), s(CL2), v(NEGM)))
+    for k in range(16):
+        L.append("v_exp_f32 %s, %s" % (v(S + k), v(S + k)))
+    # P^T operands in place.  k-step kk owns registers b = S+8kk .. +7, holding p of tokens
+    # (8(2kk)+4g+0..3, 8(2kk+1)+4g+0..3); pairs (b0,b1) (b2,b3) (b4,b5) (b6,b7) -> b0..b3.
+    for kk in range(2):
+        b = S + 8 * kk
+        for j in range(4):
+            L.append("v_cvt_pk_f16_f32 %s, %s, %s" % (v(b + j), v(b + 2 * j), v(b + 2 * j + 1)))
+        for j in range(4):
+            acc = T[j & 1]
+            c = "0" if kk == 0 and j < 2 else v(acc)
+            L.append("v_dot2_f32_f16 %s, %s, %s, %s" % (v(acc), v(b + j), s(ONES), c))
+    L.append("s_nop 2")   # a dot product's result may be read by another kind of VALU instruction three wait states later
+    L.append("v_add_f32 %s, %s, %s" % (v(T[0]), v(T[0]), v(T[1])))
+    L.append("v_add_f32 %s, %s, %s" % (v(LRUN), v(LRUN), v(T[0])))
+    if first_tile:
+        L.append("s_mov_b64 %s, 0" % s(RSC, 2))     # the accumulators are still zero: nothing to rescale
+    return L
+
+
+def p_write_items():
+    """P^T operands of the wave's 32 rows, the rescale factors of those rows and the wave's flag word -> LDS."""
+    I = []
+    I.append("v_add_u32 %s, %s, %s" % (v(T[2]), s(WOFS), v(PADDR)))
+    I.append(lambda: lds.op("ds_write_b128 %s, %s" % (v(T[2]), v(S, 4)), ("w", 0)))
+    I.append(lambda: lds.op("ds_write_b128 %s, %s offset:1024" % (v(T[2]), v(S + 8, 4)), ("w", 1)))
+    I.append("v_add_u32 %s, %s, %s" % (v(T[3]), s(W4), v(PADDR)))
+    I.append(lambda: lds.op("ds_write_b32 %s, %s offset:%d" % (v(T[3]), v(ALPHA), AOFF - PBUF), ("w", 2)))
+    I.append("v_mov_b32 %s, %s" % (v(T[0]), s(RSC)))
+    I.append("v_or_b32 %s, %s, %s" % (v(T[0]), s(RSC + 1), v(T[0])))
+    I.append("v_mov_b32 %s, %s" % (v(T[1]), s(FADR)))
+    I.append(lambda: lds.op("ds_write_b32 %s, %s" % (v(T[1]), v(T[0])), ("w", 3)))
+    return I
+
+
+def mask_tail():
+    """Last tile of a sequence only: tokens >= n_valid get score -inf.  element k is token 8*(k/4) + 4g + k%4."""
+    lab = label("full")
+    e("s_cmp_ge_u32 %s, 32" % s(NVAL))
+    e("s_cbranch_scc1 %s" % lab)
+    e("v_mov_b32 %s, 0xff800000" % v(T[0]))
+    e("v_mbcnt_lo_u32_b32 %s, -1, 0" % v(T[2]))
+    e("v_mbcnt_hi_u32_b32 %s, -1, %s" % (v(T[2]), v(T[2])))
+    e("v_lshrrev_b32 %s, 5, %s" % (v(T[2]), v(T[2])))
+    e("v_lshlrev_b32 %s, 2, %s" % (v(T[2]), v(T[2])))                       # 4g
+    for k in range(16):
+        e("v_add_u32 %s, %d, %s" % (v(T[1]), 8 * (k // 4) + (k % 4), v(T[2])))
+        e("v_cmp_gt_u32 vcc, %s, %s" % (s(NVAL), v(T[1])))                  # valid if n_valid > token
+        e("s_nop 1")
+        e("v_cndmask_b32 %s, %s, %s, vcc" % (v(S + k), v(T[0]), v(S + k)))
+    e("%s:" % lab)
+
+
+def canon_tags():
+    """LDS reads in flight at the top of every iteration, in issue order (see handover)."""
+    return [("k", p) for p in range(KRING - 1)] + [("p", 0), ("p", 1), ("p", 2)]
+
+
+def handover(k_off, tail, resc):
+    """Behind the barrier that ends a tile: the flag words of the four waves, the first K fragments of the next K.Q^T (tile
+    buffer at s[k_off]) and the first P^T fragments of the tile whose P.V comes next, around the last two P.V MFMAs of the
+    tile that ends (they still use ring slot 3, which fragment 3 takes afterwards); then the accumulators take the new row
+    maxima if some wave's flag is up (out of line, rare)."""
+    e("v_mov_b32 %s, 0x%x" % (v(T[4]), FOFF))
+    lds.op("ds_read_b128 %s, %s" % (v(T[0], 4), v(T[4])), ("f",))
+    e("v_add_u32 %s, %s, %s" % (v(KADDR), s(k_off), v(KADDR_LANE)))
+    k_warm()
+    p_read(0)
+    p_read(1)
+    p_read(2)
+    for sl in tail:
+        sl()
+    lds.need(("f",))
+    e("v_or3_b32 %s, %s, %s, %s" % (v(T[0]), v(T[0]), v(T[1]), v(T[2])))
+    e("v_or_b32 %s, %s, %s" % (v(T[0]), v(T[0]), v(T[3])))
+    e("v_cmp_ne_u32 vcc, 0, %s" % v(T[0]))
+    lab_resc, lab_back = label("resc"), label("back")
+    e("s_cmp_lg_u64 vcc, 0")
+    e("s_cbranch_scc1 %s" % lab_resc)
+    e("%s:" % lab_back)
+    resc.append((lab_resc, lab_back))
+    assert lds.pending == canon_tags(), (lds.pending, canon_tags())
+
+
+def rescale_block(ret_label):
+    """Rare path, entered when no MFMA is left to issue on the old maxima: acc[cb][hb] *= alpha[hb] (per lane = per row)."""
+    e("s_nop 7")
+    e("s_nop 7")
+    e("s_nop 3")
+    e("ds_read_b128 %s, %s offset:%d" % (v(T[4], 4), v(PADDR), AOFF - PBUF))
+    e("s_waitcnt lgkmcnt(0)")
+    for cb in range(4):
+        for hb in range(4):
+            base = 16 * (4 * cb + hb)
+            for i in range(0, 16, 4):
+                for j in range(4):
+                    e("v_accvgpr_read_b32 %s, %s" % (v(T[j]), a(base + i + j)))
+                for j in range(4):
+                    e("v_mul_f32 %s, %s, %s" % (v(T[j]), v(T[j]), v(T[4 + hb])))
+                for j in range(4):
+                    e("v_accvgpr_write_b32 %s, %s" % (a(base + i + j), v(T[j])))
+    e("s_nop 7")
+    e("s_nop 7")
+    e("s_branch %s" % ret_label)
+
+
+STAMPS = []
+
+
+def stamp(name):
+    """--clk builds: shader-clock time stamp into LDS (FOFF + 64 + 8 * index + 256 * wave), by lane 0."""
+    if not CLK:
+        return
+    k = len(STAMPS)
+    STAMPS.append(name)
+    e("s_memtime %s" % s(S0, 2))
+    e("s_waitcnt lgkmcnt(0)")
+    e("v_mov_b32 %s, %s" % (v(X0), s(S0)))
+    e("s_mul_i32 %s, %s, 256" % (s(S1), s(WAVE)))
+    e("s_add_u32 %s, %s, 0x%x" % (s(S1), s(S1), FOFF + 64 + 8 * k))
+    e("v_mov_b32 %s, %s" % (v(X1), s(S1)))
+    e("ds_write_b32 %s, %s" % (v(X1), v(X0)))
+    e("s_waitcnt lgkmcnt(0)")
+
+
+def iteration(resc):
+    """Tile IT: see the module docstring."""
+    e("; ---- iteration")
+    e("s_add_u32 %s, %s, 1" % (s(S0), s(IT)))
+    e("s_lshl_b32 %s, %s, 5" % (s(S0), s(S0)))
+    e("s_add_u32 %s, %s, %s" % (s(S0), s(S0), s(KVB)))
+    e("s_sub_u32 %s, %s, %s" % (s(NVAL), s(KVE), s(S0)))
+    e("s_min_u32 %s, %s, 32" % (s(NVAL), s(NVAL)))                    # valid tokens of tile IT+1
+    e("s_mov_b32 %s, 0" % s(VMW))
+    lab_last, lab_nodma, lab_p2, lab_end = label("last"), label("nodma"), label("p2"), label("iend")
+    e("v_add_u32 %s, %s, %s" % (v(VADDR), s(OFF0), v(VADDR_LANE)))
+    e("s_add_u32 %s, %s, 1" % (s(TMP), s(IT)))
+    e("s_cmp_ge_u32 %s, %s" % (s(TMP), s(NT)))
+    e("s_cbranch_scc1 %s" % lab_last)
+    e("s_add_u32 %s, %s, 3" % (s(TMP), s(IT)))
+    e("s_cmp_ge_u32 %s, %s" % (s(TMP), s(NT)))
+    e("s_cbranch_scc1 %s" % lab_nodma)
+
+    def v_stream(n_conv, tmp):
+        """Part 1: reads of all eight V^T fragments of tile IT (two fragments ahead of their conversion) and conversion of
+        the first n_conv, as one ordered stream: the conversions share two temporaries."""
+        items = v_read_items(0) + v_read_items(1)
+        for f in range(8):
+            if f < n_conv:
+                items += v_conv_items(f, tmp)
+            if f + 2 < 8:
+                items += v_read_items(f + 2)
+        return spread(items, 0, 35)
+
+    def part1(dma):
+        lds.reset(canon_tags())
+        run_slots(qk_slots(), 0, [spread(dma, 0, 35), v_stream(CONV_P1, (T[0], T[1]))])
+
+    # ---- part 1 with the LDS-DMA loads of tile IT+3
+    e("s_mov_b32 %s, 1" % s(VMW))
+    dma = dma_tile_lines(TMP, OFF3)
+    part1(dma)
+    state_a = list(lds.pending)
+    e("s_branch %s" % lab_p2)
+    e("%s:" % lab_nodma)
+    part1([None] * len(dma))
+    assert lds.pending == state_a, (lds.pending, state_a)
+    # ---- part 2: P.V of tile IT, softmax of tile IT+1 in its shadow
+    e("%s:" % lab_p2)
+    pv = pv_slots()
+    conv2 = []
+    for f in range(CONV_P1, 8):
+        conv2 += v_conv_items(f, (DT[0], DT[1]))
+    conv2 = spread(conv2, 37, 48) if conv2 else []      # one ordered stream (shared temporaries), done before k-step 1 starts at slot 52
+
+    def qk_done():
+        e("s_nop 7")                    # the last K.Q^T MFMA has written S (two P.V MFMAs and these wait states behind it)
+        e("s_nop 1")
+        mask_tail()
+    sm = softmax_lines()
+    streams = [conv2, spread(sm, 38, 60)]
+    left = run_slots(pv[:26], 36, streams, {38: [qk_done]})
+    assert not left, left
+    # every P^T fragment of tile IT is in registers (or on its way: waited for here) before any wave overwrites P
+    lds.drain()
+    e("s_barrier")
+    for it_ in p_write_items():
+        emit_item(it_)
+    for sl in pv[26:30]:
+        sl()
+    lds.drain()
+    # the loads of tile IT+2 have landed (those of tile IT+3, issued in this iteration, may still be in flight: loads
+    # complete in order); every wave is done with the buffers of tiles IT (V) and IT+1 (K), and P[IT+1] is written
+    lab_w0, lab_wd = label("w0"), label("wd")
+    e("s_cmp_eq_u32 %s, 0" % s(VMW))
+    e("s_cbranch_scc1 %s" % lab_w0)
+    e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
+    e("s_branch %s" % lab_wd)
+    e("%s:" % lab_w0)
+    e("s_waitcnt vmcnt(0)")
+    e("%s:" % lab_wd)
+    e("s_barrier")
+    handover(OFF2, pv[30:], resc)
+    e("s_branch %s" % lab_end)
+    # ---- last tile: P.V only
+    e("%s:" % lab_last)
+    lds.reset(canon_tags())
+    for f in range(8):
+        for it_ in v_read_items(f):
+            emit_item(it_)
+    for f in range(8):
+        for it_ in v_conv_items(f, (T[0], T[1])):
+            emit_item(it_)
+    for sl in pv_slots():
+        sl()
+    lds.drain()
+    e("%s:" % lab_end)
+    e("s_mov_b32 %s, %s" % (s(TMP), s(OFF0)))
+    e("s_mov_b32 %s, %s" % (s(OFF0), s(OFF1)))
+    e("s_mov_b32 %s, %s" % (s(OFF1), s(OFF2)))
+    e("s_mov_b32 %s, %s" % (s(OFF2), s(OFF3)))
+    e("s_mov_b32 %s, %s" % (s(OFF3), s(TMP)))
+    e("s_add_u32 %s, %s, 1" % (s(IT), s(IT)))
+
+
+def main():
+    # ------------------------------------------------------------------ entry: inputs -> fixed registers
+    e("s_mov_b64 %s, %%[kv]" % s(KV, 2))
+    e("s_mov_b64 %s, %%[bt]" % s(BT, 2))
+    e("s_mov_b32 %s, %%[kvb]" % s(KVB))
+    e("s_mov_b32 %s, %%[kve]" % s(KVE))
+    e("s_mov_b32 %s, %%[cl2]" % s(CL2))
+    e("s_mov_b32 %s, %%[npp]" % s(NPP))
+    e("s_mov_b32 %s, %%[nb1]" % s(NB1))
+    e("s_mov_b32 %s, %%[flg]" % s(FLG))
+    e("s_mov_b32 %s, %%[ntl]" % s(NT))
+    e("s_mov_b32 %s, %%[ostr]" % s(OSTR))
+    e("s_mov_b32 %s, %%[pg0]" % s(PGZ))
+    e("s_mov_b64 %s, %%[qp]" % s(QP, 2))
+    e("s_mov_b64 %s, %%[ob]" % s(OB, 2))
+    e("s_mov_b64 %s, %%[mlb]" % s(MLB, 2))
+    e("s_mov_b32 %s, %%[rstr]" % s(RSTR))
+    e("s_mov_b32 %s, %%[nrv]" % s(NRV))
+    e("v_mov_b32 %s, %%[tid]" % v(X0))
+    e("s_mov_b32 %s, 0x%08x" % (s(THR), TAU_BITS))
+    e("s_mov_b32 %s, 0x3c003c00" % s(ONES))
+    e("v_and_b32 %s, 63, %s" % (v(LANE), v(X0)))
+    e("v_lshrrev_b32 %s, 6, %s" % (v(X1), v(X0)))
+    e("s_nop 0")
+    e("v_readfirstlane_b32 %s, %s" % (s(WAVE), v(X1)))
+    e("s_lshl_b32 %s, %s, 2" % (s(W4), s(WAVE)))
+    e("s_lshl_b32 %s, %s, 11" % (s(WOFS), s(WAVE)))
+    e("s_add_u32 %s, %s, 0x%x" % (s(FADR), s(W4), FOFF))
+    stamp("entry")
+    # lane geometry
+    e("v_and_b32 %s, 31, %s" % (v(X0), v(LANE)))                       # rl
+    e("v_lshrrev_b32 %s, 5, %s" % (v(X1), v(LANE)))                    # g
+    e("v_lshlrev_b32 %s, 2, %s" % (v(T[0]), v(X1)))                    # 4g
+    e("v_lshlrev_b32 %s, 4, %s" % (v(X2), v(X1)))                      # 16g
+    e("s_mov_b32 %s, %d" % (s(SPITCH), PITCH))
+    e("v_mad_u32_u24 %s, %s, %s, %s" % (v(KADDR_LANE), v(X0), s(SPITCH), v(X2)))
+    e("v_bfe_u32 %s, %s, 2, 2" % (v(X0), v(LANE)))                     # (lane & 15) >> 2
+    e("v_add_u32 %s, %s, %s" % (v(X0), v(T[0]), v(X0)))                # 4g + ...
+    e("v_bfe_u32 %s, %s, 4, 1" % (v(X1), v(LANE)))                     # (lane >> 4) & 1
+    e("v_lshlrev_b32 %s, 5, %s" % (v(X1), v(X1)))                      # *16 elements *2 bytes
+    e("v_and_b32 %s, 3, %s" % (v(X2), v(LANE)))
+    e("v_lshlrev_b32 %s, 3, %s" % (v(X2), v(X2)))                      # *4 elements *2 bytes
+    e("v_add_u32 %s, %s, %s" % (v(X1), v(X1), v(X2)))
+    e("v_mad_u32_u24 %s, %s, %s, %s" % (v(VADDR_LANE), v(X0), s(SPITCH), v(X1)))
+    # the wave's 128 output columns start at column 128 w (256 bytes into the rows); FLG bit 4: V is columns 64 .. 575 of
+    # the rows instead of 0 .. 511 (second pass of a 576-wide V)
+    e("s_lshl_b32 %s, %s, 8" % (s(S0), s(WAVE)))
+    e("s_bitcmp1_b32 %s, 4" % s(FLG))
+    e("s_cselect_b32 %s, 128, 0" % s(S1))
+    e("s_add_u32 %s, %s, %s" % (s(S0), s(S0), s(S1)))
+    e("v_add_u32 %s, %s, %s" % (v(VADDR_LANE), s(S0), v(VADDR_LANE)))
+    e("v_lshlrev_b32 %s, 4, %s" % (v(PADDR), v(LANE)))
+    e("v_add_u32 %s, 0x%x, %s" % (v(PADDR), PBUF, v(PADDR)))
+    # ------------------------------------------------------------------ page ids of this split -> one lane each
+    lab_nobt = label("nobt")
+    e("s_lshr_b32 %s, %s, 7" % (s(PG0), s(KVB)))
+    e("v_mov_b32 %s, 0" % v(PAGES))
+    e("s_cmp_eq_u64 %s, 0" % s(BT, 2))
+    e("s_cbranch_scc1 %s" % lab_nobt)
+    e("s_add_u32 %s, %s, 127" % (s(S0), s(KVE)))
+    e("s_lshr_b32 %s, %s, 7" % (s(S0), s(S0)))
+    e("s_sub_u32 %s, %s, %s" % (s(S0), s(S0), s(PG0)))                   # pages in this split (<= 64)
+    e("v_cmp_gt_u32 vcc, %s, %s" % (s(S0), v(LANE)))
+    e("s_mov_b64 %s, exec" % s(EXS, 2))
+    e("s_nop 1")
+    e("s_and_b64 exec, exec, vcc")
+    e("v_add_u32 %s, %s, %s" % (v(X0), s(PG0), v(LANE)))
+    e("v_lshlrev_b32 %s, 2, %s" % (v(X0), v(X0)))
+    e("global_load_dword %s, %s, %s" % (v(PAGES), v(X0), s(BT, 2)))
+    e("s_mov_b64 exec, %s" % s(EXS, 2))
+    e("%s:" % lab_nobt)
+    # ------------------------------------------------------------------ Q operands: 36 coalesced 16-byte loads per lane from
+    # the packed image, in flight together with the page ids
+    e("v_lshlrev_b32 %s, 4, %s" % (v(X0), v(LANE)))
+    e("s_mul_i32 %s, %s, %d" % (s(S0), s(WAVE), 36 * 1024))
+    e("s_add_u32 %s, %s, %s" % (s(QP), s(QP), s(S0)))
+    e("s_addc_u32 %s, %s, 0" % (s(QP + 1), s(QP + 1)))
+    nq = 36
+    for ks in range(nq):
+        if ks and ks % 4 == 0:
+            e("s_add_u32 %s, %s, 4096" % (s(QP), s(QP)))
+            e("s_addc_u32 %s, %s, 0" % (s(QP + 1), s(QP + 1)))
+        e("global_load_dwordx4 %s, %s, %s offset:%d" % (v(Q0 + 4 * ks, 4), v(X0), s(QP, 2), (ks % 4) * 1024))
+    n_early = nq
+    # ------------------------------------------------------------------ state
+    e("v_mov_b32 %s, 0xff800000" % v(MRUN))
+    e("v_mov_b32 %s, 0" % v(LRUN))
+    e("s_mov_b32 %s, 0" % s(OFF0))
+    e("s_mov_b32 %s, %d" % (s(OFF1), TILE_BYTES))
+    e("s_mov_b32 %s, %d" % (s(OFF2), 2 * TILE_BYTES))
+    e("s_mov_b32 %s, %d" % (s(OFF3), 3 * TILE_BYTES))
+    e("s_mov_b32 %s, 0" % s(IT))
+    for ln in dma_table_lines(LANE, (T[0], T[1], T[2], T[3], T[4])):
+        e(ln)
+    # The first tiles can be requested before the page ids are there when the split starts on a page boundary: they lie in
+    # the first page, whose id came as a scalar.  Otherwise wait for the ids (loads return in order: only the Q loads may
+    # still be in flight).
+    lab_al = label("aligned")
+    e("s_and_b32 %s, %s, 127" % (s(S0), s(KVB)))
+    e("s_cmp_eq_u32 %s, 0" % s(S0))
+    e("s_cbranch_scc1 %s" % lab_al)
+    e("s_waitcnt vmcnt(%d)" % n_early)
+    e("v_max_i32 %s, 0, %s" % (v(PAGES), v(PAGES)))
+    e("v_min_i32 %s, %s, %s" % (v(PAGES), s(NPP), v(PAGES)))
+    e("%s:" % lab_al)
+    # ------------------------------------------------------------------ tiles 0, 1, 2 -> LDS; go on as soon as Q and tile 0 are there
+    lab_w0, lab_w1, lab_wd = label("pw0"), label("pw1"), label("pwd")
+    e("s_mov_b32 %s, 0" % s(TMP))
+    for ln in dma_tile_lines(TMP, OFF0, True):
+        e(ln)
+    for i in range(256):
+        e("v_accvgpr_write_b32 %s, 0" % a(i))
+    e("s_cmp_lt_u32 %s, 2" % s(NT))
+    e("s_cbranch_scc1 %s" % lab_w0)
+    e("s_mov_b32 %s, 1" % s(TMP))
+    for ln in dma_tile_lines(TMP, OFF1, True):
+        e(ln)
+    e("s_cmp_lt_u32 %s, 3" % s(NT))
+    e("s_cbranch_scc1 %s" % lab_w1)
+    e("s_mov_b32 %s, 2" % s(TMP))
+    for ln in dma_tile_lines(TMP, OFF2, True):
+        e(ln)
+    e("s_waitcnt vmcnt(%d)" % (2 * DMA_PER_TILE))
+    e("s_branch %s" % lab_wd)
+    e("%s:" % lab_w1)
+    e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
+    e("s_branch %s" % lab_wd)
+    e("%s:" % lab_w0)
+    e("s_waitcnt vmcnt(0)")
+    e("%s:" % lab_wd)
+    # page ids outside the pool can only come from table entries that are never used; clamped so that no address leaves the pool
+    e("v_max_i32 %s, 0, %s" % (v(PAGES), v(PAGES)))
+    e("v_min_i32 %s, %s, %s" % (v(PAGES), s(NPP), v(PAGES)))
+    e("s_barrier")                      # tile 0 is complete; every wave has read its hand-off record
+    stamp("q+tile0")
+    e("v_add_u32 %s, %s, %s" % (v(KADDR), s(OFF0), v(KADDR_LANE)))
+    k_warm()
+    for slot in qk_slots():
+        slot()
+    e("s_sub_u32 %s, %s, %s" % (s(NVAL), s(KVE), s(KVB)))
+    e("s_min_u32 %s, %s, 32" % (s(NVAL), s(NVAL)))
+    e("s_nop 7")
+    e("s_nop 7")
+    mask_tail()
+    for ln in softmax_lines(first_tile=True):
+        e(ln)
+    for it_ in p_write_items():
+        emit_item(it_)
+    lds.drain()
+    # tile 1 has landed (tile 2 may still be in flight)
+    lab_t1, lab_t1d = label("t1"), label("t1d")
+    e("s_cmp_lt_u32 %s, 3" % s(NT))
+    e("s_cbranch_scc1 %s" % lab_t1)
+    e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
+    e("s_branch %s" % lab_t1d)
+    e("%s:" % lab_t1)
+    e("s_waitcnt vmcnt(0)")
+    e("%s:" % lab_t1d)
+    e("s_barrier")
+    resc = []
+    handover(OFF1, [], resc)
+    stamp("tile0")
+    # ------------------------------------------------------------------ main loop
+    lab_loop, lab_end = label("loop"), label("end")
+    e("%s:" % lab_loop)
+    iteration(resc)
+    e("s_cmp_lt_u32 %s, %s" % (s(IT), s(NT)))
+    e("s_cbranch_scc1 %s" % lab_loop)
+    e("s_branch %s" % lab_end)
+    for lab, back in resc:
+        e("%s:" % lab)
+        rescale_block(back)
+    e("%s:" % lab_end)
+    stamp("loop")
+    # ------------------------------------------------------------------ epilogue
+    e("s_barrier")                      # no wave is still reading rescale factors: their area carries 1 / l next
+    e("s_nop 7")
+    e("s_nop 7")
+    e("s_nop 7")
+    # l of the wave's own rows: l(lane) + l(lane ^ 32); 1 / l with one Newton step (l = 0 still gives inf / NaN)
+    e("v_mov_b32 %s, %s" % (v(T[0]), v(LRUN)))
+    e("v_mov_b32 %s, %s" % (v(T[1]), v(LRUN)))
+    e("s_nop 1")
+    e("v_permlane32_swap_b32 %s, %s" % (v(T[0]), v(T[1])))
+    e("s_nop 1")
+    e("v_add_f32 %s, %s, %s" % (v(LRUN), v(T[0]), v(T[1])))
+    e("v_rcp_f32 %s, %s" % (v(T[2]), v(LRUN)))
+    e("s_nop 0")
+    e("v_fma_f32 %s, -%s, %s, 2.0" % (v(T[3]), v(LRUN), v(T[2])))
+    e("v_mul_f32 %s, %s, %s" % (v(T[3]), v(T[2]), v(T[3])))
+    e("s_mov_b32 %s, 0x1f8" % s(SCLS))
+    e("v_cmp_class_f32 vcc, %s, %s" % (v(T[3]), s(SCLS)))   # finite?
+    e("s_nop 1")
+    e("v_cndmask_b32 %s, %s, %s, vcc" % (v(T[2]), v(T[2]), v(T[3])))
+    # every wave needs 1 / l of all 128 rows: through the rescale-factor area, [lane][hb]
+    e("v_add_u32 %s, %s, %s" % (v(T[3]), s(W4), v(PADDR)))
+    e("ds_write_b32 %s, %s offset:%d" % (v(T[3]), v(T[2]), AOFF - PBUF))
+    e("s_waitcnt lgkmcnt(0)")
+    e("s_barrier")
+    e("ds_read_b128 %s, %s offset:%d" % (v(T[4], 4), v(PADDR), AOFF - PBUF))   # T[4 + hb] = 1 / l of row 32 hb + lane % 32
+    # lanes whose row exists, per row block: lane % 32 < n_rows_valid - 32 hb
+    e("v_mbcnt_lo_u32_b32 %s, -1, 0" % v(X0))
+    e("v_mbcnt_hi_u32_b32 %s, -1, %s" % (v(X0), v(X0)))               # lane
+    e("v_and_b32 %s, 31, %s" % (v(X1), v(X0)))                         # rl
+    for hb in range(4):
+        e("s_sub_i32 %s, %s, %d" % (s(S0), s(NRV), 32 * hb))
+        e("v_cmp_gt_i32 vcc, %s, %s" % (s(S0), v(X1)))
+        e("s_mov_b64 %s, vcc" % s(VM[hb], 2))
+    e("s_mov_b64 %s, exec" % s(EXS, 2))
+    e("v_lshrrev_b32 %s, 5, %s" % (v(X2), v(X0)))                      # g
+    e("s_waitcnt lgkmcnt(0)")
+    lab_pstore, lab_sdone = label("pstore"), label("sdone")
+    if NO_STORE:
+        e("s_branch %s" % lab_sdone)
+    e("s_bitcmp1_b32 %s, 0" % s(FLG))
+    e("s_cbranch_scc0 %s" % lab_pstore)
+    # f32 rows (final output, or f32 partials): element (row, column) at OB + row * RSTR + column * 4.
+    # acc[cb][hb] register 4 q + c of lane (rl, g) is row 32 hb + rl, column 128 w + 32 cb + 8 q + 4 g + c.
+    e("v_mul_lo_u32 %s, %s, %s" % (v(T[0]), v(X1), s(RSTR)))
+    e("v_lshlrev_b32 %s, 4, %s" % (v(T[1]), v(X2)))
+    e("v_add_u32 %s, %s, %s" % (v(T[0]), v(T[0]), v(T[1])))
+    e("s_lshl_b32 %s, %s, 9" % (s(S0), s(WAVE)))
+    e("v_add_u32 %s, %s, %s" % (v(T[0]), s(S0), v(T[0])))              # rl * RSTR + 16 g + 512 w
+    e("s_lshl_b32 %s, %s, 5" % (s(S1), s(RSTR)))                       # 32 rows
+    e("s_mov_b64 %s, %s" % (s(SB, 2), s(OB, 2)))
+    for hb in range(4):
+        e("s_mov_b64 exec, %s" % s(VM[hb], 2))
+        for cb in range(4):
+            for q in range(4):
+                r = S if (cb * 4 + q) % 2 == 0 else S + 4          # alternate two 4-register staging groups
+                for c in range(4):
+                    e("v_accvgpr_read_b32 %s, %s" % (v(r + c), a(16 * (4 * cb + hb) + 4 * q + c)))
+                for c in range(4):
+                    e("v_mul_f32 %s, %s, %s" % (v(r + c), v(r + c), v(T[4 + hb])))
+                e("global_store_dwordx4 %s, %s, %s offset:%d" % (v(T[0]), v(r, 4), s(SB, 2), (32 * cb + 8 * q) * 4))
+        e("s_add_u32 %s, %s, %s" % (s(SB), s(SB), s(S1)))
+        e("s_addc_u32 %s, %s, 0" % (s(SB + 1), s(SB + 1)))
+    e("s_branch %s" % lab_sdone)
+    e("%s:" % lab_pstore)
+    # f16 partials O / l, layout [column / 8][row][8 halves]: the 8 bytes of lane (rl, g) for column group 16 w + 4 cb + q
+    # of row 32 hb + rl sit at OB + (16 w + 4 cb + q) * OSTR + (32 hb + rl) * 16 + 8 g  (OSTR = rows of a slot * 16)
+    e("v_lshlrev_b32 %s, 4, %s" % (v(T[0]), v(X1)))
+    e("v_lshlrev_b32 %s, 3, %s" % (v(T[1]), v(X2)))
+    e("v_add_u32 %s, %s, %s" % (v(T[0]), v(T[0]), v(T[1])))            # rl * 16 + 8 g
+    e("s_lshl_b32 %s, %s, 4" % (s(S0), s(WAVE)))
+    e("s_mul_i32 %s, %s, %s" % (s(S0), s(S0), s(OSTR)))                # 16 w * OSTR  (< 2^31: OSTR <= 2^27 / 64 is checked on the host)
+    e("s_add_u32 %s, %s, %s" % (s(S2), s(OB), s(S0)))
+    e("s_addc_u32 %s, %s, 0" % (s(S3), s(OB + 1)))
+    for hb in range(4):
+        e("s_mov_b64 exec, %s" % s(VM[hb], 2))
+        e("s_mov_b64 %s, %s" % (s(SB, 2), s(S2, 2)))
+        for cb in range(4):
+            for q in range(4):
+                r = S if (cb * 4 + q) % 2 == 0 else S + 4
+                for c in range(4):
+                    e("v_accvgpr_read_b32 %s, %s" % (v(r + c), a(16 * (4 * cb + hb) + 4 * q + c)))
+                for c in range(4):
+                    e("v_mul_f32 %s, %s, %s" % (v(r + c), v(r + c), v(T[4 + hb])))
+                e("v_cvt_pk_f16_f32 %s, %s, %s" % (v(r), v(r), v(r + 1)))
+                e("v_cvt_pk_f16_f32 %s, %s, %s" % (v(r + 1), v(r + 2), v(r + 3)))
+                e("s_nop 0")
+                e("global_store_dwordx2 %s, %s, %s offset:%d" % (v(T[0]), v(r, 2), s(SB, 2), hb * 512))
+                e("s_add_u32 %s, %s, %s" % (s(SB), s(SB), s(OSTR)))
+                e("s_addc_u32 %s, %s, 0" % (s(SB + 1), s(SB + 1)))
+    e("%s:" % lab_sdone)
+    # (m, l) of this split for the wave's own rows, written by the g == 0 lanes when a pointer was handed over
+    lab_noml = label("noml")
+    e("s_mov_b64 exec, %s" % s(EXS, 2))
+    e("s_cmp_eq_u64 %s, 0" % s(MLB, 2))
+    e("s_cbranch_scc1 %s" % lab_noml)
+    e("s_lshl_b32 %s, %s, 5" % (s(S0), s(WAVE)))
+    e("s_sub_i32 %s, %s, %s" % (s(S0), s(NRV), s(S0)))                 # valid rows of this wave's block
+    e("v_cmp_gt_i32 vcc, %s, %s" % (s(S0), v(X0)))                     # lane < that ...
+    e("s_nop 1")
+    e("s_and_b64 exec, exec, vcc")
+    e("s_mov_b32 exec_hi, 0")                                          # ... and g == 0
+    e("v_lshlrev_b32 %s, 3, %s" % (v(T[2]), v(X0)))
+    e("s_lshl_b32 %s, %s, 8" % (s(S1), s(WAVE)))
+    e("v_add_u32 %s, %s, %s" % (v(T[2]), s(S1), v(T[2])))              # (32 w + lane) * 8
+    e("v_mov_b32 %s, %s" % (v(T[0]), v(MRUN)))
+    e("v_mov_b32 %s, %s" % (v(T[1]), v(LRUN)))
+    e("s_nop 0")
+    e("global_store_dwordx2 %s, %s, %s" % (v(T[2]), v(T[0], 2), s(MLB, 2)))
+    e("%s:" % lab_noml)
+    e("s_mov_b64 exec, %s" % s(EXS, 2))
+    e("s_waitcnt vmcnt(0)")
+    stamp("epilogue")
+
+    print("// generated by gen_decode_cs_asm.py%s -- do not edit" % (" --f16" if F16KV else ""))
+    for ln in out:
+        print('"%s\\n\\t"' % ln)
+    if CLK:
+        sys.stderr.write("stamps: %s\n" % ", ".join(STAMPS))
+
+
+main()

@@ -20,9 +20,12 @@ namespace {
 
 // LDS: 4 resident 16-bit tiles (bf16 / f16 KV), or 3 of them behind 2 raw Q8_0 tiles; then the hand-off area,
 // 32 bytes per thread: mask offset, out pointer, (m,l) pointer, debug pointer
+// The column-split programs (SRC_*_CS) keep behind the four tiles: the P^T exchange buffer (8 KB; the hand-off records share it, they
+// are read before P is first written), the rescale factors (1 KB) and the waves' flag words (64 bytes).
+constexpr bool is_cs(int kvt) { return kvt == SRC_BF16_CS || kvt == SRC_F16_CS; }
 constexpr int handoff_off(int kvt) { return kvt == SRC_Q8 ? 3 * TILE_BYTES + 2 * Q8_TILE_RAW : 4 * TILE_BYTES; }
 constexpr int SCHED_MAX_SEQ = 256;                   // balanced schedule: sequences per launch
-constexpr int sched_off(int kvt) { return handoff_off(kvt) + NTHREADS * 32; }   // prefix sums of the sequences' tile counts
+constexpr int sched_off(int kvt) { return handoff_off(kvt) + (is_cs(kvt) ? 8192 + 1024 + 64 : NTHREADS * 32); }   // prefix sums of the sequences' tile counts
 constexpr int lds_total(int kvt) { return sched_off(kvt) + (2 * SCHED_MAX_SEQ + 8) * 4; }   // prefix sums, then the lengths
 
 #define MLA_DECODE_CLOBBERS \
@@ -63,6 +66,13 @@ constexpr int lds_total(int kvt) { return sched_off(kvt) + (2 * SCHED_MAX_SEQ + 
     "a214", "a215", "a216", "a217", "a218", "a219", "a220", "a221", "a222", "a223", "a224", "a225", "a226", "a227", \
     "a228", "a229", "a230", "a231", "a232", "a233", "a234", "a235", "a236", "a237", "a238", "a239", "a240", "a241", \
     "a242", "a243", "a244", "a245", "a246", "a247", "a248", "a249", "a250", "a251", "a252", "a253", "a254", "a255"
+
+#define MLA_DECODE_CS_CLOBBERS MLA_DECODE_CLOBBERS, "s84", "s85", "s86", "s87", "s88", "s89", "s90", "s91", "s92", "s93", "s94", "s95", "s96", "s97", "s98", "s99"
+
+#define MLA_DECODE_CS_INPUTS                                                                                       \
+    [kv] "s"(kv_base), [bt] "s"(bt_row), [kvb] "s"(s_kvb), [kve] "s"(s_kve), [cl2] "s"(c_log2_bits), [npp] "s"(s_npp), \
+    [nb1] "s"(s_nb1), [flg] "s"(s_flg), [ntl] "s"(s_ntl), [ostr] "s"(s_ostr), [qp] "s"(qpack), [pg0] "s"(s_pg0),  \
+    [ob] "s"(out_base), [mlb] "s"(ml_base), [rstr] "s"(s_rstr), [nrv] "s"(s_nrv), [tid] "v"(tid)
 
 #define MLA_DECODE_INPUTS                                                                                          \
     [kv] "s"(kv_base), [bt] "s"(bt_row), [kvb] "s"(s_kvb), [kve] "s"(s_kve), [cl2] "s"(c_log2_bits), [npp] "s"(s_npp), \
@@ -341,7 +351,25 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
     const int s_scale = __builtin_amdgcn_readfirstlane(__float_as_int(p.scale));
     const int s_ostr = __builtin_amdgcn_readfirstlane(p.slot_rows * 16);  // bytes between the partial rows of column groups c and c+1
 
-    if constexpr (KVT == SRC_Q8 && MASK) {
+    // column-split programs: every wave stores 128 columns of all 128 rows, so the output is described by scalars -- the block's
+    // first row in dst (final rows) or in its partial slot, the byte pitch of f32 rows, and the number of rows that exist
+    const int lrow0 = p.balanced == 2 ? 0 : by * 128;
+    const char * out_base = direct ? (const char *) (p.dst + ((int64_t) b * p.n_rows + by * 128) * p.dst_stride + p.v_col0)
+                          : p.part_f32 ? (const char *) ((float *) p.part_o + ((int64_t) slot * p.slot_rows + lrow0) * p.dv_total)
+                                       : (const char *) (p.part_o + pblock + (int64_t) lrow0 * 8);
+    const char * ml_base  = direct ? nullptr : (const char *) (p.part_ml + ((int64_t) slot * p.slot_rows + lrow0) * 2);
+    const int s_rstr = __builtin_amdgcn_readfirstlane((int) ((direct ? p.dst_stride : (int64_t) p.dv_total) * 4));
+    const int s_nrv  = __builtin_amdgcn_readfirstlane(min(max(p.n_rows - by * 128, 0), 128));
+
+    if constexpr (KVT == SRC_BF16_CS) {
+        asm volatile(
+#include "mla_decode_cs_bf16.inc"
+            : : MLA_DECODE_CS_INPUTS : MLA_DECODE_CS_CLOBBERS);
+    } else if constexpr (KVT == SRC_F16_CS) {
+        asm volatile(
+#include "mla_decode_cs_f16.inc"
+            : : MLA_DECODE_CS_INPUTS : MLA_DECODE_CS_CLOBBERS);
+    } else if constexpr (KVT == SRC_Q8 && MASK) {
         asm volatile(
 #include "mla_decode_asm_q8_mask.inc"
             : : MLA_DECODE_INPUTS : MLA_DECODE_CLOBBERS);
@@ -588,13 +616,23 @@ static hipError_t launch_variant(const KParams & kp, dim3 grid, hipStream_t st) 
     return hipGetLastError();
 }
 
+static bool decode_cs_applicable(const KParams & kp, int kv_type) {
+    if (kv_type != MLA_TYPE_BF16 && kv_type != MLA_TYPE_F16) return false;
+    if (kp.mask || kp.bf16_direct || kp.q_as_q8) return false;
+    const int tail = kp.n_rows % 128;
+    return (tail == 0 || tail > 96) && kp.slot_rows < (1 << 22);
+}
+
 hipError_t launch_decode_fast(const KParams & kp, int kv_type, dim3 grid, hipStream_t st, bool with_prepass) {
     // the small passes ahead of the kernel run per (row block, sequence), whatever the kernel's own grid is
     const unsigned n_rb = (unsigned) ((kp.n_rows + 127) / 128), n_seq = (unsigned) kp.n_seq_sched, extra = kp.balanced == 1 ? 1 : 0;
     const bool m = kp.mask != nullptr;
     // bf16 tiles are converted to f16 inside LDS unless the caller asks for the hi + lo program, or a single wave of a workgroup
     // has rows (16- and 32-head decode): one computing wave is not bound by its MFMAs, and the hi + lo program is the more exact
-    const bool bf16_cvt = !kp.bf16_direct && kp.n_rows > 32;
+    // column-split programs (every wave computes S for its own 32 rows and P.V for its own 128 columns): blocks of 128 rows in
+    // which all four waves have rows, no mask, not the Q8_0 expansion; bf16 K enters as bf16, so the Q image is the bf16 one
+    const bool cs = decode_cs_applicable(kp, kv_type);
+    const bool bf16_cvt = !cs && !kp.bf16_direct && kp.n_rows > 32;
     if (!with_prepass) { /* the workspace still holds the Q image and the mask extents of an earlier launch of the same call */ }
     else if (kv_type == MLA_TYPE_Q8_0 || kp.q_as_q8) hipLaunchKernelGGL(mla_q_pack_q8_kernel, dim3(n_rb, n_seq, KSTEPS / 2 + extra), dim3(NTHREADS), 0, st, kp);
     else if (kv_type == MLA_TYPE_F16) hipLaunchKernelGGL(mla_q_pack_kernel<1>, dim3(n_rb, n_seq, KSTEPS + extra), dim3(NTHREADS), 0, st, kp);
@@ -602,6 +640,8 @@ hipError_t launch_decode_fast(const KParams & kp, int kv_type, dim3 grid, hipStr
     else                              hipLaunchKernelGGL(mla_q_pack_kernel<0>, dim3(n_rb, n_seq, KSTEPS + extra), dim3(NTHREADS), 0, st, kp);
     if (m && with_prepass) hipLaunchKernelGGL(mla_mask_extent_kernel, dim3(n_rb, MASK_EXT_CHUNKS), dim3(NTHREADS), 0, st, kp);
     if (kv_type == MLA_TYPE_Q8_0) return m ? launch_variant<SRC_Q8, true>(kp, grid, st) : launch_variant<SRC_Q8, false>(kp, grid, st);
+    if (cs && kv_type == MLA_TYPE_F16) return launch_variant<SRC_F16_CS, false>(kp, grid, st);
+    if (cs)                            return launch_variant<SRC_BF16_CS, false>(kp, grid, st);
     if (kv_type == MLA_TYPE_F16)  return m ? launch_variant<SRC_F16, true>(kp, grid, st) : launch_variant<SRC_F16, false>(kp, grid, st);
     if (bf16_cvt)                 return m ? launch_variant<SRC_BF16_CVT, true>(kp, grid, st) : launch_variant<SRC_BF16_CVT, false>(kp, grid, st);
     return m ? launch_variant<SRC_BF16, true>(kp, grid, st) : launch_variant<SRC_BF16, false>(kp, grid, st);

@@ -151,11 +151,13 @@ def test_planner_schedules_without_gpu():
     assert rc == 0 and info.variant == 0 and info.rows_per_wg == 64
 
 
-@pytest.mark.parametrize("flags,name", [([], "mla_decode_asm.inc"), (["--f16"], "mla_decode_asm_f16.inc"), (["--mask"], "mla_decode_asm_mask.inc"),
-                                        (["--f16", "--mask"], "mla_decode_asm_f16_mask.inc"), (["--q8"], "mla_decode_asm_q8.inc"),
-                                        (["--q8", "--mask"], "mla_decode_asm_q8_mask.inc"), (["--cvt"], "mla_decode_asm_cvt.inc"),
-                                        (["--cvt", "--mask"], "mla_decode_asm_cvt_mask.inc")])
-def test_committed_wave_programs_are_what_the_generator_emits(flags, name):
+@pytest.mark.parametrize("gen,flags,name", [("gen_decode_asm.py", [], "mla_decode_asm.inc"), ("gen_decode_asm.py", ["--f16"], "mla_decode_asm_f16.inc"),
+                                            ("gen_decode_asm.py", ["--mask"], "mla_decode_asm_mask.inc"),
+                                            ("gen_decode_asm.py", ["--f16", "--mask"], "mla_decode_asm_f16_mask.inc"), ("gen_decode_asm.py", ["--q8"], "mla_decode_asm_q8.inc"),
+                                            ("gen_decode_asm.py", ["--q8", "--mask"], "mla_decode_asm_q8_mask.inc"), ("gen_decode_asm.py", ["--cvt"], "mla_decode_asm_cvt.inc"),
+                                            ("gen_decode_asm.py", ["--cvt", "--mask"], "mla_decode_asm_cvt_mask.inc"),
+                                            ("gen_decode_cs_asm.py", [], "mla_decode_cs_bf16.inc"), ("gen_decode_cs_asm.py", ["--f16"], "mla_decode_cs_f16.inc")])
+def test_committed_wave_programs_are_what_the_generator_emits(gen, flags, name):
     """The instruction streams the decode kernel includes are generated files: each equals the generator's output.  None of
     them touches v252..v255: the asm block's clobber list ends at v251, and the compiler keeps there what lives across the
     block (the lanes it spills scalar registers to among it)."""
@@ -163,15 +165,16 @@ def test_committed_wave_programs_are_what_the_generator_emits(flags, name):
     import subprocess
     import sys
     csrc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "jittorinfer_amd", "csrc")
-    got = subprocess.run([sys.executable, os.path.join(csrc, "gen_decode_asm.py")] + flags, capture_output=True, text=True, check=True).stdout
+    got = subprocess.run([sys.executable, os.path.join(csrc, gen)] + flags, capture_output=True, text=True, check=True).stdout
     with open(os.path.join(csrc, name)) as f:
-        assert got == f.read(), "%s is stale: regenerate it with gen_decode_asm.py %s" % (name, " ".join(flags))
+        assert got == f.read(), "%s is stale: regenerate it with %s %s" % (name, gen, " ".join(flags))
     for m in re.finditer(r"\bv(\d+)\b|\bv\[(\d+):(\d+)\]", got):
         hi = int(m.group(1)) if m.group(1) else int(m.group(3))
         assert hi <= 251, "%s uses %s" % (name, m.group(0))
-    for m in re.finditer(r"\bs(\d+)\b|\bs\[(\d+):(\d+)\]", got):      # scalar registers: inside the clobbered range s40..s83
+    top = 99 if gen == "gen_decode_cs_asm.py" else 83
+    for m in re.finditer(r"\bs(\d+)\b|\bs\[(\d+):(\d+)\]", got):      # scalar registers: inside the clobbered range s40..s83 (s99)
         lo, hi = (int(m.group(1)),) * 2 if m.group(1) else (int(m.group(2)), int(m.group(3)))
-        assert 40 <= lo and hi <= 83, "%s uses %s" % (name, m.group(0))
+        assert 40 <= lo and hi <= top, "%s uses %s" % (name, m.group(0))
 
 
 def test_python_constants_match_the_header():
