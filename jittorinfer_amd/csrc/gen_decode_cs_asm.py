@@ -21,6 +21,7 @@ ARGS = sys.argv[1:]
 F16KV = "--f16" in ARGS                      # f16 KV rows: f16 MFMA for K.Q^T, V^T fragments used as they are
 CLK = "--clk" in ARGS                        # timing builds: s_memtime stamps left in LDS at the end
 NO_STORE = "--no-store" in ARGS              # timing experiments only (wrong results)
+NO_LOOP_DMA = "--no-loop-dma" in ARGS        # timing experiments only (wrong results): the loop computes on whatever the tile buffers hold
 MF_QK = "v_mfma_f32_32x32x16_f16" if F16KV else "v_mfma_f32_32x32x16_bf16"
 MF_PV = "v_mfma_f32_32x32x16_f16"
 
@@ -41,7 +42,7 @@ FOFF = AOFF + 1024                           # one word per wave: non-zero when 
 CPR = 73                                     # 16-byte chunks per padded row
 WAVE_CHUNKS = 8 * CPR                        # each wave moves rows 8w .. 8w+7 of a tile
 DMA_PER_TILE = 10
-KRING, PRING = 5, 4
+KRING, PRING = 6, 4                          # K fragment ring: five slots of its own, the sixth in T[4:7] (free while K.Q^T runs)
 
 # ---- VGPR map (v252..v255 are left to the compiler: the clobber list of the asm block ends at v251)
 Q0 = 0
@@ -68,6 +69,11 @@ RSC, ONES, OSTR, QP, OB, MLB, RSTR, NRV = 72, 74, 75, 76, 78, 80, 82, 83
 W4, WOFS, FADR, PGZ, SPITCH, SCLS = 84, 85, 86, 87, 88, 89
 VM = [90, 92, 94, 96]   # epilogue: lanes whose row of row block hb exists
 SB = 98                 # epilogue: running store base
+# LDS-DMA loads (the epilogue's row masks take these registers afterwards): wave * bytes a wave copies per tile; the four clamp
+# offsets of the current tile; the first of them for the last tile of the piece; number of tiles - 1
+WDMA, CL, LAST0, NTM1 = 90, [91, 92, 93, 94], 95, 96
+DMA_BIAS = 3072         # the k-th load behind an M0 update carries the instruction offset 1024 k, which moves both addresses: the
+                        # table offsets are (true offset - 1024 k + 3072) and the tile base is taken 3072 bytes low
 TAU_BITS = 0x41000000   # 8.0f
 
 out = []
@@ -163,15 +169,13 @@ def run_slots(slots, first_index, streams, events=None):
 
 # ---------------------------------------------------------------------------------------------------------------
 def tile_base_lines(tile_sreg, first_page_scalar=False):
-    """Scalar lines: s[TB:TB+1] = address of the first row of tile s[tile_sreg]; s[NVM1] = its valid rows - 1.
-    first_page_scalar: a tile inside the split's first page takes the page id from s[PGZ] instead of the lane of PAGES
-    (the prologue's tiles, issued while the vector load of the page ids may still be in flight)."""
+    """Scalar lines: s[TB:TB+1] = address of the first row of tile s[tile_sreg], less DMA_BIAS (s[KV] is kept that much low).
+    The page id comes from the lane of PAGES that holds the tile's page (for a cache without a table PAGES holds the
+    logical pages themselves).  first_page_scalar: a tile inside the split's first page takes the id from s[PGZ] (the
+    prologue's tiles, issued while the vector load of the page ids may still be in flight)."""
     L = []
     L.append("s_lshl_b32 %s, %s, 5" % (s(S0), s(tile_sreg)))
     L.append("s_add_u32 %s, %s, %s" % (s(S0), s(S0), s(KVB)))                      # S0 = first token of the tile
-    L.append("s_sub_u32 %s, %s, %s" % (s(S1), s(KVE), s(S0)))
-    L.append("s_min_u32 %s, %s, 32" % (s(S1), s(S1)))
-    L.append("s_sub_u32 %s, %s, 1" % (s(NVM1), s(S1)))
     L.append("s_lshr_b32 %s, %s, 7" % (s(S1), s(S0)))                             # logical page
     L.append("s_sub_u32 %s, %s, %s" % (s(S1), s(S1), s(PG0)))                     # index into the preloaded lanes
     L.append("v_readlane_b32 %s, %s, %s" % (s(S2), v(PAGES), s(S1)))
@@ -180,11 +184,9 @@ def tile_base_lines(tile_sreg, first_page_scalar=False):
         L.append("s_cselect_b32 %s, %s, %s" % (s(S2), s(PGZ), s(S2)))
     L.append("s_lshl_b32 %s, %s, 7" % (s(S2), s(S2)))
     L.append("s_and_b32 %s, %s, 127" % (s(S3), s(S0)))
-    L.append("s_add_u32 %s, %s, %s" % (s(S2), s(S2), s(S3)))                      # pool row when paged
-    L.append("s_cmp_eq_u64 %s, 0" % s(BT, 2))
-    L.append("s_cselect_b32 %s, %s, %s" % (s(S0), s(S0), s(S2)))                  # no table: the logical row itself
-    L.append("s_mul_hi_u32 %s, %s, %s" % (s(S1), s(S0), s(NB1)))
-    L.append("s_mul_i32 %s, %s, %s" % (s(S0), s(S0), s(NB1)))
+    L.append("s_add_u32 %s, %s, %s" % (s(S2), s(S2), s(S3)))                      # row in the pool / in the cache
+    L.append("s_mul_hi_u32 %s, %s, %s" % (s(S1), s(S2), s(NB1)))
+    L.append("s_mul_i32 %s, %s, %s" % (s(S0), s(S2), s(NB1)))
     L.append("s_add_u32 %s, %s, %s" % (s(TB), s(KV), s(S0)))
     L.append("s_addc_u32 %s, %s, %s" % (s(TB + 1), s(KV + 1), s(S1)))
     return L
@@ -193,7 +195,8 @@ def tile_base_lines(tile_sreg, first_page_scalar=False):
 def dma_table_lines(lane, tmp):
     """Once per kernel: where the 16 bytes that lane l of LDS-DMA slot j copies sit inside a tile.  The LDS side of a slot
     is 64 consecutive 16-byte chunks of the padded tile (73 chunks per row, the 73rd is padding); the global side is
-    row * nb1 + min(column chunk, 71) * 16 -- at most 31 * 1152 + 1136, so two offsets share a register."""
+    row * nb1 + min(column chunk, 71) * 16 -- at most 31 * 1152 + 1136 -- stored with the bias the instruction offsets
+    ask for (see DMA_BIAS), two 16-bit values per register."""
     L = []
     row, col, x0, x1, x2 = tmp
     L.append("v_mov_b32 %s, %s" % (v(col), v(lane)))
@@ -203,6 +206,7 @@ def dma_table_lines(lane, tmp):
         L.append("v_min_u32 %s, 71, %s" % (v(x1), v(col)))
         L.append("v_lshlrev_b32 %s, 4, %s" % (v(x1), v(x1)))
         L.append("v_mad_u32_u24 %s, %s, %s, %s" % (v(x0), v(row), s(NB1), v(x1)))
+        L.append("v_add_u32 %s, %d, %s" % (v(x0), DMA_BIAS - 1024 * (j % 4), v(x0)))
         if j % 2 == 0:
             L.append("v_mov_b32 %s, %s" % (v(PT[j // 2]), v(x0)))
         else:
@@ -220,37 +224,41 @@ def dma_table_lines(lane, tmp):
 
 def dma_tile_lines(tile_sreg, off_sreg, first_page_scalar=False):
     """Instruction list (to be interleaved) that issues the LDS-DMA loads of tile s[tile_sreg] into the buffer at LDS
-    offset s[off_sreg].  Rows past the end of the sequence are replaced by the last 16 bytes of the last valid row (any
-    finite data will do: their probabilities are exactly 0): one v_min against that offset."""
+    offset s[off_sreg].  In the last tile of the piece rows past the end of the sequence are replaced by the last 16 bytes
+    of the last valid row (any finite data will do: their probabilities are exactly 0): the table offsets are clamped to
+    that row's last chunk (one SDWA instruction unpacks and clamps); in every other tile the clamp is out of reach."""
     L = tile_base_lines(tile_sreg, first_page_scalar)
-    L.append("s_mul_i32 %s, %s, %s" % (s(S3), s(NVM1), s(NB1)))
-    L.append("s_add_u32 %s, %s, %d" % (s(S3), s(S3), 71 * 16))
-    L.append("s_mul_i32 %s, %s, %d" % (s(DMAB), s(WAVE), WAVE_CHUNKS * 16))
-    L.append("s_add_u32 %s, %s, %s" % (s(DMAB), s(DMAB), s(off_sreg)))
+    L.append("s_cmp_eq_u32 %s, %s" % (s(tile_sreg), s(NTM1)))
+    L.append("s_cselect_b32 %s, %s, 0xffff" % (s(CL[0]), s(LAST0)))
+    for c in range(1, 4):
+        L.append("s_sub_u32 %s, %s, %d" % (s(CL[c]), s(CL[0]), 1024 * c))
+    L.append("s_add_u32 %s, %s, %s" % (s(DMAB), s(WDMA), s(off_sreg)))
     for j in range(10):
         t = DT[j & 1]
-        if j % 2 == 0:
-            L.append("v_and_b32 %s, 0xffff, %s" % (v(t), v(PT[j // 2])))
-        else:
-            L.append("v_lshrrev_b32 %s, 16, %s" % (v(t), v(PT[j // 2])))
-        L.append("v_min_u32 %s, %s, %s" % (v(t), s(S3), v(t)))
+        c = j % 4
+        unpack = "v_min_u32_sdwa %s, %s, %s dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:WORD_%d" % (v(t), s(CL[c]), v(PT[j // 2]), j % 2)
+        if c == 0:
+            L.append("s_add_u32 m0, %s, %d" % (s(DMAB), 4096 * (j // 4)))     # (the unpack below fills the wait state M0 needs)
+        L.append(unpack)
         if j == 9:
             # 8 chunks left per wave: lanes 0..7 only.  One atomic group: nothing may be scheduled inside the exec window.
-            L.append("\\n\\t".join(["s_add_u32 m0, %s, %d" % (s(DMAB), j * 1024),
-                                    "s_mov_b64 %s, exec" % s(EXS, 2),
+            L.append("\\n\\t".join(["s_mov_b64 %s, exec" % s(EXS, 2),
                                     "s_mov_b64 exec, 0xff",
-                                    "global_load_lds_dwordx4 %s, %s" % (v(t), s(TB, 2)),
+                                    "global_load_lds_dwordx4 %s, %s offset:%d" % (v(t), s(TB, 2), 1024 * c),
                                     "s_mov_b64 exec, %s" % s(EXS, 2)]))
         else:
-            L.append("\\n\\t".join(["s_add_u32 m0, %s, %d" % (s(DMAB), j * 1024),
-                                    "s_nop 0",
-                                    "global_load_lds_dwordx4 %s, %s" % (v(t), s(TB, 2))]))
+            L.append("global_load_lds_dwordx4 %s, %s offset:%d" % (v(t), s(TB, 2), 1024 * c))
     return L
 
 
 # ---------------------------------------------------------------------------------------------------------------
+def kf_reg(p):
+    slot = p % KRING
+    return KF + 4 * slot if slot < 5 else T[4]
+
+
 def k_read(p):
-    lds.op("ds_read_b128 %s, %s offset:%d" % (v(KF + 4 * (p % KRING), 4), v(KADDR), p * 32), ("k", p))
+    lds.op("ds_read_b128 %s, %s offset:%d" % (v(kf_reg(p), 4), v(KADDR), p * 32), ("k", p))
 
 
 def k_warm():
@@ -266,7 +274,7 @@ def qk_slots():
         def slot():
             lds.need(("k", ks + 1) if ks % 2 == 0 and ("k", ks + 1) in lds.pending else ("k", ks))   # fragments return in order
             c = "0" if ks == 0 else v(S, 16)
-            e("%s %s, %s, %s, %s" % (MF_QK, v(S, 16), v(KF + 4 * (ks % KRING), 4), v(Q0 + 4 * ks, 4), c))
+            e("%s %s, %s, %s, %s" % (MF_QK, v(S, 16), v(kf_reg(ks), 4), v(Q0 + 4 * ks, 4), c))
             if ks + depth < 36:
                 k_read(ks + depth)
         return slot
@@ -422,20 +430,30 @@ def canon_tags():
     return [("k", p) for p in range(KRING - 1)] + [("p", 0), ("p", 1), ("p", 2)]
 
 
-def handover(k_off, tail, resc):
-    """Behind the barrier that ends a tile: the flag words of the four waves, the first K fragments of the next K.Q^T (tile
-    buffer at s[k_off]) and the first P^T fragments of the tile whose P.V comes next, around the last two P.V MFMAs of the
-    tile that ends (they still use ring slot 3, which fragment 3 takes afterwards); then the accumulators take the new row
-    maxima if some wave's flag is up (out of line, rare)."""
+def handover(tail, resc):
+    """Behind the barrier that ends a tile (tile IT is the one whose P.V comes next): the flag words of the four waves, the
+    first K fragments of the next K.Q^T (tile IT+1, buffer at s[OFF1]) and the first P^T fragments of tile IT, around the
+    last four P.V MFMAs of the tile that ends (they still use ring slot 3, which fragment 3 takes afterwards), with the
+    scalars of the coming iteration in their shadow; then the accumulators take the new row maxima if some wave's flag is
+    up (out of line, rare)."""
     e("v_mov_b32 %s, 0x%x" % (v(T[4]), FOFF))
     lds.op("ds_read_b128 %s, %s" % (v(T[0], 4), v(T[4])), ("f",))
-    e("v_add_u32 %s, %s, %s" % (v(KADDR), s(k_off), v(KADDR_LANE)))
+    e("v_add_u32 %s, %s, %s" % (v(KADDR), s(OFF1), v(KADDR_LANE)))
     k_warm()
     p_read(0)
     p_read(1)
     p_read(2)
-    for sl in tail:
-        sl()
+    top = ["s_add_u32 %s, %s, 1" % (s(S0), s(IT)),
+           "s_lshl_b32 %s, %s, 5" % (s(S0), s(S0)),
+           "s_add_u32 %s, %s, %s" % (s(S0), s(S0), s(KVB)),
+           "s_sub_u32 %s, %s, %s" % (s(NVAL), s(KVE), s(S0)),
+           "s_min_u32 %s, %s, 32" % (s(NVAL), s(NVAL)),                    # valid tokens of tile IT+1
+           "v_add_u32 %s, %s, %s" % (v(VADDR), s(OFF0), v(VADDR_LANE))]  # V^T fragments of tile IT
+    if tail:
+        run_slots(tail, 0, [spread(top, 0, len(tail) - 1)])
+    else:
+        for ln in top:
+            e(ln)
     lds.need(("f",))
     e("v_or3_b32 %s, %s, %s, %s" % (v(T[0]), v(T[0]), v(T[1]), v(T[2])))
     e("v_or_b32 %s, %s, %s" % (v(T[0]), v(T[0]), v(T[3])))
@@ -470,42 +488,63 @@ def rescale_block(ret_label):
     e("s_branch %s" % ret_label)
 
 
-STAMPS = []
+CLK_PREV = 97                   # --clk builds: last time stamp
+LAPS = ["prologue to Q + tile 0", "first tile", "parts 1 and 2", "barrier (P read by all)", "P write + 4 MFMA", "tile-load wait", "barrier (tile end)"]
 
 
-def stamp(name):
-    """--clk builds: shader-clock time stamp into LDS (FOFF + 64 + 8 * index + 256 * wave), by lane 0."""
+def lap(k):
+    """--clk builds: adds the shader cycles since the last lap to accumulator k of this wave in LDS (FOFF + 64 + 32 w + 4 k;
+    lane 0 adds).  Only placed where no LDS access is in flight and X0 / DT are free."""
     if not CLK:
         return
-    k = len(STAMPS)
-    STAMPS.append(name)
+    assert not lds.pending, lds.pending
     e("s_memtime %s" % s(S0, 2))
     e("s_waitcnt lgkmcnt(0)")
-    e("v_mov_b32 %s, %s" % (v(X0), s(S0)))
-    e("s_mul_i32 %s, %s, 256" % (s(S1), s(WAVE)))
-    e("s_add_u32 %s, %s, 0x%x" % (s(S1), s(S1), FOFF + 64 + 8 * k))
-    e("v_mov_b32 %s, %s" % (v(X1), s(S1)))
-    e("ds_write_b32 %s, %s" % (v(X1), v(X0)))
-    e("s_waitcnt lgkmcnt(0)")
+    if k >= 0:
+        e("s_sub_u32 %s, %s, %s" % (s(S1), s(S0), s(CLK_PREV)))
+        e("v_mov_b32 %s, %s" % (v(X0), s(S1)))
+        e("s_lshl_b32 %s, %s, 5" % (s(S1), s(WAVE)))
+        e("s_add_u32 %s, %s, 0x%x" % (s(S1), s(S1), FOFF + 64 + 4 * k))
+        e("v_mov_b32 %s, %s" % (v(DT[0]), s(S1)))
+        e("s_mov_b64 exec, 1")
+        e("ds_add_u32 %s, %s" % (v(DT[0]), v(X0)))
+        e("s_mov_b64 exec, -1")
+        e("s_waitcnt lgkmcnt(0)")
+    e("s_mov_b32 %s, %s" % (s(CLK_PREV), s(S0)))
 
 
-def iteration(resc):
-    """Tile IT: see the module docstring."""
+def clk_init():
+    if CLK:
+        e("v_mov_b32 %s, 0" % v(X0))
+        e("s_lshl_b32 %s, %s, 5" % (s(S1), s(WAVE)))
+        e("s_add_u32 %s, %s, 0x%x" % (s(S1), s(S1), FOFF + 64))
+        e("v_mov_b32 %s, %s" % (v(DT[0]), s(S1)))
+        for k in range(8):
+            e("ds_write_b32 %s, %s offset:%d" % (v(DT[0]), v(X0), 4 * k))
+        e("s_waitcnt lgkmcnt(0)")
+
+
+def clk_dump():
+    pass
+
+
+B2_AT = _opt("--b2-at", 20)       # P.V slot ahead of which the barrier "every wave has read P of this tile" sits
+PW_AT = _opt("--pw-at", 24)       # P.V slot ahead of which P of the next tile is written (the softmax is done by then)
+
+
+def iteration(resc, lab_loop):
+    """Tile IT: see the module docstring.  s[NVAL] and v[VADDR] were set by the hand-over before."""
     e("; ---- iteration")
-    e("s_add_u32 %s, %s, 1" % (s(S0), s(IT)))
-    e("s_lshl_b32 %s, %s, 5" % (s(S0), s(S0)))
-    e("s_add_u32 %s, %s, %s" % (s(S0), s(S0), s(KVB)))
-    e("s_sub_u32 %s, %s, %s" % (s(NVAL), s(KVE), s(S0)))
-    e("s_min_u32 %s, %s, 32" % (s(NVAL), s(NVAL)))                    # valid tokens of tile IT+1
     e("s_mov_b32 %s, 0" % s(VMW))
-    lab_last, lab_nodma, lab_p2, lab_end = label("last"), label("nodma"), label("p2"), label("iend")
-    e("v_add_u32 %s, %s, %s" % (v(VADDR), s(OFF0), v(VADDR_LANE)))
+    lab_last, lab_nodma, lab_p2 = label("last"), label("nodma"), label("p2")
     e("s_add_u32 %s, %s, 1" % (s(TMP), s(IT)))
     e("s_cmp_ge_u32 %s, %s" % (s(TMP), s(NT)))
     e("s_cbranch_scc1 %s" % lab_last)
     e("s_add_u32 %s, %s, 3" % (s(TMP), s(IT)))
     e("s_cmp_ge_u32 %s, %s" % (s(TMP), s(NT)))
     e("s_cbranch_scc1 %s" % lab_nodma)
+    if NO_LOOP_DMA:
+        e("s_branch %s" % lab_nodma)
 
     def v_stream(n_conv, tmp):
         """Part 1: reads of all eight V^T fragments of tile IT (two fragments ahead of their conversion) and conversion of
@@ -533,6 +572,9 @@ def iteration(resc):
     assert lds.pending == state_a, (lds.pending, state_a)
     # ---- part 2: P.V of tile IT, softmax of tile IT+1 in its shadow
     e("%s:" % lab_p2)
+    if CLK:
+        lds.drain()
+        lap(0)
     pv = pv_slots()
     conv2 = []
     for f in range(CONV_P1, 8):
@@ -540,19 +582,20 @@ def iteration(resc):
     conv2 = spread(conv2, 37, 48) if conv2 else []      # one ordered stream (shared temporaries), done before k-step 1 starts at slot 52
 
     def qk_done():
-        e("s_nop 7")                    # the last K.Q^T MFMA has written S (two P.V MFMAs and these wait states behind it)
-        e("s_nop 1")
+        e("s_nop 1")                    # the last K.Q^T MFMA has written S: two P.V MFMAs (8 passes each) were issued behind it
         mask_tail()
+
+    def p_read_by_all():
+        # every P^T fragment of tile IT is in this wave's registers (the last read was issued at slot 16) before any wave overwrites P
+        lds.drain()
+        e("s_barrier")
     sm = softmax_lines()
-    streams = [conv2, spread(sm, 38, 60)]
-    left = run_slots(pv[:26], 36, streams, {38: [qk_done]})
+    streams = [conv2, spread(sm, 38, 36 + PW_AT - 1)]
+    left = run_slots(pv[:PW_AT], 36, streams, {38: [qk_done], 36 + B2_AT: [p_read_by_all]})
     assert not left, left
-    # every P^T fragment of tile IT is in registers (or on its way: waited for here) before any wave overwrites P
-    lds.drain()
-    e("s_barrier")
     for it_ in p_write_items():
         emit_item(it_)
-    for sl in pv[26:30]:
+    for sl in pv[PW_AT:28]:
         sl()
     lds.drain()
     # the loads of tile IT+2 have landed (those of tile IT+3, issued in this iteration, may still be in flight: loads
@@ -565,9 +608,17 @@ def iteration(resc):
     e("%s:" % lab_w0)
     e("s_waitcnt vmcnt(0)")
     e("%s:" % lab_wd)
+    if CLK:
+        lap(1)
     e("s_barrier")
-    handover(OFF2, pv[30:], resc)
-    e("s_branch %s" % lab_end)
+    e("s_mov_b32 %s, %s" % (s(TMP), s(OFF0)))
+    e("s_mov_b32 %s, %s" % (s(OFF0), s(OFF1)))
+    e("s_mov_b32 %s, %s" % (s(OFF1), s(OFF2)))
+    e("s_mov_b32 %s, %s" % (s(OFF2), s(OFF3)))
+    e("s_mov_b32 %s, %s" % (s(OFF3), s(TMP)))
+    e("s_add_u32 %s, %s, 1" % (s(IT), s(IT)))
+    handover(pv[28:], resc)
+    e("s_branch %s" % lab_loop)          # (tile IT exists: the iteration before was not the last)
     # ---- last tile: P.V only
     e("%s:" % lab_last)
     lds.reset(canon_tags())
@@ -580,13 +631,6 @@ def iteration(resc):
     for sl in pv_slots():
         sl()
     lds.drain()
-    e("%s:" % lab_end)
-    e("s_mov_b32 %s, %s" % (s(TMP), s(OFF0)))
-    e("s_mov_b32 %s, %s" % (s(OFF0), s(OFF1)))
-    e("s_mov_b32 %s, %s" % (s(OFF1), s(OFF2)))
-    e("s_mov_b32 %s, %s" % (s(OFF2), s(OFF3)))
-    e("s_mov_b32 %s, %s" % (s(OFF3), s(TMP)))
-    e("s_add_u32 %s, %s, 1" % (s(IT), s(IT)))
 
 
 def main():
@@ -617,7 +661,8 @@ def main():
     e("s_lshl_b32 %s, %s, 2" % (s(W4), s(WAVE)))
     e("s_lshl_b32 %s, %s, 11" % (s(WOFS), s(WAVE)))
     e("s_add_u32 %s, %s, 0x%x" % (s(FADR), s(W4), FOFF))
-    stamp("entry")
+    clk_init()
+    lap(-1)
     # lane geometry
     e("v_and_b32 %s, 31, %s" % (v(X0), v(LANE)))                       # rl
     e("v_lshrrev_b32 %s, 5, %s" % (v(X1), v(LANE)))                    # g
@@ -642,11 +687,14 @@ def main():
     e("v_add_u32 %s, %s, %s" % (v(VADDR_LANE), s(S0), v(VADDR_LANE)))
     e("v_lshlrev_b32 %s, 4, %s" % (v(PADDR), v(LANE)))
     e("v_add_u32 %s, 0x%x, %s" % (v(PADDR), PBUF, v(PADDR)))
-    # ------------------------------------------------------------------ page ids of this split -> one lane each
+    # ------------------------------------------------------------------ page ids of this split -> one lane each.  A cache without
+    # a table: the logical pages themselves (and no clamp against a pool size)
     lab_nobt = label("nobt")
     e("s_lshr_b32 %s, %s, 7" % (s(PG0), s(KVB)))
-    e("v_mov_b32 %s, 0" % v(PAGES))
+    e("v_add_u32 %s, %s, %s" % (v(PAGES), s(PG0), v(LANE)))
     e("s_cmp_eq_u64 %s, 0" % s(BT, 2))
+    e("s_cselect_b32 %s, 0x7fffffff, %s" % (s(NPP), s(NPP)))
+    e("s_cselect_b32 %s, %s, %s" % (s(PGZ), s(PG0), s(PGZ)))
     e("s_cbranch_scc1 %s" % lab_nobt)
     e("s_add_u32 %s, %s, 127" % (s(S0), s(KVE)))
     e("s_lshr_b32 %s, %s, 7" % (s(S0), s(S0)))
@@ -660,19 +708,6 @@ def main():
     e("global_load_dword %s, %s, %s" % (v(PAGES), v(X0), s(BT, 2)))
     e("s_mov_b64 exec, %s" % s(EXS, 2))
     e("%s:" % lab_nobt)
-    # ------------------------------------------------------------------ Q operands: 36 coalesced 16-byte loads per lane from
-    # the packed image, in flight together with the page ids
-    e("v_lshlrev_b32 %s, 4, %s" % (v(X0), v(LANE)))
-    e("s_mul_i32 %s, %s, %d" % (s(S0), s(WAVE), 36 * 1024))
-    e("s_add_u32 %s, %s, %s" % (s(QP), s(QP), s(S0)))
-    e("s_addc_u32 %s, %s, 0" % (s(QP + 1), s(QP + 1)))
-    nq = 36
-    for ks in range(nq):
-        if ks and ks % 4 == 0:
-            e("s_add_u32 %s, %s, 4096" % (s(QP), s(QP)))
-            e("s_addc_u32 %s, %s, 0" % (s(QP + 1), s(QP + 1)))
-        e("global_load_dwordx4 %s, %s, %s offset:%d" % (v(Q0 + 4 * ks, 4), v(X0), s(QP, 2), (ks % 4) * 1024))
-    n_early = nq
     # ------------------------------------------------------------------ state
     e("v_mov_b32 %s, 0xff800000" % v(MRUN))
     e("v_mov_b32 %s, 0" % v(LRUN))
@@ -681,24 +716,46 @@ def main():
     e("s_mov_b32 %s, %d" % (s(OFF2), 2 * TILE_BYTES))
     e("s_mov_b32 %s, %d" % (s(OFF3), 3 * TILE_BYTES))
     e("s_mov_b32 %s, 0" % s(IT))
+    e("s_sub_u32 %s, %s, %d" % (s(KV), s(KV), DMA_BIAS))
+    e("s_subb_u32 %s, %s, 0" % (s(KV + 1), s(KV + 1)))
+    e("s_mul_i32 %s, %s, %d" % (s(WDMA), s(WAVE), WAVE_CHUNKS * 16))
+    e("s_sub_u32 %s, %s, 1" % (s(NTM1), s(NT)))
+    # clamp offset of the last tile: its last valid row's last chunk, (n_valid - 1) * nb1 + 71 * 16, with the bias
+    e("s_sub_u32 %s, %s, %s" % (s(S0), s(KVE), s(KVB)))
+    e("s_lshl_b32 %s, %s, 5" % (s(S1), s(NTM1)))
+    e("s_sub_u32 %s, %s, %s" % (s(S0), s(S0), s(S1)))
+    e("s_sub_u32 %s, %s, 1" % (s(S0), s(S0)))
+    e("s_mul_i32 %s, %s, %s" % (s(S0), s(S0), s(NB1)))
+    e("s_add_u32 %s, %s, %d" % (s(LAST0), s(S0), 71 * 16 + DMA_BIAS))
     for ln in dma_table_lines(LANE, (T[0], T[1], T[2], T[3], T[4])):
         e(ln)
-    # The first tiles can be requested before the page ids are there when the split starts on a page boundary: they lie in
-    # the first page, whose id came as a scalar.  Otherwise wait for the ids (loads return in order: only the Q loads may
-    # still be in flight).
+    lap(3)
+    # Tile 0 can be requested before the page ids are there when the split starts on a page boundary: it lies in the first
+    # page, whose id came as a scalar.  Otherwise wait for the ids (the only load in flight).
     lab_al = label("aligned")
     e("s_and_b32 %s, %s, 127" % (s(S0), s(KVB)))
     e("s_cmp_eq_u32 %s, 0" % s(S0))
     e("s_cbranch_scc1 %s" % lab_al)
-    e("s_waitcnt vmcnt(%d)" % n_early)
+    e("s_waitcnt vmcnt(0)")
     e("v_max_i32 %s, 0, %s" % (v(PAGES), v(PAGES)))
     e("v_min_i32 %s, %s, %s" % (v(PAGES), s(NPP), v(PAGES)))
     e("%s:" % lab_al)
-    # ------------------------------------------------------------------ tiles 0, 1, 2 -> LDS; go on as soon as Q and tile 0 are there
-    lab_w0, lab_w1, lab_wd = label("pw0"), label("pw1"), label("pwd")
+    # ------------------------------------------------------------------ tile 0, then the Q operands (36 coalesced 16-byte loads per
+    # lane from the packed image), then tiles 1 and 2; go on as soon as tile 0 and Q are there
     e("s_mov_b32 %s, 0" % s(TMP))
     for ln in dma_tile_lines(TMP, OFF0, True):
         e(ln)
+    e("v_lshlrev_b32 %s, 4, %s" % (v(X0), v(LANE)))
+    e("s_mul_i32 %s, %s, %d" % (s(S0), s(WAVE), 36 * 1024))
+    e("s_add_u32 %s, %s, %s" % (s(QP), s(QP), s(S0)))
+    e("s_addc_u32 %s, %s, 0" % (s(QP + 1), s(QP + 1)))
+    for ks in range(36):
+        if ks and ks % 4 == 0:
+            e("s_add_u32 %s, %s, 4096" % (s(QP), s(QP)))
+            e("s_addc_u32 %s, %s, 0" % (s(QP + 1), s(QP + 1)))
+        e("global_load_dwordx4 %s, %s, %s offset:%d" % (v(Q0 + 4 * ks, 4), v(X0), s(QP, 2), (ks % 4) * 1024))
+    lap(4)
+    lab_w0, lab_w1, lab_wd = label("pw0"), label("pw1"), label("pwd")
     for i in range(256):
         e("v_accvgpr_write_b32 %s, 0" % a(i))
     e("s_cmp_lt_u32 %s, 2" % s(NT))
@@ -711,6 +768,7 @@ def main():
     e("s_mov_b32 %s, 2" % s(TMP))
     for ln in dma_tile_lines(TMP, OFF2, True):
         e(ln)
+    lap(5)
     e("s_waitcnt vmcnt(%d)" % (2 * DMA_PER_TILE))
     e("s_branch %s" % lab_wd)
     e("%s:" % lab_w1)
@@ -723,7 +781,6 @@ def main():
     e("v_max_i32 %s, 0, %s" % (v(PAGES), v(PAGES)))
     e("v_min_i32 %s, %s, %s" % (v(PAGES), s(NPP), v(PAGES)))
     e("s_barrier")                      # tile 0 is complete; every wave has read its hand-off record
-    stamp("q+tile0")
     e("v_add_u32 %s, %s, %s" % (v(KADDR), s(OFF0), v(KADDR_LANE)))
     k_warm()
     for slot in qk_slots():
@@ -749,20 +806,17 @@ def main():
     e("%s:" % lab_t1d)
     e("s_barrier")
     resc = []
-    handover(OFF1, [], resc)
-    stamp("tile0")
+    handover([], resc)
     # ------------------------------------------------------------------ main loop
     lab_loop, lab_end = label("loop"), label("end")
     e("%s:" % lab_loop)
-    iteration(resc)
-    e("s_cmp_lt_u32 %s, %s" % (s(IT), s(NT)))
-    e("s_cbranch_scc1 %s" % lab_loop)
+    iteration(resc, lab_loop)
     e("s_branch %s" % lab_end)
     for lab, back in resc:
         e("%s:" % lab)
         rescale_block(back)
     e("%s:" % lab_end)
-    stamp("loop")
+    clk_dump()
     # ------------------------------------------------------------------ epilogue
     e("s_barrier")                      # no wave is still reading rescale factors: their area carries 1 / l next
     e("s_nop 7")
@@ -875,13 +929,12 @@ def main():
     e("%s:" % lab_noml)
     e("s_mov_b64 exec, %s" % s(EXS, 2))
     e("s_waitcnt vmcnt(0)")
-    stamp("epilogue")
 
     print("// generated by gen_decode_cs_asm.py%s -- do not edit" % (" --f16" if F16KV else ""))
     for ln in out:
         print('"%s\\n\\t"' % ln)
     if CLK:
-        sys.stderr.write("stamps: %s\n" % ", ".join(STAMPS))
+        sys.stderr.write("laps: %s\n" % "; ".join(LAPS))
 
 
 main()
