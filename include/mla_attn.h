@@ -55,6 +55,7 @@ extern "C" {
 #define MLA_ERR_WORKSPACE     (-4)
 #define MLA_ERR_NULL          (-5)
 #define MLA_ERR_UNSUPPORTED   (-6)
+#define MLA_ERR_TOO_LARGE     (-7) /* mla_attn_launch_static: the call needs more scratch than MLA_ATTN_STATIC_WORKSPACE_MAX */
 
 #define MLA_PAGE_TOKENS 128
 
@@ -141,6 +142,16 @@ int    mla_attn_launch_combine(const mla_attn_args * args, void * stream);
  * mla_attn_launch or mla_attn_launch_partials has run with the same arguments and workspace.  No counterpart in
  * the reference. */
 int    mla_attn_launch_kernel(const mla_attn_args * args, void * stream);
+
+/* mla_attn_launch with the library's own scratch instead of `workspace` (args->workspace and workspace_size are ignored).
+ * No counterpart in the reference.  For callers that cannot allocate device memory around the call: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  The scratch is a fixed array of
+ * MLA_ATTN_STATIC_WORKSPACE_MAX bytes that every device the library runs on holds until the process ends; a call whose
+ * mla_attn_workspace_size() exceeds it returns MLA_ERR_TOO_LARGE (the headline decode step, 32 sequences x 128 heads x 8192
+ * keys, needs 43 MB).  Allocates nothing.  All calls on one device share the array: calls that overlap in time on the same
+ * device (different streams or threads) race; calls on one stream, or otherwise ordered, do not. */
+#define MLA_ATTN_STATIC_WORKSPACE_MAX ((size_t) 48 << 20)
+int    mla_attn_launch_static(const mla_attn_args * args, void * stream);
 
 /* dst[i] = src[i] for n_bytes (multiple of 16) */
 int mla_hbm_copy_launch(const void * src, void * dst, size_t n_bytes, void * stream);

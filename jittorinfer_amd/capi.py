@@ -8,6 +8,8 @@ MLA_TYPE_F32, MLA_TYPE_F16, MLA_TYPE_Q8_0, MLA_TYPE_BF16 = 0, 1, 8, 30
 MLA_FLAG_F16_ACC_STRICT = 1
 MLA_FLAG_UNIFORM_SPLITS = 2
 MLA_FLAG_BF16_DIRECT = 4
+MLA_ERR_TOO_LARGE = -7
+MLA_ATTN_STATIC_WORKSPACE_MAX = 48 << 20
 PAGE_TOKENS = 128
 ROW_BYTES = {MLA_TYPE_F16: 1152, MLA_TYPE_BF16: 1152, MLA_TYPE_Q8_0: 612}
 
@@ -55,7 +57,7 @@ def library():
         lib.mla_attn_plan.argtypes = [C.POINTER(MlaAttnArgs), C.POINTER(MlaPlanInfo)]
         lib.mla_attn_launch.restype = C.c_int
         lib.mla_attn_launch.argtypes = [C.POINTER(MlaAttnArgs), C.c_void_p]
-        for name in ("mla_attn_launch_partials", "mla_attn_launch_combine", "mla_attn_launch_kernel"):
+        for name in ("mla_attn_launch_partials", "mla_attn_launch_combine", "mla_attn_launch_kernel", "mla_attn_launch_static"):
             getattr(lib, name).restype = C.c_int
             getattr(lib, name).argtypes = [C.POINTER(MlaAttnArgs), C.c_void_p]
         lib.mla_hbm_copy_launch.restype = C.c_int

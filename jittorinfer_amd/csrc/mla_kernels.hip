@@ -660,6 +660,11 @@ __global__ void __launch_bounds__(256) mla_hbm_copy_kernel(const u32x4 * __restr
 // host side
 // ---------------------------------------------------------------------------------------------------------------
 
+// Scratch of mla_attn_launch_static: one copy per device, at the address hipGetSymbolAddress reports there (g_scratch_ptr).
+// In host code the array's name is only a handle for that lookup, never an address.
+static __device__ __align__(256) unsigned char scratch[MLA_ATTN_STATIC_WORKSPACE_MAX];
+static void * g_scratch_ptr[MLA_MAX_DEVICES];
+
 struct Plan {
     int    variant;  // 0 tiled, 1 strict f16
     int    wm, wd, rblk, n_row_blocks;
@@ -961,6 +966,36 @@ static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
 }
 
 int mla_attn_launch(const mla_attn_args * a, void * stream) { return launch_phases(a, stream, 7); }
+
+// mla_attn_launch for callers that cannot allocate a workspace: the split-K partials, the Q operand image, the mask extents
+// and the schedule live in a file-scope device array.  Each device holds its own copy of the array at its own address, which
+// hipGetSymbolAddress returns with that device current (looked up once per device, on the first call there); the kernels get
+// that address exactly as they get a caller's workspace.  Nothing in the array has to start at zero: every kernel writes what a
+// later kernel of the same call reads.  Calls that overlap in time on one device share the array and race.
+int mla_attn_launch_static(const mla_attn_args * a, void * stream) {
+    if (!a) return MLA_ERR_NULL;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int) e;
+    if (dev < 0 || dev >= MLA_MAX_DEVICES) return (int) hipErrorInvalidDevice;
+    void * ptr = g_scratch_ptr[dev];
+    if (!ptr) {   // (two threads that get here together look up the same address)
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int) e;
+        if (!ptr) return (int) hipErrorInvalidSymbol;
+        g_scratch_ptr[dev] = ptr;
+    }
+    mla_attn_args b = *a;
+    b.workspace      = nullptr;
+    b.workspace_size = 0;
+    Plan pl;
+    const int rc = make_plan(&b, &pl);
+    if (rc) return rc;
+    if (plan_ws(pl) > MLA_ATTN_STATIC_WORKSPACE_MAX) return MLA_ERR_TOO_LARGE;
+    b.workspace      = ptr;
+    b.workspace_size = MLA_ATTN_STATIC_WORKSPACE_MAX;
+    return launch_phases(&b, stream, 7);
+}
 int mla_attn_launch_partials(const mla_attn_args * a, void * stream) { return launch_phases(a, stream, 5); }
 int mla_attn_launch_kernel(const mla_attn_args * a, void * stream) { return launch_phases(a, stream, 1); }
 int mla_attn_launch_combine(const mla_attn_args * a, void * stream) { return launch_phases(a, stream, 2); }
