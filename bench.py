@@ -533,33 +533,37 @@ def main():
         torch.cuda.synchronize()
         graph.replay()          # untimed: first replay uploads the graph
         torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        graph.replay()          # K steps
-        torch.cuda.synchronize()
-        ms_per_step = (time.perf_counter() - t0) * 1e3 / a.steps
-        # spread of the same measurement: nine more replays of the K steps, each bracketed the same way
-        replays = [ms_per_step * 1e3]
-        for _ in range(9):
+        # the K steps are timed several times over (each replay bracketed by a synchronize on both sides) until at least
+        # 50 ms and 11 replays are on the clock; the reported step is the median replay, the spread is kept beside it
+        replays = []
+        while len(replays) < 11 or (sum(replays) * a.steps < 50e3 and len(replays) < 200):
             t0 = time.perf_counter()
             graph.replay()
             torch.cuda.synchronize()
             replays.append((time.perf_counter() - t0) * 1e6 / a.steps)
+        first_replay_us = replays[0]
         replays.sort()
-        step_stats = {"median": 0.5 * (replays[4] + replays[5]), "p10": replays[1], "p90": replays[8], "replays_of_k_steps": len(replays)}
+        n = len(replays)
+        ms_per_step = 0.5 * (replays[(n - 1) // 2] + replays[n // 2]) * 1e-3
+        step_stats = {"median": ms_per_step * 1e3, "p10": replays[n // 10], "p90": replays[(9 * n) // 10], "first": first_replay_us, "replays_of_k_steps": n}
     else:
         step_stats = None
 
-    # ---- the dominant kernel alone (the split-K decode kernel, without the Q pre-pack and the combine pass): HIP events
-    # on the launch stream around K back-to-back launches (the stream is in order, so this is K kernel durations plus the
-    # gaps between them)
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record(stream)
-    for i in range(a.steps):
-        step(i, lib.mla_attn_launch_kernel)   # the Q operand image in the workspace is the one the steps above wrote
-    e1.record(stream)
-    torch.cuda.synchronize()
-    kern_ms = e0.elapsed_time(e1) / a.steps
-    # spread over single launches: an event between every two launches of the same loop
+    # ---- the kernels that make up the node without the Q pre-pack: the split-K decode kernel and the combine pass, K times
+    # back to back with HIP events on the launch stream around them (the stream is in order, so this is K times their
+    # durations plus the gaps between them); then the decode kernel alone the same way, and with an event between every two
+    # launches for the spread
+    def timed(fns):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for i in range(a.steps):
+            for fn in fns:
+                step(i, fn)
+        e1.record(stream)
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / a.steps
+    node_ms = timed([lib.mla_attn_launch_kernel, lib.mla_attn_launch_combine])   # the Q operand image in the workspace is the one the steps above wrote
+    kern_ms = timed([lib.mla_attn_launch_kernel])
     marks = [torch.cuda.Event(enable_timing=True) for _ in range(a.steps + 1)]
     marks[0].record(stream)
     for i in range(a.steps):
@@ -569,18 +573,14 @@ def main():
     per_launch = sorted(marks[i].elapsed_time(marks[i + 1]) * 1e3 for i in range(a.steps))
     pick = lambda f: per_launch[min(len(per_launch) - 1, int(f * len(per_launch)))]
     kern_stats = {"mean": kern_ms * 1e3, "median": pick(0.5), "p10": pick(0.1), "p90": pick(0.9)}
-    # and whole steps with events (decode + combine)
-    e0.record(stream)
-    for i in range(a.steps):
-        step(i)
-    e1.record(stream)
-    torch.cuda.synchronize()
-    step_ms_events = e0.elapsed_time(e1) / a.steps
+    # and whole steps with events (pre-pack + decode + combine)
+    step_ms_events = timed([lib.mla_attn_launch])
 
     kv_bytes = a.batch * a.ctx * KV_ROW_BYTES
     flops = a.batch * a.ctx * a.heads * FLOP_PER_TOKEN_HEAD
     value = kv_bytes / (ms_per_step * 1e-3) / 1e9
-    achieved = kv_bytes / (kern_ms * 1e-3) / 1e9
+    achieved = kv_bytes / (node_ms * 1e-3) / 1e9          # decode kernel + combine pass
+    achieved_decode = kv_bytes / (kern_ms * 1e-3) / 1e9
 
     if a.copy_calibration > 0:
         dst_copy = torch.empty_like(pools[0])
@@ -598,8 +598,9 @@ def main():
 
     # HBM bytes of one decode-kernel launch, from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by what the same
     # counters read for the library's copy kernel; figures and commands in profiles/mla_decode_kernel_c3_pmc.md
-    traffic = None
+    traffic, traffic_source = None, None
     if a.batch == 32 and a.heads == 128 and a.ctx == 8192 and a.kv == "bf16":
+        traffic_source = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of the decode kernel, scaled by the copy kernel's readings: profiles/mla_decode_kernel_c3_pmc.md (a measured constant of that profile, not of this run)"
         fetch_kib, write_kib = (150524, 34048) if a.bf16_direct else (150051, 35072)   # KiB per dispatch, mean
         traffic = int(fetch_kib * 1024 * (294912 / 147466.0) + write_kib * 1024)
     res = {
@@ -617,10 +618,11 @@ def main():
         "tokens_per_s": a.batch / (ms_per_step * 1e-3),
         "pct_hbm_peak": 100.0 * value / HBM_PEAK_GBPS,
         "tflops": flops / (ms_per_step * 1e-3) / 1e12,
-        "roofline": {"bound": "hbm", "kernel": "mla_decode_kernel<%s>" % a.kv, "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic,
-                     "algorithmic_bytes_per_launch": kv_bytes, "kernel_us": kern_stats,
-                     "mfma_tflops": flops / (kern_ms * 1e-3) / 1e12},
+        "roofline": {"bound": "hbm", "kernel": "mla_decode_kernel<%s> + mla_attn_combine_kernel" % a.kv, "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic, "traffic_source": traffic_source,
+                     "algorithmic_bytes_per_launch": kv_bytes, "kernels_us": node_ms * 1e3,
+                     "decode_kernel_alone": {"achieved": achieved_decode, "frac": achieved_decode / HBM_PEAK_GBPS, "kernel_us": kern_stats},
+                     "mfma_tflops": flops / (node_ms * 1e-3) / 1e12},
         "cpu_baseline": cpu,
         "parity": parity,
     }

@@ -438,12 +438,13 @@ __device__ __forceinline__ void partial_slots(const KParams & p, int b, int row,
 
 // Log-sum-exp merge of the split-K partials: out = sum_c (O_c/l_c) l_c 2^(m_c - M) / sum_c l_c 2^(m_c - M).
 // Partials hold O_c/l_c as f16, laid out [seq][split][column/8][row][8].  One thread = one (row, group of 8 columns):
-// 16-byte loads, lanes along rows (contiguous in the partial layout), splits in groups of 8 so that all the loads of a
-// group are in flight together.  grid = (ceil(rows/32), ceil(dv/64), n_seq), block = 256 = 32 rows x 8 column groups.
+// 16-byte loads, splits in groups of 8 so that all the loads of a group are in flight together.  A wave covers 16 rows x 4
+// column groups: it reads runs of 256 bytes (16 rows of one column group are contiguous in the partial layout) and writes 128
+// contiguous bytes per row.  grid = (ceil(rows/16), ceil(dv/128), n_seq), block = 256 = 16 rows x 16 column groups.
 __global__ void __launch_bounds__(256) mla_attn_combine_kernel(const KParams p) {
     const int b = blockIdx.z;
-    const int row = blockIdx.x * 32 + (threadIdx.x & 31);
-    const int cg  = blockIdx.y * 8 + (threadIdx.x >> 5);
+    const int row = blockIdx.x * 16 + (threadIdx.x & 15);
+    const int cg  = blockIdx.y * 16 + (threadIdx.x >> 4);
     const int seq_len = p.block_table ? min(p.seq_lens[b], (int) p.bt_stride * MLA_PAGE_TOKENS) : (int) p.n_kv;
     if (row >= p.n_rows || cg * 8 >= p.dv_total) return;
     int slot0, nvalid, lrow;
@@ -927,7 +928,7 @@ static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
             hipLaunchKernelGGL(mla_attn_combine_f32_kernel, g, dim3(256), 0, st, kp, groups);
             return (int) hipGetLastError();
         }
-        dim3 g((unsigned) ((kp.n_rows + 31) / 32), (unsigned) ((dv + 63) / 64), (unsigned) a->n_seq);
+        dim3 g((unsigned) ((kp.n_rows + 15) / 16), (unsigned) ((dv + 127) / 128), (unsigned) a->n_seq);
         hipLaunchKernelGGL(mla_attn_combine_kernel, g, dim3(256), 0, st, kp);
         return (int) hipGetLastError();
     };
