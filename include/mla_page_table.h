@@ -14,6 +14,11 @@
  *   mla_page_table_seq_cp           llama_kv_cache_seq_cp, :242-283 (whole pages are shared by reference count; a partly
  *                                   filled last page is given to the destination as a fresh page whose rows must be copied:
  *                                   the copy is reported to the caller)
+ *   mla_page_table_seq_unshare      no call of its own in the reference: its cells carry a set of sequence ids each
+ *                                   (llama_kv_cell::seq_id, src/llama-kv-cache.h:12-27), so removing a suffix of one sequence
+ *                                   (:182-240) leaves the other's cells in place and the next find_slot takes other cells; with
+ *                                   pages the same sequence of calls -- copy, roll the copy or the source back into the
+ *                                   shared prefix, append -- needs the partly used shared page copied first
  *   mla_page_table_seq_keep         llama_kv_cache_seq_keep, :285-313
  *   mla_page_table_used_cells       llama_get_kv_cache_used_cells, :480-482 (tokens held, shared pages counted once)
  *   mla_page_table_fill_inputs      the mask builder of llama_set_inputs, src/llama-context.cpp:326-447: instead of the
@@ -34,7 +39,8 @@ extern "C" {
 #define MLA_PT_ERR_NO_SPACE   (-1) /* not enough free pages, or a sequence would exceed max_blocks pages */
 #define MLA_PT_ERR_BAD_ARG    (-2) /* sequence id out of range, negative position, null pointer */
 #define MLA_PT_ERR_NOT_CONTIG (-3) /* a position that neither extends its sequence by one nor overwrites an existing cell */
-#define MLA_PT_ERR_UNSUPPORTED (-4) /* seq_rm of a range that is neither a suffix nor the whole sequence */
+#define MLA_PT_ERR_UNSUPPORTED (-4) /* seq_rm of a range that is neither a suffix nor the whole sequence; find_slot: overwriting a row of
+                                       a page that another sequence maps too, or appending into one (see mla_page_table_seq_unshare) */
 
 typedef struct mla_page_table mla_page_table;
 
@@ -55,6 +61,13 @@ int mla_page_table_seq_rm(mla_page_table * t, int32_t seq_id, int32_t p0, int32_
  * device when the last page is only partly filled (copy_n_rows = 0 when there is none). */
 int mla_page_table_seq_cp(mla_page_table * t, int32_t seq_src, int32_t seq_dst, int32_t p0, int32_t p1,
                           int32_t * copy_src_row, int32_t * copy_dst_row, int32_t * copy_n_rows);
+
+/* Gives the sequence a private copy of its last page when that page is only partly used by it (length not a multiple of 128)
+ * and other sequences map it too -- the state a seq_cp followed by seq_rm(seq, p0 inside the shared pages) leaves.  Until then
+ * find_slot refuses to append to the sequence (MLA_PT_ERR_UNSUPPORTED): the new rows would overwrite the other sequences'.
+ * copy_src_row / copy_dst_row / copy_n_rows (each may be NULL) receive the row run the caller copies on the device
+ * (copy_n_rows = 0: nothing to do).  MLA_PT_ERR_NO_SPACE when no page is free. */
+int mla_page_table_seq_unshare(mla_page_table * t, int32_t seq_id, int32_t * copy_src_row, int32_t * copy_dst_row, int32_t * copy_n_rows);
 
 /* Removes every sequence but seq_id. */
 int mla_page_table_seq_keep(mla_page_table * t, int32_t seq_id);

@@ -74,6 +74,7 @@ def library():
         lib.mla_page_table_find_slot.argtypes = [C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p]
         lib.mla_page_table_seq_rm.argtypes = [C.c_void_p, C.c_int32, C.c_int32, C.c_int32]
         lib.mla_page_table_seq_cp.argtypes = [C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_int32] + [C.POINTER(C.c_int32)] * 3
+        lib.mla_page_table_seq_unshare.argtypes = [C.c_void_p, C.c_int32] + [C.POINTER(C.c_int32)] * 3
         lib.mla_page_table_seq_keep.argtypes = [C.c_void_p, C.c_int32]
         for name in ("mla_page_table_seq_len", "mla_page_table_free_pages", "mla_page_table_used_cells"):
             getattr(lib, name).restype = C.c_int32
@@ -385,6 +386,17 @@ class PageTable:
         rc = self._lib.mla_page_table_seq_cp(self._h, src, dst, p0, p1, C.byref(a), C.byref(b), C.byref(n))
         if rc != 0:
             raise ValueError("mla_page_table_seq_cp: %d" % rc)
+        return a.value, b.value, n.value
+
+    def seq_unshare(self, seq_id):
+        """Gives the sequence a private copy of a partly used last page that other sequences map too (after seq_cp + a roll-back
+        into the shared prefix); returns (src_row, dst_row, n_rows) to copy on the device (n_rows may be 0), None when no page is free."""
+        a, b, n = C.c_int32(0), C.c_int32(0), C.c_int32(0)
+        rc = self._lib.mla_page_table_seq_unshare(self._h, seq_id, C.byref(a), C.byref(b), C.byref(n))
+        if rc == -1:
+            return None
+        if rc != 0:
+            raise ValueError("mla_page_table_seq_unshare: %d" % rc)
         return a.value, b.value, n.value
 
     def seq_keep(self, seq_id):

@@ -70,8 +70,13 @@ int mla_page_table_find_slot(mla_page_table * t, int32_t n_tokens, const int32_t
         const int32_t s = seq_id[i];
         if (!seq_ok(t, s) || pos[i] < 0) return MLA_PT_ERR_BAD_ARG;
         if (pos[i] > new_len[s]) return MLA_PT_ERR_NOT_CONTIG;
-        if (pos[i] == new_len[s]) new_len[s]++;
-        // pages shared after seq_cp are full and read-only: overwriting a position inside one is not supported
+        if (pos[i] == new_len[s]) {
+            // appending into a page another sequence also maps (a copy that was rolled back into its shared prefix) would
+            // overwrite that sequence's rows: the caller gives the sequence a private tail first (mla_page_table_seq_unshare)
+            if (pos[i] == t->len[s] && pos[i] % PAGE != 0 && t->refcount[t->pages[s][pos[i] / PAGE]] > 1) return MLA_PT_ERR_UNSUPPORTED;
+            new_len[s]++;
+        }
+        // pages shared after seq_cp are read-only: overwriting a position inside one is not supported
         else if (pos[i] < t->len[s] && t->refcount[t->pages[s][pos[i] / PAGE]] > 1) return MLA_PT_ERR_UNSUPPORTED;
     }
     int64_t need = 0;
@@ -148,6 +153,25 @@ int mla_page_table_seq_cp(mla_page_table * t, int32_t seq_src, int32_t seq_dst, 
     return 0;
 }
 
+int mla_page_table_seq_unshare(mla_page_table * t, int32_t seq_id, int32_t * copy_src_row, int32_t * copy_dst_row, int32_t * copy_n_rows) {
+    if (!seq_ok(t, seq_id)) return MLA_PT_ERR_BAD_ARG;
+    if (copy_n_rows) *copy_n_rows = 0;
+    const int32_t tail = t->len[seq_id] % PAGE;
+    if (tail == 0 || t->pages[seq_id].empty()) return 0;          // the next token opens a fresh page anyway
+    const int32_t old = t->pages[seq_id].back();
+    if (t->refcount[old] == 1) return 0;                          // already private
+    if (t->free_list.empty()) return MLA_PT_ERR_NO_SPACE;
+    const int32_t p = t->free_list.back();
+    t->free_list.pop_back();
+    t->refcount[p] = 1;
+    t->refcount[old]--;                                           // (> 0: the other sequences keep it)
+    t->pages[seq_id].back() = p;
+    if (copy_src_row) *copy_src_row = old * PAGE;
+    if (copy_dst_row) *copy_dst_row = p * PAGE;
+    if (copy_n_rows) *copy_n_rows = tail;
+    return 0;
+}
+
 int mla_page_table_seq_keep(mla_page_table * t, int32_t seq_id) {
     if (!seq_ok(t, seq_id)) return MLA_PT_ERR_BAD_ARG;
     for (int32_t s = 0; s < t->n_seq_max; s++) if (s != seq_id) truncate(t, s, 0);
@@ -160,16 +184,15 @@ int32_t mla_page_table_free_pages(const mla_page_table * t) { return t ? (int32_
 
 int32_t mla_page_table_used_cells(const mla_page_table * t) {
     if (!t) return MLA_PT_ERR_BAD_ARG;
-    // tokens held, a page shared by several sequences counted once (it is full by construction)
-    int64_t cells = 0;
-    std::vector<char> seen(t->n_pages, 0);
+    // tokens held, a page shared by several sequences counted once, by the sequence that uses most of it
+    std::vector<int32_t> used(t->n_pages, 0);
     for (int32_t s = 0; s < t->n_seq_max; s++)
         for (size_t b = 0; b < t->pages[s].size(); b++) {
             const int32_t p = t->pages[s][b];
-            if (seen[p]) continue;
-            seen[p] = 1;
-            cells += std::min<int32_t>(PAGE, t->len[s] - (int32_t) b * PAGE);
+            used[p] = std::max(used[p], std::min<int32_t>(PAGE, t->len[s] - (int32_t) b * PAGE));
         }
+    int64_t cells = 0;
+    for (int32_t c : used) cells += c;
     return (int32_t) cells;
 }
 

@@ -144,3 +144,109 @@ def test_seq_cp_shares_full_pages_and_reports_the_tail_copy():
     assert t.seq_rm(0) and t.seq_len(0) == 0
     assert t.free_pages == 10 - 3                                               # the shared pages live on with sequence 1
     assert t.seq_keep(2) and t.free_pages == 10
+
+
+def test_append_after_rolling_back_into_a_shared_page_needs_a_private_copy():
+    """seq_cp shares full pages; rolling one of the two sequences back into a shared page and appending again must not
+    write into rows the other sequence still maps: find_slot refuses until seq_unshare has given the sequence its own page
+    (the reference's per-cell sequence sets make the same sequence of calls safe, src/llama-kv-cache.cpp:182-240, :347-404)."""
+    t = J.PageTable(8, 2, 4)
+    t.find_slot([0] * 200, list(range(200)))
+    t.seq_cp(0, 1)
+    bt, sl = t.fill_inputs([0, 1])
+    assert bt[0, 0] == bt[1, 0] and list(sl) == [200, 200]
+    assert t.seq_rm(0, 100, -1) and t.seq_len(0) == 100          # sequence 0 keeps 100 tokens of the shared page
+    free = t.free_pages
+    with pytest.raises(ValueError):
+        t.find_slot([0], [100])                                   # row 100 of the shared page is sequence 1's position 100
+    assert t.free_pages == free and t.seq_len(0) == 100
+    src, dst, n = t.seq_unshare(0)
+    bt2, sl2 = t.fill_inputs([0, 1])
+    assert n == 100 and src == bt[1, 0] * 128 and dst == bt2[0, 0] * 128 and bt2[0, 0] != bt2[1, 0]
+    assert t.free_pages == free - 1
+    rows = t.find_slot([0], [100])
+    assert rows[0] == bt2[0, 0] * 128 + 100
+    assert list(t.fill_inputs([1])[0][0, :2]) == list(bt[1, :2])  # sequence 1 is untouched
+    assert t.seq_unshare(0) == (0, 0, 0) and t.seq_unshare(1) == (0, 0, 0)   # nothing shared and partly used any more
+    # the copy rolled back instead of the source: same rule
+    t2 = J.PageTable(8, 2, 4)
+    t2.find_slot([0] * 130, list(range(130)))
+    t2.seq_cp(0, 1)
+    assert t2.seq_rm(1, 64, -1)
+    with pytest.raises(ValueError):
+        t2.find_slot([1], [64])
+    assert t2.seq_unshare(1)[2] == 64 and t2.find_slot([1], [64]) is not None
+    # a roll-back to a page boundary needs nothing: the next token opens a fresh page
+    t3 = J.PageTable(8, 2, 4)
+    t3.find_slot([0] * 300, list(range(300)))
+    t3.seq_cp(0, 1)
+    assert t3.seq_rm(1, 128, -1) and t3.seq_unshare(1) == (0, 0, 0) and t3.find_slot([1], [128]) is not None
+
+
+def test_random_copies_and_roll_backs_never_alias_rows():
+    """Contents model: every find_slot row gets a fresh value written, seq_cp / seq_unshare copy the row runs they report, and
+    after every operation each sequence must still read back exactly what was written at its own positions -- a page shared
+    by mistake, or a tail copy left out, shows up as a foreign value."""
+    rng = np.random.default_rng(7)
+    n_pages, n_seq, max_blocks = 48, 5, 8
+    t = J.PageTable(n_pages, n_seq, max_blocks)
+    store = np.full(n_pages * PAGE, -1, np.int64)
+    want = [[] for _ in range(n_seq)]
+    stamp = 0
+    refused = 0
+    for step in range(600):
+        op = rng.random()
+        s = int(rng.integers(0, n_seq))
+        if op < 0.55:
+            n = int(rng.choice([1, 1, 7, 100, 129]))
+            if rng.random() < 0.2 and want[s]:
+                pos = [len(want[s]) - 1]                      # re-decode the last position
+            else:
+                pos = list(range(len(want[s]), len(want[s]) + n))
+            try:
+                rows = t.find_slot([s] * len(pos), pos)
+            except ValueError:
+                refused += 1                                  # a shared page in the way: take a private copy and try again
+                cp = t.seq_unshare(s)
+                if cp is None:
+                    continue
+                a, b, k = cp
+                store[b:b + k] = store[a:a + k]
+                try:
+                    rows = t.find_slot([s] * len(pos), pos)
+                except ValueError:                            # an overwrite inside a shared full page stays unsupported
+                    assert pos[0] < len(want[s])
+                    continue
+            if rows is None:
+                continue
+            for r, p_ in zip(rows, pos):
+                stamp += 1
+                store[r] = stamp
+                if p_ == len(want[s]):
+                    want[s].append(stamp)
+                else:
+                    want[s][p_] = stamp
+        elif op < 0.75:
+            d = int(rng.integers(0, n_seq))
+            cp = None
+            try:
+                cp = t.seq_cp(s, d)
+            except ValueError:
+                continue
+            if cp is None:
+                continue
+            a, b, k = cp
+            store[b:b + k] = store[a:a + k]
+            if d != s:
+                want[d] = list(want[s])
+        else:
+            p0 = int(rng.integers(0, len(want[s]) + 1))
+            assert t.seq_rm(s, p0, -1)
+            del want[s][p0:]
+        bt, sl = t.fill_inputs(np.arange(n_seq))
+        for q in range(n_seq):
+            assert sl[q] == len(want[q])
+            if want[q]:
+                pos = np.arange(len(want[q]))
+                assert (store[bt[q, pos // PAGE] * PAGE + pos % PAGE] == np.array(want[q])).all(), (step, q)
+    assert refused > 0     # the case this test is for did occur
