@@ -83,8 +83,14 @@ void * ggml_backend_hip_mla_reg(void);
  * against the real headers without running anything on a GPU. */
 int mla_ggml_abi_table(int i, const char ** name, int64_t * value);
 
-/* no counterpart: supports_op's verdict for one FLASH_ATTN_EXT node plus the violated clause (for diagnostics). */
+/* no counterpart: supports_op's verdict for one node (any op) plus the violated clause (for diagnostics). */
 int mla_ggml_supports_node(const void * ggml_tensor_node, const char ** why);
+
+/* no counterpart: the argument block graph_compute builds for this node, handed to its launcher's check (mla_attn_plan,
+ * mla_kv_write_check, mla_copy_f32_check, mla_rope_check, mla_mul_mat_check): 0 when the launch would accept it.  The node
+ * must have the sources its op needs; nothing is read from the device.  supports_op makes the same call, so for every
+ * node it accepts this returns 0 -- tests/test_supports_op.py checks that over generated nodes. */
+int mla_ggml_node_launch_check(const void * ggml_tensor_node);
 
 /* no counterpart: frees a buffer obtained from this backend's buffer type when no ggml is present in the process
  * to do it (what ggml_backend_buffer_free does, ggml/src/ggml-backend.cpp). */

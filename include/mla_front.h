@@ -52,6 +52,10 @@ typedef struct mla_rope_args {
 } mla_rope_args;
 
 int mla_rope_launch(const mla_rope_args * args, void * stream);
+/* The argument checks of the launch alone (the value the launch would return before it touches the device): what the
+ * plugin's supports_op asks, in the place of ggml_backend_cann_supports_op's per-op clauses
+ * (ggml/src/ggml-cann/ggml-cann.cpp:1994-2145).  Only the low bits of the addresses are looked at. */
+int mla_rope_check(const mla_rope_args * args);
 
 typedef struct mla_mul_mat_args {
     int32_t      w_type;  /* type of src0: MLA_TYPE_F16 | MLA_TYPE_BF16 */
@@ -67,6 +71,7 @@ typedef struct mla_mul_mat_args {
 } mla_mul_mat_args;
 
 int mla_mul_mat_launch(const mla_mul_mat_args * args, void * stream);
+int mla_mul_mat_check(const mla_mul_mat_args * args);   /* as mla_rope_check */
 
 typedef struct mla_copy_args {
     const void * src;
@@ -77,6 +82,7 @@ typedef struct mla_copy_args {
 } mla_copy_args;
 
 int mla_copy_f32_launch(const mla_copy_args * args, void * stream);
+int mla_copy_f32_check(const mla_copy_args * args);     /* as mla_rope_check */
 
 #ifdef __cplusplus
 }

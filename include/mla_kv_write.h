@@ -49,6 +49,10 @@ typedef struct mla_kv_write_args {
 } mla_kv_write_args;
 
 int mla_kv_write_launch(const mla_kv_write_args * args, void * stream);
+/* The argument checks of the launch alone (the value the launch would return before it touches the device), for the
+ * plugin's supports_op (the reference's counterpart: ggml_backend_cann_supports_op, ggml/src/ggml-cann/ggml-cann.cpp:1994-2145).
+ * Only the low bits of the addresses are looked at. */
+int mla_kv_write_check(const mla_kv_write_args * args);
 
 #ifdef __cplusplus
 }

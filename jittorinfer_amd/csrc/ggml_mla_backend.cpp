@@ -272,6 +272,39 @@ const tensor * view_root(const tensor * t, size_t * offs) {
     return t;
 }
 
+// The address the launchers' alignment checks see: the tensor's own once it is allocated, before that a stand-in with the
+// same low bits (every ggml buffer aligns its tensors to at least 32 bytes, TENSOR_ALIGNMENT in ggml-impl.h, so the offset
+// of a view inside its root decides).
+const void * addr_of(const tensor * t) {
+    if (!t) return nullptr;
+    if (t->data) return t->data;
+    size_t offs;
+    (void) view_root(t, &offs);
+    return (const void *) ((uintptr_t) 1 << 20 | offs);
+}
+
+// Every *_ok function below does two things: the clauses only the graph can show (which tensor is a view of which, how
+// dst relates to the sources), and then the argument block graph_compute would pass, handed to the launcher's own check
+// -- so a node the device reports as supported is one the launch accepts (ggml_backend_sched sends a refused node to
+// the CPU backend instead, ggml-backend.cpp:820-846).
+
+void fill_attn_args(const tensor * dst, mla_attn_args * a) {
+    const tensor * q = dst->src[0], * k = dst->src[1], * v = dst->src[2], * mask = dst->src[3];
+    const tensor * bt = dst->src[4], * lens = dst->src[5];
+    memset(a, 0, sizeof(*a));
+    a->n_seq = (int32_t) q->ne[3]; a->n_head = (int32_t) q->ne[2]; a->n_tok = (int32_t) q->ne[1];
+    a->dk = 576; a->dv = (int32_t) v->ne[0];
+    a->q_type = MLA_TYPE_F32; a->kv_type = k->type;
+    memcpy(&a->scale, (const char *) dst->op_params + 0, 4);
+    memcpy(&a->max_bias, (const char *) dst->op_params + 4, 4);
+    memcpy(&a->logit_softcap, (const char *) dst->op_params + 8, 4);
+    a->q = addr_of(q); a->q_nb1 = (int64_t) q->nb[1]; a->q_nb2 = (int64_t) q->nb[2]; a->q_nb3 = (int64_t) q->nb[3];
+    a->kv = addr_of(k); a->kv_nb1 = (int64_t) k->nb[1]; a->kv_nb3 = k->ne[3] == 1 ? 0 : (int64_t) k->nb[3]; a->n_kv = k->ne[1];
+    if (mask) { a->mask = addr_of(mask); a->mask_nb1 = (int64_t) mask->nb[1]; a->mask_ne0 = mask->ne[0]; }
+    if (bt) { a->block_table = (const int32_t *) addr_of(bt); a->bt_stride = bt->ne[0]; a->seq_lens = (const int32_t *) addr_of(lens); }
+    a->dst = (float *) addr_of(dst); a->dst_nb1 = (int64_t) dst->nb[1];
+}
+
 // Fills `why` (if given) with the first violated clause of the node contract.
 bool mla_node_ok(const tensor * dst, const char ** why) {
     const char * dummy;
@@ -281,6 +314,7 @@ bool mla_node_ok(const tensor * dst, const char ** why) {
     if (!q || !k || !v) { *why = "missing q/k/v"; return false; }
     if (q->type != TYPE_F32 || q->nb[0] != 4) { *why = "q must be F32 with contiguous rows"; return false; }
     if (q->ne[0] != 576 || k->ne[0] != 576) { *why = "head size must be 576 (512 latent + 64 rope)"; return false; }
+    if (q->ne[1] < 1 || q->ne[2] < 1 || q->ne[3] < 1 || q->ne[1] > 0x7fffffff || q->ne[2] > 0x7fffffff || q->ne[3] > 0x7fffffff) { *why = "q must have 1 .. 2^31-1 tokens, heads and sequences"; return false; }
     if (k->type != TYPE_F16 && k->type != TYPE_BF16 && k->type != TYPE_Q8_0) { *why = "k must be F16, BF16 or Q8_0"; return false; }
     if (k->ne[2] != 1) { *why = "MLA has a single latent KV head"; return false; }
     if (k->nb[0] != type_size(k->type)) { *why = "k rows must be contiguous"; return false; }
@@ -299,32 +333,65 @@ bool mla_node_ok(const tensor * dst, const char ** why) {
         if (mask->type != TYPE_F16 || !is_contiguous(mask) || mask->ne[2] != 1 || mask->ne[3] != 1) { *why = "mask must be contiguous F16 2-D"; return false; }
         if (mask->ne[1] < q->ne[1]) { *why = "mask has fewer rows than query tokens"; return false; }
     }
-    float max_bias;
-    memcpy(&max_bias, (const char *) dst->op_params + 4, 4);
-    if (max_bias > 0.0f && !mask) { *why = "max_bias needs a mask"; return false; }
     if ((bt != nullptr) != (lens != nullptr)) { *why = "block table and sequence lengths come together"; return false; }
     if (bt) {
         if (bt->type != TYPE_I32 || lens->type != TYPE_I32 || !is_contiguous(bt) || !is_contiguous(lens)) { *why = "block table / lengths must be contiguous I32"; return false; }
         if (bt->ne[1] != q->ne[3] || nelements(lens) != q->ne[3]) { *why = "block table / lengths must have one row per sequence"; return false; }
         if (k->ne[3] != 1) { *why = "with a block table k is the page pool [576, rows, 1, 1]"; return false; }
-        if (k->ne[1] % MLA_PAGE_TOKENS) { *why = "page pool must hold whole 128-token pages"; return false; }
+        // every position a sequence can reach has a mask column
+        if (mask && mask->ne[0] < bt->ne[0] * MLA_PAGE_TOKENS) { *why = "mask narrower than the block table's reach"; return false; }
     } else {
         if (k->ne[3] != q->ne[3] && k->ne[3] != 1) { *why = "k batch must equal q batch or be 1"; return false; }
         if (mask && mask->ne[0] < k->ne[1]) { *why = "mask narrower than n_kv"; return false; }
     }
-    return true;
+    mla_attn_args a;
+    fill_attn_args(dst, &a);
+    mla_attn_plan_info info;
+    switch (mla_attn_plan(&a, &info)) {
+        case 0: return true;
+        case MLA_ERR_BAD_ALIGNMENT: *why = "q, dst rows must be 16-byte aligned, k rows 16-byte (Q8_0: 2-byte) aligned and hold 576 values"; return false;
+        case MLA_ERR_UNSUPPORTED: *why = "max_bias needs a mask"; return false;
+        default: *why = "shape outside the launch limits (rows <= 2^31-1, page pool of whole 128-token pages, <= 2^23 pages per sequence)"; return false;
+    }
 }
 
 // The KV cache write of llm_attn_mla (src/llama-graph-attn.cpp:236-241): CPY of f32 rows [576, n_tok] into a contiguous
 // view of a BF16 / F16 / Q8_0 cache with the same number of elements; and SCATTER_UPDATE (ggml.c:3203-3223): rows of
 // `updates` (cache type or F32) into rows indices[i] of a [576, n_rows] cache.
+void fill_kv_cpy_args(const tensor * op, mla_kv_write_args * a) {
+    const tensor * src = op->src[0];
+    memset(a, 0, sizeof(*a));
+    a->n_tok = (int32_t) src->ne[1]; a->src_type = MLA_TYPE_F32; a->kv_type = op->type;
+    a->src = addr_of(src); a->src_nb1 = (int64_t) src->nb[1];
+    a->kv = const_cast<void *>(addr_of(op)); a->kv_nb1 = op->type == TYPE_Q8_0 ? 612 : 1152; a->n_kv_rows = src->ne[1]; a->row0 = 0;
+}
+
+void fill_kv_scatter_args(const tensor * op, mla_kv_write_args * a) {
+    const tensor * var = op->src[0], * idx = op->src[1], * upd = op->src[2];
+    memset(a, 0, sizeof(*a));
+    a->n_tok = (int32_t) upd->ne[1]; a->src_type = upd->type == TYPE_F32 ? MLA_TYPE_F32 : var->type; a->kv_type = var->type;
+    a->src = addr_of(upd); a->src_nb1 = (int64_t) upd->nb[1];
+    a->kv = const_cast<void *>(addr_of(var)); a->kv_nb1 = (int64_t) var->nb[1]; a->n_kv_rows = var->ne[1];
+    a->rows = addr_of(idx); a->rows_type = idx->type == TYPE_I64 ? 1 : 0;
+}
+
+const char * kv_write_why(int rc) {
+    return rc == MLA_ERR_BAD_ALIGNMENT ? "rows must be 16-byte aligned (Q8_0 cache: 2-byte, Q8_0 row copies: 4-byte)"
+         : rc == MLA_ERR_BAD_SHAPE     ? "rows shorter than 576 values"
+                                       : "refused by the launch check";
+}
+
 bool kv_cpy_ok(const tensor * op, const char ** why) {
     const char * dummy; if (!why) why = &dummy;
     const tensor * src = op->src[0];
     if (!src || src->type != TYPE_F32 || src->ne[0] != 576 || src->ne[2] != 1 || src->ne[3] != 1) { *why = "source must be F32 [576, n_tok]"; return false; }
-    if (src->nb[0] != 4 || (src->nb[1] & 15)) { *why = "source rows must be dense and 16-byte aligned"; return false; }
+    if (src->nb[0] != 4 || src->ne[1] > 0x7fffffff) { *why = "source rows must be dense, at most 2^31-1 of them"; return false; }
     if (op->type != TYPE_BF16 && op->type != TYPE_F16 && op->type != TYPE_Q8_0) { *why = "destination must be BF16, F16 or Q8_0"; return false; }
     if (!is_contiguous(op) || nelements(op) != nelements(src)) { *why = "destination must be a contiguous view with as many elements"; return false; }
+    mla_kv_write_args a;
+    fill_kv_cpy_args(op, &a);
+    const int rc = mla_kv_write_check(&a);
+    if (rc) { *why = kv_write_why(rc); return false; }
     return true;
 }
 
@@ -336,19 +403,45 @@ bool kv_scatter_ok(const tensor * op, const char ** why) {
     if (var->type != TYPE_BF16 && var->type != TYPE_F16 && var->type != TYPE_Q8_0) { *why = "cache must be BF16, F16 or Q8_0"; return false; }
     if (upd->type != var->type && upd->type != TYPE_F32) { *why = "updates must have the cache type or be F32"; return false; }
     if ((idx->type != TYPE_I32 && idx->type != TYPE_I64) || !is_contiguous(idx) || idx->ne[0] != upd->ne[1]) { *why = "indices must be contiguous I32/I64, one per update row"; return false; }
+    if (var->nb[0] != type_size(var->type) || upd->nb[0] != type_size(upd->type)) { *why = "cache and update rows must be dense"; return false; }
+    if (var->ne[1] > 0x7fffffff || upd->ne[1] > 0x7fffffff) { *why = "too many rows"; return false; }
+    {   // the node's result is the cache itself, updated in place (ggml.c:3203-3223 makes it a view of src[0])
+        size_t oo, vo;
+        if (view_root(op, &oo) != view_root(var, &vo) || oo != vo) { *why = "the node must be a view of the cache"; return false; }
+    }
+    mla_kv_write_args a;
+    fill_kv_scatter_args(op, &a);
+    const int rc = mla_kv_write_check(&a);
+    if (rc) { *why = kv_write_why(rc); return false; }
     return true;
 }
 
 // The nodes llm_attn_mla and the DeepSeek-V2 graph put either side of the attention node
 // (src/llama-graph-deepseek2.cpp:216-233, src/llama-graph-attn.cpp:264-277, :303-323): CONT and CONCAT of f32 tensors with
-// dense rows, ROPE (normal / NeoX pairing, f32), MUL_MAT of an F16 / BF16 src0 with an f32 src1.
+// dense rows, ROPE (normal / NeoX pairing, f32), and the two per-head products with the halves of kv_b: the absorb
+// product q_nope . wk_b ([n_tok x 128] . [128 x 512] per head) and the un-absorb product wv_b . kqv ([n_tok x 512] . [512 x 128]).
 bool f32_rows(const tensor * t) { return t && t->type == TYPE_F32 && t->nb[0] == 4 && !(t->nb[1] & 3) && !(t->nb[2] & 3) && !(t->nb[3] & 3); }
+
+void fill_copy_args(const void * src, const size_t * src_nb, const int64_t * ne, const void * dst, const size_t * dst_nb, mla_copy_args * a) {
+    a->src = src; a->dst = const_cast<void *>(dst);
+    for (int i = 0; i < 4; i++) { a->ne[i] = ne[i]; a->src_nb[i] = (int64_t) src_nb[i]; a->dst_nb[i] = (int64_t) dst_nb[i]; }
+}
+
+// CONT: the destination is walked in the source's shape -- same element order (ggml_cont_2d)
+void fill_cont_args(const tensor * op, mla_copy_args * a) {
+    const tensor * src = op->src[0];
+    const size_t dnb[4] = { 4, (size_t) src->ne[0] * 4, (size_t) (src->ne[0] * src->ne[1]) * 4, (size_t) (src->ne[0] * src->ne[1] * src->ne[2]) * 4 };
+    fill_copy_args(addr_of(src), src->nb, src->ne, addr_of(op), dnb, a);
+}
 
 bool cont_ok(const tensor * op, const char ** why) {
     const char * dummy; if (!why) why = &dummy;
     const tensor * src = op->src[0];
     if (!f32_rows(src)) { *why = "source must be F32 with dense rows"; return false; }
     if (op->type != TYPE_F32 || !is_contiguous(op) || nelements(op) != nelements(src)) { *why = "destination must be contiguous F32 with as many elements"; return false; }
+    mla_copy_args a;
+    fill_cont_args(op, &a);
+    if (mla_copy_f32_check(&a)) { *why = "refused by the launch check"; return false; }
     return true;
 }
 
@@ -360,21 +453,51 @@ bool concat_ok(const tensor * op, const char ** why) {
     if (dim < 0 || dim > 3) { *why = "bad dimension"; return false; }
     for (int i = 0; i < 4; i++)
         if (i == dim ? op->ne[i] != a->ne[i] + b->ne[i] : (op->ne[i] != a->ne[i] || op->ne[i] != b->ne[i])) { *why = "shapes do not concatenate"; return false; }
+    mla_copy_args c;
+    fill_copy_args(addr_of(a), a->nb, a->ne, addr_of(op), op->nb, &c);
+    if (mla_copy_f32_check(&c)) { *why = "refused by the launch check"; return false; }
+    fill_copy_args(addr_of(b), b->nb, b->ne, (const char *) addr_of(op) + (size_t) a->ne[dim] * op->nb[dim], op->nb, &c);
+    if (mla_copy_f32_check(&c)) { *why = "refused by the launch check"; return false; }
     return true;
+}
+
+void fill_rope_args(const tensor * op, mla_rope_args * a) {
+    const tensor * x = op->src[0];
+    memset(a, 0, sizeof(*a));
+    a->src = addr_of(x); a->dst = const_cast<void *>(addr_of(op)); a->pos = (const int32_t *) addr_of(op->src[1]);
+    a->freq_factors = op->src[2] ? (const float *) addr_of(op->src[2]) : nullptr;
+    for (int i = 0; i < 4; i++) { a->ne[i] = x->ne[i]; a->src_nb[i] = (int64_t) x->nb[i]; a->dst_nb[i] = (int64_t) op->nb[i]; }
+    int32_t prm[11]; memcpy(prm, op->op_params, sizeof(prm));   // ggml.c:3431-3441
+    a->n_dims = prm[1]; a->mode = prm[2]; a->n_ctx_orig = prm[4];
+    memcpy(&a->freq_base, prm + 5, 4); memcpy(&a->freq_scale, prm + 6, 4); memcpy(&a->ext_factor, prm + 7, 4);
+    memcpy(&a->attn_factor, prm + 8, 4); memcpy(&a->beta_fast, prm + 9, 4); memcpy(&a->beta_slow, prm + 10, 4);
 }
 
 bool rope_ok(const tensor * op, const char ** why) {
     const char * dummy; if (!why) why = &dummy;
     const tensor * x = op->src[0], * pos = op->src[1], * ff = op->src[2];
-    int32_t prm[5]; memcpy(prm, op->op_params, sizeof(prm));
     if (!f32_rows(x) || !f32_rows(op)) { *why = "source and destination must be F32 with dense rows"; return false; }
     for (int i = 0; i < 4; i++) if (op->ne[i] != x->ne[i]) { *why = "shape mismatch"; return false; }
     if (!pos || pos->type != TYPE_I32 || !is_contiguous(pos) || nelements(pos) != x->ne[2]) { *why = "positions must be contiguous I32, one per token"; return false; }
-    if (prm[2] != MLA_ROPE_MODE_NORM && prm[2] != MLA_ROPE_MODE_NEOX) { *why = "only the normal and the NeoX pairing"; return false; }
-    if (prm[1] <= 0 || (prm[1] & 1) || prm[1] > x->ne[0] || prm[1] > 512) { *why = "n_dims must be even, <= ne0 and <= 512"; return false; }
-    if (ff && (ff->type != TYPE_F32 || !is_contiguous(ff) || ff->ne[0] < prm[1] / 2)) { *why = "frequency factors must be contiguous F32 [n_dims/2]"; return false; }
-    if (x->ne[2] > 65535 || x->ne[3] > 65535) { *why = "too many tokens for one launch"; return false; }
-    return true;
+    mla_rope_args a;
+    fill_rope_args(op, &a);
+    if (ff && (ff->type != TYPE_F32 || !is_contiguous(ff) || ff->ne[0] < a.n_dims / 2)) { *why = "frequency factors must be contiguous F32 [n_dims/2]"; return false; }
+    switch (mla_rope_check(&a)) {
+        case 0: return true;
+        case MLA_ERR_UNSUPPORTED: *why = "only the normal and the NeoX pairing"; return false;
+        default: *why = "n_dims must be even, <= ne0 and <= 512; at most 65535 tokens per launch"; return false;
+    }
+}
+
+void fill_mul_mat_args(const tensor * op, mla_mul_mat_args * a) {
+    const tensor * w = op->src[0], * x = op->src[1];
+    memset(a, 0, sizeof(*a));
+    a->w_type = w->type; a->w = addr_of(w); a->x = addr_of(x); a->dst = const_cast<void *>(addr_of(op));
+    a->K = w->ne[0]; a->N = w->ne[1]; a->w_ne2 = w->ne[2]; a->w_ne3 = w->ne[3];
+    a->M = x->ne[1]; a->ne2 = x->ne[2]; a->ne3 = x->ne[3];
+    a->w_nb1 = (int64_t) w->nb[1]; a->w_nb2 = (int64_t) w->nb[2]; a->w_nb3 = (int64_t) w->nb[3];
+    a->x_nb1 = (int64_t) x->nb[1]; a->x_nb2 = (int64_t) x->nb[2]; a->x_nb3 = (int64_t) x->nb[3];
+    a->d_nb1 = (int64_t) op->nb[1]; a->d_nb2 = (int64_t) op->nb[2]; a->d_nb3 = (int64_t) op->nb[3];
 }
 
 bool mul_mat_ok(const tensor * op, const char ** why) {
@@ -383,12 +506,20 @@ bool mul_mat_ok(const tensor * op, const char ** why) {
     if (!w || !x) { *why = "missing operand"; return false; }
     if ((w->type != TYPE_F16 && w->type != TYPE_BF16) || w->nb[0] != 2) { *why = "src0 must be F16 or BF16 with dense rows"; return false; }
     if (x->type != TYPE_F32 || x->nb[0] != 4 || op->type != TYPE_F32 || op->nb[0] != 4) { *why = "src1 and dst must be F32 with dense rows"; return false; }
-    if (w->ne[0] != x->ne[0] || w->ne[0] < 16 || w->ne[0] % 16) { *why = "K must be a multiple of 16"; return false; }
+    if (w->ne[0] != x->ne[0]) { *why = "src0 and src1 rows differ in length"; return false; }
     if (op->ne[0] != w->ne[1] || op->ne[1] != x->ne[1] || op->ne[2] != x->ne[2] || op->ne[3] != x->ne[3]) { *why = "dst must be [N, M, ne12, ne13]"; return false; }
-    if (w->ne[2] < 1 || w->ne[3] < 1 || x->ne[2] % w->ne[2] || x->ne[3] % w->ne[3]) { *why = "src0 does not broadcast over src1's batches"; return false; }
-    for (int i = 1; i < 4; i++) if ((w->nb[i] & 15) || (x->nb[i] & 15) || (op->nb[i] & 3)) { *why = "rows must be 16-byte aligned"; return false; }
-    if (x->ne[2] * x->ne[3] > 65535) { *why = "too many batches for one launch"; return false; }
-    return true;
+    // only the two products the kernels were built and measured for: one small matrix per head, one side of it the
+    // latent width.  A model's other F16 / BF16 products (wq, wo, the FFN) stay with the backend that owns their weights.
+    const int64_t K = w->ne[0], N = w->ne[1];
+    if (!((K == 512 && N <= 512) || (N == 512 && K <= 512)) || w->ne[2] != x->ne[2] || w->ne[3] != 1) { *why = "only the per-head absorb ([K<=512] x 512) and un-absorb (512 x [N<=512]) products"; return false; }
+    mla_mul_mat_args a;
+    fill_mul_mat_args(op, &a);
+    switch (mla_mul_mat_check(&a)) {
+        case 0: return true;
+        case MLA_ERR_BAD_ALIGNMENT: *why = "rows must be 16-byte aligned"; return false;
+        case MLA_ERR_UNSUPPORTED: *why = "K must be a multiple of 16"; return false;
+        default: *why = "too many batches or rows for one launch"; return false;
+    }
 }
 
 bool device_supports_op(backend_device *, const tensor * op) {
@@ -442,23 +573,12 @@ int compute_flash_attn(backend_ctx * ctx, const tensor * dst) {
                   k ? k->name : "-", k ? (long long) k->ne[0] : 0, k ? (long long) k->ne[1] : 0, k ? (long long) k->ne[2] : 0, k ? (long long) k->ne[3] : 0);
         return STATUS_FAILED;
     }
-    const tensor * q = dst->src[0], * k = dst->src[1], * v = dst->src[2], * mask = dst->src[3];
-    const tensor * bt = dst->src[4], * lens = dst->src[5];
+    const tensor * q = dst->src[0], * k = dst->src[1], * v = dst->src[2], * bt = dst->src[4];
     if (!q->data || !k->data || !dst->data || v->data != k->data) { log_error("node '%s': operands not allocated, or v does not alias k", dst->name); return STATUS_FAILED; }
+    for (int i = 3; i < 6; i++) if (dst->src[i] && !dst->src[i]->data) { log_error("node '%s': operands not allocated", dst->name); return STATUS_FAILED; }
 
     mla_attn_args a;
-    memset(&a, 0, sizeof(a));
-    a.n_seq = (int32_t) q->ne[3]; a.n_head = (int32_t) q->ne[2]; a.n_tok = (int32_t) q->ne[1];
-    a.dk = 576; a.dv = (int32_t) v->ne[0];
-    a.q_type = MLA_TYPE_F32; a.kv_type = k->type;
-    memcpy(&a.scale, (const char *) dst->op_params + 0, 4);
-    memcpy(&a.max_bias, (const char *) dst->op_params + 4, 4);
-    memcpy(&a.logit_softcap, (const char *) dst->op_params + 8, 4);
-    a.q = q->data; a.q_nb1 = (int64_t) q->nb[1]; a.q_nb2 = (int64_t) q->nb[2]; a.q_nb3 = (int64_t) q->nb[3];
-    a.kv = k->data; a.kv_nb1 = (int64_t) k->nb[1]; a.kv_nb3 = k->ne[3] == 1 ? 0 : (int64_t) k->nb[3]; a.n_kv = k->ne[1];
-    if (mask) { a.mask = mask->data; a.mask_nb1 = (int64_t) mask->nb[1]; a.mask_ne0 = mask->ne[0]; }
-    if (bt) { a.block_table = (const int32_t *) bt->data; a.bt_stride = bt->ne[0]; a.seq_lens = (const int32_t *) lens->data; }
-    a.dst = (float *) dst->data; a.dst_nb1 = (int64_t) dst->nb[1];
+    fill_attn_args(dst, &a);
     if (ctx->f16_strict && k->type == TYPE_F16 && !bt) a.flags |= MLA_FLAG_F16_ACC_STRICT;
     if (ctx->bf16_direct) a.flags |= MLA_FLAG_BF16_DIRECT;
 
@@ -480,32 +600,22 @@ int compute_flash_attn(backend_ctx * ctx, const tensor * dst) {
 int compute_kv_write(backend_ctx * ctx, const tensor * dst) {
     const char * why = nullptr;
     mla_kv_write_args a;
-    memset(&a, 0, sizeof(a));
     if (dst->op == OP_CPY) {
         if (!kv_cpy_ok(dst, &why)) { log_error("CPY node '%s' rejected: %s", dst->name, why); return STATUS_FAILED; }
-        const tensor * src = dst->src[0];
-        a.n_tok = (int32_t) src->ne[1]; a.src_type = MLA_TYPE_F32; a.kv_type = dst->type;
-        a.src = src->data; a.src_nb1 = (int64_t) src->nb[1];
-        a.kv = dst->data; a.kv_nb1 = dst->type == TYPE_Q8_0 ? 612 : 1152; a.n_kv_rows = src->ne[1]; a.row0 = 0;
+        if (!dst->src[0]->data || !dst->data) { log_error("node '%s': operands not allocated", dst->name); return STATUS_FAILED; }
+        fill_kv_cpy_args(dst, &a);
     } else {
         if (!kv_scatter_ok(dst, &why)) { log_error("SCATTER_UPDATE node '%s' rejected: %s", dst->name, why); return STATUS_FAILED; }
-        const tensor * var = dst->src[0], * idx = dst->src[1], * upd = dst->src[2];
-        a.n_tok = (int32_t) upd->ne[1]; a.src_type = upd->type == TYPE_F32 ? MLA_TYPE_F32 : var->type; a.kv_type = var->type;
-        a.src = upd->data; a.src_nb1 = (int64_t) upd->nb[1];
-        a.kv = var->data; a.kv_nb1 = (int64_t) var->nb[1]; a.n_kv_rows = var->ne[1];
-        a.rows = idx->data; a.rows_type = idx->type == TYPE_I64 ? 1 : 0;
+        for (int i = 0; i < 3; i++) if (!dst->src[i]->data) { log_error("node '%s': operands not allocated", dst->name); return STATUS_FAILED; }
+        fill_kv_scatter_args(dst, &a);
     }
-    if (!a.src || !a.kv) { log_error("node '%s': operands not allocated", dst->name); return STATUS_FAILED; }
     const int rc = mla_kv_write_launch(&a, ctx->stream);
     if (rc != 0) { log_error("mla_kv_write_launch failed for node '%s': %d", dst->name, rc); return STATUS_FAILED; }
     return STATUS_SUCCESS;
 }
 
-int launch_copy(backend_ctx * ctx, const tensor * node, const void * src, const size_t * src_nb, const int64_t * ne, void * dst, const size_t * dst_nb) {
-    mla_copy_args a;
-    a.src = src; a.dst = dst;
-    for (int i = 0; i < 4; i++) { a.ne[i] = ne[i]; a.src_nb[i] = (int64_t) src_nb[i]; a.dst_nb[i] = (int64_t) dst_nb[i]; }
-    const int rc = mla_copy_f32_launch(&a, ctx->stream);
+int launch_copy(backend_ctx * ctx, const tensor * node, const mla_copy_args * a) {
+    const int rc = mla_copy_f32_launch(a, ctx->stream);
     if (rc != 0) { log_error("mla_copy_f32_launch failed for node '%s': %d", node->name, rc); return STATUS_FAILED; }
     return STATUS_SUCCESS;
 }
@@ -516,44 +626,32 @@ int compute_front(backend_ctx * ctx, const tensor * dst) {
     if (!dst->data) { log_error("node '%s': destination not allocated", dst->name); return STATUS_FAILED; }
     if (dst->op == OP_CONT) {
         if (!cont_ok(dst, &why)) { log_error("CONT node '%s' rejected: %s", dst->name, why); return STATUS_FAILED; }
-        const tensor * src = dst->src[0];   // the destination is walked in the source's shape: same element order (ggml_cont_2d)
-        const size_t dnb[4] = { 4, (size_t) src->ne[0] * 4, (size_t) (src->ne[0] * src->ne[1]) * 4, (size_t) (src->ne[0] * src->ne[1] * src->ne[2]) * 4 };
-        return launch_copy(ctx, dst, src->data, src->nb, src->ne, dst->data, dnb);
+        mla_copy_args a;
+        fill_cont_args(dst, &a);
+        return launch_copy(ctx, dst, &a);
     }
     if (dst->op == OP_CONCAT) {
         if (!concat_ok(dst, &why)) { log_error("CONCAT node '%s' rejected: %s", dst->name, why); return STATUS_FAILED; }
         const tensor * a = dst->src[0], * b = dst->src[1];
         int32_t dim; memcpy(&dim, dst->op_params, 4);
-        const int st = launch_copy(ctx, dst, a->data, a->nb, a->ne, dst->data, dst->nb);
+        mla_copy_args c;
+        fill_copy_args(a->data, a->nb, a->ne, dst->data, dst->nb, &c);
+        const int st = launch_copy(ctx, dst, &c);
         if (st != STATUS_SUCCESS) return st;
-        return launch_copy(ctx, dst, b->data, b->nb, b->ne, (char *) dst->data + (size_t) a->ne[dim] * dst->nb[dim], dst->nb);
+        fill_copy_args(b->data, b->nb, b->ne, (char *) dst->data + (size_t) a->ne[dim] * dst->nb[dim], dst->nb, &c);
+        return launch_copy(ctx, dst, &c);
     }
     if (dst->op == OP_ROPE) {
         if (!rope_ok(dst, &why)) { log_error("ROPE node '%s' rejected: %s", dst->name, why); return STATUS_FAILED; }
-        const tensor * x = dst->src[0];
         mla_rope_args a;
-        memset(&a, 0, sizeof(a));
-        a.src = x->data; a.dst = dst->data; a.pos = (const int32_t *) dst->src[1]->data;
-        a.freq_factors = dst->src[2] ? (const float *) dst->src[2]->data : nullptr;
-        for (int i = 0; i < 4; i++) { a.ne[i] = x->ne[i]; a.src_nb[i] = (int64_t) x->nb[i]; a.dst_nb[i] = (int64_t) dst->nb[i]; }
-        int32_t prm[11]; memcpy(prm, dst->op_params, sizeof(prm));   // ggml.c:3431-3441
-        a.n_dims = prm[1]; a.mode = prm[2]; a.n_ctx_orig = prm[4];
-        memcpy(&a.freq_base, prm + 5, 4); memcpy(&a.freq_scale, prm + 6, 4); memcpy(&a.ext_factor, prm + 7, 4);
-        memcpy(&a.attn_factor, prm + 8, 4); memcpy(&a.beta_fast, prm + 9, 4); memcpy(&a.beta_slow, prm + 10, 4);
+        fill_rope_args(dst, &a);
         const int rc = mla_rope_launch(&a, ctx->stream);
         if (rc != 0) { log_error("mla_rope_launch failed for node '%s': %d", dst->name, rc); return STATUS_FAILED; }
         return STATUS_SUCCESS;
     }
     if (!mul_mat_ok(dst, &why)) { log_error("MUL_MAT node '%s' rejected: %s", dst->name, why); return STATUS_FAILED; }
-    const tensor * w = dst->src[0], * x = dst->src[1];
     mla_mul_mat_args a;
-    memset(&a, 0, sizeof(a));
-    a.w_type = w->type; a.w = w->data; a.x = x->data; a.dst = dst->data;
-    a.K = w->ne[0]; a.N = w->ne[1]; a.w_ne2 = w->ne[2]; a.w_ne3 = w->ne[3];
-    a.M = x->ne[1]; a.ne2 = x->ne[2]; a.ne3 = x->ne[3];
-    a.w_nb1 = (int64_t) w->nb[1]; a.w_nb2 = (int64_t) w->nb[2]; a.w_nb3 = (int64_t) w->nb[3];
-    a.x_nb1 = (int64_t) x->nb[1]; a.x_nb2 = (int64_t) x->nb[2]; a.x_nb3 = (int64_t) x->nb[3];
-    a.d_nb1 = (int64_t) dst->nb[1]; a.d_nb2 = (int64_t) dst->nb[2]; a.d_nb3 = (int64_t) dst->nb[3];
+    fill_mul_mat_args(dst, &a);
     const int rc = mla_mul_mat_launch(&a, ctx->stream);
     if (rc != 0) { log_error("mla_mul_mat_launch failed for node '%s': %d", dst->name, rc); return STATUS_FAILED; }
     return STATUS_SUCCESS;
@@ -808,8 +906,42 @@ void mla_ggml_buffer_free(void * buffer) {
 
 int mla_ggml_supports_node(const void * node, const char ** why) {
     const tensor * t = (const tensor *) node;
-    if (t->op != OP_FLASH_ATTN_EXT) { if (why) *why = "not a FLASH_ATTN_EXT node"; return 0; }
-    return mla_node_ok(t, why) ? 1 : 0;
+    const char * dummy; if (!why) why = &dummy;
+    *why = "";
+    if (is_noop(t->op)) return 1;
+    switch (t->op) {
+        case OP_FLASH_ATTN_EXT: return mla_node_ok(t, why) ? 1 : 0;
+        case OP_CPY: return kv_cpy_ok(t, why) ? 1 : 0;
+        case OP_SCATTER_UPDATE: return kv_scatter_ok(t, why) ? 1 : 0;
+        case OP_CONT: return cont_ok(t, why) ? 1 : 0;
+        case OP_CONCAT: return concat_ok(t, why) ? 1 : 0;
+        case OP_ROPE: return rope_ok(t, why) ? 1 : 0;
+        case OP_MUL_MAT: return mul_mat_ok(t, why) ? 1 : 0;
+        default: *why = "op not taken by this backend"; return 0;
+    }
+}
+
+int mla_ggml_node_launch_check(const void * node) {
+    const tensor * t = (const tensor *) node;
+    switch (t->op) {
+        case OP_FLASH_ATTN_EXT: { mla_attn_args a; fill_attn_args(t, &a); mla_attn_plan_info info; return mla_attn_plan(&a, &info); }
+        case OP_CPY: { mla_kv_write_args a; fill_kv_cpy_args(t, &a); return mla_kv_write_check(&a); }
+        case OP_SCATTER_UPDATE: { mla_kv_write_args a; fill_kv_scatter_args(t, &a); return mla_kv_write_check(&a); }
+        case OP_CONT: { mla_copy_args a; fill_cont_args(t, &a); return mla_copy_f32_check(&a); }
+        case OP_CONCAT: {
+            const tensor * x = t->src[0], * y = t->src[1];
+            int32_t dim; memcpy(&dim, t->op_params, 4);
+            mla_copy_args c;
+            fill_copy_args(addr_of(x), x->nb, x->ne, addr_of(t), t->nb, &c);
+            const int rc = mla_copy_f32_check(&c);
+            if (rc) return rc;
+            fill_copy_args(addr_of(y), y->nb, y->ne, (const char *) addr_of(t) + (size_t) x->ne[dim] * t->nb[dim], t->nb, &c);
+            return mla_copy_f32_check(&c);
+        }
+        case OP_ROPE: { mla_rope_args a; fill_rope_args(t, &a); return mla_rope_check(&a); }
+        case OP_MUL_MAT: { mla_mul_mat_args a; fill_mul_mat_args(t, &a); return mla_mul_mat_check(&a); }
+        default: return is_noop(t->op) ? 0 : MLA_ERR_UNSUPPORTED;
+    }
 }
 
 }  // extern "C"

@@ -397,7 +397,7 @@ inline bool al16(const void * ptr) { return ((uintptr_t) ptr & 15) == 0; }
 
 }  // namespace
 
-extern "C" int mla_rope_launch(const mla_rope_args * a, void * stream) {
+extern "C" int mla_rope_check(const mla_rope_args * a) {
     if (!a) return MLA_ERR_NULL;
     for (int i = 0; i < 4; i++) if (a->ne[i] < 0) return MLA_ERR_BAD_SHAPE;
     if (a->n_dims <= 0 || (a->n_dims & 1) || a->n_dims > a->ne[0] || a->n_dims > 2 * ROPE_MAX_PAIRS) return MLA_ERR_BAD_SHAPE;
@@ -408,6 +408,13 @@ extern "C" int mla_rope_launch(const mla_rope_args * a, void * stream) {
     if (a->ne[2] > 65535 || a->ne[3] > 65535) return MLA_ERR_BAD_SHAPE;
     for (int i = 1; i < 4; i++) if ((a->src_nb[i] & 3) || (a->dst_nb[i] & 3)) return MLA_ERR_BAD_ALIGNMENT;
     if (((uintptr_t) a->src & 3) || ((uintptr_t) a->dst & 3)) return MLA_ERR_BAD_ALIGNMENT;
+    return 0;
+}
+
+extern "C" int mla_rope_launch(const mla_rope_args * a, void * stream) {
+    const int rc = mla_rope_check(a);
+    if (rc) return rc;
+    if (a->ne[0] * a->ne[1] * a->ne[2] * a->ne[3] == 0) return 0;
 
     RopeP p;
     p.src = (const char *) a->src; p.dst = (char *) a->dst;
@@ -439,7 +446,7 @@ extern "C" int mla_rope_launch(const mla_rope_args * a, void * stream) {
     return (int) hipGetLastError();
 }
 
-extern "C" int mla_mul_mat_launch(const mla_mul_mat_args * a, void * stream) {
+extern "C" int mla_mul_mat_check(const mla_mul_mat_args * a) {
     if (!a) return MLA_ERR_NULL;
     if (a->w_type != MLA_TYPE_F16 && a->w_type != MLA_TYPE_BF16) return MLA_ERR_BAD_TYPE;
     if (a->K < 0 || a->N < 0 || a->M < 0 || a->w_ne2 < 1 || a->w_ne3 < 1 || a->ne2 < 0 || a->ne3 < 0) return MLA_ERR_BAD_SHAPE;
@@ -452,6 +459,13 @@ extern "C" int mla_mul_mat_launch(const mla_mul_mat_args * a, void * stream) {
         (a->x_nb3 & 15) || ((uintptr_t) a->dst & 3) || (a->d_nb1 & 3) || (a->d_nb2 & 3) || (a->d_nb3 & 3))
         return MLA_ERR_BAD_ALIGNMENT;
     if (a->w_nb1 < a->K * 2 || a->x_nb1 < a->K * 4 || a->d_nb1 < a->N * 4) return MLA_ERR_BAD_SHAPE;
+    return 0;
+}
+
+extern "C" int mla_mul_mat_launch(const mla_mul_mat_args * a, void * stream) {
+    const int rc = mla_mul_mat_check(a);
+    if (rc) return rc;
+    if (a->N * a->M * a->ne2 * a->ne3 == 0) return 0;
     MmP p;
     p.w = (const char *) a->w; p.x = (const char *) a->x; p.dst = (char *) a->dst;
     p.K = a->K; p.N = a->N; p.M = a->M; p.ne2 = a->ne2;
@@ -464,19 +478,24 @@ extern "C" int mla_mul_mat_launch(const mla_mul_mat_args * a, void * stream) {
     return (int) e;
 }
 
-extern "C" int mla_copy_f32_launch(const mla_copy_args * a, void * stream) {
+extern "C" int mla_copy_f32_check(const mla_copy_args * a) {
     if (!a) return MLA_ERR_NULL;
     for (int i = 0; i < 4; i++) if (a->ne[i] < 0) return MLA_ERR_BAD_SHAPE;
     if (a->src_nb[0] != 4 || a->dst_nb[0] != 4) return MLA_ERR_BAD_SHAPE;
+    if (a->ne[0] * a->ne[1] * a->ne[2] * a->ne[3] == 0) return 0;
+    if (!a->src || !a->dst) return MLA_ERR_NULL;
+    for (int i = 1; i < 4; i++) if ((a->src_nb[i] & 3) || (a->dst_nb[i] & 3)) return MLA_ERR_BAD_ALIGNMENT;
+    if (((uintptr_t) a->src & 3) || ((uintptr_t) a->dst & 3)) return MLA_ERR_BAD_ALIGNMENT;
+    return 0;
+}
+
+extern "C" int mla_copy_f32_launch(const mla_copy_args * a, void * stream) {
+    const int rc = mla_copy_f32_check(a);
+    if (rc) return rc;
     const int64_t n = a->ne[0] * a->ne[1] * a->ne[2] * a->ne[3];
     if (n == 0) return 0;
-    if (!a->src || !a->dst) return MLA_ERR_NULL;
     bool v4 = a->ne[0] % 4 == 0 && al16(a->src) && al16(a->dst);
-    for (int i = 1; i < 4; i++) {
-        if ((a->src_nb[i] & 3) || (a->dst_nb[i] & 3)) return MLA_ERR_BAD_ALIGNMENT;
-        v4 = v4 && !(a->src_nb[i] & 15) && !(a->dst_nb[i] & 15);
-    }
-    if (((uintptr_t) a->src & 3) || ((uintptr_t) a->dst & 3)) return MLA_ERR_BAD_ALIGNMENT;
+    for (int i = 1; i < 4; i++) v4 = v4 && !(a->src_nb[i] & 15) && !(a->dst_nb[i] & 15);
     CopyP p;
     p.src = (const char *) a->src; p.dst = (char *) a->dst;
     p.ne0 = v4 ? a->ne[0] / 4 : a->ne[0]; p.ne1 = a->ne[1]; p.ne2 = a->ne[2];

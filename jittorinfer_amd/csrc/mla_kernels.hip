@@ -585,7 +585,8 @@ __global__ void __launch_bounds__(576) mla_f16_strict_kernel(const KParams p, co
         const int n = min(STRICT_CHUNK, (int) p.n_kv - c0);
         for (int k = tid; k < n; k += nth) {
             const int ic = c0 + k;
-            const float mv = mask_row ? slope * f16_bits_to_f32(*(const unsigned short *) (mask_row + (int64_t) ic * 2)) : 0.0f;
+            // (a key past the mask's width counts as masked, as in the other kernels)
+            const float mv = !mask_row ? 0.0f : ic < p.mask_ne0 ? slope * f16_bits_to_f32(*(const unsigned short *) (mask_row + (int64_t) ic * 2)) : -INFINITY;
             float sv = -INFINITY;   // ggml-cpu skips a key whose mask value is -inf (ggml-cpu.c:12041-12044)
             if (mv != -INFINITY) {
                 sv = srow[ic] * scale_eff;

@@ -98,7 +98,7 @@ template <int KVT> hipError_t launch_kvt(const WParams & p, bool convert, hipStr
 
 }  // namespace
 
-extern "C" int mla_kv_write_launch(const mla_kv_write_args * a, void * stream) {
+extern "C" int mla_kv_write_check(const mla_kv_write_args * a) {
     if (!a) return MLA_ERR_NULL;
     if (a->n_tok < 0 || a->n_kv_rows < 0) return MLA_ERR_BAD_SHAPE;
     if (a->kv_type != MLA_TYPE_BF16 && a->kv_type != MLA_TYPE_F16 && a->kv_type != MLA_TYPE_Q8_0) return MLA_ERR_BAD_TYPE;
@@ -118,6 +118,14 @@ extern "C" int mla_kv_write_launch(const mla_kv_write_args * a, void * stream) {
     if (a->block_table) {
         if (!a->seq_ids || !a->positions || a->bt_stride < 1) return MLA_ERR_NULL;
     } else if (!a->rows && (a->row0 < 0 || a->row0 + a->n_tok > a->n_kv_rows)) return MLA_ERR_BAD_SHAPE;
+    return 0;
+}
+
+extern "C" int mla_kv_write_launch(const mla_kv_write_args * a, void * stream) {
+    const int rc = mla_kv_write_check(a);
+    if (rc) return rc;
+    if (a->n_tok == 0) return 0;
+    const bool convert = a->src_type == MLA_TYPE_F32;
 
     WParams p;
     p.src = (const char *) a->src; p.src_nb1 = a->src_nb1;

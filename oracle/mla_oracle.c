@@ -28,9 +28,9 @@
  * the reference asserts DV == DK (ggml-cpu.c:11943) and output columns are independent, so with DV == DK
  * this is the reference's computation and with DV < DK it is its first DV output columns.
  *
- * Pinning: see tests/test_oracle.py (closed forms, brute force, exhaustive conversions) and
- * tests/test_oracle_vs_ref.py (differential against the reference's own compiled ggml-cpu, when
- * oracle/_ref is built).  Golden vectors produced by the compiled reference are in tests/golden/.
+ * Pinning: see tests/test_oracle.py (closed forms, brute force, exhaustive conversions, and the
+ * differential against the reference's own compiled ggml-cpu when oracle/_ref is built) and
+ * tests/test_golden.py (the vectors in tests/golden/, produced by the compiled reference).
  */
 #include <math.h>
 #include <stdint.h>

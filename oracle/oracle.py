@@ -409,6 +409,10 @@ def _ref_front():
                                        C.POINTER(RopeParams), C.c_void_p, C.c_int]
         r.ref_mla_unabsorb.restype = C.c_int
         r.ref_mla_unabsorb.argtypes = [C.c_char_p, C.c_int, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]
+        r.ref_mla_layer.restype = C.c_int
+        r.ref_mla_layer.argtypes = [C.c_char_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int64, C.c_int64, C.c_int, C.c_void_p, C.c_void_p,
+                                    C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p,
+                                    C.c_int]
         r._front_ready = True
     return r
 
@@ -464,3 +468,31 @@ def ref_mla_unabsorb(kqv, wkv_b, w_type, n_head, so_path=None, n_threads=4):
     if rc != 0:
         raise RuntimeError("ref_mla_unabsorb failed: %d" % rc)
     return out
+
+
+def ref_mla_layer(mode, k_type, w_type, n_head, n_ctx, steps, wkv_b, kq_scale, so_path=None, v_type=TYPE_F16, block_table=None,
+                  n_threads=4):
+    """Steps of llm_attn_mla on one KV cache.  mode 0: the unfused graph the reference emits (src/llama-graph-attn.cpp:233-323)
+    on its ggml-cpu, with a K cache of k_type and a transposed V cache of v_type; mode 1 / 2: the one-node form on the backend
+    plugin at so_path under ggml_backend_sched, the cache written by CPY (1) or as a page pool by SCATTER_UPDATE with a block
+    table (2).  steps = [(q f32 [n_tok, n_head, 192], kv_cur f32 [n_tok, 576]), ...], appended to the one sequence in order.
+    Returns (outputs [f32 [n_tok, 128 * n_head] per step], on_backend flags per step, cache bytes after the last step)."""
+    n_tok = np.array([q.shape[0] for q, _ in steps], dtype=np.int32)
+    kv_head = np.concatenate([[0], np.cumsum(n_tok)[:-1]]).astype(np.int32)
+    q = np.ascontiguousarray(np.concatenate([np.asarray(q, dtype=np.float32).reshape(-1) for q, _ in steps]))
+    kv = np.ascontiguousarray(np.concatenate([np.asarray(k, dtype=np.float32).reshape(-1) for _, k in steps]))
+    for qq, kk in steps:
+        assert qq.shape[1:] == (n_head, 192) and kk.shape == (qq.shape[0], 576)
+    wkv_b = np.ascontiguousarray(wkv_b)
+    out = np.full((int(n_tok.sum()), n_head * 128), np.nan, dtype=np.float32)
+    where = np.zeros(len(steps), dtype=np.int32)
+    cache = np.zeros((n_ctx, 612 if k_type == TYPE_Q8_0 else 1152), dtype=np.uint8)
+    bt = None if block_table is None else np.ascontiguousarray(block_table, dtype=np.int32)
+    rc = _ref_front().ref_mla_layer(_so(so_path), mode, k_type, v_type, w_type, n_head, n_ctx, len(steps), n_tok.ctypes.data,
+                                    kv_head.ctypes.data, q.ctypes.data, kv.ctypes.data, wkv_b.ctypes.data, kq_scale,
+                                    None if bt is None else bt.ctypes.data, 0 if bt is None else bt.shape[-1], out.ctypes.data,
+                                    where.ctypes.data, cache.ctypes.data, n_threads)
+    if rc != 0:
+        raise RuntimeError("ref_mla_layer(mode %d) failed: %d" % (mode, rc))
+    ends = np.cumsum(n_tok)
+    return [out[e - n:e] for e, n in zip(ends, n_tok)], where, cache

@@ -12,8 +12,12 @@
  *   ref_rope / ref_mul_mat        one ROPE / MUL_MAT node on ggml-cpu, or on a loaded backend
  *   ref_mla_q_states / _unabsorb  the query side and the output side of llm_attn_mla around the attention node
  *                                 (src/llama-graph-attn.cpp:264-277, :303-323), on ggml-cpu or on a loaded backend
+ *   ref_mla_layer                 whole steps of llm_attn_mla on one KV cache: the graph the reference emits (unfused,
+ *                                 src/llama-graph-attn.cpp:233-323) on ggml-cpu, or the one-node form on a loaded backend
+ *                                 through ggml_backend_sched
  *   ref_abi_table                 sizeof/offsetof/enum facts of the structs a backend must mirror
  */
+#include <math.h>
 #include <stddef.h>
 #include <stdint.h>
 #include <stdio.h>
@@ -494,6 +498,213 @@ int ref_mla_unabsorb(const char * so_path, int w_type, int64_t H, int64_t n_tok,
         if (!rc) ggml_backend_tensor_get(o, out, 0, ggml_nbytes(o));
     }
     front_close(&rt);
+    return rc;
+}
+
+/* ------------------------------------------------------------------ one attention layer, several steps on one cache
+ *
+ * mode 0  the graph llm_attn_mla builds today (src/llama-graph-attn.cpp:233-323), on the reference's ggml-cpu: the new
+ *         rows copied into the K cache (k_type, [576, n_ctx]) and, transposed, into the V cache (v_type, [n_ctx, 512]);
+ *         q_states = concat(q_nope . wk_b, q_pe); kq = mul_mat(k, q) at f32 precision; soft_max_ext with the f32 mask
+ *         and kq_scale; kqv = mul_mat(v, kq); mul_mat with wv_b; permute; cont_2d.
+ * mode 1  the one-node form on the backend loaded from so_path, scheduled by ggml_backend_sched over {that backend, CPU}
+ *         as llama_decode schedules its graphs (ggml-backend.cpp:1493-1587): ONE latent cache (k_type, [576, n_ctx]) in
+ *         the backend's buffer written by the same ggml_cpy; q_states as above; ggml_flash_attn_ext(q_states, k,
+ *         v = the first 512 columns of k, f16 mask) at f32 precision; the first 512 floats of its rows -> wv_b -> permute
+ *         -> cont_2d.
+ * mode 2  as mode 1 with the cache as a pool of 128-row pages: the new rows go in by ggml_scatter_update (ggml.c:3203-3223)
+ *         at rows block_table[pos / 128] * 128 + pos % 128, the node carries the block table and the sequence length in
+ *         src[4] / src[5], and only a step of several tokens carries a (causal) mask.
+ *
+ * One sequence; step s appends n_tok[s] tokens at positions kv_head[s] .. (every step's kv_head is the number of tokens
+ * before it).  q: per step f32 [n_tok][H][128 + 64] (q_nope | q_pe, q_pe already rotated), kv_cur: per step f32
+ * [n_tok][576], both concatenated over the steps; wkv_b = w_type [512, H * (128 + 128)] as the model stores it.
+ * out: per step f32 [n_tok][128 * H], concatenated.  on_backend[s] (modes 1, 2): bit 0 = the cache write ran on the
+ * loaded backend, bit 1 = the attention node, bit 2 = every MUL_MAT, bit 3 = CONCAT, bit 4 = CONT.
+ * cache_out (may be NULL): the K / latent cache bytes after the last step.
+ */
+struct layer_io {
+    struct ggml_tensor *q, *kv_cur, *mask, *idx, *bt, *lens, *out, *write, *fa;
+};
+
+static struct ggml_tensor * layer_q_states(struct ggml_context * c, struct ggml_tensor * tq, struct ggml_tensor * tw, int64_t H, int64_t n_tok) {
+    const int64_t NOPE = 128, ROPE = 64, LORA = 512;
+    struct ggml_tensor * q_nope = ggml_view_3d(c, tq, NOPE, H, n_tok, ggml_row_size(tq->type, NOPE + ROPE), ggml_row_size(tq->type, (NOPE + ROPE) * H), 0);
+    struct ggml_tensor * q_pe   = ggml_view_3d(c, tq, ROPE, H, n_tok, ggml_row_size(tq->type, NOPE + ROPE), ggml_row_size(tq->type, (NOPE + ROPE) * H),
+                                               ggml_row_size(tq->type, NOPE));
+    struct ggml_tensor * wk_b   = ggml_view_3d(c, tw, NOPE, LORA, H, ggml_row_size(tw->type, NOPE), ggml_row_size(tw->type, NOPE * LORA), 0);
+    q_nope = ggml_mul_mat(c, wk_b, ggml_permute(c, q_nope, 0, 2, 1, 3));
+    return ggml_concat(c, q_nope, ggml_permute(c, q_pe, 0, 2, 1, 3), 0); /* [576, n_tok, H] */
+}
+
+static struct ggml_tensor * layer_unabsorb(struct ggml_context * c, struct ggml_tensor * kqv /* [512, n_tok, H] */, struct ggml_tensor * tw, int64_t H, int64_t n_tok) {
+    const int64_t NOPE = 128, LORA = 512, DV = 128;
+    struct ggml_tensor * wv_b = ggml_view_3d(c, tw, LORA, DV, H, ggml_row_size(tw->type, LORA), ggml_row_size(tw->type, LORA * DV),
+                                             ggml_row_size(tw->type, LORA * NOPE * H));
+    struct ggml_tensor * o = ggml_mul_mat(c, wv_b, kqv);
+    return ggml_cont_2d(c, ggml_permute(c, o, 0, 2, 1, 3), DV * H, n_tok);
+}
+
+int ref_mla_layer(const char * so_path, int mode, int k_type, int v_type, int w_type, int64_t H, int64_t n_ctx, int n_steps,
+                  const int32_t * n_tok_s, const int32_t * kv_head_s, const float * q, const float * kv_cur, const void * wkv_b,
+                  float kq_scale, const int32_t * block_table, int64_t max_blocks, float * out, int32_t * on_backend,
+                  void * cache_out, int n_threads) {
+    const int64_t D = 576, LORA = 512, QW = 192, DV = 128;
+    const enum ggml_type kt = (enum ggml_type) k_type, vt = (enum ggml_type) v_type, wt = (enum ggml_type) w_type;
+    if (mode < 0 || mode > 2 || (mode == 2 && (!block_table || n_ctx % 128))) return -1;
+    ggml_backend_t be = NULL, cpu = NULL;
+    if (mode == 0) {
+        be = ggml_backend_cpu_init();
+        if (be) ggml_backend_cpu_set_n_threads(be, n_threads);
+    } else {
+        ggml_backend_reg_t reg = ggml_backend_load(so_path);
+        if (!reg) return -10;
+        if (ggml_backend_reg_dev_count(reg) < 1) return -11;
+        be  = ggml_backend_dev_init(ggml_backend_reg_dev_get(reg, 0), NULL);
+        cpu = ggml_backend_init_by_type(GGML_BACKEND_DEVICE_TYPE_CPU, NULL);
+        if (!cpu) { if (be) ggml_backend_free(be); return -15; }
+    }
+    if (!be) return -12;
+    int                   rc = 0;
+    ggml_backend_sched_t  sched = NULL;
+    struct ggml_context * g = NULL;
+    /* the cache(s) and the weight live in the executor's buffer for the whole run (src/llama-kv-cache.cpp:82-90, :153-158) */
+    struct ggml_init_params ipk = { ggml_tensor_overhead() * 8, NULL, true };
+    struct ggml_context *   ck  = ggml_init(ipk);
+    struct ggml_tensor *    k_l = ggml_new_tensor_1d(ck, kt, D * n_ctx);
+    struct ggml_tensor *    v_l = mode == 0 ? ggml_new_tensor_1d(ck, vt, LORA * n_ctx) : NULL;
+    struct ggml_tensor *    tw  = ggml_new_tensor_2d(ck, wt, LORA, H * (128 + DV));
+    ggml_backend_buffer_t   bufk = ggml_backend_alloc_ctx_tensors(ck, be);
+    if (!bufk) { rc = -18; goto done; }
+    ggml_backend_buffer_clear(bufk, 0);
+    ggml_backend_tensor_set(tw, wkv_b, 0, ggml_nbytes(tw));
+    if (mode != 0) {
+        ggml_backend_t             backends[2] = { be, cpu };
+        ggml_backend_buffer_type_t bufts[2]    = { ggml_backend_get_default_buffer_type(be), ggml_backend_get_default_buffer_type(cpu) };
+        sched = ggml_backend_sched_new(backends, bufts, 2, GGML_DEFAULT_GRAPH_SIZE, false);
+        if (!sched) { rc = -16; goto done; }
+    }
+
+    for (int s = 0; s < n_steps; s++) {
+        const int64_t n_tok = n_tok_s[s], kv_head = kv_head_s[s];
+        int64_t       n_kv  = GGML_PAD(kv_head + n_tok, 32); /* llama_kv_cache_get_padding without flash attention */
+        if (n_kv > n_ctx) n_kv = n_ctx;
+        if (kv_head + n_tok > n_ctx || (mode == 2 && kv_head + n_tok > max_blocks * 128)) { rc = -2; goto done; }
+        struct ggml_init_params ip = { ggml_tensor_overhead() * 96 + ggml_graph_overhead(), NULL, true };
+        g = ggml_init(ip);
+        struct ggml_cgraph * gf = ggml_new_graph(g);
+        struct layer_io io;
+        memset(&io, 0, sizeof(io));
+        io.q      = ggml_new_tensor_2d(g, GGML_TYPE_F32, QW * H, n_tok);
+        io.kv_cur = ggml_new_tensor_2d(g, GGML_TYPE_F32, D, n_tok);
+        ggml_set_input(io.q);
+        ggml_set_input(io.kv_cur);
+        const int64_t mask_w = mode == 2 ? max_blocks * 128 : n_kv;
+        if (mode != 2 || n_tok > 1) {
+            io.mask = ggml_new_tensor_2d(g, mode == 0 ? GGML_TYPE_F32 : GGML_TYPE_F16, mask_w, GGML_PAD(n_tok, GGML_KQ_MASK_PAD));
+            ggml_set_input(io.mask);
+        }
+        struct ggml_tensor * k;
+        if (mode == 2) {
+            io.idx  = ggml_new_tensor_1d(g, GGML_TYPE_I32, n_tok);
+            io.bt   = ggml_new_tensor_2d(g, GGML_TYPE_I32, max_blocks, 1);
+            io.lens = ggml_new_tensor_1d(g, GGML_TYPE_I32, 1);
+            ggml_set_input(io.idx); ggml_set_input(io.bt); ggml_set_input(io.lens);
+            k = io.write = ggml_scatter_update(g, ggml_reshape_2d(g, k_l, D, n_ctx), io.idx, io.kv_cur);
+        } else {
+            io.write = ggml_cpy(g, io.kv_cur, ggml_view_1d(g, k_l, n_tok * D, ggml_row_size(kt, D) * kv_head));
+            ggml_build_forward_expand(gf, io.write);
+            k = ggml_view_2d(g, k_l, D, n_kv, ggml_row_size(kt, D), 0);
+        }
+        struct ggml_tensor * q_states = layer_q_states(g, io.q, tw, H, n_tok);
+        if (mode == 0) {
+            struct ggml_tensor * v_cache_view = ggml_view_2d(g, v_l, n_tok, LORA, n_ctx * ggml_element_size(v_l), kv_head * ggml_element_size(v_l));
+            struct ggml_tensor * v_cur        = ggml_transpose(g, ggml_view_2d(g, io.kv_cur, LORA, n_tok, ggml_row_size(GGML_TYPE_F32, D), 0));
+            ggml_build_forward_expand(gf, ggml_cpy(g, v_cur, v_cache_view));
+            struct ggml_tensor * v  = ggml_view_2d(g, v_l, n_kv, LORA, ggml_element_size(v_l) * n_ctx, 0);
+            struct ggml_tensor * q2 = ggml_view_2d(g, q_states, D, H * n_tok, ggml_row_size(GGML_TYPE_F32, D), 0);
+            struct ggml_tensor * kq = ggml_mul_mat(g, k, q2);
+            ggml_mul_mat_set_prec(kq, GGML_PREC_F32);
+            kq = ggml_view_3d(g, kq, n_kv, n_tok, H, ggml_row_size(GGML_TYPE_F32, n_kv), ggml_row_size(GGML_TYPE_F32, n_kv * n_tok), 0);
+            kq = ggml_soft_max_ext(g, kq, io.mask, kq_scale, 0.0f);
+            kq = ggml_view_2d(g, kq, n_kv, n_tok * H, ggml_row_size(GGML_TYPE_F32, n_kv), 0);
+            struct ggml_tensor * kqv = ggml_mul_mat(g, v, kq);
+            kqv    = ggml_view_3d(g, kqv, LORA, n_tok, H, ggml_row_size(GGML_TYPE_F32, LORA), ggml_row_size(GGML_TYPE_F32, LORA * n_tok), 0);
+            io.out = layer_unabsorb(g, kqv, tw, H, n_tok);
+        } else {
+            struct ggml_tensor * v = ggml_view_2d(g, k, LORA, k->ne[1], k->nb[1], 0);
+            io.fa = ggml_flash_attn_ext(g, q_states, k, v, io.mask, kq_scale, 0.0f, 0.0f);
+            ggml_flash_attn_ext_set_prec(io.fa, GGML_PREC_F32);
+            io.fa->src[4] = io.bt;
+            io.fa->src[5] = io.lens;
+            /* [576, H, n_tok]: the first 512 floats of every row, seen as [512, n_tok, H] */
+            struct ggml_tensor * kqv = ggml_view_3d(g, io.fa, LORA, H, n_tok, io.fa->nb[1], io.fa->nb[2], 0);
+            io.out = layer_unabsorb(g, ggml_permute(g, kqv, 0, 2, 1, 3), tw, H, n_tok);
+        }
+        ggml_set_output(io.out);
+        ggml_build_forward_expand(gf, io.out);
+
+        ggml_backend_buffer_t bufg = NULL;
+        if (mode == 0) {
+            bufg = ggml_backend_alloc_ctx_tensors(g, be);
+            if (!bufg) { rc = -18; goto done; }
+        } else {
+            ggml_backend_sched_reset(sched);
+            if (!ggml_backend_sched_alloc_graph(sched, gf)) { rc = -16; goto done; }
+            int32_t where = 0x1c;
+            for (int i = 0; i < ggml_graph_n_nodes(gf); i++) {
+                struct ggml_tensor * n  = ggml_graph_node(gf, i);
+                const int            on = ggml_backend_sched_get_tensor_backend(sched, n) == be;
+                if (n == io.write && on) where |= 1;
+                if (n == io.fa && on) where |= 2;
+                if (n->op == GGML_OP_MUL_MAT && !on) where &= ~4;
+                if (n->op == GGML_OP_CONCAT && !on) where &= ~8;
+                if (n->op == GGML_OP_CONT && !on) where &= ~16;
+            }
+            if (on_backend) on_backend[s] = where;
+        }
+        ggml_backend_tensor_set(io.q, q, 0, ggml_nbytes(io.q));
+        ggml_backend_tensor_set(io.kv_cur, kv_cur, 0, ggml_nbytes(io.kv_cur));
+        if (io.mask) { /* causal over the cells of this one sequence: cell j holds position j (src/llama-context.cpp:364-404) */
+            const int64_t rows = io.mask->ne[1];
+            void *        md   = malloc((size_t) rows * mask_w * 4);
+            for (int64_t i = 0; i < rows; i++)
+                for (int64_t j = 0; j < mask_w; j++) {
+                    const int open = i < n_tok && j <= kv_head + i;
+                    if (mode == 0) ((float *) md)[i * mask_w + j] = open ? 0.0f : -INFINITY;
+                    else ((uint16_t *) md)[i * mask_w + j] = open ? 0 : 0xfc00;
+                }
+            ggml_backend_tensor_set(io.mask, md, 0, ggml_nbytes(io.mask));
+            free(md);
+        }
+        if (mode == 2) {
+            int32_t * rows = (int32_t *) malloc(sizeof(int32_t) * n_tok);
+            for (int64_t i = 0; i < n_tok; i++) rows[i] = block_table[(kv_head + i) / 128] * 128 + (int32_t) ((kv_head + i) % 128);
+            const int32_t len = (int32_t) (kv_head + n_tok);
+            ggml_backend_tensor_set(io.idx, rows, 0, ggml_nbytes(io.idx));
+            ggml_backend_tensor_set(io.bt, block_table, 0, ggml_nbytes(io.bt));
+            ggml_backend_tensor_set(io.lens, &len, 0, sizeof(len));
+            free(rows);
+        }
+        const enum ggml_status st = mode == 0 ? ggml_backend_graph_compute(be, gf) : ggml_backend_sched_graph_compute(sched, gf);
+        if (st != GGML_STATUS_SUCCESS) rc = (int) st ? (int) st : -19;
+        else ggml_backend_tensor_get(io.out, out, 0, ggml_nbytes(io.out));
+        if (bufg) ggml_backend_buffer_free(bufg);
+        ggml_free(g);
+        g = NULL;
+        if (rc) goto done;
+        q      += QW * H * n_tok;
+        kv_cur += D * n_tok;
+        out    += DV * H * n_tok;
+    }
+    if (cache_out) ggml_backend_tensor_get(k_l, cache_out, 0, ggml_nbytes(k_l));
+done:
+    if (g) ggml_free(g);
+    if (sched) ggml_backend_sched_free(sched);
+    if (bufk) ggml_backend_buffer_free(bufk);
+    ggml_free(ck);
+    if (cpu) ggml_backend_free(cpu);
+    ggml_backend_free(be);
     return rc;
 }
 

@@ -143,12 +143,15 @@ def test_rope_node_through_the_plugin(gpu, mode):
 
 
 def test_mul_mat_node_the_plugin_leaves_to_other_backends(gpu):
-    """An F32 src0 is not taken (supports_op false -> the driver reports the node index), nothing is computed wrongly."""
+    """An F32 src0, or a BF16 product that is not one of the layer's two per-head products, is not taken (supports_op false
+    -> the driver reports the node index); nothing is computed wrongly."""
     rng = np.random.default_rng(520)
-    a = rng.standard_normal((2, 32, 64)).astype(np.float32)
-    b = rng.standard_normal((2, 5, 64)).astype(np.float32)
+    a = rng.standard_normal((2, 512, 128)).astype(np.float32)
+    b = rng.standard_normal((2, 5, 128)).astype(np.float32)
     with pytest.raises(RuntimeError, match="-100"):
         O.ref_mul_mat(a, O.TYPE_F32, b, so_path=_so())
+    with pytest.raises(RuntimeError, match="-100"):
+        O.ref_mul_mat(O.f32_to_bf16(a[:, :32, :64].copy()), O.TYPE_BF16, b[:, :, :64].copy(), so_path=_so())
     w = O.f32_to_bf16(a)
     got = O.ref_mul_mat(w, O.TYPE_BF16, b, so_path=_so())
     assert O.errors(got, O.ref_mul_mat(w, O.TYPE_BF16, b))[1] < 2e-6
