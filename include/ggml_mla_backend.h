@@ -32,9 +32,13 @@
  *                           the permuted result, src/llama-graph-attn.cpp:322)
  *   GGML_OP_ROPE            src[0] F32 [ne0, heads, n_tok, *], src[1] I32 [n_tok] positions, src[2] optional F32 frequency
  *                           factors; op_params of ggml_rope_ext (ggml/src/ggml.c:3413-3449), mode 0 or 2
- *   GGML_OP_MUL_MAT         src[0] F16 | BF16 [K, N, h, *] (K % 16 == 0, rows 16-byte aligned), src[1] F32 [K, M, H, *],
- *                           dst F32 [N, M, H, *]: the absorb products q_nope x wk_b and wv_b x kqv
- *                           (src/llama-graph-attn.cpp:264-275, :303-317)
+ *   GGML_OP_MUL_MAT         src[0] F16 | BF16 [K, N, H] (K % 16 == 0, rows 16-byte aligned), src[1] F32 [K, M, H, *],
+ *                           dst F32 [N, M, H, *], one matrix per head with K = 512 >= N or N = 512 >= K: the absorb
+ *                           products q_nope x wk_b and wv_b x kqv (src/llama-graph-attn.cpp:264-275, :303-317) and
+ *                           nothing else -- a model's other F16 / BF16 products stay with the backend that owns them
+ * For every one of these ops supports_op runs the argument checks of the launch itself (shapes, strides, 16-byte
+ * alignment of rows and of view offsets), so a node it accepts is one graph_compute runs; a node it refuses is placed on
+ * another backend by the scheduler.
  *   GGML_OP_CONCAT          F32 operands with dense rows along any dimension (q_states = concat(q_nope_absorbed, q_pe),
  *                           src/llama-graph-attn.cpp:277; kv_states, src/llama-graph-deepseek2.cpp:235)
  * Every other op except the no-op view ops (NONE, RESHAPE, VIEW, PERMUTE, TRANSPOSE) is reported unsupported, so
@@ -48,9 +52,16 @@
  *   event_new / event_free / event_synchronize and the backend's event_record / event_wait: HIP events on the
  *                          backend's stream, which ggml_backend_sched uses to keep several copies of a graph's inputs in
  *                          flight (ggml/src/ggml-backend.cpp:1508-1530, :1576-1580, :1630-1634)
- * F16 KV: the node accumulates V in f32 (closer to the exact value than ggml-cpu's f16 accumulator, which is 4e-3 away);
- * a backend initialised with params containing "f16_acc=strict" (ggml_backend_dev_init(dev, params)), or with
- * GGML_HIP_MLA_F16_ACC=strict in the environment, replays the reference's accumulator instead (ggml-cpu.c:12066-12080).
+ * F16 KV: the node accumulates V in f32 by default.  That is what the graph the reference emits for MLA does -- llm_attn_mla
+ * builds mul_mat(v, softmax(..)) (src/llama-graph-attn.cpp:287-317), whose F16 dot product sums in f32 -- and the default
+ * agrees with that graph to 4e-4 rel-L2 (tests/test_layer_graph.py).  ggml-cpu's fused FLASH_ATTN_EXT node is the odd one:
+ * it keeps the V accumulator in f16 (ggml-cpu.c:12066-12080) and lands 1.4e-3 (77 keys) to 3.9e-3 (1024 keys) rel-L2 from
+ * the exact value of the same rounded inputs, where the default lands 2e-4 away -- so against ggml-cpu's fused node the
+ * default is outside the 1e-3 tolerance by that much (tests/test_backend_gpu.py states both numbers).  A backend
+ * initialised with params containing "f16_acc=strict" (ggml_backend_dev_init(dev, params)), or with
+ * GGML_HIP_MLA_F16_ACC=strict in the environment, replays ggml-cpu's f16 accumulator step for step instead (1.1e-4 from
+ * ggml-cpu's node; contiguous caches only; 4 times slower on a decode step): for bit-for-bit comparisons with ggml-cpu's
+ * fused node, not for serving.
  * BF16 KV, more than 32 attention rows per sequence: the decode kernel converts the cache tiles to f16 on the way (exact for magnitudes in [2^-14, 65504], which a
  * latent cache holds; see MLA_FLAG_BF16_DIRECT in mla_attn.h); params containing "bf16=direct", or GGML_HIP_MLA_BF16=direct
  * in the environment, keep the tiles in bf16 for caches with values outside that range.

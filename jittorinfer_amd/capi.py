@@ -102,18 +102,31 @@ class MlaKvWriteArgs(C.Structure):
 _workspaces = {}
 
 
-def _workspace(device, nbytes):
+def _workspace(device, nbytes, stream=None):
+    """The scratch area of a launch: one per (device, stream) -- launches on different streams run side by side and each
+    needs its own partials, Q image and schedule -- and grow-only.  Growing waits for the stream first (launches already
+    queued still use the old area) and is refused while the stream is being captured into a graph, whose replays would
+    keep the address of an area that no longer exists: size the first, uncaptured call for the largest batch."""
     import torch
-    ws = _workspaces.get(device)
+    if stream is None:
+        stream = torch.cuda.current_stream(device).cuda_stream
+    key = (device, int(stream))
+    ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError("the attention workspace would have to %s during graph capture: run one launch of the largest "
+                               "shape on this stream before capturing" % ("grow" if ws is not None else "be allocated"))
+        if ws is not None:
+            torch.cuda.synchronize(device)
         ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
-        _workspaces[device] = ws
+        _workspaces[key] = ws
     return ws
 
 
 def make_args(q, k, kv_type, dv=512, mask=None, scale=1.0, max_bias=0.0, logit_softcap=0.0, block_table=None,
-              seq_lens=None, out=None, n_splits=0, flags=0, rows_per_wg=0):
-    """Builds (args, out, keepalive) from torch tensors on one gfx950 device.
+              seq_lens=None, out=None, n_splits=0, flags=0, rows_per_wg=0, stream=None):
+    """Builds (args, out, keepalive) from torch tensors on one gfx950 device, for a launch on `stream` (a raw handle; None: the
+    current torch stream) -- the workspace is that stream's.
 
     q     float32 [n_seq, n_head, n_tok, 576] (any strides with a contiguous last dim)
     k     the latent KV rows: [n_seq, n_kv, row] (uint8/int16/bfloat16/float16 with `row` 1152/612 bytes) or,
@@ -153,7 +166,7 @@ def make_args(q, k, kv_type, dv=512, mask=None, scale=1.0, max_bias=0.0, logit_s
     a.n_splits = n_splits
     a.rows_per_wg = rows_per_wg
     need = library().mla_attn_workspace_size(C.byref(a))
-    ws = _workspace(q.device, need)
+    ws = _workspace(q.device, need, stream)
     a.workspace, a.workspace_size = ws.data_ptr(), ws.numel()
     return a, out, (q, k, mask, block_table, seq_lens, ws)
 
@@ -166,7 +179,7 @@ def ggml_flash_attn_ext(q, k, kv_type, dv=512, mask=None, scale=1.0, max_bias=0.
     import torch
     if not q.is_cuda:
         raise RuntimeError("jittorinfer_amd runs on a gfx950 GPU only (there is no CPU path)")
-    a, out, keep = make_args(q, k, kv_type, dv, mask, scale, max_bias, logit_softcap, block_table, seq_lens, out, n_splits, flags, rows_per_wg)
+    a, out, keep = make_args(q, k, kv_type, dv, mask, scale, max_bias, logit_softcap, block_table, seq_lens, out, n_splits, flags, rows_per_wg, stream)
     st = stream if stream is not None else torch.cuda.current_stream(q.device).cuda_stream
     rc = library().mla_attn_launch(C.byref(a), C.c_void_p(st))
     if rc != 0:

@@ -57,6 +57,12 @@ def test_f16_cache_with_the_reference_accumulator_on_request(gpu, monkeypatch):
     e_fast, e_strict = O.errors(fast, cpu), O.errors(strict, cpu)
     print("vs ggml-cpu: f32 accumulation", e_fast, "replay", e_strict)
     U.check(strict, cpu, "strict replay vs ggml-cpu")
+    # the numbers include/ggml_mla_backend.h states for the default: outside the tolerance against ggml-cpu's fused node
+    # because that node is 3.9e-3 from the exact value of the same rounded inputs, and the default is 2e-4 from it (the probabilities meet V as f16)
+    exact = O.flash_attn_ext_f64(q, k, O.TYPE_F16, dv=576, scale=U.SCALE)
+    e_cpu_exact, e_fast_exact = O.errors(cpu, exact), O.errors(fast, exact)
+    print("vs the exact value: ggml-cpu", e_cpu_exact, "default", e_fast_exact)
+    assert 2e-3 < e_fast[1] < 6e-3 and 2e-3 < e_cpu_exact[1] < 6e-3 and e_fast_exact[1] < 3e-4
     assert e_strict[1] < 0.5 * e_fast[1]
 
 

@@ -474,3 +474,43 @@ def test_balanced_schedule_of_a_masked_launch_with_many_row_blocks(gpu):
     want = O.flash_attn_ext(q, k, O.TYPE_BF16, dv=512, mask=mask, scale=U.SCALE)
     assert np.isnan(want[0, 5]).all() and np.isnan(want[0, 8:16]).all()
     print(U.check(got[..., :512], want, "masked launch, balanced schedule"))
+
+
+def test_workspace_is_per_stream_and_does_not_grow_under_capture(gpu):
+    """The binding keeps one scratch area per (device, stream): launches on two streams must not share partials, a
+    larger launch on a stream gets a larger area after the stream has drained, and growth during graph capture is refused
+    (the graph would replay into freed memory)."""
+    import torch
+    import jittorinfer_amd as J
+    rng = np.random.default_rng(3)
+    pool, bt, seqs = U.make_paged(rng, [900, 700], O.TYPE_BF16)
+    q = rng.standard_normal((2, 128, 1, 576)).astype(np.float32)
+    tq, tk = torch.from_numpy(q).to(gpu), torch.from_numpy(pool.view(np.int16)).to(gpu)
+    tb, tl = torch.from_numpy(bt).to(gpu), torch.tensor([900, 700], dtype=torch.int32, device=gpu)
+    kw = dict(dv=512, scale=U.SCALE, block_table=tb, seq_lens=tl)
+    s1, s2 = torch.cuda.Stream(gpu), torch.cuda.Stream(gpu)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(s1):
+        a1, o1, k1 = J.capi.make_args(tq, tk, J.MLA_TYPE_BF16, **kw)
+    with torch.cuda.stream(s2):
+        a2, o2, k2 = J.capi.make_args(tq, tk, J.MLA_TYPE_BF16, **kw)
+    assert a1.workspace != a2.workspace
+    with torch.cuda.stream(s1):
+        r1 = J.ggml_flash_attn_ext(tq, tk, J.MLA_TYPE_BF16, **kw)
+    with torch.cuda.stream(s2):
+        r2 = J.ggml_flash_attn_ext(tq, tk, J.MLA_TYPE_BF16, **kw)
+    torch.cuda.synchronize()
+    assert torch.equal(r1[..., :512], r2[..., :512])
+    print(U.check(r1.cpu().numpy()[..., :512], U.oracle_per_seq(q, seqs, O.TYPE_BF16, 512), "two streams"))
+    # a stream that has never launched, under capture: no area yet, and none may be made now
+    s3 = torch.cuda.Stream(gpu)
+    graph = torch.cuda.CUDAGraph()
+    out3, one = torch.zeros((2, 1, 128, 576), dtype=torch.float32, device=gpu), torch.zeros(1, device=gpu)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(s3):
+        graph.capture_begin()
+        one.add_(1.0)
+        with pytest.raises(RuntimeError, match="graph capture"):
+            J.capi.make_args(tq, tk, J.MLA_TYPE_BF16, out=out3, **kw)
+        graph.capture_end()
+    torch.cuda.synchronize()
