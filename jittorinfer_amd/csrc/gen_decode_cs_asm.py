@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Generates mla_decode_cs_*.inc: the gfx950 instruction streams of the pipelined MLA decode kernel in its
 "column-split" form (one inline-asm block each inside mla_decode_kernel.hip).
-Usage: python gen_decode_cs_asm.py [--f16] > mla_decode_cs_[bf16|f16].inc
+Usage: python gen_decode_cs_asm.py [--f16] [--mask] > mla_decode_cs_[bf16|f16][_mask].inc
 
 Work of one wave w of a 4-wave workgroup (128 attention rows x one KV split), per 32-token tile `it`:
     part 1   S = K[it+1].Q^T for the wave's own 32 rows (36 MFMA, Q resident in 144 VGPRs, K fragments from LDS);
@@ -14,6 +14,9 @@ A wave thus owns 128 columns of all 128 rows of O (16 accumulator blocks of 32 x
 four MFMAs, so the transposing reads (the slow kind) drop to a quarter, and with 8 fragments per wave and tile the bf16 -> f16
 conversion fits in registers: no pass over the tile in LDS, no tile buffer held for it, two tiles of loads in flight.
 bf16 K is multiplied as bf16 (exact products either way); P and V meet as f16, which keeps 11 bits of P.
+--mask: an additive f16 mask row per query token (ggml-cpu.c:12041-12057: s * scale + mask): the 16 mask values of a lane's 16
+tokens of tile it+1 are loaded at the top of iteration `it` (four 8-byte loads) and enter the scores ahead of the softmax; the
+eight registers they live in come out of the K and P^T fragment rings.
 """
 import sys
 
@@ -22,6 +25,8 @@ F16KV = "--f16" in ARGS                      # f16 KV rows: f16 MFMA for K.Q^T, 
 CLK = "--clk" in ARGS                        # timing builds: s_memtime stamps left in LDS at the end
 NO_STORE = "--no-store" in ARGS              # timing experiments only (wrong results)
 NO_LOOP_DMA = "--no-loop-dma" in ARGS        # timing experiments only (wrong results): the loop computes on whatever the tile buffers hold
+MASK = "--mask" in ARGS                      # additive f16 mask rows (one per query token)
+assert not (MASK and CLK)
 MF_QK = "v_mfma_f32_32x32x16_f16" if F16KV else "v_mfma_f32_32x32x16_bf16"
 MF_PV = "v_mfma_f32_32x32x16_f16"
 
@@ -42,7 +47,9 @@ FOFF = AOFF + 1024                           # one word per wave: non-zero when 
 CPR = 73                                     # 16-byte chunks per padded row
 WAVE_CHUNKS = 8 * CPR                        # each wave moves rows 8w .. 8w+7 of a tile
 DMA_PER_TILE = 10
-KRING, PRING = 6, 4                          # K fragment ring: five slots of its own, the sixth in T[4:7] (free while K.Q^T runs)
+# K fragment ring: five slots of its own, the sixth in T[4:7] (free while K.Q^T runs); mask builds give the last slot of each
+# ring to the mask values
+KRING, PRING = (5, 3) if MASK else (6, 4)
 
 # ---- VGPR map (v252..v255 are left to the compiler: the clobber list of the asm block ends at v251)
 Q0 = 0
@@ -58,6 +65,8 @@ X0 = 249
 DT = [250, 251]         # address temporaries of the LDS-DMA slots; conversion temporaries in part 2
 X1, X2 = 250, 251       # prologue / epilogue temporaries
 NEGM, ALPHA, TMAX = T[5], T[6], T[7]   # live inside the softmax only
+MKR = [204, 205, 206, 207, 224, 225, 226, 227]   # mask builds: the 16 f16 mask values of this lane's 16 tokens of a tile
+MOFF = X0               # mask builds: byte offset of this lane's first mask element inside a tile's 64 mask bytes (from the end of the prologue on)
 LANE = T[7]             # prologue only
 N_VGPR = 252
 # ---- SGPR map (all inside the clobbered range s40..s99)
@@ -74,6 +83,7 @@ SB = 98                 # epilogue: running store base
 WDMA, CL, LAST0, NTM1 = 90, [91, 92, 93, 94], 95, 96
 DMA_BIAS = 3072         # the k-th load behind an M0 update carries the instruction offset 1024 k, which moves both addresses: the
                         # table offsets are (true offset - 1024 k + 3072) and the tile base is taken 3072 bytes low
+SCL, L2E, MSK = 98, 99, 76   # mask builds: scale, log2(e) (SB's registers until the epilogue), mask base (QP's registers once Q is requested)
 TAU_BITS = 0x41000000   # 8.0f
 
 out = []
@@ -254,7 +264,7 @@ def dma_tile_lines(tile_sreg, off_sreg, first_page_scalar=False):
 # ---------------------------------------------------------------------------------------------------------------
 def kf_reg(p):
     slot = p % KRING
-    return KF + 4 * slot if slot < 5 else T[4]
+    return KF + 4 * slot if slot < KRING - 1 else T[4]
 
 
 def k_read(p):
@@ -341,6 +351,13 @@ def softmax_lines(first_tile=False):
     l += sum of the rounded p (the output stays an exact weighted mean of V rows)."""
     L = []
     m = [T[0], T[1], T[2], T[3], T[4]]
+    if MASK:
+        # u = s * scale + mask (the order of ggml-cpu.c:12048-12057); element k = token 8 (k / 4) + 4 g + k % 4, whose mask value is
+        # half k % 2 of register 2 (k / 4) + (k % 4) / 2
+        for k in range(16):
+            h = k % 2
+            L.append("v_fma_mix_f32 %s, %s, %s, %s op_sel:[0,0,%d] op_sel_hi:[0,0,1]" % (v(S + k), v(S + k), s(SCL), v(MKR[2 * (k // 4) + (k % 4) // 2]), h))
+    CS = L2E if MASK else CL2           # factor from the values in S to log2 units
     L.append("v_max3_f32 %s, %s, %s, %s" % (v(m[0]), v(S + 0), v(S + 1), v(S + 2)))
     L.append("v_max3_f32 %s, %s, %s, %s" % (v(m[1]), v(S + 3), v(S + 4), v(S + 5)))
     L.append("v_max3_f32 %s, %s, %s, %s" % (v(m[2]), v(S + 6), v(S + 7), v(S + 8)))
@@ -354,7 +371,7 @@ def softmax_lines(first_tile=False):
     L.append("v_permlane32_swap_b32 %s, %s" % (v(m[0]), v(m[1])))
     L.append("s_nop 1")
     L.append("v_max_f32 %s, %s, %s" % (v(TMAX), v(m[0]), v(m[1])))
-    L.append("v_mul_f32 %s, %s, %s" % (v(TMAX), s(CL2), v(TMAX)))           # log2 units (the factor is > 0)
+    L.append("v_mul_f32 %s, %s, %s" % (v(TMAX), s(CS), v(TMAX)))            # log2 units (the factor is > 0)
     L.append("v_add_f32 %s, %s, %s" % (v(m[2]), s(THR), v(MRUN)))           # m_run + TAU  (-inf stays -inf)
     L.append("v_sub_f32 %s, %s, %s" % (v(m[3]), v(MRUN), v(TMAX)))          # m_run - tmax
     L.append("v_exp_f32 %s, %s" % (v(m[3]), v(m[3])))                       # 2^(m_run - tmax); 0 when m_run = -inf
@@ -371,7 +388,7 @@ def softmax_lines(first_tile=False):
     L.append("s_nop 0")
     L.append("v_cndmask_b32 %s, %s, 0, vcc" % (v(NEGM), v(NEGM)))
     for k in range(16):
-        L.append("v_fma_f32 %s, %s, %s, %s" % (v(S + k), v(S + k), s(CL2), v(NEGM)))
+        L.append("v_fma_f32 %s, %s, %s, %s" % (v(S + k), v(S + k), s(CS), v(NEGM)))
     for k in range(16):
         L.append("v_exp_f32 %s, %s" % (v(S + k), v(S + k)))
     # P^T operands in place.  k-step kk owns registers b = S+8kk .. +7, holding p of tokens
@@ -425,9 +442,31 @@ def mask_tail():
     e("%s:" % lab)
 
 
+def mask_loads(tile_sreg):
+    """Mask builds: the 64 mask bytes of tile s[tile_sreg] for this lane's query token -> MKR (four 8-byte loads)."""
+    e("s_lshl_b32 %s, %s, 6" % (s(S0), s(tile_sreg)))
+    e("s_add_u32 %s, %s, %s" % (s(S0), s(MSK), s(S0)))
+    e("s_addc_u32 %s, %s, 0" % (s(S1), s(MSK + 1)))
+    for j in range(4):
+        e("global_load_dwordx2 %s, %s, %s offset:%d" % (v(MKR[2 * j], 2), v(MOFF), s(S0, 2), 16 * j))
+
+
+def mask_wait():
+    """Mask builds: the mask values requested at the top of the iteration are there (loads return in order: only the tile
+    loads issued behind them, if any, may still be in flight)."""
+    lab_m0, lab_md = label("m0"), label("md")
+    e("s_cmp_eq_u32 %s, 0" % s(VMW))
+    e("s_cbranch_scc1 %s" % lab_m0)
+    e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
+    e("s_branch %s" % lab_md)
+    e("%s:" % lab_m0)
+    e("s_waitcnt vmcnt(0)")
+    e("%s:" % lab_md)
+
+
 def canon_tags():
     """LDS reads in flight at the top of every iteration, in issue order (see handover)."""
-    return [("k", p) for p in range(KRING - 1)] + [("p", 0), ("p", 1), ("p", 2)]
+    return [("k", p) for p in range(KRING - 1)] + [("p", f) for f in range(PRING - 1)]
 
 
 def handover(tail, resc):
@@ -440,9 +479,10 @@ def handover(tail, resc):
     lds.op("ds_read_b128 %s, %s" % (v(T[0], 4), v(T[4])), ("f",))
     e("v_add_u32 %s, %s, %s" % (v(KADDR), s(OFF1), v(KADDR_LANE)))
     k_warm()
-    p_read(0)
-    p_read(1)
-    p_read(2)
+    # fragment 7, which the tail MFMAs still use, sits in ring slot 7 % PRING: a fragment that shares it is requested behind them
+    early = [f for f in range(PRING - 1) if not tail or f % PRING != 7 % PRING]
+    for f in early:
+        p_read(f)
     top = ["s_add_u32 %s, %s, 1" % (s(S0), s(IT)),
            "s_lshl_b32 %s, %s, 5" % (s(S0), s(S0)),
            "s_add_u32 %s, %s, %s" % (s(S0), s(S0), s(KVB)),
@@ -454,6 +494,10 @@ def handover(tail, resc):
     else:
         for ln in top:
             e(ln)
+    for f in range(PRING - 1):
+        if f not in early:
+            assert f > max(early)      # fragments return in order
+            p_read(f)
     lds.need(("f",))
     e("v_or3_b32 %s, %s, %s, %s" % (v(T[0]), v(T[0]), v(T[1]), v(T[2])))
     e("v_or_b32 %s, %s, %s" % (v(T[0]), v(T[0]), v(T[3])))
@@ -540,6 +584,8 @@ def iteration(resc, lab_loop):
     e("s_add_u32 %s, %s, 1" % (s(TMP), s(IT)))
     e("s_cmp_ge_u32 %s, %s" % (s(TMP), s(NT)))
     e("s_cbranch_scc1 %s" % lab_last)
+    if MASK:
+        mask_loads(TMP)              # mask of tile IT+1: behind the loads of tile IT+2, ahead of those of tile IT+3
     e("s_add_u32 %s, %s, 3" % (s(TMP), s(IT)))
     e("s_cmp_ge_u32 %s, %s" % (s(TMP), s(NT)))
     e("s_cbranch_scc1 %s" % lab_nodma)
@@ -584,6 +630,8 @@ def iteration(resc, lab_loop):
     def qk_done():
         e("s_nop 1")                    # the last K.Q^T MFMA has written S: two P.V MFMAs (8 passes each) were issued behind it
         mask_tail()
+        if MASK:
+            mask_wait()
 
     def p_read_by_all():
         # every P^T fragment of tile IT is in this wave's registers (the last read was issued at slot 16) before any wave overwrites P
@@ -652,6 +700,9 @@ def main():
     e("s_mov_b32 %s, %%[rstr]" % s(RSTR))
     e("s_mov_b32 %s, %%[nrv]" % s(NRV))
     e("v_mov_b32 %s, %%[tid]" % v(X0))
+    if MASK:
+        e("s_mov_b32 %s, %%[scl]" % s(SCL))
+        e("s_mov_b32 %s, 0x3fb8aa3b" % s(L2E))
     e("s_mov_b32 %s, 0x%08x" % (s(THR), TAU_BITS))
     e("s_mov_b32 %s, 0x3c003c00" % s(ONES))
     e("v_and_b32 %s, 63, %s" % (v(LANE), v(X0)))
@@ -754,6 +805,15 @@ def main():
             e("s_add_u32 %s, %s, 4096" % (s(QP), s(QP)))
             e("s_addc_u32 %s, %s, 0" % (s(QP + 1), s(QP + 1)))
         e("global_load_dwordx4 %s, %s, %s offset:%d" % (v(Q0 + 4 * ks, 4), v(X0), s(QP, 2), (ks % 4) * 1024))
+    if MASK:
+        # mask rows start at key kv_begin of this piece; QP's registers and X0 are free now
+        e("s_mov_b64 %s, %%[msk]" % s(MSK, 2))
+        e("s_lshl_b32 %s, %s, 1" % (s(S0), s(KVB)))
+        e("s_add_u32 %s, %s, %s" % (s(MSK), s(MSK), s(S0)))
+        e("s_addc_u32 %s, %s, 0" % (s(MSK + 1), s(MSK + 1)))
+        e("v_mov_b32 %s, %%[moff]" % v(MOFF))
+        e("s_mov_b32 %s, 0" % s(TMP))
+        mask_loads(TMP)
     lap(4)
     lab_w0, lab_w1, lab_wd = label("pw0"), label("pw1"), label("pwd")
     for i in range(256):
@@ -930,7 +990,7 @@ def main():
     e("s_mov_b64 exec, %s" % s(EXS, 2))
     e("s_waitcnt vmcnt(0)")
 
-    print("// generated by gen_decode_cs_asm.py%s -- do not edit" % (" --f16" if F16KV else ""))
+    print("// generated by gen_decode_cs_asm.py%s%s -- do not edit" % (" --f16" if F16KV else "", " --mask" if MASK else ""))
     for ln in out:
         print('"%s\\n\\t"' % ln)
     if CLK:

@@ -74,6 +74,8 @@ constexpr int lds_total(int kvt) { return sched_off(kvt) + (2 * SCHED_MAX_SEQ + 
     [nb1] "s"(s_nb1), [flg] "s"(s_flg), [ntl] "s"(s_ntl), [ostr] "s"(s_ostr), [qp] "s"(qpack), [pg0] "s"(s_pg0),  \
     [ob] "s"(out_base), [mlb] "s"(ml_base), [rstr] "s"(s_rstr), [nrv] "s"(s_nrv), [tid] "v"(tid)
 
+#define MLA_DECODE_CS_MASK_INPUTS MLA_DECODE_CS_INPUTS, [msk] "s"(mask_base), [scl] "s"(s_scale), [moff] "v"(mask_off)
+
 #define MLA_DECODE_INPUTS                                                                                          \
     [kv] "s"(kv_base), [bt] "s"(bt_row), [kvb] "s"(s_kvb), [kve] "s"(s_kve), [cl2] "s"(c_log2_bits), [npp] "s"(s_npp), \
     [nb1] "s"(s_nb1), [flg] "s"(s_flg), [ntl] "s"(s_ntl), [ostr] "s"(s_ostr), [qp] "s"(qpack), [msk] "s"(mask_base),  \
@@ -361,7 +363,18 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
     const int s_rstr = __builtin_amdgcn_readfirstlane((int) ((direct ? p.dst_stride : (int64_t) p.dv_total) * 4));
     const int s_nrv  = __builtin_amdgcn_readfirstlane(min(max(p.n_rows - by * 128, 0), 128));
 
-    if constexpr (KVT == SRC_BF16_CS) {
+    // mask builds of the column-split programs: byte offset of this lane's first mask element (its query token's row, tokens 4g.. of a tile)
+    const int mask_off = MASK ? (int) ((int64_t) (min(row, p.n_rows - 1) / p.n_head) * p.mask_nb1 + 8 * g) : 0;
+
+    if constexpr (KVT == SRC_BF16_CS && MASK) {
+        asm volatile(
+#include "mla_decode_cs_bf16_mask.inc"
+            : : MLA_DECODE_CS_MASK_INPUTS : MLA_DECODE_CS_CLOBBERS);
+    } else if constexpr (KVT == SRC_F16_CS && MASK) {
+        asm volatile(
+#include "mla_decode_cs_f16_mask.inc"
+            : : MLA_DECODE_CS_MASK_INPUTS : MLA_DECODE_CS_CLOBBERS);
+    } else if constexpr (KVT == SRC_BF16_CS) {
         asm volatile(
 #include "mla_decode_cs_bf16.inc"
             : : MLA_DECODE_CS_INPUTS : MLA_DECODE_CS_CLOBBERS);
@@ -618,7 +631,7 @@ static hipError_t launch_variant(const KParams & kp, dim3 grid, hipStream_t st) 
 
 static bool decode_cs_applicable(const KParams & kp, int kv_type) {
     if (kv_type != MLA_TYPE_BF16 && kv_type != MLA_TYPE_F16) return false;
-    if (kp.mask || kp.bf16_direct || kp.q_as_q8) return false;
+    if (kp.bf16_direct || kp.q_as_q8) return false;
     const int tail = kp.n_rows % 128;
     return (tail == 0 || tail > 96) && kp.slot_rows < (1 << 22);
 }
@@ -630,7 +643,7 @@ hipError_t launch_decode_fast(const KParams & kp, int kv_type, dim3 grid, hipStr
     // bf16 tiles are converted to f16 inside LDS unless the caller asks for the hi + lo program, or a single wave of a workgroup
     // has rows (16- and 32-head decode): one computing wave is not bound by its MFMAs, and the hi + lo program is the more exact
     // column-split programs (every wave computes S for its own 32 rows and P.V for its own 128 columns): blocks of 128 rows in
-    // which all four waves have rows, no mask, not the Q8_0 expansion; bf16 K enters as bf16, so the Q image is the bf16 one
+    // which all four waves have rows, not the Q8_0 expansion; bf16 K enters as bf16, so the Q image is the bf16 one
     const bool cs = decode_cs_applicable(kp, kv_type);
     const bool bf16_cvt = !cs && !kp.bf16_direct && kp.n_rows > 32;
     if (!with_prepass) { /* the workspace still holds the Q image and the mask extents of an earlier launch of the same call */ }
@@ -640,8 +653,8 @@ hipError_t launch_decode_fast(const KParams & kp, int kv_type, dim3 grid, hipStr
     else                              hipLaunchKernelGGL(mla_q_pack_kernel<0>, dim3(n_rb, n_seq, KSTEPS + extra), dim3(NTHREADS), 0, st, kp);
     if (m && with_prepass) hipLaunchKernelGGL(mla_mask_extent_kernel, dim3(n_rb, MASK_EXT_CHUNKS), dim3(NTHREADS), 0, st, kp);
     if (kv_type == MLA_TYPE_Q8_0) return m ? launch_variant<SRC_Q8, true>(kp, grid, st) : launch_variant<SRC_Q8, false>(kp, grid, st);
-    if (cs && kv_type == MLA_TYPE_F16) return launch_variant<SRC_F16_CS, false>(kp, grid, st);
-    if (cs)                            return launch_variant<SRC_BF16_CS, false>(kp, grid, st);
+    if (cs && kv_type == MLA_TYPE_F16) return m ? launch_variant<SRC_F16_CS, true>(kp, grid, st) : launch_variant<SRC_F16_CS, false>(kp, grid, st);
+    if (cs)                            return m ? launch_variant<SRC_BF16_CS, true>(kp, grid, st) : launch_variant<SRC_BF16_CS, false>(kp, grid, st);
     if (kv_type == MLA_TYPE_F16)  return m ? launch_variant<SRC_F16, true>(kp, grid, st) : launch_variant<SRC_F16, false>(kp, grid, st);
     if (bf16_cvt)                 return m ? launch_variant<SRC_BF16_CVT, true>(kp, grid, st) : launch_variant<SRC_BF16_CVT, false>(kp, grid, st);
     return m ? launch_variant<SRC_BF16, true>(kp, grid, st) : launch_variant<SRC_BF16, false>(kp, grid, st);
