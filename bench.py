@@ -598,11 +598,15 @@ def main():
 
     # HBM bytes of one decode-kernel launch, from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by what the same
     # counters read for the library's copy kernel; figures and commands in profiles/mla_decode_kernel_c3_pmc.md
-    traffic, traffic_source = None, None
+    traffic, traffic_source, traffic_decode = None, None, None
     if a.batch == 32 and a.heads == 128 and a.ctx == 8192 and a.kv == "bf16":
-        traffic_source = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of the decode kernel, scaled by the copy kernel's readings: profiles/mla_decode_kernel_c3_pmc.md (a measured constant of that profile, not of this run)"
-        fetch_kib, write_kib = (150524, 34048) if a.bf16_direct else (150051, 35072)   # KiB per dispatch, mean
-        traffic = int(fetch_kib * 1024 * (294912 / 147466.0) + write_kib * 1024)
+        traffic_source = ("rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of the decode kernel and of the combine pass, scaled by the copy kernel's readings: "
+                          "profiles/mla_decode_kernel_c3_pmc.md (measured constants of that profile, not of this run)")
+        # KiB per dispatch, mean: decode kernel (fetch, write), combine pass (fetch, write)
+        d_f, d_w, c_f, c_w = (150524, 34048, 16677, 8192) if a.bf16_direct else (150613, 35584, 16548, 8192)
+        scale_f = 294912 / 147466.0   # the copy kernel reads 294 912 KiB and FETCH_SIZE reports 147 466
+        traffic_decode = int(d_f * 1024 * scale_f + d_w * 1024)
+        traffic = traffic_decode + int(c_f * 1024 * scale_f + c_w * 1024)
     res = {
         "metric": "mla_paged_decode_kv_read_bandwidth", "value": value, "unit": "GB/s",
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms_per_step,
@@ -621,7 +625,7 @@ def main():
         "roofline": {"bound": "hbm", "kernel": "mla_decode_kernel<%s> + mla_attn_combine_kernel" % a.kv, "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic, "traffic_source": traffic_source,
                      "algorithmic_bytes_per_launch": kv_bytes, "kernels_us": node_ms * 1e3,
-                     "decode_kernel_alone": {"achieved": achieved_decode, "frac": achieved_decode / HBM_PEAK_GBPS, "kernel_us": kern_stats},
+                     "decode_kernel_alone": {"achieved": achieved_decode, "frac": achieved_decode / HBM_PEAK_GBPS, "kernel_us": kern_stats, "traffic": traffic_decode},
                      "mfma_tflops": flops / (node_ms * 1e-3) / 1e12},
         "cpu_baseline": cpu,
         "parity": parity,
