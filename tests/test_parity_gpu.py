@@ -311,3 +311,27 @@ def test_bf16_few_rows_keep_the_direct_program(gpu):
         assert np.array_equal(a.view(np.int32), b.view(np.int32))
         want = U.oracle_per_seq(q, seqs, O.TYPE_BF16, 512)
         print(n_head, U.check(a[..., :512], want, "few rows", max_abs=2e-5, rel_l2=2e-5))
+
+
+def test_q8_0_cache_with_arbitrary_block_scales(gpu):
+    """A Q8_0 cache as the reference's quantizer leaves it -- every block its own scale d = amax / 127, not the power of two of
+    BASELINE's config 5 -- through the paged decode path (128 heads, ragged lengths, KV splits) and through a masked launch:
+    the f16 MFMA operand f16(q * d) then carries a rounding of its own (2^-12 relative per value), and the result still
+    meets the stated tolerance at these lengths.  (A sequence of one or two keys can reach 2.2e-3 in single elements: an
+    output element is then the rounded operand itself; tests/test_sweep_gpu.py allows 3e-3 for that.)"""
+    rng = np.random.default_rng(88)
+    lens = [2900, 700, 1311, 130, 4097, 64]
+    pool, bt, seqs = U.make_paged(rng, lens, O.TYPE_Q8_0)          # q8_scale None: quantize_row_q8_0 of N(0, 1) rows
+    d = pool.reshape(-1, 18, 34)[:, :, :2].copy().view(np.float16)
+    assert len(np.unique(d)) > 1000                                 # the scales really are arbitrary
+    q = rng.standard_normal((len(lens), 128, 1, 576)).astype(np.float32)
+    got = _run(gpu, q, pool, O.TYPE_Q8_0, bt=bt, lens=lens, scale=U.SCALE)[..., :512]
+    want = U.oracle_per_seq(q, seqs, O.TYPE_Q8_0, 512)
+    print(U.check(got, want, "Q8_0, arbitrary scales, paged decode"))
+    n_kv, n_tok = 1024, 8
+    q = rng.standard_normal((1, 16, n_tok, 576)).astype(np.float32)
+    k = U.encode_kv(rng.standard_normal((1, n_kv, 576)).astype(np.float32), O.TYPE_Q8_0)
+    m = np.where(np.arange(n_kv)[None, :] > 900 + 10 * np.arange(n_tok)[:, None], -np.inf, 0.0).astype(np.float16)
+    got = _run(gpu, q, k, O.TYPE_Q8_0, mask=m.view(np.uint16), scale=U.SCALE)[..., :512]
+    want = O.flash_attn_ext(q, k, O.TYPE_Q8_0, dv=512, mask=m.view(np.uint16), scale=U.SCALE)
+    print(U.check(got, want, "Q8_0, arbitrary scales, masked"))
