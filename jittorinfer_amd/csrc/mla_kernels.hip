@@ -511,7 +511,7 @@ __global__ void __launch_bounds__(256) mla_attn_combine_f32_kernel(const KParams
     const float2 * ml = (const float2 *) p.part_ml + (int64_t) slot0 * p.slot_rows + lrow;
     const float *  po = (const float *) p.part_o + ((int64_t) slot0 * p.slot_rows + lrow) * p.dv_total + cg * 4;
     const int64_t ml_step = p.slot_rows, po_step = (int64_t) p.slot_rows * p.dv_total;
-    constexpr int G = 16;   // small problems are latency-bound: a ragged batch has up to 32 one-page pieces per sequence
+    constexpr int G = 32;   // small problems are latency-bound: a ragged batch has up to 32 one-page pieces per sequence, all in flight at once
     float M = -INFINITY, L = 0.f;
     f32x4 o = { 0.f, 0.f, 0.f, 0.f };
     for (int c0 = 0; c0 < nvalid; c0 += G) {   // groups of G splits: their loads are in flight together
