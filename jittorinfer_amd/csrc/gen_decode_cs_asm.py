@@ -26,6 +26,7 @@ CLK = "--clk" in ARGS                        # timing builds: s_memtime stamps l
 NO_STORE = "--no-store" in ARGS              # timing experiments only (wrong results)
 NO_LOOP_DMA = "--no-loop-dma" in ARGS        # timing experiments only (wrong results): the loop computes on whatever the tile buffers hold
 MASK = "--mask" in ARGS                      # additive f16 mask rows (one per query token)
+KS = "--ks" in ARGS                          # at most 32 rows: the four waves split the 576 columns of K.Q^T (see ks_main)
 assert not (MASK and CLK)
 MF_QK = "v_mfma_f32_32x32x16_f16" if F16KV else "v_mfma_f32_32x32x16_bf16"
 MF_PV = "v_mfma_f32_32x32x16_f16"
@@ -681,7 +682,9 @@ def iteration(resc, lab_loop):
     lds.drain()
 
 
-def main():
+def prologue_head():
+    """Inputs -> fixed registers, lane geometry, the page ids of the piece, running state, the tile loads' offset table; ends
+    when tile 0 can be requested."""
     # ------------------------------------------------------------------ entry: inputs -> fixed registers
     e("s_mov_b64 %s, %%[kv]" % s(KV, 2))
     e("s_mov_b64 %s, %%[bt]" % s(BT, 2))
@@ -791,6 +794,10 @@ def main():
     e("v_max_i32 %s, 0, %s" % (v(PAGES), v(PAGES)))
     e("v_min_i32 %s, %s, %s" % (v(PAGES), s(NPP), v(PAGES)))
     e("%s:" % lab_al)
+
+
+def main():
+    prologue_head()
     # ------------------------------------------------------------------ tile 0, then the Q operands (36 coalesced 16-byte loads per
     # lane from the packed image), then tiles 1 and 2; go on as soon as tile 0 and Q are there
     e("s_mov_b32 %s, 0" % s(TMP))
@@ -877,8 +884,16 @@ def main():
         rescale_block(back)
     e("%s:" % lab_end)
     clk_dump()
+    epilogue(4)
+    emit()
+
+
+def epilogue(nhb):
+    """1 / l of the rows, then the stores: nhb = 4: the wave's 128 columns of all 128 rows, 1 / l exchanged through LDS; nhb = 1 (the
+    k-split program): 32 rows, every wave has l itself."""
     # ------------------------------------------------------------------ epilogue
-    e("s_barrier")                      # no wave is still reading rescale factors: their area carries 1 / l next
+    if nhb == 4:
+        e("s_barrier")                  # no wave is still reading rescale factors: their area carries 1 / l next
     e("s_nop 7")
     e("s_nop 7")
     e("s_nop 7")
@@ -897,17 +912,20 @@ def main():
     e("v_cmp_class_f32 vcc, %s, %s" % (v(T[3]), s(SCLS)))   # finite?
     e("s_nop 1")
     e("v_cndmask_b32 %s, %s, %s, vcc" % (v(T[2]), v(T[2]), v(T[3])))
-    # every wave needs 1 / l of all 128 rows: through the rescale-factor area, [lane][hb]
-    e("v_add_u32 %s, %s, %s" % (v(T[3]), s(W4), v(PADDR)))
-    e("ds_write_b32 %s, %s offset:%d" % (v(T[3]), v(T[2]), AOFF - PBUF))
-    e("s_waitcnt lgkmcnt(0)")
-    e("s_barrier")
-    e("ds_read_b128 %s, %s offset:%d" % (v(T[4], 4), v(PADDR), AOFF - PBUF))   # T[4 + hb] = 1 / l of row 32 hb + lane % 32
+    if nhb == 4:
+        # every wave needs 1 / l of all 128 rows: through the rescale-factor area, [lane][hb]
+        e("v_add_u32 %s, %s, %s" % (v(T[3]), s(W4), v(PADDR)))
+        e("ds_write_b32 %s, %s offset:%d" % (v(T[3]), v(T[2]), AOFF - PBUF))
+        e("s_waitcnt lgkmcnt(0)")
+        e("s_barrier")
+        e("ds_read_b128 %s, %s offset:%d" % (v(T[4], 4), v(PADDR), AOFF - PBUF))   # T[4 + hb] = 1 / l of row 32 hb + lane % 32
+    else:
+        e("v_mov_b32 %s, %s" % (v(T[4]), v(T[2])))
     # lanes whose row exists, per row block: lane % 32 < n_rows_valid - 32 hb
     e("v_mbcnt_lo_u32_b32 %s, -1, 0" % v(X0))
     e("v_mbcnt_hi_u32_b32 %s, -1, %s" % (v(X0), v(X0)))               # lane
     e("v_and_b32 %s, 31, %s" % (v(X1), v(X0)))                         # rl
-    for hb in range(4):
+    for hb in range(nhb):
         e("s_sub_i32 %s, %s, %d" % (s(S0), s(NRV), 32 * hb))
         e("v_cmp_gt_i32 vcc, %s, %s" % (s(S0), v(X1)))
         e("s_mov_b64 %s, vcc" % s(VM[hb], 2))
@@ -928,7 +946,7 @@ def main():
     e("v_add_u32 %s, %s, %s" % (v(T[0]), s(S0), v(T[0])))              # rl * RSTR + 16 g + 512 w
     e("s_lshl_b32 %s, %s, 5" % (s(S1), s(RSTR)))                       # 32 rows
     e("s_mov_b64 %s, %s" % (s(SB, 2), s(OB, 2)))
-    for hb in range(4):
+    for hb in range(nhb):
         e("s_mov_b64 exec, %s" % s(VM[hb], 2))
         for cb in range(4):
             for q in range(4):
@@ -951,7 +969,7 @@ def main():
     e("s_mul_i32 %s, %s, %s" % (s(S0), s(S0), s(OSTR)))                # 16 w * OSTR  (< 2^31: OSTR <= 2^27 / 64 is checked on the host)
     e("s_add_u32 %s, %s, %s" % (s(S2), s(OB), s(S0)))
     e("s_addc_u32 %s, %s, 0" % (s(S3), s(OB + 1)))
-    for hb in range(4):
+    for hb in range(nhb):
         e("s_mov_b64 exec, %s" % s(VM[hb], 2))
         e("s_mov_b64 %s, %s" % (s(SB, 2), s(S2, 2)))
         for cb in range(4):
@@ -973,6 +991,9 @@ def main():
     e("s_mov_b64 exec, %s" % s(EXS, 2))
     e("s_cmp_eq_u64 %s, 0" % s(MLB, 2))
     e("s_cbranch_scc1 %s" % lab_noml)
+    if nhb == 1:
+        e("s_cmp_lg_u32 %s, 0" % s(WAVE))      # every wave holds (m, l) of the 32 rows: the first one writes them
+        e("s_cbranch_scc1 %s" % lab_noml)
     e("s_lshl_b32 %s, %s, 5" % (s(S0), s(WAVE)))
     e("s_sub_i32 %s, %s, %s" % (s(S0), s(NRV), s(S0)))                 # valid rows of this wave's block
     e("v_cmp_gt_i32 vcc, %s, %s" % (s(S0), v(X0)))                     # lane < that ...
@@ -990,11 +1011,262 @@ def main():
     e("s_mov_b64 exec, %s" % s(EXS, 2))
     e("s_waitcnt vmcnt(0)")
 
-    print("// generated by gen_decode_cs_asm.py%s%s -- do not edit" % (" --f16" if F16KV else "", " --mask" if MASK else ""))
+
+# ---------------------------------------------------------------------------------------------------------------
+# --ks: the program for at most 32 rows per sequence (a decode step of a 16- or 32-head model).  One row block, so the column-split
+# programs would leave K.Q^T to one wave; here the four waves split its 576 columns instead:
+#   wave w:  S_w = K[it+1][:, 144 w .. 144 w + 143] . Q[:, the same columns]^T   (9 MFMA; the wave holds a quarter of Q, 36 VGPRs)
+#            S_w -> LDS (4 KB per wave), barrier, every wave reads the four partial tiles and adds them in the same order, so all
+#            four hold the same scores, run the same softmax and reach the same maxima, sums and rescale decisions: P^T never
+#            goes through LDS, no flags, no factors
+#            O^T[128 w .. 128 w + 127][32 rows] += V[it]^T . P[it]^T   (8 MFMA)
+# 17 MFMAs per wave and tile instead of 68 / 100 on one wave.  Three tile buffers (loads two tiles ahead, requested as soon as every
+# wave is done with the buffer); the exchange area takes the fourth one's place.
+SQ, XR = 36, 52           # partial scores of this wave; the four waves' partial tiles as read back
+XOFF = 3 * TILE_BYTES     # exchange area: [wave][quarter of the 16 registers][lane][16 bytes] = 16 KB
+
+
+def ks_qk_slots():
+    depth = KRING - 1
+
+    def mk(ks):
+        def slot():
+            lds.need(("k", ks))
+            e("%s %s, %s, %s, %s" % (MF_QK, v(SQ, 16), v(kf_reg(ks), 4), v(Q0 + 4 * ks, 4), "0" if ks == 0 else v(SQ, 16)))
+            if ks + depth < 9:
+                k_read(ks + depth)
+        return slot
+    return [mk(ks) for ks in range(9)]
+
+
+def ks_scores():
+    """The MFMA slots of K.Q^T of the tile at v[KADDR] for this wave's quarter of the columns; the first K fragments are requested here."""
+    for p_ in range(min(KRING - 1, 9)):
+        k_read(p_)
+    return ks_qk_slots()
+
+
+def ks_exchange_write():
+    e("s_nop 7")                       # the last MFMA's result
+    e("s_nop 7")
+    e("s_nop 3")
+    e("v_add_u32 %s, %s, %s" % (v(T[2]), s(WOFS), v(PADDR)))
+    for q in range(4):
+        lds.op("ds_write_b128 %s, %s offset:%d" % (v(T[2]), v(SQ + 4 * q, 4), 1024 * q), ("x", q))
+    lds.drain()
+    e("s_barrier")
+
+
+def ks_exchange_read_items():
+    return [(lambda w=w, q=q: lds.op("ds_read_b128 %s, %s offset:%d" % (v(XR + 16 * w + 4 * q, 4), v(PADDR), 4096 * w + 1024 * q), ("xr", w, q)))
+            for w in range(4) for q in range(4)]
+
+
+def ks_sum_lines():
+    L = []
+    for k in range(16):
+        L.append("v_add_f32 %s, %s, %s" % (v(S + k), v(XR + k), v(XR + 16 + k)))
+    for k in range(16):
+        L.append("v_add_f32 %s, %s, %s" % (v(S + k), v(S + k), v(XR + 32 + k)))
+    for k in range(16):
+        L.append("v_add_f32 %s, %s, %s" % (v(S + k), v(S + k), v(XR + 48 + k)))
+    return L
+
+
+def ks_pv(n):
+    """MFMA n of the 8 of O^T += V^T.P^T: the P^T operands are this wave's own registers (S+0..3, S+8..11)."""
+    kk, cb = n // 4, n % 4
+    e("%s %s, %s, %s, %s" % (MF_PV, a(64 * cb, 16), v(VF + 4 * (4 * kk + cb), 4), v(S + 8 * kk, 4), a(64 * cb, 16)))
+
+
+def ks_v_items():
+    items = []
+    for f in range(8):
+        items += v_read_items(f)
+    for f in range(8):
+        items += v_conv_items(f, (DT[0], DT[1]))
+    return items
+
+
+def ks_rescale_block(ret_label):
+    """Rare path: the running maxima moved; acc[cb] *= alpha (per lane = per row).  Entered long after the last MFMA was issued."""
+    e("s_nop 7")
+    for cb in range(4):
+        for i in range(0, 16, 4):
+            for j in range(4):
+                e("v_accvgpr_read_b32 %s, %s" % (v(T[j]), a(64 * cb + i + j)))
+            for j in range(4):
+                e("v_mul_f32 %s, %s, %s" % (v(T[j]), v(T[j]), v(ALPHA)))
+            for j in range(4):
+                e("v_accvgpr_write_b32 %s, %s" % (a(64 * cb + i + j), v(T[j])))
+    e("s_nop 7")
+    e("s_branch %s" % ret_label)
+
+
+def ks_tail(first_tile, resc):
+    """Once the four partial tiles are back: their sum -> S, the keys past the end masked, softmax -> P^T operands in S, the
+    accumulators rescaled if some row's maximum moved."""
+    for ln in ks_sum_lines():
+        e(ln)
+    mask_tail()
+    for ln in softmax_lines(first_tile=first_tile):
+        e(ln)
+    if not first_tile:
+        lab_resc, lab_back = label("resc"), label("back")
+        e("s_cmp_lg_u64 %s, 0" % s(RSC, 2))
+        e("s_cbranch_scc1 %s" % lab_resc)
+        e("%s:" % lab_back)
+        resc.append((lab_resc, lab_back))
+
+
+def ks_main():
+    assert not MASK and not CLK
+    prologue_head()
+    e("s_mul_i32 %s, %s, 288" % (s(S0), s(WAVE)))                      # this wave's k-steps 9 w ..: 32 bytes each
+    e("v_add_u32 %s, %s, %s" % (v(KADDR_LANE), s(S0), v(KADDR_LANE)))
+    e("v_lshlrev_b32 %s, 4, %s" % (v(PADDR), v(LANE)))
+    e("v_add_u32 %s, 0x%x, %s" % (v(PADDR), XOFF, v(PADDR)))
+    e("s_lshl_b32 %s, %s, 12" % (s(WOFS), s(WAVE)))
+    # ------------------------------------------------------------------ tile 0, the wave's quarter of the Q operands, tiles 1 and 2
+    e("s_mov_b32 %s, 0" % s(TMP))
+    for ln in dma_tile_lines(TMP, OFF0, True):
+        e(ln)
+    e("v_lshlrev_b32 %s, 4, %s" % (v(X0), v(LANE)))
+    e("s_mul_i32 %s, %s, %d" % (s(S0), s(WAVE), 9 * 1024))
+    e("s_add_u32 %s, %s, %s" % (s(QP), s(QP), s(S0)))
+    e("s_addc_u32 %s, %s, 0" % (s(QP + 1), s(QP + 1)))
+    for ks in range(9):
+        if ks and ks % 4 == 0:
+            e("s_add_u32 %s, %s, 4096" % (s(QP), s(QP)))
+            e("s_addc_u32 %s, %s, 0" % (s(QP + 1), s(QP + 1)))
+        e("global_load_dwordx4 %s, %s, %s offset:%d" % (v(Q0 + 4 * ks, 4), v(X0), s(QP, 2), (ks % 4) * 1024))
+    for cb in range(4):
+        for i in range(16):
+            e("v_accvgpr_write_b32 %s, 0" % a(64 * cb + i))
+    lab_w0, lab_w1, lab_wd = label("pw0"), label("pw1"), label("pwd")
+    e("s_cmp_lt_u32 %s, 2" % s(NT))
+    e("s_cbranch_scc1 %s" % lab_w0)
+    e("s_mov_b32 %s, 1" % s(TMP))
+    for ln in dma_tile_lines(TMP, OFF1, True):
+        e(ln)
+    e("s_cmp_lt_u32 %s, 3" % s(NT))
+    e("s_cbranch_scc1 %s" % lab_w1)
+    e("s_mov_b32 %s, 2" % s(TMP))
+    for ln in dma_tile_lines(TMP, OFF2, True):
+        e(ln)
+    e("s_waitcnt vmcnt(%d)" % (2 * DMA_PER_TILE))
+    e("s_branch %s" % lab_wd)
+    e("%s:" % lab_w1)
+    e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
+    e("s_branch %s" % lab_wd)
+    e("%s:" % lab_w0)
+    e("s_waitcnt vmcnt(0)")
+    e("%s:" % lab_wd)
+    e("v_max_i32 %s, 0, %s" % (v(PAGES), v(PAGES)))
+    e("v_min_i32 %s, %s, %s" % (v(PAGES), s(NPP), v(PAGES)))
+    e("s_barrier")                      # tile 0 is complete
+    e("v_add_u32 %s, %s, %s" % (v(KADDR), s(OFF0), v(KADDR_LANE)))
+    lds.reset([])
+    for slot in ks_scores():
+        slot()
+    ks_exchange_write()
+    for it_ in ks_exchange_read_items():
+        it_()
+    e("s_sub_u32 %s, %s, %s" % (s(NVAL), s(KVE), s(KVB)))
+    e("s_min_u32 %s, %s, 32" % (s(NVAL), s(NVAL)))
+    lds.drain()
+    resc = []
+    ks_tail(True, resc)
+    lab_t1, lab_t1d = label("t1"), label("t1d")
+    e("s_cmp_lt_u32 %s, 3" % s(NT))
+    e("s_cbranch_scc1 %s" % lab_t1)
+    e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
+    e("s_branch %s" % lab_t1d)
+    e("%s:" % lab_t1)
+    e("s_waitcnt vmcnt(0)")
+    e("%s:" % lab_t1d)
+    e("s_barrier")                      # tile 1 is complete; every wave has read the partial tiles
+    # ------------------------------------------------------------------ main loop: tile IT is the one whose P.V comes next
+    lab_loop, lab_last, lab_nodma, lab_dd, lab_end = (label(x) for x in ("loop", "last", "nodma", "dd", "end"))
+    e("%s:" % lab_loop)
+    e("s_mov_b32 %s, 0" % s(VMW))
+    e("v_add_u32 %s, %s, %s" % (v(VADDR), s(OFF0), v(VADDR_LANE)))
+    e("s_add_u32 %s, %s, 1" % (s(TMP), s(IT)))
+    e("s_cmp_ge_u32 %s, %s" % (s(TMP), s(NT)))
+    e("s_cbranch_scc1 %s" % lab_last)
+    e("v_add_u32 %s, %s, %s" % (v(KADDR), s(OFF1), v(KADDR_LANE)))
+    e("s_lshl_b32 %s, %s, 5" % (s(S0), s(TMP)))
+    e("s_add_u32 %s, %s, %s" % (s(S0), s(S0), s(KVB)))
+    e("s_sub_u32 %s, %s, %s" % (s(NVAL), s(KVE), s(S0)))
+    e("s_min_u32 %s, %s, 32" % (s(NVAL), s(NVAL)))                     # valid keys of tile IT+1
+    # part 1: the partial scores of tile IT+1, with the V^T fragments of tile IT (reads, conversion) in their shadow and behind
+    lds.reset([])
+    qk = ks_scores()
+    vit = ks_v_items()
+    n_in = 40 if not F16KV else len(vit)
+    run_slots(qk, 0, [spread(vit[:n_in], 0, 8)])
+    for it_ in vit[n_in:]:
+        emit_item(it_)
+    ks_exchange_write()                 # barrier: every wave is done with tile IT's V rows and tile IT+1's K rows
+    # the buffer of tile IT takes tile IT+3
+    e("s_add_u32 %s, %s, 3" % (s(TMP), s(IT)))
+    e("s_cmp_ge_u32 %s, %s" % (s(TMP), s(NT)))
+    e("s_cbranch_scc1 %s" % lab_nodma)
+    e("s_mov_b32 %s, 1" % s(VMW))
+    for ln in dma_tile_lines(TMP, OFF0):
+        e(ln)
+    e("%s:" % lab_nodma)
+    # part 2: P.V of tile IT (P^T of tile IT is still in S) with the reads of the partial tiles in between; then S <- scores of tile IT+1
+    # (the V^T fragments were waited for before the exchange barrier: ks_exchange_write drains)
+    xr = ks_exchange_read_items()
+    lds.reset([])
+    for n in range(8):
+        ks_pv(n)
+        xr[2 * n]()
+        xr[2 * n + 1]()
+    lds.drain()
+    ks_tail(False, resc)
+    lab_w0b, lab_wdb = label("w0"), label("wd")
+    e("s_cmp_eq_u32 %s, 0" % s(VMW))
+    e("s_cbranch_scc1 %s" % lab_w0b)
+    e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
+    e("s_branch %s" % lab_wdb)
+    e("%s:" % lab_w0b)
+    e("s_waitcnt vmcnt(0)")
+    e("%s:" % lab_wdb)
+    e("s_barrier")                      # tile IT+2 is complete; every wave has read the partial tiles
+    e("s_mov_b32 %s, %s" % (s(TMP), s(OFF0)))
+    e("s_mov_b32 %s, %s" % (s(OFF0), s(OFF1)))
+    e("s_mov_b32 %s, %s" % (s(OFF1), s(OFF2)))
+    e("s_mov_b32 %s, %s" % (s(OFF2), s(TMP)))
+    e("s_add_u32 %s, %s, 1" % (s(IT), s(IT)))
+    e("s_branch %s" % lab_loop)
+    # ---- last tile: P.V only
+    e("%s:" % lab_last)
+    lds.reset([])
+    for it_ in ks_v_items():
+        emit_item(it_)
+    lds.drain()
+    for n in range(8):
+        ks_pv(n)
+    e("s_branch %s" % lab_end)
+    for lab, back in resc:
+        e("%s:" % lab)
+        ks_rescale_block(back)
+    e("%s:" % lab_end)
+    epilogue(1)
+    emit()
+
+
+def emit():
+    print("// generated by gen_decode_cs_asm.py%s%s%s -- do not edit" % (" --ks" if KS else "", " --f16" if F16KV else "", " --mask" if MASK else ""))
     for ln in out:
         print('"%s\\n\\t"' % ln)
     if CLK:
         sys.stderr.write("laps: %s\n" % "; ".join(LAPS))
 
 
-main()
+if KS:
+    ks_main()
+else:
+    main()

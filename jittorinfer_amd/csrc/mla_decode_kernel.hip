@@ -22,7 +22,7 @@ namespace {
 // 32 bytes per thread: mask offset, out pointer, (m,l) pointer, debug pointer
 // The column-split programs (SRC_*_CS) keep behind the four tiles: the P^T exchange buffer (8 KB; the hand-off records share it, they
 // are read before P is first written), the rescale factors (1 KB) and the waves' flag words (64 bytes).
-constexpr bool is_cs(int kvt) { return kvt == SRC_BF16_CS || kvt == SRC_F16_CS; }
+constexpr bool is_cs(int kvt) { return kvt == SRC_BF16_CS || kvt == SRC_F16_CS || kvt == SRC_BF16_KS || kvt == SRC_F16_KS; }
 constexpr int handoff_off(int kvt) { return kvt == SRC_Q8 ? 3 * TILE_BYTES + 2 * Q8_TILE_RAW : 4 * TILE_BYTES; }
 constexpr int SCHED_MAX_SEQ = 256;                   // balanced schedule: sequences per launch
 constexpr int sched_off(int kvt) { return handoff_off(kvt) + (is_cs(kvt) ? 8192 + 1024 + 64 : NTHREADS * 32); }   // prefix sums of the sequences' tile counts
@@ -374,6 +374,14 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
         asm volatile(
 #include "mla_decode_cs_f16_mask.inc"
             : : MLA_DECODE_CS_MASK_INPUTS : MLA_DECODE_CS_CLOBBERS);
+    } else if constexpr (KVT == SRC_BF16_KS) {
+        asm volatile(
+#include "mla_decode_ks_bf16.inc"
+            : : MLA_DECODE_CS_INPUTS : MLA_DECODE_CS_CLOBBERS);
+    } else if constexpr (KVT == SRC_F16_KS) {
+        asm volatile(
+#include "mla_decode_ks_f16.inc"
+            : : MLA_DECODE_CS_INPUTS : MLA_DECODE_CS_CLOBBERS);
     } else if constexpr (KVT == SRC_BF16_CS) {
         asm volatile(
 #include "mla_decode_cs_bf16.inc"
@@ -636,6 +644,13 @@ static bool decode_cs_applicable(const KParams & kp, int kv_type) {
     return (tail == 0 || tail > 96) && kp.slot_rows < (1 << 22);
 }
 
+// At most 32 rows per sequence (a decode step of a 16- or 32-head model): the four waves split the 576 columns of K.Q^T between
+// them instead of leaving it to the one wave that has rows (gen_decode_cs_asm.py --ks)
+static bool decode_ks_applicable(const KParams & kp, int kv_type) {
+    if (kv_type != MLA_TYPE_BF16 && kv_type != MLA_TYPE_F16) return false;
+    return !kp.mask && !kp.bf16_direct && !kp.q_as_q8 && kp.n_rows <= 32 && kp.slot_rows < (1 << 22);
+}
+
 hipError_t launch_decode_fast(const KParams & kp, int kv_type, dim3 grid, hipStream_t st, bool with_prepass) {
     // the small passes ahead of the kernel run per (row block, sequence), whatever the kernel's own grid is
     const unsigned n_rb = (unsigned) ((kp.n_rows + 127) / 128), n_seq = (unsigned) kp.n_seq_sched, extra = kp.balanced == 1 ? 1 : 0;
@@ -644,7 +659,7 @@ hipError_t launch_decode_fast(const KParams & kp, int kv_type, dim3 grid, hipStr
     // has rows (16- and 32-head decode): one computing wave is not bound by its MFMAs, and the hi + lo program is the more exact
     // column-split programs (every wave computes S for its own 32 rows and P.V for its own 128 columns): blocks of 128 rows in
     // which all four waves have rows, not the Q8_0 expansion; bf16 K enters as bf16, so the Q image is the bf16 one
-    const bool cs = decode_cs_applicable(kp, kv_type);
+    const bool cs = decode_cs_applicable(kp, kv_type), ks = decode_ks_applicable(kp, kv_type);
     const bool bf16_cvt = !cs && !kp.bf16_direct && kp.n_rows > 32;
     if (!with_prepass) { /* the workspace still holds the Q image and the mask extents of an earlier launch of the same call */ }
     else if (kv_type == MLA_TYPE_Q8_0 || kp.q_as_q8) hipLaunchKernelGGL(mla_q_pack_q8_kernel, dim3(n_rb, n_seq, KSTEPS / 2 + extra), dim3(NTHREADS), 0, st, kp);
@@ -653,6 +668,7 @@ hipError_t launch_decode_fast(const KParams & kp, int kv_type, dim3 grid, hipStr
     else                              hipLaunchKernelGGL(mla_q_pack_kernel<0>, dim3(n_rb, n_seq, KSTEPS + extra), dim3(NTHREADS), 0, st, kp);
     if (m && with_prepass) hipLaunchKernelGGL(mla_mask_extent_kernel, dim3(n_rb, MASK_EXT_CHUNKS), dim3(NTHREADS), 0, st, kp);
     if (kv_type == MLA_TYPE_Q8_0) return m ? launch_variant<SRC_Q8, true>(kp, grid, st) : launch_variant<SRC_Q8, false>(kp, grid, st);
+    if (ks) return kv_type == MLA_TYPE_F16 ? launch_variant<SRC_F16_KS, false>(kp, grid, st) : launch_variant<SRC_BF16_KS, false>(kp, grid, st);
     if (cs && kv_type == MLA_TYPE_F16) return m ? launch_variant<SRC_F16_CS, true>(kp, grid, st) : launch_variant<SRC_F16_CS, false>(kp, grid, st);
     if (cs)                            return m ? launch_variant<SRC_BF16_CS, true>(kp, grid, st) : launch_variant<SRC_BF16_CS, false>(kp, grid, st);
     if (kv_type == MLA_TYPE_F16)  return m ? launch_variant<SRC_F16, true>(kp, grid, st) : launch_variant<SRC_F16, false>(kp, grid, st);

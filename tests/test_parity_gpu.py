@@ -297,20 +297,31 @@ def test_bf16_direct_program_and_values_beyond_the_f16_range(gpu, masked):
     assert np.isfinite(conv[..., :512][~np.isnan(want)]).all()      # saturated, never infinite
 
 
-def test_bf16_few_rows_keep_the_direct_program(gpu):
-    """With at most 32 attention rows per sequence (a 16- or 32-head decode step) one wave of a workgroup computes and the
-    conversion of the tiles buys nothing: such launches run the hi + lo bf16 program whether the flag is set or not."""
+@pytest.mark.parametrize("k_type", [O.TYPE_BF16, O.TYPE_F16])
+def test_few_rows_k_split_program(gpu, k_type):
+    """At most 32 attention rows per sequence (a decode step of a 16- or 32-head model, 1 or 2 query tokens of 16 heads): the
+    four waves of a workgroup split the 576 columns of K.Q^T and exchange partial score tiles instead of leaving the product
+    to the one wave that has rows.  Paged with KV splits (f16 and f32 partials), one piece per sequence (final rows), lengths
+    that end inside a tile; the 576-wide V in its two passes; MLA_FLAG_BF16_DIRECT still selects the hi + lo bf16 program,
+    which is held more tightly."""
     import jittorinfer_amd as J
     rng = np.random.default_rng(99)
-    lens = [700, 129, 300]
-    pool, bt, seqs = U.make_paged(rng, lens, O.TYPE_BF16)
-    for n_head in (16, 32):
-        q = rng.standard_normal((3, n_head, 1, 576)).astype(np.float32)
-        a = _run(gpu, q, pool, O.TYPE_BF16, bt=bt, lens=lens, scale=U.SCALE)
-        b = _run(gpu, q, pool, O.TYPE_BF16, bt=bt, lens=lens, scale=U.SCALE, flags=J.MLA_FLAG_BF16_DIRECT)
-        assert np.array_equal(a.view(np.int32), b.view(np.int32))
-        want = U.oracle_per_seq(q, seqs, O.TYPE_BF16, 512)
-        print(n_head, U.check(a[..., :512], want, "few rows", max_abs=2e-5, rel_l2=2e-5))
+    lens = [700, 129, 300, 1, 33, 2048]
+    pool, bt, seqs = U.make_paged(rng, lens, k_type)
+    f64 = k_type == O.TYPE_F16     # (ggml-cpu's f16 accumulator: the f32-accumulating kernels are held to the exact value)
+    for n_head, n_tok in ((16, 1), (32, 1), (16, 2), (24, 1)):
+        q = rng.standard_normal((len(lens), n_head, n_tok, 576)).astype(np.float32)
+        want = np.stack([(O.flash_attn_ext_f64 if f64 else O.flash_attn_ext)(q[b:b + 1], k[None], k_type, dv=512, scale=U.SCALE)[0] for b, k in enumerate(seqs)])
+        for n_splits in (0, 1, 3):
+            a = _run(gpu, q, pool, k_type, bt=bt, lens=lens, scale=U.SCALE, n_splits=n_splits)
+            print(n_head, n_tok, n_splits, U.check(a[..., :512], want, "few rows, k-split program"))
+        if k_type == O.TYPE_BF16:
+            b = _run(gpu, q, pool, k_type, bt=bt, lens=lens, scale=U.SCALE, flags=J.MLA_FLAG_BF16_DIRECT)
+            print(n_head, U.check(b[..., :512], want, "few rows, hi + lo program", max_abs=2e-5, rel_l2=2e-5))
+    q = rng.standard_normal((len(lens), 16, 1, 576)).astype(np.float32)
+    a = _run(gpu, q, pool, k_type, dv=576, bt=bt, lens=lens, scale=U.SCALE)
+    want = np.stack([(O.flash_attn_ext_f64 if f64 else O.flash_attn_ext)(q[b:b + 1], k[None], k_type, dv=576, scale=U.SCALE)[0] for b, k in enumerate(seqs)])
+    print(U.check(a, want, "few rows, V := K"))
 
 
 def test_q8_0_cache_with_arbitrary_block_scales(gpu):
