@@ -498,28 +498,19 @@ __global__ void __launch_bounds__(256) mla_attn_combine_kernel(const KParams p) 
 // The same merge over f32 partials (rows of dv_total floats; small problems).  One thread = one (row, group of 4 columns),
 // lanes along the columns of a row.  grid = (ceil(rows/2), 1, n_seq), block = 256 = 2 rows x 128 column groups (dv <= 512)
 // or (rows, 1, n_seq) with 144 active threads for dv = 576: blockDim covers one or two rows, see the launch.
-__global__ void __launch_bounds__(256) mla_attn_combine_f32_kernel(const KParams p, int groups_per_row) {
-    const int b = blockIdx.z;
-    const int rows_per_block = 256 / groups_per_row;
-    const int row = blockIdx.x * rows_per_block + threadIdx.x / groups_per_row;
-    const int cg  = threadIdx.x % groups_per_row;
-    const int seq_len = p.block_table ? min(p.seq_lens[b], (int) p.bt_stride * MLA_PAGE_TOKENS) : (int) p.n_kv;
-    if (row >= p.n_rows || threadIdx.x >= rows_per_block * groups_per_row || cg * 4 >= p.dv_total) return;
-    int slot0, nvalid, lrow;
-    partial_slots(p, b, row, seq_len, slot0, nvalid, lrow);
-    if (nvalid < 0) return;
-    const float2 * ml = (const float2 *) p.part_ml + (int64_t) slot0 * p.slot_rows + lrow;
-    const float *  po = (const float *) p.part_o + ((int64_t) slot0 * p.slot_rows + lrow) * p.dv_total + cg * 4;
-    const int64_t ml_step = p.slot_rows, po_step = (int64_t) p.slot_rows * p.dv_total;
-    constexpr int G = 32;   // small problems are latency-bound: a ragged batch has up to 32 one-page pieces per sequence, all in flight at once
+// G splits are loaded together (a split past the end is a duplicate of the last one with weight 0): small problems are
+// latency-bound, so the group should cover every split of a row in one round -- a ragged batch of short sequences has up to 32
+// one-page pieces per sequence -- without issuing many times the loads a row with two or three splits needs.
+template <int G>
+__device__ __forceinline__ void combine_f32_row(const KParams & p, const float2 * ml, const float * po, int64_t ml_step, int64_t po_step, int nvalid, float * dst) {
     float M = -INFINITY, L = 0.f;
     f32x4 o = { 0.f, 0.f, 0.f, 0.f };
-    for (int c0 = 0; c0 < nvalid; c0 += G) {   // groups of G splits: their loads are in flight together
+    for (int c0 = 0; c0 < nvalid; c0 += G) {
         float2 mlv[G];
         f32x4  xv[G];
 #pragma unroll
         for (int k = 0; k < G; k++) {
-            const int c = min(c0 + k, nvalid - 1);  // past the end: a duplicate of the last split, given weight 0 below
+            const int c = min(c0 + k, nvalid - 1);
             mlv[k] = ml[c * ml_step];
             xv[k]  = *(const f32x4 *) (po + c * po_step);
         }
@@ -540,7 +531,26 @@ __global__ void __launch_bounds__(256) mla_attn_combine_f32_kernel(const KParams
         }
     }
     const float inv = 1.0f / L;  // no valid key at all: 0 * inf = NaN, like the reference
-    *(f32x4 *) (p.dst + ((int64_t) b * p.n_rows + row) * p.dst_stride + p.v_col0 + cg * 4) = f32x4{ o.x * inv, o.y * inv, o.z * inv, o.w * inv };
+    *(f32x4 *) dst = f32x4{ o.x * inv, o.y * inv, o.z * inv, o.w * inv };
+}
+
+__global__ void __launch_bounds__(256) mla_attn_combine_f32_kernel(const KParams p, int groups_per_row) {
+    const int b = blockIdx.z;
+    const int rows_per_block = 256 / groups_per_row;
+    const int row = blockIdx.x * rows_per_block + threadIdx.x / groups_per_row;
+    const int cg  = threadIdx.x % groups_per_row;
+    const int seq_len = p.block_table ? min(p.seq_lens[b], (int) p.bt_stride * MLA_PAGE_TOKENS) : (int) p.n_kv;
+    if (row >= p.n_rows || threadIdx.x >= rows_per_block * groups_per_row || cg * 4 >= p.dv_total) return;
+    int slot0, nvalid, lrow;
+    partial_slots(p, b, row, seq_len, slot0, nvalid, lrow);
+    if (nvalid < 0) return;
+    const float2 * ml = (const float2 *) p.part_ml + (int64_t) slot0 * p.slot_rows + lrow;
+    const float *  po = (const float *) p.part_o + ((int64_t) slot0 * p.slot_rows + lrow) * p.dv_total + cg * 4;
+    const int64_t ml_step = p.slot_rows, po_step = (int64_t) p.slot_rows * p.dv_total;
+    float * dst = p.dst + ((int64_t) b * p.n_rows + row) * p.dst_stride + p.v_col0 + cg * 4;
+    if (nvalid <= 4)       combine_f32_row<4>(p, ml, po, ml_step, po_step, nvalid, dst);
+    else if (nvalid <= 16) combine_f32_row<16>(p, ml, po, ml_step, po_step, nvalid, dst);
+    else                   combine_f32_row<32>(p, ml, po, ml_step, po_step, nvalid, dst);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
