@@ -100,24 +100,23 @@ class MlaKvWriteArgs(C.Structure):
 
 
 _workspaces = {}
+_retired = []
 
 
 def _workspace(device, nbytes, stream=None):
     """The scratch area of a launch: one per (device, stream) -- launches on different streams run side by side and each
-    needs its own partials, Q image and schedule -- and grow-only.  Growing waits for the stream first (launches already
-    queued still use the old area) and is refused while the stream is being captured into a graph, whose replays would
-    keep the address of an area that no longer exists: size the first, uncaptured call for the largest batch."""
+    needs its own partials, Q image and schedule -- and grow-only.  An area that has been handed out is never freed: a
+    launch queued on another thread's behalf or recorded into a HIP graph keeps its address, so a larger request gets a new
+    area and the old one is only retired (a few tens of MB per size step).  Under graph capture the new area comes from the
+    graph's own memory pool, like any tensor made during capture."""
     import torch
     if stream is None:
         stream = torch.cuda.current_stream(device).cuda_stream
     key = (device, int(stream))
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
-        if torch.cuda.is_current_stream_capturing():
-            raise RuntimeError("the attention workspace would have to %s during graph capture: run one launch of the largest "
-                               "shape on this stream before capturing" % ("grow" if ws is not None else "be allocated"))
         if ws is not None:
-            torch.cuda.synchronize(device)
+            _retired.append(ws)
         ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws

@@ -554,7 +554,7 @@ __global__ void __launch_bounds__(NTHREADS) mla_q_pack_q8_kernel(const KParams p
 
 }  // namespace
 
-size_t decode_fast_lds_bytes(int kv_type) { return (size_t) lds_total(kv_type == MLA_TYPE_Q8_0 ? SRC_Q8 : SRC_BF16); }
+size_t decode_fast_lds_bytes(int kv_type) { return (size_t) lds_total(kv_type == MLA_TYPE_Q8_0 ? SRC_Q8 : SRC_BF16_CS); }   // (the largest of the programs for that type)
 
 size_t decode_fast_qpack_bytes(int n_seq, int n_row_blocks) { return (size_t) n_seq * n_row_blocks * 4 * KSTEPS * 1024; }
 

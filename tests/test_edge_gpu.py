@@ -476,10 +476,10 @@ def test_balanced_schedule_of_a_masked_launch_with_many_row_blocks(gpu):
     print(U.check(got[..., :512], want, "masked launch, balanced schedule"))
 
 
-def test_workspace_is_per_stream_and_does_not_grow_under_capture(gpu):
-    """The binding keeps one scratch area per (device, stream): launches on two streams must not share partials, a
-    larger launch on a stream gets a larger area after the stream has drained, and growth during graph capture is refused
-    (the graph would replay into freed memory)."""
+def test_workspace_is_per_stream_and_survives_growth_and_capture(gpu):
+    """The binding keeps one scratch area per (device, stream): launches on two streams must not share partials; a larger
+    launch gets a new area while the old one stays allocated (a graph that recorded its address replays correctly
+    afterwards); a first launch on a stream that is being captured allocates from the graph's pool and replays correctly."""
     import torch
     import jittorinfer_amd as J
     rng = np.random.default_rng(3)
@@ -488,6 +488,7 @@ def test_workspace_is_per_stream_and_does_not_grow_under_capture(gpu):
     tq, tk = torch.from_numpy(q).to(gpu), torch.from_numpy(pool.view(np.int16)).to(gpu)
     tb, tl = torch.from_numpy(bt).to(gpu), torch.tensor([900, 700], dtype=torch.int32, device=gpu)
     kw = dict(dv=512, scale=U.SCALE, block_table=tb, seq_lens=tl)
+    want = U.oracle_per_seq(q, seqs, O.TYPE_BF16, 512)
     s1, s2 = torch.cuda.Stream(gpu), torch.cuda.Stream(gpu)
     torch.cuda.synchronize()
     with torch.cuda.stream(s1):
@@ -501,16 +502,24 @@ def test_workspace_is_per_stream_and_does_not_grow_under_capture(gpu):
         r2 = J.ggml_flash_attn_ext(tq, tk, J.MLA_TYPE_BF16, **kw)
     torch.cuda.synchronize()
     assert torch.equal(r1[..., :512], r2[..., :512])
-    print(U.check(r1.cpu().numpy()[..., :512], U.oracle_per_seq(q, seqs, O.TYPE_BF16, 512), "two streams"))
-    # a stream that has never launched, under capture: no area yet, and none may be made now
-    s3 = torch.cuda.Stream(gpu)
+    print(U.check(r1.cpu().numpy()[..., :512], want, "two streams"))
+    # a stream that has never launched, under capture (what `with torch.cuda.graph(g):` does): the area is made then and there
+    out3 = torch.zeros((2, 1, 128, 576), dtype=torch.float32, device=gpu)
     graph = torch.cuda.CUDAGraph()
-    out3, one = torch.zeros((2, 1, 128, 576), dtype=torch.float32, device=gpu), torch.zeros(1, device=gpu)
     torch.cuda.synchronize()
-    with torch.cuda.stream(s3):
-        graph.capture_begin()
-        one.add_(1.0)
-        with pytest.raises(RuntimeError, match="graph capture"):
-            J.capi.make_args(tq, tk, J.MLA_TYPE_BF16, out=out3, **kw)
-        graph.capture_end()
+    with torch.cuda.graph(graph):
+        J.ggml_flash_attn_ext(tq, tk, J.MLA_TYPE_BF16, out=out3, **kw)
     torch.cuda.synchronize()
+    # a much larger launch on the first stream replaces its area; the graph and the earlier argument block keep theirs
+    big_pool, big_bt, _ = U.make_paged(rng, [128] * 64, O.TYPE_BF16)
+    bq = torch.from_numpy(rng.standard_normal((64, 128, 1, 576)).astype(np.float32)).to(gpu)
+    with torch.cuda.stream(s1):
+        J.ggml_flash_attn_ext(bq, torch.from_numpy(big_pool.view(np.int16)).to(gpu), J.MLA_TYPE_BF16, dv=512, scale=U.SCALE,
+                              block_table=torch.from_numpy(big_bt).to(gpu), seq_lens=torch.full((64,), 128, dtype=torch.int32, device=gpu), n_splits=1)
+    torch.cuda.synchronize()
+    for it in range(2):
+        out3.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out3[..., :512], r1[..., :512]), "replay %d" % it
