@@ -78,6 +78,7 @@ struct KParams {
     int             q_as_q8;       // the KV rows are the f16 expansion of a Q8_0 cache: Q is quantized the Q8_0 way
     int             bf16_direct;   // bf16 KV: the hi + lo program instead of the one that converts the tiles to f16 (MLA_FLAG_BF16_DIRECT)
     int             rows_contig;  // kv rows are packed (kv_nb1 == row bytes): whole tiles are one contiguous run
+    int             mask_ext_in_pack;  // Q pre-pack launch: its last 16 layers of blocks scan the mask extents
 };
 
 template <typename T, typename U> __device__ __forceinline__ T bitcast(U u) { return __builtin_bit_cast(T, u); }

@@ -427,51 +427,19 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
   }
 }
 
-// Q f32 -> the decode kernel's MFMA operand image, rounded to the KV type as ggml-cpu rounds it (ggml-cpu.c:12034-12035):
-// out[((seq*n_row_blocks + rb)*4 + wave)*36 + ks][lane] = 8 values of row rb*128 + wave*32 + lane%32,
-// columns 16*ks + 8*(lane/32) .. +7.  Rows past n_rows repeat the last row (their results are never stored);
-// a group of 32 rows that lies past n_rows entirely is left unwritten, its wave of the decode kernel neither loads nor computes.
-// grid = (n_row_blocks, n_seq, 36 k-steps), block = 256: one 16-byte output per thread.
-// MODE 0: bf16 operands; 1: f16; 2: rounded to bf16 as for MODE 0, then written as f16 (exact inside the f16 range,
-// +-65504 beyond it) for the program that converts its bf16 tiles to f16.
-template <int MODE> __device__ __forceinline__ unsigned int pack_q2(float a, float b) {
-    if constexpr (MODE == 2) {
-        const auto h = __builtin_amdgcn_cvt_pkrtz(round_trip<false>(a), round_trip<false>(b));
-        return bitcast<unsigned int>(h);
-    } else return pack2<MODE == 1>(a, b);
-}
-template <int MODE>
-__global__ void __launch_bounds__(NTHREADS) mla_q_pack_kernel(const KParams p) {
-    if (blockIdx.z == gridDim.z - 1 && p.balanced == 1) {   // balanced schedule: one extra layer of blocks, the first of which builds it
-        if (blockIdx.x == 0 && blockIdx.y == 0) sched_prefix(p);
-        return;
-    }
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int g = lane >> 5, rl = lane & 31;
-    const int b = blockIdx.y, ks = blockIdx.z;
-    if ((int) blockIdx.x * 128 + wave * 32 >= p.n_rows) return;   // a wave of the decode kernel without a row: it computes nothing, its image is never used
-    const int row = min((int) blockIdx.x * 128 + wave * 32 + rl, p.n_rows - 1);
-    const int tq = row / p.n_head, head = row - tq * p.n_head;
-    const float * qrow = (const float *) (p.q + (int64_t) tq * p.q_nb1 + (int64_t) head * p.q_nb2 + (int64_t) b * p.q_nb3) + 8 * g;
-    u32x4 * out = (u32x4 *) p.q_pack + ((((int64_t) b * gridDim.x + blockIdx.x) * 4 + wave) * KSTEPS) * 64 + lane;
-    const f32x4 x0 = *(const f32x4 *) (qrow + 16 * ks);
-    const f32x4 x1 = *(const f32x4 *) (qrow + 16 * ks + 4);
-    out[ks * 64] = u32x4{ pack_q2<MODE>(x0.x, x0.y), pack_q2<MODE>(x0.z, x0.w), pack_q2<MODE>(x1.x, x1.y), pack_q2<MODE>(x1.z, x1.w) };
-}
-
 // Per block of 128 rows and per sixteenth of the mask row: the first key and one past the last key that any of the
 // block's query tokens may attend to (mask value != -inf); n_kv, 0 when there is none.  The attention kernel merges the
 // 16 pairs and rounds outwards to tiles.  grid = (n_row_blocks, 16), block = 256.  The mask is shared by all sequences
 // (ggml-cpu.c:12024).
 constexpr int MASK_EXT_CHUNKS = 16;
-__global__ void __launch_bounds__(NTHREADS) mla_mask_extent_kernel(const KParams p) {
+__device__ __forceinline__ void mask_extent_block(const KParams & p, int rb, int chunk) {
     __shared__ int red_hi[NTHREADS], red_lo[NTHREADS];
     const int tid = threadIdx.x;
-    const int r0 = blockIdx.x * 128, r1 = min(r0 + 127, p.n_rows - 1);
+    const int r0 = rb * 128, r1 = min(r0 + 127, p.n_rows - 1);
     const int t0 = r0 / p.n_head, t1 = r1 / p.n_head;
     const int n_kv = (int) (p.block_table ? p.bt_stride * MLA_PAGE_TOKENS : p.n_kv);
     const int n8 = n_kv / 8;   // groups of 8 mask values (16 bytes); n_kv is a multiple of 32 on this path
-    const int g0 = (int) ((int64_t) n8 * blockIdx.y / MASK_EXT_CHUNKS), g1 = (int) ((int64_t) n8 * (blockIdx.y + 1) / MASK_EXT_CHUNKS);
+    const int g0 = (int) ((int64_t) n8 * chunk / MASK_EXT_CHUNKS), g1 = (int) ((int64_t) n8 * (chunk + 1) / MASK_EXT_CHUNKS);
     int hi = 0, lo = n_kv;
     for (int t = t0; t <= t1; t++) {
         const char * mrow = p.mask + (int64_t) t * p.mask_nb1;
@@ -509,16 +477,58 @@ __global__ void __launch_bounds__(NTHREADS) mla_mask_extent_kernel(const KParams
         __syncthreads();
     }
     if (tid == 0) {
-        p.mask_ext[(blockIdx.x * MASK_EXT_CHUNKS + blockIdx.y) * 2]     = red_lo[0];
-        p.mask_ext[(blockIdx.x * MASK_EXT_CHUNKS + blockIdx.y) * 2 + 1] = red_hi[0];
+        p.mask_ext[(rb * MASK_EXT_CHUNKS + chunk) * 2]     = red_lo[0];
+        p.mask_ext[(rb * MASK_EXT_CHUNKS + chunk) * 2 + 1] = red_hi[0];
     }
 }
+__global__ void __launch_bounds__(NTHREADS) mla_mask_extent_kernel(const KParams p) { mask_extent_block(p, blockIdx.x, blockIdx.y); }
 
+// The pipelined kernel's launches fold the extent scan into the Q pre-pack launch: MASK_EXT_CHUNKS more layers of blocks behind
+// the pack layers (one launch and one dispatch hand-over less ahead of the decode kernel).  True when this block was one of them.
+__device__ __forceinline__ bool pack_launch_extent_layer(const KParams & p) {
+    if (!p.mask_ext_in_pack || blockIdx.z + MASK_EXT_CHUNKS < gridDim.z) return false;
+    if (blockIdx.y == 0) mask_extent_block(p, blockIdx.x, (int) (blockIdx.z + MASK_EXT_CHUNKS - gridDim.z));
+    return true;
+}
+
+// Q f32 -> the decode kernel's MFMA operand image, rounded to the KV type as ggml-cpu rounds it (ggml-cpu.c:12034-12035):
+// out[((seq*n_row_blocks + rb)*4 + wave)*36 + ks][lane] = 8 values of row rb*128 + wave*32 + lane%32,
+// columns 16*ks + 8*(lane/32) .. +7.  Rows past n_rows repeat the last row (their results are never stored);
+// a group of 32 rows that lies past n_rows entirely is left unwritten, its wave of the decode kernel neither loads nor computes.
+// grid = (n_row_blocks, n_seq, 36 k-steps), block = 256: one 16-byte output per thread.
+// MODE 0: bf16 operands; 1: f16; 2: rounded to bf16 as for MODE 0, then written as f16 (exact inside the f16 range,
+// +-65504 beyond it) for the program that converts its bf16 tiles to f16.
+template <int MODE> __device__ __forceinline__ unsigned int pack_q2(float a, float b) {
+    if constexpr (MODE == 2) {
+        const auto h = __builtin_amdgcn_cvt_pkrtz(round_trip<false>(a), round_trip<false>(b));
+        return bitcast<unsigned int>(h);
+    } else return pack2<MODE == 1>(a, b);
+}
+template <int MODE>
+__global__ void __launch_bounds__(NTHREADS) mla_q_pack_kernel(const KParams p) {
+    if (pack_launch_extent_layer(p)) return;
+    if (blockIdx.z == gridDim.z - 1 && p.balanced == 1) {   // balanced schedule: one extra layer of blocks, the first of which builds it
+        if (blockIdx.x == 0 && blockIdx.y == 0) sched_prefix(p);
+        return;
+    }
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int g = lane >> 5, rl = lane & 31;
+    const int b = blockIdx.y, ks = blockIdx.z;
+    if ((int) blockIdx.x * 128 + wave * 32 >= p.n_rows) return;   // a wave of the decode kernel without a row: it computes nothing, its image is never used
+    const int row = min((int) blockIdx.x * 128 + wave * 32 + rl, p.n_rows - 1);
+    const int tq = row / p.n_head, head = row - tq * p.n_head;
+    const float * qrow = (const float *) (p.q + (int64_t) tq * p.q_nb1 + (int64_t) head * p.q_nb2 + (int64_t) b * p.q_nb3) + 8 * g;
+    u32x4 * out = (u32x4 *) p.q_pack + ((((int64_t) b * gridDim.x + blockIdx.x) * 4 + wave) * KSTEPS) * 64 + lane;
+    const f32x4 x0 = *(const f32x4 *) (qrow + 16 * ks);
+    const f32x4 x1 = *(const f32x4 *) (qrow + 16 * ks + 4);
+    out[ks * 64] = u32x4{ pack_q2<MODE>(x0.x, x0.y), pack_q2<MODE>(x0.z, x0.w), pack_q2<MODE>(x1.x, x1.y), pack_q2<MODE>(x1.z, x1.w) };
+}
 
 // The same image for Q8_0 KV: ggml-cpu quantizes Q to Q8_0 when K is Q8_0 (ggml-cpu.c:313-322, :12034-12035): per block of 32
 // d = amax/127 (stored as f16), id = 127/amax, q = round-half-even(x*id) (ggml-cpu-quants.c:855-900); the MFMA operand is the
 // dequantized value q * f16(d), rounded to f16.  grid = (n_row_blocks, n_seq, 18 blocks), block = 256: two k-steps per thread.
 __global__ void __launch_bounds__(NTHREADS) mla_q_pack_q8_kernel(const KParams p) {
+    if (pack_launch_extent_layer(p)) return;
     if (blockIdx.z == gridDim.z - 1 && p.balanced == 1) {   // balanced schedule: one extra layer of blocks, the first of which builds it
         if (blockIdx.x == 0 && blockIdx.y == 0) sched_prefix(p);
         return;
@@ -661,12 +671,18 @@ hipError_t launch_decode_fast(const KParams & kp, int kv_type, dim3 grid, hipStr
     // which all four waves have rows, not the Q8_0 expansion; bf16 K enters as bf16, so the Q image is the bf16 one
     const bool cs = decode_cs_applicable(kp, kv_type), ks = decode_ks_applicable(kp, kv_type);
     const bool bf16_cvt = !cs && !kp.bf16_direct && kp.n_rows > 32;
+    // the scan of the mask extents rides in the pack launch (a masked launch has no balanced page schedule, so its layers and the
+    // schedule layer never meet; if they ever did, the scan would keep a launch of its own)
+    const bool fold = m && !extra;
+    KParams pk = kp;
+    pk.mask_ext_in_pack = fold ? 1 : 0;
+    const unsigned ext = fold ? MASK_EXT_CHUNKS : 0;
     if (!with_prepass) { /* the workspace still holds the Q image and the mask extents of an earlier launch of the same call */ }
-    else if (kv_type == MLA_TYPE_Q8_0 || kp.q_as_q8) hipLaunchKernelGGL(mla_q_pack_q8_kernel, dim3(n_rb, n_seq, KSTEPS / 2 + extra), dim3(NTHREADS), 0, st, kp);
-    else if (kv_type == MLA_TYPE_F16) hipLaunchKernelGGL(mla_q_pack_kernel<1>, dim3(n_rb, n_seq, KSTEPS + extra), dim3(NTHREADS), 0, st, kp);
-    else if (bf16_cvt)                hipLaunchKernelGGL(mla_q_pack_kernel<2>, dim3(n_rb, n_seq, KSTEPS + extra), dim3(NTHREADS), 0, st, kp);
-    else                              hipLaunchKernelGGL(mla_q_pack_kernel<0>, dim3(n_rb, n_seq, KSTEPS + extra), dim3(NTHREADS), 0, st, kp);
-    if (m && with_prepass) hipLaunchKernelGGL(mla_mask_extent_kernel, dim3(n_rb, MASK_EXT_CHUNKS), dim3(NTHREADS), 0, st, kp);
+    else if (kv_type == MLA_TYPE_Q8_0 || kp.q_as_q8) hipLaunchKernelGGL(mla_q_pack_q8_kernel, dim3(n_rb, n_seq, KSTEPS / 2 + extra + ext), dim3(NTHREADS), 0, st, pk);
+    else if (kv_type == MLA_TYPE_F16) hipLaunchKernelGGL(mla_q_pack_kernel<1>, dim3(n_rb, n_seq, KSTEPS + extra + ext), dim3(NTHREADS), 0, st, pk);
+    else if (bf16_cvt)                hipLaunchKernelGGL(mla_q_pack_kernel<2>, dim3(n_rb, n_seq, KSTEPS + extra + ext), dim3(NTHREADS), 0, st, pk);
+    else                              hipLaunchKernelGGL(mla_q_pack_kernel<0>, dim3(n_rb, n_seq, KSTEPS + extra + ext), dim3(NTHREADS), 0, st, pk);
+    if (m && !fold && with_prepass) hipLaunchKernelGGL(mla_mask_extent_kernel, dim3(n_rb, MASK_EXT_CHUNKS), dim3(NTHREADS), 0, st, kp);
     if (kv_type == MLA_TYPE_Q8_0) return m ? launch_variant<SRC_Q8, true>(kp, grid, st) : launch_variant<SRC_Q8, false>(kp, grid, st);
     if (ks) return kv_type == MLA_TYPE_F16 ? launch_variant<SRC_F16_KS, false>(kp, grid, st) : launch_variant<SRC_BF16_KS, false>(kp, grid, st);
     if (cs && kv_type == MLA_TYPE_F16) return m ? launch_variant<SRC_F16_CS, true>(kp, grid, st) : launch_variant<SRC_F16_CS, false>(kp, grid, st);
