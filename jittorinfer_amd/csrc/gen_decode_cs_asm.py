@@ -682,9 +682,10 @@ def iteration(resc, lab_loop):
     lds.drain()
 
 
-def prologue_head():
+def prologue_head(early=None):
     """Inputs -> fixed registers, lane geometry, the page ids of the piece, running state, the tile loads' offset table; ends
-    when tile 0 can be requested."""
+    when tile 0 can be requested.  early: emitted once the wave and lane numbers are known (loads that should be on their way
+    while the rest is set up; v[36:167] and the scalar temporaries are its own until the end of the prologue)."""
     # ------------------------------------------------------------------ entry: inputs -> fixed registers
     e("s_mov_b64 %s, %%[kv]" % s(KV, 2))
     e("s_mov_b64 %s, %%[bt]" % s(BT, 2))
@@ -717,6 +718,8 @@ def prologue_head():
     e("s_add_u32 %s, %s, 0x%x" % (s(FADR), s(W4), FOFF))
     clk_init()
     lap(-1)
+    if early:
+        early()
     # lane geometry
     e("v_and_b32 %s, 31, %s" % (v(X0), v(LANE)))                       # rl
     e("v_lshrrev_b32 %s, 5, %s" % (v(X1), v(LANE)))                    # g
@@ -798,8 +801,24 @@ def prologue_head():
 
 def main():
     prologue_head()
-    # ------------------------------------------------------------------ tile 0, then the Q operands (36 coalesced 16-byte loads per
-    # lane from the packed image), then tiles 1 and 2; go on as soon as tile 0 and Q are there
+    # ------------------------------------------------------------------ the Q operands and tile 0.  FLG bit 6: the C++ prologue left this
+    # wave's 32 rows, rounded to the KV type, in tile buffer `wave` in the layout of a KV tile, so an operand is read like a K
+    # fragment, and once every wave has its operands the buffers are free for tile 0.  Otherwise: tile 0, then the operands from the
+    # packed image (36 coalesced 16-byte loads per lane).  Tiles 1 and 2 follow; go on as soon as tile 0 and Q are there
+    lab_img, lab_qd = label("qimg"), label("qdone")
+    e("s_bitcmp1_b32 %s, 6" % s(FLG))
+    e("s_cbranch_scc0 %s" % lab_img)
+    e("s_mul_i32 %s, %s, %d" % (s(S0), s(WAVE), TILE_BYTES))
+    e("v_add_u32 %s, %s, %s" % (v(X0), s(S0), v(KADDR_LANE)))
+    for ks in range(36):
+        e("ds_read_b128 %s, %s offset:%d" % (v(Q0 + 4 * ks, 4), v(X0), 32 * ks))
+    e("s_waitcnt lgkmcnt(0)")
+    e("s_barrier")
+    e("s_mov_b32 %s, 0" % s(TMP))
+    for ln in dma_tile_lines(TMP, OFF0, True):
+        e(ln)
+    e("s_branch %s" % lab_qd)
+    e("%s:" % lab_img)
     e("s_mov_b32 %s, 0" % s(TMP))
     for ln in dma_tile_lines(TMP, OFF0, True):
         e(ln)
@@ -812,6 +831,7 @@ def main():
             e("s_add_u32 %s, %s, 4096" % (s(QP), s(QP)))
             e("s_addc_u32 %s, %s, 0" % (s(QP + 1), s(QP + 1)))
         e("global_load_dwordx4 %s, %s, %s offset:%d" % (v(Q0 + 4 * ks, 4), v(X0), s(QP, 2), (ks % 4) * 1024))
+    e("%s:" % lab_qd)
     if MASK:
         # mask rows start at key kv_begin of this piece; QP's registers and X0 are free now
         e("s_mov_b64 %s, %%[msk]" % s(MSK, 2))
@@ -1119,52 +1139,107 @@ def ks_tail(first_tile, resc):
         resc.append((lab_resc, lab_back))
 
 
+KS_RP, KS_LOFF, KS_WADDR, KS_BUF = 164, 166, 167, 36
+
+
+def ks_q_issue():
+    """The loads of this wave's quarter of Q (144 columns of the 32 rows, f32 in global memory), first thing in the program: their
+    way to the MFMA operands is the longest (registers, rounding, LDS, registers).  Where each row's quarter starts comes from a
+    table the C++ prologue left behind the exchange buffer (lane r of the table read holds row r's address); one 16-byte load per
+    lane and row, lanes past the 36th repeat the 36th."""
+    pairs = [S0, S2, QP, SB]
+    e("v_and_b32 %s, 31, %s" % (v(X0), v(LANE)))
+    e("v_lshlrev_b32 %s, 3, %s" % (v(X0), v(X0)))
+    e("s_lshl_b32 %s, %s, 8" % (s(S0), s(WAVE)))
+    e("s_add_u32 %s, %s, 0x%x" % (s(S0), s(S0), AOFF))
+    e("v_add_u32 %s, %s, %s" % (v(X0), s(S0), v(X0)))
+    e("ds_read_b64 %s, %s" % (v(KS_RP, 2), v(X0)))
+    e("v_min_u32 %s, 35, %s" % (v(X1), v(LANE)))
+    e("v_lshlrev_b32 %s, 4, %s" % (v(KS_LOFF), v(X1)))                 # byte offset of the lane's load inside the quarter row
+    e("v_lshlrev_b32 %s, 3, %s" % (v(X1), v(X1)))
+    e("s_mul_i32 %s, %s, 288" % (s(S0), s(WAVE)))
+    e("s_add_u32 %s, %s, %d" % (s(S0), s(S0), 2 * TILE_BYTES))
+    e("v_add_u32 %s, %s, %s" % (v(KS_WADDR), s(S0), v(X1)))            # where the lane's 8 bytes of row 0 go: tile buffer 2
+    e("s_waitcnt lgkmcnt(0)")
+    for batch in range(8):
+        for j in range(4):
+            r = 4 * batch + j
+            e("v_readlane_b32 %s, %s, %d" % (s(pairs[j]), v(KS_RP), r))
+            e("v_readlane_b32 %s, %s, %d" % (s(pairs[j] + 1), v(KS_RP + 1), r))
+        e("s_nop 4")                                                   # a lane read's scalar result may not be an address for 5 cycles
+        for j in range(4):
+            r = 4 * batch + j
+            e("global_load_dwordx4 %s, %s, %s" % (v(KS_BUF + 4 * r, 4), v(KS_LOFF), s(pairs[j], 2)))
+
+
+def ks_q_round(behind):
+    """The quarter of Q, as it arrives, -> tile buffer 2, rounded to the KV type (to nearest even, as ggml-cpu rounds Q:
+    ggml-cpu.c:12034-12035) in the layout of a KV tile.  behind: loads issued after the last of Q's (None: wait for everything)."""
+    cvt = "v_cvt_pk_f16_f32" if F16KV else "v_cvt_pk_bf16_f32"
+    if behind is None:
+        e("s_waitcnt vmcnt(0)")
+    for r in range(32):
+        b = KS_BUF + 4 * r
+        if behind is not None:
+            e("s_waitcnt vmcnt(%d)" % (31 - r + behind))
+        e("%s %s, %s, %s" % (cvt, v(b), v(b), v(b + 1)))
+        e("%s %s, %s, %s" % (cvt, v(b + 1), v(b + 2), v(b + 3)))
+        e("ds_write_b64 %s, %s offset:%d" % (v(KS_WADDR), v(b, 2), r * PITCH))
+    e("s_waitcnt lgkmcnt(0)")
+
+
 def ks_main():
     assert not MASK and not CLK
-    prologue_head()
+    prologue_head(ks_q_issue)
     e("s_mul_i32 %s, %s, 288" % (s(S0), s(WAVE)))                      # this wave's k-steps 9 w ..: 32 bytes each
     e("v_add_u32 %s, %s, %s" % (v(KADDR_LANE), s(S0), v(KADDR_LANE)))
     e("v_lshlrev_b32 %s, 4, %s" % (v(PADDR), v(LANE)))
     e("v_add_u32 %s, 0x%x, %s" % (v(PADDR), XOFF, v(PADDR)))
     e("s_lshl_b32 %s, %s, 12" % (s(WOFS), s(WAVE)))
-    # ------------------------------------------------------------------ tile 0, the wave's quarter of the Q operands, tiles 1 and 2
+    # ------------------------------------------------------------------ tiles 0 and 1 are requested; the wave's quarter of Q (on its way
+    # since the top of the program) goes through tile buffer 2 (every wave its own columns of the 32 rows, in the layout of a KV
+    # tile: an operand is read like a K fragment); tile 2 is requested once every wave has its operands
     e("s_mov_b32 %s, 0" % s(TMP))
     for ln in dma_tile_lines(TMP, OFF0, True):
         e(ln)
-    e("v_lshlrev_b32 %s, 4, %s" % (v(X0), v(LANE)))
-    e("s_mul_i32 %s, %s, %d" % (s(S0), s(WAVE), 9 * 1024))
-    e("s_add_u32 %s, %s, %s" % (s(QP), s(QP), s(S0)))
-    e("s_addc_u32 %s, %s, 0" % (s(QP + 1), s(QP + 1)))
-    for ks in range(9):
-        if ks and ks % 4 == 0:
-            e("s_add_u32 %s, %s, 4096" % (s(QP), s(QP)))
-            e("s_addc_u32 %s, %s, 0" % (s(QP + 1), s(QP + 1)))
-        e("global_load_dwordx4 %s, %s, %s offset:%d" % (v(Q0 + 4 * ks, 4), v(X0), s(QP, 2), (ks % 4) * 1024))
-    for cb in range(4):
-        for i in range(16):
-            e("v_accvgpr_write_b32 %s, 0" % a(64 * cb + i))
-    lab_w0, lab_w1, lab_wd = label("pw0"), label("pw1"), label("pwd")
+    # behind Q's loads: the page ids (when there is a table; counted as absent, which at worst waits for one load more) and the
+    # 10 loads of each tile
+    lab_w0, lab_wd, lab_qr = label("pw0"), label("pwd"), label("qr")
     e("s_cmp_lt_u32 %s, 2" % s(NT))
     e("s_cbranch_scc1 %s" % lab_w0)
     e("s_mov_b32 %s, 1" % s(TMP))
     for ln in dma_tile_lines(TMP, OFF1, True):
         e(ln)
+    ks_q_round(2 * DMA_PER_TILE)
+    e("s_branch %s" % lab_qr)
+    e("%s:" % lab_w0)
+    ks_q_round(None)
+    e("%s:" % lab_qr)
+    e("v_add_u32 %s, %d, %s" % (v(X0), 2 * TILE_BYTES, v(KADDR_LANE)))
+    for ks in range(9):
+        e("ds_read_b128 %s, %s offset:%d" % (v(Q0 + 4 * ks, 4), v(X0), 32 * ks))
+    for cb in range(4):
+        for i in range(16):
+            e("v_accvgpr_write_b32 %s, 0" % a(64 * cb + i))
+    lab_one = label("pone")
+    e("s_cmp_lt_u32 %s, 2" % s(NT))
+    e("s_cbranch_scc1 %s" % lab_one)
+    e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
+    e("s_branch %s" % lab_wd)
+    e("%s:" % lab_one)
+    e("s_waitcnt vmcnt(0)")
+    e("%s:" % lab_wd)
+    e("s_waitcnt lgkmcnt(0)")
+    e("v_max_i32 %s, 0, %s" % (v(PAGES), v(PAGES)))
+    e("v_min_i32 %s, %s, %s" % (v(PAGES), s(NPP), v(PAGES)))
+    e("s_barrier")                      # tile 0 is complete; every wave has its Q operands
+    lab_no2 = label("no2")
     e("s_cmp_lt_u32 %s, 3" % s(NT))
-    e("s_cbranch_scc1 %s" % lab_w1)
+    e("s_cbranch_scc1 %s" % lab_no2)
     e("s_mov_b32 %s, 2" % s(TMP))
     for ln in dma_tile_lines(TMP, OFF2, True):
         e(ln)
-    e("s_waitcnt vmcnt(%d)" % (2 * DMA_PER_TILE))
-    e("s_branch %s" % lab_wd)
-    e("%s:" % lab_w1)
-    e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
-    e("s_branch %s" % lab_wd)
-    e("%s:" % lab_w0)
-    e("s_waitcnt vmcnt(0)")
-    e("%s:" % lab_wd)
-    e("v_max_i32 %s, 0, %s" % (v(PAGES), v(PAGES)))
-    e("v_min_i32 %s, %s, %s" % (v(PAGES), s(NPP), v(PAGES)))
-    e("s_barrier")                      # tile 0 is complete
+    e("%s:" % lab_no2)
     e("v_add_u32 %s, %s, %s" % (v(KADDR), s(OFF0), v(KADDR_LANE)))
     lds.reset([])
     for slot in ks_scores():

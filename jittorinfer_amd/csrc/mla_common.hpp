@@ -33,7 +33,8 @@ constexpr float LOG2E     = 1.4426950408889634f;
 
 enum { SRC_BF16 = 0, SRC_F16 = 1, SRC_Q8 = 2, SRC_BF16_CVT = 3,     // SRC_BF16_CVT: decode kernel only (bf16 tiles converted to f16 inside LDS)
        SRC_BF16_CS = 4, SRC_F16_CS = 5,                             // decode kernel only: the column-split programs (gen_decode_cs_asm.py)
-       SRC_BF16_KS = 6, SRC_F16_KS = 7 };                           // and its k-split programs for at most 32 rows (gen_decode_cs_asm.py --ks)
+       SRC_BF16_KS = 6, SRC_F16_KS = 7,                             // and its k-split programs for at most 32 rows (gen_decode_cs_asm.py --ks)
+       SRC_BF16_CSQ = 8, SRC_F16_CSQ = 9 };                         // column-split programs behind a prologue that rounds Q itself (no pre-pack pass)
 
 struct KParams {
     const char *    q;
@@ -79,6 +80,7 @@ struct KParams {
     int             bf16_direct;   // bf16 KV: the hi + lo program instead of the one that converts the tiles to f16 (MLA_FLAG_BF16_DIRECT)
     int             rows_contig;  // kv rows are packed (kv_nb1 == row bytes): whole tiles are one contiguous run
     int             mask_ext_in_pack;  // Q pre-pack launch: its last 16 layers of blocks scan the mask extents
+    int             q_in_kernel;   // pipelined kernel: the wave program rounds Q itself (no pre-pack pass, no operand image)
 };
 
 template <typename T, typename U> __device__ __forceinline__ T bitcast(U u) { return __builtin_bit_cast(T, u); }

@@ -22,7 +22,7 @@ namespace {
 // 32 bytes per thread: mask offset, out pointer, (m,l) pointer, debug pointer
 // The column-split programs (SRC_*_CS) keep behind the four tiles: the P^T exchange buffer (8 KB; the hand-off records share it, they
 // are read before P is first written), the rescale factors (1 KB) and the waves' flag words (64 bytes).
-constexpr bool is_cs(int kvt) { return kvt == SRC_BF16_CS || kvt == SRC_F16_CS || kvt == SRC_BF16_KS || kvt == SRC_F16_KS; }
+constexpr bool is_cs(int kvt) { return kvt == SRC_BF16_CS || kvt == SRC_F16_CS || kvt == SRC_BF16_KS || kvt == SRC_F16_KS || kvt == SRC_BF16_CSQ || kvt == SRC_F16_CSQ; }
 constexpr int handoff_off(int kvt) { return kvt == SRC_Q8 ? 3 * TILE_BYTES + 2 * Q8_TILE_RAW : 4 * TILE_BYTES; }
 constexpr int SCHED_MAX_SEQ = 256;                   // balanced schedule: sequences per launch
 constexpr int sched_off(int kvt) { return handoff_off(kvt) + (is_cs(kvt) ? 8192 + 1024 + 64 : NTHREADS * 32); }   // prefix sums of the sequences' tile counts
@@ -115,7 +115,8 @@ __device__ __forceinline__ void sched_first_piece(const KParams & p, const int *
     if (pos >= end) return;
     int lo = 0, hi = p.n_units - 1;   // the item that holds unit `pos`: the last i with S[i] <= pos (it has units)
     while (lo < hi) { const int mid = (lo + hi + 1) >> 1; if (S[mid] <= pos) lo = mid; else hi = mid - 1; }
-    const int it = lo, first = S[it], piece_end = min(S[it + 1], end), base = S[SCHED_MAX_SEQ + 8 + it];
+    // (the second table holds the first keys of the row blocks' key ranges, or -- paged batch -- the sequence lengths: pages start at key 0)
+    const int it = lo, first = S[it], piece_end = min(S[it + 1], end), base = p.balanced == 1 ? 0 : S[SCHED_MAX_SEQ + 8 + it];
     hdr[0] = it;
     hdr[1] = base + (pos - first) * unit_tokens;
     hdr[2] = base + (piece_end - first) * unit_tokens;
@@ -145,6 +146,60 @@ __device__ __forceinline__ void sched_prefix(const KParams & p) {
     int hdr[8];
     sched_first_piece(p, S, t, MLA_PAGE_TOKENS, hdr);
     for (int i = 0; i < 8; i++) p.wg_first[8 * t + i] = hdr[i];
+}
+
+// Q for the column-split and k-split programs: they take their MFMA operands out of LDS, where this leaves the rows of Q --
+// f32 in global memory -- rounded to the KV type as ggml-cpu rounds them (ggml-cpu.c:12034-12035; one v_cvt_pk instruction per
+// pair: round to nearest even) and laid out like a KV tile (row pitch PITCH), so that the program reads an operand the way it
+// reads a K fragment.  No pass over Q ahead of the kernel, no operand image in the workspace.
+// NROW rows from row0 on (rows past n_rows repeat the last one: their results are never stored), C4 groups of 4 columns from
+// byte col0 of the f32 rows on; a row is one run of 16-byte loads, its address a scalar.  Everything but `lane` is uniform.
+template <bool F16> __device__ __forceinline__ u32x2 round4(const f32x4 x) {
+    typedef float f32x2v __attribute__((ext_vector_type(2)));
+    const f32x2v lo = { x.x, x.y }, hi = { x.z, x.w };
+    if constexpr (F16) {
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        return u32x2{ bitcast<unsigned int>(__builtin_convertvector(lo, h2)), bitcast<unsigned int>(__builtin_convertvector(hi, h2)) };
+    } else {
+        typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+        return u32x2{ bitcast<unsigned int>(__builtin_convertvector(lo, b2)), bitcast<unsigned int>(__builtin_convertvector(hi, b2)) };
+    }
+}
+// Lane r < 32 works out where row row0 + r of Q starts (rows past n_rows: the last one) and leaves the address of its byte col0 in
+// this wave's table of 32 entries in LDS.
+__device__ __forceinline__ void q_row_table(const KParams & p, int b, int row0, int col0, unsigned long long * rowptr, int lane) {
+    const int row = min(row0 + (lane & 31), p.n_rows - 1), tq = row / p.n_head, head = row - tq * p.n_head;
+    if (lane < 32) rowptr[lane] = (unsigned long long) (p.q + (int64_t) b * p.q_nb3 + (int64_t) tq * p.q_nb1 + (int64_t) head * p.q_nb2 + col0);
+}
+template <bool F16, int NROW, int C4>
+__device__ __forceinline__ void stage_q_rows(const KParams & p, int b, int row0, int col0, unsigned char * lds, unsigned long long * rowptr, int lane) {
+    constexpr int NLD = (C4 + 63) / 64;   // loads per row; in the last one the lanes past the end of the row repeat its last group
+    constexpr int GRP = 8, NG = NROW / GRP;   // rows per group; the loads of the next group are issued ahead of the work on this one
+    q_row_table(p, b, row0, col0, rowptr, lane);   // the loop below is straight-line code with scalar row addresses
+    const int lane_last = min(lane, C4 - 64 * (NLD - 1) - 1);
+    f32x4 x[2][GRP][NLD];
+    auto load = [&](int g) {
+#pragma unroll
+        for (int r = 0; r < GRP; r++) {
+            const unsigned long long a = rowptr[g * GRP + r];
+            typedef const __attribute__((address_space(1))) char * gptr;
+            const gptr qrow = (gptr) (((unsigned long long) (unsigned int) __builtin_amdgcn_readfirstlane((int) (a >> 32)) << 32) |
+                                      (unsigned int) __builtin_amdgcn_readfirstlane((int) a));
+#pragma unroll
+            for (int k = 0; k < NLD; k++)
+                x[g & 1][r][k] = *(const __attribute__((address_space(1))) f32x4 *) (qrow + 1024 * k + 16 * (k == NLD - 1 ? lane_last : lane));
+        }
+    };
+    load(0);
+#pragma unroll
+    for (int g = 0; g < NG; g++) {
+        if (g + 1 < NG) load(g + 1);
+#pragma unroll
+        for (int r = 0; r < GRP; r++)
+#pragma unroll
+            for (int k = 0; k < NLD; k++)
+                *(u32x2 *) (lds + (g * GRP + r) * PITCH + 512 * k + 8 * (k == NLD - 1 ? lane_last : lane)) = round4<F16>(x[g & 1][r][k]);
+    }
 }
 
 // The wave-level program is generated by gen_decode_asm.py (register map, LDS-DMA issue, MFMA/VALU interleave).
@@ -212,6 +267,26 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
         }
         int hdr[8];
         sched_first_piece(p, sched, bx, TILE_TOK, hdr);
+        for (int i = 0; i < 8; i++) first_piece[i] = __builtin_amdgcn_readfirstlane(hdr[i]);
+        if (first_piece[1] >= first_piece[2]) return;
+        run_pos = first_piece[5]; run_end = first_piece[6]; run_item = first_piece[0] + 1;
+    } else if (p.balanced && p.q_in_kernel) {
+        // paged batch without a pre-pass (the program rounds Q itself): every workgroup scans the page counts of the sequences
+        // itself (one round of loads, a 256-thread scan and the look-up of its first page: cheaper than a launch ahead of the
+        // kernel); the first workgroup leaves the prefix sums for the combine pass
+        const int t = threadIdx.x;
+        int pages = 0, len = 0;
+        if (t < p.n_units) {
+            len   = p.seq_lens[t];
+            pages = (max(min(len, (int) p.bt_stride * MLA_PAGE_TOKENS), 0) + MLA_PAGE_TOKENS - 1) / MLA_PAGE_TOKENS;
+        }
+        sched_scan(sched, pages, len, p.n_units);
+        if (bx == 0) {
+            if (t <= p.n_units) p.sched[t] = sched[t];
+            if (t == 0 && p.n_units == SCHED_MAX_SEQ) p.sched[SCHED_MAX_SEQ] = sched[SCHED_MAX_SEQ];
+        }
+        int hdr[8];
+        sched_first_piece(p, sched, bx, MLA_PAGE_TOKENS, hdr);
         for (int i = 0; i < 8; i++) first_piece[i] = __builtin_amdgcn_readfirstlane(hdr[i]);
         if (first_piece[1] >= first_piece[2]) return;
         run_pos = first_piece[5]; run_end = first_piece[6]; run_item = first_piece[0] + 1;
@@ -329,7 +404,17 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
         h[2] = (unsigned long long) mlptr;
         h[3] = (unsigned long long) p.debug_ptr;
     }
-    // this wave's packed Q operands: [seq][row block][wave][k-step][lane][16 bytes], written by mla_q_pack_kernel
+    // Q without the pre-pack pass.  Column-split programs, in the builds the launcher picks for it (SRC_*_CSQ): this wave's 32 rows ->
+    // tile buffer `wave`.  k-split programs, always: the program fetches and rounds its quarter of the columns itself, behind its first
+    // tile loads; it only needs to know where the rows start.  The tables sit behind the P^T exchange buffer.
+    unsigned long long * q_rows = (unsigned long long *) (smem + HANDOFF_OFF + 8192) + wave * 32;
+    if constexpr (KVT == SRC_BF16_CSQ || KVT == SRC_F16_CSQ) {
+        stage_q_rows<KVT == SRC_F16_CSQ, 32, 144>(p, b, by * 128 + wave * 32, 0, smem + wave * TILE_BYTES, q_rows, lane);
+    } else if constexpr (KVT == SRC_BF16_KS || KVT == SRC_F16_KS) {
+        q_row_table(p, b, 0, wave * 576, q_rows, lane);
+    }
+    // this wave's packed Q operands: [seq][row block][wave][k-step][lane][16 bytes], written by mla_q_pack_kernel (the programs
+    // that take Q from LDS get no image)
     const char * qpack = (const char *) p.q_pack + ((((int64_t) b * ((p.n_rows + 127) / 128) + by) * 4) * KSTEPS) * 1024;  // + wave*36 KB, added in the wave program
     const char *    kv_base = p.kv + (p.block_table ? 0 : (int64_t) b * p.kv_nb3);
     const int32_t * bt_row  = p.block_table ? p.block_table + (int64_t) b * p.bt_stride : nullptr;
@@ -340,9 +425,9 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
     const int s_npp  = __builtin_amdgcn_readfirstlane(p.n_pool_pages - 1);
     const int s_nb1  = __builtin_amdgcn_readfirstlane((int) p.kv_nb1);
     // bit 0: f32 row store; bit 4: V starts at column 64; bit 5: none of this wave's 32 rows exists (it only moves tiles and,
-    // in the Q8_0 programs, dequantizes its share of them)
+    // in the Q8_0 programs, dequantizes its share of them); bit 6 (column-split programs): the Q operands wait in the tile buffers
     const int s_flg  = __builtin_amdgcn_readfirstlane((direct || p.part_f32 ? 1 : 0) | (p.v_col0 ? 16 : 0) |
-                                                      (by * 128 + wave * 32 >= p.n_rows ? 32 : 0) | p.debug_flags);
+                                                      (by * 128 + wave * 32 >= p.n_rows ? 32 : 0) | (p.q_in_kernel ? 64 : 0) | p.debug_flags);
     const int s_ntl  = __builtin_amdgcn_readfirstlane(n_tiles);
     // id of the split's first page as a scalar: the first tiles are requested before the vector load of all page ids is back
     int pg0 = 0;
@@ -366,11 +451,11 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
     // mask builds of the column-split programs: byte offset of this lane's first mask element (its query token's row, tokens 4g.. of a tile)
     const int mask_off = MASK ? (int) ((int64_t) (min(row, p.n_rows - 1) / p.n_head) * p.mask_nb1 + 8 * g) : 0;
 
-    if constexpr (KVT == SRC_BF16_CS && MASK) {
+    if constexpr ((KVT == SRC_BF16_CS || KVT == SRC_BF16_CSQ) && MASK) {
         asm volatile(
 #include "mla_decode_cs_bf16_mask.inc"
             : : MLA_DECODE_CS_MASK_INPUTS : MLA_DECODE_CS_CLOBBERS);
-    } else if constexpr (KVT == SRC_F16_CS && MASK) {
+    } else if constexpr ((KVT == SRC_F16_CS || KVT == SRC_F16_CSQ) && MASK) {
         asm volatile(
 #include "mla_decode_cs_f16_mask.inc"
             : : MLA_DECODE_CS_MASK_INPUTS : MLA_DECODE_CS_CLOBBERS);
@@ -382,11 +467,11 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
         asm volatile(
 #include "mla_decode_ks_f16.inc"
             : : MLA_DECODE_CS_INPUTS : MLA_DECODE_CS_CLOBBERS);
-    } else if constexpr (KVT == SRC_BF16_CS) {
+    } else if constexpr (KVT == SRC_BF16_CS || KVT == SRC_BF16_CSQ) {
         asm volatile(
 #include "mla_decode_cs_bf16.inc"
             : : MLA_DECODE_CS_INPUTS : MLA_DECODE_CS_CLOBBERS);
-    } else if constexpr (KVT == SRC_F16_CS) {
+    } else if constexpr (KVT == SRC_F16_CS || KVT == SRC_F16_CSQ) {
         asm volatile(
 #include "mla_decode_cs_f16.inc"
             : : MLA_DECODE_CS_INPUTS : MLA_DECODE_CS_CLOBBERS);
@@ -661,30 +746,40 @@ static bool decode_ks_applicable(const KParams & kp, int kv_type) {
     return !kp.mask && !kp.bf16_direct && !kp.q_as_q8 && kp.n_rows <= 32 && kp.slot_rows < (1 << 22);
 }
 
-hipError_t launch_decode_fast(const KParams & kp, int kv_type, dim3 grid, hipStream_t st, bool with_prepass) {
+hipError_t launch_decode_fast(const KParams & kp_in, int kv_type, dim3 grid, hipStream_t st, bool with_prepass) {
     // the small passes ahead of the kernel run per (row block, sequence), whatever the kernel's own grid is
-    const unsigned n_rb = (unsigned) ((kp.n_rows + 127) / 128), n_seq = (unsigned) kp.n_seq_sched, extra = kp.balanced == 1 ? 1 : 0;
-    const bool m = kp.mask != nullptr;
+    const unsigned n_rb = (unsigned) ((kp_in.n_rows + 127) / 128), n_seq = (unsigned) kp_in.n_seq_sched, extra = kp_in.balanced == 1 ? 1 : 0;
+    const bool m = kp_in.mask != nullptr;
     // bf16 tiles are converted to f16 inside LDS unless the caller asks for the hi + lo program, or a single wave of a workgroup
     // has rows (16- and 32-head decode): one computing wave is not bound by its MFMAs, and the hi + lo program is the more exact
     // column-split programs (every wave computes S for its own 32 rows and P.V for its own 128 columns): blocks of 128 rows in
     // which all four waves have rows, not the Q8_0 expansion; bf16 K enters as bf16, so the Q image is the bf16 one
-    const bool cs = decode_cs_applicable(kp, kv_type), ks = decode_ks_applicable(kp, kv_type);
-    const bool bf16_cvt = !cs && !kp.bf16_direct && kp.n_rows > 32;
-    // the scan of the mask extents rides in the pack launch (a masked launch has no balanced page schedule, so its layers and the
-    // schedule layer never meet; if they ever did, the scan would keep a launch of its own)
-    const bool fold = m && !extra;
-    KParams pk = kp;
-    pk.mask_ext_in_pack = fold ? 1 : 0;
+    const bool cs = decode_cs_applicable(kp_in, kv_type), ks = decode_ks_applicable(kp_in, kv_type);
+    const bool bf16_cvt = !cs && !kp_in.bf16_direct && kp_in.n_rows > 32;
+    // Q without the pre-pack pass: the k-split programs always round their quarter of Q themselves (144 columns of 32 rows per wave,
+    // fetched behind the first tile loads); the column-split programs when every block of 128 rows is visited by one workgroup (one
+    // split: a prefill chunk) -- the f32 rows are twice the bytes of the operand image, which pays when they are read once and not
+    // when the 8 splits of a decode step each read them.  Ahead of such a launch only the scan of the mask extents (masked launches)
+    // is left, and nothing at all ahead of an unmasked one.
+    const bool q_in_kernel = ks || (cs && kp_in.n_splits == 1 && !kp_in.balanced);
+    KParams kp = kp_in;
+    kp.q_in_kernel = q_in_kernel ? 1 : 0;
+    // elsewhere the scan of the mask extents rides in the pack launch (a masked launch has no balanced page schedule, so its layers
+    // and the schedule layer never meet; if they ever did, the scan would keep a launch of its own)
+    const bool fold = m && !extra && !q_in_kernel;
+    kp.mask_ext_in_pack = fold ? 1 : 0;
     const unsigned ext = fold ? MASK_EXT_CHUNKS : 0;
     if (!with_prepass) { /* the workspace still holds the Q image and the mask extents of an earlier launch of the same call */ }
-    else if (kv_type == MLA_TYPE_Q8_0 || kp.q_as_q8) hipLaunchKernelGGL(mla_q_pack_q8_kernel, dim3(n_rb, n_seq, KSTEPS / 2 + extra + ext), dim3(NTHREADS), 0, st, pk);
-    else if (kv_type == MLA_TYPE_F16) hipLaunchKernelGGL(mla_q_pack_kernel<1>, dim3(n_rb, n_seq, KSTEPS + extra + ext), dim3(NTHREADS), 0, st, pk);
-    else if (bf16_cvt)                hipLaunchKernelGGL(mla_q_pack_kernel<2>, dim3(n_rb, n_seq, KSTEPS + extra + ext), dim3(NTHREADS), 0, st, pk);
-    else                              hipLaunchKernelGGL(mla_q_pack_kernel<0>, dim3(n_rb, n_seq, KSTEPS + extra + ext), dim3(NTHREADS), 0, st, pk);
+    else if (q_in_kernel) { /* nothing: a balanced page schedule is worked out by the workgroups themselves */ }
+    else if (kv_type == MLA_TYPE_Q8_0 || kp.q_as_q8) hipLaunchKernelGGL(mla_q_pack_q8_kernel, dim3(n_rb, n_seq, KSTEPS / 2 + extra + ext), dim3(NTHREADS), 0, st, kp);
+    else if (kv_type == MLA_TYPE_F16) hipLaunchKernelGGL(mla_q_pack_kernel<1>, dim3(n_rb, n_seq, KSTEPS + extra + ext), dim3(NTHREADS), 0, st, kp);
+    else if (bf16_cvt)                hipLaunchKernelGGL(mla_q_pack_kernel<2>, dim3(n_rb, n_seq, KSTEPS + extra + ext), dim3(NTHREADS), 0, st, kp);
+    else                              hipLaunchKernelGGL(mla_q_pack_kernel<0>, dim3(n_rb, n_seq, KSTEPS + extra + ext), dim3(NTHREADS), 0, st, kp);
     if (m && !fold && with_prepass) hipLaunchKernelGGL(mla_mask_extent_kernel, dim3(n_rb, MASK_EXT_CHUNKS), dim3(NTHREADS), 0, st, kp);
     if (kv_type == MLA_TYPE_Q8_0) return m ? launch_variant<SRC_Q8, true>(kp, grid, st) : launch_variant<SRC_Q8, false>(kp, grid, st);
     if (ks) return kv_type == MLA_TYPE_F16 ? launch_variant<SRC_F16_KS, false>(kp, grid, st) : launch_variant<SRC_BF16_KS, false>(kp, grid, st);
+    if (cs && q_in_kernel && kv_type == MLA_TYPE_F16) return m ? launch_variant<SRC_F16_CSQ, true>(kp, grid, st) : launch_variant<SRC_F16_CSQ, false>(kp, grid, st);
+    if (cs && q_in_kernel)             return m ? launch_variant<SRC_BF16_CSQ, true>(kp, grid, st) : launch_variant<SRC_BF16_CSQ, false>(kp, grid, st);
     if (cs && kv_type == MLA_TYPE_F16) return m ? launch_variant<SRC_F16_CS, true>(kp, grid, st) : launch_variant<SRC_F16_CS, false>(kp, grid, st);
     if (cs)                            return m ? launch_variant<SRC_BF16_CS, true>(kp, grid, st) : launch_variant<SRC_BF16_CS, false>(kp, grid, st);
     if (kv_type == MLA_TYPE_F16)  return m ? launch_variant<SRC_F16, true>(kp, grid, st) : launch_variant<SRC_F16, false>(kp, grid, st);
