@@ -17,6 +17,10 @@ bf16 K is multiplied as bf16 (exact products either way); P and V meet as f16, w
 --mask: an additive f16 mask row per query token (ggml-cpu.c:12041-12057: s * scale + mask): the 16 mask values of a lane's 16
 tokens of tile it+1 are loaded at the top of iteration `it` (four 8-byte loads) and enter the scores ahead of the softmax; the
 eight registers they live in come out of the K and P^T fragment rings.
+--mask --bias: the remaining terms of ggml-cpu.c:12041-12057, u = softcap * tanh(s * scale / softcap) + slope(head) * mask.  The slope
+(ggml-cpu.c:11985-11989, :12006-12008; 1 without ALiBi) is a per-lane input that stays in a register the program never writes; the
+soft cap runs as tanh(x) = 1 - 2 / (1 + 2^(2 x log2 e)) on v_exp_f32 / v_rcp_f32, and since a constant added to every logit of a
+row changes neither the probabilities nor the split-K merge, the program keeps -2 softcap / (1 + e^(2x)) and drops the "+ softcap".
 """
 import sys
 
@@ -27,7 +31,8 @@ NO_STORE = "--no-store" in ARGS              # timing experiments only (wrong re
 NO_LOOP_DMA = "--no-loop-dma" in ARGS        # timing experiments only (wrong results): the loop computes on whatever the tile buffers hold
 MASK = "--mask" in ARGS                      # additive f16 mask rows (one per query token)
 KS = "--ks" in ARGS                          # at most 32 rows: the four waves split the 576 columns of K.Q^T (see ks_main)
-assert not (MASK and CLK)
+BIAS = "--bias" in ARGS                      # mask builds: ALiBi slope per head on the mask, tanh soft cap on the logits
+assert not (MASK and CLK) and (MASK or not BIAS)
 MF_QK = "v_mfma_f32_32x32x16_f16" if F16KV else "v_mfma_f32_32x32x16_bf16"
 MF_PV = "v_mfma_f32_32x32x16_f16"
 
@@ -69,7 +74,8 @@ NEGM, ALPHA, TMAX = T[5], T[6], T[7]   # live inside the softmax only
 MKR = [204, 205, 206, 207, 224, 225, 226, 227]   # mask builds: the 16 f16 mask values of this lane's 16 tokens of a tile
 MOFF = X0               # mask builds: byte offset of this lane's first mask element inside a tile's 64 mask bytes (from the end of the prologue on)
 LANE = T[7]             # prologue only
-N_VGPR = 252
+SLOPE = 252             # bias builds: ALiBi slope of this lane's row (one register more than the other builds own)
+N_VGPR = 253 if BIAS else 252
 # ---- SGPR map (all inside the clobbered range s40..s99)
 KV, BT, KVB, KVE, CL2, NPP, NB1, FLG = 40, 42, 44, 45, 46, 47, 48, 49
 NT, IT, OFF0, OFF1, OFF2, OFF3, WAVE, TMP = 50, 51, 52, 53, 54, 55, 56, 57
@@ -85,6 +91,8 @@ WDMA, CL, LAST0, NTM1 = 90, [91, 92, 93, 94], 95, 96
 DMA_BIAS = 3072         # the k-th load behind an M0 update carries the instruction offset 1024 k, which moves both addresses: the
                         # table offsets are (true offset - 1024 k + 3072) and the tile base is taken 3072 bytes low
 SCL, L2E, MSK = 98, 99, 76   # mask builds: scale, log2(e) (SB's registers until the epilogue), mask base (QP's registers once Q is requested)
+K1, K2 = CL2, NPP            # bias builds: 2 log2(e) scale / softcap (the input that carries c_log2 elsewhere) and -2 softcap, 0 = no soft
+                             # cap (NPP's register once the page ids are clamped)
 TAU_BITS = 0x41000000   # 8.0f
 
 out = []
@@ -357,7 +365,10 @@ def softmax_lines(first_tile=False):
         # half k % 2 of register 2 (k / 4) + (k % 4) / 2
         for k in range(16):
             h = k % 2
-            L.append("v_fma_mix_f32 %s, %s, %s, %s op_sel:[0,0,%d] op_sel_hi:[0,0,1]" % (v(S + k), v(S + k), s(SCL), v(MKR[2 * (k // 4) + (k % 4) // 2]), h))
+            if BIAS:   # the logits were scaled (and capped) by bias_block(): u += slope * mask
+                L.append("v_fma_mix_f32 %s, %s, %s, %s op_sel:[%d,0,0] op_sel_hi:[1,0,0]" % (v(S + k), v(MKR[2 * (k // 4) + (k % 4) // 2]), v(SLOPE), v(S + k), h))
+            else:
+                L.append("v_fma_mix_f32 %s, %s, %s, %s op_sel:[0,0,%d] op_sel_hi:[0,0,1]" % (v(S + k), v(S + k), s(SCL), v(MKR[2 * (k // 4) + (k % 4) // 2]), h))
     CS = L2E if MASK else CL2           # factor from the values in S to log2 units
     L.append("v_max3_f32 %s, %s, %s, %s" % (v(m[0]), v(S + 0), v(S + 1), v(S + 2)))
     L.append("v_max3_f32 %s, %s, %s, %s" % (v(m[1]), v(S + 3), v(S + 4), v(S + 5)))
@@ -423,6 +434,29 @@ def p_write_items():
     I.append("v_mov_b32 %s, %s" % (v(T[1]), s(FADR)))
     I.append(lambda: lds.op("ds_write_b32 %s, %s" % (v(T[1]), v(T[0])), ("w", 3)))
     return I
+
+
+def bias_block():
+    """Bias builds, once the scores of a tile are complete: S <- s * scale, or, with a soft cap, -2 softcap / (1 + 2^(s K1))
+    (= softcap * tanh(s * scale / softcap) - softcap).  Not in the shadow of MFMAs: the two forms are a branch apart."""
+    lab_plain, lab_done = label("nocap"), label("capd")
+    e("s_cmp_eq_u32 %s, 0" % s(K2))
+    e("s_cbranch_scc1 %s" % lab_plain)
+    for k in range(16):
+        e("v_mul_f32 %s, %s, %s" % (v(S + k), s(K1), v(S + k)))
+    for k in range(16):
+        e("v_exp_f32 %s, %s" % (v(S + k), v(S + k)))
+    for k in range(16):
+        e("v_add_f32 %s, 1.0, %s" % (v(S + k), v(S + k)))
+    for k in range(16):
+        e("v_rcp_f32 %s, %s" % (v(S + k), v(S + k)))
+    for k in range(16):
+        e("v_mul_f32 %s, %s, %s" % (v(S + k), s(K2), v(S + k)))
+    e("s_branch %s" % lab_done)
+    e("%s:" % lab_plain)
+    for k in range(16):
+        e("v_mul_f32 %s, %s, %s" % (v(S + k), s(SCL), v(S + k)))
+    e("%s:" % lab_done)
 
 
 def mask_tail():
@@ -633,6 +667,8 @@ def iteration(resc, lab_loop):
         mask_tail()
         if MASK:
             mask_wait()
+        if BIAS:
+            bias_block()
 
     def p_read_by_all():
         # every P^T fragment of tile IT is in this wave's registers (the last read was issued at slot 16) before any wave overwrites P
@@ -838,7 +874,15 @@ def main():
         e("s_lshl_b32 %s, %s, 1" % (s(S0), s(KVB)))
         e("s_add_u32 %s, %s, %s" % (s(MSK), s(MSK), s(S0)))
         e("s_addc_u32 %s, %s, 0" % (s(MSK + 1), s(MSK + 1)))
-        e("v_mov_b32 %s, %%[moff]" % v(MOFF))
+        if BIAS:   # (one vector input less: the offset is the first word of this thread's hand-off record)
+            e("v_lshlrev_b32 %s, 5, %s" % (v(MOFF), v(LANE)))
+            e("s_lshl_b32 %s, %s, 11" % (s(S0), s(WAVE)))
+            e("s_add_u32 %s, %s, 0x%x" % (s(S0), s(S0), HOFF))
+            e("v_add_u32 %s, %s, %s" % (v(MOFF), s(S0), v(MOFF)))
+            e("ds_read_b32 %s, %s" % (v(MOFF), v(MOFF)))
+            e("s_waitcnt lgkmcnt(0)")
+        else:
+            e("v_mov_b32 %s, %%[moff]" % v(MOFF))
         e("s_mov_b32 %s, 0" % s(TMP))
         mask_loads(TMP)
     lap(4)
@@ -867,6 +911,16 @@ def main():
     # page ids outside the pool can only come from table entries that are never used; clamped so that no address leaves the pool
     e("v_max_i32 %s, 0, %s" % (v(PAGES), v(PAGES)))
     e("v_min_i32 %s, %s, %s" % (v(PAGES), s(NPP), v(PAGES)))
+    if BIAS:
+        # the last 8 bytes of this thread's hand-off record: its row's slope, and -2 softcap
+        e("v_lshlrev_b32 %s, 5, %s" % (v(DT[0]), v(LANE)))
+        e("s_lshl_b32 %s, %s, 11" % (s(S0), s(WAVE)))
+        e("s_add_u32 %s, %s, 0x%x" % (s(S0), s(S0), HOFF + 24))
+        e("v_add_u32 %s, %s, %s" % (v(DT[0]), s(S0), v(DT[0])))
+        e("ds_read_b64 %s, %s" % (v(DT[0], 2), v(DT[0])))
+        e("s_waitcnt lgkmcnt(0)")
+        e("v_mov_b32 %s, %s" % (v(SLOPE), v(DT[0])))
+        e("v_readfirstlane_b32 %s, %s" % (s(K2), v(DT[1])))
     e("s_barrier")                      # tile 0 is complete; every wave has read its hand-off record
     e("v_add_u32 %s, %s, %s" % (v(KADDR), s(OFF0), v(KADDR_LANE)))
     k_warm()
@@ -877,6 +931,8 @@ def main():
     e("s_nop 7")
     e("s_nop 7")
     mask_tail()
+    if BIAS:
+        bias_block()
     for ln in softmax_lines(first_tile=True):
         e(ln)
     for it_ in p_write_items():
@@ -1334,7 +1390,7 @@ def ks_main():
 
 
 def emit():
-    print("// generated by gen_decode_cs_asm.py%s%s%s -- do not edit" % (" --ks" if KS else "", " --f16" if F16KV else "", " --mask" if MASK else ""))
+    print("// generated by gen_decode_cs_asm.py%s%s%s%s -- do not edit" % (" --ks" if KS else "", " --f16" if F16KV else "", " --mask" if MASK else "", " --bias" if BIAS else ""))
     for ln in out:
         print('"%s\\n\\t"' % ln)
     if CLK:

@@ -1,5 +1,6 @@
 // Pipelined split-K flash-decode kernel for the common MLA decode shape on gfx950:
-// bf16 or f16 latent KV rows of 576 (V = first 512 columns), no mask / ALiBi / softcap, any number of rows
+// bf16, f16 or Q8_0 latent KV rows of 576 (V = first 512 columns), with or without an f16 mask (ALiBi and the soft cap in the masked
+// column-split programs), any number of rows
 // (query token x head pairs) in blocks of 128 per workgroup.
 //
 // One workgroup = 4 waves = 128 rows x one KV split.  Per 32-token tile:
@@ -22,7 +23,7 @@ namespace {
 // 32 bytes per thread: mask offset, out pointer, (m,l) pointer, debug pointer
 // The column-split programs (SRC_*_CS) keep behind the four tiles: the P^T exchange buffer (8 KB; the hand-off records share it, they
 // are read before P is first written), the rescale factors (1 KB) and the waves' flag words (64 bytes).
-constexpr bool is_cs(int kvt) { return kvt == SRC_BF16_CS || kvt == SRC_F16_CS || kvt == SRC_BF16_KS || kvt == SRC_F16_KS || kvt == SRC_BF16_CSQ || kvt == SRC_F16_CSQ; }
+constexpr bool is_cs(int kvt) { return kvt == SRC_BF16_CS || kvt == SRC_F16_CS || kvt == SRC_BF16_KS || kvt == SRC_F16_KS || kvt == SRC_BF16_CSQ || kvt == SRC_F16_CSQ || kvt == SRC_BF16_CSB || kvt == SRC_F16_CSB; }
 constexpr int handoff_off(int kvt) { return kvt == SRC_Q8 ? 3 * TILE_BYTES + 2 * Q8_TILE_RAW : 4 * TILE_BYTES; }
 constexpr int SCHED_MAX_SEQ = 256;                   // balanced schedule: sequences per launch
 constexpr int sched_off(int kvt) { return handoff_off(kvt) + (is_cs(kvt) ? 8192 + 1024 + 64 : NTHREADS * 32); }   // prefix sums of the sequences' tile counts
@@ -75,6 +76,9 @@ constexpr int lds_total(int kvt) { return sched_off(kvt) + (2 * SCHED_MAX_SEQ + 
     [ob] "s"(out_base), [mlb] "s"(ml_base), [rstr] "s"(s_rstr), [nrv] "s"(s_nrv), [tid] "v"(tid)
 
 #define MLA_DECODE_CS_MASK_INPUTS MLA_DECODE_CS_INPUTS, [msk] "s"(mask_base), [scl] "s"(s_scale), [moff] "v"(mask_off)
+// (bias builds: one vector register more is the program's own, the mask offset comes through the hand-off record instead)
+#define MLA_DECODE_CS_BIAS_INPUTS MLA_DECODE_CS_INPUTS, [msk] "s"(mask_base), [scl] "s"(s_scale)
+#define MLA_DECODE_CS_BIAS_CLOBBERS MLA_DECODE_CS_CLOBBERS, "v252"
 
 #define MLA_DECODE_INPUTS                                                                                          \
     [kv] "s"(kv_base), [bt] "s"(bt_row), [kvb] "s"(s_kvb), [kve] "s"(s_kve), [cl2] "s"(c_log2_bits), [npp] "s"(s_npp), \
@@ -396,13 +400,24 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
                                : p.part_f32    ? (void *) ((float *) p.part_o + prow * p.dv_total + 4 * g)
                                                : (void *) (p.part_o + pblock + (int64_t) lrow * 8 + 4 * g)) : nullptr;
     float * mlptr = (!direct && g == 0 && row_valid) ? p.part_ml + prow * 2 : nullptr;
+    // bias builds (ALiBi slope, soft cap; ggml-cpu.c:12041-12057): the launcher has put scale / softcap into p.scale,
+    // 2 log2(e) scale / softcap into p.c_log2_bits and -2 softcap (0: no soft cap) into p.softcap; the last 8 bytes of the hand-off
+    // record are the slope of this thread's row's head (ggml-cpu.c:11985-11989, :12006-12008) and that -2 softcap; see
+    // gen_decode_cs_asm.py
+    constexpr bool BIAS = KVT == SRC_BF16_CSB || KVT == SRC_F16_CSB;
+    float slope = 1.0f;
+    if (BIAS && p.max_bias > 0.0f) {
+        const int r = min(row, p.n_rows - 1), head = r - (r / p.n_head) * p.n_head;
+        slope = head < p.n_head_log2 ? powf(p.m0, (float) (head + 1)) : powf(p.m1, (float) (2 * (head - p.n_head_log2) + 1));
+    }
     {
         unsigned long long * h = (unsigned long long *) (smem + HANDOFF_OFF + tid * 32);
         // mask builds: byte offset of this lane's first mask element (its query token's row, tokens 4g.. of a tile)
         h[0] = MASK ? (unsigned long long) ((int64_t) (min(row, p.n_rows - 1) / p.n_head) * p.mask_nb1 + 8 * g) : 0;
         h[1] = (unsigned long long) optr;
         h[2] = (unsigned long long) mlptr;
-        h[3] = (unsigned long long) p.debug_ptr;
+        h[3] = BIAS ? (unsigned long long) (unsigned int) __float_as_int(slope) | ((unsigned long long) (unsigned int) __float_as_int(p.softcap) << 32)
+                    : (unsigned long long) p.debug_ptr;
     }
     // Q without the pre-pack pass.  Column-split programs, in the builds the launcher picks for it (SRC_*_CSQ): this wave's 32 rows ->
     // tile buffer `wave`.  k-split programs, always: the program fetches and rounds its quarter of the columns itself, behind its first
@@ -451,7 +466,15 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
     // mask builds of the column-split programs: byte offset of this lane's first mask element (its query token's row, tokens 4g.. of a tile)
     const int mask_off = MASK ? (int) ((int64_t) (min(row, p.n_rows - 1) / p.n_head) * p.mask_nb1 + 8 * g) : 0;
 
-    if constexpr ((KVT == SRC_BF16_CS || KVT == SRC_BF16_CSQ) && MASK) {
+    if constexpr (KVT == SRC_BF16_CSB) {
+        asm volatile(
+#include "mla_decode_cs_bf16_bias.inc"
+            : : MLA_DECODE_CS_BIAS_INPUTS : MLA_DECODE_CS_BIAS_CLOBBERS);
+    } else if constexpr (KVT == SRC_F16_CSB) {
+        asm volatile(
+#include "mla_decode_cs_f16_bias.inc"
+            : : MLA_DECODE_CS_BIAS_INPUTS : MLA_DECODE_CS_BIAS_CLOBBERS);
+    } else if constexpr ((KVT == SRC_BF16_CS || KVT == SRC_BF16_CSQ) && MASK) {
         asm volatile(
 #include "mla_decode_cs_bf16_mask.inc"
             : : MLA_DECODE_CS_MASK_INPUTS : MLA_DECODE_CS_CLOBBERS);
@@ -677,7 +700,14 @@ bool decode_fast_applicable(const mla_attn_args * a) {
     if ((a->dv != 512 && a->dv != 576) || (a->flags & MLA_FLAG_F16_ACC_STRICT)) return false;   // 576: two passes, V = columns 0.. and 64..
     const bool q8_copy = decode_fast_q8_copy_rows(a) > 0;
     if (a->kv_type == MLA_TYPE_Q8_0 && !q8_copy && !q8_raw_tiles_ok(a)) return false;
-    if (a->logit_softcap != 0.0f || a->max_bias > 0.0f) return false;
+    if (a->logit_softcap != 0.0f || a->max_bias > 0.0f) {
+        // ALiBi / soft cap: the masked column-split programs have a build for them (16-bit rows, a mask, blocks of 128 rows in
+        // which every wave has rows); everything else goes to the general kernel
+        const int64_t n_rows = (int64_t) a->n_tok * a->n_head, tail = n_rows % 128;
+        if (!a->mask || a->kv_type == MLA_TYPE_Q8_0 || (a->flags & MLA_FLAG_BF16_DIRECT)) return false;
+        if (!(tail == 0 || tail > 96) || n_rows >= (1 << 22)) return false;
+        if (a->logit_softcap != 0.0f && !(a->logit_softcap > 0.0f && a->logit_softcap < INFINITY)) return false;
+    }
     // 16-bit rows must be packed: the per-lane offsets of the tile copy are kept as 16-bit values (31 * 1152 + 1136 < 65536)
     if (a->kv_type != MLA_TYPE_Q8_0 && a->kv_nb1 != ROW_BYTES) return false;   // (the f16 copy of a Q8_0 cache is packed by construction)
     if (a->mask) {
@@ -761,7 +791,8 @@ hipError_t launch_decode_fast(const KParams & kp_in, int kv_type, dim3 grid, hip
     // split: a prefill chunk) -- the f32 rows are twice the bytes of the operand image, which pays when they are read once and not
     // when the 8 splits of a decode step each read them.  Ahead of such a launch only the scan of the mask extents (masked launches)
     // is left, and nothing at all ahead of an unmasked one.
-    const bool q_in_kernel = ks || (cs && kp_in.n_splits == 1 && !kp_in.balanced);
+    const bool bias = kp_in.softcap != 0.0f || kp_in.max_bias > 0.0f;   // (decode_fast_applicable let it through: masked, column-split)
+    const bool q_in_kernel = ks || (cs && !bias && kp_in.n_splits == 1 && !kp_in.balanced);
     KParams kp = kp_in;
     kp.q_in_kernel = q_in_kernel ? 1 : 0;
     // elsewhere the scan of the mask extents rides in the pack launch (a masked launch has no balanced page schedule, so its layers
@@ -778,6 +809,15 @@ hipError_t launch_decode_fast(const KParams & kp_in, int kv_type, dim3 grid, hip
     if (m && !fold && with_prepass) hipLaunchKernelGGL(mla_mask_extent_kernel, dim3(n_rb, MASK_EXT_CHUNKS), dim3(NTHREADS), 0, st, kp);
     if (kv_type == MLA_TYPE_Q8_0) return m ? launch_variant<SRC_Q8, true>(kp, grid, st) : launch_variant<SRC_Q8, false>(kp, grid, st);
     if (ks) return kv_type == MLA_TYPE_F16 ? launch_variant<SRC_F16_KS, false>(kp, grid, st) : launch_variant<SRC_BF16_KS, false>(kp, grid, st);
+    if (bias) {
+        if (!cs || !m) return hipErrorInvalidValue;
+        // what the bias builds expect in place of scale, scale * log2(e) and softcap (see the kernel)
+        if (kp.softcap != 0.0f) kp.scale = kp.scale / kp.softcap;
+        const float k1 = 2.0f * 1.44269504088896340736f * kp.scale;
+        kp.c_log2_bits = __builtin_bit_cast(int, k1);
+        kp.softcap = kp.softcap != 0.0f ? -2.0f * kp.softcap : 0.0f;   // (not -0: the program tests the bits)
+        return kv_type == MLA_TYPE_F16 ? launch_variant<SRC_F16_CSB, true>(kp, grid, st) : launch_variant<SRC_BF16_CSB, true>(kp, grid, st);
+    }
     if (cs && q_in_kernel && kv_type == MLA_TYPE_F16) return m ? launch_variant<SRC_F16_CSQ, true>(kp, grid, st) : launch_variant<SRC_F16_CSQ, false>(kp, grid, st);
     if (cs && q_in_kernel)             return m ? launch_variant<SRC_BF16_CSQ, true>(kp, grid, st) : launch_variant<SRC_BF16_CSQ, false>(kp, grid, st);
     if (cs && kv_type == MLA_TYPE_F16) return m ? launch_variant<SRC_F16_CS, true>(kp, grid, st) : launch_variant<SRC_F16_CS, false>(kp, grid, st);

@@ -145,7 +145,9 @@ def test_planner_schedules_without_gpu():
     assert rc == 0 and info.variant == 2 and info.balanced == 0 and info.n_splits == 8
     rc, info, _ = _plan(dv=576)                                  # V := K: two passes of the pipelined kernel (columns 0.., 64..)
     assert rc == 0 and info.variant == 2 and info.n_passes == 2 and info.balanced == 1
-    rc, info, _ = _plan(dv=576, max_bias=8.0, mask=131072, mask_nb1=16384, mask_ne0=8192)   # ALiBi: the general kernel, 2 x 288 columns
+    rc, info, _ = _plan(dv=576, max_bias=8.0, mask=131072, mask_nb1=16384, mask_ne0=8192)   # ALiBi with a mask over 16-bit rows: the pipelined kernel has a build for it
+    assert rc == 0 and info.variant == 2 and info.n_passes == 2
+    rc, info, _ = _plan(dv=576, max_bias=8.0, mask=131072, mask_nb1=16384, mask_ne0=8192, kv_type=J.MLA_TYPE_Q8_0, kv_nb1=612)   # not over Q8_0 rows: the general kernel, 2 x 288 columns
     assert rc == 0 and info.variant == 0 and info.n_passes == 2
     rc, info, _ = _plan(logit_softcap=30.0)                      # softcap: general kernel, 64 rows per workgroup
     assert rc == 0 and info.variant == 0 and info.rows_per_wg == 64
@@ -158,12 +160,14 @@ def test_planner_schedules_without_gpu():
                                             ("gen_decode_asm.py", ["--cvt", "--mask"], "mla_decode_asm_cvt_mask.inc"),
                                             ("gen_decode_cs_asm.py", [], "mla_decode_cs_bf16.inc"), ("gen_decode_cs_asm.py", ["--f16"], "mla_decode_cs_f16.inc"),
                                             ("gen_decode_cs_asm.py", ["--mask"], "mla_decode_cs_bf16_mask.inc"),
+                                            ("gen_decode_cs_asm.py", ["--mask", "--bias"], "mla_decode_cs_bf16_bias.inc"),
+                                            ("gen_decode_cs_asm.py", ["--f16", "--mask", "--bias"], "mla_decode_cs_f16_bias.inc"),
                                             ("gen_decode_cs_asm.py", ["--f16", "--mask"], "mla_decode_cs_f16_mask.inc"),
                                             ("gen_decode_cs_asm.py", ["--ks"], "mla_decode_ks_bf16.inc"), ("gen_decode_cs_asm.py", ["--ks", "--f16"], "mla_decode_ks_f16.inc")])
 def test_committed_wave_programs_are_what_the_generator_emits(gen, flags, name):
     """The instruction streams the decode kernel includes are generated files: each equals the generator's output.  None of
     them touches v252..v255: the asm block's clobber list ends at v251, and the compiler keeps there what lives across the
-    block (the lanes it spills scalar registers to among it)."""
+    block (the lanes it spills scalar registers to among it).  The bias builds own v252 as well: their clobber list names it."""
     import re
     import subprocess
     import sys
@@ -173,7 +177,7 @@ def test_committed_wave_programs_are_what_the_generator_emits(gen, flags, name):
         assert got == f.read(), "%s is stale: regenerate it with %s %s" % (name, gen, " ".join(flags))
     for m in re.finditer(r"\bv(\d+)\b|\bv\[(\d+):(\d+)\]", got):
         hi = int(m.group(1)) if m.group(1) else int(m.group(3))
-        assert hi <= 251, "%s uses %s" % (name, m.group(0))
+        assert hi <= (252 if "--bias" in flags else 251), "%s uses %s" % (name, m.group(0))
     top = 99 if gen == "gen_decode_cs_asm.py" else 83
     for m in re.finditer(r"\bs(\d+)\b|\bs\[(\d+):(\d+)\]", got):      # scalar registers: inside the clobbered range s40..s83 (s99)
         lo, hi = (int(m.group(1)),) * 2 if m.group(1) else (int(m.group(2)), int(m.group(3)))

@@ -346,3 +346,59 @@ def test_q8_0_cache_with_arbitrary_block_scales(gpu):
     got = _run(gpu, q, k, O.TYPE_Q8_0, mask=m.view(np.uint16), scale=U.SCALE)[..., :512]
     want = O.flash_attn_ext(q, k, O.TYPE_Q8_0, dv=512, mask=m.view(np.uint16), scale=U.SCALE)
     print(U.check(got, want, "Q8_0, arbitrary scales, masked"))
+
+
+@pytest.mark.parametrize("k_type", [O.TYPE_BF16, O.TYPE_F16])
+@pytest.mark.parametrize("max_bias,softcap", [(8.0, 0.0), (0.0, 30.0), (4.0, 5.0)])
+@pytest.mark.parametrize("paged", [False, True])
+def test_alibi_and_softcap_on_the_pipelined_kernel(gpu, k_type, max_bias, softcap, paged):
+    """ALiBi slopes and the tanh soft cap (ggml-cpu.c:11985-11989, :12041-12057) in the masked column-split programs: 2 query
+    tokens x 128 heads (two blocks of 128 rows; the heads past the 64th use the second slope family when n_head_log2 < n_head
+    -- here n_head_log2 = 128, so a 96-head case is added through the 48-head shape below), a mask with holes and graded values.
+    Expected values: float64 numpy on the rounded operands (for bf16 also the oracle)."""
+    import torch
+    import jittorinfer_amd as J
+    rng = np.random.default_rng(int(max_bias * 10 + softcap) + k_type)
+    for n_head, n_tok in ((128, 2), (48, 8)):   # 256 and 384 rows; 48 heads: n_head_log2 = 32, heads 32.. use m1
+        n_seq, n_kv = 2, 640
+        q = rng.standard_normal((n_seq, n_head, n_tok, 576)).astype(np.float32)
+        kf32 = rng.standard_normal((n_seq, n_kv, 576)).astype(np.float32)
+        m = (rng.standard_normal((n_tok, n_kv)) * 2.0).astype(np.float32)
+        m[rng.random((n_tok, n_kv)) < 0.3] = -np.inf
+        m[:, 600:] = -np.inf
+        mask = m.astype(np.float16)
+        if paged:
+            pool, bt, seqs = U.make_paged(rng, [n_kv] * n_seq, k_type)
+            kw = dict(bt=bt, lens=[n_kv] * n_seq)
+            k, kv_rows = pool, np.stack(seqs)
+        else:
+            k = U.encode_kv(kf32, k_type)
+            kw, kv_rows = {}, k
+        tq = torch.from_numpy(q).to(gpu)
+        tk = torch.from_numpy(k.view(np.int16) if k.dtype == np.uint16 else k).to(gpu)
+        tm = torch.from_numpy(mask).to(gpu)
+        out = torch.empty((n_seq, n_tok, n_head, 576), dtype=torch.float32, device=gpu)
+        kt = J.MLA_TYPE_BF16 if k_type == O.TYPE_BF16 else J.MLA_TYPE_F16
+        extra = dict(max_bias=max_bias, logit_softcap=softcap)
+        if paged:
+            extra.update(block_table=torch.from_numpy(bt).to(gpu), seq_lens=torch.tensor([n_kv] * n_seq, dtype=torch.int32, device=gpu))
+        info = J.plan(tq, tk, kt, dv=512, mask=tm, scale=U.SCALE, out=out, **extra)
+        assert info["variant"] == 2, info     # the pipelined kernel, not the general one
+        got = _run(gpu, q, k, k_type, mask=mask.view(np.uint16), scale=U.SCALE, max_bias=max_bias, logit_softcap=softcap, **kw)[..., :512]
+        # float64 on the operands as the kernel sees them
+        kd = (O.bf16_to_f32(kv_rows) if k_type == O.TYPE_BF16 else O.f16_to_f32(kv_rows)).astype(np.float64)
+        qd = (O.bf16_to_f32(O.f32_to_bf16(q)) if k_type == O.TYPE_BF16 else O.f16_to_f32(O.f32_to_f16(q))).astype(np.float64)
+        n_log2 = 1 << int(np.floor(np.log2(n_head)))
+        m0, m1 = 2.0 ** (-max_bias / n_log2), 2.0 ** (-max_bias / 2 / n_log2)
+        slopes = np.array([1.0 if max_bias == 0 else (m0 ** (h + 1) if h < n_log2 else m1 ** (2 * (h - n_log2) + 1)) for h in range(n_head)])
+        s = np.einsum("bhtd,bkd->bhtk", qd, kd) * U.SCALE
+        if softcap:
+            s = softcap * np.tanh(s / softcap)
+        s = s + slopes[None, :, None, None] * mask.astype(np.float64)[None, None]
+        p = np.exp(s - s.max(-1, keepdims=True))
+        p /= p.sum(-1, keepdims=True)
+        want = np.einsum("bhtk,bkd->bthd", p, kd[..., :512])
+        print(U.check(got, want, "bias %g cap %g heads %d" % (max_bias, softcap, n_head)))
+        if k_type == O.TYPE_BF16 and not paged:
+            want_o = O.flash_attn_ext(q, k, k_type, dv=512, mask=mask.view(np.uint16), scale=U.SCALE, max_bias=max_bias, softcap=softcap)
+            print(U.check(got, want_o, "the same against the oracle"))
