@@ -20,6 +20,16 @@
  *                                   pages the same sequence of calls -- copy, roll the copy or the source back into the
  *                                   shared prefix, append -- needs the partly used shared page copied first
  *   mla_page_table_seq_keep         llama_kv_cache_seq_keep, :285-313
+ *   mla_page_table_seq_add          llama_kv_cache_seq_add, :285-345: the reference marks the cache has_shift, and its next
+ *                                   update aborts on that (GGML_ASSERT(!lctx.kv_self.has_shift), "we do not support shift",
+ *                                   src/llama-execute-kvupdate.cpp:151-155: the keys in the cache were rotated for their old
+ *                                   positions and nothing re-rotates them).  Here the call itself is refused and nothing
+ *                                   changes; like the reference's it succeeds when the range holds no cell or delta is 0
+ *   mla_page_table_defrag           llama_kv_cache_defrag, :470-475, and the row moves of build_defrag,
+ *                                   src/llama-graph-defrag.cpp:23-84 (ggml_cpy of cell runs into the holes that seq_rm left).
+ *                                   With pages there is nothing to move: what seq_rm frees are whole pages, which go back to the
+ *                                   free list, and any free page serves any sequence through the block table; the only slack
+ *                                   is the unused tail of a sequence's last page (under 128 cells per sequence)
  *   mla_page_table_used_cells       llama_get_kv_cache_used_cells, :480-482 (tokens held, shared pages counted once)
  *   mla_page_table_fill_inputs      the mask builder of llama_set_inputs, src/llama-context.cpp:326-447: instead of the
  *                                   O(n_tokens x n_kv) f16 mask it fills the I32 block table [n_seqs][max_blocks] and the I32
@@ -40,7 +50,8 @@ extern "C" {
 #define MLA_PT_ERR_BAD_ARG    (-2) /* sequence id out of range, negative position, null pointer */
 #define MLA_PT_ERR_NOT_CONTIG (-3) /* a position that neither extends its sequence by one nor overwrites an existing cell */
 #define MLA_PT_ERR_UNSUPPORTED (-4) /* seq_rm of a range that is neither a suffix nor the whole sequence; find_slot: overwriting a row of
-                                       a page that another sequence maps too, or appending into one (see mla_page_table_seq_unshare) */
+                                       a page that another sequence maps too, or appending into one (see mla_page_table_seq_unshare);
+                                       seq_add that would move a cached position */
 
 typedef struct mla_page_table mla_page_table;
 
@@ -68,6 +79,13 @@ int mla_page_table_seq_cp(mla_page_table * t, int32_t seq_src, int32_t seq_dst, 
  * copy_src_row / copy_dst_row / copy_n_rows (each may be NULL) receive the row run the caller copies on the device
  * (copy_n_rows = 0: nothing to do).  MLA_PT_ERR_NO_SPACE when no page is free. */
 int mla_page_table_seq_unshare(mla_page_table * t, int32_t seq_id, int32_t * copy_src_row, int32_t * copy_dst_row, int32_t * copy_n_rows);
+
+/* Adds delta to positions [p0, p1) of a sequence: 0 when the range holds no cell or delta == 0, else MLA_PT_ERR_UNSUPPORTED
+ * (nothing changed). */
+int mla_page_table_seq_add(mla_page_table * t, int32_t seq_id, int32_t p0, int32_t p1, int32_t delta);
+
+/* Compacts the cache: *n_moves (may be NULL) receives the number of row runs the caller has to copy on the device, always 0. */
+int mla_page_table_defrag(mla_page_table * t, int32_t * n_moves);
 
 /* Removes every sequence but seq_id. */
 int mla_page_table_seq_keep(mla_page_table * t, int32_t seq_id);

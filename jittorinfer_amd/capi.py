@@ -76,6 +76,8 @@ def library():
         lib.mla_page_table_seq_cp.argtypes = [C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_int32] + [C.POINTER(C.c_int32)] * 3
         lib.mla_page_table_seq_unshare.argtypes = [C.c_void_p, C.c_int32] + [C.POINTER(C.c_int32)] * 3
         lib.mla_page_table_seq_keep.argtypes = [C.c_void_p, C.c_int32]
+        lib.mla_page_table_seq_add.argtypes = [C.c_void_p] + [C.c_int32] * 4
+        lib.mla_page_table_defrag.argtypes = [C.c_void_p, C.POINTER(C.c_int32)]
         for name in ("mla_page_table_seq_len", "mla_page_table_free_pages", "mla_page_table_used_cells"):
             getattr(lib, name).restype = C.c_int32
         lib.mla_page_table_seq_len.argtypes = [C.c_void_p, C.c_int32]
@@ -413,6 +415,18 @@ class PageTable:
 
     def seq_keep(self, seq_id):
         return self._lib.mla_page_table_seq_keep(self._h, seq_id) == 0
+
+    def seq_add(self, seq_id, p0, p1, delta):
+        """True when nothing had to move (no cell in the range, or delta 0); False: refused, cached positions cannot be shifted."""
+        return self._lib.mla_page_table_seq_add(self._h, seq_id, p0, p1, delta) == 0
+
+    def defrag(self):
+        """Number of row runs to copy on the device: always 0, freed pages need no compaction."""
+        n = C.c_int32(-1)
+        rc = self._lib.mla_page_table_defrag(self._h, C.byref(n))
+        if rc != 0:
+            raise ValueError("mla_page_table_defrag: %d" % rc)
+        return n.value
 
     def seq_len(self, seq_id):
         return self._lib.mla_page_table_seq_len(self._h, seq_id)

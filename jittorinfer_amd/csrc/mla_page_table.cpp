@@ -172,6 +172,21 @@ int mla_page_table_seq_unshare(mla_page_table * t, int32_t seq_id, int32_t * cop
     return 0;
 }
 
+int mla_page_table_seq_add(mla_page_table * t, int32_t seq_id, int32_t p0, int32_t p1, int32_t delta) {
+    if (!seq_ok(t, seq_id)) return MLA_PT_ERR_BAD_ARG;
+    if (p0 < 0) p0 = 0;
+    const int32_t n = t->len[seq_id];
+    if (p1 < 0 || p1 > n) p1 = n;
+    if (p0 >= p1 || delta == 0) return 0;   // no cell in the range, or nothing to add: the reference returns early too
+    return MLA_PT_ERR_UNSUPPORTED;          // a shift of cached positions: the rows hold keys rotated for their old positions
+}
+
+int mla_page_table_defrag(mla_page_table * t, int32_t * n_moves) {
+    if (!t) return MLA_PT_ERR_BAD_ARG;
+    if (n_moves) *n_moves = 0;   // freed cells are whole pages on the free list, and any free page serves any sequence
+    return 0;
+}
+
 int mla_page_table_seq_keep(mla_page_table * t, int32_t seq_id) {
     if (!seq_ok(t, seq_id)) return MLA_PT_ERR_BAD_ARG;
     for (int32_t s = 0; s < t->n_seq_max; s++) if (s != seq_id) truncate(t, s, 0);

@@ -250,3 +250,28 @@ def test_random_copies_and_roll_backs_never_alias_rows():
                 pos = np.arange(len(want[q]))
                 assert (store[bt[q, pos // PAGE] * PAGE + pos % PAGE] == np.array(want[q])).all(), (step, q)
     assert refused > 0     # the case this test is for did occur
+
+
+def test_seq_add_and_defrag_counterparts():
+    """llama_kv_cache_seq_add (src/llama-kv-cache.cpp:285-345) succeeds without effect when the range holds no cell, and a real
+    shift is what the reference aborts on at its next cache update (src/llama-execute-kvupdate.cpp:151-155): refused here, table
+    unchanged.  llama_kv_cache_defrag (:470-475): holes are whole pages on the free list, so there is never a row to move."""
+    t = J.PageTable(8, 2, 6)
+    assert t.find_slot([0] * 300, list(range(300))) is not None
+    bt0, lens0 = t.fill_inputs([0, 1])
+    assert t.seq_add(0, 300, -1, -7)          # no cell at or past position 300
+    assert t.seq_add(0, 50, 50, -7)           # empty range
+    assert t.seq_add(0, 0, -1, 0)             # nothing to add
+    assert t.seq_add(1, 0, -1, 5)             # an empty sequence
+    assert not t.seq_add(0, 100, -1, -50)     # a context shift
+    assert not t.seq_add(0, 0, -1, 3)
+    bt1, lens1 = t.fill_inputs([0, 1])
+    assert np.array_equal(bt0, bt1) and np.array_equal(lens0, lens1) and t.seq_len(0) == 300
+    # holes come back as whole pages and are reused as they are: nothing to compact, before or after
+    assert t.defrag() == 0
+    assert t.seq_rm(0, 130, -1) and t.free_pages == 6
+    assert t.find_slot([1] * 700, list(range(700))) is not None and t.free_pages == 0
+    assert t.defrag() == 0 and t.seq_len(0) == 130 and t.seq_len(1) == 700
+    rows0 = set(t.find_slot([0] * 130, list(range(130))))
+    rows1 = set(t.find_slot([1] * 700, list(range(700))))
+    assert len(rows0) == 130 and len(rows1) == 700 and not (rows0 & rows1)
