@@ -544,38 +544,33 @@ __device__ __forceinline__ void mask_extent_block(const KParams & p, int rb, int
     __shared__ int red_hi[NTHREADS], red_lo[NTHREADS];
     const int tid = threadIdx.x;
     const int r0 = rb * 128, r1 = min(r0 + 127, p.n_rows - 1);
-    const int t0 = r0 / p.n_head, t1 = r1 / p.n_head;
+    const int t0 = r0 / p.n_head, n_t = r1 / p.n_head - t0 + 1;
     const int n_kv = (int) (p.block_table ? p.bt_stride * MLA_PAGE_TOKENS : p.n_kv);
     const int n8 = n_kv / 8;   // groups of 8 mask values (16 bytes); n_kv is a multiple of 32 on this path
-    const int g0 = (int) ((int64_t) n8 * chunk / MASK_EXT_CHUNKS), g1 = (int) ((int64_t) n8 * (chunk + 1) / MASK_EXT_CHUNKS);
+    const int g0 = (int) ((int64_t) n8 * chunk / MASK_EXT_CHUNKS), ng = (int) ((int64_t) n8 * (chunk + 1) / MASK_EXT_CHUNKS) - g0;
+    // the (token, group) pairs of this sixteenth form one list, eight 16-byte loads per thread in flight: a loop over the tokens
+    // would be a chain of load latencies when the rows are short (a prefill chunk: many tokens per block, few thousand keys)
+    const int64_t total = (int64_t) n_t * ng;
     int hi = 0, lo = n_kv;
-    for (int t = t0; t <= t1; t++) {
-        const char * mrow = p.mask + (int64_t) t * p.mask_nb1;
-        int i1 = g0 + tid;
-        for (; i1 + 3 * NTHREADS < g1; i1 += 4 * NTHREADS) {   // long rows: four groups per thread in flight, the scan is a chain of load latencies otherwise
-            const int i0 = i1;
-            u32x2 a[4], b[4];
+    constexpr int U = 8;
+    for (int64_t base = tid; base < total; base += U * NTHREADS) {
+        u32x4 w[U];
+        int   g[U];
 #pragma unroll
-            for (int u = 0; u < 4; u++) {
-                const int i = i0 + u * NTHREADS;
-                a[u] = *(const u32x2 *) (mrow + 16 * (int64_t) i);   // rows are 8-byte aligned
-                b[u] = *(const u32x2 *) (mrow + 16 * (int64_t) i + 8);
-            }
-#pragma unroll
-            for (int u = 0; u < 4; u++) {
-                const int i = i0 + u * NTHREADS;
-                const unsigned w[4] = { a[u].x, a[u].y, b[u].x, b[u].y };
-#pragma unroll
-                for (int e = 0; e < 8; e++)
-                    if (((w[e >> 1] >> (16 * (e & 1))) & 0xffff) != 0xfc00u) { lo = min(lo, 8 * i + e); hi = max(hi, 8 * i + e + 1); }
-            }
+        for (int u = 0; u < U; u++) {
+            const int64_t idx = min(base + u * NTHREADS, total - 1);   // past the end: the last pair again
+            const int t = (int) (idx / ng);
+            g[u] = g0 + (int) (idx - (int64_t) t * ng);
+            const char * a = p.mask + (int64_t) (t0 + t) * p.mask_nb1 + 16 * (int64_t) g[u];   // rows are 8-byte aligned
+            const u32x2 x = *(const u32x2 *) a, y = *(const u32x2 *) (a + 8);
+            w[u] = u32x4{ x.x, x.y, y.x, y.y };
         }
-        for (int i = i1; i < g1; i += NTHREADS) {
-            const u32x2 a = *(const u32x2 *) (mrow + 16 * (int64_t) i), b = *(const u32x2 *) (mrow + 16 * (int64_t) i + 8);
-            const unsigned w[4] = { a.x, a.y, b.x, b.y };
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const unsigned v[4] = { w[u].x, w[u].y, w[u].z, w[u].w };
 #pragma unroll
             for (int e = 0; e < 8; e++)
-                if (((w[e >> 1] >> (16 * (e & 1))) & 0xffff) != 0xfc00u) { lo = min(lo, 8 * i + e); hi = max(hi, 8 * i + e + 1); }
+                if (((v[e >> 1] >> (16 * (e & 1))) & 0xffff) != 0xfc00u) { lo = min(lo, 8 * g[u] + e); hi = max(hi, 8 * g[u] + e + 1); }
         }
     }
     red_hi[tid] = hi; red_lo[tid] = lo;
