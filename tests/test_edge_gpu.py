@@ -63,6 +63,44 @@ def test_partial_row_blocks_masked(gpu):
     print(U.check(got[..., :512], want, "partial row blocks, masked"))
 
 
+@pytest.mark.parametrize("k_type", [O.TYPE_BF16, O.TYPE_F16, O.TYPE_Q8_0])
+def test_fewer_than_sixteen_rows(gpu, k_type):
+    """1, 2, 5, 8 and 15 attention rows per sequence (a model with few heads per device, single-head probes): the pipelined
+    kernel takes them too -- the k-split programs without a mask over 16-bit rows, the row-split programs with a mask or over
+    Q8_0 rows.  Paged with ragged lengths (an empty sequence among them) and contiguous with a mask that has holes and a
+    fully masked row."""
+    import torch
+    import jittorinfer_amd as J
+    rng = np.random.default_rng(21 + k_type)
+    lens = [0, 1, 33, 129, 700, 2048]
+    pool, bt, seqs = U.make_paged(rng, np.maximum(lens, 1), k_type)
+    seqs = [s[:l] for s, l in zip(seqs, lens)]
+    kt = {O.TYPE_BF16: J.MLA_TYPE_BF16, O.TYPE_F16: J.MLA_TYPE_F16, O.TYPE_Q8_0: J.MLA_TYPE_Q8_0}[k_type]
+    for n_head, n_tok in ((1, 1), (2, 1), (5, 1), (8, 1), (5, 3), (1, 2)):
+        q = rng.standard_normal((len(lens), n_head, n_tok, 576)).astype(np.float32)
+        for n_splits in (0, 2):
+            got = _run(gpu, q, pool, k_type, bt=bt, lens=lens, scale=U.SCALE, n_splits=n_splits)
+            print(n_head, n_tok, n_splits, U.check(got[..., :512], _want(q, seqs, k_type), "fewer than 16 rows, paged"))
+        n_kv = 320
+        k = U.encode_kv(rng.standard_normal((2, n_kv, 576)).astype(np.float32), k_type)
+        m = (rng.standard_normal((n_tok, n_kv)) * 1.5).astype(np.float32)
+        m[rng.random((n_tok, n_kv)) < 0.4] = -np.inf
+        m[:, 290:] = -np.inf
+        if n_tok > 1:
+            m[1, :] = -np.inf                                 # a query token that may attend to nothing: NaN rows, like the reference's
+        mask = m.astype(np.float16).view(np.uint16)
+        q2 = q[:2]
+        tq = torch.from_numpy(q2).to(gpu)
+        tk = torch.from_numpy(k.view(np.int16) if k.dtype == np.uint16 else k).to(gpu)
+        out = torch.empty((2, n_tok, n_head, 576), dtype=torch.float32, device=gpu)
+        info = J.plan(tq, tk, kt, dv=512, mask=torch.from_numpy(mask.view(np.float16)).to(gpu), scale=U.SCALE, out=out)
+        assert info["variant"] == 2, info                     # the pipelined kernel
+        got = _run(gpu, q2, k, k_type, mask=mask, scale=U.SCALE)
+        fn = O.flash_attn_ext_f64 if k_type == O.TYPE_F16 else O.flash_attn_ext
+        want = fn(q2, k, k_type, dv=512, mask=mask, scale=U.SCALE)
+        print(n_head, n_tok, U.check(got[..., :512], want, "fewer than 16 rows, masked", max_abs=3e-3 if k_type == O.TYPE_Q8_0 else U.MAX_ABS_TOL))
+
+
 def test_strided_q(gpu):
     """Q handed over as a permuted view ([seq, tok, head, 576] storage), the layout a fused Q projection would leave."""
     import torch
