@@ -16,18 +16,6 @@ The two 16-register score/P groups swap roles every tile, so the loop body is em
 """
 import sys
 
-DEBUG = "--debug" in sys.argv
-NO_LOOP_DMA = "--no-loop-dma" in sys.argv   # timing experiments only (wrong results)
-NO_PV = "--no-pv" in sys.argv
-NO_QK = "--no-qk" in sys.argv
-NO_SM = "--no-softmax" in sys.argv
-DMA_PLACE = "pv" if "--dma-pv" in sys.argv else "bulk" if "--dma-bulk" in sys.argv else "a"
-NO_VREAD = "--no-vread" in sys.argv
-NO_KREAD = "--no-kread" in sys.argv
-NO_DQ_VALU = "--no-dq-valu" in sys.argv   # timing experiments: Q8_0 dequantizer without its arithmetic / without its LDS traffic
-NO_DQ_LDS = "--no-dq-lds" in sys.argv
-NO_STORE = "--no-store" in sys.argv
-NO_QLOAD = "--no-qload" in sys.argv
 CLKP = "--clk-parts" in sys.argv    # with --clk: accumulate the cycles of part 1 / part 2 of the iterations instead of the waits
 CLK = "--clk" in sys.argv or CLKP           # timing experiments only: s_memtime stamps, written to the hand-off area at the end
 MASK = "--mask" in sys.argv  # additive f16 mask rows (one per query token), added to the scaled scores
@@ -78,7 +66,6 @@ DROW, DCOL, VOFF, PAGES = 241, 242, 243, 244
 LANE, KADDR, VADDR, TMAX = 245, 246, 247, 248
 X0, X1, X2 = 249, 250, 251
 N_VGPR = 252
-DBG, TIDR = 230, 248   # debug builds only: T[6:7] holds the debug pointer until the main loop; TMAX's register keeps tid
 # ---- SGPR map (all inside the clobbered range s40..s79)
 KV, BT, KVB, KVE, CL2, NPP, NB1, FLG = 40, 42, 44, 45, 46, 47, 48, 49
 NT, IT, OFF0, OFF1, OFF2, WAVE, TB, TMP, NVM1 = 50, 51, 52, 53, 54, 55, 56, 58, 59
@@ -123,8 +110,6 @@ class Lds:
         self.pending = []
 
     def read(self, line, tag):
-        if (NO_VREAD and tag[0] == "v") or (NO_KREAD and tag[0] == "k") or (NO_DQ_LDS and tag[0] in "rw"):
-            return
         e(line)
         self.pending.append(tag)
 
@@ -298,9 +283,6 @@ def q8_dequant_items(raw_sreg, dst_sreg, tile_plus):
             lds.need(("r", u, 1))
             e("v_alignbyte_b32 %s, %s, %s, %s" % (v(w[0]), v(w[1]), v(w[0]), s(SH)))      # values 0..3
         I.append(first)
-        if NO_DQ_VALU:
-            I.append(lambda u=u: lds.read("ds_write_b128 %s, %s offset:%d" % (v(DSTA), v(DQ_OUT, 4), 128 * u), ("w", u)))
-            continue
         I.append("v_alignbyte_b32 %s, %s, %s, %s" % (v(w[1]), v(w[2]), v(w[1]), s(SH)))   # values 4..7
         I.append("v_perm_b32 %s, %s, %s, %s" % (v(d), v(d), v(d), s(PSEL)))              # d in both halves
         I.append("v_and_b32 %s, %s, %s" % (v(d), v(d), v(DZ)))
@@ -426,15 +408,12 @@ def k_read(kaddr, p):
 
 def k_warm(kaddr):
     """First K fragments of a tile into the ring."""
-    if not NO_QK:
-        for p in range(KRING - 1):
-            k_read(kaddr, p)
+    for p in range(KRING - 1):
+        k_read(kaddr, p)
 
 
 def qk_slots(sreg, kaddr):
     """36 MFMA slots of S = K.Q^T into v[sreg:sreg+15]; K fragments come through a ring (k_warm first)."""
-    if NO_QK:
-        return [(lambda: None) for _ in range(36)]
     depth = KRING - 1
 
     def mk(ks):
@@ -463,15 +442,14 @@ def v_read(vaddr, idx):
 
 def v_warm(vaddr):
     """First V^T fragments of a tile into the ring (issued at the end of the previous tile)."""
-    if not NO_PV:
-        for idx in range(VRING - 1):
-            v_read(vaddr, idx)
+    for idx in range(VRING - 1):
+        v_read(vaddr, idx)
 
 
 def canon_tags():
     """LDS reads in flight at the top of every iteration, in issue order (see tile_handover)."""
-    vt = lambda idx: [] if NO_PV or NO_VREAD else [("v", idx, 0), ("v", idx, 1)]
-    kt = [] if NO_QK or NO_KREAD else [("k", p) for p in range(KRING - 1)]
+    vt = lambda idx: [("v", idx, 0), ("v", idx, 1)]
+    kt = [("k", p) for p in range(KRING - 1)]
     t = []
     for idx in range(2, VRING - 1):
         t += vt(idx)
@@ -483,11 +461,10 @@ def tile_handover(kaddr_off, vaddr_off, last_slots, sync):
     MFMA time: first fragment reads of the next iteration (V^T of tile IT+1 from the buffer at s[vaddr_off], K of tile
     IT+2 from s[kaddr_off]) around the wait for the tile loads and the workgroup barrier (`sync` emits them).
     Ring slots 0 and 1 of the V^T ring are still needed by the last two MFMAs, so fragments 0 and 1 follow them."""
-    if not NO_PV:
-        lds.need(("v", 31, 1))          # every read of tile IT's buffer has returned: the buffer may be overwritten
-        e("v_add_u32 %s, %s, %s" % (v(VADDR), s(vaddr_off), v(VADDR_LANE)))
-        for idx in range(2, VRING - 1):
-            v_read(VADDR, idx)
+    lds.need(("v", 31, 1))          # every read of tile IT's buffer has returned: the buffer may be overwritten
+    e("v_add_u32 %s, %s, %s" % (v(VADDR), s(vaddr_off), v(VADDR_LANE)))
+    for idx in range(2, VRING - 1):
+        v_read(VADDR, idx)
     if Q8 or CVTB:
         lds.need(("w", 8))              # this wave's share of the next f16 tile is written
     sync()
@@ -496,8 +473,7 @@ def tile_handover(kaddr_off, vaddr_off, last_slots, sync):
     for n in range(2):
         if n < len(last_slots):
             last_slots[n]()
-        if not NO_PV:
-            v_read(VADDR, n)
+        v_read(VADDR, n)
     assert lds.pending == canon_tags(), (lds.pending, canon_tags())
 
 
@@ -505,8 +481,6 @@ def pv_slots(vaddr, greg):
     """MFMA slots of O^T += V^T.P^T for the tile whose P^T operands sit in group `greg`
     (hi halves of k-step kk in greg+8kk .. +3, lo halves in greg+8kk+4 .. +7).  16 d-blocks x 2 k-steps, fragments
     through a ring (v_warm first), d-blocks in pairs so that MFMAs on the same accumulator are never adjacent."""
-    if NO_PV:
-        return []
     depth = VRING - 1
 
     def mf(idx, lo, pre):
@@ -547,8 +521,6 @@ def softmax_lines(sreg):
     1 where the max stayed) and RSC (non-zero when some lane changed its max; the accumulators are rescaled by the
     caller once the MFMAs of the current tile are done) -> p = 2^(s*c - m) -> l += sum p -> P^T operands in place:
     k-step kk: hi halves in sreg+8kk..+3, lo halves in sreg+8kk+4..+7."""
-    if NO_SM:
-        return ["s_mov_b64 %s, 0" % s(RSC, 2)]
     L = []
     m = [T[0], T[1], T[2], T[3], T[4]]
     if MASK:
@@ -695,8 +667,6 @@ def iteration(g_cur, g_next, tag):
     e("s_add_u32 %s, %s, 3" % (s(TMP), s(IT)))
     e("s_cmp_ge_u32 %s, %s" % (s(TMP), s(NT)))
     e("s_cbranch_scc1 %s" % lab_nodma)
-    if NO_LOOP_DMA:
-        e("s_branch %s" % lab_nodma)
 
     def part1(dma):
         lds.pending = canon_tags()
@@ -839,8 +809,6 @@ def main():
     e("s_mov_b32 %s, %%[pg0]" % s(PGZ))
     e("s_mov_b64 %s, %%[qp]" % s(QP, 2))
     e("v_mov_b32 %s, %%[tid]" % v(X0))
-    if DEBUG:
-        e("v_mov_b32 %s, %s" % (v(TIDR), v(X0)))
     e("s_mov_b32 %s, 0x%08x" % (s(THR), 0x41000000))  # TAU = 8.0f
     if not SPLIT:
         e("s_mov_b32 %s, 0x3c003c00" % s(ONES))
@@ -911,7 +879,7 @@ def main():
     e("%s:" % lab_nobt)
     # ------------------------------------------------------------------ Q operands: 36 coalesced 16-byte loads per lane from
     # the packed image, in flight together with the page ids
-    nq = 0 if NO_QLOAD else 36
+    nq = 36
     e("v_lshlrev_b32 %s, 4, %s" % (v(X0), v(LANE)))
     e("s_mul_i32 %s, %s, %d" % (s(S0), s(WAVE), 36 * 1024))
     e("s_add_u32 %s, %s, %s" % (s(QP), s(QP), s(S0)))
@@ -1201,30 +1169,6 @@ def main():
             e("s_branch %s" % LAB_EXIT)
             e("%s:" % lab_busy)
     stamp(1)
-    if DEBUG:
-        # FLG bit 1: dump LDS tile 0 (2336 chunks) to the debug pointer and stop
-        lab = label("nodump1")
-        e("s_bitcmp1_b32 %s, 1" % s(FLG))
-        e("s_cbranch_scc0 %s" % lab)
-        for k in range(10):
-            lab2 = label("skipchunk")
-            e("v_add_u32 %s, %d, %s" % (v(X1), 256 * k, v(TIDR)))
-            e("v_cmp_gt_u32 vcc, %d, %s" % (32 * CPR, v(X1)))
-            e("s_mov_b64 %s, exec" % s(EXS, 2))
-            e("s_nop 1")
-            e("s_and_b64 exec, exec, vcc")
-            e("v_lshlrev_b32 %s, 4, %s" % (v(X1), v(X1)))
-            e("v_add_u32 %s, %s, %s" % (v(X2), s(OFF0), v(X1)))
-            e("ds_read_b128 %s, %s" % (v(SA, 4), v(X2)))
-            e("v_add_co_u32 %s, vcc, %s, %s" % (v(SB), v(DBG), v(X1)))
-            e("s_nop 1")
-            e("v_addc_co_u32 %s, vcc, 0, %s, vcc" % (v(SB + 1), v(DBG + 1)))
-            e("s_waitcnt lgkmcnt(0)")
-            e("global_store_dwordx4 %s, %s, off" % (v(SB, 2), v(SA, 4)))
-            e("s_mov_b64 exec, %s" % s(EXS, 2))
-        e("s_waitcnt vmcnt(0)")
-        e("s_endpgm")
-        e("%s:" % lab)
     e("v_add_u32 %s, %s, %s" % (v(KADDR), s(OFF0), v(KADDR_LANE)))
     k_warm(KADDR)
     for slot in qk_slots(SA, KADDR):
@@ -1314,8 +1258,6 @@ def main():
     # Split-K partial: f16, layout [column/8][row][8] so that the 64 lanes of a wave write 512 contiguous bytes;
     # the out pointer already includes row*16 + g*8 bytes and every (i, j) step advances it by n_rows*16 bytes.
     lab_pstore, lab_sdone = label("pstore"), label("sdone")
-    if NO_STORE:
-        e("s_branch %s" % lab_sdone)
     e("s_bitcmp1_b32 %s, 0" % s(FLG))
     e("s_cbranch_scc0 %s" % lab_pstore)
     for i in range(16):

@@ -27,8 +27,6 @@ import sys
 ARGS = sys.argv[1:]
 F16KV = "--f16" in ARGS                      # f16 KV rows: f16 MFMA for K.Q^T, V^T fragments used as they are
 CLK = "--clk" in ARGS                        # timing builds: s_memtime stamps left in LDS at the end
-NO_STORE = "--no-store" in ARGS              # timing experiments only (wrong results)
-NO_LOOP_DMA = "--no-loop-dma" in ARGS        # timing experiments only (wrong results): the loop computes on whatever the tile buffers hold
 MASK = "--mask" in ARGS                      # additive f16 mask rows (one per query token)
 KS = "--ks" in ARGS                          # at most 32 rows: the four waves split the 576 columns of K.Q^T (see ks_main)
 BIAS = "--bias" in ARGS                      # mask builds: ALiBi slope per head on the mask, tanh soft cap on the logits
@@ -624,8 +622,6 @@ def iteration(resc, lab_loop):
     e("s_add_u32 %s, %s, 3" % (s(TMP), s(IT)))
     e("s_cmp_ge_u32 %s, %s" % (s(TMP), s(NT)))
     e("s_cbranch_scc1 %s" % lab_nodma)
-    if NO_LOOP_DMA:
-        e("s_branch %s" % lab_nodma)
 
     def v_stream(n_conv, tmp):
         """Part 1: reads of all eight V^T fragments of tile IT (two fragments ahead of their conversion) and conversion of
@@ -1009,8 +1005,6 @@ def epilogue(nhb):
     e("v_lshrrev_b32 %s, 5, %s" % (v(X2), v(X0)))                      # g
     e("s_waitcnt lgkmcnt(0)")
     lab_pstore, lab_sdone = label("pstore"), label("sdone")
-    if NO_STORE:
-        e("s_branch %s" % lab_sdone)
     e("s_bitcmp1_b32 %s, 0" % s(FLG))
     e("s_cbranch_scc0 %s" % lab_pstore)
     # f32 rows (final output, or f32 partials): element (row, column) at OB + row * RSTR + column * 4.

@@ -61,8 +61,6 @@ struct KParams {
     int             n_head_log2;
     int             c_log2_bits;   // bit pattern of scale * log2(e)
     void *          q_pack;        // decode kernel: Q in MFMA operand layout (workspace)
-    int             debug_flags;   // development builds of the decode kernel only
-    void *          debug_ptr;
     int             n_pool_pages;  // block-table mode: pages in the pool
     int *           mask_ext;      // pipelined kernel with a mask: per block of 128 rows, 16 pairs (first, one past the last key that is not masked for all its rows) (workspace)
     int             rel_splits;    // the KV splits divide that key range (every split writes its (m, l), -inf when it has no key)

@@ -20,7 +20,7 @@ namespace mla {
 namespace {
 
 // LDS: 4 resident 16-bit tiles (bf16 / f16 KV), or 3 of them behind 2 raw Q8_0 tiles; then the hand-off area,
-// 32 bytes per thread: mask offset, out pointer, (m,l) pointer, debug pointer
+// 32 bytes per thread: mask offset, out pointer, (m,l) pointer, 8 bytes for the bias builds (slope, soft cap)
 // The column-split programs (SRC_*_CS) keep behind the four tiles: the P^T exchange buffer (8 KB; the hand-off records share it, they
 // are read before P is first written), the rescale factors (1 KB) and the waves' flag words (64 bytes).
 constexpr bool is_cs(int kvt) { return kvt == SRC_BF16_CS || kvt == SRC_F16_CS || kvt == SRC_BF16_KS || kvt == SRC_F16_KS || kvt == SRC_BF16_CSQ || kvt == SRC_F16_CSQ || kvt == SRC_BF16_CSB || kvt == SRC_F16_CSB; }
@@ -417,7 +417,7 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
         h[1] = (unsigned long long) optr;
         h[2] = (unsigned long long) mlptr;
         h[3] = BIAS ? (unsigned long long) (unsigned int) __float_as_int(slope) | ((unsigned long long) (unsigned int) __float_as_int(p.softcap) << 32)
-                    : (unsigned long long) p.debug_ptr;
+                    : 0ull;
     }
     // Q without the pre-pack pass.  Column-split programs, in the builds the launcher picks for it (SRC_*_CSQ): this wave's 32 rows ->
     // tile buffer `wave`.  k-split programs, always: the program fetches and rounds its quarter of the columns itself, behind its first
@@ -442,7 +442,7 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
     // bit 0: f32 row store; bit 4: V starts at column 64; bit 5: none of this wave's 32 rows exists (it only moves tiles and,
     // in the Q8_0 programs, dequantizes its share of them); bit 6 (column-split programs): the Q operands wait in the tile buffers
     const int s_flg  = __builtin_amdgcn_readfirstlane((direct || p.part_f32 ? 1 : 0) | (p.v_col0 ? 16 : 0) |
-                                                      (by * 128 + wave * 32 >= p.n_rows ? 32 : 0) | (p.q_in_kernel ? 64 : 0) | p.debug_flags);
+                                                      (by * 128 + wave * 32 >= p.n_rows ? 32 : 0) | (p.q_in_kernel ? 64 : 0));
     const int s_ntl  = __builtin_amdgcn_readfirstlane(n_tiles);
     // id of the split's first page as a scalar: the first tiles are requested before the vector load of all page ids is back
     int pg0 = 0;
