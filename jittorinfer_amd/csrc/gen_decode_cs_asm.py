@@ -831,12 +831,31 @@ def prologue_head(early=None):
     e("%s:" % lab_al)
 
 
+def q_image_issue():
+    """The 36 coalesced 16-byte loads per lane of this wave's Q operands from the packed image, first thing in the program, so that
+    they are on their way while the prologue sets up its tables (not when FLG bit 6 says the operands wait in LDS)."""
+    lab = label("qlds")
+    e("s_bitcmp1_b32 %s, 6" % s(FLG))
+    e("s_cbranch_scc1 %s" % lab)
+    e("v_lshlrev_b32 %s, 4, %s" % (v(X0), v(LANE)))
+    e("s_mul_i32 %s, %s, %d" % (s(S0), s(WAVE), 36 * 1024))
+    e("s_add_u32 %s, %s, %s" % (s(QP), s(QP), s(S0)))
+    e("s_addc_u32 %s, %s, 0" % (s(QP + 1), s(QP + 1)))
+    for ks in range(36):
+        if ks and ks % 4 == 0:
+            e("s_add_u32 %s, %s, 4096" % (s(QP), s(QP)))
+            e("s_addc_u32 %s, %s, 0" % (s(QP + 1), s(QP + 1)))
+        e("global_load_dwordx4 %s, %s, %s offset:%d" % (v(Q0 + 4 * ks, 4), v(X0), s(QP, 2), (ks % 4) * 1024))
+    e("%s:" % lab)
+
+
 def main():
-    prologue_head()
+    prologue_head(q_image_issue)
     # ------------------------------------------------------------------ the Q operands and tile 0.  FLG bit 6: the C++ prologue left this
     # wave's 32 rows, rounded to the KV type, in tile buffer `wave` in the layout of a KV tile, so an operand is read like a K
-    # fragment, and once every wave has its operands the buffers are free for tile 0.  Otherwise: tile 0, then the operands from the
-    # packed image (36 coalesced 16-byte loads per lane).  Tiles 1 and 2 follow; go on as soon as tile 0 and Q are there
+    # fragment, and once every wave has its operands the buffers are free for tile 0.  Otherwise the operands are on their way from
+    # the packed image since the top of the program (q_image_issue): tile 0.  Tiles 1 and 2 follow; go on as soon as tile 0 and Q
+    # are there
     lab_img, lab_qd = label("qimg"), label("qdone")
     e("s_bitcmp1_b32 %s, 6" % s(FLG))
     e("s_cbranch_scc0 %s" % lab_img)
@@ -854,15 +873,6 @@ def main():
     e("s_mov_b32 %s, 0" % s(TMP))
     for ln in dma_tile_lines(TMP, OFF0, True):
         e(ln)
-    e("v_lshlrev_b32 %s, 4, %s" % (v(X0), v(LANE)))
-    e("s_mul_i32 %s, %s, %d" % (s(S0), s(WAVE), 36 * 1024))
-    e("s_add_u32 %s, %s, %s" % (s(QP), s(QP), s(S0)))
-    e("s_addc_u32 %s, %s, 0" % (s(QP + 1), s(QP + 1)))
-    for ks in range(36):
-        if ks and ks % 4 == 0:
-            e("s_add_u32 %s, %s, 4096" % (s(QP), s(QP)))
-            e("s_addc_u32 %s, %s, 0" % (s(QP + 1), s(QP + 1)))
-        e("global_load_dwordx4 %s, %s, %s offset:%d" % (v(Q0 + 4 * ks, 4), v(X0), s(QP, 2), (ks % 4) * 1024))
     e("%s:" % lab_qd)
     if MASK:
         # mask rows start at key kv_begin of this piece; QP's registers and X0 are free now
