@@ -1207,7 +1207,7 @@ def ks_q_issue():
     way to the MFMA operands is the longest (registers, rounding, LDS, registers).  Where each row's quarter starts comes from a
     table the C++ prologue left behind the exchange buffer (lane r of the table read holds row r's address); one 16-byte load per
     lane and row, lanes past the 36th repeat the 36th."""
-    pairs = [S0, S2, QP, SB]
+    pairs = [S0, S2, RSC, EXS]         # (scalar temporaries of later phases: nothing of the prologue lives in them yet)
     e("v_and_b32 %s, 31, %s" % (v(X0), v(LANE)))
     e("v_lshlrev_b32 %s, 3, %s" % (v(X0), v(X0)))
     e("s_lshl_b32 %s, %s, 8" % (s(S0), s(WAVE)))
@@ -1249,13 +1249,19 @@ def ks_q_round(behind):
 
 
 def ks_main():
-    assert not MASK and not CLK
+    assert not CLK and not BIAS
     prologue_head(ks_q_issue)
     e("s_mul_i32 %s, %s, 288" % (s(S0), s(WAVE)))                      # this wave's k-steps 9 w ..: 32 bytes each
     e("v_add_u32 %s, %s, %s" % (v(KADDR_LANE), s(S0), v(KADDR_LANE)))
     e("v_lshlrev_b32 %s, 4, %s" % (v(PADDR), v(LANE)))
     e("v_add_u32 %s, 0x%x, %s" % (v(PADDR), XOFF, v(PADDR)))
     e("s_lshl_b32 %s, %s, 12" % (s(WOFS), s(WAVE)))
+    if MASK:
+        # mask rows start at key kv_begin of this piece (the operand image's registers are free: this program has none)
+        e("s_mov_b64 %s, %%[msk]" % s(MSK, 2))
+        e("s_lshl_b32 %s, %s, 1" % (s(S0), s(KVB)))
+        e("s_add_u32 %s, %s, %s" % (s(MSK), s(MSK), s(S0)))
+        e("s_addc_u32 %s, %s, 0" % (s(MSK + 1), s(MSK + 1)))
     # ------------------------------------------------------------------ tiles 0 and 1 are requested; the wave's quarter of Q (on its way
     # since the top of the program) goes through tile buffer 2 (every wave its own columns of the 32 rows, in the layout of a KV
     # tile: an operand is read like a K fragment); tile 2 is requested once every wave has its operands
@@ -1293,6 +1299,19 @@ def ks_main():
     e("v_max_i32 %s, 0, %s" % (v(PAGES), v(PAGES)))
     e("v_min_i32 %s, %s, %s" % (v(PAGES), s(NPP), v(PAGES)))
     e("s_barrier")                      # tile 0 is complete; every wave has its Q operands
+    if MASK:
+        # the mask values of tile 0 (the byte offset of this lane's first one: its row's token, tokens 4 g .. of a tile, is the
+        # first word of this thread's hand-off record), ahead of tile 2's request
+        e("v_mbcnt_lo_u32_b32 %s, -1, 0" % v(MOFF))
+        e("v_mbcnt_hi_u32_b32 %s, -1, %s" % (v(MOFF), v(MOFF)))
+        e("v_lshlrev_b32 %s, 5, %s" % (v(MOFF), v(MOFF)))
+        e("s_lshl_b32 %s, %s, 11" % (s(S0), s(WAVE)))
+        e("s_add_u32 %s, %s, 0x%x" % (s(S0), s(S0), HOFF))
+        e("v_add_u32 %s, %s, %s" % (v(MOFF), s(S0), v(MOFF)))
+        e("ds_read_b32 %s, %s" % (v(MOFF), v(MOFF)))
+        e("s_waitcnt lgkmcnt(0)")
+        e("s_mov_b32 %s, 0" % s(TMP))
+        mask_loads(TMP)
     lab_no2 = label("no2")
     e("s_cmp_lt_u32 %s, 3" % s(NT))
     e("s_cbranch_scc1 %s" % lab_no2)
@@ -1310,6 +1329,16 @@ def ks_main():
     e("s_sub_u32 %s, %s, %s" % (s(NVAL), s(KVE), s(KVB)))
     e("s_min_u32 %s, %s, 32" % (s(NVAL), s(NVAL)))
     lds.drain()
+    if MASK:
+        # the mask values are there once at most tile 2's loads are in flight
+        lab_m1, lab_m1d = label("mt1"), label("mt1d")
+        e("s_cmp_lt_u32 %s, 3" % s(NT))
+        e("s_cbranch_scc1 %s" % lab_m1)
+        e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
+        e("s_branch %s" % lab_m1d)
+        e("%s:" % lab_m1)
+        e("s_waitcnt vmcnt(0)")
+        e("%s:" % lab_m1d)
     resc = []
     ks_tail(True, resc)
     lab_t1, lab_t1d = label("t1"), label("t1d")
@@ -1334,6 +1363,8 @@ def ks_main():
     e("s_add_u32 %s, %s, %s" % (s(S0), s(S0), s(KVB)))
     e("s_sub_u32 %s, %s, %s" % (s(NVAL), s(KVE), s(S0)))
     e("s_min_u32 %s, %s, 32" % (s(NVAL), s(NVAL)))                     # valid keys of tile IT+1
+    if MASK:
+        mask_loads(TMP)                 # mask of tile IT+1: behind the loads of tile IT+2, ahead of those of tile IT+3
     # part 1: the partial scores of tile IT+1, with the V^T fragments of tile IT (reads, conversion) in their shadow and behind
     lds.reset([])
     qk = ks_scores()
@@ -1360,6 +1391,8 @@ def ks_main():
         xr[2 * n]()
         xr[2 * n + 1]()
     lds.drain()
+    if MASK:
+        mask_wait()
     ks_tail(False, resc)
     lab_w0b, lab_wdb = label("w0"), label("wd")
     e("s_cmp_eq_u32 %s, 0" % s(VMW))

@@ -413,7 +413,9 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
     {
         unsigned long long * h = (unsigned long long *) (smem + HANDOFF_OFF + tid * 32);
         // mask builds: byte offset of this lane's first mask element (its query token's row, tokens 4g.. of a tile)
-        h[0] = MASK ? (unsigned long long) ((int64_t) (min(row, p.n_rows - 1) / p.n_head) * p.mask_nb1 + 8 * g) : 0;
+        // (the k-split programs: every wave works on the same 32 rows, its lanes' rows do not depend on the wave)
+        constexpr bool KS_ROWS = KVT == SRC_BF16_KS || KVT == SRC_F16_KS;
+        h[0] = MASK ? (unsigned long long) ((int64_t) (min(KS_ROWS ? by * 128 + rl : row, p.n_rows - 1) / p.n_head) * p.mask_nb1 + 8 * g) : 0;
         h[1] = (unsigned long long) optr;
         h[2] = (unsigned long long) mlptr;
         h[3] = BIAS ? (unsigned long long) (unsigned int) __float_as_int(slope) | ((unsigned long long) (unsigned int) __float_as_int(p.softcap) << 32)
@@ -482,6 +484,14 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) {
         asm volatile(
 #include "mla_decode_cs_f16_mask.inc"
             : : MLA_DECODE_CS_MASK_INPUTS : MLA_DECODE_CS_CLOBBERS);
+    } else if constexpr (KVT == SRC_BF16_KS && MASK) {
+        asm volatile(
+#include "mla_decode_ks_bf16_mask.inc"
+            : : MLA_DECODE_CS_BIAS_INPUTS : MLA_DECODE_CS_CLOBBERS);
+    } else if constexpr (KVT == SRC_F16_KS && MASK) {
+        asm volatile(
+#include "mla_decode_ks_f16_mask.inc"
+            : : MLA_DECODE_CS_BIAS_INPUTS : MLA_DECODE_CS_CLOBBERS);
     } else if constexpr (KVT == SRC_BF16_KS) {
         asm volatile(
 #include "mla_decode_ks_bf16.inc"
@@ -769,7 +779,8 @@ static bool decode_cs_applicable(const KParams & kp, int kv_type) {
 // them instead of leaving it to the one wave that has rows (gen_decode_cs_asm.py --ks)
 static bool decode_ks_applicable(const KParams & kp, int kv_type) {
     if (kv_type != MLA_TYPE_BF16 && kv_type != MLA_TYPE_F16) return false;
-    return !kp.mask && !kp.bf16_direct && !kp.q_as_q8 && kp.n_rows <= 32 && kp.slot_rows < (1 << 22);
+    const bool bias = kp.softcap != 0.0f || kp.max_bias > 0.0f;
+    return !bias && !kp.bf16_direct && !kp.q_as_q8 && kp.n_rows <= 32 && kp.slot_rows < (1 << 22);
 }
 
 hipError_t launch_decode_fast(const KParams & kp_in, int kv_type, dim3 grid, hipStream_t st, bool with_prepass) {
@@ -804,6 +815,7 @@ hipError_t launch_decode_fast(const KParams & kp_in, int kv_type, dim3 grid, hip
     else                              hipLaunchKernelGGL(mla_q_pack_kernel<0>, dim3(n_rb, n_seq, KSTEPS + extra + ext), dim3(NTHREADS), 0, st, kp);
     if (m && !fold && with_prepass) hipLaunchKernelGGL(mla_mask_extent_kernel, dim3(n_rb, MASK_EXT_CHUNKS), dim3(NTHREADS), 0, st, kp);
     if (kv_type == MLA_TYPE_Q8_0) return m ? launch_variant<SRC_Q8, true>(kp, grid, st) : launch_variant<SRC_Q8, false>(kp, grid, st);
+    if (ks && m) return kv_type == MLA_TYPE_F16 ? launch_variant<SRC_F16_KS, true>(kp, grid, st) : launch_variant<SRC_BF16_KS, true>(kp, grid, st);
     if (ks) return kv_type == MLA_TYPE_F16 ? launch_variant<SRC_F16_KS, false>(kp, grid, st) : launch_variant<SRC_BF16_KS, false>(kp, grid, st);
     if (bias) {
         if (!cs || !m) return hipErrorInvalidValue;
