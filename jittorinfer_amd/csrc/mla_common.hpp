@@ -45,6 +45,7 @@ struct KParams {
     int64_t         n_kv;
     const char *    mask;
     int64_t         mask_nb1, mask_ne0;
+    int64_t         mask_nb3;      // bytes from one sequence's mask rows to the next one's (0: all sequences share the rows)
     const int32_t * block_table;
     int64_t         bt_stride;
     const int32_t * seq_lens;
@@ -78,8 +79,14 @@ struct KParams {
     int             q_as_q8;       // the KV rows are the f16 expansion of a Q8_0 cache: Q is quantized the Q8_0 way
     int             bf16_direct;   // bf16 KV: the hi + lo program instead of the one that converts the tiles to f16 (MLA_FLAG_BF16_DIRECT)
     int             rows_contig;  // kv rows are packed (kv_nb1 == row bytes): whole tiles are one contiguous run
-    int             mask_ext_in_pack;  // Q pre-pack launch: its last 16 layers of blocks scan the mask extents
+    int             mask_ext_in_pack;  // Q pre-pack launch: its last 16 mask_ext_sub layers of blocks scan the mask extents
+    int             mask_ext_sub;      // 1, or the tokens of a row block that get a block each in that scan (a launch issued in two forms)
     int             q_in_kernel;   // pipelined kernel: the wave program rounds Q itself (no pre-pack pass, no operand image)
+    // A masked launch of few heads that is issued in two forms, of which the device runs one (see mla_decode_dual_kernel):
+    int             dual;          //   0: no; 1: these are the parameters of the row-block form (balanced == 2); 2: of the token form
+                                   //   (balanced == 3: every query token a sequence of one token, its mask row that sequence's mask)
+                                   //   mask_ext then holds 16 pairs per query token in both
+    int *           form;          //   the form that ran (2 / 3), left by the kernel for the combine pass (workspace)
 };
 
 template <typename T, typename U> __device__ __forceinline__ T bitcast(U u) { return __builtin_bit_cast(T, u); }
@@ -132,7 +139,7 @@ inline hipError_t raise_lds_limit(const void * fn, bool (&done)[MLA_MAX_DEVICES]
 int64_t    decode_fast_q8_copy_rows(const mla_attn_args * a);   // > 0: Q8_0 + mask on rows the wave program cannot tile runs on an f16 copy of that many rows (workspace)
 hipError_t launch_mask_extent(const KParams & kp, hipStream_t st);   // fills kp.mask_ext: 16 key pairs per block of 128 rows
 hipError_t launch_q8_to_f16(const char * src, int64_t src_nb1, int64_t src_nb3, int64_t rows_per_batch, void * dst, int64_t n_rows, hipStream_t st);
-hipError_t launch_decode_fast(const KParams & kp, int kv_type, dim3 grid, hipStream_t st, bool with_prepass);
+hipError_t launch_decode_fast(const KParams & kp, int kv_type, dim3 grid, hipStream_t st, bool with_prepass, const KParams * tok = nullptr);
 size_t     decode_fast_lds_bytes(int kv_type);
 size_t     decode_fast_qpack_bytes(int n_seq, int n_row_blocks);
 

@@ -19,6 +19,7 @@
 
 #include "mla_common.hpp"
 #include <string.h>
+#include <algorithm>
 #include <stdlib.h>
 
 using namespace mla;
@@ -417,17 +418,21 @@ __global__ void __launch_bounds__(NTHREADS) mla_attn_tile_kernel(const KParams p
 // schedule: the workgroups whose runs of the unit list touch the item (the sequence b, or with a mask the row block of
 // the row), slot = workgroup + item (see mla_decode_kernel), each holding p.slot_rows rows; lrow = the row inside a slot.
 // nvalid < 0: one workgroup had the whole item and wrote the final rows itself.
-__device__ __forceinline__ void partial_slots(const KParams & p, int b, int row, int seq_len, int & slot0, int & nvalid, int & lrow) {
+// A launch issued in two forms (p.dual; the combine pass gets the row-block form's parameters): p.form tells which one ran; in the
+// token form an item is a query token and a slot holds its n_head rows.
+__device__ __forceinline__ void partial_slots(const KParams & p, int b, int row, int seq_len, int & slot0, int & nvalid, int & lrow, int & slot_rows) {
     lrow = row;
+    slot_rows = p.slot_rows;
     if (!p.balanced) {
         nvalid = (seq_len + p.split_tokens - 1) / p.split_tokens;
         nvalid = p.rel_splits ? p.n_splits : min(nvalid, p.n_splits);
         slot0  = b * p.n_splits;
         return;
     }
-    const int item = p.balanced == 2 ? row / 128 : b;
+    int item = p.balanced == 2 ? row / 128 : b, n_units = p.n_units;
     if (p.balanced == 2) lrow = row - item * 128;
-    const int before = p.sched[item], mine = p.sched[item + 1] - before, total = p.sched[p.n_units];
+    if (p.dual && *p.form == 3) { item = row / p.n_head; lrow = row - item * p.n_head; slot_rows = p.n_head; n_units = p.n_tok; }
+    const int before = p.sched[item], mine = p.sched[item + 1] - before, total = p.sched[n_units];
     const int quota = (total + p.n_wg - 1) / p.n_wg;
     if (mine == 0) { slot0 = 0; nvalid = 0; return; }
     const int w0 = before / quota, w1 = (before + mine - 1) / quota;
@@ -447,13 +452,13 @@ __global__ void __launch_bounds__(256) mla_attn_combine_kernel(const KParams p) 
     const int cg  = blockIdx.y * 16 + (threadIdx.x >> 4);
     const int seq_len = p.block_table ? min(p.seq_lens[b], (int) p.bt_stride * MLA_PAGE_TOKENS) : (int) p.n_kv;
     if (row >= p.n_rows || cg * 8 >= p.dv_total) return;
-    int slot0, nvalid, lrow;
-    partial_slots(p, b, row, seq_len, slot0, nvalid, lrow);
+    int slot0, nvalid, lrow, slot_rows;
+    partial_slots(p, b, row, seq_len, slot0, nvalid, lrow, slot_rows);
     if (nvalid < 0) return;
 
-    const float2 *   ml = (const float2 *) p.part_ml + (int64_t) slot0 * p.slot_rows + lrow;
-    const _Float16 * po = p.part_o + (int64_t) slot0 * p.slot_rows * p.dv_total + ((int64_t) cg * p.slot_rows + lrow) * 8;
-    const int64_t ml_step = p.slot_rows, po_step = (int64_t) p.slot_rows * p.dv_total;
+    const float2 *   ml = (const float2 *) p.part_ml + (int64_t) slot0 * slot_rows + lrow;
+    const _Float16 * po = p.part_o + (int64_t) slot0 * slot_rows * p.dv_total + ((int64_t) cg * slot_rows + lrow) * 8;
+    const int64_t ml_step = slot_rows, po_step = (int64_t) slot_rows * p.dv_total;
 
     float M = -INFINITY, L = 0.f;
     float o[8] = { 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f };
@@ -541,12 +546,12 @@ __global__ void __launch_bounds__(256) mla_attn_combine_f32_kernel(const KParams
     const int cg  = threadIdx.x % groups_per_row;
     const int seq_len = p.block_table ? min(p.seq_lens[b], (int) p.bt_stride * MLA_PAGE_TOKENS) : (int) p.n_kv;
     if (row >= p.n_rows || threadIdx.x >= rows_per_block * groups_per_row || cg * 4 >= p.dv_total) return;
-    int slot0, nvalid, lrow;
-    partial_slots(p, b, row, seq_len, slot0, nvalid, lrow);
+    int slot0, nvalid, lrow, slot_rows;
+    partial_slots(p, b, row, seq_len, slot0, nvalid, lrow, slot_rows);
     if (nvalid < 0) return;
-    const float2 * ml = (const float2 *) p.part_ml + (int64_t) slot0 * p.slot_rows + lrow;
-    const float *  po = (const float *) p.part_o + ((int64_t) slot0 * p.slot_rows + lrow) * p.dv_total + cg * 4;
-    const int64_t ml_step = p.slot_rows, po_step = (int64_t) p.slot_rows * p.dv_total;
+    const float2 * ml = (const float2 *) p.part_ml + (int64_t) slot0 * slot_rows + lrow;
+    const float *  po = (const float *) p.part_o + ((int64_t) slot0 * slot_rows + lrow) * p.dv_total + cg * 4;
+    const int64_t ml_step = slot_rows, po_step = (int64_t) slot_rows * p.dv_total;
     float * dst = p.dst + ((int64_t) b * p.n_rows + row) * p.dst_stride + p.v_col0 + cg * 4;
     if (nvalid <= 4)       combine_f32_row<4>(p, ml, po, ml_step, po_step, nvalid, dst);
     else if (nvalid <= 16) combine_f32_row<16>(p, ml, po, ml_step, po_step, nvalid, dst);
@@ -687,6 +692,7 @@ struct Plan {
     int64_t kvcopy_rows;
     int    part_f32;
     int    balanced, n_wg, n_units;   // balanced schedule of the pipelined kernel (1: ragged paged decode, 2: masked launch)
+    int    dual;                      // the masked launch is issued in two forms, see token_form_candidate
 };
 
 int validate(const mla_attn_args * a) {
@@ -718,6 +724,20 @@ int validate(const mla_attn_args * a) {
     if (a->n_splits < 0) return MLA_ERR_BAD_SHAPE;
     if (a->rows_per_wg != 0 && a->rows_per_wg != 32 && a->rows_per_wg != 64 && a->rows_per_wg != 128) return MLA_ERR_BAD_SHAPE;
     return 0;
+}
+
+// The reference's batched decode with few heads per device (one cache shared by the sequences, one query token each, the f16 mask
+// selects each token's cells; 16 heads at tensor-parallel degree 8): a block of 128 rows holds the rows of 8 tokens and visits the
+// cells of all 8, seven eighths of them masked for any one row.  Taken token by token -- every query token a sequence of its own
+// with one token of n_head rows (at most 32: the k-split program), all on the same cache, its mask row that sequence's mask -- a
+// workgroup only visits the cells its token may attend to.  For a prompt chunk of one sequence it is the other way round: the
+// tokens of a block share their cells, and the token form would read them once per token.  The arguments do not tell the two
+// apart, the mask on the device does: such a launch is issued in both forms at once, to a kernel that holds the programs of both;
+// every workgroup adds up the tiles either form would visit (from the mask extents) and runs the cheaper one.
+static bool token_form_candidate(const mla_attn_args * a, const Plan & pl) {
+    return pl.variant == 2 && pl.balanced == 2 && a->n_tok <= 256 && a->n_head <= 32 && (int64_t) a->n_tok * a->n_head > 32 &&
+           (a->kv_type == MLA_TYPE_BF16 || a->kv_type == MLA_TYPE_F16) && !(a->flags & MLA_FLAG_BF16_DIRECT) &&
+           a->logit_softcap == 0.0f && !(a->max_bias > 0.0f);
 }
 
 int make_plan(const mla_attn_args * a, Plan * pl) {
@@ -793,9 +813,16 @@ int make_plan(const mla_attn_args * a, Plan * pl) {
             pl->ws_sched = (size_t) ((pl->n_units + 1 + 63) / 64 * 64 + pl->n_wg * 8) * sizeof(int);
         }
     }
+    if (token_form_candidate(a, *pl)) {
+        pl->dual = 1;
+        pl->ws_maskext = (size_t) a->n_tok * 16 * 2 * sizeof(int);   // 16 pairs per query token
+        pl->ws_sched   = (size_t) ((std::max(pl->n_units, a->n_tok) + 1 + 63) / 64 * 64 + pl->n_wg * 8) * sizeof(int);
+    }
     if (pl->n_splits > 1) {
         // f32 partials while they are small (no second rounding of O on top of the MFMA operands' one), f16 beyond: there the
         // partial traffic counts, and the rounding (2^-12 relative per split) is averaged over long contexts
+        // (the two forms of a launch issued in both share the area: the token form's n_wg + n_tok slots of n_head <= 32 rows fit
+        // into the row-block form's n_wg + n_units slots of 128 rows)
         const size_t n_slots = pl->balanced ? (size_t) pl->n_wg + pl->n_units : (size_t) a->n_seq * pl->n_splits;
         const size_t slot_rows = pl->balanced == 2 ? 128 : (size_t) n_rows;
         const size_t n_part = n_slots * slot_rows * (pl->variant == 2 ? 512 : a->dv);
@@ -854,7 +881,7 @@ int mla_attn_plan(const mla_attn_args * args, mla_attn_plan_info * out) {
     out->split_tokens = pl.split_tokens;
     out->n_passes     = pl.n_passes;
     out->lds_bytes    = (int64_t) pl.lds_bytes;
-    out->balanced     = pl.balanced;
+    out->balanced     = pl.dual ? 4 : pl.balanced;
     out->n_workgroups = pl.balanced ? pl.n_wg : pl.n_splits * pl.n_row_blocks * a_n_seq;
     return 0;
 }
@@ -872,7 +899,7 @@ static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
     KParams kp{};
     kp.q = (const char *) a->q; kp.q_nb1 = a->q_nb1; kp.q_nb2 = a->q_nb2; kp.q_nb3 = a->q_nb3;
     kp.kv = (const char *) a->kv; kp.kv_nb1 = a->kv_nb1; kp.kv_nb3 = a->kv_nb3; kp.n_kv = a->n_kv;
-    kp.mask = (const char *) a->mask; kp.mask_nb1 = a->mask_nb1; kp.mask_ne0 = a->mask_ne0;
+    kp.mask = (const char *) a->mask; kp.mask_nb1 = a->mask_nb1; kp.mask_ne0 = a->mask_ne0; kp.mask_nb3 = 0;   // (shared by the sequences, ggml-cpu.c:12024)
     kp.block_table = a->block_table; kp.bt_stride = a->bt_stride; kp.seq_lens = a->seq_lens;
     kp.dst = a->dst; kp.dst_stride = a->dst_nb1 / 4;
     kp.n_head = a->n_head; kp.n_tok = a->n_tok; kp.n_rows = a->n_tok * a->n_head;
@@ -898,7 +925,16 @@ static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
     kp.q_pack = ws + align256(pl.ws_part_o) + align256(pl.ws_part_ml) + align256(pl.ws_scores);
     kp.mask_ext = pl.ws_maskext ? (int *) (ws + align256(pl.ws_part_o) + align256(pl.ws_part_ml) + align256(pl.ws_scores) + align256(pl.ws_qpack)) : nullptr;
     kp.sched = (int *) (ws + align256(pl.ws_part_o) + align256(pl.ws_part_ml) + align256(pl.ws_scores) + align256(pl.ws_qpack) + align256(pl.ws_maskext));
-    kp.wg_first = kp.sched + (pl.n_units + 1 + 63) / 64 * 64;
+    kp.wg_first = kp.sched + (std::max(pl.n_units, pl.dual ? a->n_tok : 0) + 1 + 63) / 64 * 64;
+    // the token form of a launch issued in two forms (see token_form_candidate): every query token a sequence of one token
+    KParams kt = kp;
+    if (pl.dual) {
+        kp.dual = 1; kt.dual = 2;
+        kp.form = kt.form = kp.wg_first;   // (a masked launch has no use for that table)
+        kt.q_nb3 = a->q_nb1; kt.kv_nb3 = 0; kt.mask_nb3 = a->mask_nb1;
+        kt.n_tok = 1; kt.n_rows = a->n_head; kt.slot_rows = a->n_head;
+        kt.balanced = 3; kt.n_units = a->n_tok; kt.n_seq_sched = a->n_tok;
+    }
 
     if (pl.variant == 1) {
         if (!(phases & 1)) return 0;
@@ -951,7 +987,8 @@ static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
         for (int pass = 0; pass < pl.n_passes; pass++) {
             kp.v_col0 = pass * 64;
             if (phases & 1) {
-                const hipError_t e = launch_decode_fast(kp, kv_type, grid, st, (phases & 4) != 0 && pass == 0);
+                kt.v_col0 = kp.v_col0; kt.dv_total = kp.dv_total;
+                const hipError_t e = launch_decode_fast(kp, kv_type, grid, st, (phases & 4) != 0 && pass == 0, pl.dual ? &kt : nullptr);
                 if (e != hipSuccess) return (int) e;
             }
             // the partials of a pass are consumed before the next pass overwrites them; a combine-only call finishes the last pass

@@ -151,6 +151,17 @@ def test_planner_schedules_without_gpu():
     assert rc == 0 and info.variant == 0 and info.n_passes == 2
     rc, info, _ = _plan(logit_softcap=30.0)                      # softcap: general kernel, 64 rows per workgroup
     assert rc == 0 and info.variant == 0 and info.rows_per_wg == 64
+    # the reference's decode batch: one cache, one query token per sequence, the mask picks every token's cells
+    batch = dict(n_seq=1, n_tok=32, block_table=0, seq_lens=0, bt_stride=0, n_kv=32 * 8192, kv_nb3=0, mask=131072, mask_nb1=2 * 32 * 8192, mask_ne0=32 * 8192)
+    rc, info, _ = _plan(**batch)                                 # 128 heads: a query token fills a block of 128 rows
+    assert rc == 0 and info.variant == 2 and info.balanced == 2 and info.n_row_blocks == 32
+    rc, info, ws = _plan(n_head=16, **batch)                     # 16 heads: issued both as row blocks and token by token
+    assert rc == 0 and info.variant == 2 and info.balanced == 4 and info.n_row_blocks == 4 and info.n_workgroups == 256
+    assert ws >= (256 + 4) * 128 * 512 * 2 + 32 * 16 * 8         # the row-block form's partials hold the token form's; 16 key pairs per token
+    for kw in (dict(n_head=16, n_tok=2), dict(n_head=16, n_tok=257), dict(n_head=64), dict(n_head=16, kv_type=J.MLA_TYPE_Q8_0, kv_nb1=612),
+               dict(n_head=16, flags=J.MLA_FLAG_BF16_DIRECT), dict(n_head=16, max_bias=8.0)):
+        rc, info, _ = _plan(**{**batch, **kw})                  # at most 32 rows, more than 256 tokens, more than 32 heads, Q8_0 rows, ...: one form
+        assert rc == 0 and info.balanced in (0, 2), kw
 
 
 @pytest.mark.parametrize("gen,flags,name", [("gen_decode_asm.py", [], "mla_decode_asm.inc"), ("gen_decode_asm.py", ["--f16"], "mla_decode_asm_f16.inc"),

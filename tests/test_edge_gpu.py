@@ -421,6 +421,62 @@ def test_reference_style_batched_decode_through_the_mask(gpu, k_type, n_splits):
     print(U.check(got[..., :512], want, "batched decode through the mask"))
 
 
+@pytest.mark.parametrize("k_type", [O.TYPE_BF16, O.TYPE_F16])
+@pytest.mark.parametrize("n_head,n_tok", [(16, 32), (32, 64), (24, 37), (16, 256), (8, 16), (16, 3)])
+def test_few_heads_masked_launch_issued_in_two_forms(gpu, k_type, n_head, n_tok):
+    """A masked launch over one cache with at most 32 heads and at most 256 query tokens is issued both as row blocks of 128
+    rows and token by token (every token a sequence of n_head rows); the device runs the form with fewer tiles to visit.
+    Three masks over the same cache and queries: a decode batch (every token its own cells, shuffled, with gaps, one token
+    without any cell -> NaN rows, one with a hole) where the token form runs; a prompt chunk (causal over one sequence) where
+    the row-block form runs; two sequences with half of the tokens each.  24 heads: tokens straddle the row blocks."""
+    import torch
+    import jittorinfer_amd as J
+    rng = np.random.default_rng(1000 * n_head + n_tok)
+    n_kv = 4096
+    k = U.encode_kv(rng.standard_normal((1, n_kv, 576)).astype(np.float32), k_type)
+    q = rng.standard_normal((1, n_head, n_tok, 576)).astype(np.float32)
+    masks = {}
+    m = np.full((n_tok, n_kv), -np.inf, dtype=np.float32)       # decode batch
+    pos, budget = 5, n_kv // n_tok
+    for t in rng.permutation(n_tok):
+        l = int(rng.integers(1, budget - 2))
+        if t != 1:
+            m[t, pos:pos + l] = 0.0
+        pos += l + int(rng.integers(0, 3))
+    t_hole = int(np.argmax((m == 0).sum(1)))
+    cells = np.flatnonzero(m[t_hole] == 0)
+    if len(cells) > 4:
+        m[t_hole, cells[1]:cells[len(cells) // 2]] = -np.inf
+    masks["decode batch"] = m
+    m = np.full((n_tok, n_kv), -np.inf, dtype=np.float32)       # prompt chunk: token t sees cells 100 .. 100 + past + t
+    past = 1500
+    for t in range(n_tok):
+        m[t, 100:100 + past + t + 1] = 0.0
+    masks["prompt chunk"] = m
+    m = np.full((n_tok, n_kv), -np.inf, dtype=np.float32)       # two sequences, each a chunk of half of the tokens
+    for t in range(n_tok):
+        first = t < n_tok // 2
+        base, i = (64, t) if first else (2200, t - n_tok // 2)
+        m[t, base:base + 700 + i + 1] = 0.0
+    masks["two sequences"] = m
+    tq, tk = torch.from_numpy(q).to(gpu), torch.from_numpy(k.view(np.int16)).to(gpu)
+    for what, m in masks.items():
+        mask = m.astype(np.float16).view(np.uint16)
+        tm = torch.from_numpy(mask.view(np.float16)).to(gpu)
+        info = J.plan(tq, tk, k_type, dv=512, scale=U.SCALE, mask=tm)
+        assert info["variant"] == 2 and info["balanced"] == 4     # 4: both forms are launched
+        got = _run(gpu, q, k, k_type, mask=mask, scale=U.SCALE)
+        want = (O.flash_attn_ext_f64 if k_type == O.TYPE_F16 else O.flash_attn_ext)(q, k, k_type, dv=512, mask=mask, scale=U.SCALE)
+        if what == "decode batch":
+            assert np.isnan(want[0, 1]).all()
+        print(what, U.check(got[..., :512], want, what))
+    if n_tok == 32:                                                # the 576-wide V: both forms in each of the two passes
+        mask = masks["decode batch"].astype(np.float16).view(np.uint16)
+        got = _run(gpu, q, k, k_type, dv=576, mask=mask, scale=U.SCALE)
+        want = (O.flash_attn_ext_f64 if k_type == O.TYPE_F16 else O.flash_attn_ext)(q, k, k_type, dv=576, mask=mask, scale=U.SCALE)
+        print(U.check(got, want, "V := K"))
+
+
 def _run_flags(gpu, q, pool, k_type, bt, lens, flags):
     import torch
     import jittorinfer_amd as J
