@@ -315,15 +315,16 @@ def other_config(a, dev, lib, J):
             pool = pool.reshape(1, B * L, 612)
         else:
             pool = (torch.randn((1, B * L, 576), generator=g, device=dev) * 0.5).to(torch.bfloat16).view(torch.int16)
-        q = torch.randn((1, 128, B, 576), generator=g, device=dev)
+        H = a.heads   # (--heads 16: the same batch at tensor-parallel degree 8)
+        q = torch.randn((1, H, B, 576), generator=g, device=dev)
         mask = torch.full((64, B * L), float("-inf"), dtype=torch.float16, device=dev)
         # --ragged: every sequence owns a slot of 8192 cells of the shared cache but has filled only 2048 .. 8192 of them
         lens = [int(x) for x in rng.integers(2048, 8193, B)] if a.ragged else [L] * B
         for b in range(B):
             mask[b, b * L:b * L + lens[b]] = 0
-        out = torch.empty((1, B, 128, 576), dtype=torch.float32, device=dev)
-        n_head, n_tok, kv, kvt = 128, B, ("q8_0" if a.kv == "q8_0" else "bf16"), (J.MLA_TYPE_Q8_0 if a.kv == "q8_0" else J.MLA_TYPE_BF16)
-        name = "BASELINE configs[2] without the block table: one shared cache of 262144 cells, 32 query tokens, f16 mask selects each token's %s cells" % ("2048..8192" if a.ragged else "8192")
+        out = torch.empty((1, B, H, 576), dtype=torch.float32, device=dev)
+        n_head, n_tok, kv, kvt = H, B, ("q8_0" if a.kv == "q8_0" else "bf16"), (J.MLA_TYPE_Q8_0 if a.kv == "q8_0" else J.MLA_TYPE_BF16)
+        name = "BASELINE configs[2] without the block table: one shared cache of 262144 cells, 32 query tokens x %d heads, f16 mask selects each token's %s cells" % (H, "2048..8192" if a.ragged else "8192")
     elif a.config == "c4":
         lens, n_head, n_tok, kv, kvt = [2560] * 4, 16, 512, "bf16", J.MLA_TYPE_BF16
         mask = torch.where(torch.arange(2560, device=dev)[None, :] > 2048 + torch.arange(512, device=dev)[:, None], float("-inf"), 0.0).to(torch.float16)
