@@ -422,7 +422,7 @@ def test_reference_style_batched_decode_through_the_mask(gpu, k_type, n_splits):
 
 
 @pytest.mark.parametrize("k_type", [O.TYPE_BF16, O.TYPE_F16])
-@pytest.mark.parametrize("n_head,n_tok", [(16, 32), (32, 64), (24, 37), (16, 256), (8, 16), (16, 3)])
+@pytest.mark.parametrize("n_head,n_tok", [(16, 32), (32, 64), (24, 37), (16, 256), (8, 16), (16, 3), (16, 20), (1, 200)])
 def test_few_heads_masked_launch_issued_in_two_forms(gpu, k_type, n_head, n_tok):
     """A masked launch over one cache with at most 32 heads and at most 256 query tokens is issued both as row blocks of 128
     rows and token by token (every token a sequence of n_head rows); the device runs the form with fewer tiles to visit.
