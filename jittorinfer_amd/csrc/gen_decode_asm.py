@@ -796,6 +796,10 @@ def main():
     if CLK:
         e("s_mov_b32 s92, 0")
         e("s_mov_b32 s93, 0")
+    # Nothing of the compiled code ahead of the program may still be in flight: a scalar load whose value that code no longer needs
+    # (hoisted above a branch, say) may have been given a register of this program's, and would land on top of what the program
+    # has put there since -- the hardware keeps no order between a load's return and later writes to its destination.
+    e("s_waitcnt vmcnt(0) lgkmcnt(0)")
     e("s_mov_b64 %s, %%[kv]" % s(KV, 2))
     e("s_mov_b64 %s, %%[bt]" % s(BT, 2))
     e("s_mov_b32 %s, %%[kvb]" % s(KVB))

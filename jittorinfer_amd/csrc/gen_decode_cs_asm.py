@@ -719,6 +719,10 @@ def prologue_head(early=None):
     when tile 0 can be requested.  early: emitted once the wave and lane numbers are known (loads that should be on their way
     while the rest is set up; v[36:167] and the scalar temporaries are its own until the end of the prologue)."""
     # ------------------------------------------------------------------ entry: inputs -> fixed registers
+    # Nothing of the compiled code ahead of the program may still be in flight: a scalar load whose value that code no longer needs
+    # (hoisted above a branch, say) may have been given a register of this program's, and would land on top of what the program
+    # has put there since -- the hardware keeps no order between a load's return and later writes to its destination.
+    e("s_waitcnt vmcnt(0) lgkmcnt(0)")
     e("s_mov_b64 %s, %%[kv]" % s(KV, 2))
     e("s_mov_b64 %s, %%[bt]" % s(BT, 2))
     e("s_mov_b32 %s, %%[kvb]" % s(KVB))
