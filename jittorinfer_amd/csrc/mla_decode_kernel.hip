@@ -326,15 +326,59 @@ __device__ __forceinline__ void decode_body() {
             tiles = mask_item_tiles(p.mask_ext, t, p.n_units, (int) p.n_kv, base);
         }
         sched_scan(sched, tiles, base, p.n_units);
+        // Aligned schedule.  Equal runs of the tile list cross from one item into the next wherever they happen to, and a workgroup
+        // whose run does pays a second prologue and epilogue (the Q operands again, another set of partial rows: about what 5 tiles
+        // cost) -- with 16 items of 260 tiles (a prompt chunk of 128 tokens x 16 heads) nearly every item boundary falls inside a
+        // run.  If a run length q within ALIGN_TRY - 1 tiles of the equal share exists for which giving every item ceil(tiles / q)
+        // workgroups of its own needs no more workgroups than there are, that is done instead: item i's workgroups divide its
+        // tiles evenly, nobody crosses.  W[i] (LDS; the first workgroup leaves it for the combine pass) = workgroups before item i.
+        constexpr int ALIGN_TRY = 5;
+        int * W = (int *) smem + 2048, * need_w = W + 2 * SCHED_MAX_SEQ + 8;   // (the tile buffers are not in use yet)
+        int q_al = 0;
+        {
+            const int q_min = max((sched[p.n_units] + p.n_wg - 1) / p.n_wg, 1);
+            int need[ALIGN_TRY];
+#pragma unroll
+            for (int k = 0; k < ALIGN_TRY; k++) {
+                need[k] = (tiles + q_min + k - 1) / (q_min + k);
+                for (int d = 32; d > 0; d >>= 1) need[k] += __shfl_xor(need[k], d, 64);
+                if ((t & 63) == 0) need_w[(t >> 6) * ALIGN_TRY + k] = need[k];
+            }
+            __syncthreads();
+#pragma unroll
+            for (int k = ALIGN_TRY - 1; k >= 0; k--)
+                if (need_w[k] + need_w[ALIGN_TRY + k] + need_w[2 * ALIGN_TRY + k] + need_w[3 * ALIGN_TRY + k] <= p.n_wg) q_al = q_min + k;
+            q_al = __builtin_amdgcn_readfirstlane(q_al);
+            __syncthreads();   // (need_w is read: the scan below and, later, the tile buffers may overwrite it)
+        }
+        if (q_al) sched_scan(W, (tiles + q_al - 1) / q_al, 0, p.n_units);
         if (bx == 0) {
             if (t <= p.n_units) p.sched[t] = sched[t];
             if (t == 0 && p.n_units == SCHED_MAX_SEQ) p.sched[SCHED_MAX_SEQ] = sched[SCHED_MAX_SEQ];
+            if (t == 0) p.wg_first[1] = q_al ? 1 : 0;
+            if (q_al) {
+                if (t <= p.n_units) p.wg_first[8 + t] = W[t];
+                if (t == 0 && p.n_units == SCHED_MAX_SEQ) p.wg_first[8 + SCHED_MAX_SEQ] = W[SCHED_MAX_SEQ];
+            }
         }
-        int hdr[8];
-        sched_first_piece(p, sched, bx, TILE_TOK, hdr);
-        for (int i = 0; i < 8; i++) first_piece[i] = __builtin_amdgcn_readfirstlane(hdr[i]);
-        if (first_piece[1] >= first_piece[2]) return;
-        run_pos = first_piece[5]; run_end = first_piece[6]; run_item = first_piece[0] + 1;
+        if (q_al) {
+            if (bx >= W[p.n_units]) return;
+            int lo = 0, hi = p.n_units - 1;   // the item whose workgroups include bx: the last i with W[i] <= bx
+            while (lo < hi) { const int mid = (lo + hi + 1) >> 1; if (W[mid] <= bx) lo = mid; else hi = mid - 1; }
+            const int k = bx - W[lo], w = W[lo + 1] - W[lo], u = sched[lo + 1] - sched[lo], b0 = sched[SCHED_MAX_SEQ + 8 + lo];
+            first_piece[0] = __builtin_amdgcn_readfirstlane(lo);
+            first_piece[1] = __builtin_amdgcn_readfirstlane(b0 + (int) ((int64_t) k * u / w) * TILE_TOK);
+            first_piece[2] = __builtin_amdgcn_readfirstlane(b0 + (int) ((int64_t) (k + 1) * u / w) * TILE_TOK);
+            first_piece[4] = __builtin_amdgcn_readfirstlane(w == 1);
+            first_piece[7] = (int) p.n_kv;
+            __syncthreads();   // (W is read; the tile buffers may be written)
+        } else {
+            int hdr[8];
+            sched_first_piece(p, sched, bx, TILE_TOK, hdr);
+            for (int i = 0; i < 8; i++) first_piece[i] = __builtin_amdgcn_readfirstlane(hdr[i]);
+            if (first_piece[1] >= first_piece[2]) return;
+            run_pos = first_piece[5]; run_end = first_piece[6]; run_item = first_piece[0] + 1;
+        }
     } else if (p.balanced && p.q_in_kernel) {
         // paged batch without a pre-pass (the program rounds Q itself): every workgroup scans the page counts of the sequences
         // itself (one round of loads, a 256-thread scan and the look-up of its first page: cheaper than a launch ahead of the

@@ -432,6 +432,13 @@ __device__ __forceinline__ void partial_slots(const KParams & p, int b, int row,
     int item = p.balanced == 2 ? row / 128 : b, n_units = p.n_units;
     if (p.balanced == 2) lrow = row - item * 128;
     if (p.dual && *p.form == 3) { item = row / p.n_head; lrow = row - item * p.n_head; slot_rows = p.n_head; n_units = p.n_tok; }
+    if (p.balanced >= 2 && p.wg_first[1]) {   // aligned schedule of a masked launch: every item has workgroups of its own
+        const int * W = p.wg_first + 8;
+        nvalid = W[item + 1] - W[item];
+        slot0  = nvalid ? W[item] + item : 0;
+        if (nvalid == 1) nvalid = -1;
+        return;
+    }
     const int before = p.sched[item], mine = p.sched[item + 1] - before, total = p.sched[n_units];
     const int quota = (total + p.n_wg - 1) / p.n_wg;
     if (mine == 0) { slot0 = 0; nvalid = 0; return; }
