@@ -477,6 +477,51 @@ def test_few_heads_masked_launch_issued_in_two_forms(gpu, k_type, n_head, n_tok)
         print(U.check(got, want, "V := K"))
 
 
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_random_masked_launches_over_one_cache(gpu, seed):
+    """Randomised masked launches over one contiguous cache (the reference's own graph form): 1 to 128 heads, 1 to 300 query
+    tokens, every token a window of its own (some empty -> NaN rows, some with a hole), windows of neighbouring tokens disjoint,
+    nested or overlapping at random -- which decides whether the launch runs as row blocks or token by token, with equal runs
+    of the tile list or with workgroups of its own for every item -- bf16 and f16 cells, both V widths."""
+    import torch
+    import jittorinfer_amd as J
+    rng = np.random.default_rng(4242 + seed)
+    seen = set()
+    for case in range(14):
+        n_head = int(rng.choice([1, 3, 8, 16, 16, 24, 32, 32, 48, 64, 128]))
+        n_tok = int(rng.choice([1, 2, 5, 8, 17, 32, 64, 100, 300])) if n_head <= 32 else int(rng.choice([1, 2, 5, 8, 17]))
+        n_kv = 32 * int(rng.integers(4, 129))
+        k_type = O.TYPE_BF16 if rng.integers(2) else O.TYPE_F16
+        dv = 576 if rng.integers(5) == 0 else 512
+        style = int(rng.integers(3))      # 0: decode batch (disjoint windows), 1: prompt chunk (nested windows), 2: anything
+        m = np.full((n_tok, n_kv), -np.inf, dtype=np.float32)
+        for t in range(n_tok):
+            if rng.integers(12) == 0:
+                continue
+            if style == 0:
+                w = max(1, n_kv // n_tok)
+                lo, hi = t * w + int(rng.integers(0, max(1, w // 3))), (t + 1) * w
+            elif style == 1:
+                lo, hi = 7, min(n_kv, max(8, n_kv - n_tok + t))
+            else:
+                lo = int(rng.integers(0, n_kv)); hi = min(n_kv, lo + int(rng.integers(1, n_kv)))
+            hi = min(max(hi, lo + 1), n_kv)
+            m[t, lo:hi] = (rng.standard_normal(hi - lo) * 0.5).astype(np.float32) if rng.integers(3) == 0 else 0.0
+            if hi - lo > 6 and rng.integers(4) == 0:
+                m[t, lo + 2:lo + 2 + (hi - lo) // 2] = -np.inf
+        mask = m.astype(np.float16).view(np.uint16)
+        q = rng.standard_normal((1, n_head, n_tok, 576)).astype(np.float32)
+        k = U.encode_kv(rng.standard_normal((1, n_kv, 576)).astype(np.float32), k_type)
+        tq, tk = torch.from_numpy(q).to(gpu), torch.from_numpy(k.view(np.int16)).to(gpu)
+        tm = torch.from_numpy(mask.view(np.float16)).to(gpu)
+        info = J.plan(tq, tk, k_type, dv=dv, scale=U.SCALE, mask=tm)
+        seen.add((info["variant"], info["balanced"]))
+        got = _run(gpu, q, k, k_type, dv=dv, mask=mask, scale=U.SCALE)[..., :dv]
+        want = (O.flash_attn_ext_f64 if k_type == O.TYPE_F16 else O.flash_attn_ext)(q, k, k_type, dv=dv, mask=mask, scale=U.SCALE)
+        U.check(got, want, "case %d: H %d tok %d n_kv %d type %d dv %d style %d plan %s" % (case, n_head, n_tok, n_kv, k_type, dv, style, info))
+    print(sorted(seen))
+
+
 def _run_flags(gpu, q, pool, k_type, bt, lens, flags):
     import torch
     import jittorinfer_amd as J
