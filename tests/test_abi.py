@@ -151,6 +151,13 @@ def test_planner_schedules_without_gpu():
     assert rc == 0 and info.variant == 0 and info.n_passes == 2
     rc, info, _ = _plan(logit_softcap=30.0)                      # softcap: general kernel, 64 rows per workgroup
     assert rc == 0 and info.variant == 0 and info.rows_per_wg == 64
+    one = dict(n_seq=1, n_head=16, block_table=0, seq_lens=0, bt_stride=0, kv_nb3=0, kv_type=J.MLA_TYPE_F16)
+    rc, info, _ = _plan(n_kv=1024, **one)                        # configs[0]: one short sequence, splits of one 32-key tile
+    assert rc == 0 and info.variant == 2 and info.n_splits == 32 and info.split_tokens == 32
+    rc, info, _ = _plan(n_kv=4096, **one)                        # more tiles than 1 MB of partials allows splits: whole pages again
+    assert rc == 0 and info.n_splits == 32 and info.split_tokens == 128
+    rc, info, _ = _plan(n_kv=1024, **{**one, "n_head": 128})
+    assert rc == 0 and info.n_splits == 8 and info.split_tokens == 128
     # the reference's decode batch: one cache, one query token per sequence, the mask picks every token's cells
     batch = dict(n_seq=1, n_tok=32, block_table=0, seq_lens=0, bt_stride=0, n_kv=32 * 8192, kv_nb3=0, mask=131072, mask_nb1=2 * 32 * 8192, mask_ne0=32 * 8192)
     rc, info, _ = _plan(**batch)                                 # 128 heads: a query token fills a block of 128 rows
