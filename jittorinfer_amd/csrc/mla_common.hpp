@@ -66,12 +66,15 @@ struct KParams {
     int *           mask_ext;      // pipelined kernel with a mask: per block of 128 rows, 16 pairs (first, one past the last key that is not masked for all its rows) (workspace)
     int             rel_splits;    // the KV splits divide that key range (every split writes its (m, l), -inf when it has no key)
     int             balanced;      // pipelined kernel: 1 = ragged paged decode, workgroups take equal runs of the page list of all
-                                   // sequences; 2 = masked launch, equal runs of the tile list of the row blocks' key ranges
+                                   // sequences; 2 = masked launch, equal runs of the tile list of the row blocks' key ranges; 3 = the same with
+                                   // every query token as an item (the token form of a launch issued in two forms, see `dual`)
     int             n_wg;          //   workgroups (grid = (n_wg, 1, 1)); partial slot of workgroup v's piece of item i = v + i
-    int             n_units;       //   items: sequences (1) / row blocks (2)
+    int             n_units;       //   items: sequences (1) / row blocks (2) / query tokens (3)
     int             slot_rows;     // rows per partial slot: n_rows, or 128 with balanced == 2
     int             n_seq_sched;   // sequences of the launch (grids of the pre-pack passes)
-    int *           wg_first;      //   [n_wg][8] first piece of every workgroup (balanced == 1; workspace, written by the pre-pass)
+    int *           wg_first;      //   [n_wg][8] first piece of every workgroup (balanced == 1; workspace, written by the pre-pass).  Masked launches
+                                   //   (balanced >= 2) keep there, written by the kernel's first workgroup for the combine pass: [1] = the schedule is
+                                   //   the aligned one, [8 ..] = workgroups before every item in that schedule
     int *           sched;         //   [n_units + 1] units before each item / in total (workspace; written by the pre-pass (1) or by the
                                    //   first workgroup of the kernel itself (2); the combine pass reads it)
     int             v_col0;        // pipelined kernel: V = columns v_col0 .. v_col0 + 511 of the rows (0, or 64 in the second pass of a

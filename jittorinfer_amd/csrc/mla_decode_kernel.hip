@@ -129,8 +129,9 @@ constexpr int lds_total(int kvt) { return sched_off(kvt) + (2 * SCHED_MAX_SEQ + 
 
 // Balanced schedule.  The work of a launch is a list of units -- the 128-token pages of the sequences of a paged decode
 // batch (p.balanced == 1), or the 32-token tiles of the key ranges the row blocks of a masked launch may attend to
-// (p.balanced == 2) -- and each of p.n_wg workgroups takes an equal run of that list, piece by piece where the run
-// crosses from one item (sequence / row block) to the next.
+// (p.balanced == 2; 3: of the key ranges of its query tokens, each taken as a sequence of its own) -- and each of p.n_wg
+// workgroups takes an equal run of that list, piece by piece where the run crosses from one item (sequence / row block / token)
+// to the next; a masked launch gives every item workgroups of its own instead where that costs next to nothing (see the kernel).
 //
 // sched_scan: S (LDS, 2 * SCHED_MAX_SEQ + 8 ints) <- S[i] = units of the items before i (i <= n_units), and from
 // S[SCHED_MAX_SEQ + 8] the `base` of every item; `count`, `base` belong to item threadIdx.x.  All 256 threads call it.
