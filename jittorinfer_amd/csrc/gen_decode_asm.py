@@ -1318,6 +1318,9 @@ def main():
     print("// generated by gen_decode_asm.py%s%s -- do not edit" % (" --q8" if Q8 else " --f16" if "--f16" in sys.argv else "", " --mask" if MASK else ""))
     for ln in out:
         print('"%s\\n\\t"' % ln)
+    # and nothing of the program is in flight when the compiled code goes on (the mirror image of the wait at the top: an LDS read
+    # or a load requested ahead for a tile that never came would land in a register that code has taken since)
+    print('"s_waitcnt vmcnt(0) lgkmcnt(0)\\n\\t"')
 
 
 main()

@@ -1434,6 +1434,9 @@ def emit():
     print("// generated by gen_decode_cs_asm.py%s%s%s%s -- do not edit" % (" --ks" if KS else "", " --f16" if F16KV else "", " --mask" if MASK else "", " --bias" if BIAS else ""))
     for ln in out:
         print('"%s\\n\\t"' % ln)
+    # and nothing of the program is in flight when the compiled code goes on (the mirror image of the wait at the top: an LDS read
+    # or a load requested ahead for a tile that never came would land in a register that code has taken since)
+    print('"s_waitcnt vmcnt(0) lgkmcnt(0)\\n\\t"')
     if CLK:
         sys.stderr.write("laps: %s\n" % "; ".join(LAPS))
 
