@@ -30,7 +30,7 @@ constexpr int sched_off(int kvt) { return handoff_off(kvt) + (is_cs(kvt) ? 8192 
 constexpr int lds_total(int kvt) { return sched_off(kvt) + (2 * SCHED_MAX_SEQ + 8) * 4; }   // prefix sums, then the lengths
 
 #define MLA_DECODE_CLOBBERS \
-    "memory", "vcc", "scc", "m0", "s40", "s41", "s42", "s43", "s44", "s45", "s46", "s47", "s48", "s49", "s50", "s51", \
+    "memory", "vcc", "scc", "s40", "s41", "s42", "s43", "s44", "s45", "s46", "s47", "s48", "s49", "s50", "s51", \
     "s52", "s53", "s54", "s55", "s56", "s57", "s58", "s59", "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", \
     "s68", "s69", "s70", "s71", "s72", "s73", "s74", "s75", "s76", "s77", "s78", "s79", "s80", "s81", "s82", "s83", "v0", "v1", "v2", "v3", "v4", \
     "v5", "v6", "v7", "v8", "v9", "v10", "v11", "v12", "v13", "v14", "v15", "v16", "v17", "v18", "v19", "v20", "v21", \
@@ -70,7 +70,7 @@ constexpr int lds_total(int kvt) { return sched_off(kvt) + (2 * SCHED_MAX_SEQ + 
 
 // the k-split programs leave v192 .. v203 alone (the compiler keeps spilled scalars there)
 #define MLA_DECODE_KS_BASE_CLOBBERS \
-    "memory", "vcc", "scc", "m0", "s40", "s41", "s42", "s43", "s44", "s45", "s46", "s47", "s48", "s49", "s50", "s51", \
+    "memory", "vcc", "scc", "s40", "s41", "s42", "s43", "s44", "s45", "s46", "s47", "s48", "s49", "s50", "s51", \
     "s52", "s53", "s54", "s55", "s56", "s57", "s58", "s59", "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", \
     "s68", "s69", "s70", "s71", "s72", "s73", "s74", "s75", "s76", "s77", "s78", "s79", "s80", "s81", "s82", "s83", "v0", "v1", "v2", "v3", "v4", \
     "v5", "v6", "v7", "v8", "v9", "v10", "v11", "v12", "v13", "v14", "v15", "v16", "v17", "v18", "v19", "v20", "v21", \
@@ -655,7 +655,7 @@ __device__ __forceinline__ void decode_body() {
 }
 
 template <int KVT, bool MASK>
-__global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams p) { decode_body<KVT, MASK, 0, false>(); }
+__global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams) { decode_body<KVT, MASK, 0, false>(); }   // (the body reads the argument segment)
 
 // A masked launch of few heads issued in two forms (the launcher's comment tells why): pb describes it as row blocks of 128 rows
 // (balanced == 2), pt token by token (balanced == 3: every query token a sequence of one token, its mask row that sequence's

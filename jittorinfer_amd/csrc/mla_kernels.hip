@@ -239,7 +239,7 @@ __global__ void __launch_bounds__(NTHREADS) mla_attn_tile_kernel(const KParams p
             for (int w = tid; w < TILE_TOK * 18; w += NTHREADS) {
                 const int r  = w / 18;
                 const int bk = w - r * 18;
-                const LDS_PTR(const unsigned short) src = (LDS_PTR(const unsigned short)) (raw + r * Q8_ROW + bk * 34);
+                LDS_PTR(const unsigned short) src = (LDS_PTR(const unsigned short)) (raw + r * Q8_ROW + bk * 34);
                 const float d = f16_bits_to_f32(src[0]);
                 unsigned int o[16];
 #pragma unroll
@@ -514,7 +514,7 @@ __global__ void __launch_bounds__(256) mla_attn_combine_kernel(const KParams p) 
 // latency-bound, so the group should cover every split of a row in one round -- a ragged batch of short sequences has up to 32
 // one-page pieces per sequence -- without issuing many times the loads a row with two or three splits needs.
 template <int G>
-__device__ __forceinline__ void combine_f32_row(const KParams & p, const float2 * ml, const float * po, int64_t ml_step, int64_t po_step, int nvalid, float * dst) {
+__device__ __forceinline__ void combine_f32_row(const float2 * ml, const float * po, int64_t ml_step, int64_t po_step, int nvalid, float * dst) {
     float M = -INFINITY, L = 0.f;
     f32x4 o = { 0.f, 0.f, 0.f, 0.f };
     for (int c0 = 0; c0 < nvalid; c0 += G) {
@@ -552,7 +552,7 @@ __global__ void __launch_bounds__(256) mla_attn_combine_f32_kernel(const KParams
     const int row = blockIdx.x * rows_per_block + threadIdx.x / groups_per_row;
     const int cg  = threadIdx.x % groups_per_row;
     const int seq_len = p.block_table ? min(p.seq_lens[b], (int) p.bt_stride * MLA_PAGE_TOKENS) : (int) p.n_kv;
-    if (row >= p.n_rows || threadIdx.x >= rows_per_block * groups_per_row || cg * 4 >= p.dv_total) return;
+    if (row >= p.n_rows || (int) threadIdx.x >= rows_per_block * groups_per_row || cg * 4 >= p.dv_total) return;
     int slot0, nvalid, lrow, slot_rows;
     partial_slots(p, b, row, seq_len, slot0, nvalid, lrow, slot_rows);
     if (nvalid < 0) return;
@@ -560,9 +560,9 @@ __global__ void __launch_bounds__(256) mla_attn_combine_f32_kernel(const KParams
     const float *  po = (const float *) p.part_o + ((int64_t) slot0 * slot_rows + lrow) * p.dv_total + cg * 4;
     const int64_t ml_step = slot_rows, po_step = (int64_t) slot_rows * p.dv_total;
     float * dst = p.dst + ((int64_t) b * p.n_rows + row) * p.dst_stride + p.v_col0 + cg * 4;
-    if (nvalid <= 4)       combine_f32_row<4>(p, ml, po, ml_step, po_step, nvalid, dst);
-    else if (nvalid <= 16) combine_f32_row<16>(p, ml, po, ml_step, po_step, nvalid, dst);
-    else                   combine_f32_row<32>(p, ml, po, ml_step, po_step, nvalid, dst);
+    if (nvalid <= 4)       combine_f32_row<4>(ml, po, ml_step, po_step, nvalid, dst);
+    else if (nvalid <= 16) combine_f32_row<16>(ml, po, ml_step, po_step, nvalid, dst);
+    else                   combine_f32_row<32>(ml, po, ml_step, po_step, nvalid, dst);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
