@@ -195,6 +195,10 @@ def test_committed_wave_programs_are_what_the_generator_emits(gen, flags, name):
     got = subprocess.run([sys.executable, os.path.join(csrc, gen)] + flags, capture_output=True, text=True, check=True).stdout
     with open(os.path.join(csrc, name)) as f:
         assert got == f.read(), "%s is stale: regenerate it with %s %s" % (name, gen, " ".join(flags))
+    # a program takes and leaves the machine with nothing in flight: what the compiled code ahead of it left outstanding could land on
+    # a register the program has written since, and the other way round
+    lines = [ln for ln in got.splitlines() if ln.startswith('"')]
+    assert lines[0] == '"s_waitcnt vmcnt(0) lgkmcnt(0)\\n\\t"' and lines[-1] == lines[0], (lines[0], lines[-1])
     for m in re.finditer(r"\bv(\d+)\b|\bv\[(\d+):(\d+)\]", got):
         hi = int(m.group(1)) if m.group(1) else int(m.group(3))
         assert hi <= (252 if "--bias" in flags else 251), "%s uses %s" % (name, m.group(0))
