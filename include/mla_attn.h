@@ -124,7 +124,8 @@ typedef struct mla_attn_plan_info {
     int32_t balanced;     /* 1 = paged decode with the balanced schedule: n_workgroups workgroups take equal runs of the batch's
                              page list (n_splits / split_tokens then describe the uniform plan it replaces); 2 = a masked launch
                              over one cache, equal runs of the 32-key tiles its blocks of 128 rows may attend to; 4 = such a
-                             launch with at most 32 heads and 256 query tokens: issued both in that form and token by token
+                             launch with few heads (up to 32; 33 to 64 that do not divide 128, or of Q8_0 cells) and at most 256
+                             query tokens: issued both in that form and token by token
                              (every query token's rows a workgroup's rows), the device runs the one with fewer tiles to visit */
     int32_t n_workgroups;
 } mla_attn_plan_info;

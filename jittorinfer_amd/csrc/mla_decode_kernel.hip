@@ -702,7 +702,9 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_dual_kernel(const KParams
     __syncthreads();
     const int blk = __builtin_amdgcn_readfirstlane(tot[0] + tot[2] + tot[4] + tot[6]);
     const int tok = __builtin_amdgcn_readfirstlane(tot[1] + tot[3] + tot[5] + tot[7]);
-    const bool token_form = 2 * (int64_t) tok <= 3 * (int64_t) blk;
+    // (a token of 33 to 64 rows runs the row-split program on two of the four waves: a tile of it costs nearly what a row block's
+    // does -- 32 tokens x 8192 cells at 64 heads: 80 against 83 us -- so that form only runs where it visits fewer tiles)
+    const bool token_form = pt.n_rows <= 32 ? 2 * (int64_t) tok <= 3 * (int64_t) blk : 16 * (int64_t) tok <= 15 * (int64_t) blk;
     if (blockIdx.x == 0 && t == 0) *pb.form = token_form ? 3 : 2;   // for the combine pass
     static_assert(sizeof(KParams) % 8 == 0, "the second KParams follows the first without padding");
     if (token_form) decode_body<KVT_TOK, true, (int) sizeof(KParams), true>();
@@ -752,9 +754,9 @@ __device__ __forceinline__ void mask_extent_block_tokens(const KParams & p, int 
 // 16 pairs and rounds outwards to tiles.  grid = (n_row_blocks, 16), block = 256.  The mask is shared by all sequences
 // (ggml-cpu.c:12024).
 // A launch issued in two forms (p.dual) keeps the pairs per query token instead -- the token form's items; a row block's range is the
-// merge of its tokens' -- and scans them with one block per (token, sixteenth) when the row blocks are few: a decode batch has few of
-// them and a mask row as long as the whole cache (`sub` numbers the tokens of the row block, p.mask_ext_sub > 1 of them), or else
-// with a wave per token.  A token whose heads straddle two row blocks is scanned for both, with the same result.
+// merge of its tokens' -- and scans them with one block per (token, sixteenth) when the mask rows are long: a decode batch has few
+// row blocks and a mask row as long as the whole cache (`sub` numbers the tokens of the row block, p.mask_ext_sub > 1 of them), or
+// else with a wave per token.  A token whose heads straddle two row blocks is scanned for both, with the same result.
 __device__ __forceinline__ void mask_extent_block(const KParams & p, int rb, int chunk, int sub) {
     __shared__ int red_hi[NTHREADS], red_lo[NTHREADS];
     const int tid = threadIdx.x;
@@ -826,6 +828,23 @@ __device__ __forceinline__ bool pack_launch_extent_layer(const KParams & p) {
 // grid = (n_row_blocks, n_seq, 36 k-steps), block = 256: one 16-byte output per thread.
 // MODE 0: bf16 operands; 1: f16; 2: rounded to bf16 as for MODE 0, then written as f16 (exact inside the f16 range,
 // +-65504 beyond it) for the program that converts its bf16 tiles to f16.
+// Which rows a wave of a pack launch rounds, and where to.  A launch issued in two forms whose token form takes an operand image
+// (p.tok_q_pack) has more layers of blocks along y: layer 0 is the one sequence in its row-block form; the waves of block
+// (x, y >= 1) take query tokens as sequences of one token of n_head <= 64 rows each, one wave (two from 33 heads on) per token:
+// four (two) tokens to a block.  `wave`: the wave of the decode kernel whose operands these are.
+struct PackWhere { int rb, b, n_rb, n_rows, wave; int64_t q_nb3; void * image; bool token; };
+__device__ __forceinline__ int pack_tokens_per_block(int n_head) { return n_head <= 32 ? 4 : 2; }
+__device__ __forceinline__ bool pack_where(const KParams & p, int wave, PackWhere & w) {
+    w = PackWhere{ (int) blockIdx.x, (int) blockIdx.y, (int) gridDim.x, p.n_rows, wave, p.q_nb3, p.q_pack, false };
+    if (p.tok_q_pack && blockIdx.y >= 1) {
+        const int tpb = pack_tokens_per_block(p.n_head), wpt = 4 / tpb;
+        const int t = (((int) blockIdx.y - 1) * (int) gridDim.x + (int) blockIdx.x) * tpb + wave / wpt;
+        if (t >= p.n_tok) return false;
+        w = PackWhere{ 0, t, 1, p.n_head, wave % wpt, p.q_nb1, p.tok_q_pack, true };
+    }
+    return true;
+}
+
 template <int MODE> __device__ __forceinline__ unsigned int pack_q2(float a, float b) {
     if constexpr (MODE == 2) {
         const auto h = __builtin_amdgcn_cvt_pkrtz(round_trip<false>(a), round_trip<false>(b));
@@ -841,14 +860,22 @@ __global__ void __launch_bounds__(NTHREADS) mla_q_pack_kernel(const KParams p) {
     }
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int g = lane >> 5, rl = lane & 31;
-    const int b = blockIdx.y, ks = blockIdx.z;
-    if ((int) blockIdx.x * 128 + wave * 32 >= p.n_rows) return;   // a wave of the decode kernel without a row: it computes nothing, its image is never used
-    const int row = min((int) blockIdx.x * 128 + wave * 32 + rl, p.n_rows - 1);
+    const int ks = blockIdx.z;
+    PackWhere w;
+    if (!pack_where(p, wave, w)) return;
+    if (w.rb * 128 + w.wave * 32 >= w.n_rows) return;   // a wave of the decode kernel without a row: it computes nothing, its image is never used
+    const int row = min(w.rb * 128 + w.wave * 32 + rl, w.n_rows - 1);
     const int tq = row / p.n_head, head = row - tq * p.n_head;
-    const float * qrow = (const float *) (p.q + (int64_t) tq * p.q_nb1 + (int64_t) head * p.q_nb2 + (int64_t) b * p.q_nb3) + 8 * g;
-    u32x4 * out = (u32x4 *) p.q_pack + ((((int64_t) b * gridDim.x + blockIdx.x) * 4 + wave) * KSTEPS) * 64 + lane;
+    const float * qrow = (const float *) (p.q + (int64_t) tq * p.q_nb1 + (int64_t) head * p.q_nb2 + (int64_t) w.b * w.q_nb3) + 8 * g;
+    u32x4 * out = (u32x4 *) w.image + ((((int64_t) w.b * w.n_rb + w.rb) * 4 + w.wave) * KSTEPS) * 64 + lane;
     const f32x4 x0 = *(const f32x4 *) (qrow + 16 * ks);
     const f32x4 x1 = *(const f32x4 *) (qrow + 16 * ks + 4);
+    // (the token form of a launch issued in two forms may want another rounding than the row-block form: p.tok_mode)
+    if (w.token && p.tok_mode != MODE) {
+        if (p.tok_mode == 2) out[ks * 64] = u32x4{ pack_q2<2>(x0.x, x0.y), pack_q2<2>(x0.z, x0.w), pack_q2<2>(x1.x, x1.y), pack_q2<2>(x1.z, x1.w) };
+        else                 out[ks * 64] = u32x4{ pack_q2<1>(x0.x, x0.y), pack_q2<1>(x0.z, x0.w), pack_q2<1>(x1.x, x1.y), pack_q2<1>(x1.z, x1.w) };
+        return;
+    }
     out[ks * 64] = u32x4{ pack_q2<MODE>(x0.x, x0.y), pack_q2<MODE>(x0.z, x0.w), pack_q2<MODE>(x1.x, x1.y), pack_q2<MODE>(x1.z, x1.w) };
 }
 
@@ -863,11 +890,15 @@ __global__ void __launch_bounds__(NTHREADS) mla_q_pack_q8_kernel(const KParams p
     }
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int g = lane >> 5, rl = lane & 31;
-    const int b = blockIdx.y, j = blockIdx.z;
-    const int row = min((int) blockIdx.x * 128 + wave * 32 + rl, p.n_rows - 1);
+    const int j = blockIdx.z;
+    PackWhere w;
+    if (!pack_where(p, wave, w)) return;
+    // (the row-block form writes the image of every wave, rows past the end repeating the last one: the Q8_0 program loads it in
+    // waves without a row too; the token form leaves such a wave's part as it is -- its values are never used)
+    const int row = min(w.rb * 128 + w.wave * 32 + rl, w.n_rows - 1);
     const int tq = row / p.n_head, head = row - tq * p.n_head;
-    const float * qrow = (const float *) (p.q + (int64_t) tq * p.q_nb1 + (int64_t) head * p.q_nb2 + (int64_t) b * p.q_nb3);
-    u32x4 * out = (u32x4 *) p.q_pack + ((((int64_t) b * gridDim.x + blockIdx.x) * 4 + wave) * KSTEPS) * 64 + lane;
+    const float * qrow = (const float *) (p.q + (int64_t) tq * p.q_nb1 + (int64_t) head * p.q_nb2 + (int64_t) w.b * w.q_nb3);
+    u32x4 * out = (u32x4 *) w.image + ((((int64_t) w.b * w.n_rb + w.rb) * 4 + w.wave) * KSTEPS) * 64 + lane;
     f32x4 x[4];
     x[0] = *(const f32x4 *) (qrow + 32 * j + 8 * g);
     x[1] = *(const f32x4 *) (qrow + 32 * j + 8 * g + 4);
@@ -1028,27 +1059,43 @@ hipError_t launch_decode_fast(const KParams & kp_in, int kv_type, dim3 grid, hip
     const bool q_in_kernel = ks || (cs && !bias && kp_in.n_splits == 1 && !kp_in.balanced);
     KParams kp = kp_in;
     kp.q_in_kernel = q_in_kernel ? 1 : 0;
+    // a launch issued in two forms: what its token form runs, and whether that takes an operand image of its own
+    const bool tok_ks = tok && decode_ks_applicable(*tok, kv_type);
+    if (tok && (!m || ks || bias || kp.bf16_direct || kp.q_as_q8 || q_in_kernel)) return hipErrorInvalidValue;
+    if (tok && !tok_ks && tok->n_rows > 64) return hipErrorInvalidValue;
+    kp.tok_q_pack = tok && !tok_ks ? tok->q_pack : nullptr;
+    kp.tok_mode   = kv_type == MLA_TYPE_F16 ? 1 : 2;
+    const unsigned tok_blocks = (unsigned) ((kp.n_tok + (kp.n_head <= 32 ? 4 : 2) - 1) / (kp.n_head <= 32 ? 4 : 2));   // (pack_tokens_per_block)
+    const unsigned tok_layers = kp.tok_q_pack ? (tok_blocks + n_rb - 1) / n_rb : 0;
     // elsewhere the scan of the mask extents rides in the pack launch (a masked launch has no balanced page schedule, so its layers
     // and the schedule layer never meet; if they ever did, the scan would keep a launch of its own)
     const bool fold = m && !extra && !q_in_kernel;
     // (a launch issued in two forms scans per query token: 16 layers for each of the tokens a row block can hold)
-    const int ext_sub = kp.dual && n_rb * MASK_EXT_CHUNKS < 256 ? min(kp.n_tok, 127 / kp.n_head + 2) : 1;
+    // long mask rows -- a decode batch: the row spans the whole cache; a sixteenth of it is a block's worth of 16-byte groups from
+    // 32768 keys on -- get a block per (token, sixteenth), shorter ones (a prompt chunk) a wave per token
+    const int ext_sub = kp.dual && kp.n_kv >= 32768 ? min(kp.n_tok, 127 / kp.n_head + 2) : 1;
     kp.mask_ext_in_pack = fold ? 1 : 0;
     kp.mask_ext_sub = ext_sub;
     const unsigned ext = fold ? MASK_EXT_CHUNKS * ext_sub : 0;
     if (!with_prepass) { /* the workspace still holds the Q image and the mask extents of an earlier launch of the same call */ }
     else if (q_in_kernel) { /* nothing: a balanced page schedule is worked out by the workgroups themselves */ }
-    else if (kv_type == MLA_TYPE_Q8_0 || kp.q_as_q8) hipLaunchKernelGGL(mla_q_pack_q8_kernel, dim3(n_rb, n_seq, KSTEPS / 2 + extra + ext), dim3(NTHREADS), 0, st, kp);
-    else if (kv_type == MLA_TYPE_F16) hipLaunchKernelGGL(mla_q_pack_kernel<1>, dim3(n_rb, n_seq, KSTEPS + extra + ext), dim3(NTHREADS), 0, st, kp);
-    else if (bf16_cvt)                hipLaunchKernelGGL(mla_q_pack_kernel<2>, dim3(n_rb, n_seq, KSTEPS + extra + ext), dim3(NTHREADS), 0, st, kp);
-    else                              hipLaunchKernelGGL(mla_q_pack_kernel<0>, dim3(n_rb, n_seq, KSTEPS + extra + ext), dim3(NTHREADS), 0, st, kp);
+    else if (kv_type == MLA_TYPE_Q8_0 || kp.q_as_q8) hipLaunchKernelGGL(mla_q_pack_q8_kernel, dim3(n_rb, n_seq + tok_layers, KSTEPS / 2 + extra + ext), dim3(NTHREADS), 0, st, kp);
+    else if (kv_type == MLA_TYPE_F16) hipLaunchKernelGGL(mla_q_pack_kernel<1>, dim3(n_rb, n_seq + tok_layers, KSTEPS + extra + ext), dim3(NTHREADS), 0, st, kp);
+    else if (bf16_cvt)                hipLaunchKernelGGL(mla_q_pack_kernel<2>, dim3(n_rb, n_seq + tok_layers, KSTEPS + extra + ext), dim3(NTHREADS), 0, st, kp);
+    else                              hipLaunchKernelGGL(mla_q_pack_kernel<0>, dim3(n_rb, n_seq + tok_layers, KSTEPS + extra + ext), dim3(NTHREADS), 0, st, kp);
     if (m && !fold && with_prepass) hipLaunchKernelGGL(mla_mask_extent_kernel, dim3(n_rb, MASK_EXT_CHUNKS, ext_sub), dim3(NTHREADS), 0, st, kp);
     if (tok) {
-        if (!m || ks || bias || kp.bf16_direct || kp.q_as_q8 || (kv_type != MLA_TYPE_BF16 && kv_type != MLA_TYPE_F16)) return hipErrorInvalidValue;
+        // the row-block form as chosen above; the token form: the k-split program up to 32 rows of 16-bit cells (it rounds Q itself), else
+        // the row-split program of the cache type, whose operand image the pack launch above has written token by token
         KParams kt = *tok;
-        kt.q_in_kernel = 1;   // (the k-split program)
-        if (cs) return kv_type == MLA_TYPE_F16 ? launch_dual<SRC_F16_CS, SRC_F16_KS>(kp, kt, grid, st) : launch_dual<SRC_BF16_CS, SRC_BF16_KS>(kp, kt, grid, st);
-        return kv_type == MLA_TYPE_F16 ? launch_dual<SRC_F16, SRC_F16_KS>(kp, kt, grid, st) : launch_dual<SRC_BF16_CVT, SRC_BF16_KS>(kp, kt, grid, st);
+        kt.q_in_kernel = tok_ks ? 1 : 0;
+        if (kv_type == MLA_TYPE_Q8_0) return launch_dual<SRC_Q8, SRC_Q8>(kp, kt, grid, st);
+        if (kv_type == MLA_TYPE_F16) {
+            if (cs) return tok_ks ? launch_dual<SRC_F16_CS, SRC_F16_KS>(kp, kt, grid, st) : launch_dual<SRC_F16_CS, SRC_F16>(kp, kt, grid, st);
+            return tok_ks ? launch_dual<SRC_F16, SRC_F16_KS>(kp, kt, grid, st) : launch_dual<SRC_F16, SRC_F16>(kp, kt, grid, st);
+        }
+        if (cs) return tok_ks ? launch_dual<SRC_BF16_CS, SRC_BF16_KS>(kp, kt, grid, st) : launch_dual<SRC_BF16_CS, SRC_BF16_CVT>(kp, kt, grid, st);
+        return tok_ks ? launch_dual<SRC_BF16_CVT, SRC_BF16_KS>(kp, kt, grid, st) : launch_dual<SRC_BF16_CVT, SRC_BF16_CVT>(kp, kt, grid, st);
     }
     if (kv_type == MLA_TYPE_Q8_0) return m ? launch_variant<SRC_Q8, true>(kp, grid, st) : launch_variant<SRC_Q8, false>(kp, grid, st);
     if (ks && m) return kv_type == MLA_TYPE_F16 ? launch_variant<SRC_F16_KS, true>(kp, grid, st) : launch_variant<SRC_BF16_KS, true>(kp, grid, st);

@@ -741,10 +741,18 @@ int validate(const mla_attn_args * a) {
 // tokens of a block share their cells, and the token form would read them once per token.  The arguments do not tell the two
 // apart, the mask on the device does: such a launch is issued in both forms at once, to a kernel that holds the programs of both;
 // every workgroup adds up the tiles either form would visit (from the mask extents) and runs the cheaper one.
+// Up to 32 heads of 16-bit cells the token form is the k-split program; from 33 to 64 heads, and for Q8_0 cells the wave program copies
+// as raw tiles, it is the row-split program of the cache type (one or two of its four waves with rows), which takes an operand
+// image of its own (token_image_bytes; written by more layers of the pack launch).  Not 64 heads of 16-bit cells: a row block is
+// two tokens exactly, the token form never visits fewer tiles and its tile costs the same (32 tokens x 8192 cells: 99.5 us
+// per step against 98.3 us).  48 heads: 113 -> 98 us; Q8_0 cells, 16 / 32 / 64 heads: 105 -> 85, 94 -> 86, 95 -> 89 us.
 static bool token_form_candidate(const mla_attn_args * a, const Plan & pl) {
-    return pl.variant == 2 && pl.balanced == 2 && a->n_tok <= 256 && a->n_head <= 32 && (int64_t) a->n_tok * a->n_head > 32 &&
-           (a->kv_type == MLA_TYPE_BF16 || a->kv_type == MLA_TYPE_F16) && !(a->flags & MLA_FLAG_BF16_DIRECT) &&
-           a->logit_softcap == 0.0f && !(a->max_bias > 0.0f);
+    if (a->n_head > 32 && a->kv_type != MLA_TYPE_Q8_0 && 128 % a->n_head == 0) return false;
+    return pl.variant == 2 && pl.balanced == 2 && a->n_tok <= 256 && a->n_head <= 64 && (int64_t) a->n_tok * a->n_head > 32 && a->n_tok > 1 &&
+           pl.kvcopy_rows == 0 && !(a->flags & MLA_FLAG_BF16_DIRECT) && a->logit_softcap == 0.0f && !(a->max_bias > 0.0f);
+}
+static size_t token_image_bytes(const mla_attn_args * a) {
+    return a->kv_type == MLA_TYPE_Q8_0 || a->n_head > 32 ? decode_fast_qpack_bytes(a->n_tok, 1) : 0;
 }
 
 int make_plan(const mla_attn_args * a, Plan * pl) {
@@ -837,6 +845,7 @@ int make_plan(const mla_attn_args * a, Plan * pl) {
     if (token_form_candidate(a, *pl)) {
         pl->dual = 1;
         pl->ws_maskext = (size_t) a->n_tok * 16 * 2 * sizeof(int);   // 16 pairs per query token
+        pl->ws_qpack  += token_image_bytes(a);
         pl->ws_sched   = (size_t) ((std::max(pl->n_units, a->n_tok) + 1 + 63) / 64 * 64 + pl->n_wg * 8) * sizeof(int);
     }
     if (pl->n_splits > 1) {
@@ -953,6 +962,7 @@ static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
         kp.dual = 1; kt.dual = 2;
         kp.form = kt.form = kp.wg_first;   // (a masked launch has no use for that table)
         kt.q_nb3 = a->q_nb1; kt.kv_nb3 = 0; kt.mask_nb3 = a->mask_nb1;
+        kt.q_pack = (char *) kp.q_pack + decode_fast_qpack_bytes(a->n_seq, pl.n_row_blocks);   // (behind the row-block form's image)
         kt.n_tok = 1; kt.n_rows = a->n_head; kt.slot_rows = a->n_head;
         kt.balanced = 3; kt.n_units = a->n_tok; kt.n_seq_sched = a->n_tok;
     }

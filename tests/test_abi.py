@@ -165,9 +165,13 @@ def test_planner_schedules_without_gpu():
     rc, info, ws = _plan(n_head=16, **batch)                     # 16 heads: issued both as row blocks and token by token
     assert rc == 0 and info.variant == 2 and info.balanced == 4 and info.n_row_blocks == 4 and info.n_workgroups == 256
     assert ws >= (256 + 4) * 128 * 512 * 2 + 32 * 16 * 8         # the row-block form's partials hold the token form's; 16 key pairs per token
-    for kw in (dict(n_head=16, n_tok=2), dict(n_head=16, n_tok=257), dict(n_head=64), dict(n_head=16, kv_type=J.MLA_TYPE_Q8_0, kv_nb1=612),
+    for kw in (dict(n_head=48), dict(n_head=16, kv_type=J.MLA_TYPE_Q8_0, kv_nb1=612), dict(n_head=64, kv_type=J.MLA_TYPE_Q8_0, kv_nb1=612)):
+        rc, info, ws2 = _plan(**{**batch, **kw})                # up to 64 heads, and Q8_0 cells: the token form is the row-split program
+        assert rc == 0 and info.balanced == 4, kw
+        assert ws2 >= 32 * 4 * 36 * 1024                        # ... which takes an operand image per token
+    for kw in (dict(n_head=16, n_tok=2), dict(n_head=16, n_tok=257), dict(n_head=65), dict(n_head=64), dict(n_head=48, n_tok=1),
                dict(n_head=16, flags=J.MLA_FLAG_BF16_DIRECT), dict(n_head=16, max_bias=8.0)):
-        rc, info, _ = _plan(**{**batch, **kw})                  # at most 32 rows, more than 256 tokens, more than 32 heads, Q8_0 rows, ...: one form
+        rc, info, _ = _plan(**{**batch, **kw})                  # at most 32 rows, more than 256 tokens, more than 64 heads, two tokens to a row block exactly, ...: one form
         assert rc == 0 and info.balanced in (0, 2), kw
 
 
