@@ -92,11 +92,13 @@ def test_scheduler_set_up_as_llama_sets_it_up(gpu, paged):
 
 
 @pytest.mark.parametrize("use_sched", [False, True])
-def test_batched_decode_through_the_mask_as_llama_builds_it(gpu, use_sched):
+@pytest.mark.parametrize("n_head", [128, 16])
+def test_batched_decode_through_the_mask_as_llama_builds_it(gpu, use_sched, n_head):
     """The reference's decode batch: one shared cache, one query token per sequence, the f16 mask padded to 64 rows selects
     each token's own cells (src/llama-context.cpp:364-404); V is the 512-wide latent prefix view of K.  The reference's
-    compiled ggml drives the plugin; the pipelined masked kernel computes the node."""
-    rng = np.random.default_rng(23)
+    compiled ggml drives the plugin; the pipelined masked kernel computes the node (16 heads: issued as row blocks and token
+    by token, the device runs the token form)."""
+    rng = np.random.default_rng(23 + n_head)
     n_kv, lens = 1024, [200, 256, 31, 300]
     k = U.encode_kv(rng.standard_normal((1, n_kv, 576)).astype(np.float32), O.TYPE_BF16)
     m = np.full((len(lens), n_kv), -np.inf, dtype=np.float32)
@@ -105,7 +107,7 @@ def test_batched_decode_through_the_mask_as_llama_builds_it(gpu, use_sched):
         m[s, pos:pos + l] = 0.0
         pos += l + 20
     mask = m.astype(np.float16).view(np.uint16)
-    q = rng.standard_normal((1, 128, len(lens), 576)).astype(np.float32)
+    q = rng.standard_normal((1, n_head, len(lens), 576)).astype(np.float32)
     got, info = O.ref_backend_flash_attn_ext(_so(), q, k, O.TYPE_BF16, dv=512, mask=mask, scale=U.SCALE, use_sched=use_sched)
     want = O.flash_attn_ext(q, k, O.TYPE_BF16, dv=512, mask=mask, scale=U.SCALE)
     print(U.check(got[..., :512], want, "masked batched decode through the reference's ggml"))
