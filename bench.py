@@ -339,6 +339,14 @@ def other_config(a, dev, lib, J):
         out = torch.empty((len(lens), n_tok, n_head, 576), dtype=torch.float32, device=dev)
     kw = dict(dv=512, scale=scale, mask=mask, block_table=bt, seq_lens=sl, out=out, n_splits=a.splits, rows_per_wg=a.rows_per_wg,
               flags=(J.MLA_FLAG_UNIFORM_SPLITS if a.uniform_splits else 0) | (J.MLA_FLAG_BF16_DIRECT if a.bf16_direct else 0))
+    if a.reuse_mask_extents:
+        # the node of a layer after the first of a graph: the mask is the one whose extents the launch before left in the workspace
+        assert mask is not None, "--reuse-mask-extents needs a masked config"
+        ar0, _, keep0 = J.capi.make_args(q, pool, kvt, **kw)
+        rc = lib.mla_attn_launch(C.byref(ar0), C.c_void_p(torch.cuda.current_stream(dev).cuda_stream))
+        assert rc == 0, rc
+        torch.cuda.synchronize()
+        kw["flags"] |= J.MLA_FLAG_MASK_EXTENTS_VALID
     ar, _, keep = J.capi.make_args(q, pool, kvt, **kw)
     plan = J.plan(q, pool, kvt, **kw)
     stream = torch.cuda.current_stream(dev)
@@ -452,6 +460,7 @@ def main():
                     help="also launch the library's plain copy kernel N times over one KV pool (known byte count) so that a "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run can be scaled")
     ap.add_argument("--kv", default="bf16", choices=["bf16", "f16", "q8_0"], help="storage type of the latent KV pool (the headline config is bf16; q8_0 only with --config kvwrite)")
+    ap.add_argument("--reuse-mask-extents", action="store_true", help="masked configs: time the launch of a layer after the first of a graph, which finds the key extents of the shared mask in the workspace (MLA_FLAG_MASK_EXTENTS_VALID)")
     ap.add_argument("--ragged", action="store_true", help="--config c3mask: sequence lengths uniform in [2048, 8192] instead of 8192")
     ap.add_argument("--uniform-splits", action="store_true", help="paged decode: equal KV splits per sequence (MLA_FLAG_UNIFORM_SPLITS) instead of the balanced schedule")
     ap.add_argument("--bf16-direct", action="store_true", help="bf16 KV: the hi + lo bf16 program (MLA_FLAG_BF16_DIRECT) instead of the default one that converts the tiles to f16 inside LDS")

@@ -103,6 +103,12 @@ int mla_ggml_supports_node(const void * ggml_tensor_node, const char ** why);
  * node it accepts this returns 0 -- tests/test_supports_op.py checks that over generated nodes. */
 int mla_ggml_node_launch_check(const void * ggml_tensor_node);
 
+/* no counterpart: how many FLASH_ATTN_EXT nodes this process has launched with the key extents of their mask taken from the
+ * node before them in the same graph (the layers of one llama graph share their mask tensor,
+ * src/llama-graph-deepseek2.cpp:99-103) instead of scanning the mask again; GGML_HIP_MLA_MASK_EXTENTS=rescan, or
+ * "mask_extents=rescan" in the params of init_backend, turns that off.  For tests and diagnostics. */
+int64_t mla_ggml_mask_extent_reuses(void);
+
 /* no counterpart: frees a buffer obtained from this backend's buffer type when no ggml is present in the process
  * to do it (what ggml_backend_buffer_free does, ggml/src/ggml-backend.cpp). */
 void mla_ggml_buffer_free(void * ggml_backend_buffer);

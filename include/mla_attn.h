@@ -40,6 +40,11 @@ extern "C" {
 #define MLA_FLAG_UNIFORM_SPLITS 2u /* paged decode: give every sequence the same number of equal KV splits (sized for the longest
                                       sequence the block table can hold) instead of the balanced schedule that deals equal
                                       runs of the batch's whole page list to the workgroups; for comparing the two */
+#define MLA_FLAG_MASK_EXTENTS_VALID 8u /* masked launch: the workspace still holds the key extents of this mask, left there by the
+                                      launch before it, which had the same arguments except q, kv and dst (the attention nodes of
+                                      the layers of one graph share their mask, src/llama-graph-deepseek2.cpp:99-103): the scan of
+                                      the mask is left out.  The caller vouches for it; nothing else may have used the workspace
+                                      in between. */
 #define MLA_FLAG_BF16_DIRECT 4u    /* BF16 KV, pipelined kernel: multiply the bf16 tiles as they are, with the probabilities fed as
                                       hi + lo bf16 halves (100 MFMAs per 32 keys).  Without the flag, and with more than 32
                                       attention rows (heads x query tokens) per sequence, the tiles are converted

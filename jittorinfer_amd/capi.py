@@ -8,6 +8,7 @@ MLA_TYPE_F32, MLA_TYPE_F16, MLA_TYPE_Q8_0, MLA_TYPE_BF16 = 0, 1, 8, 30
 MLA_FLAG_F16_ACC_STRICT = 1
 MLA_FLAG_UNIFORM_SPLITS = 2
 MLA_FLAG_BF16_DIRECT = 4
+MLA_FLAG_MASK_EXTENTS_VALID = 8
 MLA_ERR_TOO_LARGE = -7
 MLA_ATTN_STATIC_WORKSPACE_MAX = 48 << 20
 PAGE_TOKENS = 128

@@ -20,6 +20,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <atomic>
 #include <mutex>
 #include <string>
 #include <vector>
@@ -69,12 +70,20 @@ struct backend_ctx {
     size_t      workspace_size = 0;
     bool        f16_strict     = false;   // F16 KV: replay ggml-cpu's f16 accumulator instead of accumulating in f32
     bool        bf16_direct    = false;   // BF16 KV: the hi + lo bf16 program instead of the one that converts the tiles to f16 (MLA_FLAG_BF16_DIRECT)
+    // The attention nodes of the layers of one graph share their mask (one KQ_mask tensor per graph, src/llama-graph-deepseek2.cpp:99-103):
+    // the key extents the first of them leaves in the workspace serve the others (MLA_FLAG_MASK_EXTENTS_VALID).  ext_key: the
+    // arguments of the launch whose extents the workspace holds, q / kv / dst blanked; valid inside one graph_compute call, while no
+    // node writes the mask and nothing else uses the workspace.
+    bool          reuse_mask_extents = true;
+    bool          ext_key_valid      = false;
+    mla_attn_args ext_key;
 };
 
 std::vector<device_ctx *>     g_device_ctx;
 std::vector<backend_device *> g_devices;
 backend_reg                   g_reg;
 std::once_flag                g_once;
+std::atomic<int64_t>          g_mask_extent_reuses{ 0 };
 uint8_t                       g_guid[16] = { 0x6d, 0x6c, 0x61, 0x2d, 0x68, 0x69, 0x70, 0x2d, 0x67, 0x66, 0x78, 0x39, 0x35, 0x30, 0x00, 0x01 };
 
 int64_t nelements(const tensor * t) { return t->ne[0] * t->ne[1] * t->ne[2] * t->ne[3]; }
@@ -587,13 +596,20 @@ int compute_flash_attn(backend_ctx * ctx, const tensor * dst) {
         // grow the scratch area; work already queued on the stream may still be using the old one
         if (!HIP_OK(hipStreamSynchronize(ctx->stream))) return STATUS_FAILED;
         if (ctx->workspace) (void) hipFree(ctx->workspace);
-        ctx->workspace = nullptr; ctx->workspace_size = 0;
+        ctx->workspace = nullptr; ctx->workspace_size = 0; ctx->ext_key_valid = false;
         if (!HIP_OK(hipMalloc(&ctx->workspace, need))) { log_error("workspace of %zu bytes: out of memory", need); return STATUS_ALLOC_FAILED; }
         ctx->workspace_size = need;
     }
     a.workspace = ctx->workspace; a.workspace_size = ctx->workspace_size;
+    mla_attn_args key;       // (what the extents depend on: everything but the operands that change from layer to layer)
+    memcpy(&key, &a, sizeof(key));
+    key.q = nullptr; key.kv = nullptr; key.dst = nullptr;
+    const bool same_mask = a.mask && ctx->reuse_mask_extents && ctx->ext_key_valid && memcmp(&key, &ctx->ext_key, sizeof(key)) == 0;
+    if (same_mask) { a.flags |= MLA_FLAG_MASK_EXTENTS_VALID; g_mask_extent_reuses++; }
     const int rc = mla_attn_launch(&a, ctx->stream);
+    ctx->ext_key_valid = false;
     if (rc != 0) { log_error("mla_attn_launch failed for node '%s': %d", dst->name, rc); return STATUS_FAILED; }
+    if (a.mask) { memcpy(&ctx->ext_key, &key, sizeof(key)); ctx->ext_key_valid = true; }
     return STATUS_SUCCESS;
 }
 
@@ -660,9 +676,16 @@ int compute_front(backend_ctx * ctx, const tensor * dst) {
 int backend_graph_compute(backend * be, cgraph * g) {
     backend_ctx * ctx = (backend_ctx *) be->context;
     if (!HIP_OK(hipSetDevice(ctx->device))) return STATUS_FAILED;
+    ctx->ext_key_valid = false;   // (the mask is an input of the graph: it may have been set anew since the last call)
     for (int i = 0; i < g->n_nodes; i++) {
         const tensor * node = g->nodes[i];
         if (is_empty(node) || is_noop(node->op)) continue;
+        // a node that writes into the mask whose extents the workspace holds (none of the reference's graphs has one) ends their validity
+        if (ctx->ext_key_valid && node->data && ctx->ext_key.mask && node->op != OP_FLASH_ATTN_EXT) {
+            const char * m0 = (const char *) ctx->ext_key.mask, * m1 = m0 + (size_t) ctx->ext_key.mask_nb1 * (size_t) ctx->ext_key.n_tok;
+            const char * d0 = (const char *) node->data, * d1 = d0 + tensor_nbytes(node);
+            if (d0 < m1 && m0 < d1) ctx->ext_key_valid = false;
+        }
         int st;
         switch (node->op) {
             case OP_FLASH_ATTN_EXT: st = compute_flash_attn(ctx, node); break;
@@ -740,6 +763,8 @@ backend * device_init_backend(backend_device * dev, const char * params) {
     ctx->f16_strict = (params && strstr(params, "f16_acc=strict")) || (env && strcmp(env, "strict") == 0);
     const char * env_bf = getenv("GGML_HIP_MLA_BF16");
     ctx->bf16_direct = (params && strstr(params, "bf16=direct")) || (env_bf && strcmp(env_bf, "direct") == 0);
+    const char * env_ext = getenv("GGML_HIP_MLA_MASK_EXTENTS");   // "rescan": every attention node scans its mask itself
+    ctx->reuse_mask_extents = !((params && strstr(params, "mask_extents=rescan")) || (env_ext && strcmp(env_ext, "rescan") == 0));
     if (!HIP_OK(hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking))) { delete ctx; return nullptr; }
     return new backend{ &g_guid, k_backend_iface, dev, ctx };
 }
@@ -886,6 +911,8 @@ void * ggml_backend_init(void) {
 }
 
 int ggml_backend_score(void) { return gfx950_device_count() > 0 ? 100 : 0; }
+
+int64_t mla_ggml_mask_extent_reuses(void) { return g_mask_extent_reuses.load(); }
 
 void * ggml_backend_hip_mla_reg(void) { return ggml_backend_init(); }
 

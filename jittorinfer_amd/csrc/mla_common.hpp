@@ -145,7 +145,7 @@ inline hipError_t raise_lds_limit(const void * fn, bool (&done)[MLA_MAX_DEVICES]
 int64_t    decode_fast_q8_copy_rows(const mla_attn_args * a);   // > 0: Q8_0 + mask on rows the wave program cannot tile runs on an f16 copy of that many rows (workspace)
 hipError_t launch_mask_extent(const KParams & kp, hipStream_t st);   // fills kp.mask_ext: 16 key pairs per block of 128 rows
 hipError_t launch_q8_to_f16(const char * src, int64_t src_nb1, int64_t src_nb3, int64_t rows_per_batch, void * dst, int64_t n_rows, hipStream_t st);
-hipError_t launch_decode_fast(const KParams & kp, int kv_type, dim3 grid, hipStream_t st, bool with_prepass, const KParams * tok = nullptr);
+hipError_t launch_decode_fast(const KParams & kp, int kv_type, dim3 grid, hipStream_t st, bool with_prepass, const KParams * tok = nullptr, bool scan_mask = true);
 size_t     decode_fast_lds_bytes(int kv_type);
 size_t     decode_fast_qpack_bytes(int n_seq, int n_row_blocks);
 

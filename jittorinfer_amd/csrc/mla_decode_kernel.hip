@@ -1040,7 +1040,8 @@ static hipError_t launch_dual(const KParams & kb, const KParams & kt, dim3 grid,
 }
 
 // tok: the same launch in its token form, when it is issued in both (masked, 16-bit rows, no bias; see mla_decode_dual_kernel)
-hipError_t launch_decode_fast(const KParams & kp_in, int kv_type, dim3 grid, hipStream_t st, bool with_prepass, const KParams * tok) {
+// scan_mask false: the mask extents in the workspace are still those of this mask (MLA_FLAG_MASK_EXTENTS_VALID)
+hipError_t launch_decode_fast(const KParams & kp_in, int kv_type, dim3 grid, hipStream_t st, bool with_prepass, const KParams * tok, bool scan_mask) {
     // the small passes ahead of the kernel run per (row block, sequence), whatever the kernel's own grid is
     const unsigned n_rb = (unsigned) ((kp_in.n_rows + 127) / 128), n_seq = (unsigned) kp_in.n_seq_sched, extra = kp_in.balanced == 1 ? 1 : 0;
     const bool m = kp_in.mask != nullptr;
@@ -1069,7 +1070,7 @@ hipError_t launch_decode_fast(const KParams & kp_in, int kv_type, dim3 grid, hip
     const unsigned tok_layers = kp.tok_q_pack ? (tok_blocks + n_rb - 1) / n_rb : 0;
     // elsewhere the scan of the mask extents rides in the pack launch (a masked launch has no balanced page schedule, so its layers
     // and the schedule layer never meet; if they ever did, the scan would keep a launch of its own)
-    const bool fold = m && !extra && !q_in_kernel;
+    const bool fold = m && !extra && !q_in_kernel && scan_mask;
     // (a launch issued in two forms scans per query token: 16 layers for each of the tokens a row block can hold)
     // long mask rows -- a decode batch: the row spans the whole cache; a sixteenth of it is a block's worth of 16-byte groups from
     // 32768 keys on -- get a block per (token, sixteenth), shorter ones (a prompt chunk) a wave per token
@@ -1083,7 +1084,7 @@ hipError_t launch_decode_fast(const KParams & kp_in, int kv_type, dim3 grid, hip
     else if (kv_type == MLA_TYPE_F16) hipLaunchKernelGGL(mla_q_pack_kernel<1>, dim3(n_rb, n_seq + tok_layers, KSTEPS + extra + ext), dim3(NTHREADS), 0, st, kp);
     else if (bf16_cvt)                hipLaunchKernelGGL(mla_q_pack_kernel<2>, dim3(n_rb, n_seq + tok_layers, KSTEPS + extra + ext), dim3(NTHREADS), 0, st, kp);
     else                              hipLaunchKernelGGL(mla_q_pack_kernel<0>, dim3(n_rb, n_seq + tok_layers, KSTEPS + extra + ext), dim3(NTHREADS), 0, st, kp);
-    if (m && !fold && with_prepass) hipLaunchKernelGGL(mla_mask_extent_kernel, dim3(n_rb, MASK_EXT_CHUNKS, ext_sub), dim3(NTHREADS), 0, st, kp);
+    if (m && !fold && with_prepass && scan_mask) hipLaunchKernelGGL(mla_mask_extent_kernel, dim3(n_rb, MASK_EXT_CHUNKS, ext_sub), dim3(NTHREADS), 0, st, kp);
     if (tok) {
         // the row-block form as chosen above; the token form: the k-split program up to 32 rows of 16-bit cells (it rounds Q itself), else
         // the row-split program of the cache type, whose operand image the pack launch above has written token by token

@@ -995,7 +995,8 @@ static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
         kp.rows_contig = 1; kp.q_as_q8 = 1;
         kv_type = MLA_TYPE_F16;
     }
-    if (pl.variant == 0 && kp.mask_ext && (phases & 4)) {
+    const bool scan_mask = !(a->flags & MLA_FLAG_MASK_EXTENTS_VALID);
+    if (pl.variant == 0 && kp.mask_ext && (phases & 4) && scan_mask) {
         const hipError_t e = launch_mask_extent(kp, st);
         if (e != hipSuccess) return (int) e;
     }
@@ -1019,7 +1020,7 @@ static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
             kp.v_col0 = pass * 64;
             if (phases & 1) {
                 kt.v_col0 = kp.v_col0; kt.dv_total = kp.dv_total;
-                const hipError_t e = launch_decode_fast(kp, kv_type, grid, st, (phases & 4) != 0 && pass == 0, pl.dual ? &kt : nullptr);
+                const hipError_t e = launch_decode_fast(kp, kv_type, grid, st, (phases & 4) != 0 && pass == 0, pl.dual ? &kt : nullptr, scan_mask);
                 if (e != hipSuccess) return (int) e;
             }
             // the partials of a pass are consumed before the next pass overwrites them; a combine-only call finishes the last pass

@@ -72,7 +72,7 @@ def ref():
         _ref.ref_backend_flash_attn_ext.restype = C.c_int
         _ref.ref_backend_flash_attn_ext.argtypes = [C.c_char_p, C.c_int] + [C.c_int64] * 6 + [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64,
                                                     C.c_void_p, C.c_int64, C.c_void_p, C.c_float, C.c_float, C.c_float, C.c_int,
-                                                    C.c_void_p, C.c_char_p, C.c_size_t]
+                                                    C.c_void_p, C.c_char_p, C.c_size_t, C.c_void_p, C.c_void_p]
         _ref.ref_kv_cpy.restype = C.c_int
         _ref.ref_kv_cpy.argtypes = [C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_int]
         _ref.ref_backend_kv_cpy.restype = C.c_int
@@ -216,9 +216,11 @@ def ref_flash_attn_ext(q, k, k_type, mask=None, scale=1.0, max_bias=0.0, softcap
 
 
 def ref_backend_flash_attn_ext(so_path, q, k, k_type, dv=576, mask=None, block_table=None, seq_lens=None, scale=1.0,
-                               max_bias=0.0, softcap=0.0, use_sched=False):
+                               max_bias=0.0, softcap=0.0, use_sched=False, q_second=None):
     """Run the node on a backend .so loaded by the reference's ggml_backend_load, through its ggml-backend API.
-    k: [n_seq, n_kv, row] or, with a block table, the pool [n_rows, row].  Returns (float32 [n_seq, n_tok, n_head, 576], info)."""
+    k: [n_seq, n_kv, row] or, with a block table, the pool [n_rows, row].  Returns (float32 [n_seq, n_tok, n_head, 576], info).
+    q_second: the graph gets a second attention node over the same cache and mask with these queries (as the layers of one llama
+    graph share their mask); the result is then (out, out_second, info)."""
     r = ref()
     if r is None:
         raise RuntimeError("oracle/_ref is not built")
@@ -236,14 +238,22 @@ def ref_backend_flash_attn_ext(so_path, q, k, k_type, dv=576, mask=None, block_t
         seq_lens = np.ascontiguousarray(seq_lens, dtype=np.int32)
         max_blocks = block_table.shape[1]
     out = np.full((n3, N, H, DK), np.nan, dtype=np.float32)
+    out_b = None
+    if q_second is not None:
+        q_second = np.ascontiguousarray(q_second, dtype=np.float32)
+        assert q_second.shape == q.shape
+        out_b = np.full((n3, N, H, DK), np.nan, dtype=np.float32)
     info = C.create_string_buffer(512)
     rc = r.ref_backend_flash_attn_ext(so_path.encode(), k_type, DK, dv, N, H, n3, n_kv, q.ctypes.data, k.ctypes.data,
                                       mask.ctypes.data if mask is not None else None, mask_ne0,
                                       block_table.ctypes.data if block_table is not None else None, max_blocks,
                                       seq_lens.ctypes.data if seq_lens is not None else None,
-                                      scale, max_bias, softcap, int(use_sched), out.ctypes.data, info, 512)
+                                      scale, max_bias, softcap, int(use_sched), out.ctypes.data, info, 512,
+                                      q_second.ctypes.data if q_second is not None else None, out_b.ctypes.data if out_b is not None else None)
     if rc != 0:
         raise RuntimeError("ref_backend_flash_attn_ext failed: %d (%s)" % (rc, info.value.decode()))
+    if q_second is not None:
+        return out, out_b, info.value.decode()
     return out, info.value.decode()
 
 

@@ -96,6 +96,7 @@ int ref_flash_attn_ext(int k_type, int64_t DK, int64_t n_tok, int64_t n_head, in
 struct fa_graph {
     struct ggml_context * ctx;
     struct ggml_tensor *  tq, *tm, *tb, *tl, *q_in, *fa, *o;
+    struct ggml_tensor *  tq_b, *fa_b;   /* second_node: another query tensor and another node over the same cache and mask */
     struct ggml_cgraph *  gf;
 };
 
@@ -104,7 +105,7 @@ struct fa_graph {
 static int fa_graph_build(struct fa_graph * g, struct ggml_tensor * tk_in, struct ggml_tensor ** tk_out, enum ggml_type kt,
                           int64_t DK, int64_t dv, int64_t n_tok, int64_t n_head, int64_t n3, int64_t n_kv, int paged,
                           int with_mask, int64_t mask_ne0, int64_t max_blocks, float scale, float max_bias, float softcap,
-                          int cpu_ops) {
+                          int cpu_ops, int second_node) {
     struct ggml_init_params ip = { ggml_tensor_overhead() * 32 + ggml_graph_overhead() + 4096, NULL, true };
     memset(g, 0, sizeof(*g));
     g->ctx = ggml_init(ip);
@@ -129,6 +130,17 @@ static int fa_graph_build(struct fa_graph * g, struct ggml_tensor * tk_in, struc
     ggml_set_output(g->o);
     g->gf = ggml_new_graph(ctx);
     ggml_build_forward_expand(g->gf, g->o);
+    if (second_node) {
+        /* the attention nodes of the layers of one llama graph share one mask tensor (src/llama-graph-deepseek2.cpp:99-103) */
+        g->tq_b = ggml_new_tensor_4d(ctx, GGML_TYPE_F32, DK, n_tok, n_head, n3);
+        ggml_set_input(g->tq_b);
+        g->fa_b = ggml_flash_attn_ext(ctx, g->tq_b, tk, tv, g->tm, scale, max_bias, softcap);
+        ggml_flash_attn_ext_set_prec(g->fa_b, GGML_PREC_F32);
+        g->fa_b->src[4] = g->tb;
+        g->fa_b->src[5] = g->tl;
+        ggml_set_output(g->fa_b);
+        ggml_build_forward_expand(g->gf, g->fa_b);
+    }
     if (tk_out) *tk_out = tk;
     return 0;
 }
@@ -137,7 +149,7 @@ int ref_backend_flash_attn_ext(const char * so_path, int k_type, int64_t DK, int
                                int64_t n3, int64_t n_kv, const float * q, const void * k, const uint16_t * mask,
                                int64_t mask_ne0, const int32_t * block_table, int64_t max_blocks,
                                const int32_t * seq_lens, float scale, float max_bias, float softcap, int use_sched,
-                               float * dst, char * info, size_t info_len) {
+                               float * dst, char * info, size_t info_len, const float * q_b, float * dst_b) {
     static ggml_backend_reg_t reg = NULL;
     static char               loaded_path[4096];
     if (!reg || strcmp(loaded_path, so_path) != 0) {
@@ -201,7 +213,7 @@ int ref_backend_flash_attn_ext(const char * so_path, int k_type, int64_t DK, int
     for (int run = 0; run < n_runs; run++) {
         const float run_scale = run == 1 ? 0.5f * scale : scale;
         rc = fa_graph_build(&g, tk, use_sched ? NULL : &tk, kt, DK, dv, n_tok, n_head, n3, n_kv, paged, mask != NULL, mask_ne0,
-                            max_blocks, run_scale, max_bias, softcap, use_sched == 2);
+                            max_blocks, run_scale, max_bias, softcap, use_sched == 2, q_b != NULL);
         if (rc) goto done;
         if (!ggml_backend_dev_supports_op(dev, g.fa)) { rc = -14; goto done; }
         if (use_sched) {
@@ -218,6 +230,7 @@ int ref_backend_flash_attn_ext(const char * so_path, int k_type, int64_t DK, int
             ggml_backend_tensor_set(tk, k, 0, ggml_nbytes(tk));
         }
         ggml_backend_tensor_set(g.tq, run == 1 ? q2 : q, 0, ggml_nbytes(g.tq));
+        if (g.tq_b) ggml_backend_tensor_set(g.tq_b, q_b, 0, ggml_nbytes(g.tq_b));
         if (g.tm) {
             const size_t nrow = (size_t) g.tm->ne[1];
             uint16_t *   md   = (uint16_t *) malloc(nrow * mask_ne0 * 2);
@@ -239,6 +252,7 @@ int ref_backend_flash_attn_ext(const char * so_path, int k_type, int64_t DK, int
         }
         if (st != GGML_STATUS_SUCCESS) { rc = (int) st ? (int) st : -19; goto done; }
         const size_t nb = ggml_nbytes(g.o);
+        if (g.fa_b && run == 0) ggml_backend_tensor_get(g.fa_b, dst_b, 0, ggml_nbytes(g.fa_b));
         if (run == 1) {
             /* softmax(0.5 * scale * (2Q).K) is softmax(scale * Q.K) bit for bit: doubling is exact in every rounding step */
             d2 = (float *) malloc(nb);

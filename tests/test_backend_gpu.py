@@ -113,6 +113,37 @@ def test_batched_decode_through_the_mask_as_llama_builds_it(gpu, use_sched, n_he
     print(U.check(got[..., :512], want, "masked batched decode through the reference's ggml"))
 
 
+@pytest.mark.parametrize("n_head", [128, 16])
+@pytest.mark.parametrize("rescan", [False, True])
+def test_two_attention_nodes_of_one_graph_share_the_mask(gpu, monkeypatch, n_head, rescan):
+    """The layers of one llama graph share their mask tensor: the second attention node of a graph finds the key extents of the
+    mask in the plugin's workspace, left there by the first, and leaves out the scan (GGML_HIP_MLA_MASK_EXTENTS=rescan: every
+    node scans for itself).  Two nodes over one cache and one mask with different queries, both against the oracle; then the
+    same graph with another mask -- the extents of the first graph must not survive into the second call."""
+    if rescan:
+        monkeypatch.setenv("GGML_HIP_MLA_MASK_EXTENTS", "rescan")
+    import ctypes
+    lib = ctypes.CDLL(_so())
+    lib.mla_ggml_mask_extent_reuses.restype = ctypes.c_int64
+    before = lib.mla_ggml_mask_extent_reuses()
+    rng = np.random.default_rng(61 + n_head)
+    n_kv, lens = 1536, [300, 512, 77, 400]
+    k = U.encode_kv(rng.standard_normal((1, n_kv, 576)).astype(np.float32), O.TYPE_BF16)
+    qa = rng.standard_normal((1, n_head, len(lens), 576)).astype(np.float32)
+    qb = rng.standard_normal((1, n_head, len(lens), 576)).astype(np.float32)
+    for shift in (0, 40):                       # the second graph: every sequence sits 40 cells further on
+        m = np.full((len(lens), n_kv), -np.inf, dtype=np.float32)
+        pos = shift
+        for s, l in enumerate(lens):
+            m[s, pos:pos + l] = 0.0
+            pos += l + 20
+        mask = m.astype(np.float16).view(np.uint16)
+        got_a, got_b, info = O.ref_backend_flash_attn_ext(_so(), qa, k, O.TYPE_BF16, dv=512, mask=mask, scale=U.SCALE, q_second=qb)
+        print(U.check(got_a[..., :512], O.flash_attn_ext(qa, k, O.TYPE_BF16, dv=512, mask=mask, scale=U.SCALE), "first node, shift %d" % shift))
+        print(U.check(got_b[..., :512], O.flash_attn_ext(qb, k, O.TYPE_BF16, dv=512, mask=mask, scale=U.SCALE), "second node, shift %d" % shift))
+    assert lib.mla_ggml_mask_extent_reuses() - before == (0 if rescan else 2)    # the second node of each of the two graphs
+
+
 @pytest.mark.parametrize("w_type", [O.TYPE_BF16, O.TYPE_F16])
 @pytest.mark.parametrize("n_tok", [1, 32, 150])
 def test_query_side_and_output_side_graphs_through_the_plugin(gpu, w_type, n_tok):

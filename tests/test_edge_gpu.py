@@ -569,6 +569,45 @@ def test_repeated_launches_give_identical_results(gpu, k_type):
         assert bool(torch.isfinite(ref).all())
 
 
+@pytest.mark.parametrize("k_type", [O.TYPE_BF16, O.TYPE_Q8_0])
+@pytest.mark.parametrize("n_head,n_tok", [(128, 8), (16, 32), (16, 1), (48, 5)])
+def test_mask_extents_left_by_the_launch_before(gpu, k_type, n_head, n_tok):
+    """MLA_FLAG_MASK_EXTENTS_VALID: a launch with the same mask and shapes as the one before it on the same workspace, other
+    queries and another cache, leaves out the scan of the mask and gives the result of a launch that scans (every kernel path that
+    takes a mask: column-split, both forms of a few-head launch, k-split, row-split, Q8_0; contiguous and paged)."""
+    import torch
+    import jittorinfer_amd as J
+    rng = np.random.default_rng(900 + n_head + n_tok)
+    n_kv = 2048
+    q8s = 1.0 / 32 if k_type == O.TYPE_Q8_0 else None
+    m = np.full((n_tok, n_kv), -np.inf, dtype=np.float32)
+    for t in range(n_tok):
+        lo = int(rng.integers(0, n_kv - 64)); hi = min(n_kv, lo + int(rng.integers(33, 700)))
+        m[t, lo:hi] = 0.0
+    tm = torch.from_numpy(m.astype(np.float16)).to(gpu)
+    for paged in (False, True):
+        outs = []
+        for layer in range(2):      # two "layers": other queries, another cache; the second is launched twice, with and without the flag
+            q = torch.from_numpy(rng.standard_normal((1, n_head, n_tok, 576)).astype(np.float32)).to(gpu)
+            kf = rng.standard_normal((1, n_kv, 576)).astype(np.float32)
+            if paged:
+                pool, bt, _ = U.make_paged(rng, [n_kv], k_type, q8_scale=q8s)
+                kw = dict(block_table=torch.from_numpy(bt).to(gpu), seq_lens=torch.tensor([n_kv], dtype=torch.int32, device=gpu))
+                k = torch.from_numpy(pool.view(np.int16) if pool.dtype == np.uint16 else pool).to(gpu)
+            else:
+                enc = U.encode_kv(kf, k_type, q8_scale=q8s)
+                kw = {}
+                k = torch.from_numpy(enc.view(np.int16) if enc.dtype == np.uint16 else enc).to(gpu)
+            out = torch.full((1, n_tok, n_head, 576), float("nan"), dtype=torch.float32, device=gpu)
+            J.ggml_flash_attn_ext(q, k, k_type, dv=512, scale=U.SCALE, mask=tm, out=out, **kw)
+            if layer == 1:
+                again = torch.full_like(out, float("nan"))
+                J.ggml_flash_attn_ext(q, k, k_type, dv=512, scale=U.SCALE, mask=tm, out=again, flags=J.MLA_FLAG_MASK_EXTENTS_VALID, **kw)
+                torch.cuda.synchronize()
+                assert torch.equal(again[..., :512], out[..., :512]), "paged %d: the launch that reuses the extents differs" % paged
+                assert bool(torch.isfinite(out[..., :512]).all())
+
+
 def _run_flags(gpu, q, pool, k_type, bt, lens, flags):
     import torch
     import jittorinfer_amd as J
