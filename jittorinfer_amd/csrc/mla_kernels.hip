@@ -507,6 +507,92 @@ __global__ void __launch_bounds__(256) mla_attn_combine_kernel(const KParams p) 
     *(f32x4 *) (out + 4) = f32x4{ o[4] * inv, o[5] * inv, o[6] * inv, o[7] * inv };
 }
 
+// The same merge for rows with many splits (one or two long sequences: 256 pieces of one row's output): the walk over the splits of
+// a row is a chain of load latencies when one thread makes it, so SL = 4 or 16 lanes share it -- lane `sl` of such a group takes
+// splits sl, sl + SL, ... (up to 16 of them in flight), and the group merges its (M, L, O) triples with lane shuffles at the end.
+// A wave covers 64 / SL rows x one group of 8 columns x SL split lanes.  grid = (ceil(rows * SL / 64), dv/32, n_seq), block = 256 =
+// 4 waves = 4 column groups.  One sequence of 128 heads x 131 072 keys in 256 splits: step 96.3 us with one thread per (row, column
+// group), 72.1 us with four lanes, 67.7 us with sixteen (the decode kernel alone: 47 us).
+template <int G, int SL>
+__device__ __forceinline__ void combine_wide_walk(const float2 * ml, const _Float16 * po, int64_t ml_step, int64_t po_step, int nvalid, int sl, float & M, float & L, float (&o)[8]) {
+    for (int c0 = sl; c0 < nvalid; c0 += SL * G) {
+        float2 mlv[G];
+        u32x4  hv[G];
+#pragma unroll
+        for (int k = 0; k < G; k++) {
+            const int c = min(c0 + SL * k, nvalid - 1);  // past the end: a duplicate of the last split, given weight 0 below
+            mlv[k] = ml[c * ml_step];
+            hv[k]  = *(const u32x4 *) (po + c * po_step);
+        }
+        float Mg = M;
+#pragma unroll
+        for (int k = 0; k < G; k++) if (c0 + SL * k < nvalid) Mg = fmaxf(Mg, mlv[k].x);
+        if (Mg == -INFINITY) continue;  // every split so far saw only masked keys
+        const float r = fast_exp2(M - Mg);  // 0 when M was -inf
+        M = Mg;
+        L *= r;
+#pragma unroll
+        for (int k = 0; k < 8; k++) o[k] *= r;
+#pragma unroll
+        for (int k = 0; k < G; k++) {
+            const float w = (c0 + SL * k < nvalid && mlv[k].x != -INFINITY) ? mlv[k].y * fast_exp2(mlv[k].x - M) : 0.f;
+            L += w;
+            if (w == 0.f) continue;  // its partial may hold anything (0/0 of a split without a key), never multiply it in
+            const unsigned h[4] = { hv[k].x, hv[k].y, hv[k].z, hv[k].w };
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                o[2 * e]     += f16_bits_to_f32(h[e] & 0xffff) * w;
+                o[2 * e + 1] += f16_bits_to_f32(h[e] >> 16) * w;
+            }
+        }
+    }
+}
+template <int SL>
+__global__ void __launch_bounds__(256) mla_attn_combine_wide_kernel(const KParams p) {
+    const int b = blockIdx.z, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int sl = lane % SL;
+    const int row = blockIdx.x * (64 / SL) + lane / SL;
+    const int cg  = blockIdx.y * 4 + wave;
+    const int seq_len = p.block_table ? min(p.seq_lens[b], (int) p.bt_stride * MLA_PAGE_TOKENS) : (int) p.n_kv;
+    // (rows past the end keep their lanes: the shuffles below want whole groups; they work on the last row and store nothing)
+    const int rrow = min(row, p.n_rows - 1);
+    if (cg * 8 >= p.dv_total) return;
+    int slot0, nvalid, lrow, slot_rows;
+    partial_slots(p, b, rrow, seq_len, slot0, nvalid, lrow, slot_rows);
+    if (nvalid < 0) return;   // (the same for the lanes of a group)
+
+    const float2 *   ml = (const float2 *) p.part_ml + (int64_t) slot0 * slot_rows + lrow;
+    const _Float16 * po = p.part_o + (int64_t) slot0 * slot_rows * p.dv_total + ((int64_t) cg * slot_rows + lrow) * 8;
+    const int64_t ml_step = slot_rows, po_step = (int64_t) slot_rows * p.dv_total;
+
+    float M = -INFINITY, L = 0.f;
+    float o[8] = { 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f };
+    // 16 splits per lane in flight, or 4 when the row has few (the host picks this kernel by the longest rows of the launch)
+    if (nvalid > 4 * SL) combine_wide_walk<16, SL>(ml, po, ml_step, po_step, nvalid, sl, M, L, o);
+    else                 combine_wide_walk<4, SL>(ml, po, ml_step, po_step, nvalid, sl, M, L, o);
+    // the group's triples -> one: common maximum, rescale, add
+    float Mq = M;
+#pragma unroll
+    for (int d = 1; d < SL; d <<= 1) Mq = fmaxf(Mq, __shfl_xor(Mq, d, 64));
+    const float rs = (M == -INFINITY) ? 0.f : fast_exp2(M - Mq);   // (a lane without a valid split: nothing to add; Mq = -inf too: L stays 0)
+    L *= rs;
+#pragma unroll
+    for (int k = 0; k < 8; k++) o[k] *= rs;
+#pragma unroll
+    for (int d = 1; d < SL; d <<= 1) {
+        L += __shfl_xor(L, d, 64);
+#pragma unroll
+        for (int k = 0; k < 8; k++) o[k] += __shfl_xor(o[k], d, 64);
+    }
+    if (row >= p.n_rows || sl >= 4) return;
+    const float inv = 1.0f / L;  // no valid key at all: 0 * inf = NaN, like the reference
+    float * out = p.dst + ((int64_t) b * p.n_rows + row) * p.dst_stride + p.v_col0 + cg * 8 + 2 * sl;   // lane sl stores columns 2 sl, 2 sl + 1
+    float2 v;
+    v.x = (sl == 0 ? o[0] : sl == 1 ? o[2] : sl == 2 ? o[4] : o[6]) * inv;
+    v.y = (sl == 0 ? o[1] : sl == 1 ? o[3] : sl == 2 ? o[5] : o[7]) * inv;
+    *(float2 *) out = v;
+}
+
 // The same merge over f32 partials (rows of dv_total floats; small problems).  One thread = one (row, group of 4 columns),
 // lanes along the columns of a row.  grid = (ceil(rows/2), 1, n_seq), block = 256 = 2 rows x 128 column groups (dv <= 512)
 // or (rows, 1, n_seq) with 144 active threads for dv = 576: blockDim covers one or two rows, see the launch.
@@ -1005,6 +1091,18 @@ static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
             const int groups = dv / 4, rows_per_block = 256 / groups;   // 128 -> 2 rows, 144 -> 1 row
             dim3 g((unsigned) ((kp.n_rows + rows_per_block - 1) / rows_per_block), 1, (unsigned) a->n_seq);
             hipLaunchKernelGGL(mla_attn_combine_f32_kernel, g, dim3(256), 0, st, kp, groups);
+            return (int) hipGetLastError();
+        }
+        // rows with many splits (few long sequences): four lanes share the walk over a row's splits
+        const int splits_per_row = pl.balanced ? (pl.n_wg + pl.n_units - 1) / pl.n_units : pl.n_splits;
+        if (splits_per_row > 128) {   // (sixteen lanes pay from about 200 splits on: 256 splits 72.1 -> 67.7 us per step, 128 splits 64.1 -> 67.8)
+            dim3 gw((unsigned) ((kp.n_rows + 3) / 4), (unsigned) ((dv + 31) / 32), (unsigned) a->n_seq);
+            hipLaunchKernelGGL(mla_attn_combine_wide_kernel<16>, gw, dim3(256), 0, st, kp);
+            return (int) hipGetLastError();
+        }
+        if (splits_per_row > 16) {
+            dim3 gw((unsigned) ((kp.n_rows + 15) / 16), (unsigned) ((dv + 31) / 32), (unsigned) a->n_seq);
+            hipLaunchKernelGGL(mla_attn_combine_wide_kernel<4>, gw, dim3(256), 0, st, kp);
             return (int) hipGetLastError();
         }
         dim3 g((unsigned) ((kp.n_rows + 15) / 16), (unsigned) ((dv + 127) / 128), (unsigned) a->n_seq);

@@ -608,6 +608,41 @@ def test_mask_extents_left_by_the_launch_before(gpu, k_type, n_head, n_tok):
                 assert bool(torch.isfinite(out[..., :512]).all())
 
 
+@pytest.mark.parametrize("form", ["paged", "masked"])
+def test_one_long_sequence_in_256_splits(gpu, form):
+    """One or two long sequences of 128 heads: the planner deals the keys out to 256 workgroups, every output row has up to 256 f16
+    partials, and the combine pass for such rows lets four lanes share the walk over a row's splits.  Paged (33 000 and 20 000 keys:
+    a balanced page schedule across both) and masked over one cache (two query tokens with windows of their own, one of them with a
+    hole)."""
+    import torch
+    import jittorinfer_amd as J
+    rng = np.random.default_rng(77)
+    if form == "paged":
+        lens = [33000, 20000]
+        pool, bt, seqs = U.make_paged(rng, lens, O.TYPE_BF16)
+        q = rng.standard_normal((2, 128, 1, 576)).astype(np.float32)
+        tq, tk = torch.from_numpy(q).to(gpu), torch.from_numpy(pool.view(np.int16)).to(gpu)
+        info = J.plan(tq, tk, O.TYPE_BF16, dv=512, scale=U.SCALE, block_table=torch.from_numpy(bt).to(gpu), seq_lens=torch.tensor(lens, dtype=torch.int32, device=gpu))
+        assert info["variant"] == 2 and info["balanced"] == 1 and info["n_workgroups"] == 256
+        got = _run(gpu, q, pool, O.TYPE_BF16, bt=bt, lens=lens, scale=U.SCALE)
+        want = U.oracle_per_seq(q, seqs, O.TYPE_BF16, 512)
+    else:
+        n_kv = 40960
+        k = U.encode_kv(rng.standard_normal((1, n_kv, 576)).astype(np.float32), O.TYPE_BF16)
+        q = rng.standard_normal((1, 128, 2, 576)).astype(np.float32)
+        m = np.full((2, n_kv), -np.inf, dtype=np.float32)
+        m[0, 100:36000] = 0.0
+        m[0, 5000:9000] = -np.inf
+        m[1, 20000:40900] = 0.0
+        mask = m.astype(np.float16).view(np.uint16)
+        tq, tk = torch.from_numpy(q).to(gpu), torch.from_numpy(k.view(np.int16)).to(gpu)
+        info = J.plan(tq, tk, O.TYPE_BF16, dv=512, scale=U.SCALE, mask=torch.from_numpy(mask.view(np.float16)).to(gpu))
+        assert info["variant"] == 2 and info["balanced"] == 2 and info["n_row_blocks"] == 2
+        got = _run(gpu, q, k, O.TYPE_BF16, mask=mask, scale=U.SCALE)
+        want = O.flash_attn_ext(q, k, O.TYPE_BF16, dv=512, mask=mask, scale=U.SCALE)
+    print(U.check(got[..., :512], want, "many splits per row, " + form))
+
+
 def _run_flags(gpu, q, pool, k_type, bt, lens, flags):
     import torch
     import jittorinfer_amd as J
