@@ -651,6 +651,67 @@ __global__ void __launch_bounds__(256) mla_attn_combine_f32_kernel(const KParams
     else                   combine_f32_row<32>(ml, po, ml_step, po_step, nvalid, dst);
 }
 
+// f32 partials, rows with more than 32 splits (a single sequence of a decode step: 64 one-page splits at 8192 keys, 256 pieces at
+// 131 072): the four waves of a block share the walk over the splits of one row -- wave w takes splits w, w + 4, ..., 16 in flight,
+// for 64 groups of 4 columns -- and meet in LDS.  grid = (rows, ceil(dv / 256), n_seq), block = 256.
+__global__ void __launch_bounds__(256) mla_attn_combine_f32_wide_kernel(const KParams p) {
+    __shared__ float red[4][6][64];
+    constexpr int G = 16;
+    const int b = blockIdx.z, row = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int cg = min((int) blockIdx.y * 64 + lane, p.dv_total / 4 - 1);   // (lanes past the row's end repeat its last group and store nothing)
+    const int seq_len = p.block_table ? min(p.seq_lens[b], (int) p.bt_stride * MLA_PAGE_TOKENS) : (int) p.n_kv;
+    int slot0, nvalid, lrow, slot_rows;
+    partial_slots(p, b, row, seq_len, slot0, nvalid, lrow, slot_rows);
+    if (nvalid < 0) return;   // (uniform over the block: one row)
+    const float2 * ml = (const float2 *) p.part_ml + (int64_t) slot0 * slot_rows + lrow;
+    const float *  po = (const float *) p.part_o + ((int64_t) slot0 * slot_rows + lrow) * p.dv_total + cg * 4;
+    const int64_t ml_step = slot_rows, po_step = (int64_t) slot_rows * p.dv_total;
+    float M = -INFINITY, L = 0.f;
+    f32x4 o = { 0.f, 0.f, 0.f, 0.f };
+    for (int c0 = wave; c0 < nvalid; c0 += 4 * G) {
+        float2 mlv[G];
+        f32x4  xv[G];
+#pragma unroll
+        for (int k = 0; k < G; k++) {
+            const int c = min(c0 + 4 * k, nvalid - 1);
+            mlv[k] = ml[c * ml_step];
+            xv[k]  = *(const f32x4 *) (po + c * po_step);
+        }
+        float Mg = M;
+#pragma unroll
+        for (int k = 0; k < G; k++) if (c0 + 4 * k < nvalid) Mg = fmaxf(Mg, mlv[k].x);
+        if (Mg == -INFINITY) continue;  // every split so far saw only masked keys
+        const float r = fast_exp2(M - Mg);  // 0 when M was -inf
+        M = Mg;
+        L *= r;
+        o.x *= r; o.y *= r; o.z *= r; o.w *= r;
+#pragma unroll
+        for (int k = 0; k < G; k++) {
+            const float w = (c0 + 4 * k < nvalid && mlv[k].x != -INFINITY) ? mlv[k].y * fast_exp2(mlv[k].x - M) : 0.f;
+            L += w;
+            if (w == 0.f) continue;  // that split saw only masked keys (or is padding): its partial may hold anything
+            o.x += xv[k].x * w; o.y += xv[k].y * w; o.z += xv[k].z * w; o.w += xv[k].w * w;
+        }
+    }
+    red[wave][0][lane] = M; red[wave][1][lane] = L;
+    red[wave][2][lane] = o.x; red[wave][3][lane] = o.y; red[wave][4][lane] = o.z; red[wave][5][lane] = o.w;
+    __syncthreads();
+    if (wave != 0 || (int) blockIdx.y * 64 + lane >= p.dv_total / 4) return;
+    float Mq = fmaxf(fmaxf(red[0][0][lane], red[1][0][lane]), fmaxf(red[2][0][lane], red[3][0][lane]));
+    float Lq = 0.f;
+    f32x4 oq = { 0.f, 0.f, 0.f, 0.f };
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+        const float mw = red[w][0][lane];
+        const float rs = mw == -INFINITY ? 0.f : fast_exp2(mw - Mq);   // (a wave without a valid split adds nothing)
+        Lq += red[w][1][lane] * rs;
+        oq.x += red[w][2][lane] * rs; oq.y += red[w][3][lane] * rs; oq.z += red[w][4][lane] * rs; oq.w += red[w][5][lane] * rs;
+    }
+    const float inv = 1.0f / Lq;  // no valid key at all: 0 * inf = NaN, like the reference
+    float * dst = p.dst + ((int64_t) b * p.n_rows + row) * p.dst_stride + p.v_col0 + cg * 4;
+    *(f32x4 *) dst = f32x4{ oq.x * inv, oq.y * inv, oq.z * inv, oq.w * inv };
+}
+
 // ---------------------------------------------------------------------------------------------------------------
 // Strict replay of ggml-cpu's f16 accumulator for F16 KV (ggml-cpu.c:12066-12080 with the x86 F16 vector forms
 // :621-659, :718-765: f32 FMA, result rounded to f16 after every scale and every multiply-add, keys in order).
@@ -1087,6 +1148,12 @@ static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
         if (e != hipSuccess) return (int) e;
     }
     auto combine = [&](int dv) -> int {
+        const int splits_per_row = pl.balanced ? (pl.n_wg + pl.n_units - 1) / pl.n_units : pl.n_splits;
+        if (pl.part_f32 && splits_per_row > 32) {   // (one or two sequences: the waves of a block share the walk over a row's splits)
+            dim3 gw((unsigned) kp.n_rows, (unsigned) ((dv / 4 + 63) / 64), (unsigned) a->n_seq);
+            hipLaunchKernelGGL(mla_attn_combine_f32_wide_kernel, gw, dim3(256), 0, st, kp);
+            return (int) hipGetLastError();
+        }
         if (pl.part_f32) {
             const int groups = dv / 4, rows_per_block = 256 / groups;   // 128 -> 2 rows, 144 -> 1 row
             dim3 g((unsigned) ((kp.n_rows + rows_per_block - 1) / rows_per_block), 1, (unsigned) a->n_seq);
@@ -1094,7 +1161,6 @@ static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
             return (int) hipGetLastError();
         }
         // rows with many splits (few long sequences): four lanes share the walk over a row's splits
-        const int splits_per_row = pl.balanced ? (pl.n_wg + pl.n_units - 1) / pl.n_units : pl.n_splits;
         if (splits_per_row > 128) {   // (sixteen lanes pay from about 200 splits on: 256 splits 72.1 -> 67.7 us per step, 128 splits 64.1 -> 67.8)
             dim3 gw((unsigned) ((kp.n_rows + 3) / 4), (unsigned) ((dv + 31) / 32), (unsigned) a->n_seq);
             hipLaunchKernelGGL(mla_attn_combine_wide_kernel<16>, gw, dim3(256), 0, st, kp);

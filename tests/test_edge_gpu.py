@@ -608,16 +608,32 @@ def test_mask_extents_left_by_the_launch_before(gpu, k_type, n_head, n_tok):
                 assert bool(torch.isfinite(out[..., :512]).all())
 
 
-@pytest.mark.parametrize("form", ["paged", "masked"])
+@pytest.mark.parametrize("form", ["paged", "masked", "few heads", "contiguous"])
 def test_one_long_sequence_in_256_splits(gpu, form):
     """One or two long sequences of 128 heads: the planner deals the keys out to 256 workgroups, every output row has up to 256 f16
     partials, and the combine pass for such rows lets four lanes share the walk over a row's splits.  Paged (33 000 and 20 000 keys:
     a balanced page schedule across both) and masked over one cache (two query tokens with windows of their own, one of them with a
-    hole)."""
+    hole).  With f32 partials (16 heads over 33 000 paged keys: 256 pieces; 128 heads over 8192 contiguous keys: 64 one-page splits;
+    V := K in its two passes) the four waves of a block share the walk."""
     import torch
     import jittorinfer_amd as J
     rng = np.random.default_rng(77)
-    if form == "paged":
+    if form == "few heads":
+        lens = [33000]
+        pool, bt, seqs = U.make_paged(rng, lens, O.TYPE_F16)
+        q = rng.standard_normal((1, 16, 1, 576)).astype(np.float32)
+        got = _run(gpu, q, pool, O.TYPE_F16, bt=bt, lens=lens, scale=U.SCALE)
+        want = np.stack([O.flash_attn_ext_f64(q[b:b + 1], k[None], O.TYPE_F16, dv=512, scale=U.SCALE)[0] for b, k in enumerate(seqs)])
+    elif form == "contiguous":
+        k = U.encode_kv(rng.standard_normal((1, 8192, 576)).astype(np.float32), O.TYPE_BF16)
+        q = rng.standard_normal((1, 128, 1, 576)).astype(np.float32)
+        tq, tk = torch.from_numpy(q).to(gpu), torch.from_numpy(k.view(np.int16)).to(gpu)
+        assert J.plan(tq, tk, O.TYPE_BF16, dv=576, scale=U.SCALE)["n_splits"] == 64
+        got = _run(gpu, q, k, O.TYPE_BF16, dv=576, scale=U.SCALE)
+        want = O.flash_attn_ext(q, k, O.TYPE_BF16, dv=576, scale=U.SCALE)
+        print(U.check(got, want, "many splits per row, V := K"))
+        return
+    elif form == "paged":
         lens = [33000, 20000]
         pool, bt, seqs = U.make_paged(rng, lens, O.TYPE_BF16)
         q = rng.standard_normal((2, 128, 1, 576)).astype(np.float32)
