@@ -945,14 +945,16 @@ int make_plan(const mla_attn_args * a, Plan * pl) {
     const int64_t pages_per_split = (n_pages + splits - 1) / splits;
     pl->split_tokens = (int) (pages_per_split * MLA_PAGE_TOKENS);
     pl->n_splits     = (int) ((n_pages + pages_per_split - 1) / pages_per_split);
-    // A launch that leaves most CUs without a workgroup even with one page per split and whose partials stay tiny (one short
-    // sequence of a few heads: BASELINE's configs[0]) is split by 32-key tiles instead: the wave programs start a split at any tile
-    // (a page holds four), and what a workgroup of such a launch spends per tile it saves in full (14.4 -> 13.0 us there).  Not
-    // beyond 1 MB of f32 partials: from there on the combine pass loses more than the kernel gains (16 heads x 4096 keys in 128
-    // splits: 17.1 -> 23.4 us).
+    // A launch that leaves most CUs without a workgroup even with one page per split and whose partials stay small (one or two short
+    // sequences of a few heads: BASELINE's configs[0]) is split by 32-key tiles instead: the wave programs start a split at any tile
+    // (a page holds four), and what a workgroup of such a launch spends per tile it saves in full (configs[0] 14.4 -> 13.0 us; one
+    // sequence of 16 heads x 4096 keys 17.2 -> 14.9 us, two 19.1 -> 16.2 us).  Up to 4 MB of f32 partials for at most 32 rows, 1 MB
+    // beyond (128 rows: a partial is 64 KB of f32, twice a tile of KV; every finer split measured slower there): past that the
+    // combine pass loses more than the kernel gains (16 heads x 8192 keys in 256 splits: 17.5 -> 21.3 us).
     if (pl->variant == 2 && a->n_splits == 0 && pages_per_split == 1 && !a->mask && a->kv_type != MLA_TYPE_Q8_0) {
         const int64_t n_tiles = (max_len + TILE_TOK - 1) / TILE_TOK, wgs = (int64_t) a->n_seq * pl->n_row_blocks;
-        const int64_t want = std::min<int64_t>({ n_tiles, 256 / wgs, ((int64_t) 1 << 20) / ((int64_t) a->n_seq * n_rows * 512 * 4) });
+        const int64_t lim = (int64_t) (n_rows <= 32 ? 4 : 1) << 20;
+        const int64_t want = std::min<int64_t>({ n_tiles, 256 / wgs, lim / ((int64_t) a->n_seq * n_rows * 512 * 4) });
         if (want > pl->n_splits) {
             const int64_t tiles_per_split = (n_tiles + want - 1) / want;
             pl->split_tokens = (int) (tiles_per_split * TILE_TOK);

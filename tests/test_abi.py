@@ -154,8 +154,10 @@ def test_planner_schedules_without_gpu():
     one = dict(n_seq=1, n_head=16, block_table=0, seq_lens=0, bt_stride=0, kv_nb3=0, kv_type=J.MLA_TYPE_F16)
     rc, info, _ = _plan(n_kv=1024, **one)                        # configs[0]: one short sequence, splits of one 32-key tile
     assert rc == 0 and info.variant == 2 and info.n_splits == 32 and info.split_tokens == 32
-    rc, info, _ = _plan(n_kv=4096, **one)                        # more tiles than 1 MB of partials allows splits: whole pages again
-    assert rc == 0 and info.n_splits == 32 and info.split_tokens == 128
+    rc, info, _ = _plan(n_kv=4096, **one)                        # 128 tiles: 4 MB of f32 partials, the most a few-head launch gets
+    assert rc == 0 and info.n_splits == 128 and info.split_tokens == 32
+    rc, info, _ = _plan(n_kv=16384, **one)                       # more tiles than that allows splits: whole pages again
+    assert rc == 0 and info.n_splits == 128 and info.split_tokens == 128
     rc, info, _ = _plan(n_kv=1024, **{**one, "n_head": 128})
     assert rc == 0 and info.n_splits == 8 and info.split_tokens == 128
     # the reference's decode batch: one cache, one query token per sequence, the mask picks every token's cells
