@@ -77,7 +77,7 @@ N_VGPR = 253 if BIAS else 252
 # ---- SGPR map (all inside the clobbered range s40..s99)
 KV, BT, KVB, KVE, CL2, NPP, NB1, FLG = 40, 42, 44, 45, 46, 47, 48, 49
 NT, IT, OFF0, OFF1, OFF2, OFF3, WAVE, TMP = 50, 51, 52, 53, 54, 55, 56, 57
-TB, NVM1, VMW, EXS = 58, 60, 61, 62
+TB, PMASK, VMW, EXS = 58, 60, 61, 62         # PMASK: 127 with a block table (token inside its page), all ones without
 S0, S1, S2, S3, DMAB, NVAL, THR, PG0 = 64, 65, 66, 67, 68, 69, 70, 71
 RSC, ONES, OSTR, QP, OB, MLB, RSTR, NRV = 72, 74, 75, 76, 78, 80, 82, 83
 W4, WOFS, FADR, PGZ, SPITCH, SCLS = 84, 85, 86, 87, 88, 89
@@ -187,8 +187,9 @@ def run_slots(slots, first_index, streams, events=None):
 # ---------------------------------------------------------------------------------------------------------------
 def tile_base_lines(tile_sreg, first_page_scalar=False):
     """Scalar lines: s[TB:TB+1] = address of the first row of tile s[tile_sreg], less DMA_BIAS (s[KV] is kept that much low).
-    The page id comes from the lane of PAGES that holds the tile's page (for a cache without a table PAGES holds the
-    logical pages themselves).  first_page_scalar: a tile inside the split's first page takes the id from s[PGZ] (the
+    The page id comes from the lane of PAGES that holds the tile's page -- at most 64 pages per split, the launcher sees to that.
+    A cache without a table has no such limit: its PAGES and s[PGZ] are 0 and s[PMASK] keeps all bits of the token, so the row is
+    the token itself whatever lane the (wrapping) index picks.  first_page_scalar: a tile inside the split's first page takes the id from s[PGZ] (the
     prologue's tiles, issued while the vector load of the page ids may still be in flight)."""
     L = []
     L.append("s_lshl_b32 %s, %s, 5" % (s(S0), s(tile_sreg)))
@@ -200,7 +201,7 @@ def tile_base_lines(tile_sreg, first_page_scalar=False):
         L.append("s_cmp_eq_u32 %s, 0" % s(S1))
         L.append("s_cselect_b32 %s, %s, %s" % (s(S2), s(PGZ), s(S2)))
     L.append("s_lshl_b32 %s, %s, 7" % (s(S2), s(S2)))
-    L.append("s_and_b32 %s, %s, 127" % (s(S3), s(S0)))
+    L.append("s_and_b32 %s, %s, %s" % (s(S3), s(S0), s(PMASK)))                 # token inside the page; the whole token without a table
     L.append("s_add_u32 %s, %s, %s" % (s(S2), s(S2), s(S3)))                      # row in the pool / in the cache
     L.append("s_mul_hi_u32 %s, %s, %s" % (s(S1), s(S2), s(NB1)))
     L.append("s_mul_i32 %s, %s, %s" % (s(S0), s(S2), s(NB1)))
@@ -781,14 +782,16 @@ def prologue_head(early=None):
     e("v_lshlrev_b32 %s, 4, %s" % (v(PADDR), v(LANE)))
     e("v_add_u32 %s, 0x%x, %s" % (v(PADDR), PBUF, v(PADDR)))
     # ------------------------------------------------------------------ page ids of this split -> one lane each.  A cache without
-    # a table: the logical pages themselves (and no clamp against a pool size)
+    # a table: page 0 everywhere and the whole token as the offset inside it (and no clamp against a pool size)
     lab_nobt = label("nobt")
     e("s_lshr_b32 %s, %s, 7" % (s(PG0), s(KVB)))
-    e("v_add_u32 %s, %s, %s" % (v(PAGES), s(PG0), v(LANE)))
+    e("v_mov_b32 %s, 0" % v(PAGES))
     e("s_cmp_eq_u64 %s, 0" % s(BT, 2))
     e("s_cselect_b32 %s, 0x7fffffff, %s" % (s(NPP), s(NPP)))
-    e("s_cselect_b32 %s, %s, %s" % (s(PGZ), s(PG0), s(PGZ)))
+    e("s_cselect_b32 %s, 0, %s" % (s(PGZ), s(PGZ)))
+    e("s_cselect_b32 %s, -1, 127" % s(PMASK))
     e("s_cbranch_scc1 %s" % lab_nobt)
+    e("v_add_u32 %s, %s, %s" % (v(PAGES), s(PG0), v(LANE)))
     e("s_add_u32 %s, %s, 127" % (s(S0), s(KVE)))
     e("s_lshr_b32 %s, %s, 7" % (s(S0), s(S0)))
     e("s_sub_u32 %s, %s, %s" % (s(S0), s(S0), s(PG0)))                   # pages in this split (<= 64)

@@ -303,6 +303,11 @@ __device__ __forceinline__ void decode_body() {
             const unsigned id = (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
             const unsigned v  = (id & 7) * (G >> 3) + (id >> 3);
             bx = v % gridDim.x; by = (v / gridDim.x) % gridDim.y; bz = v / (gridDim.x * gridDim.y);
+            // A masked launch with one split per row block -- a prompt chunk, whose row blocks see more keys the later their tokens
+            // come -- would give the first XCD the shortest row blocks of a sequence and the last the longest (512 tokens x 128 heads
+            // from an empty cache: 2 against 16 tiles).  The row blocks are therefore taken in folded order 0, R-1, 1, R-2, ...: any run
+            // of an even number of them has the same number of keys as any other, and the blocks of one sequence still share an XCD.
+            if (MASK && gridDim.x == 1 && !p.balanced) by = (by & 1) ? (int) gridDim.y - 1 - (by >> 1) : (by >> 1);
         }
     }
 
@@ -809,6 +814,48 @@ __device__ __forceinline__ void mask_extent_block(const KParams & p, int rb, int
 // grid = (n_row_blocks, 16), or for a launch issued in two forms (n_row_blocks, 16, tokens per row block)
 __global__ void __launch_bounds__(NTHREADS) mla_mask_extent_kernel(const KParams p) { mask_extent_block(p, blockIdx.x, blockIdx.y, blockIdx.z); }
 
+// The same scan with a wave per (row block, sixteenth), four to a block, for launches of many row blocks whose sixteenths are short
+// (a prompt chunk of 512 tokens x 128 heads: 8192 pairs of 4 groups each, for which a block of 256 threads and its barriers are
+// all overhead: 20.9 -> 3 us).  grid = ceil(n_row_blocks * 16 / 4), block = 256.
+__global__ void __launch_bounds__(NTHREADS) mla_mask_extent_wave_kernel(const KParams p, int n_rb) {
+    const int lane = threadIdx.x & 63, pair = (int) blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (pair >= n_rb * MASK_EXT_CHUNKS) return;
+    const int rb = pair / MASK_EXT_CHUNKS, chunk = pair - rb * MASK_EXT_CHUNKS;
+    const int r0 = rb * 128, r1 = min(r0 + 127, p.n_rows - 1);
+    const int t0 = r0 / p.n_head, n_t = r1 / p.n_head - t0 + 1;
+    const int n_kv = (int) (p.block_table ? p.bt_stride * MLA_PAGE_TOKENS : p.n_kv);
+    const int n8 = n_kv / 8;
+    const int g0 = (int) ((int64_t) n8 * chunk / MASK_EXT_CHUNKS), ng = (int) ((int64_t) n8 * (chunk + 1) / MASK_EXT_CHUNKS) - g0;
+    const int64_t total = (int64_t) n_t * ng;
+    int hi = 0, lo = n_kv;
+    constexpr int U = 4;
+    for (int64_t base = lane; base < total; base += U * 64) {
+        u32x4 w[U];
+        int   g[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int64_t idx = min(base + u * 64, total - 1);   // past the end: the last pair again
+            const int t = (int) (idx / ng);
+            g[u] = g0 + (int) (idx - (int64_t) t * ng);
+            const char * a = p.mask + (int64_t) (t0 + t) * p.mask_nb1 + 16 * (int64_t) g[u];   // rows are 8-byte aligned
+            const u32x2 x = *(const u32x2 *) a, y = *(const u32x2 *) (a + 8);
+            w[u] = u32x4{ x.x, x.y, y.x, y.y };
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const unsigned v[4] = { w[u].x, w[u].y, w[u].z, w[u].w };
+#pragma unroll
+            for (int e = 0; e < 8; e++)
+                if (((v[e >> 1] >> (16 * (e & 1))) & 0xffff) != 0xfc00u) { lo = min(lo, 8 * g[u] + e); hi = max(hi, 8 * g[u] + e + 1); }
+        }
+    }
+    for (int d = 32; d > 0; d >>= 1) { lo = min(lo, __shfl_xor(lo, d, 64)); hi = max(hi, __shfl_xor(hi, d, 64)); }
+    if (lane == 0) {
+        p.mask_ext[pair * 2]     = lo;
+        p.mask_ext[pair * 2 + 1] = hi;
+    }
+}
+
 // The pipelined kernel's launches fold the extent scan into the Q pre-pack launch: MASK_EXT_CHUNKS more layers of blocks behind
 // the pack layers (one launch and one dispatch hand-over less ahead of the decode kernel).  True when this block was one of them.
 __device__ __forceinline__ bool pack_launch_extent_layer(const KParams & p) {
@@ -1084,7 +1131,15 @@ hipError_t launch_decode_fast(const KParams & kp_in, int kv_type, dim3 grid, hip
     else if (kv_type == MLA_TYPE_F16) hipLaunchKernelGGL(mla_q_pack_kernel<1>, dim3(n_rb, n_seq + tok_layers, KSTEPS + extra + ext), dim3(NTHREADS), 0, st, kp);
     else if (bf16_cvt)                hipLaunchKernelGGL(mla_q_pack_kernel<2>, dim3(n_rb, n_seq + tok_layers, KSTEPS + extra + ext), dim3(NTHREADS), 0, st, kp);
     else                              hipLaunchKernelGGL(mla_q_pack_kernel<0>, dim3(n_rb, n_seq + tok_layers, KSTEPS + extra + ext), dim3(NTHREADS), 0, st, kp);
-    if (m && !fold && with_prepass && scan_mask) hipLaunchKernelGGL(mla_mask_extent_kernel, dim3(n_rb, MASK_EXT_CHUNKS, ext_sub), dim3(NTHREADS), 0, st, kp);
+    if (m && !fold && with_prepass && scan_mask) {
+        // many row blocks with little to scan per (row block, sixteenth): a wave per pair instead of a block
+        const int64_t n_kv_m = kp.block_table ? kp.bt_stride * MLA_PAGE_TOKENS : kp.n_kv;
+        const int64_t per_pair = (int64_t) (127 / kp.n_head + 2) * (n_kv_m / 8 / MASK_EXT_CHUNKS + 1);
+        if (!kp.dual && n_rb * MASK_EXT_CHUNKS >= 1024 && per_pair <= 1024)
+            hipLaunchKernelGGL(mla_mask_extent_wave_kernel, dim3((n_rb * MASK_EXT_CHUNKS + 3) / 4), dim3(NTHREADS), 0, st, kp, (int) n_rb);
+        else
+            hipLaunchKernelGGL(mla_mask_extent_kernel, dim3(n_rb, MASK_EXT_CHUNKS, ext_sub), dim3(NTHREADS), 0, st, kp);
+    }
     if (tok) {
         // the row-block form as chosen above; the token form: the k-split program up to 32 rows of 16-bit cells (it rounds Q itself), else
         // the row-split program of the cache type, whose operand image the pack launch above has written token by token
