@@ -39,7 +39,8 @@ extern "C" {
                                       instead of accumulating in f32; sequential over keys, a correctness mode */
 #define MLA_FLAG_UNIFORM_SPLITS 2u /* paged decode: give every sequence the same number of equal KV splits (sized for the longest
                                       sequence the block table can hold) instead of the balanced schedule that deals equal
-                                      runs of the batch's whole page list to the workgroups; for comparing the two */
+                                      runs of the batch's whole page list to the workgroups, and the sequences of a batch of
+                                      more than 256 in batch order instead of longest first; for comparing the two */
 #define MLA_FLAG_MASK_EXTENTS_VALID 8u /* masked launch: the workspace still holds the key extents of this mask, left there by the
                                       launch before it, which had the same arguments except q, kv and dst (the attention nodes of
                                       the layers of one graph share their mask, src/llama-graph-deepseek2.cpp:99-103): the scan of

@@ -90,6 +90,8 @@ struct KParams {
                                    //   (balanced == 3: every query token a sequence of one token, its mask row that sequence's mask)
                                    //   mask_ext then holds 16 pairs per query token in both
     int *           form;          //   the form that ran (2 / 3), left by the kernel for the combine pass (workspace)
+    const int *     seq_order;     // a paged decode batch of more than 256 sequences, a workgroup each: the sequences by falling length (workspace,
+                                   //   written by the pre-pass; workgroups are dispatched in that order); nullptr: the order of the batch
     void *          tok_q_pack;    //   row-block form's parameters, pack launch: the token form's operand image, [token][wave][k-step][lane][16 B]
                                    //   (nullptr: its program rounds Q itself), and the rounding it wants (1: f16, 2: bf16 written as f16)
     int             tok_mode;

@@ -311,6 +311,11 @@ __device__ __forceinline__ void decode_body() {
         }
     }
 
+    // A paged decode batch of more than 256 sequences with a workgroup each (grid = (1, 1, sequences)) runs in rounds, in dispatch
+    // order: the sequences are taken longest first, so that the workgroups that start last are the short ones (512 ragged sequences
+    // of 128 heads: 851 -> 7xx us).  Consecutive dispatch indices go to different XCDs, which spreads every length over all of them.
+    if (!MASK && p.seq_order) bz = p.seq_order[blockIdx.z];
+
     // Balanced schedule (p.balanced; a ragged decode batch): the pages of all sequences form one list, every workgroup
     // takes an equal run of it (grid = (n_wg, 1, 1), bx = its place), and a run that crosses a sequence boundary is worked
     // off piece by piece.  Piece of workgroup v in sequence b -> partial slot v + b: the slots of one sequence are
@@ -811,6 +816,20 @@ __device__ __forceinline__ void mask_extent_block(const KParams & p, int rb, int
         p.mask_ext[(slot * MASK_EXT_CHUNKS + chunk) * 2 + 1] = red_hi[0];
     }
 }
+// order[r] = the sequence with the r-th largest length (ties in batch order).  n <= 4096; grid = ceil(n / 256), block = 256.
+constexpr int SEQ_ORDER_MAX = 4096;
+__global__ void __launch_bounds__(NTHREADS) mla_seq_order_kernel(const int32_t * lens, int n, int * order) {
+    __shared__ int L[SEQ_ORDER_MAX];
+    for (int j = threadIdx.x; j < n; j += NTHREADS) L[j] = lens[j];
+    __syncthreads();
+    const int i = blockIdx.x * NTHREADS + threadIdx.x;
+    if (i >= n) return;
+    const int li = L[i];
+    int rank = 0;
+    for (int j = 0; j < n; j++) rank += (L[j] > li) || (L[j] == li && j < i);
+    order[rank] = i;
+}
+
 // grid = (n_row_blocks, 16), or for a launch issued in two forms (n_row_blocks, 16, tokens per row block)
 __global__ void __launch_bounds__(NTHREADS) mla_mask_extent_kernel(const KParams p) { mask_extent_block(p, blockIdx.x, blockIdx.y, blockIdx.z); }
 
@@ -1125,6 +1144,10 @@ hipError_t launch_decode_fast(const KParams & kp_in, int kv_type, dim3 grid, hip
     kp.mask_ext_in_pack = fold ? 1 : 0;
     kp.mask_ext_sub = ext_sub;
     const unsigned ext = fold ? MASK_EXT_CHUNKS * ext_sub : 0;
+    if (with_prepass && kp.seq_order) {
+        if (n_seq > (unsigned) SEQ_ORDER_MAX || grid.x != 1 || grid.y != 1 || grid.z != n_seq) return hipErrorInvalidValue;
+        hipLaunchKernelGGL(mla_seq_order_kernel, dim3((n_seq + NTHREADS - 1) / NTHREADS), dim3(NTHREADS), 0, st, kp.seq_lens, (int) n_seq, (int *) kp.seq_order);
+    }
     if (!with_prepass) { /* the workspace still holds the Q image and the mask extents of an earlier launch of the same call */ }
     else if (q_in_kernel) { /* nothing: a balanced page schedule is worked out by the workgroups themselves */ }
     else if (kv_type == MLA_TYPE_Q8_0 || kp.q_as_q8) hipLaunchKernelGGL(mla_q_pack_q8_kernel, dim3(n_rb, n_seq + tok_layers, KSTEPS / 2 + extra + ext), dim3(NTHREADS), 0, st, kp);

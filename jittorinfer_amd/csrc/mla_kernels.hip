@@ -847,6 +847,7 @@ struct Plan {
     int    part_f32;
     int    balanced, n_wg, n_units;   // balanced schedule of the pipelined kernel (1: ragged paged decode, 2: masked launch)
     int    dual;                      // the masked launch is issued in two forms, see token_form_candidate
+    int    seq_sorted;                // paged decode of more than 256 sequences: workgroups take the sequences longest first
 };
 
 int validate(const mla_attn_args * a) {
@@ -991,6 +992,13 @@ int make_plan(const mla_attn_args * a, Plan * pl) {
             pl->ws_sched = (size_t) ((pl->n_units + 1 + 63) / 64 * 64 + pl->n_wg * 8) * sizeof(int);
         }
     }
+    // A paged decode batch of more than 256 sequences with a workgroup each runs in rounds: its sequences are taken longest first
+    // (an order the pre-pass writes; ws_sched holds it)
+    if (pl->variant == 2 && !pl->balanced && pl->n_splits == 1 && pl->n_row_blocks == 1 && a->block_table && !a->mask &&
+        a->n_seq > 256 && a->n_seq <= 4096 && !(a->flags & MLA_FLAG_UNIFORM_SPLITS)) {
+        pl->seq_sorted = 1;
+        pl->ws_sched = (size_t) a->n_seq * sizeof(int);
+    }
     if (token_form_candidate(a, *pl)) {
         pl->dual = 1;
         pl->ws_maskext = (size_t) a->n_tok * 16 * 2 * sizeof(int);   // 16 pairs per query token
@@ -1105,6 +1113,7 @@ static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
     kp.mask_ext = pl.ws_maskext ? (int *) (ws + align256(pl.ws_part_o) + align256(pl.ws_part_ml) + align256(pl.ws_scores) + align256(pl.ws_qpack)) : nullptr;
     kp.sched = (int *) (ws + align256(pl.ws_part_o) + align256(pl.ws_part_ml) + align256(pl.ws_scores) + align256(pl.ws_qpack) + align256(pl.ws_maskext));
     kp.wg_first = kp.sched + (std::max(pl.n_units, pl.dual ? a->n_tok : 0) + 1 + 63) / 64 * 64;
+    kp.seq_order = pl.seq_sorted ? kp.sched : nullptr;
     // the token form of a launch issued in two forms (see token_form_candidate): every query token a sequence of one token
     KParams kt = kp;
     if (pl.dual) {

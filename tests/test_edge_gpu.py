@@ -860,3 +860,27 @@ def test_prompt_chunk_behind_a_long_cache_without_a_table(gpu):
             worst = max(worst, float(np.abs(out[0, t, h, :512].cpu().numpy() - want).max()))
         print("tokens %d past %d: worst sampled difference %.2e" % (n_tok, past, worst))
         assert worst < U.MAX_ABS_TOL, (n_tok, past, worst)
+
+
+def test_paged_decode_of_more_than_256_sequences_longest_first(gpu):
+    """A paged decode batch of more than 256 sequences of 128 heads is a workgroup per sequence, in rounds; the workgroups take the
+    sequences by falling length (an order the pre-pass writes into the workspace).  300 ragged sequences, some empty, some equal:
+    against the oracle, and bit for bit against the same launch in batch order (MLA_FLAG_UNIFORM_SPLITS)."""
+    import torch
+    import jittorinfer_amd as J
+    rng = np.random.default_rng(300)
+    lens = [int(x) for x in rng.integers(1, 140, size=300)]
+    lens[7], lens[150], lens[299] = 0, 600, 333
+    lens[20:24] = [77, 77, 77, 77]
+    pool, bt, seqs = U.make_paged(rng, np.maximum(lens, 1), O.TYPE_BF16)
+    seqs = [s[:l] for s, l in zip(seqs, lens)]
+    q = rng.standard_normal((300, 128, 1, 576)).astype(np.float32)
+    tq, tk = torch.from_numpy(q).to(gpu), torch.from_numpy(pool.view(np.int16)).to(gpu)
+    tb, tl = torch.from_numpy(bt).to(gpu), torch.from_numpy(np.asarray(lens, dtype=np.int32)).to(gpu)
+    info = J.plan(tq, tk, O.TYPE_BF16, dv=512, scale=U.SCALE, block_table=tb, seq_lens=tl)
+    assert info["variant"] == 2 and info["n_splits"] == 1 and info["balanced"] == 0 and info["n_workgroups"] == 300, info
+    got, _ = _run_flags(gpu, q, pool, O.TYPE_BF16, bt, lens, 0)
+    same, _ = _run_flags(gpu, q, pool, O.TYPE_BF16, bt, lens, J.MLA_FLAG_UNIFORM_SPLITS)
+    assert np.array_equal(got, same, equal_nan=True), "longest first and batch order differ"
+    want = U.oracle_per_seq(q, seqs, O.TYPE_BF16, 512)
+    print(U.check(got, want, "300 sequences, longest first"))
