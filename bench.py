@@ -329,10 +329,26 @@ def other_config(a, dev, lib, J):
         lens, n_head, n_tok, kv, kvt = [2560] * 4, 16, 512, "bf16", J.MLA_TYPE_BF16
         mask = torch.where(torch.arange(2560, device=dev)[None, :] > 2048 + torch.arange(512, device=dev)[:, None], float("-inf"), 0.0).to(torch.float16)
         name = "BASELINE configs[3]: chunked prefill B=4 H=16, 512 new on 2048 cached tokens, causal f16 mask, bf16 pages"
+    elif a.config == "ragged":
+        # a paged decode batch of any size with lengths uniform in [256, ctx] (more than 256 sequences: one workgroup each, longest first)
+        lens, n_head, n_tok, kv, kvt = [int(x) for x in rng.integers(256, a.ctx + 1, a.batch)], a.heads, 1, "bf16", J.MLA_TYPE_BF16
+        name = "paged MLA decode B=%d H=%d L~U[256,%d], bf16 pages" % (a.batch, a.heads, a.ctx)
+    elif a.config == "chunk":
+        # one prompt chunk of --tokens tokens behind --cached cached ones: a contiguous cache without a block table, causal f16 mask
+        n_old, n_tok, n_head, kv, kvt = a.cached, a.tokens, a.heads, "bf16", J.MLA_TYPE_BF16
+        n_kv = (n_old + n_tok + 31) // 32 * 32
+        g = torch.Generator(device=dev)
+        g.manual_seed(a.seed)
+        pool = (torch.randn((1, n_kv, 576), generator=g, device=dev) * 0.5).to(torch.bfloat16).view(torch.int16)
+        q = torch.randn((1, n_head, n_tok, 576), generator=g, device=dev)
+        mask = torch.where(torch.arange(n_kv, device=dev)[None, :] > n_old + torch.arange(n_tok, device=dev)[:, None], float("-inf"), 0.0).to(torch.float16)
+        out = torch.empty((1, n_tok, n_head, 576), dtype=torch.float32, device=dev)
+        lens = [n_old + n_tok]
+        name = "prompt chunk: %d new on %d cached tokens, H=%d, one contiguous bf16 cache, causal f16 mask" % (n_tok, n_old, n_head)
     else:
         lens, n_head, n_tok, kv, kvt = [int(x) for x in rng.integers(2048, 8193, 64)], 128, 1, "q8_0", J.MLA_TYPE_Q8_0
         name = "BASELINE configs[4]: paged MLA decode B=64 H=128 L~U[2048,8192], Q8_0 pages"
-    if a.config == "c3mask":
+    if a.config in ("c3mask", "chunk"):
         bt = sl = None
     else:
         q, pool, bt, sl = build_paged(dev, lens, n_head, n_tok, kv, a.seed)
@@ -388,8 +404,8 @@ def other_config(a, dev, lib, J):
     e1.record(stream)
     torch.cuda.synchronize()
     kern_ms = e0.elapsed_time(e1) / a.steps
-    if a.config == "c4":
-        n_old = 2048
+    if a.config in ("c4", "chunk"):
+        n_old = 2048 if a.config == "c4" else n_old
         kv_bytes = sum(lens) * KV_ROW_BYTES
         flops = len(lens) * n_head * FLOP_PER_TOKEN_HEAD * (n_tok * n_old + n_tok * (n_tok + 1) // 2)
         roof = {"bound": "mfma", "achieved": flops / (kern_ms * 1e-3) / 1e12, "peak": 2500.0, "unit": "TFLOP/s"}
@@ -461,11 +477,12 @@ def main():
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run can be scaled")
     ap.add_argument("--kv", default="bf16", choices=["bf16", "f16", "q8_0"], help="storage type of the latent KV pool (the headline config is bf16; q8_0 only with --config kvwrite)")
     ap.add_argument("--reuse-mask-extents", action="store_true", help="masked configs: time the launch of a layer after the first of a graph, which finds the key extents of the shared mask in the workspace (MLA_FLAG_MASK_EXTENTS_VALID)")
+    ap.add_argument("--cached", type=int, default=0, help="--config chunk: tokens already in the cache ahead of the chunk")
     ap.add_argument("--ragged", action="store_true", help="--config c3mask: sequence lengths uniform in [2048, 8192] instead of 8192")
     ap.add_argument("--uniform-splits", action="store_true", help="paged decode: equal KV splits per sequence (MLA_FLAG_UNIFORM_SPLITS) instead of the balanced schedule")
     ap.add_argument("--bf16-direct", action="store_true", help="bf16 KV: the hi + lo bf16 program (MLA_FLAG_BF16_DIRECT) instead of the default one that converts the tiles to f16 inside LDS")
     ap.add_argument("--eager", action="store_true", help="time the K steps as K eager launch sequences instead of one replay of a HIP graph that holds them")
-    ap.add_argument("--config", default="c3", choices=["c2", "c3", "c3mask", "c4", "c5", "kvwrite", "rope", "absorb", "unabsorb", "layer"],
+    ap.add_argument("--config", default="c3", choices=["c2", "c3", "c3mask", "c4", "c5", "ragged", "chunk", "kvwrite", "rope", "absorb", "unabsorb", "layer"],
                     help="c3 (default) is the headline workload; the others time BASELINE's remaining GPU configs and the cache write for the profiles")
     a = ap.parse_args()
     if a.gpus != 1:

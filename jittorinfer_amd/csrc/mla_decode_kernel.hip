@@ -816,46 +816,59 @@ __device__ __forceinline__ void mask_extent_block(const KParams & p, int rb, int
         p.mask_ext[(slot * MASK_EXT_CHUNKS + chunk) * 2 + 1] = red_hi[0];
     }
 }
-// order[r] = the sequence with the r-th largest length (ties in batch order).  n <= 4096; grid = ceil(n / 256), block = 256.
+// order[r] = the sequence with the r-th largest length (ties in batch order).  n <= 4096; grid = ceil(n / 64), block = 256: a block ranks
+// 64 sequences, each of its four waves counting the keys (length, 4095 - index) above a sequence's own in a quarter of all n, read from LDS
+// two to a 16-byte load (one thread per sequence over all n, one length per iteration, was a chain of LDS latencies: 20 us for 512
+// sequences, now 5).
 constexpr int SEQ_ORDER_MAX = 4096;
 __global__ void __launch_bounds__(NTHREADS) mla_seq_order_kernel(const int32_t * lens, int n, int * order) {
-    __shared__ int L[SEQ_ORDER_MAX];
-    for (int j = threadIdx.x; j < n; j += NTHREADS) L[j] = lens[j];
+    __shared__ __attribute__((aligned(16))) long long K[SEQ_ORDER_MAX];
+    __shared__ int part[4][64];
+    const int n2 = (n + 1) & ~1;
+    for (int j = threadIdx.x; j < n2; j += NTHREADS)
+        K[j] = j < n ? ((long long) lens[j] << 32) | (unsigned) (SEQ_ORDER_MAX - 1 - j) : (long long) 0x8000000000000000ull;   // padding: below every key
     __syncthreads();
-    const int i = blockIdx.x * NTHREADS + threadIdx.x;
-    if (i >= n) return;
-    const int li = L[i];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, i = min((int) blockIdx.x * 64 + lane, n - 1);
+    const long long ki = K[i];
+    typedef long long ll2 __attribute__((ext_vector_type(2)));
+    const ll2 * K2 = (const ll2 *) K;
+    const int pairs = n2 / 2, j0 = pairs * wave / 4, j1 = pairs * (wave + 1) / 4;
     int rank = 0;
-    for (int j = 0; j < n; j++) rank += (L[j] > li) || (L[j] == li && j < i);
-    order[rank] = i;
+#pragma unroll 8
+    for (int j = j0; j < j1; j++) {
+        const ll2 v = K2[j];
+        rank += (int) (v.x > ki) + (int) (v.y > ki);
+    }
+    part[wave][lane] = rank;
+    __syncthreads();
+    if (wave == 0 && (int) blockIdx.x * 64 + lane < n) order[part[0][lane] + part[1][lane] + part[2][lane] + part[3][lane]] = i;
 }
 
 // grid = (n_row_blocks, 16), or for a launch issued in two forms (n_row_blocks, 16, tokens per row block)
 __global__ void __launch_bounds__(NTHREADS) mla_mask_extent_kernel(const KParams p) { mask_extent_block(p, blockIdx.x, blockIdx.y, blockIdx.z); }
 
-// The same scan with a wave per (row block, sixteenth), four to a block, for launches of many row blocks whose sixteenths are short
-// (a prompt chunk of 512 tokens x 128 heads: 8192 pairs of 4 groups each, for which a block of 256 threads and its barriers are
-// all overhead: 20.9 -> 3 us).  grid = ceil(n_row_blocks * 16 / 4), block = 256.
+// The same scan with 16 lanes per (row block, sixteenth) and a block per row block, for launches of many row blocks whose sixteenths
+// are short (a prompt chunk of 512 tokens x 128 heads: 8192 pairs of 4 groups each, for which a block of 256 threads and its barriers
+// are all overhead: 20.9 -> 5 us).  grid = n_row_blocks, block = 256.
 __global__ void __launch_bounds__(NTHREADS) mla_mask_extent_wave_kernel(const KParams p, int n_rb) {
-    const int lane = threadIdx.x & 63, pair = (int) blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (pair >= n_rb * MASK_EXT_CHUNKS) return;
-    const int rb = pair / MASK_EXT_CHUNKS, chunk = pair - rb * MASK_EXT_CHUNKS;
+    const int sub = threadIdx.x & 15, chunk = threadIdx.x >> 4, rb = blockIdx.x;
+    if (rb >= n_rb) return;
     const int r0 = rb * 128, r1 = min(r0 + 127, p.n_rows - 1);
     const int t0 = r0 / p.n_head, n_t = r1 / p.n_head - t0 + 1;
     const int n_kv = (int) (p.block_table ? p.bt_stride * MLA_PAGE_TOKENS : p.n_kv);
     const int n8 = n_kv / 8;
     const int g0 = (int) ((int64_t) n8 * chunk / MASK_EXT_CHUNKS), ng = (int) ((int64_t) n8 * (chunk + 1) / MASK_EXT_CHUNKS) - g0;
-    const int64_t total = (int64_t) n_t * ng;
+    const int total = n_t * ng;   // (the launcher takes this form for at most 1024 (token, group) pairs per sixteenth)
     int hi = 0, lo = n_kv;
     constexpr int U = 4;
-    for (int64_t base = lane; base < total; base += U * 64) {
+    for (int base = sub; base < total; base += U * 16) {
         u32x4 w[U];
         int   g[U];
 #pragma unroll
         for (int u = 0; u < U; u++) {
-            const int64_t idx = min(base + u * 64, total - 1);   // past the end: the last pair again
-            const int t = (int) (idx / ng);
-            g[u] = g0 + (int) (idx - (int64_t) t * ng);
+            const int idx = min(base + u * 16, total - 1);   // past the end: the last pair again
+            const int t = idx / ng;
+            g[u] = g0 + idx - t * ng;
             const char * a = p.mask + (int64_t) (t0 + t) * p.mask_nb1 + 16 * (int64_t) g[u];   // rows are 8-byte aligned
             const u32x2 x = *(const u32x2 *) a, y = *(const u32x2 *) (a + 8);
             w[u] = u32x4{ x.x, x.y, y.x, y.y };
@@ -868,10 +881,10 @@ __global__ void __launch_bounds__(NTHREADS) mla_mask_extent_wave_kernel(const KP
                 if (((v[e >> 1] >> (16 * (e & 1))) & 0xffff) != 0xfc00u) { lo = min(lo, 8 * g[u] + e); hi = max(hi, 8 * g[u] + e + 1); }
         }
     }
-    for (int d = 32; d > 0; d >>= 1) { lo = min(lo, __shfl_xor(lo, d, 64)); hi = max(hi, __shfl_xor(hi, d, 64)); }
-    if (lane == 0) {
-        p.mask_ext[pair * 2]     = lo;
-        p.mask_ext[pair * 2 + 1] = hi;
+    for (int d = 8; d > 0; d >>= 1) { lo = min(lo, __shfl_xor(lo, d, 64)); hi = max(hi, __shfl_xor(hi, d, 64)); }
+    if (sub == 0) {
+        p.mask_ext[(rb * MASK_EXT_CHUNKS + chunk) * 2]     = lo;
+        p.mask_ext[(rb * MASK_EXT_CHUNKS + chunk) * 2 + 1] = hi;
     }
 }
 
@@ -1146,7 +1159,7 @@ hipError_t launch_decode_fast(const KParams & kp_in, int kv_type, dim3 grid, hip
     const unsigned ext = fold ? MASK_EXT_CHUNKS * ext_sub : 0;
     if (with_prepass && kp.seq_order) {
         if (n_seq > (unsigned) SEQ_ORDER_MAX || grid.x != 1 || grid.y != 1 || grid.z != n_seq) return hipErrorInvalidValue;
-        hipLaunchKernelGGL(mla_seq_order_kernel, dim3((n_seq + NTHREADS - 1) / NTHREADS), dim3(NTHREADS), 0, st, kp.seq_lens, (int) n_seq, (int *) kp.seq_order);
+        hipLaunchKernelGGL(mla_seq_order_kernel, dim3((n_seq + 63) / 64), dim3(NTHREADS), 0, st, kp.seq_lens, (int) n_seq, (int *) kp.seq_order);
     }
     if (!with_prepass) { /* the workspace still holds the Q image and the mask extents of an earlier launch of the same call */ }
     else if (q_in_kernel) { /* nothing: a balanced page schedule is worked out by the workgroups themselves */ }
@@ -1155,11 +1168,11 @@ hipError_t launch_decode_fast(const KParams & kp_in, int kv_type, dim3 grid, hip
     else if (bf16_cvt)                hipLaunchKernelGGL(mla_q_pack_kernel<2>, dim3(n_rb, n_seq + tok_layers, KSTEPS + extra + ext), dim3(NTHREADS), 0, st, kp);
     else                              hipLaunchKernelGGL(mla_q_pack_kernel<0>, dim3(n_rb, n_seq + tok_layers, KSTEPS + extra + ext), dim3(NTHREADS), 0, st, kp);
     if (m && !fold && with_prepass && scan_mask) {
-        // many row blocks with little to scan per (row block, sixteenth): a wave per pair instead of a block
+        // many row blocks with little to scan per (row block, sixteenth): 16 lanes per pair instead of a block
         const int64_t n_kv_m = kp.block_table ? kp.bt_stride * MLA_PAGE_TOKENS : kp.n_kv;
         const int64_t per_pair = (int64_t) (127 / kp.n_head + 2) * (n_kv_m / 8 / MASK_EXT_CHUNKS + 1);
         if (!kp.dual && n_rb * MASK_EXT_CHUNKS >= 1024 && per_pair <= 1024)
-            hipLaunchKernelGGL(mla_mask_extent_wave_kernel, dim3((n_rb * MASK_EXT_CHUNKS + 3) / 4), dim3(NTHREADS), 0, st, kp, (int) n_rb);
+            hipLaunchKernelGGL(mla_mask_extent_wave_kernel, dim3(n_rb), dim3(NTHREADS), 0, st, kp, (int) n_rb);
         else
             hipLaunchKernelGGL(mla_mask_extent_kernel, dim3(n_rb, MASK_EXT_CHUNKS, ext_sub), dim3(NTHREADS), 0, st, kp);
     }
