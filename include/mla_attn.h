@@ -148,7 +148,7 @@ int    mla_attn_launch_partials(const mla_attn_args * args, void * stream);
 int    mla_attn_launch_combine(const mla_attn_args * args, void * stream);
 
 /* mla_attn_launch_partials without the small passes that run ahead of the pipelined kernel (the Q operand image and,
- * with a mask, its key extents): the one kernel that reads the KV rows, alone, for timing it.  Valid only after
+ * with a mask, its key extents; the order of the sequences of a large batch): the one kernel that reads the KV rows, alone, for timing it.  Valid only after
  * mla_attn_launch or mla_attn_launch_partials has run with the same arguments and workspace.  No counterpart in
  * the reference. */
 int    mla_attn_launch_kernel(const mla_attn_args * args, void * stream);
