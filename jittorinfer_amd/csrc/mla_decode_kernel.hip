@@ -313,7 +313,7 @@ __device__ __forceinline__ void decode_body() {
 
     // A paged decode batch of more than 256 sequences with a workgroup each (grid = (1, 1, sequences)) runs in rounds, in dispatch
     // order: the sequences are taken longest first, so that the workgroups that start last are the short ones (512 ragged sequences
-    // of 128 heads: 851 -> 7xx us).  Consecutive dispatch indices go to different XCDs, which spreads every length over all of them.
+    // of 128 heads: 815 -> 720 us per step).  Consecutive dispatch indices go to different XCDs, which spreads every length over all of them.
     if (!MASK && p.seq_order) bz = (int) min((unsigned) p.seq_order[blockIdx.z], gridDim.z - 1);   // (clamped: never a sequence that is not there)
 
     // Balanced schedule (p.balanced; a ragged decode batch): the pages of all sequences form one list, every workgroup
