@@ -35,11 +35,7 @@ MF_QK = "v_mfma_f32_32x32x16_f16" if F16KV else "v_mfma_f32_32x32x16_bf16"
 MF_PV = "v_mfma_f32_32x32x16_f16"
 
 
-def _opt(name, default):
-    return int(ARGS[ARGS.index(name) + 1]) if name in ARGS else default
-
-
-CONV_P1 = _opt("--conv-p1", 5)               # V^T fragments converted in part 1; the rest in the first half of part 2
+CONV_P1 = 5                                  # V^T fragments converted in part 1; the rest in the first half of part 2
 
 PITCH = 1168
 TILE_BYTES = 32 * PITCH
@@ -606,8 +602,12 @@ def clk_dump():
     pass
 
 
-B2_AT = _opt("--b2-at", 20)       # P.V slot ahead of which the barrier "every wave has read P of this tile" sits
-PW_AT = _opt("--pw-at", 24)       # P.V slot ahead of which P of the next tile is written (the softmax is done by then)
+# P.V slot ahead of which the barrier "every wave has read P of this tile" sits: behind the request for the tile's last P^T fragment
+# (a ring of four asks for fragment 7 at slot 16, a ring of three -- the mask builds -- at slot 20: with the barrier ahead of slot 20
+# the other waves' reads of fragment 7, wave 3's rows, raced with wave 3's write of the next tile's P), with an MFMA or two between
+# the request and the wait for it
+B2_AT = 22 if PRING == 3 else 20
+PW_AT = 24                        # P.V slot ahead of which P of the next tile is written (the softmax is done by then)
 
 
 def iteration(resc, lab_loop):
@@ -668,7 +668,8 @@ def iteration(resc, lab_loop):
             bias_block()
 
     def p_read_by_all():
-        # every P^T fragment of tile IT is in this wave's registers (the last read was issued at slot 16) before any wave overwrites P
+        # every P^T fragment of tile IT is in this wave's registers before any wave overwrites P
+        assert all(("p", f) in lds.issued for f in range(8)), "barrier ahead of the request for a P^T fragment"
         lds.drain()
         e("s_barrier")
     sm = softmax_lines()
