@@ -1,0 +1,163 @@
+"""The generated wave programs (jittorinfer_amd/csrc/mla_decode_*.inc) run on the CPU, in the emulator of tests/wave_emu.py, for all
+four waves of a workgroup: their results against a float64 attention over the same piece of the cache, and the emulator's hazard
+report -- registers used while a load into them is in flight, LDS words one wave writes and another reads (or overwrites) without
+"wait, barrier" in between, accesses outside the buffers -- which has to be empty.  Every conditional branch of a program has to go
+both ways over the scenarios of its family, so that the report covers the paths a launch can take (no tile load left to request,
+the last tile, a ragged end, the rescale of the accumulators, each kind of store)."""
+import numpy as np
+import pytest
+
+from tests import wave_emu as E
+from tests import wave_scenarios as S
+
+MAX_ABS, REL_L2 = 2e-3, 1e-3        # the tolerance of the kernels' parity tests
+
+
+def _check(got, want, what):
+    err = np.abs(got - want).max()
+    rel = np.linalg.norm(got - want) / max(np.linalg.norm(want), 1e-30)
+    assert err <= MAX_ABS * max(1.0, np.abs(want).max()) and rel <= REL_L2, "%s: max-abs %.3g rel-L2 %.3g" % (what, err, rel)
+
+
+class Coverage:
+    """Which way every conditional branch of a program went, over all scenarios run on it."""
+
+    def __init__(self):
+        self.seen = {}
+
+    def install(self, wg):
+        cov = self.seen
+
+        def wrap(fn):
+            def h(w, o, m):
+                jump = fn(w, o, m)
+                cov.setdefault(w.pc, set()).add(jump is not None)
+                return jump
+            return h
+        wg.branch_handlers = {k: wrap(E.HANDLERS[k]) for k in ("s_cbranch_scc0", "s_cbranch_scc1")}
+
+    def missing(self, wg):
+        """Branches that did not go both ways.  One cannot: the rescale test behind the first tile of the column-split programs (the
+        first softmax clears its flag: the accumulators are still zero), the first branch to a label of that kind."""
+        out = []
+        first_resc = next((pc for pc, ins in enumerate(wg.instrs) if ins[0] == "s_cbranch_scc1" and ins[1][0][1].startswith("Lresc")), None)
+        for pc, ins in enumerate(wg.instrs):
+            if ins[0].startswith("s_cbranch") and self.seen.get(pc, set()) != {True, False}:
+                if pc == first_resc and self.seen.get(pc) == {False} and "_cs_" in wg.name:
+                    continue
+                out.append((pc, ins[3], sorted(self.seen.get(pc, set()))))
+        return out
+
+
+def run_cs(name, cov, f16, mask_build=False, bias_build=False, n_rows=128, kv=(0, 128), seq_len=None, paged=None, f32_rows=True, final=True,
+           q_in_lds=False, boost=False, seed=0, n_head=None, softcap=0.0, alibi=False, v_col0=False):
+    rng = np.random.default_rng(seed)
+    n_head = n_head or n_rows
+    mask = None
+    seq_len = kv[1] if seq_len is None else seq_len
+    paged = (not mask_build) if paged is None else paged
+    if mask_build:
+        n_kv = (seq_len + 31) // 32 * 32
+        mask = np.where(rng.random(((n_rows + n_head - 1) // n_head, n_kv)) < 0.25, -np.inf, rng.standard_normal(((n_rows + n_head - 1) // n_head, n_kv)) * (0.5 if alibi else 0.0))
+        mask[:, seq_len:] = -np.inf
+        mask[:, kv[0]] = 0.0              # (no row of the piece without a key: such rows are the launcher's business)
+        if not paged:         # (a masked launch over a cache without a table covers whole tiles; with a table the lengths may be ragged)
+            kv, seq_len = (kv[0], min(n_kv, (kv[1] + 31) // 32 * 32)), n_kv
+    piece = S.Piece(rng, f16, n_rows=n_rows, kv_begin=kv[0], kv_end=kv[1], seq_len=seq_len, paged=paged, mask=mask, n_head=n_head,
+                    k_boost=(lambda t: 4.0 ** ((t - kv[0]) // 32)) if boost else None)
+    slopes = None
+    if alibi:
+        slopes = (2.0 ** (-8.0 * (np.arange(128) % n_head + 1) / n_head)).astype(np.float32)
+    scale = S.SCALE
+    inputs = S.cs_inputs(piece, piece.gmem, f32_rows=f32_rows, final=final, scale=scale, mask_build=mask_build)
+    lds_init = S.cs_handoff(piece, bias_build, slopes, -2.0 * softcap if softcap else 0.0)
+    if bias_build:        # the launcher hands scale / softcap, 2 log2(e) scale / softcap and -2 softcap where the plain builds find scale and scale log2(e)
+        base = inputs
+
+        def inputs(w, base=base):
+            d = base(w)
+            if softcap:
+                d["scl"] = int(np.array([scale / softcap], np.float32).view(np.uint32)[0])
+                d["cl2"] = int(np.array([2.0 * np.log2(np.e) * scale / softcap], np.float32).view(np.uint32)[0])
+            return d
+    if q_in_lds:          # the operands wait in the tile buffers: wave w's 32 rows in buffer w, laid out like a tile of the cache
+        rows = np.zeros((4, 32, S.PITCH // 2), np.uint16)
+        rows[:, :, :576] = piece.q_bits.reshape(4, 32, 576)
+        lds_init = lds_init + [(w * S.TILE_BYTES, rows[w]) for w in range(4)]
+        base2 = inputs
+
+        def inputs(w, base2=base2):
+            d = base2(w)
+            d["flg"] |= 64
+            d["qp"] = 0
+            return d
+    if v_col0:
+        base3 = inputs
+
+        def inputs(w, base3=base3):
+            d = base3(w)
+            d["flg"] |= 16
+            return d
+    wg = E.Workgroup(S.program_text(name), 4, piece.gmem, inputs, lds_init=lds_init)
+    wg.name = name
+    cov.install(wg)
+    findings = wg.run()
+    assert not findings, "%s: %s" % (name, findings[:5])
+    want, m_want, l_want = piece.reference(scale=scale, softcap=softcap, slopes=slopes, v0=64 if v_col0 else 0)   # (V = columns 64 .. 575 in the second pass of a 576-wide V)
+    if f32_rows:
+        got = piece.gmem.array("out").view(np.float32).reshape(128, 512)[:n_rows].astype(np.float64)
+    else:   # f16 partials, [column / 8][row][8]
+        got = piece.gmem.array("out").view(np.float16).reshape(64, 128, 8).transpose(1, 0, 2).reshape(128, 512)[:n_rows].astype(np.float64)
+    _check(got, want, name)
+    if not final:
+        ml = piece.gmem.array("ml").view(np.float32).reshape(128, 2)[:n_rows].astype(np.float64)
+        lse = ml[:, 0] + np.log2(ml[:, 1])
+        if softcap:         # the capped logits are kept less the cap: a constant per row
+            lse = lse + softcap * np.log2(np.e)
+        assert np.abs(lse - (m_want + np.log2(l_want))).max() < 1e-3, "%s: (m, l) of the piece" % name
+    return wg
+
+
+CS_SCENARIOS = [
+    dict(kv=(0, 128)),                                                     # four tiles: one round of tile loads in the loop, then none
+    dict(kv=(0, 32), final=False, f32_rows=False),                         # one tile, f16 partial rows
+    dict(kv=(128, 128 + 64), seq_len=400, final=False),                    # two tiles inside a longer sequence, f32 partial rows
+    dict(kv=(96, 96 + 96 - 5), paged=True),                                # a split that starts inside a page; ragged end
+    dict(kv=(0, 7 * 32 + 1), paged=False),                                 # contiguous cache, eight tiles, one key in the last
+    dict(kv=(0, 160), boost=True),                                         # the running maxima move: accumulators rescaled
+    dict(kv=(0, 96), n_rows=100, final=False, f32_rows=False),             # the last wave has 4 rows
+    dict(kv=(0, 64), q_in_lds=True),                                       # Q rounded by the kernel's own prologue, waiting in LDS
+    dict(kv=(0, 96), v_col0=True),                                         # second pass of a 576-wide V
+    dict(kv=(256, 256 + 19), seq_len=256 + 19),                            # one ragged tile
+]
+
+
+@pytest.mark.parametrize("name,f16", [("mla_decode_cs_bf16.inc", False), ("mla_decode_cs_f16.inc", True)])
+def test_column_split_programs(name, f16):
+    cov = Coverage()
+    for k, sc in enumerate(CS_SCENARIOS):
+        wg = run_cs(name, cov, f16, seed=k, **sc)
+    assert not cov.missing(wg), cov.missing(wg)
+
+
+@pytest.mark.parametrize("name,f16", [("mla_decode_cs_bf16_mask.inc", False), ("mla_decode_cs_f16_mask.inc", True)])
+def test_masked_column_split_programs(name, f16):
+    cov = Coverage()
+    for k, sc in enumerate(CS_SCENARIOS):
+        sc = {kk: vv for kk, vv in sc.items() if kk != "paged"}
+        wg = run_cs(name, cov, f16, mask_build=True, seed=10 + k, n_head=16, **sc)
+    wg = run_cs(name, cov, f16, mask_build=True, seed=30, kv=(0, 128), paged=True, n_head=128)
+    wg = run_cs(name, cov, f16, mask_build=True, seed=31, kv=(0, 19), paged=True, n_head=64)
+    wg = run_cs(name, cov, f16, mask_build=True, seed=32, kv=(32, 128 + 7), paged=True, n_head=32)
+    assert not cov.missing(wg), cov.missing(wg)
+
+
+@pytest.mark.parametrize("name,f16", [("mla_decode_cs_bf16_bias.inc", False), ("mla_decode_cs_f16_bias.inc", True)])
+def test_bias_column_split_programs(name, f16):
+    cov = Coverage()
+    for k, sc in enumerate(CS_SCENARIOS):
+        sc = {kk: vv for kk, vv in sc.items() if kk != "paged"}
+        wg = run_cs(name, cov, f16, mask_build=True, bias_build=True, seed=40 + k, n_head=32, alibi=k % 2 == 0, softcap=30.0 if k % 3 else 0.0, **sc)
+    wg = run_cs(name, cov, f16, mask_build=True, bias_build=True, seed=61, kv=(0, 19), paged=True, n_head=64, alibi=True)
+    wg = run_cs(name, cov, f16, mask_build=True, bias_build=True, seed=62, kv=(32, 128 + 7), paged=True, n_head=32, softcap=20.0)
+    assert not cov.missing(wg), cov.missing(wg)
