@@ -371,6 +371,8 @@ class Wave:
             self.set_exec(val)
         elif k == "exec_hi":
             self.set_exec((self.exec & 0xffffffff) | ((val & 0xffffffff) << 32))
+        elif k == "exec_lo":
+            self.set_exec((self.exec & ~0xffffffff) | (val & 0xffffffff))
         elif k == "m0":
             self.m0 = val & 0xffffffff
         else:
@@ -1041,6 +1043,8 @@ def _(w, o, m):
 
 # ---- global memory
 def _gaddr(w, voff, sbase, m):
+    if sbase[0] == "label" and sbase[1] == "off":       # no scalar base: the address is a register pair
+        return (w.rv(voff, 0).astype(np.uint64) | (w.rv(voff, 1).astype(np.uint64) << np.uint64(32))) + np.uint64(m.get("offset", 0))
     return (np.uint64(w.rs(sbase, 2)) + w.rv(voff).astype(np.uint64) + np.uint64(m.get("offset", 0))).astype(np.uint64)
 
 
@@ -1063,7 +1067,7 @@ HANDLERS["global_load_dwordx4"] = _gload(4)
 @op("global_load_lds_dwordx4")
 def _(w, o, m):
     wg = w.wg
-    addr = _gaddr(w, o[0], o[1], m)
+    addr = _gaddr(w, o[0], o[1], m)       # (the instruction offset moves the LDS address as well as the global one)
     data, bad = wg.gmem.read(addr, 16, w.em)
     if bad.any():
         wg.report("global-oob", w.index, w.pc, "tile copy reads outside the scenario's buffers, lanes %s, e.g. 0x%x" % (np.nonzero(bad)[0][:4], int(addr[bad][0])))
