@@ -22,6 +22,8 @@ HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 / fp16 MFMA rate
 KV_ROW_BYTES = 1152     # 576 bf16
 FLOP_PER_TOKEN_HEAD = 2 * 576 + 2 * 512
+# the commit and date at which profiles/mla_decode_kernel_c3_pmc.md's FETCH_SIZE / WRITE_SIZE readings (the `traffic` constants below) were taken
+TRAFFIC_PROFILE_COMMIT = ("e0ae410", "2026-11-25")
 
 
 def build_workload(dev, n_seq, n_head, ctx, n_pools, seed, kv="bf16"):
@@ -576,11 +578,25 @@ def main():
     else:
         step_stats = None
 
-    # ---- the kernels that make up the node without the Q pre-pack: the split-K decode kernel and the combine pass, K times
-    # back to back with HIP events on the launch stream around them (the stream is in order, so this is K times their
-    # durations plus the gaps between them); then the decode kernel alone the same way, and with an event between every two
-    # launches for the spread
-    def timed(fns):
+    # ---- the kernels that make up the node without the Q pre-pack: the split-K decode kernel and the combine pass, with a HIP
+    # event on the launch stream between every two steps (the stream is in order: an interval is one launch's duration plus the
+    # hand-over to the next); mean, median and spread all come from those K intervals.  Then the decode kernel alone the same
+    # way, whole steps (pre-pack + decode + combine) the same way, and, labelled as what it is, K decode launches back to back
+    # between one pair of events (a launch's first workgroups start while the last of the one before still run, so this is
+    # the rate of a stream of launches, not the duration of one)
+    def per_launch(fns):
+        marks = [torch.cuda.Event(enable_timing=True) for _ in range(a.steps + 1)]
+        marks[0].record(stream)
+        for i in range(a.steps):
+            for fn in fns:
+                step(i, fn)
+            marks[i + 1].record(stream)
+        torch.cuda.synchronize()
+        us = sorted(marks[i].elapsed_time(marks[i + 1]) * 1e3 for i in range(a.steps))
+        pick = lambda f: us[min(len(us) - 1, int(f * len(us)))]
+        return {"mean": sum(us) / len(us), "median": 0.5 * (us[(len(us) - 1) // 2] + us[len(us) // 2]), "p10": pick(0.1), "p90": pick(0.9), "launches": len(us)}
+
+    def back_to_back(fns):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record(stream)
         for i in range(a.steps):
@@ -588,20 +604,12 @@ def main():
                 step(i, fn)
         e1.record(stream)
         torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / a.steps
-    node_ms = timed([lib.mla_attn_launch_kernel, lib.mla_attn_launch_combine])   # the Q operand image in the workspace is the one the steps above wrote
-    kern_ms = timed([lib.mla_attn_launch_kernel])
-    marks = [torch.cuda.Event(enable_timing=True) for _ in range(a.steps + 1)]
-    marks[0].record(stream)
-    for i in range(a.steps):
-        step(i, lib.mla_attn_launch_kernel)
-        marks[i + 1].record(stream)
-    torch.cuda.synchronize()
-    per_launch = sorted(marks[i].elapsed_time(marks[i + 1]) * 1e3 for i in range(a.steps))
-    pick = lambda f: per_launch[min(len(per_launch) - 1, int(f * len(per_launch)))]
-    kern_stats = {"mean": kern_ms * 1e3, "median": pick(0.5), "p10": pick(0.1), "p90": pick(0.9)}
-    # and whole steps with events (pre-pack + decode + combine)
-    step_ms_events = timed([lib.mla_attn_launch])
+        return e0.elapsed_time(e1) * 1e3 / a.steps
+    node_stats = per_launch([lib.mla_attn_launch_kernel, lib.mla_attn_launch_combine])   # the Q operand image in the workspace is the one the steps above wrote
+    kern_stats = per_launch([lib.mla_attn_launch_kernel])
+    kern_stats["back_to_back"] = back_to_back([lib.mla_attn_launch_kernel])
+    step_stats_events = per_launch([lib.mla_attn_launch])
+    node_ms, kern_ms, step_ms_events = node_stats["mean"] * 1e-3, kern_stats["mean"] * 1e-3, step_stats_events["mean"] * 1e-3
 
     kv_bytes = a.batch * a.ctx * KV_ROW_BYTES
     flops = a.batch * a.ctx * a.heads * FLOP_PER_TOKEN_HEAD
@@ -626,14 +634,19 @@ def main():
     # HBM bytes of one decode-kernel launch, from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by what the same
     # counters read for the library's copy kernel; figures and commands in profiles/mla_decode_kernel_c3_pmc.md
     traffic, traffic_source, traffic_decode = None, None, None
+    measured_plan = {"variant": 2, "n_splits": 8, "balanced": 1, "n_workgroups": 256, "lds_bytes": 160864}   # the launch the constants below were taken on
     if a.batch == 32 and a.heads == 128 and a.ctx == 8192 and a.kv == "bf16":
-        traffic_source = ("rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of the decode kernel and of the combine pass, scaled by the copy kernel's readings: "
-                          "profiles/mla_decode_kernel_c3_pmc.md (measured constants of that profile, not of this run)")
-        # KiB per dispatch, mean: decode kernel (fetch, write), combine pass (fetch, write)
-        d_f, d_w, c_f, c_w = (150524, 34048, 16677, 8192) if a.bf16_direct else (150613, 35584, 16548, 8192)
-        scale_f = 294912 / 147466.0   # the copy kernel reads 294 912 KiB and FETCH_SIZE reports 147 466
-        traffic_decode = int(d_f * 1024 * scale_f + d_w * 1024)
-        traffic = traffic_decode + int(c_f * 1024 * scale_f + c_w * 1024)
+        differs = {k: (plan.get(k), v) for k, v in measured_plan.items() if plan.get(k) != v}
+        if differs:
+            traffic_source = "not reported: the plan of this launch differs from the one profiles/mla_decode_kernel_c3_pmc.md was measured on: %s" % differs
+        else:
+            traffic_source = ("rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of the decode kernel and of the combine pass, scaled by the copy kernel's readings: "
+                              "profiles/mla_decode_kernel_c3_pmc.md (constants of that profile, taken at commit %s on %s, not of this run)" % TRAFFIC_PROFILE_COMMIT)
+            # KiB per dispatch, mean: decode kernel (fetch, write), combine pass (fetch, write)
+            d_f, d_w, c_f, c_w = (150524, 34048, 16677, 8192) if a.bf16_direct else (150613, 35584, 16548, 8192)
+            scale_f = 294912 / 147466.0   # the copy kernel reads 294 912 KiB and FETCH_SIZE reports 147 466
+            traffic_decode = int(d_f * 1024 * scale_f + d_w * 1024)
+            traffic = traffic_decode + int(c_f * 1024 * scale_f + c_w * 1024)
     res = {
         "metric": "mla_paged_decode_kv_read_bandwidth", "value": value, "unit": "GB/s",
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms_per_step,
@@ -644,14 +657,14 @@ def main():
         "us_per_step": ms_per_step * 1e3,
         "launch": "eager" if a.eager else "hip graph replay of the K steps",
         "us_per_step_eager": eager_ms_per_step * 1e3,
-        "us_per_step_events": step_ms_events * 1e3,
+        "us_per_step_events": step_stats_events,
         "us_per_step_spread": step_stats,
         "tokens_per_s": a.batch / (ms_per_step * 1e-3),
         "pct_hbm_peak": 100.0 * value / HBM_PEAK_GBPS,
         "tflops": flops / (ms_per_step * 1e-3) / 1e12,
         "roofline": {"bound": "hbm", "kernel": "mla_decode_kernel<%s> + mla_attn_combine_kernel" % a.kv, "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic, "traffic_source": traffic_source,
-                     "algorithmic_bytes_per_launch": kv_bytes, "kernels_us": node_ms * 1e3,
+                     "algorithmic_bytes_per_launch": kv_bytes, "kernels_us": node_stats,
                      "decode_kernel_alone": {"achieved": achieved_decode, "frac": achieved_decode / HBM_PEAK_GBPS, "kernel_us": kern_stats, "traffic": traffic_decode},
                      "mfma_tflops": flops / (node_ms * 1e-3) / 1e12},
         "cpu_baseline": cpu,

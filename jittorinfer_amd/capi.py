@@ -108,21 +108,38 @@ _retired = []
 
 def _workspace(device, nbytes, stream=None):
     """The scratch area of a launch: one per (device, stream) -- launches on different streams run side by side and each
-    needs its own partials, Q image and schedule -- and grow-only.  An area that has been handed out is never freed: a
-    launch queued on another thread's behalf or recorded into a HIP graph keeps its address, so a larger request gets a new
-    area and the old one is only retired (a few tens of MB per size step).  Under graph capture the new area comes from the
-    graph's own memory pool, like any tensor made during capture."""
+    needs its own partials, Q image and schedule.  An area that has been handed out is not freed while work may use it: a launch
+    queued earlier or recorded into a HIP graph keeps its address, so a larger request gets a new area and the old one is retired.
+    Areas grow by at least half (requests that creep up -- a decode loop adding one key per step -- retire O(log size) areas, not
+    one per step); release_workspaces() drops what has been retired.  Under graph capture the new area comes from the graph's own
+    memory pool, like any tensor made during capture."""
     import torch
     if stream is None:
         stream = torch.cuda.current_stream(device).cuda_stream
     key = (device, int(stream))
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
+        have = 0
         if ws is not None:
             _retired.append(ws)
-        ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+            have = ws.numel()
+        ws = torch.empty(max(nbytes, have + have // 2, 1 << 20), dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws
+
+
+def release_workspaces(stream=None, device=None):
+    """Drops the retired scratch areas and, for a stream that is given (a raw handle; with its device), that stream's current one --
+    to be called when the stream is destroyed, or at any point where no launch that used them is still queued or held in a HIP
+    graph that will be replayed: the call synchronizes the device first and refuses to run under graph capture."""
+    import torch
+    if torch.cuda.is_current_stream_capturing():
+        raise RuntimeError("release_workspaces: not under graph capture")
+    torch.cuda.synchronize(device)
+    _retired.clear()
+    if stream is not None:
+        dev = torch.device("cuda", torch.cuda.current_device()) if device is None else device
+        _workspaces.pop((dev, int(stream)), None)
 
 
 def make_args(q, k, kv_type, dv=512, mask=None, scale=1.0, max_bias=0.0, logit_softcap=0.0, block_table=None,

@@ -601,9 +601,14 @@ int compute_flash_attn(backend_ctx * ctx, const tensor * dst) {
         ctx->workspace_size = need;
     }
     a.workspace = ctx->workspace; a.workspace_size = ctx->workspace_size;
-    mla_attn_args key;       // (what the extents depend on: everything but the operands that change from layer to layer)
+    // what the extents, their layout and their place in the workspace depend on: everything but the operands that change from layer
+    // to layer -- and of those the alignment, which the planner looks at (a Q8_0 cache that is not 16-byte aligned runs on an f16 copy,
+    // with extents per row block where the aligned form has them per token)
+    mla_attn_args key;
     memcpy(&key, &a, sizeof(key));
-    key.q = nullptr; key.kv = nullptr; key.dst = nullptr;
+    key.q   = (const void *) ((uintptr_t) a.q & 15);
+    key.kv  = (const void *) ((uintptr_t) a.kv & 15);
+    key.dst = (float *) ((uintptr_t) a.dst & 15);
     const bool same_mask = a.mask && ctx->reuse_mask_extents && ctx->ext_key_valid && memcmp(&key, &ctx->ext_key, sizeof(key)) == 0;
     if (same_mask) { a.flags |= MLA_FLAG_MASK_EXTENTS_VALID; g_mask_extent_reuses++; }
     const int rc = mla_attn_launch(&a, ctx->stream);

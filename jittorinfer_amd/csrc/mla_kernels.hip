@@ -449,34 +449,37 @@ __device__ __forceinline__ void partial_slots(const KParams & p, int b, int row,
 }
 
 // Log-sum-exp merge of the split-K partials: out = sum_c (O_c/l_c) l_c 2^(m_c - M) / sum_c l_c 2^(m_c - M).
-// Partials hold O_c/l_c as f16, laid out [seq][split][column/8][row][8].  One thread = one (row, group of 8 columns):
-// 16-byte loads, splits in groups of 8 so that all the loads of a group are in flight together.  A wave covers 16 rows x 4
-// column groups: it reads runs of 256 bytes (16 rows of one column group are contiguous in the partial layout) and writes 128
-// contiguous bytes per row.  grid = (ceil(rows/16), ceil(dv/128), n_seq), block = 256 = 16 rows x 16 column groups.
+// Partials hold O_c/l_c as f16, laid out [seq][split][column/8][row][8].  One thread = one row and two groups of 8 columns 128
+// columns apart: 16-byte loads, splits in groups of 8 so that all the loads of a group (8 (m, l) pairs, 16 partial chunks) are in
+// flight together, and the weights of a group of splits are worked out once for both column groups.  A wave covers 16 rows x 4
+// column groups (twice): it reads runs of 256 bytes (16 rows of one column group are contiguous in the partial layout) and writes
+// 128 contiguous bytes per row.  grid = (ceil(rows/16), ceil(dv/256), n_seq), block = 256 = 16 rows x 16 column groups (x 2).
 __global__ void __launch_bounds__(256) mla_attn_combine_kernel(const KParams p) {
     const int b = blockIdx.z;
     const int row = blockIdx.x * 16 + (threadIdx.x & 15);
-    const int cg  = blockIdx.y * 16 + (threadIdx.x >> 4);
+    const int cg  = blockIdx.y * 32 + (threadIdx.x >> 4);
     const int seq_len = p.block_table ? min(p.seq_lens[b], (int) p.bt_stride * MLA_PAGE_TOKENS) : (int) p.n_kv;
     if (row >= p.n_rows || cg * 8 >= p.dv_total) return;
+    const bool two = (cg + 16) * 8 < p.dv_total;   // the second column group exists
     int slot0, nvalid, lrow, slot_rows;
     partial_slots(p, b, row, seq_len, slot0, nvalid, lrow, slot_rows);
     if (nvalid < 0) return;
 
     const float2 *   ml = (const float2 *) p.part_ml + (int64_t) slot0 * slot_rows + lrow;
     const _Float16 * po = p.part_o + (int64_t) slot0 * slot_rows * p.dv_total + ((int64_t) cg * slot_rows + lrow) * 8;
-    const int64_t ml_step = slot_rows, po_step = (int64_t) slot_rows * p.dv_total;
+    const int64_t ml_step = slot_rows, po_step = (int64_t) slot_rows * p.dv_total, second = two ? (int64_t) 16 * slot_rows * 8 : 0;
 
     float M = -INFINITY, L = 0.f;
-    float o[8] = { 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f };
+    float o[16] = { 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f };
     for (int c0 = 0; c0 < nvalid; c0 += 8) {
         float2 mlv[8];
-        u32x4  hv[8];
+        u32x4  hv[8], hw[8];
 #pragma unroll
         for (int k = 0; k < 8; k++) {
             const int c = min(c0 + k, nvalid - 1);  // past the end: a duplicate of the last split, given weight 0 below
             mlv[k] = ml[c * ml_step];
             hv[k]  = *(const u32x4 *) (po + c * po_step);
+            hw[k]  = *(const u32x4 *) (po + c * po_step + second);
         }
         float Mg = M;
 #pragma unroll
@@ -486,16 +489,16 @@ __global__ void __launch_bounds__(256) mla_attn_combine_kernel(const KParams p) 
         M = Mg;
         L *= r;
 #pragma unroll
-        for (int k = 0; k < 8; k++) o[k] *= r;
+        for (int k = 0; k < 16; k++) o[k] *= r;
 #pragma unroll
         for (int k = 0; k < 8; k++) {
             // l_c 2^(m_c - M); a split that saw only masked keys (m_c = -inf) and the padding of the group get 0
             const float w = (c0 + k < nvalid && mlv[k].x != -INFINITY) ? mlv[k].y * fast_exp2(mlv[k].x - M) : 0.f;
             L += w;
             if (w == 0.f) continue;  // its partial may hold anything (0/0 of a split without a key), never multiply it in
-            const unsigned h[4] = { hv[k].x, hv[k].y, hv[k].z, hv[k].w };
+            const unsigned h[8] = { hv[k].x, hv[k].y, hv[k].z, hv[k].w, hw[k].x, hw[k].y, hw[k].z, hw[k].w };
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
+            for (int e = 0; e < 8; e++) {
                 o[2 * e]     += f16_bits_to_f32(h[e] & 0xffff) * w;
                 o[2 * e + 1] += f16_bits_to_f32(h[e] >> 16) * w;
             }
@@ -505,6 +508,10 @@ __global__ void __launch_bounds__(256) mla_attn_combine_kernel(const KParams p) 
     float * out = p.dst + ((int64_t) b * p.n_rows + row) * p.dst_stride + p.v_col0 + cg * 8;
     *(f32x4 *) out       = f32x4{ o[0] * inv, o[1] * inv, o[2] * inv, o[3] * inv };
     *(f32x4 *) (out + 4) = f32x4{ o[4] * inv, o[5] * inv, o[6] * inv, o[7] * inv };
+    if (two) {
+        *(f32x4 *) (out + 128) = f32x4{ o[8] * inv, o[9] * inv, o[10] * inv, o[11] * inv };
+        *(f32x4 *) (out + 132) = f32x4{ o[12] * inv, o[13] * inv, o[14] * inv, o[15] * inv };
+    }
 }
 
 // The same merge for rows with many splits (one or two long sequences: 256 pieces of one row's output): the walk over the splits of
@@ -1182,7 +1189,7 @@ static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
             hipLaunchKernelGGL(mla_attn_combine_wide_kernel<4>, gw, dim3(256), 0, st, kp);
             return (int) hipGetLastError();
         }
-        dim3 g((unsigned) ((kp.n_rows + 15) / 16), (unsigned) ((dv + 127) / 128), (unsigned) a->n_seq);
+        dim3 g((unsigned) ((kp.n_rows + 15) / 16), (unsigned) ((dv + 255) / 256), (unsigned) a->n_seq);
         hipLaunchKernelGGL(mla_attn_combine_kernel, g, dim3(256), 0, st, kp);
         return (int) hipGetLastError();
     };
