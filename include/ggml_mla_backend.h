@@ -60,8 +60,14 @@
  * default is outside the 1e-3 tolerance by that much (tests/test_backend_gpu.py states both numbers).  A backend
  * initialised with params containing "f16_acc=strict" (ggml_backend_dev_init(dev, params)), or with
  * GGML_HIP_MLA_F16_ACC=strict in the environment, replays ggml-cpu's f16 accumulator step for step instead (1.1e-4 from
- * ggml-cpu's node; contiguous caches only; 4 times slower on a decode step): for bit-for-bit comparisons with ggml-cpu's
+ * ggml-cpu's node; contiguous and paged caches; 4 times slower on a decode step): for bit-for-bit comparisons with ggml-cpu's
  * fused node, not for serving.
+ * Q8_0 KV: the matrix cores are fed q * d rounded to f16 (K, V and the Q8_0-quantized Q alike) where ggml-cpu multiplies integers and
+ * scales (ggml-cpu-quants.c:3814-4241) and dequantises V to f32 (ggml-quants.c:357-373).  Over many keys the rounding averages out
+ * (4.5e-4 rel-L2 at any block scale); when two or three keys carry a row it shows in single elements, up to 2.5e-3 max-abs against
+ * the stated 2e-3 (rel-L2 stays near 3e-4).  A cache of at most one page per sequence takes the exact path by itself; params containing
+ * "q8=exact", or GGML_HIP_MLA_Q8=exact in the environment, make every Q8_0 node take it (the reference's own arithmetic, keys in
+ * order: within 1e-5 of ggml-cpu's node at any shape, 10 to 100 times slower): for comparisons, not for serving.
  * BF16 KV, more than 32 attention rows per sequence: the decode kernel converts the cache tiles to f16 on the way (exact for magnitudes in [2^-14, 65504], which a
  * latent cache holds; see MLA_FLAG_BF16_DIRECT in mla_attn.h); params containing "bf16=direct", or GGML_HIP_MLA_BF16=direct
  * in the environment, keep the tiles in bf16 for caches with values outside that range.

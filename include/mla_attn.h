@@ -36,7 +36,16 @@ extern "C" {
 
 /* flags */
 #define MLA_FLAG_F16_ACC_STRICT 1u /* F16 KV only: replay ggml-cpu's per-key f16 accumulator (ggml-cpu.c:12066-12080)
-                                      instead of accumulating in f32; sequential over keys, a correctness mode */
+                                      instead of accumulating in f32; sequential over keys, a correctness mode; over a
+                                      contiguous cache or through the block table */
+#define MLA_FLAG_Q8_EXACT 16u      /* Q8_0 KV only: the reference's own arithmetic -- Q quantized to Q8_0, integer block dots times
+                                      d_q * d_k (ggml-cpu-quants.c:3814-4241), V dequantised to f32 (ggml-quants.c:357-373), f32
+                                      accumulator, keys in order -- instead of the matrix-core path, whose operands are q * d rounded to
+                                      f16 (q * d has 19 significant bits, f16 keeps 11).  That rounding averages out over many keys
+                                      (4.5e-4 relative L2 error at any block scale) but shows in single elements when two or three
+                                      keys carry a row: up to 2.5e-3 against the stated 2e-3.  A correctness mode like the one above,
+                                      10 to 100 times slower; without the flag it is taken by itself when no sequence can hold more
+                                      than one page of keys, where it costs nothing to speak of. */
 #define MLA_FLAG_UNIFORM_SPLITS 2u /* paged decode: give every sequence the same number of equal KV splits (sized for the longest
                                       sequence the block table can hold) instead of the balanced schedule that deals equal
                                       runs of the batch's whole page list to the workgroups, and the sequences of a batch of

@@ -9,6 +9,7 @@ MLA_FLAG_F16_ACC_STRICT = 1
 MLA_FLAG_UNIFORM_SPLITS = 2
 MLA_FLAG_BF16_DIRECT = 4
 MLA_FLAG_MASK_EXTENTS_VALID = 8
+MLA_FLAG_Q8_EXACT = 16
 MLA_ERR_TOO_LARGE = -7
 MLA_ATTN_STATIC_WORKSPACE_MAX = 48 << 20
 PAGE_TOKENS = 128

@@ -40,12 +40,8 @@ Q8_WAVE_CHUNKS = 306           # a wave copies 306 of the 1224 16-byte chunks of
 CPR = 73                       # 16-byte chunks per padded row
 WAVE_CHUNKS = 8 * CPR          # 584: each wave moves rows 8w..8w+7 of a tile
 TAU = 8.0
-def _opt(name, default):
-    return int(sys.argv[sys.argv.index(name) + 1]) if name in sys.argv else default
-
-
-P1_PV = _opt("--p1pv", 24 if SPLIT else 12)   # P.V MFMAs issued among the 36 QK^T MFMAs; the rest cover the softmax
-P1_LEAD = _opt("--lead", 3)                   # P.V MFMAs at the head of an iteration (they cover the first K fragment reads)
+P1_PV = 24 if SPLIT else 12   # P.V MFMAs issued among the 36 QK^T MFMAs; the rest cover the softmax
+P1_LEAD = 3                   # P.V MFMAs at the head of an iteration (they cover the first K fragment reads)
 
 # ---- VGPR map
 Q0 = 0

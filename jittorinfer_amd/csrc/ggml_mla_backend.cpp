@@ -69,6 +69,7 @@ struct backend_ctx {
     void *      workspace      = nullptr;
     size_t      workspace_size = 0;
     bool        f16_strict     = false;   // F16 KV: replay ggml-cpu's f16 accumulator instead of accumulating in f32
+    bool        q8_exact       = false;   // Q8_0 KV: the reference's integer block dots and f32 V instead of f16 matrix-core operands (MLA_FLAG_Q8_EXACT)
     bool        bf16_direct    = false;   // BF16 KV: the hi + lo bf16 program instead of the one that converts the tiles to f16 (MLA_FLAG_BF16_DIRECT)
     // The attention nodes of the layers of one graph share their mask (one KQ_mask tensor per graph, src/llama-graph-deepseek2.cpp:99-103):
     // the key extents the first of them leaves in the workspace serve the others (MLA_FLAG_MASK_EXTENTS_VALID).  ext_key: the
@@ -588,7 +589,8 @@ int compute_flash_attn(backend_ctx * ctx, const tensor * dst) {
 
     mla_attn_args a;
     fill_attn_args(dst, &a);
-    if (ctx->f16_strict && k->type == TYPE_F16 && !bt) a.flags |= MLA_FLAG_F16_ACC_STRICT;
+    if (ctx->f16_strict && k->type == TYPE_F16) a.flags |= MLA_FLAG_F16_ACC_STRICT;
+    if (ctx->q8_exact && k->type == TYPE_Q8_0) a.flags |= MLA_FLAG_Q8_EXACT;
     if (ctx->bf16_direct) a.flags |= MLA_FLAG_BF16_DIRECT;
 
     const size_t need = mla_attn_workspace_size(&a);
@@ -766,6 +768,8 @@ backend * device_init_backend(backend_device * dev, const char * params) {
     ctx->name   = dc->name;
     const char * env = getenv("GGML_HIP_MLA_F16_ACC");
     ctx->f16_strict = (params && strstr(params, "f16_acc=strict")) || (env && strcmp(env, "strict") == 0);
+    const char * env_q8 = getenv("GGML_HIP_MLA_Q8");
+    ctx->q8_exact = (params && strstr(params, "q8=exact")) || (env_q8 && strcmp(env_q8, "exact") == 0);
     const char * env_bf = getenv("GGML_HIP_MLA_BF16");
     ctx->bf16_direct = (params && strstr(params, "bf16=direct")) || (env_bf && strcmp(env_bf, "direct") == 0);
     const char * env_ext = getenv("GGML_HIP_MLA_MASK_EXTENTS");   // "rescan": every attention node scans its mask itself

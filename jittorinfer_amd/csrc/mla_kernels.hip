@@ -720,45 +720,113 @@ __global__ void __launch_bounds__(256) mla_attn_combine_f32_wide_kernel(const KP
 }
 
 // ---------------------------------------------------------------------------------------------------------------
-// Strict replay of ggml-cpu's f16 accumulator for F16 KV (ggml-cpu.c:12066-12080 with the x86 F16 vector forms
-// :621-659, :718-765: f32 FMA, result rounded to f16 after every scale and every multiply-add, keys in order).
-// Two small kernels: scores (f32 dot of f16-rounded Q with f16 K), then one block per row walking the keys.
+// Replay of ggml-cpu's own arithmetic, key by key (ggml-cpu.c:12028-12124), for comparisons with the reference's node and for
+// problems too small for operand rounding to average out.  Two kernels: the logits' dots, then one block per row walking the keys.
+//   F16 KV, MLA_FLAG_F16_ACC_STRICT: f32 dot of f16-rounded Q with f16 K; the f16 accumulator of ggml-cpu.c:12066-12080 with the
+//     x86 F16 vector forms :621-659, :718-765 (f32 FMA, result rounded to f16 after every scale and every multiply-add).
+//   Q8_0 KV, MLA_FLAG_Q8_EXACT (and by itself for caches of at most one page per sequence): Q quantized to Q8_0 the way the x86 CPU
+//     backend does it (ggml-cpu-quants.c:855-900), the integer block dots times d_q * d_k of ggml-cpu-quants.c:3814-4241, V = q * d
+//     in f32 (ggml-quants.c:357-373) and the f32 accumulator of ggml-cpu.c:12081-12095 -- no operand is rounded to 16 bits.
+// Both over a contiguous cache or through the block table.
 // ---------------------------------------------------------------------------------------------------------------
-__global__ void mla_f16_scores_kernel(const KParams p, float * scores) {  // grid (ceil(n_kv/4), n_rows, n_seq), block 256
+__device__ __forceinline__ const char * ref_kv_row(const KParams & p, int b, int64_t ic) {
+    if (p.block_table) {
+        const int page = min(max(p.block_table[(int64_t) b * p.bt_stride + (ic >> 7)], 0), p.n_pool_pages - 1);
+        return p.kv + ((int64_t) page * MLA_PAGE_TOKENS + (ic & (MLA_PAGE_TOKENS - 1))) * p.kv_nb1;
+    }
+    return p.kv + ic * p.kv_nb1 + (int64_t) b * p.kv_nb3;
+}
+__device__ __forceinline__ int ref_seq_len(const KParams & p, int b) {
+    return p.block_table ? max(min(p.seq_lens[b], (int) p.bt_stride * MLA_PAGE_TOKENS), 0) : (int) p.n_kv;
+}
+
+// grid (ceil(max_len / 64), n_rows, n_seq), block 256: a wave takes 16 keys; scores[(b * n_rows + row) * max_len + ic]
+template <int KVT>
+__global__ void __launch_bounds__(256) mla_ref_scores_kernel(const KParams p, float * scores, const int64_t max_len) {
+    __shared__ signed char qq[DK];
+    __shared__ float dq[DK / 32];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int ic = blockIdx.x * 4 + wave, row = blockIdx.y, b = blockIdx.z;
-    if (ic >= p.n_kv) return;
+    const int row = blockIdx.y, b = blockIdx.z;
+    const int seq_len = ref_seq_len(p, b);
+    const int ic0 = blockIdx.x * 64 + wave * 16;
+    if (blockIdx.x * 64 >= seq_len) return;   // (uniform over the block)
     const int tq = row / p.n_head, head = row - tq * p.n_head;
     const float * qrow = (const float *) (p.q + (int64_t) tq * p.q_nb1 + (int64_t) head * p.q_nb2 + (int64_t) b * p.q_nb3);
-    const unsigned short * krow = (const unsigned short *) (p.kv + (int64_t) ic * p.kv_nb1 + (int64_t) b * p.kv_nb3);
-    float sum = 0.f;
-    for (int d = lane; d < DK; d += 64) sum += (float) (_Float16) qrow[d] * f16_bits_to_f32(krow[d]);
+    float * out = scores + ((int64_t) b * p.n_rows + row) * max_len;
+    if constexpr (KVT == MLA_TYPE_Q8_0) {
+        // Q -> Q8_0: per block of 32 d = amax / 127 (kept as f16), id = 127 / amax, q = round-half-even(x * id)
+        for (int e = threadIdx.x; e < DK; e += 256) {   // (the 32 lanes of a half wave hold one block)
+            const float x = qrow[e];
+            float amax = fabsf(x);
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
-    if (lane == 0) scores[((int64_t) b * p.n_rows + row) * p.n_kv + ic] = sum;
+            for (int o = 16; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+            const float id = amax != 0.f ? 127.0f / amax : 0.f;
+            qq[e] = (signed char) (int) rintf(x * id);
+            if ((e & 31) == 0) dq[e >> 5] = f16_bits_to_f32(f32_to_f16_bits(amax / 127.0f));
+        }
+        __syncthreads();
+        const int h = lane >> 5, i = lane & 31;
+        for (int k = 0; k < 16; k++) {
+            const int ic = ic0 + k;
+            if (ic >= seq_len) break;
+            const unsigned char * krow = (const unsigned char *) ref_kv_row(p, b, ic);
+            float acc = 0.f;
+#pragma unroll
+            for (int j = 0; j < 9; j++) {
+                const int blk = 2 * j + h;
+                int sumi = (int) qq[blk * 32 + i] * (int) (signed char) krow[blk * 34 + 2 + i];
+#pragma unroll
+                for (int o = 16; o > 0; o >>= 1) sumi += __shfl_xor(sumi, o, 64);
+                const float dk = f16_bits_to_f32(*(const unsigned short *) (krow + blk * 34));
+                acc += (float) sumi * (dq[blk] * dk);
+            }
+            acc += __shfl_xor(acc, 32, 64);
+            if (lane == 0) out[ic] = acc;
+        }
+    } else {
+        for (int k = 0; k < 16; k++) {
+            const int ic = ic0 + k;
+            if (ic >= seq_len) break;
+            const unsigned short * krow = (const unsigned short *) ref_kv_row(p, b, ic);
+            float sum = 0.f;
+            for (int d = lane; d < DK; d += 64) sum += (float) (_Float16) qrow[d] * f16_bits_to_f32(krow[d]);
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
+            if (lane == 0) out[ic] = sum;
+        }
+    }
 }
 
 // One block per output row, one thread per output column; the keys are walked in chunks of STRICT_CHUNK:
 //   (a) the logits of the chunk (scale, softcap, ALiBi slope x mask), one key per thread,
 //   (b) their running maximum by a prefix scan -- the maximum before key k decides which branch ggml-cpu takes at k
 //       and what it feeds expf -- which gives every key its (ms, vs) pair without walking the keys,
-//   (c) the walk itself, per column: acc = f16(acc * ms) where the maximum moved, acc = f16(fma(v, vs, acc)), S = S * ms + vs,
-//       exactly the operations of the reference, in its order; the V values of eight keys are in flight at a time.
+//   (c) the walk itself, per column: acc = acc * ms where the maximum moved, acc = fma(v, vs, acc), S = S * ms + vs, exactly the
+//       operations of the reference, in its order (F16 KV: both results rounded to f16, as its f16 accumulator does); the V values
+//       of eight keys are in flight at a time.
 constexpr int STRICT_CHUNK = 1024;
-__global__ void __launch_bounds__(576) mla_f16_strict_kernel(const KParams p, const float * scores) {  // grid (n_rows, n_seq), block 512 | 576
+template <int KVT>
+__global__ void __launch_bounds__(576) mla_ref_walk_kernel(const KParams p, const float * scores, const int64_t max_len) {  // grid (n_rows, n_seq), block 512 | 576
     __shared__ __attribute__((aligned(16))) float lg[STRICT_CHUNK], pa[STRICT_CHUNK], pb[STRICT_CHUNK];   // logits (-inf: skipped key); scan buffers, then ms / vs
     const int tid = threadIdx.x, nth = blockDim.x, row = blockIdx.x, b = blockIdx.y;
     const int tq = row / p.n_head, head = row - tq * p.n_head;
+    const int n_kv = ref_seq_len(p, b);
     float slope = 1.0f;
     if (p.max_bias > 0.0f) slope = head < p.n_head_log2 ? powf(p.m0, (float) (head + 1)) : powf(p.m1, (float) (2 * (head - p.n_head_log2) + 1));
     const float scale_eff = p.softcap != 0.0f ? p.scale / p.softcap : p.scale;
-    const char * mask_row = p.mask ? p.mask + (int64_t) tq * p.mask_nb1 : nullptr;
-    const float * srow = scores + ((int64_t) b * p.n_rows + row) * p.n_kv;
+    const char * mask_row = p.mask ? p.mask + (int64_t) tq * p.mask_nb1 + (int64_t) b * p.mask_nb3 : nullptr;
+    const float * srow = scores + ((int64_t) b * p.n_rows + row) * max_len;
     const bool col = tid < p.dv_total;
-    const char * vcol = p.kv + (int64_t) b * p.kv_nb3 + 2 * (col ? tid : 0);
+    const int  c   = col ? tid : 0;
+    // where column c sits inside a row, and (Q8_0) where its block's scale does
+    const int voff = KVT == MLA_TYPE_Q8_0 ? (c >> 5) * 34 + 2 + (c & 31) : 2 * c, doff = (c >> 5) * 34;
+    auto value = [&](const char * r) -> float {
+        if constexpr (KVT == MLA_TYPE_Q8_0) return (float) (int) *(const signed char *) (r + voff) * f16_bits_to_f32(*(const unsigned short *) (r + doff));
+        else return f16_bits_to_f32(*(const unsigned short *) (r + voff));
+    };
     float acc = 0.f, S = 0.f, M = -INFINITY;   // M: the maximum over the chunks before this one (the same in every thread)
-    for (int c0 = 0; c0 < (int) p.n_kv; c0 += STRICT_CHUNK) {
-        const int n = min(STRICT_CHUNK, (int) p.n_kv - c0);
+    for (int c0 = 0; c0 < n_kv; c0 += STRICT_CHUNK) {
+        const int n = min(STRICT_CHUNK, n_kv - c0);
         for (int k = tid; k < n; k += nth) {
             const int ic = c0 + k;
             // (a key past the mask's width counts as masked, as in the other kernels)
@@ -798,26 +866,31 @@ __global__ void __launch_bounds__(576) mla_f16_strict_kernel(const KParams p, co
         __syncthreads();
         M = fmaxf(M, m_chunk);
         if (col) {
-            const char * vp = vcol + (int64_t) c0 * p.kv_nb1;
-            unsigned short vn[8];
+            float vn[8];
 #pragma unroll
-            for (int j = 0; j < 8; j++) vn[j] = *(const unsigned short *) (vp + (int64_t) min(j, n - 1) * p.kv_nb1);
+            for (int j = 0; j < 8; j++) vn[j] = value(ref_kv_row(p, b, c0 + min(j, n - 1)));
             for (int k0 = 0; k0 < n; k0 += 8) {
-                unsigned short v8[8];
+                float v8[8];
 #pragma unroll
                 for (int j = 0; j < 8; j++) v8[j] = vn[j];
 #pragma unroll
-                for (int j = 0; j < 8; j++) vn[j] = *(const unsigned short *) (vp + (int64_t) min(k0 + 8 + j, n - 1) * p.kv_nb1);   // the next eight, in flight during this group
+                for (int j = 0; j < 8; j++) vn[j] = value(ref_kv_row(p, b, c0 + min(k0 + 8 + j, n - 1)));   // the next eight, in flight during this group
                 const f32x4 m0 = *(const f32x4 *) (pa + k0), m1 = *(const f32x4 *) (pa + k0 + 4);
                 const f32x4 w0 = *(const f32x4 *) (pb + k0), w1 = *(const f32x4 *) (pb + k0 + 4);
                 const float ms8[8] = { m0.x, m0.y, m0.z, m0.w, m1.x, m1.y, m1.z, m1.w };
                 const float vs8[8] = { w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w };
 #pragma unroll
                 for (int j = 0; j < 8; j++) {
-                    // acc * ms is the identity where the maximum did not move (ms = 1 and acc is an f16 value), so no branch on it
-                    const float scaled = (float) (_Float16) (acc * ms8[j]);
-                    const float next   = (float) (_Float16) fmaf(f16_bits_to_f32(v8[j]), vs8[j], scaled);
-                    const bool  skip   = vs8[j] < 0.0f;
+                    // acc * ms is the identity where the maximum did not move (ms = 1), so no branch on it
+                    float scaled, next;
+                    if constexpr (KVT == MLA_TYPE_F16) {
+                        scaled = (float) (_Float16) (acc * ms8[j]);
+                        next   = (float) (_Float16) fmaf(v8[j], vs8[j], scaled);
+                    } else {
+                        scaled = acc * ms8[j];
+                        next   = fmaf(v8[j], vs8[j], scaled);
+                    }
+                    const bool skip = vs8[j] < 0.0f;
                     acc = skip ? acc : next;
                     S   = skip ? S : S * ms8[j] + vs8[j];
                 }
@@ -827,6 +900,7 @@ __global__ void __launch_bounds__(576) mla_f16_strict_kernel(const KParams p, co
     }
     if (col) p.dst[((int64_t) b * p.n_rows + row) * p.dst_stride + tid] = acc * (1.0f / S);
 }
+
 
 __global__ void __launch_bounds__(256) mla_hbm_copy_kernel(const u32x4 * __restrict__ src, u32x4 * __restrict__ dst, size_t n16) {
     size_t       i      = (size_t) blockIdx.x * 256 + threadIdx.x;
@@ -864,7 +938,8 @@ int validate(const mla_attn_args * a) {
     if (a->dk != DK || (a->dv != 512 && a->dv != 576)) return MLA_ERR_BAD_SHAPE;
     if (a->q_type != MLA_TYPE_F32) return MLA_ERR_BAD_TYPE;
     if (a->kv_type != MLA_TYPE_BF16 && a->kv_type != MLA_TYPE_F16 && a->kv_type != MLA_TYPE_Q8_0) return MLA_ERR_BAD_TYPE;
-    if ((a->flags & MLA_FLAG_F16_ACC_STRICT) && (a->kv_type != MLA_TYPE_F16 || a->block_table)) return MLA_ERR_UNSUPPORTED;
+    if ((a->flags & MLA_FLAG_F16_ACC_STRICT) && a->kv_type != MLA_TYPE_F16) return MLA_ERR_UNSUPPORTED;
+    if ((a->flags & MLA_FLAG_Q8_EXACT) && a->kv_type != MLA_TYPE_Q8_0) return MLA_ERR_UNSUPPORTED;
     if (a->n_kv < 0 || a->n_kv > 0x7fffffff) return MLA_ERR_BAD_SHAPE;
     if ((int64_t) a->n_tok * a->n_head > 0x7fffffff) return MLA_ERR_BAD_SHAPE;
     if (((uintptr_t) a->q & 15) || (a->q_nb1 & 15) || (a->q_nb2 & 15) || (a->q_nb3 & 15)) return MLA_ERR_BAD_ALIGNMENT;
@@ -916,11 +991,15 @@ int make_plan(const mla_attn_args * a, Plan * pl) {
     const int64_t n_rows  = (int64_t) a->n_tok * a->n_head;
     const int64_t max_len = a->block_table ? a->bt_stride * MLA_PAGE_TOKENS : a->n_kv;
     *pl = Plan{};
-    if (a->flags & MLA_FLAG_F16_ACC_STRICT) {
+    // The replay of the reference's own arithmetic (mla_ref_scores_kernel, mla_ref_walk_kernel): asked for by flag, and taken by
+    // itself for a Q8_0 cache of at most one page per sequence -- with so few keys one of them can carry a row, and then the
+    // 16-bit operands the matrix cores are fed (q * d has 19 significant bits) show in single output elements
+    const bool q8_small = a->kv_type == MLA_TYPE_Q8_0 && max_len <= MLA_PAGE_TOKENS && (int64_t) a->n_seq * n_rows <= 16384 && a->rows_per_wg == 0;
+    if ((a->flags & (MLA_FLAG_F16_ACC_STRICT | MLA_FLAG_Q8_EXACT)) || q8_small) {
         pl->variant   = 1;
         pl->n_splits  = 1;
         pl->n_passes  = 1;
-        pl->ws_scores = (size_t) a->n_seq * n_rows * (size_t) (a->n_kv > 0 ? a->n_kv : 1) * sizeof(float);
+        pl->ws_scores = (size_t) a->n_seq * n_rows * (size_t) (max_len > 0 ? max_len : 1) * sizeof(float);
         pl->split_tokens = (int) max_len;
         return 0;
     }
@@ -1134,14 +1213,18 @@ static int launch_phases(const mla_attn_args * a, void * stream, int phases) {
 
     if (pl.variant == 1) {
         if (!(phases & 1)) return 0;
-        if (a->n_kv > 0) {
-            dim3 g1((unsigned) ((a->n_kv + 3) / 4), (unsigned) kp.n_rows, (unsigned) a->n_seq);
-            hipLaunchKernelGGL(mla_f16_scores_kernel, g1, dim3(256), 0, st, kp, scores);
+        const int64_t max_len = a->block_table ? a->bt_stride * MLA_PAGE_TOKENS : a->n_kv;
+        const bool q8 = a->kv_type == MLA_TYPE_Q8_0;
+        if (max_len > 0) {
+            dim3 g1((unsigned) ((max_len + 63) / 64), (unsigned) kp.n_rows, (unsigned) a->n_seq);
+            if (q8) hipLaunchKernelGGL(mla_ref_scores_kernel<MLA_TYPE_Q8_0>, g1, dim3(256), 0, st, kp, scores, max_len);
+            else    hipLaunchKernelGGL(mla_ref_scores_kernel<MLA_TYPE_F16>, g1, dim3(256), 0, st, kp, scores, max_len);
             hipError_t e = hipGetLastError();
             if (e != hipSuccess) return (int) e;
         }
         dim3 g2((unsigned) kp.n_rows, (unsigned) a->n_seq);
-        hipLaunchKernelGGL(mla_f16_strict_kernel, g2, dim3(a->dv == 576 ? 576 : 512), 0, st, kp, (const float *) scores);
+        if (q8) hipLaunchKernelGGL(mla_ref_walk_kernel<MLA_TYPE_Q8_0>, g2, dim3(a->dv == 576 ? 576 : 512), 0, st, kp, (const float *) scores, max_len);
+        else    hipLaunchKernelGGL(mla_ref_walk_kernel<MLA_TYPE_F16>, g2, dim3(a->dv == 576 ? 576 : 512), 0, st, kp, (const float *) scores, max_len);
         return (int) hipGetLastError();
     }
 

@@ -66,6 +66,30 @@ def test_f16_cache_with_the_reference_accumulator_on_request(gpu, monkeypatch):
     assert e_strict[1] < 0.5 * e_fast[1]
 
 
+def test_q8_0_cache_with_the_reference_arithmetic_on_request(gpu, monkeypatch):
+    """Q8_0 KV with block scales of their own (a real quantization of N(0, 3) rows) and a mask that leaves every query token three
+    keys: the matrix-core operands (q * d rounded to f16) show in single elements, the documented deviation of the default path; a
+    backend initialised with q8=exact (here through the environment) runs ggml-cpu's own arithmetic and agrees with the reference's
+    compiled node to 1e-5.  Both against ggml-cpu itself (oracle/_ref), through the plugin interface."""
+    rng = np.random.default_rng(33)
+    n_tok, n_kv = 4, 1024
+    q = (rng.standard_normal((1, 16, n_tok, 576)) * 2).astype(np.float32)
+    k = U.encode_kv((rng.standard_normal((1, n_kv, 576)) * 3).astype(np.float32), O.TYPE_Q8_0)
+    m = np.full((n_tok, n_kv), -np.inf, np.float32)
+    for t in range(n_tok):
+        m[t, rng.choice(n_kv, 3, replace=False)] = 0.0
+    mask = m.astype(np.float16).view(np.uint16)
+    cpu = O.ref_flash_attn_ext(q, k, O.TYPE_Q8_0, mask=mask, scale=U.SCALE)
+    fast, _ = O.ref_backend_flash_attn_ext(_so(), q, k, O.TYPE_Q8_0, dv=576, mask=mask, scale=U.SCALE)
+    monkeypatch.setenv("GGML_HIP_MLA_Q8", "exact")
+    exact, _ = O.ref_backend_flash_attn_ext(_so(), q, k, O.TYPE_Q8_0, dv=576, mask=mask, scale=U.SCALE)
+    e_fast, e_exact = O.errors(fast, cpu), O.errors(exact, cpu)
+    print("vs ggml-cpu: matrix-core operands", e_fast, "reference arithmetic", e_exact)
+    U.check(fast, cpu, "Q8_0 default vs ggml-cpu", max_abs=8e-3)          # values up to 12: 2^-12 of that per element
+    U.check(exact, cpu, "Q8_0 exact vs ggml-cpu", max_abs=2e-5, rel_l2=1e-5)
+    assert e_exact[0] < 0.05 * e_fast[0]
+
+
 @pytest.mark.parametrize("paged", [False, True])
 def test_scheduler_set_up_as_llama_sets_it_up(gpu, paged):
     """The scheduler as the reference's context builds it (src/llama-context-load-utils.cpp:108-131): the CPU backend's

@@ -68,6 +68,90 @@ def test_f16_strict_beyond_one_chunk_with_mask_softcap_alibi(gpu, n_kv, n_tok, d
     print(U.check(got[..., :dv], want, "strict f16, %d keys" % n_kv))
 
 
+def test_f16_strict_through_the_block_table(gpu):
+    """The replay of ggml-cpu's f16 accumulator over a paged F16 cache: ragged lengths (one of them empty-page short, one past a chunk of
+    1024 keys), a shuffled table, unused pages and page tails holding wild values; against the oracle's f16-accumulator form, which is
+    the reference's fused node (oracle/mla_oracle.c)."""
+    import jittorinfer_amd as J
+    rng = np.random.default_rng(41)
+    lens = [300, 1, 1100, 128]
+    pool, bt, seqs = U.make_paged(rng, lens, O.TYPE_F16, n_pool_pages=24)
+    q = rng.standard_normal((4, 8, 2, 576)).astype(np.float32)
+    m = (rng.standard_normal((2, 1152)) * 1.5).astype(np.float32)
+    m[rng.random((2, 1152)) < 0.3] = -np.inf
+    m[:, 0] = 0
+    mask = m.astype(np.float16).view(np.uint16)
+    got = _run(gpu, q, pool, O.TYPE_F16, mask=mask, bt=bt, lens=lens, scale=U.SCALE, flags=J.MLA_FLAG_F16_ACC_STRICT)
+    want = U.oracle_per_seq(q, seqs, O.TYPE_F16, 512, mask=mask)
+    print(U.check(got[..., :512], want, "strict f16, paged"))
+    # and the same data as one contiguous cache per sequence gives the same bits: the gather is exact
+    for b, L in enumerate(lens):
+        one = _run(gpu, q[b:b + 1], seqs[b][None], O.TYPE_F16, mask=np.ascontiguousarray(mask.reshape(2, 1152)[:, :L]), scale=U.SCALE, flags=J.MLA_FLAG_F16_ACC_STRICT)
+        assert np.array_equal(one[0, ..., :512], got[b, ..., :512])
+
+
+@pytest.mark.parametrize("paged", [False, True])
+@pytest.mark.parametrize("dv", [512, 576])
+def test_q8_exact_is_the_reference_arithmetic(gpu, paged, dv):
+    """MLA_FLAG_Q8_EXACT: Q quantized to Q8_0, integer block dots times the two scales, V dequantised to f32, f32 accumulator, keys in
+    order.  Arbitrary block scales (a real quantization of N(0, 3) rows: values up to 12, where the f16 operands of the matrix-core path
+    are off by up to 4e-3 for a key that carries a row), few open keys per row, soft cap and ALiBi: within 2e-5 of the oracle, far inside
+    the stated tolerance."""
+    import jittorinfer_amd as J
+    rng = np.random.default_rng(43 + dv)
+    lens = [200, 1300, 31]
+    n_tok, n_head = 3, 6
+    q = (rng.standard_normal((3, n_head, n_tok, 576)) * 2).astype(np.float32)
+    width = 1408
+    m = (rng.standard_normal((n_tok, width)) * 1.5).astype(np.float32)
+    m[rng.random((n_tok, width)) < 0.97] = -np.inf              # a handful of open keys per token
+    m[:, 5] = 0
+    mask = m.astype(np.float16).view(np.uint16)
+    kw = dict(scale=U.SCALE, max_bias=8.0, logit_softcap=20.0)
+    okw = dict(scale=U.SCALE, max_bias=8.0, softcap=20.0)
+    if paged:
+        pool, bt, seqs = U.make_paged(rng, lens, O.TYPE_Q8_0, n_pool_pages=20, sigma=3.0)
+        got = _run(gpu, q, pool, O.TYPE_Q8_0, dv=dv, mask=mask, bt=bt, lens=lens, flags=J.MLA_FLAG_Q8_EXACT, **kw)
+        want = np.stack([O.flash_attn_ext(q[b:b + 1], seqs[b][None], O.TYPE_Q8_0, dv=dv, mask=np.ascontiguousarray(mask[:, :lens[b]]), **okw)[0] for b in range(3)])
+    else:
+        k = U.encode_kv((rng.standard_normal((3, 1300, 576)) * 3).astype(np.float32), O.TYPE_Q8_0)
+        mk = np.ascontiguousarray(mask[:, :1300])
+        got = _run(gpu, q, k, O.TYPE_Q8_0, dv=dv, mask=mk, flags=J.MLA_FLAG_Q8_EXACT, **kw)
+        want = O.flash_attn_ext(q, k, O.TYPE_Q8_0, dv=dv, mask=mk, **okw)
+    print(U.check(got[..., :dv], want, "Q8_0 exact", max_abs=2e-5, rel_l2=2e-6))
+
+
+def test_q8_caches_of_one_page_take_the_exact_path(gpu):
+    """A Q8_0 cache no sequence of which can hold more than a page: few enough keys for one of them to carry a row, so the launch takes
+    the replay of the reference's arithmetic by itself (variant 1) and meets the stated tolerance at any block scale -- here rows of
+    N(0, 3) with one key made to dominate every row, where the matrix-core operands would be off by several 1e-3."""
+    import torch
+    import jittorinfer_amd as J
+    rng = np.random.default_rng(47)
+    for paged in (False, True):
+        lens = [128, 3, 77] if paged else [77, 77, 77]
+        q = rng.standard_normal((3, 128, 1, 576)).astype(np.float32)
+        kf = [(rng.standard_normal((L, 576)) * 3).astype(np.float32) for L in lens]
+        for b in range(3):
+            kf[b][0] = q[b, 0, 0] * 2.0                     # the first key lines up with the first head's query
+        if paged:
+            pool, bt, _ = U.make_paged(rng, lens, O.TYPE_Q8_0, n_pool_pages=5, sigma=3.0)
+            seqs = [U.encode_kv(x, O.TYPE_Q8_0) for x in kf]
+            for b in range(3):
+                pool[bt[b, 0] * 128:bt[b, 0] * 128 + lens[b]] = seqs[b]
+            info = J.plan(torch.from_numpy(q).to(gpu), torch.from_numpy(pool).to(gpu), O.TYPE_Q8_0, dv=512, scale=U.SCALE,
+                          block_table=torch.from_numpy(bt).to(gpu), seq_lens=torch.tensor(lens, dtype=torch.int32, device=gpu))
+            got = _run(gpu, q, pool, O.TYPE_Q8_0, bt=bt, lens=lens, scale=U.SCALE)
+            want = U.oracle_per_seq(q, seqs, O.TYPE_Q8_0, 512)
+        else:
+            k = U.encode_kv(np.stack(kf), O.TYPE_Q8_0)
+            info = J.plan(torch.from_numpy(q).to(gpu), torch.from_numpy(k).to(gpu), O.TYPE_Q8_0, dv=512, scale=U.SCALE)
+            got = _run(gpu, q, k, O.TYPE_Q8_0, scale=U.SCALE)
+            want = O.flash_attn_ext(q, k, O.TYPE_Q8_0, dv=512, scale=U.SCALE)
+        assert info["variant"] == 1, info
+        print(U.check(got[..., :512], want, "Q8_0, one page", max_abs=2e-5, rel_l2=2e-6))
+
+
 @pytest.mark.parametrize("k_type", [O.TYPE_BF16, O.TYPE_Q8_0])
 def test_config2_paged_decode(gpu, k_type):
     """BASELINE config 2 shape: batch 8, 16 heads, lengths uniform in [512, 4096], 512-page pool, shuffled table."""
