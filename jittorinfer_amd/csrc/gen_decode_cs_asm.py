@@ -47,6 +47,12 @@ FOFF = AOFF + 1024                           # one word per wave: non-zero when 
 CPR = 73                                     # 16-byte chunks per padded row
 WAVE_CHUNKS = 8 * CPR                        # each wave moves rows 8w .. 8w+7 of a tile
 DMA_PER_TILE = 10
+# Tile copies of the unmasked programs carry the non-temporal hint: a decode step reads every key once, and cells streamed through
+# the L2s without the hint push out what is read again -- the operand image the workgroups of a sequence share, the partials the
+# combine pass is about to read (config 3: step 92.4 -> 88.8 us; 128 sequences x 8192 keys, 16 heads: kernel 218 -> 199 us = 6.1 TB/s).
+# The masked programs also run prompt chunks, whose row blocks read the same cells one after the other (config 4 with the hint:
+# 174.8 -> 179.5 us), so theirs stay as they are.
+NT_HINT = "" if MASK else " nt"
 # K fragment ring: five slots of its own, the sixth in T[4:7] (free while K.Q^T runs); mask builds give the last slot of each
 # ring to the mask values
 KRING, PRING = (5, 3) if MASK else (6, 4)
@@ -258,10 +264,10 @@ def dma_tile_lines(tile_sreg, off_sreg, first_page_scalar=False):
             # 8 chunks left per wave: lanes 0..7 only.  One atomic group: nothing may be scheduled inside the exec window.
             L.append("\\n\\t".join(["s_mov_b64 %s, exec" % s(EXS, 2),
                                     "s_mov_b64 exec, 0xff",
-                                    "global_load_lds_dwordx4 %s, %s offset:%d" % (v(t), s(TB, 2), 1024 * c),
+                                    "global_load_lds_dwordx4 %s, %s offset:%d%s" % (v(t), s(TB, 2), 1024 * c, NT_HINT),
                                     "s_mov_b64 exec, %s" % s(EXS, 2)]))
         else:
-            L.append("global_load_lds_dwordx4 %s, %s offset:%d" % (v(t), s(TB, 2), 1024 * c))
+            L.append("global_load_lds_dwordx4 %s, %s offset:%d%s" % (v(t), s(TB, 2), 1024 * c, NT_HINT))
     return L
 
 

@@ -66,6 +66,7 @@ def _parse_instr(ln):
     for k, val in _MOD.findall(rest):
         mods[k] = [int(x) for x in val[1:-1].split(",")] if val.startswith("[") else (int(val, 0) if re.fullmatch(r"-?(0x[0-9a-f]+|\d+)", val) else val)
     rest = _MOD.sub("", rest)
+    rest = re.sub(r"\s+(nt|sc0|sc1)\b", "", rest)       # cache-policy hints of loads and stores: nothing the emulator models
     ops = [_parse_operand(x.strip()) for x in _split_operands(rest) if x.strip()]
     return (mn, ops, mods, ln)
 
