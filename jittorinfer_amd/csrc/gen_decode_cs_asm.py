@@ -30,7 +30,8 @@ CLK = "--clk" in ARGS                        # timing builds: s_memtime stamps l
 MASK = "--mask" in ARGS                      # additive f16 mask rows (one per query token)
 KS = "--ks" in ARGS                          # at most 32 rows: the four waves split the 576 columns of K.Q^T (see ks_main)
 BIAS = "--bias" in ARGS                      # mask builds: ALiBi slope per head on the mask, tanh soft cap on the logits
-assert not (MASK and CLK) and (MASK or not BIAS)
+STREAM = "--stream" in ARGS                  # mask builds: the tile copies carry the non-temporal hint (see NT_HINT)
+assert not (MASK and CLK) and (MASK or not BIAS) and (MASK or not STREAM) and not (BIAS and STREAM)
 MF_QK = "v_mfma_f32_32x32x16_f16" if F16KV else "v_mfma_f32_32x32x16_bf16"
 MF_PV = "v_mfma_f32_32x32x16_f16"
 
@@ -51,8 +52,10 @@ DMA_PER_TILE = 10
 # the L2s without the hint push out what is read again -- the operand image the workgroups of a sequence share, the partials the
 # combine pass is about to read (config 3: step 92.4 -> 88.8 us; 128 sequences x 8192 keys, 16 heads: kernel 218 -> 199 us = 6.1 TB/s).
 # The masked programs also run prompt chunks, whose row blocks read the same cells one after the other (config 4 with the hint:
-# 174.8 -> 179.5 us), so theirs stay as they are.
-NT_HINT = "" if MASK else " nt"
+# 174.8 -> 179.5 us): they come in two builds, and the launcher takes the one with the hint (--stream) when the cache is far larger
+# than the L2s can hold -- the reference's decode batch, whose mask gives every token its own cells of one big cache (config 3 in
+# that form: step 112.2 -> 109.1 us).
+NT_HINT = " nt" if STREAM or not MASK else ""
 # K fragment ring: five slots of its own, the sixth in T[4:7] (free while K.Q^T runs); mask builds give the last slot of each
 # ring to the mask values
 KRING, PRING = (5, 3) if MASK else (6, 4)
@@ -1441,7 +1444,7 @@ def ks_main():
 
 
 def emit():
-    print("// generated by gen_decode_cs_asm.py%s%s%s%s -- do not edit" % (" --ks" if KS else "", " --f16" if F16KV else "", " --mask" if MASK else "", " --bias" if BIAS else ""))
+    print("// generated by gen_decode_cs_asm.py%s%s%s%s%s -- do not edit" % (" --ks" if KS else "", " --f16" if F16KV else "", " --mask" if MASK else "", " --bias" if BIAS else "", " --stream" if STREAM else ""))
     for ln in out:
         print('"%s\\n\\t"' % ln)
     # and nothing of the program is in flight when the compiled code goes on (the mirror image of the wait at the top: an LDS read

@@ -283,7 +283,8 @@ __device__ __forceinline__ void stage_q_rows(const KP & p, int b, int row0, int 
 // leaves it few -- across the program (50 to 150 spilled scalars per kernel; a kernel that holds two bodies does not compile);
 // costs a piece 0.2 to 0.5 us of load latency, so only the kernels with two bodies ask for it.
 typedef const __attribute__((address_space(4))) KParams KParamsArg;
-template <int KVT, bool MASK, int KOFF, bool OPAQUE>
+// STREAM (masked column-split and k-split programs): the build whose tile copies carry the non-temporal hint
+template <int KVT, bool MASK, int KOFF, bool OPAQUE, bool STREAM = false>
 __device__ __forceinline__ void decode_body() {
     KParamsArg * p_ptr = (KParamsArg *) ((const __attribute__((address_space(4))) char *) __builtin_amdgcn_kernarg_segment_ptr() + KOFF);
     KParamsArg & p = *p_ptr;
@@ -595,6 +596,22 @@ __device__ __forceinline__ void decode_body() {
         asm volatile(
 #include "mla_decode_cs_f16_bias.inc"
             : : MLA_DECODE_CS_BIAS_INPUTS : MLA_DECODE_CS_BIAS_CLOBBERS);
+    } else if constexpr (KVT == SRC_BF16_CS && MASK && STREAM) {
+        asm volatile(
+#include "mla_decode_cs_bf16_mask_nt.inc"
+            : : MLA_DECODE_CS_MASK_INPUTS : MLA_DECODE_CS_CLOBBERS);
+    } else if constexpr (KVT == SRC_F16_CS && MASK && STREAM) {
+        asm volatile(
+#include "mla_decode_cs_f16_mask_nt.inc"
+            : : MLA_DECODE_CS_MASK_INPUTS : MLA_DECODE_CS_CLOBBERS);
+    } else if constexpr (KVT == SRC_BF16_KS && MASK && STREAM) {
+        asm volatile(
+#include "mla_decode_ks_bf16_mask_nt.inc"
+            : : MLA_DECODE_CS_BIAS_INPUTS : MLA_DECODE_KS_CLOBBERS);
+    } else if constexpr (KVT == SRC_F16_KS && MASK && STREAM) {
+        asm volatile(
+#include "mla_decode_ks_f16_mask_nt.inc"
+            : : MLA_DECODE_CS_BIAS_INPUTS : MLA_DECODE_KS_CLOBBERS);
     } else if constexpr ((KVT == SRC_BF16_CS || KVT == SRC_BF16_CSQ) && MASK) {
         asm volatile(
 #include "mla_decode_cs_bf16_mask.inc"
@@ -664,8 +681,8 @@ __device__ __forceinline__ void decode_body() {
   }
 }
 
-template <int KVT, bool MASK>
-__global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams) { decode_body<KVT, MASK, 0, false>(); }   // (the body reads the argument segment)
+template <int KVT, bool MASK, bool STREAM = false>
+__global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams) { decode_body<KVT, MASK, 0, false, STREAM>(); }   // (the body reads the argument segment)
 
 // A masked launch of few heads issued in two forms (the launcher's comment tells why): pb describes it as row blocks of 128 rows
 // (balanced == 2), pt token by token (balanced == 3: every query token a sequence of one token, its mask row that sequence's
@@ -673,7 +690,7 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams) { d
 // rows, the k-split program) costs about two thirds of a tile of the row-block form: when the tokens of a row block attend to
 // different cells -- a decode batch -- both forms visit as many tiles in all and the token form wins; when they attend to the same
 // cells -- a prompt chunk of one sequence -- the row-block form visits 128 / n_head times fewer.
-template <int KVT_BLK, int KVT_TOK>
+template <int KVT_BLK, int KVT_TOK, bool STREAM = false>
 __global__ void __launch_bounds__(NTHREADS) mla_decode_dual_kernel(const KParams pb, const KParams pt) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     // (the tile buffers are not in use yet)  tab: tiles and first key of the key range of every token, then of every row block --
@@ -717,8 +734,8 @@ __global__ void __launch_bounds__(NTHREADS) mla_decode_dual_kernel(const KParams
     const bool token_form = pt.n_rows <= 32 ? 2 * (int64_t) tok <= 3 * (int64_t) blk : 16 * (int64_t) tok <= 15 * (int64_t) blk;
     if (blockIdx.x == 0 && t == 0) *pb.form = token_form ? 3 : 2;   // for the combine pass
     static_assert(sizeof(KParams) % 8 == 0, "the second KParams follows the first without padding");
-    if (token_form) decode_body<KVT_TOK, true, (int) sizeof(KParams), true>();
-    else            decode_body<KVT_BLK, true, 0, true>();
+    if (token_form) decode_body<KVT_TOK, true, (int) sizeof(KParams), true, STREAM>();
+    else            decode_body<KVT_BLK, true, 0, true, STREAM>();
 }
 
 // The pairs of n_t query tokens from t0 on (a launch issued in two forms keeps them per token, see below) when the row blocks are
@@ -1084,14 +1101,16 @@ hipError_t launch_q8_to_f16(const char * src, int64_t src_nb1, int64_t src_nb3, 
     return hipGetLastError();
 }
 
-template <int KVT, bool MASK>
+template <int KVT, bool MASK, bool STREAM = false>
 static hipError_t launch_variant(const KParams & kp, dim3 grid, hipStream_t st) {
     static bool attr_done[MLA_MAX_DEVICES];
-    const hipError_t e = raise_lds_limit((const void *) mla_decode_kernel<KVT, MASK>, attr_done);
+    const hipError_t e = raise_lds_limit((const void *) mla_decode_kernel<KVT, MASK, STREAM>, attr_done);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((mla_decode_kernel<KVT, MASK>), grid, dim3(NTHREADS), (size_t) lds_total(KVT), st, kp);
+    hipLaunchKernelGGL((mla_decode_kernel<KVT, MASK, STREAM>), grid, dim3(NTHREADS), (size_t) lds_total(KVT), st, kp);
     return hipGetLastError();
 }
+
+constexpr int64_t STREAM_CACHE_BYTES = 96ll << 20;   // (three times what the eight L2s hold)
 
 static bool decode_cs_applicable(const KParams & kp, int kv_type) {
     if (kv_type != MLA_TYPE_BF16 && kv_type != MLA_TYPE_F16) return false;
@@ -1108,13 +1127,13 @@ static bool decode_ks_applicable(const KParams & kp, int kv_type) {
     return !bias && !kp.bf16_direct && !kp.q_as_q8 && kp.n_rows <= 32 && kp.slot_rows < (1 << 22);
 }
 
-template <int KVT_BLK, int KVT_TOK>
+template <int KVT_BLK, int KVT_TOK, bool STREAM = false>
 static hipError_t launch_dual(const KParams & kb, const KParams & kt, dim3 grid, hipStream_t st) {
     static bool attr_done[MLA_MAX_DEVICES];
-    const hipError_t e = raise_lds_limit((const void *) mla_decode_dual_kernel<KVT_BLK, KVT_TOK>, attr_done);
+    const hipError_t e = raise_lds_limit((const void *) mla_decode_dual_kernel<KVT_BLK, KVT_TOK, STREAM>, attr_done);
     if (e != hipSuccess) return e;
     constexpr int lds = lds_total(KVT_BLK) > lds_total(KVT_TOK) ? lds_total(KVT_BLK) : lds_total(KVT_TOK);
-    hipLaunchKernelGGL((mla_decode_dual_kernel<KVT_BLK, KVT_TOK>), grid, dim3(NTHREADS), (size_t) lds, st, kb, kt);
+    hipLaunchKernelGGL((mla_decode_dual_kernel<KVT_BLK, KVT_TOK, STREAM>), grid, dim3(NTHREADS), (size_t) lds, st, kb, kt);
     return hipGetLastError();
 }
 
@@ -1176,12 +1195,18 @@ hipError_t launch_decode_fast(const KParams & kp_in, int kv_type, dim3 grid, hip
         else
             hipLaunchKernelGGL(mla_mask_extent_kernel, dim3(n_rb, MASK_EXT_CHUNKS, ext_sub), dim3(NTHREADS), 0, st, kp);
     }
+    // Masked launches over a cache far larger than the L2s hold (a decode batch whose mask gives every token its own cells of one big
+    // cache): the builds whose tile copies carry the non-temporal hint.  A prompt chunk re-reads the cells of its sequence from one row
+    // block to the next and wants them kept; its caches are small next to that bound (config 4: 12 MB).
+    const int64_t cache_bytes = kp.block_table ? (int64_t) kp.n_pool_pages * MLA_PAGE_TOKENS * kp.kv_nb1 : kp.n_kv * kp.kv_nb1 * (kp.kv_nb3 ? (int64_t) kp.n_seq_sched : 1);
+    const bool stream = m && cache_bytes > STREAM_CACHE_BYTES;
     if (tok) {
         // the row-block form as chosen above; the token form: the k-split program up to 32 rows of 16-bit cells (it rounds Q itself), else
         // the row-split program of the cache type, whose operand image the pack launch above has written token by token
         KParams kt = *tok;
         kt.q_in_kernel = tok_ks ? 1 : 0;
         if (kv_type == MLA_TYPE_Q8_0) return launch_dual<SRC_Q8, SRC_Q8>(kp, kt, grid, st);
+        if (stream && cs && tok_ks) return kv_type == MLA_TYPE_F16 ? launch_dual<SRC_F16_CS, SRC_F16_KS, true>(kp, kt, grid, st) : launch_dual<SRC_BF16_CS, SRC_BF16_KS, true>(kp, kt, grid, st);
         if (kv_type == MLA_TYPE_F16) {
             if (cs) return tok_ks ? launch_dual<SRC_F16_CS, SRC_F16_KS>(kp, kt, grid, st) : launch_dual<SRC_F16_CS, SRC_F16>(kp, kt, grid, st);
             return tok_ks ? launch_dual<SRC_F16, SRC_F16_KS>(kp, kt, grid, st) : launch_dual<SRC_F16, SRC_F16>(kp, kt, grid, st);
@@ -1190,6 +1215,7 @@ hipError_t launch_decode_fast(const KParams & kp_in, int kv_type, dim3 grid, hip
         return tok_ks ? launch_dual<SRC_BF16_CVT, SRC_BF16_KS>(kp, kt, grid, st) : launch_dual<SRC_BF16_CVT, SRC_BF16_CVT>(kp, kt, grid, st);
     }
     if (kv_type == MLA_TYPE_Q8_0) return m ? launch_variant<SRC_Q8, true>(kp, grid, st) : launch_variant<SRC_Q8, false>(kp, grid, st);
+    if (ks && m && stream) return kv_type == MLA_TYPE_F16 ? launch_variant<SRC_F16_KS, true, true>(kp, grid, st) : launch_variant<SRC_BF16_KS, true, true>(kp, grid, st);
     if (ks && m) return kv_type == MLA_TYPE_F16 ? launch_variant<SRC_F16_KS, true>(kp, grid, st) : launch_variant<SRC_BF16_KS, true>(kp, grid, st);
     if (ks) return kv_type == MLA_TYPE_F16 ? launch_variant<SRC_F16_KS, false>(kp, grid, st) : launch_variant<SRC_BF16_KS, false>(kp, grid, st);
     if (bias) {
@@ -1203,6 +1229,7 @@ hipError_t launch_decode_fast(const KParams & kp_in, int kv_type, dim3 grid, hip
     }
     if (cs && q_in_kernel && kv_type == MLA_TYPE_F16) return m ? launch_variant<SRC_F16_CSQ, true>(kp, grid, st) : launch_variant<SRC_F16_CSQ, false>(kp, grid, st);
     if (cs && q_in_kernel)             return m ? launch_variant<SRC_BF16_CSQ, true>(kp, grid, st) : launch_variant<SRC_BF16_CSQ, false>(kp, grid, st);
+    if (cs && m && stream) return kv_type == MLA_TYPE_F16 ? launch_variant<SRC_F16_CS, true, true>(kp, grid, st) : launch_variant<SRC_BF16_CS, true, true>(kp, grid, st);
     if (cs && kv_type == MLA_TYPE_F16) return m ? launch_variant<SRC_F16_CS, true>(kp, grid, st) : launch_variant<SRC_F16_CS, false>(kp, grid, st);
     if (cs)                            return m ? launch_variant<SRC_BF16_CS, true>(kp, grid, st) : launch_variant<SRC_BF16_CS, false>(kp, grid, st);
     if (kv_type == MLA_TYPE_F16)  return m ? launch_variant<SRC_F16, true>(kp, grid, st) : launch_variant<SRC_F16, false>(kp, grid, st);

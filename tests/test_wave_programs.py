@@ -159,7 +159,8 @@ def test_column_split_programs(name, f16):
     _only_register_loads_ahead_of_tile_copies(cov)
 
 
-@pytest.mark.parametrize("name,f16", [("mla_decode_cs_bf16_mask.inc", False), ("mla_decode_cs_f16_mask.inc", True)])
+@pytest.mark.parametrize("name,f16", [("mla_decode_cs_bf16_mask.inc", False), ("mla_decode_cs_f16_mask.inc", True),
+                                      ("mla_decode_cs_bf16_mask_nt.inc", False), ("mla_decode_cs_f16_mask_nt.inc", True)])
 def test_masked_column_split_programs(name, f16):
     cov = Coverage()
     for k, sc in enumerate(CS_SCENARIOS):
@@ -233,7 +234,8 @@ KS_SCENARIOS = [
 
 
 @pytest.mark.parametrize("name,f16,mask_build", [("mla_decode_ks_bf16.inc", False, False), ("mla_decode_ks_f16.inc", True, False),
-                                                 ("mla_decode_ks_bf16_mask.inc", False, True), ("mla_decode_ks_f16_mask.inc", True, True)])
+                                                 ("mla_decode_ks_bf16_mask.inc", False, True), ("mla_decode_ks_f16_mask.inc", True, True),
+                                                 ("mla_decode_ks_bf16_mask_nt.inc", False, True), ("mla_decode_ks_f16_mask_nt.inc", True, True)])
 def test_k_split_programs(name, f16, mask_build):
     cov = Coverage()
     for k, sc in enumerate(KS_SCENARIOS):
