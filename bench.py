@@ -23,7 +23,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 / fp16 MFMA rate
 KV_ROW_BYTES = 1152     # 576 bf16
 FLOP_PER_TOKEN_HEAD = 2 * 576 + 2 * 512
 # the commit and date at which profiles/mla_decode_kernel_c3_pmc.md's FETCH_SIZE / WRITE_SIZE readings (the `traffic` constants below) were taken
-TRAFFIC_PROFILE_COMMIT = ("e0ae410", "2026-11-25")
+TRAFFIC_PROFILE_COMMIT = ("d9e0b0a", "2026-11-26")
 
 
 def build_workload(dev, n_seq, n_head, ctx, n_pools, seed, kv="bf16"):
@@ -649,7 +649,7 @@ def main():
             traffic_source = ("rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of the decode kernel and of the combine pass, scaled by the copy kernel's readings: "
                               "profiles/mla_decode_kernel_c3_pmc.md (constants of that profile, taken at commit %s on %s, not of this run)" % TRAFFIC_PROFILE_COMMIT)
             # KiB per dispatch, mean: decode kernel (fetch, write), combine pass (fetch, write)
-            d_f, d_w, c_f, c_w = (150524, 34048, 16677, 8192) if a.bf16_direct else (150613, 35584, 16548, 8192)
+            d_f, d_w, c_f, c_w = (150524, 34048, 16677, 8192) if a.bf16_direct else (150520, 34560, 16560, 8192)
             scale_f = 294912 / 147466.0   # the copy kernel reads 294 912 KiB and FETCH_SIZE reports 147 466
             traffic_decode = int(d_f * 1024 * scale_f + d_w * 1024)
             traffic = traffic_decode + int(c_f * 1024 * scale_f + c_w * 1024)

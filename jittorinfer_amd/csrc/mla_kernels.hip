@@ -17,6 +17,7 @@
 //
 // gfx950 only: v_mfma_f32_32x32x16_*, ds_read_b64_tr_b16, 160 KB LDS, 64-wide waves.
 
+#include <atomic>
 #include "mla_common.hpp"
 #include <string.h>
 #include <algorithm>
@@ -915,7 +916,7 @@ __global__ void __launch_bounds__(256) mla_hbm_copy_kernel(const u32x4 * __restr
 // Scratch of mla_attn_launch_static: one copy per device, at the address hipGetSymbolAddress reports there (g_scratch_ptr).
 // In host code the array's name is only a handle for that lookup, never an address.
 static __device__ __align__(256) unsigned char scratch[MLA_ATTN_STATIC_WORKSPACE_MAX];
-static void * g_scratch_ptr[MLA_MAX_DEVICES];
+static std::atomic<void *> g_scratch_ptr[MLA_MAX_DEVICES];   // (per device; threads that look it up together store the same value)
 
 struct Plan {
     int    variant;  // 0 tiled, 1 strict f16
@@ -1324,12 +1325,12 @@ int mla_attn_launch_static(const mla_attn_args * a, void * stream) {
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return (int) e;
     if (dev < 0 || dev >= MLA_MAX_DEVICES) return (int) hipErrorInvalidDevice;
-    void * ptr = g_scratch_ptr[dev];
+    void * ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
     if (!ptr) {   // (two threads that get here together look up the same address)
         e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
         if (e != hipSuccess) return (int) e;
         if (!ptr) return (int) hipErrorInvalidSymbol;
-        g_scratch_ptr[dev] = ptr;
+        g_scratch_ptr[dev].store(ptr, std::memory_order_release);
     }
     mla_attn_args b = *a;
     b.workspace      = nullptr;
