@@ -212,8 +212,9 @@ def front_config(a, dev, lib, J):
 
 def layer_config(a, dev, lib, J):
     """One decode step of one attention layer between the q / kv projections and wo, every node through the C ABI:
-    rope(q_pe) and the absorb product written straight into the 576-wide Q rows, rope(k_pe) in place, the cache write
-    through the block table, paged attention, the un-absorb product written straight into the [token, head*128] rows.
+    rope(q_pe) and the absorb product written straight into the 576-wide Q rows, rope(k_pe) and the cache write through
+    the block table (these in one dispatch, k_pe rotated on its way into the cache; --front separate: a launch each, k_pe
+    rotated in place), paged attention, the un-absorb product written straight into the [token, head*128] rows.
     Config 3's shape (32 sequences, 128 heads, 8191 cached tokens + the new one); wkv_b and the KV pool of 4 layers are
     rotated between steps."""
     import torch
@@ -241,10 +242,19 @@ def layer_config(a, dev, lib, J):
     def step(i, st):
         w = wkv_b[i % layers]
         pool = pools[i % layers].view(torch.int16)
-        J.ggml_rope_ext(q[:, :, 128:], pos, out=q_states[:, :, 512:].permute(1, 0, 2), **rope_kw)
-        J.ggml_rope_ext(k_pe, pos, out=k_pe, **rope_kw)
-        J.ggml_mul_mat(w[:H * 512 * 128].view(H, 512, 128), J.MLA_TYPE_BF16, q[:, :, :128].permute(1, 0, 2), out=q_states[:, :, :512])
-        J.kv_write(kv_new, pool, J.MLA_TYPE_BF16, block_table=bt, seq_ids=seq_ids, positions=pos)
+        if a.front == "batch":
+            # the three independent nodes ahead of the attention node in one dispatch; k_pe is rotated on its way into the cache
+            fb = J.FrontBatch()
+            J.ggml_rope_ext(q[:, :, 128:], pos, out=q_states[:, :, 512:].permute(1, 0, 2), batch=fb, **rope_kw)
+            J.ggml_mul_mat(w[:H * 512 * 128].view(H, 512, 128), J.MLA_TYPE_BF16, q[:, :, :128].permute(1, 0, 2), out=q_states[:, :, :512], batch=fb)
+            J.kv_write(kv_new, pool, J.MLA_TYPE_BF16, block_table=bt, seq_ids=seq_ids, positions=pos, k_pe=kv_new[:, 512:],
+                       rope=dict(pos=pos, **rope_kw), batch=fb)
+            fb.launch(stream=st.value)
+        else:
+            J.ggml_rope_ext(q[:, :, 128:], pos, out=q_states[:, :, 512:].permute(1, 0, 2), **rope_kw)
+            J.ggml_rope_ext(k_pe, pos, out=k_pe, **rope_kw)
+            J.ggml_mul_mat(w[:H * 512 * 128].view(H, 512, 128), J.MLA_TYPE_BF16, q[:, :, :128].permute(1, 0, 2), out=q_states[:, :, :512])
+            J.kv_write(kv_new, pool, J.MLA_TYPE_BF16, block_table=bt, seq_ids=seq_ids, positions=pos)
         rc = lib.mla_attn_launch(C.byref(attn_args[i % layers][0]), st)
         if rc != 0:
             raise RuntimeError("launch failed: %d" % rc)
@@ -278,7 +288,7 @@ def layer_config(a, dev, lib, J):
     print(json.dumps({"metric": "mla_decode_layer_step_bandwidth", "value": nbytes / (ms * 1e-3) / 1e9, "unit": "GB/s", "n_gpus": 1,
                       "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak",
                       "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-                      "config": {"workload": "decode step of one MLA layer, q projection output to wo input: rope x2, absorb, cache write, paged attention (B=%d H=%d ctx=%d bf16), un-absorb; 8 kernel launches" % (B, H, ctx)},
+                      "config": {"workload": "decode step of one MLA layer, q projection output to wo input: rope x2, absorb, cache write, paged attention (B=%d H=%d ctx=%d bf16), un-absorb; %s" % (B, H, ctx, "5 kernel launches (rope of q_pe, absorb and rope of k_pe + cache write in one dispatch)" if a.front == "batch" else "8 kernel launches")},
                       "us_per_step": ms * 1e3, "eager_us_per_step": eager_ms * 1e3, "launch": "hip graph replay of the K steps",
                       "tokens_per_s": B / (ms * 1e-3),
                       "roofline": {"bound": "hbm", "kernel": "whole step", "achieved": nbytes / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
@@ -475,6 +485,7 @@ def main():
     ap.add_argument("--heads", type=int, default=128)
     ap.add_argument("--ctx", type=int, default=8192)
     ap.add_argument("--pools", type=int, default=4, help="distinct KV pools rotated between steps")
+    ap.add_argument("--front", choices=["batch", "separate"], default="batch", help="--config layer: the nodes ahead of the attention node in one dispatch (mla_front_batch_launch), or a launch each")
     ap.add_argument("--splits", type=int, default=0)
     ap.add_argument("--rows-per-wg", type=int, default=0)
     ap.add_argument("--cpu-seqs", type=int, default=32, help="sequences of the workload timed on the host cores (default: the whole step; 0 = skip)")

@@ -116,6 +116,15 @@ int mla_ggml_node_launch_check(const void * ggml_tensor_node);
  * "mask_extents=rescan" in the params of init_backend, turns that off.  For tests and diagnostics. */
 int64_t mla_ggml_mask_extent_reuses(void);
 
+/* no counterpart: the CPY / SCATTER_UPDATE / CONT / CONCAT / ROPE / MUL_MAT nodes this process has computed through
+ * graph_compute, and the dispatches (mla_front_batch_launch calls) they took: graph_compute issues the nodes between
+ * two attention nodes level by level of their dependencies, the independent ones of a level in one dispatch, where the
+ * reference's executors take a pass per node (ggml-cpu.c:15230-15268, ggml-cann.cpp:1761-1800).
+ * GGML_HIP_MLA_BATCH=off, or "batch=off" in the params of init_backend, gives every node a launch of its own.  For
+ * tests and diagnostics. */
+int64_t mla_ggml_front_dispatches(void);
+int64_t mla_ggml_front_nodes(void);
+
 /* no counterpart: frees a buffer obtained from this backend's buffer type when no ggml is present in the process
  * to do it (what ggml_backend_buffer_free does, ggml/src/ggml-backend.cpp). */
 void mla_ggml_buffer_free(void * ggml_backend_buffer);

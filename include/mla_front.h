@@ -84,6 +84,31 @@ typedef struct mla_copy_args {
 int mla_copy_f32_launch(const mla_copy_args * args, void * stream);
 int mla_copy_f32_check(const mla_copy_args * args);     /* as mla_rope_check */
 
+/* Several independent launches of this header and of include/mla_kv_write.h in one dispatch.  The nodes llm_attn_mla and
+ * the DeepSeek-V2 graph put ahead of the attention node of a decode step (src/llama-graph-deepseek2.cpp:216-236,
+ * src/llama-graph-attn.cpp:236-277) move a few MB each; as launches of their own each costs 4 - 5 us however little it
+ * does, and the reference's graph executor has no counterpart to take that away (ggml_backend_sched hands a backend its
+ * nodes as one graph, ggml/src/ggml-backend.cpp:1493-1587; what the backend makes of consecutive nodes is its own
+ * business).  The ops of a batch must be independent: none reads or writes memory that another one writes.  The result
+ * is that of launching them one after the other, in any order.  Ops whose shape has no form inside the batch kernel (a
+ * product with more than 32 rows per matrix: a prefill chunk) are launched on their own by the same call.  All ops are
+ * checked before the first is launched: an error means nothing ran. */
+#define MLA_FRONT_ROPE          0 /* args: const mla_rope_args * */
+#define MLA_FRONT_MUL_MAT       1 /* const mla_mul_mat_args * */
+#define MLA_FRONT_COPY          2 /* const mla_copy_args * */
+#define MLA_FRONT_KV_WRITE      3 /* const mla_kv_write_args *      (include/mla_kv_write.h) */
+#define MLA_FRONT_KV_WRITE_ROPE 4 /* const mla_kv_write_rope_args * (include/mla_kv_write.h) */
+#define MLA_FRONT_BATCH_MAX     8 /* ops per dispatch; a longer list takes several */
+
+typedef struct mla_front_op {
+    int32_t      kind;  /* MLA_FRONT_* */
+    int32_t      _pad;
+    const void * args;
+} mla_front_op;
+
+int mla_front_batch_launch(const mla_front_op * ops, int32_t n_ops, void * stream);
+int mla_front_batch_check(const mla_front_op * ops, int32_t n_ops);   /* as mla_rope_check, for every op */
+
 #ifdef __cplusplus
 }
 #endif

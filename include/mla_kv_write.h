@@ -24,6 +24,8 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include "mla_front.h" /* mla_rope_args */
+
 #ifdef __cplusplus
 extern "C" {
 #endif
@@ -53,6 +55,22 @@ int mla_kv_write_launch(const mla_kv_write_args * args, void * stream);
  * plugin's supports_op (the reference's counterpart: ggml_backend_cann_supports_op, ggml/src/ggml-cann/ggml-cann.cpp:1994-2145).
  * Only the low bits of the addresses are looked at. */
 int mla_kv_write_check(const mla_kv_write_args * args);
+
+/* The cache write with the rotary embedding of the row's last 64 values folded in: what the DeepSeek-V2 graph spells
+ * k_pe = ggml_rope_ext(ggml_cont(k_pe), ...); kv_states = ggml_concat(kv_compressed, k_pe, 0)
+ * (src/llama-graph-deepseek2.cpp:226-236) followed by the copy into the cache (src/llama-graph-attn.cpp:236-241), as one
+ * pass over the new rows: values 0 .. 511 of row t come from `w.src` (f32 rows; only their first 512 values are read),
+ * values 512 .. 575 are rope.src row t ([64, 1, n_tok, 1], f32, 16-byte aligned rows) rotated at rope.pos[t] with the
+ * arithmetic of mla_rope_launch (bit-identical to it), then the row is converted and written as mla_kv_write_launch
+ * writes it.  rope.n_dims must be 64, rope.mode MLA_ROPE_MODE_NORM (the pairing DeepSeek-V2/V3 use), w.src_type
+ * MLA_TYPE_F32; rope.dst is not used: the rotated k_pe exists only in the cache. */
+typedef struct mla_kv_write_rope_args {
+    mla_kv_write_args w;
+    mla_rope_args     rope;
+} mla_kv_write_rope_args;
+
+int mla_kv_write_rope_launch(const mla_kv_write_rope_args * args, void * stream);
+int mla_kv_write_rope_check(const mla_kv_write_rope_args * args);   /* as mla_kv_write_check */
 
 #ifdef __cplusplus
 }

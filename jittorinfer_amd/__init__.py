@@ -5,5 +5,5 @@ fallback: every entry point raises if the library is missing."""
 from .capi import (  # noqa: F401
     MLA_TYPE_BF16, MLA_TYPE_F16, MLA_TYPE_F32, MLA_TYPE_Q8_0, MLA_FLAG_F16_ACC_STRICT, MLA_FLAG_UNIFORM_SPLITS, MLA_FLAG_BF16_DIRECT, MLA_FLAG_MASK_EXTENTS_VALID, MLA_FLAG_Q8_EXACT,
     MlaAttnArgs, MlaPlanInfo, MlaKvWriteArgs, MlaRopeArgs, MlaMulMatArgs, MlaCopyArgs, library, library_path, ggml_flash_attn_ext,
-    kv_write, plan, hbm_copy, PageTable, ggml_rope_ext, ggml_mul_mat, copy_f32, release_workspaces,
+    kv_write, plan, hbm_copy, PageTable, ggml_rope_ext, ggml_mul_mat, copy_f32, release_workspaces, FrontBatch,
 )

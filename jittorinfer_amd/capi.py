@@ -66,9 +66,12 @@ def library():
         lib.mla_hbm_copy_launch.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
         lib.mla_kv_write_launch.restype = C.c_int
         lib.mla_kv_write_launch.argtypes = [C.POINTER(MlaKvWriteArgs), C.c_void_p]
-        for name, cls in (("mla_rope_launch", MlaRopeArgs), ("mla_mul_mat_launch", MlaMulMatArgs), ("mla_copy_f32_launch", MlaCopyArgs)):
+        for name, cls in (("mla_rope_launch", MlaRopeArgs), ("mla_mul_mat_launch", MlaMulMatArgs), ("mla_copy_f32_launch", MlaCopyArgs),
+                          ("mla_kv_write_rope_launch", MlaKvWriteRopeArgs)):
             getattr(lib, name).restype = C.c_int
             getattr(lib, name).argtypes = [C.POINTER(cls), C.c_void_p]
+        lib.mla_front_batch_launch.restype = C.c_int
+        lib.mla_front_batch_launch.argtypes = [C.POINTER(MlaFrontOp), C.c_int32, C.c_void_p]
         lib.mla_page_table_create.restype = C.c_void_p
         lib.mla_page_table_create.argtypes = [C.c_int32] * 3
         lib.mla_page_table_free.argtypes = [C.c_void_p]
@@ -224,22 +227,35 @@ def hbm_copy(src, dst, stream=None):
         raise RuntimeError("mla_hbm_copy_launch failed with code %d" % rc)
 
 
-def kv_write(src, cache, kv_type, *, row0=None, rows=None, block_table=None, seq_ids=None, positions=None, stream=None):
+def kv_write(src, cache, kv_type, *, row0=None, rows=None, block_table=None, seq_ids=None, positions=None, stream=None,
+             k_pe=None, rope=None, batch=None):
     """The KV cache write (ggml_cpy of src/llama-graph-attn.cpp:236-241 / ggml_scatter_update of :380-383) on the current
     torch stream.  src: float32 [n_tok, 576] (converted to the cache type on write) or rows already in the cache type;
     cache: [n_rows, row] in the storage type (row = 1152 or 612 bytes).  Exactly one addressing mode: row0 (consecutive
-    rows), rows (int32/int64 [n_tok] row indices), or block_table + seq_ids + positions (128-token pages)."""
+    rows), rows (int32/int64 [n_tok] row indices), or block_table + seq_ids + positions (128-token pages).
+    k_pe + rope: values 512 .. 575 of every row are k_pe (float32 [n_tok, 64], not yet rotated) rotated on the way
+    (mla_kv_write_rope_launch); rope = dict(pos=..., and the keywords of ggml_rope_ext).  batch: a FrontBatch that takes
+    the launch instead of the stream."""
     import torch
     if not src.is_cuda:
         raise RuntimeError("jittorinfer_amd runs on a gfx950 GPU only (there is no CPU path)")
-    a = MlaKvWriteArgs()
+    ra = None
+    if k_pe is not None:
+        ra = MlaKvWriteRopeArgs()
+        a = ra.w
+        kw = dict(rope)
+        rpos = kw.pop("pos")
+        assert k_pe.dtype == torch.float32 and k_pe.dim() == 2 and k_pe.shape == (src.shape[0], 64) and k_pe.stride(1) == 1
+        _fill_rope_args(ra.rope, k_pe.unsqueeze(1), rpos, k_pe.unsqueeze(1), **kw)
+    else:
+        a = MlaKvWriteArgs()
     a.n_tok = src.shape[0]
     a.kv_type = kv_type
     a.src_type = MLA_TYPE_F32 if src.dtype == torch.float32 else kv_type
     assert src.dim() == 2 and src.stride(1) == 1 and cache.dim() == 2 and cache.stride(1) == 1
     assert cache.shape[1] * cache.element_size() == ROW_BYTES[kv_type]
     if a.src_type == MLA_TYPE_F32:
-        assert src.shape[1] == 576
+        assert src.shape[1] == 576 or (ra is not None and src.shape[1] >= 512)
     else:
         assert src.shape[1] * src.element_size() == ROW_BYTES[kv_type]
     a.src, a.src_nb1 = src.data_ptr(), src.stride(0) * src.element_size()
@@ -256,10 +272,13 @@ def kv_write(src, cache, kv_type, *, row0=None, rows=None, block_table=None, seq
         assert block_table.dim() == 2 and seq_ids.numel() == a.n_tok and positions.numel() == a.n_tok
         a.block_table, a.bt_stride = block_table.data_ptr(), block_table.shape[1]
         a.seq_ids, a.positions = seq_ids.data_ptr(), positions.data_ptr()
+    if batch is not None:
+        batch.add(MLA_FRONT_KV_WRITE_ROPE if ra is not None else MLA_FRONT_KV_WRITE, ra if ra is not None else a)
+        return cache
     st = stream if stream is not None else torch.cuda.current_stream(src.device).cuda_stream
-    rc = library().mla_kv_write_launch(C.byref(a), C.c_void_p(st))
+    rc = library().mla_kv_write_rope_launch(C.byref(ra), C.c_void_p(st)) if ra is not None else library().mla_kv_write_launch(C.byref(a), C.c_void_p(st))
     if rc != 0:
-        raise RuntimeError("mla_kv_write_launch failed with code %d" % rc)
+        raise RuntimeError("mla_kv_write%s_launch failed with code %d" % ("_rope" if ra is not None else "", rc))
     return cache
 
 
@@ -285,6 +304,42 @@ class MlaCopyArgs(C.Structure):
     _fields_ = [("src", C.c_void_p), ("dst", C.c_void_p), ("ne", C.c_int64 * 4), ("src_nb", C.c_int64 * 4), ("dst_nb", C.c_int64 * 4)]
 
 
+class MlaKvWriteRopeArgs(C.Structure):
+    """mla_kv_write_rope_args of include/mla_kv_write.h."""
+    _fields_ = [("w", MlaKvWriteArgs), ("rope", MlaRopeArgs)]
+
+
+class MlaFrontOp(C.Structure):
+    """mla_front_op of include/mla_front.h."""
+    _fields_ = [("kind", C.c_int32), ("_pad", C.c_int32), ("args", C.c_void_p)]
+
+
+MLA_FRONT_ROPE, MLA_FRONT_MUL_MAT, MLA_FRONT_COPY, MLA_FRONT_KV_WRITE, MLA_FRONT_KV_WRITE_ROPE = range(5)
+
+
+class FrontBatch:
+    """Independent launches of ggml_rope_ext / ggml_mul_mat / copy_f32 / kv_write collected (pass batch=...) and issued as one
+    dispatch by launch() (mla_front_batch_launch).  None of them may read or write what another one writes."""
+
+    def __init__(self):
+        self.ops = []
+
+    def add(self, kind, args):
+        self.ops.append((kind, args))
+
+    def launch(self, stream=None, device=None):
+        import torch
+        n = len(self.ops)
+        arr = (MlaFrontOp * max(n, 1))()
+        for i, (kind, args) in enumerate(self.ops):
+            arr[i].kind, arr[i].args = kind, C.addressof(args)
+        st = stream if stream is not None else torch.cuda.current_stream(device).cuda_stream
+        rc = library().mla_front_batch_launch(arr, n, C.c_void_p(st))
+        if rc != 0:
+            raise RuntimeError("mla_front_batch_launch failed with code %d" % rc)
+        self.ops = []
+
+
 def _gpu_only(t):
     if not t.is_cuda:
         raise RuntimeError("jittorinfer_amd runs on a gfx950 GPU only (there is no CPU path)")
@@ -305,8 +360,24 @@ def _nb4(t):
     return ne, nb
 
 
+def _fill_rope_args(a, x, pos, out, *, n_dims, mode=0, n_ctx_orig=0, freq_base=10000.0, freq_scale=1.0, ext_factor=0.0, attn_factor=1.0,
+                    beta_fast=32.0, beta_slow=1.0, freq_factors=None):
+    import torch
+    assert pos.dtype == torch.int32 and pos.is_contiguous() and pos.numel() == x.shape[0]
+    ne, nb = _nb4(x)
+    _, dnb = _nb4(out)
+    a.src, a.dst, a.pos = x.data_ptr(), out.data_ptr(), pos.data_ptr()
+    a.ne[:], a.src_nb[:], a.dst_nb[:] = ne, nb, dnb
+    if freq_factors is not None:
+        assert freq_factors.dtype == torch.float32 and freq_factors.is_contiguous() and freq_factors.numel() >= n_dims // 2
+        a.freq_factors = freq_factors.data_ptr()
+    a.n_dims, a.mode, a.n_ctx_orig = n_dims, mode, n_ctx_orig
+    a.freq_base, a.freq_scale, a.ext_factor, a.attn_factor = freq_base, freq_scale, ext_factor, attn_factor
+    a.beta_fast, a.beta_slow = beta_fast, beta_slow
+
+
 def ggml_rope_ext(x, pos, *, n_dims, mode=0, n_ctx_orig=0, freq_base=10000.0, freq_scale=1.0, ext_factor=0.0, attn_factor=1.0,
-                  beta_fast=32.0, beta_slow=1.0, freq_factors=None, out=None, stream=None):
+                  beta_fast=32.0, beta_slow=1.0, freq_factors=None, out=None, stream=None, batch=None):
     """ggml_rope_ext (ggml/src/ggml.c:3495-3501) on the current torch stream.  x: float32 [n_tok, n_head, ne0] (ggml ne =
     {ne0, n_head, n_tok}), unit stride in the last dimension; pos: int32 [n_tok]; out: same shape (default: a new
     contiguous tensor; pass out=x to rotate in place)."""
@@ -318,23 +389,18 @@ def ggml_rope_ext(x, pos, *, n_dims, mode=0, n_ctx_orig=0, freq_base=10000.0, fr
         out = torch.empty(x.shape, dtype=torch.float32, device=x.device)
     assert out.shape == x.shape and out.dtype == torch.float32 and out.stride(2) == 1
     a = MlaRopeArgs()
-    ne, nb = _nb4(x)
-    _, dnb = _nb4(out)
-    a.src, a.dst, a.pos = x.data_ptr(), out.data_ptr(), pos.data_ptr()
-    a.ne[:], a.src_nb[:], a.dst_nb[:] = ne, nb, dnb
-    if freq_factors is not None:
-        assert freq_factors.dtype == torch.float32 and freq_factors.is_contiguous() and freq_factors.numel() >= n_dims // 2
-        a.freq_factors = freq_factors.data_ptr()
-    a.n_dims, a.mode, a.n_ctx_orig = n_dims, mode, n_ctx_orig
-    a.freq_base, a.freq_scale, a.ext_factor, a.attn_factor = freq_base, freq_scale, ext_factor, attn_factor
-    a.beta_fast, a.beta_slow = beta_fast, beta_slow
+    _fill_rope_args(a, x, pos, out, n_dims=n_dims, mode=mode, n_ctx_orig=n_ctx_orig, freq_base=freq_base, freq_scale=freq_scale,
+                    ext_factor=ext_factor, attn_factor=attn_factor, beta_fast=beta_fast, beta_slow=beta_slow, freq_factors=freq_factors)
+    if batch is not None:
+        batch.add(MLA_FRONT_ROPE, a)
+        return out
     rc = library().mla_rope_launch(C.byref(a), C.c_void_p(_stream(x, stream)))
     if rc != 0:
         raise RuntimeError("mla_rope_launch failed with code %d" % rc)
     return out
 
 
-def ggml_mul_mat(w, w_type, x, *, out=None, stream=None):
+def ggml_mul_mat(w, w_type, x, *, out=None, stream=None, batch=None):
     """ggml_mul_mat(src0 = w, src1 = x) for the absorb products (src/llama-graph-attn.cpp:264-275, :303-317).
     w: [w_ne2, N, K] 16-bit storage (bf16 / f16 bits, any 2-byte dtype), x: float32 [ne2, M, K], unit stride in the
     last dimension of both, ne2 % w_ne2 == 0; returns float32 [ne2, M, N]."""
@@ -353,13 +419,16 @@ def ggml_mul_mat(w, w_type, x, *, out=None, stream=None):
     a.x_nb1, a.x_nb2 = x.stride(1) * 4, x.stride(0) * 4
     a.d_nb1, a.d_nb2 = out.stride(1) * 4, out.stride(0) * 4
     a.w_nb3, a.x_nb3, a.d_nb3 = a.w_nb2 * a.w_ne2, a.x_nb2 * a.ne2, a.d_nb2 * a.ne2
+    if batch is not None:
+        batch.add(MLA_FRONT_MUL_MAT, a)
+        return out
     rc = library().mla_mul_mat_launch(C.byref(a), C.c_void_p(_stream(x, stream)))
     if rc != 0:
         raise RuntimeError("mla_mul_mat_launch failed with code %d" % rc)
     return out
 
 
-def copy_f32(src, dst, stream=None):
+def copy_f32(src, dst, stream=None, batch=None):
     """Strided float32 copy (ggml_cont; each half of ggml_concat): dst[...] = src[...], same shape, any strides with a
     unit last one."""
     import torch
@@ -371,6 +440,9 @@ def copy_f32(src, dst, stream=None):
     _, dnb = _nb4(dst)
     a.src, a.dst = src.data_ptr(), dst.data_ptr()
     a.ne[:], a.src_nb[:], a.dst_nb[:] = ne, nb, dnb
+    if batch is not None:
+        batch.add(MLA_FRONT_COPY, a)
+        return dst
     rc = library().mla_copy_f32_launch(C.byref(a), C.c_void_p(_stream(src, stream)))
     if rc != 0:
         raise RuntimeError("mla_copy_f32_launch failed with code %d" % rc)

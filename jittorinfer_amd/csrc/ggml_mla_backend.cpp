@@ -76,6 +76,8 @@ struct backend_ctx {
     // arguments of the launch whose extents the workspace holds, q / kv / dst blanked; valid inside one graph_compute call, while no
     // node writes the mask and nothing else uses the workspace.
     bool          reuse_mask_extents = true;
+    bool          log_schedule       = false;   // GGML_HIP_MLA_DEBUG=schedule: the levels front_flush issues, on stderr
+    bool          batch_front        = true;    // the nodes around the attention node as dispatches of several nodes each (front_collect / front_flush)
     bool          ext_key_valid      = false;
     mla_attn_args ext_key;
 };
@@ -680,10 +682,210 @@ int compute_front(backend_ctx * ctx, const tensor * dst) {
     return STATUS_SUCCESS;
 }
 
+// ---- the nodes around the attention node, scheduled as dispatches of several nodes each (mla_front_batch_launch)
+//
+// graph_compute collects the run of nodes between two attention nodes, works out which of them depend on which from the
+// memory they read and write, and issues them level by level: all nodes of a level in one dispatch.  The reference's
+// executors run a graph node by node (ggml-cpu: one pass of the thread pool per node, ggml-cpu.c:15230-15268; CANN: one
+// or more aclnn calls per node, ggml-cann.cpp:1761-1800); here a node of a decode step moves a few MB and a launch of its
+// own costs it 4 - 5 us.  Two rewrites shorten the dependency chains; both leave every node's own result where the graph
+// says it is, so that a consumer this backend does not see (another split of ggml_backend_sched) still finds it:
+//  * a ROPE whose source is a CONT of this run reads the CONT's source instead (the kernel takes strided rows; the CONT
+//    still runs, in the same dispatch -- unless the ROPE rotates in place in the CONT's memory, which is where the graph
+//    allocator puts it: then the CONT's result would be overwritten unread and the CONT is left out);
+//  * a cache write (CPY / SCATTER_UPDATE) whose new rows are CONCAT(latent, view of ROPE(k_pe)) reads the latent rows and
+//    the unrotated k_pe and rotates on the way (mla_kv_write_rope_launch: bit-identical to the chain); the ROPE and the
+//    CONCAT still run.
+// Neither is applied when a node between the producer and the consumer writes what the consumer would now read later.
+// The dependencies are those of the memory, not of the graph's edges: the graph allocator (ggml-alloc.c) hands a tensor's
+// memory to a later node once its last consumer in node order has run, so two nodes without an edge between them may
+// still have to keep their order.
+struct mem_range { const char * lo, * hi; };
+inline bool overlaps(const mem_range & a, const mem_range & b) { return a.lo < b.hi && b.lo < a.hi; }
+inline mem_range range_of(const tensor * t) { return mem_range{ (const char *) t->data, (const char *) t->data + tensor_nbytes(t) }; }
+
+struct front_item {
+    const tensor * node;
+    int            n_ops;
+    mla_front_op   ops[2];
+    union { mla_rope_args rope; mla_mul_mat_args mm; mla_copy_args copy; mla_kv_write_args kvw; mla_kv_write_rope_args kvr; } args[2];
+    int            n_reads;
+    mem_range      reads[6];
+    mem_range      write;
+    const tensor * rope_src;   // ROPE items: the tensor the launch reads its rows from (the node's source, or that CONT's source)
+    int            level;
+};
+
+constexpr int FRONT_WINDOW = 64;
+
+std::atomic<int64_t> g_front_dispatches{ 0 }, g_front_nodes{ 0 };
+
+int find_item(const std::vector<front_item> & w, const tensor * node) {
+    for (int i = (int) w.size() - 1; i >= 0; i--) if (w[i].node == node) return i;
+    return -1;
+}
+bool written_after(const std::vector<front_item> & w, int i, const mem_range & r) {
+    for (size_t k = (size_t) i + 1; k < w.size(); k++) if (overlaps(w[k].write, r)) return true;
+    return false;
+}
+
+// Appends `node` to the run; validation as in compute_front / compute_kv_write.
+int front_collect(std::vector<front_item> & w, const tensor * node) {
+    const char * why = nullptr;
+    for (int i = 0; i < 3; i++) if (node->src[i] && !node->src[i]->data) { log_error("node '%s': operands not allocated", node->name); return STATUS_FAILED; }
+    if (!node->data) { log_error("node '%s': destination not allocated", node->name); return STATUS_FAILED; }
+    w.emplace_back();
+    front_item & it = w.back();
+    const int self = (int) w.size() - 1;
+    memset(&it, 0, sizeof(it));
+    it.node = node; it.n_ops = 1; it.write = range_of(node);
+    auto reads = [&](const tensor * t) { if (t && it.n_reads < 6) it.reads[it.n_reads++] = range_of(t); };
+    switch (node->op) {
+        case OP_CONT: {
+            if (!cont_ok(node, &why)) { log_error("CONT node '%s' rejected: %s", node->name, why); return STATUS_FAILED; }
+            fill_cont_args(node, &it.args[0].copy);
+            it.ops[0] = mla_front_op{ MLA_FRONT_COPY, 0, &it.args[0].copy };
+            reads(node->src[0]);
+            break;
+        }
+        case OP_CONCAT: {
+            if (!concat_ok(node, &why)) { log_error("CONCAT node '%s' rejected: %s", node->name, why); return STATUS_FAILED; }
+            const tensor * a = node->src[0], * b = node->src[1];
+            int32_t dim; memcpy(&dim, node->op_params, 4);
+            fill_copy_args(a->data, a->nb, a->ne, node->data, node->nb, &it.args[0].copy);
+            fill_copy_args(b->data, b->nb, b->ne, (char *) node->data + (size_t) a->ne[dim] * node->nb[dim], node->nb, &it.args[1].copy);
+            it.n_ops = 2;
+            it.ops[0] = mla_front_op{ MLA_FRONT_COPY, 0, &it.args[0].copy };
+            it.ops[1] = mla_front_op{ MLA_FRONT_COPY, 0, &it.args[1].copy };
+            reads(a); reads(b);
+            break;
+        }
+        case OP_ROPE: {
+            if (!rope_ok(node, &why)) { log_error("ROPE node '%s' rejected: %s", node->name, why); return STATUS_FAILED; }
+            mla_rope_args & a = it.args[0].rope;
+            fill_rope_args(node, &a);
+            it.rope_src = node->src[0];
+            const tensor * x = node->src[0];
+            const int ci = x->op == OP_CONT ? find_item(w, x) : -1;
+            if (ci >= 0 && ci != self && f32_rows(x->src[0]) && x->src[0]->data) {
+                const tensor * xs = x->src[0];
+                bool same = true;
+                for (int i = 0; i < 4; i++) same = same && xs->ne[i] == x->ne[i];
+                mla_rope_args f = a;
+                f.src = xs->data;
+                for (int i = 0; i < 4; i++) f.src_nb[i] = (int64_t) xs->nb[i];
+                if (same && mla_rope_check(&f) == 0 && !written_after(w, ci, range_of(xs))) {
+                    a = f; it.rope_src = xs;
+                    // the graph allocator lets a ROPE rotate in place (ggml-alloc.c: ggml_op_can_inplace): the CONT's result is
+                    // then overwritten whole by this node, and when nothing in between reads it the CONT has no work left
+                    bool read_between = false;
+                    for (int k = ci + 1; k < self && !read_between; k++)
+                        for (int r = 0; r < w[k].n_reads && !read_between; r++) read_between = overlaps(w[k].reads[r], w[ci].write);
+                    if (node->data == x->data && tensor_nbytes(node) == tensor_nbytes(x) && !read_between) {
+                        w[ci].n_ops = 0; w[ci].n_reads = 0; w[ci].write = mem_range{ nullptr, nullptr };
+                    }
+                }
+            }
+            it.ops[0] = mla_front_op{ MLA_FRONT_ROPE, 0, &a };
+            reads(it.rope_src); reads(node->src[1]); reads(node->src[2]);
+            break;
+        }
+        case OP_MUL_MAT: {
+            if (!mul_mat_ok(node, &why)) { log_error("MUL_MAT node '%s' rejected: %s", node->name, why); return STATUS_FAILED; }
+            fill_mul_mat_args(node, &it.args[0].mm);
+            it.ops[0] = mla_front_op{ MLA_FRONT_MUL_MAT, 0, &it.args[0].mm };
+            reads(node->src[0]); reads(node->src[1]);
+            break;
+        }
+        default: {   // OP_CPY, OP_SCATTER_UPDATE
+            mla_kv_write_args & a = it.args[0].kvw;
+            const tensor * rows;
+            if (node->op == OP_CPY) {
+                if (!kv_cpy_ok(node, &why)) { log_error("CPY node '%s' rejected: %s", node->name, why); return STATUS_FAILED; }
+                fill_kv_cpy_args(node, &a);
+                rows = node->src[0];
+            } else {
+                if (!kv_scatter_ok(node, &why)) { log_error("SCATTER_UPDATE node '%s' rejected: %s", node->name, why); return STATUS_FAILED; }
+                fill_kv_scatter_args(node, &a);
+                rows = node->src[2];
+                it.write = range_of(node->src[0]);
+                reads(node->src[1]);
+            }
+            it.ops[0] = mla_front_op{ MLA_FRONT_KV_WRITE, 0, &a };
+            // new rows = CONCAT(latent [512, n_tok], view of ROPE(k_pe [64, 1, n_tok])): the rope on the way into the cache
+            const int ki = rows->op == OP_CONCAT ? find_item(w, rows) : -1;
+            bool folded = false;
+            if (ki >= 0 && ki != self && rows->type == TYPE_F32) {
+                const tensor * lat = rows->src[0], * pe = rows->src[1];
+                int32_t dim; memcpy(&dim, rows->op_params, 4);
+                size_t off = 0;
+                const tensor * r = pe ? view_root(pe, &off) : nullptr;
+                const int ri = r && r->op == OP_ROPE ? find_item(w, r) : -1;
+                if (dim == 0 && lat && lat->ne[0] == 512 && pe->ne[0] == 64 && ri >= 0 && off == 0 && is_contiguous(r) && r->ne[0] == 64 && r->ne[1] == 1 &&
+                    r->ne[3] == 1 && pe->ne[1] == r->ne[2] && pe->ne[2] == 1 && pe->ne[3] == 1 && pe->nb[1] == 256 && lat->ne[1] == rows->ne[1] && lat->ne[2] == 1 && lat->ne[3] == 1) {
+                    mla_kv_write_rope_args f;
+                    f.w = a;
+                    f.w.src = lat->data; f.w.src_nb1 = (int64_t) lat->nb[1];
+                    f.rope = w[ri].args[0].rope;
+                    const mem_range pe_src = range_of(w[ri].rope_src);
+                    if (mla_kv_write_rope_check(&f) == 0 && !written_after(w, ki, range_of(lat)) && !written_after(w, ri, pe_src) &&
+                        !written_after(w, ri, range_of(r->src[1])) && !(r->src[2] && written_after(w, ri, range_of(r->src[2])))) {
+                        it.args[0].kvr = f;
+                        it.ops[0] = mla_front_op{ MLA_FRONT_KV_WRITE_ROPE, 0, &it.args[0].kvr };
+                        reads(lat); it.reads[it.n_reads++] = pe_src; reads(r->src[1]); reads(r->src[2]);
+                        folded = true;
+                    }
+                }
+            }
+            if (!folded) reads(rows);
+            break;
+        }
+    }
+    it.level = 0;
+    for (int i = 0; i < self; i++) {
+        const front_item & e = w[i];
+        bool dep = overlaps(e.write, it.write);
+        for (int k = 0; k < it.n_reads && !dep; k++) dep = overlaps(e.write, it.reads[k]);
+        for (int k = 0; k < e.n_reads && !dep; k++) dep = overlaps(e.reads[k], it.write);
+        if (dep && e.level + 1 > it.level) it.level = e.level + 1;
+    }
+    return STATUS_SUCCESS;
+}
+
+int front_flush(backend_ctx * ctx, std::vector<front_item> & w) {
+    int max_level = -1;
+    for (const front_item & it : w) if (it.level > max_level) max_level = it.level;
+    if (ctx->log_schedule)
+        for (const front_item & it : w)
+            fprintf(stderr, "ggml-hip-mla: schedule: level %d  op %2d x%d  %-24s writes %p+%zu  reads %p %p %p\n", it.level, it.node->op, it.n_ops, it.node->name,
+                    (const void *) it.write.lo, (size_t) (it.write.hi - it.write.lo), it.n_reads > 0 ? (const void *) it.reads[0].lo : nullptr,
+                    it.n_reads > 1 ? (const void *) it.reads[1].lo : nullptr, it.n_reads > 2 ? (const void *) it.reads[2].lo : nullptr);
+    std::vector<mla_front_op> ops;
+    for (int level = 0; level <= max_level; level++) {
+        ops.clear();
+        for (const front_item & it : w)
+            if (it.level == level)
+                for (int k = 0; k < it.n_ops; k++) ops.push_back(it.ops[k]);
+        if (ops.empty()) continue;
+        const int rc = mla_front_batch_launch(ops.data(), (int32_t) ops.size(), ctx->stream);
+        if (rc != 0) {
+            for (const front_item & it : w) if (it.level == level) log_error("level %d holds node '%s'", level, it.node->name);
+            log_error("mla_front_batch_launch failed: %d", rc);
+            return STATUS_FAILED;
+        }
+        g_front_dispatches++;
+    }
+    g_front_nodes += (int64_t) w.size();
+    w.clear();
+    return STATUS_SUCCESS;
+}
+
 int backend_graph_compute(backend * be, cgraph * g) {
     backend_ctx * ctx = (backend_ctx *) be->context;
     if (!HIP_OK(hipSetDevice(ctx->device))) return STATUS_FAILED;
     ctx->ext_key_valid = false;   // (the mask is an input of the graph: it may have been set anew since the last call)
+    std::vector<front_item> window;
+    window.reserve(FRONT_WINDOW);   // the items hold pointers into themselves: the vector never grows past this
     for (int i = 0; i < g->n_nodes; i++) {
         const tensor * node = g->nodes[i];
         if (is_empty(node) || is_noop(node->op)) continue;
@@ -695,14 +897,20 @@ int backend_graph_compute(backend * be, cgraph * g) {
         }
         int st;
         switch (node->op) {
-            case OP_FLASH_ATTN_EXT: st = compute_flash_attn(ctx, node); break;
-            case OP_CPY: case OP_SCATTER_UPDATE: st = compute_kv_write(ctx, node); break;
-            case OP_CONT: case OP_CONCAT: case OP_ROPE: case OP_MUL_MAT: st = compute_front(ctx, node); break;
+            case OP_FLASH_ATTN_EXT:
+                st = front_flush(ctx, window);
+                if (st == STATUS_SUCCESS) st = compute_flash_attn(ctx, node);
+                break;
+            case OP_CPY: case OP_SCATTER_UPDATE: case OP_CONT: case OP_CONCAT: case OP_ROPE: case OP_MUL_MAT:
+                if (!ctx->batch_front) { st = node->op == OP_CPY || node->op == OP_SCATTER_UPDATE ? compute_kv_write(ctx, node) : compute_front(ctx, node); break; }
+                st = front_collect(window, node);
+                if (st == STATUS_SUCCESS && (int) window.size() == FRONT_WINDOW) st = front_flush(ctx, window);
+                break;
             default: log_error("op %d of node '%s' is not supported", node->op, node->name); return STATUS_FAILED;
         }
         if (st != STATUS_SUCCESS) return st;
     }
-    return STATUS_SUCCESS;
+    return front_flush(ctx, window);
 }
 
 // Events (ggml-backend-impl.h:120-122, :132-135, :183-185; the reference's own: ggml-cann.cpp:2192-2219, :2365-2410): what
@@ -774,6 +982,10 @@ backend * device_init_backend(backend_device * dev, const char * params) {
     ctx->bf16_direct = (params && strstr(params, "bf16=direct")) || (env_bf && strcmp(env_bf, "direct") == 0);
     const char * env_ext = getenv("GGML_HIP_MLA_MASK_EXTENTS");   // "rescan": every attention node scans its mask itself
     ctx->reuse_mask_extents = !((params && strstr(params, "mask_extents=rescan")) || (env_ext && strcmp(env_ext, "rescan") == 0));
+    const char * env_dbg = getenv("GGML_HIP_MLA_DEBUG");
+    ctx->log_schedule = env_dbg && strstr(env_dbg, "schedule");
+    const char * env_batch = getenv("GGML_HIP_MLA_BATCH");   // "off": every node a launch of its own
+    ctx->batch_front = !((params && strstr(params, "batch=off")) || (env_batch && strcmp(env_batch, "off") == 0));
     if (!HIP_OK(hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking))) { delete ctx; return nullptr; }
     return new backend{ &g_guid, k_backend_iface, dev, ctx };
 }
@@ -922,6 +1134,8 @@ void * ggml_backend_init(void) {
 int ggml_backend_score(void) { return gfx950_device_count() > 0 ? 100 : 0; }
 
 int64_t mla_ggml_mask_extent_reuses(void) { return g_mask_extent_reuses.load(); }
+int64_t mla_ggml_front_dispatches(void) { return g_front_dispatches.load(); }
+int64_t mla_ggml_front_nodes(void) { return g_front_nodes.load(); }
 
 void * ggml_backend_hip_mla_reg(void) { return ggml_backend_init(); }
 

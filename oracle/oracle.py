@@ -481,11 +481,13 @@ def ref_mla_unabsorb(kqv, wkv_b, w_type, n_head, so_path=None, n_threads=4):
 
 
 def ref_mla_layer(mode, k_type, w_type, n_head, n_ctx, steps, wkv_b, kq_scale, so_path=None, v_type=TYPE_F16, block_table=None,
-                  n_threads=4):
+                  n_threads=4, rope_in_graph=False):
     """Steps of llm_attn_mla on one KV cache.  mode 0: the unfused graph the reference emits (src/llama-graph-attn.cpp:233-323)
     on its ggml-cpu, with a K cache of k_type and a transposed V cache of v_type; mode 1 / 2: the one-node form on the backend
     plugin at so_path under ggml_backend_sched, the cache written by CPY (1) or as a page pool by SCATTER_UPDATE with a block
     table (2).  steps = [(q f32 [n_tok, n_head, 192], kv_cur f32 [n_tok, 576]), ...], appended to the one sequence in order.
+    rope_in_graph: q_pe and the last 64 values of the kv_cur rows arrive unrotated and the graph holds the model's own
+    cont / rope_ext / view / concat nodes for them (src/llama-graph-deepseek2.cpp:216-236), positions = cache positions.
     Returns (outputs [f32 [n_tok, 128 * n_head] per step], on_backend flags per step, cache bytes after the last step)."""
     n_tok = np.array([q.shape[0] for q, _ in steps], dtype=np.int32)
     kv_head = np.concatenate([[0], np.cumsum(n_tok)[:-1]]).astype(np.int32)
@@ -498,11 +500,11 @@ def ref_mla_layer(mode, k_type, w_type, n_head, n_ctx, steps, wkv_b, kq_scale, s
     where = np.zeros(len(steps), dtype=np.int32)
     cache = np.zeros((n_ctx, 612 if k_type == TYPE_Q8_0 else 1152), dtype=np.uint8)
     bt = None if block_table is None else np.ascontiguousarray(block_table, dtype=np.int32)
-    rc = _ref_front().ref_mla_layer(_so(so_path), mode, k_type, v_type, w_type, n_head, n_ctx, len(steps), n_tok.ctypes.data,
+    rc = _ref_front().ref_mla_layer(_so(so_path), mode | (8 if rope_in_graph else 0), k_type, v_type, w_type, n_head, n_ctx, len(steps), n_tok.ctypes.data,
                                     kv_head.ctypes.data, q.ctypes.data, kv.ctypes.data, wkv_b.ctypes.data, kq_scale,
                                     None if bt is None else bt.ctypes.data, 0 if bt is None else bt.shape[-1], out.ctypes.data,
                                     where.ctypes.data, cache.ctypes.data, n_threads)
     if rc != 0:
-        raise RuntimeError("ref_mla_layer(mode %d) failed: %d" % (mode, rc))
+        raise RuntimeError("ref_mla_layer(mode %d%s) failed: %d" % (mode, ", rope in the graph" if rope_in_graph else "", rc))
     ends = np.cumsum(n_tok)
     return [out[e - n:e] for e, n in zip(ends, n_tok)], where, cache

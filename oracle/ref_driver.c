@@ -538,15 +538,23 @@ int ref_mla_unabsorb(const char * so_path, int w_type, int64_t H, int64_t n_tok,
  * cache_out (may be NULL): the K / latent cache bytes after the last step.
  */
 struct layer_io {
-    struct ggml_tensor *q, *kv_cur, *mask, *idx, *bt, *lens, *out, *write, *fa;
+    struct ggml_tensor *q, *kv_cur, *mask, *idx, *bt, *lens, *out, *write, *fa, *pos;
 };
 
-static struct ggml_tensor * layer_q_states(struct ggml_context * c, struct ggml_tensor * tq, struct ggml_tensor * tw, int64_t H, int64_t n_tok) {
+/* the rotary embedding as the DeepSeek-V2 graph applies it to q_pe and k_pe (src/llama-graph-deepseek2.cpp:216-233): cont of
+ * the view, rope_ext with YaRN parameters (DeepSeek-V2's: n_rot 64, normal pairing, n_ctx_orig 4096, factor 40) */
+static struct ggml_tensor * layer_rope(struct ggml_context * c, struct ggml_tensor * pe, struct ggml_tensor * pos) {
+    pe = ggml_cont(c, pe);
+    return ggml_rope_ext(c, pe, pos, NULL, 64, 0, 4096, 10000.0f, 0.025f, 1.0f, 0.8f, 32.0f, 1.0f);
+}
+
+static struct ggml_tensor * layer_q_states(struct ggml_context * c, struct ggml_tensor * tq, struct ggml_tensor * tw, int64_t H, int64_t n_tok, struct ggml_tensor * pos) {
     const int64_t NOPE = 128, ROPE = 64, LORA = 512;
     struct ggml_tensor * q_nope = ggml_view_3d(c, tq, NOPE, H, n_tok, ggml_row_size(tq->type, NOPE + ROPE), ggml_row_size(tq->type, (NOPE + ROPE) * H), 0);
     struct ggml_tensor * q_pe   = ggml_view_3d(c, tq, ROPE, H, n_tok, ggml_row_size(tq->type, NOPE + ROPE), ggml_row_size(tq->type, (NOPE + ROPE) * H),
                                                ggml_row_size(tq->type, NOPE));
     struct ggml_tensor * wk_b   = ggml_view_3d(c, tw, NOPE, LORA, H, ggml_row_size(tw->type, NOPE), ggml_row_size(tw->type, NOPE * LORA), 0);
+    if (pos) q_pe = layer_rope(c, q_pe, pos);
     q_nope = ggml_mul_mat(c, wk_b, ggml_permute(c, q_nope, 0, 2, 1, 3));
     return ggml_concat(c, q_nope, ggml_permute(c, q_pe, 0, 2, 1, 3), 0); /* [576, n_tok, H] */
 }
@@ -565,6 +573,12 @@ int ref_mla_layer(const char * so_path, int mode, int k_type, int v_type, int w_
                   void * cache_out, int n_threads) {
     const int64_t D = 576, LORA = 512, QW = 192, DV = 128;
     const enum ggml_type kt = (enum ggml_type) k_type, vt = (enum ggml_type) v_type, wt = (enum ggml_type) w_type;
+    /* mode | 8: the rotary embedding is part of the graph, as in the model's graph: q_pe and the last 64 values of the kv_cur
+     * rows arrive unrotated, positions kv_head .. in an I32 tensor, q_pe = rope(cont(view)), k_pe = rope(cont(view)),
+     * kv_states = concat(view of the 512 latent values, view_2d(k_pe)) is what goes into the K / latent cache
+     * (src/llama-graph-deepseek2.cpp:216-236); on_backend bit 5 = every ROPE ran on the loaded backend */
+    const int rope_in_graph = (mode & 8) != 0;
+    mode &= 7;
     if (mode < 0 || mode > 2 || (mode == 2 && (!block_table || n_ctx % 128))) return -1;
     ggml_backend_t be = NULL, cpu = NULL;
     if (mode == 0) {
@@ -604,7 +618,7 @@ int ref_mla_layer(const char * so_path, int mode, int k_type, int v_type, int w_
         int64_t       n_kv  = GGML_PAD(kv_head + n_tok, 32); /* llama_kv_cache_get_padding without flash attention */
         if (n_kv > n_ctx) n_kv = n_ctx;
         if (kv_head + n_tok > n_ctx || (mode == 2 && kv_head + n_tok > max_blocks * 128)) { rc = -2; goto done; }
-        struct ggml_init_params ip = { ggml_tensor_overhead() * 96 + ggml_graph_overhead(), NULL, true };
+        struct ggml_init_params ip = { ggml_tensor_overhead() * 128 + ggml_graph_overhead(), NULL, true };
         g = ggml_init(ip);
         struct ggml_cgraph * gf = ggml_new_graph(g);
         struct layer_io io;
@@ -618,19 +632,28 @@ int ref_mla_layer(const char * so_path, int mode, int k_type, int v_type, int w_
             io.mask = ggml_new_tensor_2d(g, mode == 0 ? GGML_TYPE_F32 : GGML_TYPE_F16, mask_w, GGML_PAD(n_tok, GGML_KQ_MASK_PAD));
             ggml_set_input(io.mask);
         }
+        struct ggml_tensor * kv_states = io.kv_cur;
+        if (rope_in_graph) {
+            io.pos = ggml_new_tensor_1d(g, GGML_TYPE_I32, n_tok);
+            ggml_set_input(io.pos);
+            struct ggml_tensor * k_pe = ggml_view_3d(g, io.kv_cur, 64, 1, n_tok, io.kv_cur->nb[1], io.kv_cur->nb[1], ggml_row_size(GGML_TYPE_F32, LORA));
+            k_pe = layer_rope(g, k_pe, io.pos);
+            k_pe = ggml_view_2d(g, k_pe, 64, n_tok, ggml_row_size(k_pe->type, 64), 0);
+            kv_states = ggml_concat(g, ggml_view_2d(g, io.kv_cur, LORA, n_tok, io.kv_cur->nb[1], 0), k_pe, 0);
+        }
         struct ggml_tensor * k;
         if (mode == 2) {
             io.idx  = ggml_new_tensor_1d(g, GGML_TYPE_I32, n_tok);
             io.bt   = ggml_new_tensor_2d(g, GGML_TYPE_I32, max_blocks, 1);
             io.lens = ggml_new_tensor_1d(g, GGML_TYPE_I32, 1);
             ggml_set_input(io.idx); ggml_set_input(io.bt); ggml_set_input(io.lens);
-            k = io.write = ggml_scatter_update(g, ggml_reshape_2d(g, k_l, D, n_ctx), io.idx, io.kv_cur);
+            k = io.write = ggml_scatter_update(g, ggml_reshape_2d(g, k_l, D, n_ctx), io.idx, kv_states);
         } else {
-            io.write = ggml_cpy(g, io.kv_cur, ggml_view_1d(g, k_l, n_tok * D, ggml_row_size(kt, D) * kv_head));
+            io.write = ggml_cpy(g, kv_states, ggml_view_1d(g, k_l, n_tok * D, ggml_row_size(kt, D) * kv_head));
             ggml_build_forward_expand(gf, io.write);
             k = ggml_view_2d(g, k_l, D, n_kv, ggml_row_size(kt, D), 0);
         }
-        struct ggml_tensor * q_states = layer_q_states(g, io.q, tw, H, n_tok);
+        struct ggml_tensor * q_states = layer_q_states(g, io.q, tw, H, n_tok, io.pos);
         if (mode == 0) {
             struct ggml_tensor * v_cache_view = ggml_view_2d(g, v_l, n_tok, LORA, n_ctx * ggml_element_size(v_l), kv_head * ggml_element_size(v_l));
             struct ggml_tensor * v_cur        = ggml_transpose(g, ggml_view_2d(g, io.kv_cur, LORA, n_tok, ggml_row_size(GGML_TYPE_F32, D), 0));
@@ -665,7 +688,7 @@ int ref_mla_layer(const char * so_path, int mode, int k_type, int v_type, int w_
         } else {
             ggml_backend_sched_reset(sched);
             if (!ggml_backend_sched_alloc_graph(sched, gf)) { rc = -16; goto done; }
-            int32_t where = 0x1c;
+            int32_t where = rope_in_graph ? 0x3c : 0x1c;
             for (int i = 0; i < ggml_graph_n_nodes(gf); i++) {
                 struct ggml_tensor * n  = ggml_graph_node(gf, i);
                 const int            on = ggml_backend_sched_get_tensor_backend(sched, n) == be;
@@ -674,6 +697,7 @@ int ref_mla_layer(const char * so_path, int mode, int k_type, int v_type, int w_
                 if (n->op == GGML_OP_MUL_MAT && !on) where &= ~4;
                 if (n->op == GGML_OP_CONCAT && !on) where &= ~8;
                 if (n->op == GGML_OP_CONT && !on) where &= ~16;
+                if (n->op == GGML_OP_ROPE && !on) where &= ~32;
             }
             if (on_backend) on_backend[s] = where;
         }
@@ -690,6 +714,12 @@ int ref_mla_layer(const char * so_path, int mode, int k_type, int v_type, int w_
                 }
             ggml_backend_tensor_set(io.mask, md, 0, ggml_nbytes(io.mask));
             free(md);
+        }
+        if (io.pos) {
+            int32_t * pp = (int32_t *) malloc(sizeof(int32_t) * n_tok);
+            for (int64_t i = 0; i < n_tok; i++) pp[i] = (int32_t) (kv_head + i);
+            ggml_backend_tensor_set(io.pos, pp, 0, ggml_nbytes(io.pos));
+            free(pp);
         }
         if (mode == 2) {
             int32_t * rows = (int32_t *) malloc(sizeof(int32_t) * n_tok);

@@ -97,3 +97,56 @@ def test_args_struct_matches_header():
         size, off_kv, off_rows, off_pos = map(int, subprocess.run([exe], check=True, capture_output=True, text=True).stdout.split())
     assert C.sizeof(MlaKvWriteArgs) == size
     assert MlaKvWriteArgs.kv.offset == off_kv and MlaKvWriteArgs.rows.offset == off_rows and MlaKvWriteArgs.positions.offset == off_pos
+
+
+def test_rope_and_batch_structs_match_the_headers_and_the_checks_refuse_what_they_should():
+    """mla_kv_write_rope_args / mla_front_op mirrors against the C compiler's view, and the argument checks of
+    mla_kv_write_rope_check / mla_front_batch_check (host code: no GPU needed)."""
+    import jittorinfer_amd as J
+    from jittorinfer_amd.capi import MlaKvWriteRopeArgs, MlaFrontOp, MLA_FRONT_COPY, MLA_FRONT_KV_WRITE_ROPE
+    src = ('#include <stdio.h>\n#include <stddef.h>\n#include "mla_kv_write.h"\nint main(){printf("%zu %zu %zu %zu %d %d\\n", '
+           'sizeof(mla_kv_write_rope_args), offsetof(mla_kv_write_rope_args, rope), sizeof(mla_front_op), offsetof(mla_front_op, args), '
+           'MLA_FRONT_COPY, MLA_FRONT_KV_WRITE_ROPE);return 0;}\n')
+    with tempfile.TemporaryDirectory() as d:
+        c = os.path.join(d, "t.c")
+        exe = os.path.join(d, "t")
+        open(c, "w").write(src)
+        subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), c, "-o", exe], check=True)
+        vals = list(map(int, subprocess.run([exe], check=True, capture_output=True, text=True).stdout.split()))
+    assert vals == [C.sizeof(MlaKvWriteRopeArgs), MlaKvWriteRopeArgs.rope.offset, C.sizeof(MlaFrontOp), MlaFrontOp.args.offset,
+                    MLA_FRONT_COPY, MLA_FRONT_KV_WRITE_ROPE]
+
+    lib = J.library()
+    lib.mla_kv_write_rope_check.argtypes = [C.POINTER(MlaKvWriteRopeArgs)]
+    lib.mla_front_batch_check.argtypes = [C.POINTER(MlaFrontOp), C.c_int32]
+
+    def good():
+        a = MlaKvWriteRopeArgs()
+        a.w.n_tok, a.w.src_type, a.w.kv_type = 5, J.MLA_TYPE_F32, J.MLA_TYPE_BF16
+        a.w.src, a.w.src_nb1, a.w.kv, a.w.kv_nb1, a.w.n_kv_rows = 0x1000, 2048, 0x100000, 1152, 64
+        a.rope.src, a.rope.pos, a.rope.dst = 0x2000, 0x3000, 0x2000
+        a.rope.ne[:], a.rope.src_nb[:], a.rope.dst_nb[:] = [64, 1, 5, 1], [4, 256, 256, 1280], [4, 256, 256, 1280]
+        a.rope.n_dims, a.rope.mode, a.rope.n_ctx_orig, a.rope.freq_base, a.rope.freq_scale = 64, 0, 4096, 10000.0, 1.0
+        a.rope.attn_factor, a.rope.beta_fast, a.rope.beta_slow = 1.0, 32.0, 1.0
+        return a
+    assert lib.mla_kv_write_rope_check(C.byref(good())) == 0
+    for field, value, rc in (("rope.mode", 2, -6), ("rope.n_dims", 32, -1), ("rope.src", 0x2004, -3), ("rope.pos", None, -5),
+                             ("w.src_type", J.MLA_TYPE_BF16, -2), ("w.src_nb1", 1024, -1), ("w.row0", 60, -1)):
+        a = good()
+        obj, name = (a.rope, field[5:]) if field.startswith("rope.") else (a.w, field[2:])
+        setattr(obj, name, value)
+        assert lib.mla_kv_write_rope_check(C.byref(a)) == rc, field
+    a = good()
+    a.rope.ne[2] = 4   # one k_pe row per new token
+    assert lib.mla_kv_write_rope_check(C.byref(a)) == -1
+
+    ops = (MlaFrontOp * 3)()
+    a = good()
+    ops[0].kind, ops[0].args = MLA_FRONT_KV_WRITE_ROPE, C.addressof(a)
+    assert lib.mla_front_batch_check(ops, 1) == 0
+    assert lib.mla_front_batch_check(ops, 0) == 0 and lib.mla_front_batch_check(None, 0) == 0
+    assert lib.mla_front_batch_check(None, 1) == -5 and lib.mla_front_batch_check(ops, -1) == -1
+    ops[1].kind, ops[1].args = 9, C.addressof(a)
+    assert lib.mla_front_batch_check(ops, 2) == -2          # no such kind
+    ops[1].kind, ops[1].args = MLA_FRONT_COPY, None
+    assert lib.mla_front_batch_check(ops, 2) == -5

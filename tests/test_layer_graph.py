@@ -126,3 +126,69 @@ def test_plugin_layer_graph_at_128_heads_across_pages(gpu):
     assert (where == 0x1f).all(), where
     for s, (g, r) in enumerate(zip(got, ref)):
         print("step %d:" % s, U.check(g, r, "128 heads, step %d" % s))
+
+
+@needs_ref
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", [1, 2])
+@pytest.mark.parametrize("k_type", [O.TYPE_BF16, O.TYPE_F16, O.TYPE_Q8_0])
+def test_plugin_layer_graph_with_the_model_s_rope_nodes(gpu, k_type, mode, monkeypatch):
+    """The front of the layer as the DeepSeek-V2 graph spells it (src/llama-graph-deepseek2.cpp:216-236): cont and rope_ext of
+    q_pe and k_pe, view, concat into kv_states, then the cache write -- against the same graph in its unfused form on the
+    reference's ggml-cpu.  The plugin issues these nodes as dispatches of several nodes each, reads the rope sources through the
+    cont nodes and rotates k_pe on its way into the cache; with GGML_HIP_MLA_BATCH=off it launches node by node.  Both ways must
+    agree bit for bit, the first in at most 7 dispatches per step for its 10 nodes."""
+    import jittorinfer_amd as J
+    lib = J.library()
+    lib.mla_ggml_front_dispatches.restype = lib.mla_ggml_front_nodes.restype = __import__("ctypes").c_int64
+    n_head = 16
+    wkv_b, steps = _inputs(16, k_type, n_head)
+    ref, _, ref_cache = O.ref_mla_layer(0, k_type, W_TYPE, n_head, N_CTX, steps, wkv_b, U.SCALE, rope_in_graph=True)
+    bt = np.array([[5, 2, 7, 0]], np.int32) if mode == 2 else None
+    n_ctx = 8 * 128 if mode == 2 else N_CTX
+    d0, n0 = lib.mla_ggml_front_dispatches(), lib.mla_ggml_front_nodes()
+    got, where, cache = O.ref_mla_layer(mode, k_type, W_TYPE, n_head, n_ctx, steps, wkv_b, U.SCALE, so_path=_so(), block_table=bt, rope_in_graph=True)
+    assert (where == 0x3f).all(), where          # cache write, attention node, MUL_MATs, CONCATs, CONTs, ROPEs: all on the plugin
+    assert lib.mla_ggml_front_nodes() - n0 == 10 * len(STEPS)
+    # (13 launches per step node by node: a CONCAT is two.  How far below that the dispatches get is up to the graph allocator,
+    # which reuses the memory of tensors that are dead in node order and so makes later nodes wait for their readers.)
+    assert lib.mla_ggml_front_dispatches() - d0 <= 7 * len(STEPS)
+    monkeypatch.setenv("GGML_HIP_MLA_BATCH", "off")
+    got1, where1, cache1 = O.ref_mla_layer(mode, k_type, W_TYPE, n_head, n_ctx, steps, wkv_b, U.SCALE, so_path=_so(), block_table=bt, rope_in_graph=True)
+    monkeypatch.delenv("GGML_HIP_MLA_BATCH")
+    assert (where1 == 0x3f).all() and lib.mla_ggml_front_nodes() - n0 == 10 * len(STEPS)
+    np.testing.assert_array_equal(cache, cache1)
+    for g, g1 in zip(got, got1):
+        np.testing.assert_array_equal(g.view(np.uint32), g1.view(np.uint32))
+    n = sum(STEPS)
+    rows = cache[5 * 128:5 * 128 + n] if mode == 2 else cache[:n]
+    lat = 16 * 34 if k_type == O.TYPE_Q8_0 else 1024    # bytes of a row that hold the latent part
+    np.testing.assert_array_equal(rows[:, :lat], ref_cache[:n, :lat])
+    # the rope part: cosf / sinf of another libm, so a value may land on the neighbouring code of the cache type
+    assert np.mean(rows[:, lat:] != ref_cache[:n, lat:]) < 5e-3
+    assert rows[:, lat:].any()
+    for s, (g, r) in enumerate(zip(got, ref)):
+        print("step %d (%d tokens):" % (s, g.shape[0]), U.check(g, r, "plugin layer graph with rope nodes vs unfused graph, step %d" % s))
+
+
+@needs_ref
+def test_reference_graph_with_rope_nodes_equals_the_rotation_applied_outside_the_graph():
+    """Pins the rope front of the driver's graphs: the unfused reference graph with cont / rope_ext / concat nodes on unrotated
+    inputs gives, bit for bit, what the same graph gives on inputs rotated beforehand by the oracle's rope (itself bit-exact
+    against the compiled reference)."""
+    k_type, n_head = O.TYPE_F16, 16
+    wkv_b, steps = _inputs(21, k_type, n_head)
+    p = O.rope_params(n_dims=64, mode=0, n_ctx_orig=4096, freq_base=10000.0, freq_scale=0.025, ext_factor=1.0, attn_factor=0.8)
+    rotated, head = [], 0
+    for q, kv in steps:
+        pos = (head + np.arange(q.shape[0])).astype(np.int32)
+        q2, kv2 = q.copy(), kv.copy()
+        q2[:, :, 128:] = O.rope(np.ascontiguousarray(q[:, :, 128:]), pos, p)
+        kv2[:, 512:] = O.rope(np.ascontiguousarray(kv[:, None, 512:]), pos, p)[:, 0]
+        rotated.append((q2, kv2))
+        head += q.shape[0]
+    a, _, cache_a = O.ref_mla_layer(0, k_type, W_TYPE, n_head, N_CTX, steps, wkv_b, U.SCALE, rope_in_graph=True)
+    b, _, cache_b = O.ref_mla_layer(0, k_type, W_TYPE, n_head, N_CTX, rotated, wkv_b, U.SCALE)
+    np.testing.assert_array_equal(cache_a, cache_b)
+    for x, y in zip(a, b):
+        np.testing.assert_array_equal(x.view(np.uint32), y.view(np.uint32))
