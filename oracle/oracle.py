@@ -423,6 +423,9 @@ def _ref_front():
         r.ref_mla_layer.argtypes = [C.c_char_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int64, C.c_int64, C.c_int, C.c_void_p, C.c_void_p,
                                     C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p,
                                     C.c_int]
+        r.ref_random_front.restype = C.c_int
+        r.ref_random_front.argtypes = [C.c_char_p, C.c_uint32, C.c_int64, C.c_int64, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p,
+                                       C.c_void_p, C.c_void_p, C.POINTER(C.c_int32), C.c_int]
         r._front_ready = True
     return r
 
@@ -478,6 +481,24 @@ def ref_mla_unabsorb(kqv, wkv_b, w_type, n_head, so_path=None, n_threads=4):
     if rc != 0:
         raise RuntimeError("ref_mla_unabsorb failed: %d" % rc)
     return out
+
+
+def ref_random_front(seed, n_head, n_tok, n_ops, kv_type, a, b, pos, so_path=None, n_threads=4):
+    """A graph of cont / rope_ext / concat nodes and the k side's rope -> concat -> cpy drawn from `seed` (oracle/ref_driver.c),
+    allocated by ggml's graph allocator, on the reference's ggml-cpu (so_path None) or the backend plugin.  a: f32 [n_tok, n_head,
+    192], b: f32 [n_tok, 576], pos: int32 [n_tok].  Returns (result f32 [n_tok, n_head, 192], cache rows as bytes, nodes)."""
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    b = np.ascontiguousarray(b, dtype=np.float32)
+    pos = np.ascontiguousarray(pos, dtype=np.int32)
+    assert a.shape == (n_tok, n_head, 192) and b.shape == (n_tok, 576) and pos.shape == (n_tok,)
+    out = np.full((n_tok, n_head, 192), np.nan, dtype=np.float32)
+    cache = np.zeros((n_tok, 612 if kv_type == TYPE_Q8_0 else 1152), dtype=np.uint8)
+    n_nodes = C.c_int32(0)
+    rc = _ref_front().ref_random_front(_so(so_path), seed, n_head, n_tok, n_ops, kv_type, a.ctypes.data, b.ctypes.data, pos.ctypes.data,
+                                       out.ctypes.data, cache.ctypes.data, C.byref(n_nodes), n_threads)
+    if rc != 0:
+        raise RuntimeError("ref_random_front(seed %d) failed: %d" % (seed, rc))
+    return out, cache, n_nodes.value
 
 
 def ref_mla_layer(mode, k_type, w_type, n_head, n_ctx, steps, wkv_b, kq_scale, so_path=None, v_type=TYPE_F16, block_table=None,

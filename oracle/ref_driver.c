@@ -752,6 +752,118 @@ done:
     return rc;
 }
 
+/* ------------------------------------------------------------------ generated graphs of the nodes around the attention node
+ *
+ * A graph drawn from `seed` out of the node kinds the model's front uses -- cont of strided views, rope_ext, concat, and the
+ * k side's cont -> rope_ext -> view_2d -> concat -> cpy into a cache of kv_type -- over inputs a = f32 [192, H, T], b = f32
+ * [576, T], pos = i32 [T]; allocated with the graph allocator (ggml_gallocr: a tensor's memory goes to a later node once
+ * its last consumer in node order has run, ggml-alloc.c:553-679), run on the reference's ggml-cpu (so_path NULL) or on the
+ * loaded backend.  out: the final f32 [192, H, T] tensor; cache_out: the T cache rows; n_nodes_out: nodes in the graph.
+ * Deterministic in (seed, H, T, n_ops, kv_type): two calls build the same graph, whichever executor runs it. */
+static uint32_t rg_next(uint32_t * st) { *st = *st * 1664525u + 1013904223u; return *st >> 8; }
+
+int ref_random_front(const char * so_path, uint32_t seed, int64_t H, int64_t T, int n_ops, int kv_type, const float * a_in,
+                     const float * b_in, const int32_t * pos_in, float * out, void * cache_out, int32_t * n_nodes_out, int n_threads) {
+    ggml_backend_t be = NULL;
+    if (so_path) {
+        ggml_backend_reg_t reg = ggml_backend_load(so_path);
+        if (!reg) return -10;
+        if (ggml_backend_reg_dev_count(reg) < 1) return -11;
+        be = ggml_backend_dev_init(ggml_backend_reg_dev_get(reg, 0), NULL);
+    } else {
+        be = ggml_backend_cpu_init();
+        if (be) ggml_backend_cpu_set_n_threads(be, n_threads);
+    }
+    if (!be) return -12;
+    int rc = 0;
+    const enum ggml_type kt = (enum ggml_type) kv_type;
+    struct ggml_init_params ipk = { ggml_tensor_overhead() * 4, NULL, true };
+    struct ggml_context *   ck  = ggml_init(ipk);
+    struct ggml_tensor *    cache = ggml_new_tensor_1d(ck, kt, 576 * T);
+    ggml_backend_buffer_t   bufk = ggml_backend_alloc_ctx_tensors(ck, be);
+    struct ggml_init_params ip = { ggml_tensor_overhead() * (size_t) (8 * n_ops + 64) + ggml_graph_overhead(), NULL, true };
+    struct ggml_context *   c  = ggml_init(ip);
+    struct ggml_cgraph *    gf = ggml_new_graph(c);
+    ggml_gallocr_t          ga = NULL;
+    if (!bufk) { rc = -13; goto done; }
+    ggml_backend_buffer_clear(bufk, 0);
+    {
+        struct ggml_tensor * ta = ggml_new_tensor_3d(c, GGML_TYPE_F32, 192, H, T);
+        struct ggml_tensor * tb = ggml_new_tensor_2d(c, GGML_TYPE_F32, 576, T);
+        struct ggml_tensor * tp = ggml_new_tensor_1d(c, GGML_TYPE_I32, T);
+        ggml_set_input(ta); ggml_set_input(tb); ggml_set_input(tp);
+#define RG_ROPE(x) ggml_rope_ext(c, (x), tp, NULL, 64, 0, 4096, 10000.0f, 0.025f, 1.0f, 0.8f, 32.0f, 1.0f)
+#define RG_VIEW(src, w, off) ggml_view_3d(c, (src), (w), H, T, (src)->nb[1], (src)->nb[2], (size_t) (off) * 4)
+        enum { CAP = 256 };
+        struct ggml_tensor * w64[CAP], * w128[CAP], * w192[CAP];
+        int n64 = 0, n128 = 0, n192 = 0;
+        uint32_t st = seed * 2654435761u + 12345u;
+        w192[n192++] = ta;
+        for (int i = 0; i < n_ops && n64 < CAP - 2 && n128 < CAP - 2 && n192 < CAP - 2; i++) {
+            int kind = (int) (rg_next(&st) % 7);
+            if ((kind == 1 || kind == 3) && n64 == 0) kind = 0;
+            if (kind == 4 && (n128 == 0 || n64 == 0)) kind = n64 ? 3 : 0;
+            if (kind == 6 && n128 == 0) kind = 5;
+            switch (kind) {
+                case 0: {   /* cont of a 64-wide view of a wider tensor */
+                    const int wide = n128 && (rg_next(&st) & 1);
+                    struct ggml_tensor * src = wide ? w128[rg_next(&st) % n128] : w192[rg_next(&st) % n192];
+                    const int slots = wide ? 2 : 3;
+                    w64[n64++] = ggml_cont(c, RG_VIEW(src, 64, 64 * (rg_next(&st) % slots)));
+                    break;
+                }
+                case 1: w64[n64++] = RG_ROPE(w64[rg_next(&st) % n64]); break;
+                case 2: {   /* the model's pair: rope of the cont of a view */
+                    struct ggml_tensor * src = w192[rg_next(&st) % n192];
+                    w64[n64++] = RG_ROPE(ggml_cont(c, RG_VIEW(src, 64, 64 * (rg_next(&st) % 3))));
+                    break;
+                }
+                case 3: w128[n128++] = ggml_concat(c, w64[rg_next(&st) % n64], w64[rg_next(&st) % n64], 0); break;
+                case 4:
+                    if (rg_next(&st) & 1) w192[n192++] = ggml_concat(c, w128[rg_next(&st) % n128], w64[rg_next(&st) % n64], 0);
+                    else                  w192[n192++] = ggml_concat(c, w64[rg_next(&st) % n64], w128[rg_next(&st) % n128], 0);
+                    break;
+                case 5: w128[n128++] = ggml_cont(c, RG_VIEW(w192[rg_next(&st) % n192], 128, 64 * (rg_next(&st) % 2))); break;
+                default: w64[n64++] = RG_ROPE(RG_VIEW(w128[rg_next(&st) % n128], 64, 64 * (rg_next(&st) % 2))); break;   /* rope of a strided view */
+            }
+        }
+        /* the k side, written into the cache the way llm_attn_mla does it, ahead of the rest (src/llama-graph-attn.cpp:236-241) */
+        struct ggml_tensor * k_pe = ggml_view_3d(c, tb, 64, 1, T, tb->nb[1], tb->nb[1], 512 * 4);
+        k_pe = RG_ROPE(ggml_cont(c, k_pe));
+        k_pe = ggml_view_2d(c, k_pe, 64, T, ggml_row_size(GGML_TYPE_F32, 64), 0);
+        struct ggml_tensor * kv_states = ggml_concat(c, ggml_view_2d(c, tb, 512, T, tb->nb[1], 0), k_pe, 0);
+        ggml_build_forward_expand(gf, ggml_cpy(c, kv_states, ggml_view_1d(c, cache, 576 * T, 0)));
+        /* the result: the three newest tensors of each width, folded into one of 192 */
+        struct ggml_tensor * p64  = n64 ? w64[n64 - 1] : ggml_cont(c, RG_VIEW(ta, 64, 128));
+        struct ggml_tensor * p128 = n128 ? w128[n128 - 1] : ggml_cont(c, RG_VIEW(ta, 128, 0));
+        struct ggml_tensor * res  = ggml_concat(c, p128, p64, 0);
+        if (n192 > 1) res = ggml_concat(c, ggml_cont(c, RG_VIEW(w192[n192 - 1], 128, 64)), ggml_cont(c, RG_VIEW(res, 64, 64 * (rg_next(&st) % 3))), 0);
+        ggml_set_output(res);
+        ggml_build_forward_expand(gf, res);
+#undef RG_ROPE
+#undef RG_VIEW
+        if (n_nodes_out) *n_nodes_out = ggml_graph_n_nodes(gf);
+        for (int i = 0; i < ggml_graph_n_nodes(gf); i++)
+            if (!ggml_backend_supports_op(be, ggml_graph_node(gf, i))) { rc = -100 - i; goto done; }
+        ga = ggml_gallocr_new(ggml_backend_get_default_buffer_type(be));
+        if (!ga || !ggml_gallocr_alloc_graph(ga, gf)) { rc = -14; goto done; }
+        ggml_backend_tensor_set(ta, a_in, 0, ggml_nbytes(ta));
+        ggml_backend_tensor_set(tb, b_in, 0, ggml_nbytes(tb));
+        ggml_backend_tensor_set(tp, pos_in, 0, ggml_nbytes(tp));
+        const enum ggml_status gs = ggml_backend_graph_compute(be, gf);
+        if (gs != GGML_STATUS_SUCCESS) { rc = (int) gs ? (int) gs : -15; goto done; }
+        ggml_backend_tensor_get(res, out, 0, ggml_nbytes(res));
+        if (cache_out) ggml_backend_tensor_get(cache, cache_out, 0, ggml_nbytes(cache));
+    }
+done:
+    if (ga) ggml_gallocr_free(ga);
+    ggml_free(c);
+    if (bufk) ggml_backend_buffer_free(bufk);
+    ggml_free(ck);
+    ggml_backend_free(be);
+    return rc;
+}
+
 void ref_quantize_q8_0_ref(const float * x, void * y, int64_t k) { quantize_row_q8_0_ref(x, (block_q8_0 *) y, k); }
 void ref_quantize_q8_0_cpu(const float * x, void * y, int64_t k) { quantize_row_q8_0(x, y, k); }
 void ref_dequantize_q8_0(const void * x, float * y, int64_t k) { dequantize_row_q8_0((const block_q8_0 *) x, y, k); }

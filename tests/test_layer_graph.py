@@ -192,3 +192,43 @@ def test_reference_graph_with_rope_nodes_equals_the_rotation_applied_outside_the
     np.testing.assert_array_equal(cache_a, cache_b)
     for x, y in zip(a, b):
         np.testing.assert_array_equal(x.view(np.uint32), y.view(np.uint32))
+
+
+@needs_ref
+@pytest.mark.gpu
+@pytest.mark.parametrize("k_type", [O.TYPE_BF16, O.TYPE_Q8_0])
+def test_generated_graphs_of_front_nodes_scheduled_by_levels(gpu, k_type, monkeypatch):
+    """Graphs of cont / rope_ext / concat nodes (with the model's cont -> rope pairs, ropes of strided views, and the k side's
+    rope -> view -> concat -> cpy) drawn from a seed and laid out by ggml's graph allocator, which reuses dead tensors' memory:
+    the plugin's level schedule (dispatches of several nodes, reads through CONT nodes, the rope folded into the cache write) must
+    give, bit for bit, what it gives node by node, and both what the reference's ggml-cpu gives for the same graph (rope: cosf /
+    sinf of another libm, 4e-6 relative to the largest value per rope a value went through)."""
+    import ctypes
+    import jittorinfer_amd as J
+    lib = J.library()
+    lib.mla_ggml_front_dispatches.restype = lib.mla_ggml_front_nodes.restype = ctypes.c_int64
+    rng = np.random.default_rng(77)
+    saved = 0
+    for seed in range(40):
+        n_head, n_tok, n_ops = int(rng.integers(1, 20)), int(rng.integers(1, 40)), int(rng.integers(4, 40))
+        a = rng.standard_normal((n_tok, n_head, 192)).astype(np.float32)
+        b = rng.standard_normal((n_tok, 576)).astype(np.float32)
+        pos = rng.integers(0, 100000, size=n_tok).astype(np.int32)
+        ref, ref_cache, n_nodes = O.ref_random_front(seed, n_head, n_tok, n_ops, k_type, a, b, pos)
+        d0, n0 = lib.mla_ggml_front_dispatches(), lib.mla_ggml_front_nodes()
+        got, cache, _ = O.ref_random_front(seed, n_head, n_tok, n_ops, k_type, a, b, pos, so_path=_so())
+        d1, n1 = lib.mla_ggml_front_dispatches(), lib.mla_ggml_front_nodes()
+        monkeypatch.setenv("GGML_HIP_MLA_BATCH", "off")
+        got1, cache1, _ = O.ref_random_front(seed, n_head, n_tok, n_ops, k_type, a, b, pos, so_path=_so())
+        monkeypatch.delenv("GGML_HIP_MLA_BATCH")
+        assert lib.mla_ggml_front_nodes() == n1            # node by node: the scheduler is not in the way
+        np.testing.assert_array_equal(got.view(np.uint32), got1.view(np.uint32), err_msg="seed %d" % seed)
+        np.testing.assert_array_equal(cache, cache1, err_msg="seed %d" % seed)
+        assert not np.isnan(got).any()
+        tol = 4e-6 * n_ops * max(1.0, float(np.abs(ref).max()))
+        assert float(np.abs(got - ref).max()) <= tol, (seed, float(np.abs(got - ref).max()), tol)
+        lat = 16 * 34 if k_type == O.TYPE_Q8_0 else 1024
+        np.testing.assert_array_equal(cache[:, :lat], ref_cache[:, :lat])
+        assert np.mean(cache[:, lat:] != ref_cache[:, lat:]) < 2e-2
+        saved += (n1 - n0) - (d1 - d0)
+    assert saved > 40, saved      # dispatches saved over the 40 graphs
