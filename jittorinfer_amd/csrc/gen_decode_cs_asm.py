@@ -442,7 +442,9 @@ def p_write_items():
 
 def bias_block():
     """Bias builds, once the scores of a tile are complete: S <- s * scale, or, with a soft cap, -2 softcap / (1 + 2^(s K1))
-    (= softcap * tanh(s * scale / softcap) - softcap).  Not in the shadow of MFMAs: the two forms are a branch apart."""
+    (= softcap * tanh(s * scale / softcap) - softcap).  Not in the shadow of MFMAs: the two forms are a branch apart.  Ahead of
+    mask_tail(): the cap is bounded, so a key past the end of the sequence that was already at -inf would come back with a finite
+    logit (and count, wherever the caller's mask says nothing about the cells past the end of a paged sequence)."""
     lab_plain, lab_done = label("nocap"), label("capd")
     e("s_cmp_eq_u32 %s, 0" % s(K2))
     e("s_cbranch_scc1 %s" % lab_plain)
@@ -670,11 +672,11 @@ def iteration(resc, lab_loop):
 
     def qk_done():
         e("s_nop 1")                    # the last K.Q^T MFMA has written S: two P.V MFMAs (8 passes each) were issued behind it
+        if BIAS:
+            bias_block()                # (ahead of mask_tail: the soft cap maps -inf to a finite value)
         mask_tail()
         if MASK:
             mask_wait()
-        if BIAS:
-            bias_block()
 
     def p_read_by_all():
         # every P^T fragment of tile IT is in this wave's registers before any wave overwrites P
@@ -953,9 +955,9 @@ def main():
     e("s_min_u32 %s, %s, 32" % (s(NVAL), s(NVAL)))
     e("s_nop 7")
     e("s_nop 7")
-    mask_tail()
     if BIAS:
         bias_block()
+    mask_tail()
     for ln in softmax_lines(first_tile=True):
         e(ln)
     for it_ in p_write_items():
@@ -1205,6 +1207,8 @@ def ks_tail(first_tile, resc):
     accumulators rescaled if some row's maximum moved."""
     for ln in ks_sum_lines():
         e(ln)
+    if BIAS:
+        bias_block()
     mask_tail()
     for ln in softmax_lines(first_tile=first_tile):
         e(ln)
@@ -1266,7 +1270,7 @@ def ks_q_round(behind):
 
 
 def ks_main():
-    assert not CLK and not BIAS
+    assert not CLK and (MASK or not BIAS)
     prologue_head(ks_q_issue)
     e("s_mul_i32 %s, %s, 288" % (s(S0), s(WAVE)))                      # this wave's k-steps 9 w ..: 32 bytes each
     e("v_add_u32 %s, %s, %s" % (v(KADDR_LANE), s(S0), v(KADDR_LANE)))
@@ -1325,8 +1329,14 @@ def ks_main():
         e("s_lshl_b32 %s, %s, 11" % (s(S0), s(WAVE)))
         e("s_add_u32 %s, %s, 0x%x" % (s(S0), s(S0), HOFF))
         e("v_add_u32 %s, %s, %s" % (v(MOFF), s(S0), v(MOFF)))
+        if BIAS:
+            # the last 8 bytes of the record: the row's slope, and -2 softcap (NPP's register: the page ids are clamped)
+            e("ds_read_b64 %s, %s offset:24" % (v(DT[0], 2), v(MOFF)))
         e("ds_read_b32 %s, %s" % (v(MOFF), v(MOFF)))
         e("s_waitcnt lgkmcnt(0)")
+        if BIAS:
+            e("v_mov_b32 %s, %s" % (v(SLOPE), v(DT[0])))
+            e("v_readfirstlane_b32 %s, %s" % (s(K2), v(DT[1])))
         e("s_mov_b32 %s, 0" % s(TMP))
         mask_loads(TMP)
     lab_no2 = label("no2")

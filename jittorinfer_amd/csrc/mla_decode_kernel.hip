@@ -23,7 +23,8 @@ namespace {
 // 32 bytes per thread: mask offset, out pointer, (m,l) pointer, 8 bytes for the bias builds (slope, soft cap)
 // The column-split programs (SRC_*_CS) keep behind the four tiles: the P^T exchange buffer (8 KB; the hand-off records share it, they
 // are read before P is first written), the rescale factors (1 KB) and the waves' flag words (64 bytes).
-constexpr bool is_cs(int kvt) { return kvt == SRC_BF16_CS || kvt == SRC_F16_CS || kvt == SRC_BF16_KS || kvt == SRC_F16_KS || kvt == SRC_BF16_CSQ || kvt == SRC_F16_CSQ || kvt == SRC_BF16_CSB || kvt == SRC_F16_CSB; }
+constexpr bool is_ks(int kvt) { return kvt == SRC_BF16_KS || kvt == SRC_F16_KS || kvt == SRC_BF16_KSB || kvt == SRC_F16_KSB; }
+constexpr bool is_cs(int kvt) { return kvt == SRC_BF16_CS || kvt == SRC_F16_CS || is_ks(kvt) || kvt == SRC_BF16_CSQ || kvt == SRC_F16_CSQ || kvt == SRC_BF16_CSB || kvt == SRC_F16_CSB; }
 constexpr int handoff_off(int kvt) { return kvt == SRC_Q8 ? 3 * TILE_BYTES + 2 * Q8_TILE_RAW : 4 * TILE_BYTES; }
 constexpr int SCHED_MAX_SEQ = 256;                   // balanced schedule: sequences per launch
 constexpr int sched_off(int kvt) { return handoff_off(kvt) + (is_cs(kvt) ? 8192 + 1024 + 64 : NTHREADS * 32); }   // prefix sums of the sequences' tile counts
@@ -121,6 +122,7 @@ constexpr int lds_total(int kvt) { return sched_off(kvt) + (2 * SCHED_MAX_SEQ + 
 // (bias builds: one vector register more is the program's own, the mask offset comes through the hand-off record instead)
 #define MLA_DECODE_CS_BIAS_INPUTS MLA_DECODE_CS_INPUTS, [msk] "s"(mask_base), [scl] "s"(s_scale)
 #define MLA_DECODE_CS_BIAS_CLOBBERS MLA_DECODE_CS_CLOBBERS, "v252"
+#define MLA_DECODE_KS_BIAS_CLOBBERS MLA_DECODE_KS_CLOBBERS, "v252"
 
 #define MLA_DECODE_INPUTS                                                                                          \
     [kv] "s"(kv_base), [bt] "s"(bt_row), [kvb] "s"(s_kvb), [kve] "s"(s_kve), [cl2] "s"(c_log2_bits), [npp] "s"(s_npp), \
@@ -524,17 +526,17 @@ __device__ __forceinline__ void decode_body() {
     // 2 log2(e) scale / softcap into p.c_log2_bits and -2 softcap (0: no soft cap) into p.softcap; the last 8 bytes of the hand-off
     // record are the slope of this thread's row's head (ggml-cpu.c:11985-11989, :12006-12008) and that -2 softcap; see
     // gen_decode_cs_asm.py
-    constexpr bool BIAS = KVT == SRC_BF16_CSB || KVT == SRC_F16_CSB;
+    constexpr bool BIAS = KVT == SRC_BF16_CSB || KVT == SRC_F16_CSB || KVT == SRC_BF16_KSB || KVT == SRC_F16_KSB;
+    // (the k-split programs: every wave works on the same 32 rows, its lanes' rows do not depend on the wave)
+    constexpr bool KS_ROWS = is_ks(KVT);
     float slope = 1.0f;
     if (BIAS && p.max_bias > 0.0f) {
-        const int r = min(row, p.n_rows - 1), head = r - (r / p.n_head) * p.n_head;
+        const int r = min(KS_ROWS ? by * 128 + rl : row, p.n_rows - 1), head = r - (r / p.n_head) * p.n_head;
         slope = head < p.n_head_log2 ? powf(p.m0, (float) (head + 1)) : powf(p.m1, (float) (2 * (head - p.n_head_log2) + 1));
     }
     {
         unsigned long long * h = (unsigned long long *) (smem + HANDOFF_OFF + tid * 32);
         // mask builds: byte offset of this lane's first mask element (its query token's row, tokens 4g.. of a tile)
-        // (the k-split programs: every wave works on the same 32 rows, its lanes' rows do not depend on the wave)
-        constexpr bool KS_ROWS = KVT == SRC_BF16_KS || KVT == SRC_F16_KS;
         h[0] = MASK ? (unsigned long long) ((int64_t) (min(KS_ROWS ? by * 128 + rl : row, p.n_rows - 1) / p.n_head) * p.mask_nb1 + 8 * g) : 0;
         h[1] = (unsigned long long) optr;
         h[2] = (unsigned long long) mlptr;
@@ -547,7 +549,7 @@ __device__ __forceinline__ void decode_body() {
     unsigned long long * q_rows = (unsigned long long *) (smem + HANDOFF_OFF + 8192) + wave * 32;
     if constexpr (KVT == SRC_BF16_CSQ || KVT == SRC_F16_CSQ) {
         stage_q_rows<KVT == SRC_F16_CSQ, 32, 144>(p, b, by * 128 + wave * 32, 0, smem + wave * TILE_BYTES, q_rows, lane);
-    } else if constexpr (KVT == SRC_BF16_KS || KVT == SRC_F16_KS) {
+    } else if constexpr (is_ks(KVT)) {
         q_row_table(p, b, 0, wave * 576, q_rows, lane);
     }
     // this wave's packed Q operands: [seq][row block][wave][k-step][lane][16 bytes], written by mla_q_pack_kernel (the programs
@@ -588,7 +590,15 @@ __device__ __forceinline__ void decode_body() {
     // mask builds of the column-split programs: byte offset of this lane's first mask element (its query token's row, tokens 4g.. of a tile)
     const int mask_off = MASK ? (int) ((int64_t) (min(row, p.n_rows - 1) / p.n_head) * p.mask_nb1 + 8 * g) : 0;
 
-    if constexpr (KVT == SRC_BF16_CSB) {
+    if constexpr (KVT == SRC_BF16_KSB) {
+        asm volatile(
+#include "mla_decode_ks_bf16_bias.inc"
+            : : MLA_DECODE_CS_BIAS_INPUTS : MLA_DECODE_KS_BIAS_CLOBBERS);
+    } else if constexpr (KVT == SRC_F16_KSB) {
+        asm volatile(
+#include "mla_decode_ks_f16_bias.inc"
+            : : MLA_DECODE_CS_BIAS_INPUTS : MLA_DECODE_KS_BIAS_CLOBBERS);
+    } else if constexpr (KVT == SRC_BF16_CSB) {
         asm volatile(
 #include "mla_decode_cs_bf16_bias.inc"
             : : MLA_DECODE_CS_BIAS_INPUTS : MLA_DECODE_CS_BIAS_CLOBBERS);
@@ -1048,11 +1058,11 @@ bool decode_fast_applicable(const mla_attn_args * a) {
     const bool q8_copy = decode_fast_q8_copy_rows(a) > 0;
     if (a->kv_type == MLA_TYPE_Q8_0 && !q8_copy && !q8_raw_tiles_ok(a)) return false;
     if (a->logit_softcap != 0.0f || a->max_bias > 0.0f) {
-        // ALiBi / soft cap: the masked column-split programs have a build for them (16-bit rows, a mask, blocks of 128 rows in
-        // which every wave has rows); everything else goes to the general kernel
+        // ALiBi / soft cap: the masked column-split programs (blocks of 128 rows in which every wave has rows) and the masked k-split
+        // programs (at most 32 rows) have a build for them, over 16-bit rows; everything else goes to the general kernel
         const int64_t n_rows = (int64_t) a->n_tok * a->n_head, tail = n_rows % 128;
         if (!a->mask || a->kv_type == MLA_TYPE_Q8_0 || (a->flags & MLA_FLAG_BF16_DIRECT)) return false;
-        if (!(tail == 0 || tail > 96) || n_rows >= (1 << 22)) return false;
+        if (!(n_rows <= 32 || tail == 0 || tail > 96) || n_rows >= (1 << 22)) return false;
         if (a->logit_softcap != 0.0f && !(a->logit_softcap > 0.0f && a->logit_softcap < INFINITY)) return false;
     }
     // 16-bit rows must be packed: the per-lane offsets of the tile copy are kept as 16-bit values (31 * 1152 + 1136 < 65536)
@@ -1123,8 +1133,8 @@ static bool decode_cs_applicable(const KParams & kp, int kv_type) {
 // them instead of leaving it to the one wave that has rows (gen_decode_cs_asm.py --ks)
 static bool decode_ks_applicable(const KParams & kp, int kv_type) {
     if (kv_type != MLA_TYPE_BF16 && kv_type != MLA_TYPE_F16) return false;
-    const bool bias = kp.softcap != 0.0f || kp.max_bias > 0.0f;
-    return !bias && !kp.bf16_direct && !kp.q_as_q8 && kp.n_rows <= 32 && kp.slot_rows < (1 << 22);
+    const bool bias = kp.softcap != 0.0f || kp.max_bias > 0.0f;   // (bias builds exist for masked launches)
+    return (!bias || kp.mask) && !kp.bf16_direct && !kp.q_as_q8 && kp.n_rows <= 32 && kp.slot_rows < (1 << 22);
 }
 
 template <int KVT_BLK, int KVT_TOK, bool STREAM = false>
@@ -1215,6 +1225,15 @@ hipError_t launch_decode_fast(const KParams & kp_in, int kv_type, dim3 grid, hip
         return tok_ks ? launch_dual<SRC_BF16_CVT, SRC_BF16_KS>(kp, kt, grid, st) : launch_dual<SRC_BF16_CVT, SRC_BF16_CVT>(kp, kt, grid, st);
     }
     if (kv_type == MLA_TYPE_Q8_0) return m ? launch_variant<SRC_Q8, true>(kp, grid, st) : launch_variant<SRC_Q8, false>(kp, grid, st);
+    if (ks && bias) {
+        if (!m) return hipErrorInvalidValue;
+        // what the bias builds expect in place of scale, scale * log2(e) and softcap (see the kernel)
+        if (kp.softcap != 0.0f) kp.scale = kp.scale / kp.softcap;
+        const float k1 = 2.0f * 1.44269504088896340736f * kp.scale;
+        kp.c_log2_bits = __builtin_bit_cast(int, k1);
+        kp.softcap = kp.softcap != 0.0f ? -2.0f * kp.softcap : 0.0f;   // (not -0: the program tests the bits)
+        return kv_type == MLA_TYPE_F16 ? launch_variant<SRC_F16_KSB, true>(kp, grid, st) : launch_variant<SRC_BF16_KSB, true>(kp, grid, st);
+    }
     if (ks && m && stream) return kv_type == MLA_TYPE_F16 ? launch_variant<SRC_F16_KS, true, true>(kp, grid, st) : launch_variant<SRC_BF16_KS, true, true>(kp, grid, st);
     if (ks && m) return kv_type == MLA_TYPE_F16 ? launch_variant<SRC_F16_KS, true>(kp, grid, st) : launch_variant<SRC_BF16_KS, true>(kp, grid, st);
     if (ks) return kv_type == MLA_TYPE_F16 ? launch_variant<SRC_F16_KS, false>(kp, grid, st) : launch_variant<SRC_BF16_KS, false>(kp, grid, st);

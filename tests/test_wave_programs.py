@@ -67,7 +67,7 @@ class Coverage:
 
 
 def run_cs(name, cov, f16, mask_build=False, bias_build=False, n_rows=128, kv=(0, 128), seq_len=None, paged=None, f32_rows=True, final=True,
-           q_in_lds=False, boost=False, seed=0, n_head=None, softcap=0.0, alibi=False, v_col0=False):
+           q_in_lds=False, boost=False, seed=0, n_head=None, softcap=0.0, alibi=False, v_col0=False, open_tail=False):
     rng = np.random.default_rng(seed)
     n_head = n_head or n_rows
     mask = None
@@ -76,7 +76,8 @@ def run_cs(name, cov, f16, mask_build=False, bias_build=False, n_rows=128, kv=(0
     if mask_build:
         n_kv = (seq_len + 31) // 32 * 32
         mask = np.where(rng.random(((n_rows + n_head - 1) // n_head, n_kv)) < 0.25, -np.inf, rng.standard_normal(((n_rows + n_head - 1) // n_head, n_kv)) * (0.5 if alibi else 0.0))
-        mask[:, seq_len:] = -np.inf
+        if not open_tail:     # (open_tail: the caller's mask says nothing about the cells past the end of a paged sequence)
+            mask[:, seq_len:] = -np.inf
         mask[:, kv[0]] = 0.0              # (no row of the piece without a key: such rows are the launcher's business)
         if not paged:         # (a masked launch over a cache without a table covers whole tiles; with a table the lengths may be ragged)
             kv, seq_len = (kv[0], min(n_kv, (kv[1] + 31) // 32 * 32)), n_kv
@@ -181,12 +182,16 @@ def test_bias_column_split_programs(name, f16):
         wg = run_cs(name, cov, f16, mask_build=True, bias_build=True, seed=40 + k, n_head=32, alibi=k % 2 == 0, softcap=30.0 if k % 3 else 0.0, **sc)
     wg = run_cs(name, cov, f16, mask_build=True, bias_build=True, seed=61, kv=(0, 19), paged=True, n_head=64, alibi=True)
     wg = run_cs(name, cov, f16, mask_build=True, bias_build=True, seed=62, kv=(32, 128 + 7), paged=True, n_head=32, softcap=20.0)
+    # a small cap and a mask that is open past the end of the paged sequence: the keys of the last tile that do not exist stay out
+    # (they came back with the finite logit -softcap while the cap was applied behind the tail masking)
+    wg = run_cs(name, cov, f16, mask_build=True, bias_build=True, seed=63, kv=(32, 128 + 7), paged=True, n_head=32, softcap=1.0, open_tail=True)
+    wg = run_cs(name, cov, f16, mask_build=True, bias_build=True, seed=64, kv=(0, 19), paged=True, n_head=64, alibi=True, softcap=0.7, open_tail=True)
     assert not cov.missing(wg), cov.missing(wg)
     _only_register_loads_ahead_of_tile_copies(cov)
 
 
 def run_ks(name, cov, f16, mask_build=False, n_rows=32, kv=(0, 128), seq_len=None, paged=None, f32_rows=True, final=True, boost=False, seed=0,
-           n_head=None):
+           n_head=None, bias_build=False, softcap=0.0, alibi=False, open_tail=False):
     rng = np.random.default_rng(seed)
     n_head = n_head or n_rows
     mask = None
@@ -195,21 +200,32 @@ def run_ks(name, cov, f16, mask_build=False, n_rows=32, kv=(0, 128), seq_len=Non
     if mask_build:
         n_kv = (seq_len + 31) // 32 * 32
         n_tok = (n_rows + n_head - 1) // n_head
-        mask = np.where(rng.random((n_tok, n_kv)) < 0.25, -np.inf, 0.0)
-        mask[:, seq_len:] = -np.inf
+        mask = np.where(rng.random((n_tok, n_kv)) < 0.25, -np.inf, rng.standard_normal((n_tok, n_kv)) * (0.5 if alibi else 0.0))
+        if not open_tail:
+            mask[:, seq_len:] = -np.inf
         mask[:, kv[0]] = 0.0
         if not paged:
             kv, seq_len = (kv[0], min(n_kv, (kv[1] + 31) // 32 * 32)), n_kv
     piece = S.Piece(rng, f16, n_rows=n_rows, kv_begin=kv[0], kv_end=kv[1], seq_len=seq_len, paged=paged, mask=mask, n_head=n_head,
                     k_boost=(lambda t: 4.0 ** ((t - kv[0]) // 32)) if boost else None)
-    lds_init = S.ks_lds_init(piece)
-    wg = E.Workgroup(S.program_text(name), 4, piece.gmem, S.ks_inputs(piece, piece.gmem, f32_rows=f32_rows, final=final, mask_build=mask_build), lds_init=lds_init)
+    slopes = (2.0 ** (-8.0 * (np.arange(128) % n_head + 1) / n_head)).astype(np.float32) if alibi else None
+    lds_init = S.ks_lds_init(piece, bias_build, slopes, -2.0 * softcap if softcap else 0.0)
+    inputs = S.ks_inputs(piece, piece.gmem, f32_rows=f32_rows, final=final, mask_build=mask_build)
+    if bias_build and softcap:        # what the launcher hands the bias builds where the plain ones find scale and scale log2(e)
+        base = inputs
+
+        def inputs(w, base=base):
+            d = base(w)
+            d["scl"] = int(np.array([S.SCALE / softcap], np.float32).view(np.uint32)[0])
+            d["cl2"] = int(np.array([2.0 * np.log2(np.e) * S.SCALE / softcap], np.float32).view(np.uint32)[0])
+            return d
+    wg = E.Workgroup(S.program_text(name), 4, piece.gmem, inputs, lds_init=lds_init)
     wg.name = name
     cov.install(wg)
     findings = wg.run()
     cov.collect(wg)
     assert not findings, "%s: %s" % (name, findings[:5])
-    want, m_want, l_want = piece.reference()
+    want, m_want, l_want = piece.reference(softcap=softcap, slopes=slopes)
     if f32_rows:
         got = piece.gmem.array("out").view(np.float32).reshape(128, 512)[:n_rows].astype(np.float64)
     else:
@@ -217,7 +233,10 @@ def run_ks(name, cov, f16, mask_build=False, n_rows=32, kv=(0, 128), seq_len=Non
     _check(got, want, name)
     if not final:
         ml = piece.gmem.array("ml").view(np.float32).reshape(128, 2)[:n_rows].astype(np.float64)
-        assert np.abs(ml[:, 0] + np.log2(ml[:, 1]) - (m_want + np.log2(l_want))).max() < 1e-3, "%s: (m, l) of the piece" % name
+        lse = ml[:, 0] + np.log2(ml[:, 1])
+        if softcap:         # the capped logits are kept less the cap: a constant per row
+            lse = lse + softcap * np.log2(np.e)
+        assert np.abs(lse - (m_want + np.log2(l_want))).max() < 1e-3, "%s: (m, l) of the piece" % name
     return wg
 
 
@@ -245,6 +264,22 @@ def test_k_split_programs(name, f16, mask_build):
     if mask_build:
         wg = run_ks(name, cov, f16, mask_build=True, seed=90, kv=(0, 19), paged=True, n_head=8, n_rows=16)
         wg = run_ks(name, cov, f16, mask_build=True, seed=91, kv=(32, 128 + 7), paged=True, n_head=32)
+    assert not cov.missing(wg), cov.missing(wg)
+    _only_register_loads_ahead_of_tile_copies(cov)
+
+
+@pytest.mark.parametrize("name,f16", [("mla_decode_ks_bf16_bias.inc", False), ("mla_decode_ks_f16_bias.inc", True)])
+def test_bias_k_split_programs(name, f16):
+    """ALiBi slopes and the soft cap on the k-split programs (at most 32 rows): the scenarios of the masked builds with a slope
+    per head, a cap, both, neither; caps small enough that a key wrongly let in would show."""
+    cov = Coverage()
+    for k, sc in enumerate(KS_SCENARIOS):
+        sc = {kk: vv for kk, vv in sc.items() if kk != "paged"}
+        wg = run_ks(name, cov, f16, mask_build=True, bias_build=True, seed=170 + k, n_head=16, alibi=k % 2 == 0,
+                    softcap=0.0 if sc.get("boost") else (30.0, 0.0, 2.0)[k % 3], **sc)   # (a cap keeps the running maxima from moving)
+    wg = run_ks(name, cov, f16, mask_build=True, bias_build=True, seed=190, kv=(0, 19), paged=True, n_head=8, n_rows=16, alibi=True, softcap=0.7, open_tail=True)
+    wg = run_ks(name, cov, f16, mask_build=True, bias_build=True, seed=191, kv=(32, 128 + 7), paged=True, n_head=32, softcap=1.0, open_tail=True)
+    wg = run_ks(name, cov, f16, mask_build=True, bias_build=True, seed=192, kv=(0, 64), paged=True, n_head=4, n_rows=8, alibi=True)
     assert not cov.missing(wg), cov.missing(wg)
     _only_register_loads_ahead_of_tile_copies(cov)
 

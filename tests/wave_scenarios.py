@@ -147,9 +147,10 @@ def ks_inputs(piece, gmem_out, f32_rows=True, final=True, scale=SCALE, mask_buil
     return per_wave
 
 
-def ks_lds_init(piece):
-    """Hand-off records (first word: the mask offset of the thread's row, rows counted inside the one block of 32) and, behind the
-    exchange buffer, every wave's table of the addresses its quarter of the 32 Q rows starts at."""
+def ks_lds_init(piece, bias_build=False, slopes=None, softcap=0.0):
+    """Hand-off records (first word: the mask offset of the thread's row, rows counted inside the one block of 32; bias builds: last 8
+    bytes the row's slope and -2 softcap) and, behind the exchange buffer, every wave's table of the addresses its quarter of the 32 Q
+    rows starts at."""
     q_addr = piece.gmem.add("q_f32", piece.q_f32[:piece.n_rows])
     rec = np.zeros((256, 8), np.uint32)
     tab = np.zeros((4, 32), np.uint64)
@@ -158,6 +159,9 @@ def ks_lds_init(piece):
         row = min(lane % 32, piece.n_rows - 1)
         if piece.mask is not None:
             rec[t, 0] = (row // piece.n_head) * piece.mask_nb1 + 8 * (lane // 32)
+        if bias_build:
+            rec[t, 6] = np.array([1.0 if slopes is None else slopes[row]], np.float32).view(np.uint32)[0]
+            rec[t, 7] = np.array([softcap], np.float32).view(np.uint32)[0]
     for w in range(4):
         for r in range(32):
             tab[w, r] = q_addr + min(r, piece.n_rows - 1) * 576 * 4 + w * 576
