@@ -92,7 +92,7 @@ int mla_copy_f32_check(const mla_copy_args * args);     /* as mla_rope_check */
  * business).  The ops of a batch must be independent: none reads or writes memory that another one writes.  The result
  * is that of launching them one after the other, in any order.  Ops whose shape has no form inside the batch kernel (a
  * product with more than 32 rows per matrix: a prefill chunk) are launched on their own by the same call.  All ops are
- * checked before the first is launched: an error means nothing ran. */
+ * checked before the first is launched: a refused argument block (a negative MLA_ERR_* return) means nothing ran. */
 #define MLA_FRONT_ROPE          0 /* args: const mla_rope_args * */
 #define MLA_FRONT_MUL_MAT       1 /* const mla_mul_mat_args * */
 #define MLA_FRONT_COPY          2 /* const mla_copy_args * */
