@@ -43,7 +43,7 @@ extern "C" {
                                       accumulator, keys in order -- instead of the matrix-core path, whose operands are q * d rounded to
                                       f16 (q * d has 19 significant bits, f16 keeps 11).  That rounding averages out over many keys
                                       (4.5e-4 relative L2 error at any block scale) but shows in single elements when two or three
-                                      keys carry a row: up to 2.5e-3 against the stated 2e-3 for values of unit variance, more for larger ones.  A correctness mode like the one above,
+                                      keys carry a row: up to 4e-3 against the stated 2e-3 for values of unit variance, more for larger ones.  A correctness mode like the one above,
                                       10 to 100 times slower; without the flag it is taken by itself when no sequence can hold more
                                       than one page of keys, where it costs nothing to speak of. */
 #define MLA_FLAG_UNIFORM_SPLITS 2u /* paged decode: give every sequence the same number of equal KV splits (sized for the longest
