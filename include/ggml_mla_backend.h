@@ -66,7 +66,7 @@
  * scales (ggml-cpu-quants.c:3814-4241) and dequantises V to f32 (ggml-quants.c:357-373).  Over many keys the rounding averages out
  * (4.5e-4 rel-L2 at any block scale); when two or three keys carry a row it shows in single elements, up to 4e-3 max-abs against
  * the stated 2e-3 for values of unit variance (the largest of 4 000 random small cases: 3.9e-3; rel-L2 stays below 5e-4), and more for larger ones, since both the logits' and V's
- * rounding scale with the values: 3e-2 in single elements for rows of N(0, 3) under queries of N(0, 2) (tests/test_backend_gpu.py).  A cache of at most one page per sequence takes the exact path by itself; params containing
+ * rounding scale with the values: 3e-2 in single elements for rows of N(0, 3) under queries of N(0, 2) (tests/test_backend_gpu.py).  A cache of at most one page per sequence takes the exact path by itself (while rows x keys stay within 16 384 x 128); params containing
  * "q8=exact", or GGML_HIP_MLA_Q8=exact in the environment, make every Q8_0 node take it (the reference's own arithmetic, keys in
  * order: within 1e-5 of ggml-cpu's node at any shape, 10 to 100 times slower): for comparisons, not for serving.
  * BF16 KV, more than 32 attention rows per sequence: the decode kernel converts the cache tiles to f16 on the way (exact for magnitudes in [2^-14, 65504], which a

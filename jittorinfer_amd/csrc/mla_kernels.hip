@@ -994,8 +994,10 @@ int make_plan(const mla_attn_args * a, Plan * pl) {
     *pl = Plan{};
     // The replay of the reference's own arithmetic (mla_ref_scores_kernel, mla_ref_walk_kernel): asked for by flag, and taken by
     // itself for a Q8_0 cache of at most one page per sequence -- with so few keys one of them can carry a row, and then the
-    // 16-bit operands the matrix cores are fed (q * d has 19 significant bits) show in single output elements
-    const bool q8_small = a->kv_type == MLA_TYPE_Q8_0 && max_len <= MLA_PAGE_TOKENS && (int64_t) a->n_seq * n_rows <= 16384 && a->rows_per_wg == 0;
+    // 16-bit operands the matrix cores are fed (q * d has 19 significant bits) show in single output elements -- while the walk
+    // stays short: rows x keys up to what 16 384 rows over a full page are
+    const bool q8_small = a->kv_type == MLA_TYPE_Q8_0 && max_len <= MLA_PAGE_TOKENS && a->rows_per_wg == 0 &&
+                          (int64_t) a->n_seq * n_rows * (max_len > 0 ? max_len : 1) <= (int64_t) 16384 * MLA_PAGE_TOKENS;
     if ((a->flags & (MLA_FLAG_F16_ACC_STRICT | MLA_FLAG_Q8_EXACT)) || q8_small) {
         pl->variant   = 1;
         pl->n_splits  = 1;

@@ -150,6 +150,22 @@ def test_q8_caches_of_one_page_take_the_exact_path(gpu):
             want = O.flash_attn_ext(q, k, O.TYPE_Q8_0, dv=512, scale=U.SCALE)
         assert info["variant"] == 1, info
         print(U.check(got[..., :512], want, "Q8_0, one page", max_abs=2e-5, rel_l2=2e-6))
+    # the bound is on rows x keys: 5 sequences of 33 tokens x 128 heads over 32 keys under a mask (21 120 rows; the shape on which a
+    # wider random sweep found the matrix-core operands 3.9e-3 off) still takes the replay, the same rows over 128 keys do not
+    q = rng.standard_normal((5, 128, 33, 576)).astype(np.float32)
+    for n_kv, variant in ((32, 1), (128, 2)):
+        k = U.encode_kv(rng.standard_normal((5, n_kv, 576)).astype(np.float32), O.TYPE_Q8_0)
+        m = (rng.standard_normal((33, n_kv)) * 1.5).astype(np.float32)
+        m[rng.random((33, n_kv)) < 0.6] = -np.inf
+        m[:, 0] = 0.0
+        mask = np.zeros((64, n_kv), np.float16)
+        mask[:33] = m
+        info = J.plan(torch.from_numpy(q).to(gpu), torch.from_numpy(k).to(gpu), O.TYPE_Q8_0, dv=512, scale=U.SCALE, mask=torch.from_numpy(mask).to(gpu))
+        assert info["variant"] == variant, info
+        if variant == 1:
+            got = _run(gpu, q, k, O.TYPE_Q8_0, mask=mask.view(np.uint16), scale=U.SCALE)
+            want = O.flash_attn_ext(q, k, O.TYPE_Q8_0, dv=512, mask=mask.view(np.uint16), scale=U.SCALE)
+            print(U.check(got[..., :512], want, "Q8_0, 21 120 rows over 32 keys", max_abs=2e-5, rel_l2=2e-6))
 
 
 @pytest.mark.parametrize("k_type", [O.TYPE_BF16, O.TYPE_Q8_0])
