@@ -59,6 +59,11 @@ NT_HINT = " nt" if STREAM or not MASK else ""
 # K fragment ring: five slots of its own, the sixth in T[4:7] (free while K.Q^T runs); mask builds give the last slot of each
 # ring to the mask values
 KRING, PRING = (5, 3) if MASK else (6, 4)
+# The f16 partial rows and the (m, l) pairs are read by another kernel, on other XCDs: stored at device scope they go to memory as
+# they are written, instead of waiting in this XCD's L2 for the write-back at the end of the kernel (config 3: step -1 %, a layer's
+# decode step -1 us).  Not the f32 rows: final output written through loses the L2's merging of a row's pieces (a prompt chunk of
+# 512 tokens from an empty cache: 97 -> 142 us with the same bit on those stores).
+PARTIAL_SCOPE = " sc1"
 
 # ---- VGPR map (v252..v255 are left to the compiler: the clobber list of the asm block ends at v251)
 Q0 = 0
@@ -1081,7 +1086,7 @@ def epilogue(nhb):
                 e("v_cvt_pk_f16_f32 %s, %s, %s" % (v(r), v(r), v(r + 1)))
                 e("v_cvt_pk_f16_f32 %s, %s, %s" % (v(r + 1), v(r + 2), v(r + 3)))
                 e("s_nop 0")
-                e("global_store_dwordx2 %s, %s, %s offset:%d" % (v(T[0]), v(r, 2), s(SB, 2), hb * 512))
+                e("global_store_dwordx2 %s, %s, %s offset:%d%s" % (v(T[0]), v(r, 2), s(SB, 2), hb * 512, PARTIAL_SCOPE))
                 e("s_add_u32 %s, %s, %s" % (s(SB), s(SB), s(OSTR)))
                 e("s_addc_u32 %s, %s, 0" % (s(SB + 1), s(SB + 1)))
     e("%s:" % lab_sdone)
@@ -1105,7 +1110,7 @@ def epilogue(nhb):
     e("v_mov_b32 %s, %s" % (v(T[0]), v(MRUN)))
     e("v_mov_b32 %s, %s" % (v(T[1]), v(LRUN)))
     e("s_nop 0")
-    e("global_store_dwordx2 %s, %s, %s" % (v(T[2]), v(T[0], 2), s(MLB, 2)))
+    e("global_store_dwordx2 %s, %s, %s%s" % (v(T[2]), v(T[0], 2), s(MLB, 2), PARTIAL_SCOPE))
     e("%s:" % lab_noml)
     e("s_mov_b64 exec, %s" % s(EXS, 2))
     e("s_waitcnt vmcnt(0)")
