@@ -40,6 +40,9 @@ DMA_PER_TILE = 5 if Q8 else 10 # LDS-DMA instructions each wave issues per tile
 # through the L2s without it push out what is read again (the operand image, the partials).  Not the masked programs (prompt chunks
 # re-read their cells from one row block to the next) and not the Q8_0 programs (their kernel measured 3 % slower with it).
 NT_HINT = "" if MASK or Q8 else " nt"
+# The f16 partial rows and the (m, l) pairs go to another kernel, on other XCDs: stored at device scope they are written through as
+# they are produced instead of at the kernel's end (see gen_decode_cs_asm.py)
+PARTIAL_SCOPE = " sc1"
 Q8_WAVE_CHUNKS = 306           # a wave copies 306 of the 1224 16-byte chunks of a raw tile
 CPR = 73                       # 16-byte chunks per padded row
 WAVE_CHUNKS = 8 * CPR          # 584: each wave moves rows 8w..8w+7 of a tile
@@ -1285,7 +1288,7 @@ def main():
             e("v_cvt_pk_f16_f32 %s, %s, %s" % (v(r), v(r), v(r + 1)))
             e("v_cvt_pk_f16_f32 %s, %s, %s" % (v(r + 1), v(r + 2), v(r + 3)))
             e("s_nop 0")
-            e("global_store_dwordx2 %s, %s, off" % (v(OPTR, 2), v(r, 2)))
+            e("global_store_dwordx2 %s, %s, off%s" % (v(OPTR, 2), v(r, 2), PARTIAL_SCOPE))
             e("v_add_co_u32 %s, vcc, %s, %s" % (v(OPTR), s(OSTR), v(OPTR)))
             e("s_nop 1")
             e("v_addc_co_u32 %s, vcc, 0, %s, vcc" % (v(OPTR + 1), v(OPTR + 1)))
@@ -1298,7 +1301,7 @@ def main():
     e("v_mov_b32 %s, %s" % (v(T[0]), v(MRUN)))
     e("v_mov_b32 %s, %s" % (v(T[1]), v(LRUN)))
     e("s_nop 0")
-    e("global_store_dwordx2 %s, %s, off" % (v(MLPTR, 2), v(T[0], 2)))
+    e("global_store_dwordx2 %s, %s, off%s" % (v(MLPTR, 2), v(T[0], 2), PARTIAL_SCOPE))
     e("s_mov_b64 exec, %s" % s(EXS, 2))
     e("s_waitcnt vmcnt(0)")
     stamp(5)
