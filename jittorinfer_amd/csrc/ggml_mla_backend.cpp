@@ -728,6 +728,11 @@ bool written_after(const std::vector<front_item> & w, int i, const mem_range & r
     for (size_t k = (size_t) i + 1; k < w.size(); k++) if (overlaps(w[k].write, r)) return true;
     return false;
 }
+// ... by an item strictly between items i and j
+bool written_between(const std::vector<front_item> & w, int i, int j, const mem_range & r) {
+    for (int k = i + 1; k < j; k++) if (overlaps(w[k].write, r)) return true;
+    return false;
+}
 
 // Appends `node` to the run; validation as in compute_front / compute_kv_write.
 int front_collect(std::vector<front_item> & w, const tensor * node) {
@@ -774,7 +779,8 @@ int front_collect(std::vector<front_item> & w, const tensor * node) {
                 mla_rope_args f = a;
                 f.src = xs->data;
                 for (int i = 0; i < 4; i++) f.src_nb[i] = (int64_t) xs->nb[i];
-                if (same && mla_rope_check(&f) == 0 && !written_after(w, ci, range_of(xs))) {
+                // (the CONT's source as it was when the CONT ran, and the CONT's result as the CONT left it: nothing in between wrote either)
+                if (same && mla_rope_check(&f) == 0 && !written_after(w, ci, range_of(xs)) && !written_between(w, ci, self, range_of(x))) {
                     a = f; it.rope_src = xs;
                     // the graph allocator lets a ROPE rotate in place (ggml-alloc.c: ggml_op_can_inplace): the CONT's result is
                     // then overwritten whole by this node, and when nothing in between reads it the CONT has no work left
@@ -828,7 +834,10 @@ int front_collect(std::vector<front_item> & w, const tensor * node) {
                     f.w.src = lat->data; f.w.src_nb1 = (int64_t) lat->nb[1];
                     f.rope = w[ri].args[0].rope;
                     const mem_range pe_src = range_of(w[ri].rope_src);
-                    if (mla_kv_write_rope_check(&f) == 0 && !written_after(w, ki, range_of(lat)) && !written_after(w, ri, pe_src) &&
+                    // (what the chain read is still what it was, and its intermediate results are what it left: the rotated k_pe up to the
+                    // CONCAT, the CONCAT's rows up to this node)
+                    if (mla_kv_write_rope_check(&f) == 0 && !written_between(w, ri, ki, range_of(r)) && !written_between(w, ki, self, range_of(rows)) &&
+                        !written_after(w, ki, range_of(lat)) && !written_after(w, ri, pe_src) &&
                         !written_after(w, ri, range_of(r->src[1])) && !(r->src[2] && written_after(w, ri, range_of(r->src[2])))) {
                         it.args[0].kvr = f;
                         it.ops[0] = mla_front_op{ MLA_FRONT_KV_WRITE_ROPE, 0, &it.args[0].kvr };

@@ -800,10 +800,11 @@ int ref_random_front(const char * so_path, uint32_t seed, int64_t H, int64_t T, 
         uint32_t st = seed * 2654435761u + 12345u;
         w192[n192++] = ta;
         for (int i = 0; i < n_ops && n64 < CAP - 2 && n128 < CAP - 2 && n192 < CAP - 2; i++) {
-            int kind = (int) (rg_next(&st) % 7);
+            int kind = (int) (rg_next(&st) % 8);
             if ((kind == 1 || kind == 3) && n64 == 0) kind = 0;
             if (kind == 4 && (n128 == 0 || n64 == 0)) kind = n64 ? 3 : 0;
             if (kind == 6 && n128 == 0) kind = 5;
+            if (n64 >= CAP - 4) break;
             switch (kind) {
                 case 0: {   /* cont of a 64-wide view of a wider tensor */
                     const int wide = n128 && (rg_next(&st) & 1);
@@ -824,7 +825,13 @@ int ref_random_front(const char * so_path, uint32_t seed, int64_t H, int64_t T, 
                     else                  w192[n192++] = ggml_concat(c, w64[rg_next(&st) % n64], w128[rg_next(&st) % n128], 0);
                     break;
                 case 5: w128[n128++] = ggml_cont(c, RG_VIEW(w192[rg_next(&st) % n192], 128, 64 * (rg_next(&st) % 2))); break;
-                default: w64[n64++] = RG_ROPE(RG_VIEW(w128[rg_next(&st) % n128], 64, 64 * (rg_next(&st) % 2))); break;   /* rope of a strided view */
+                case 6: w64[n64++] = RG_ROPE(RG_VIEW(w128[rg_next(&st) % n128], 64, 64 * (rg_next(&st) % 2))); break;   /* rope of a strided view */
+                default: {  /* one cont with two consumers, one of which rotates it in place: whichever comes later in node order sees the other's work */
+                    struct ggml_tensor * t = ggml_cont(c, RG_VIEW(w192[rg_next(&st) % n192], 64, 64 * (rg_next(&st) % 3)));
+                    w64[n64++] = ggml_rope_ext_inplace(c, t, tp, NULL, 64, 0, 4096, 10000.0f, 0.025f, 1.0f, 0.8f, 32.0f, 1.0f);
+                    w64[n64++] = RG_ROPE(t);
+                    break;
+                }
             }
         }
         /* the k side, written into the cache the way llm_attn_mla does it, ahead of the rest (src/llama-graph-attn.cpp:236-241) */
