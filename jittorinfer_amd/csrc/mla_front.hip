@@ -33,13 +33,13 @@ __global__ void __launch_bounds__(256) mla_rope_kernel(const RopeP p) {
 template <bool F16, int MB>
 __global__ void __launch_bounds__(256) mla_mul_mat_kernel(const MmP p) {
     __shared__ __attribute__((aligned(16))) char lds[MM_LDS<MB>];
-    mm_body<F16, MB>(p, Blk{ blockIdx.x, blockIdx.y, blockIdx.z, gridDim.x }, lds);
+    mm_body<F16, MB>(p, xcd_grouped(Blk{ blockIdx.x, blockIdx.y, blockIdx.z, gridDim.x }, gridDim.y, gridDim.z), lds);
 }
 
 template <bool F16>
 __global__ void __launch_bounds__(256) mla_mul_mat_small_kernel(const MmP p) {
     __shared__ __attribute__((aligned(16))) char lds[MS_LDS];
-    mm_small_body<F16>(p, Blk{ blockIdx.x, blockIdx.y, blockIdx.z, gridDim.x }, lds);
+    mm_small_body<F16>(p, xcd_grouped(Blk{ blockIdx.x, blockIdx.y, blockIdx.z, gridDim.x }, gridDim.y, gridDim.z), lds);
 }
 
 // Many rows m with K = 128, 256 or 512 (a prefill chunk through the absorb products): bound by the f32 activations
@@ -192,7 +192,7 @@ struct BatchOp {
 };
 struct BatchP {
     int n;
-    unsigned first[MLA_FRONT_BATCH_MAX + 1];
+    unsigned first[MLA_FRONT_BATCH_MAX + 1];   // multiples of 8: every op's first workgroup runs on XCD 0 (xcd_grouped)
     BatchOp op[MLA_FRONT_BATCH_MAX];
 };
 
@@ -208,13 +208,14 @@ __global__ void __launch_bounds__(256) mla_front_batch_kernel(const BatchP p) {
     while (i + 1 < p.n && blockIdx.x >= p.first[i + 1]) i++;
     const BatchOp & op = p.op[i];
     const unsigned l = blockIdx.x - p.first[i];
+    if (l >= op.gx * op.gy * op.gz) return;   // the padding up to the next op's start
     const Blk b{ l % op.gx, (l / op.gx) % op.gy, l / (op.gx * op.gy), op.gx };
     switch (op.kind) {
         case B_ROPE:          rope_body(op.u.rope, b, lds); break;
-        case B_MM_SMALL:      mm_small_body<false>(op.u.mm, b, lds); break;
-        case B_MM_SMALL_F16:  mm_small_body<true>(op.u.mm, b, lds); break;
-        case B_MM_TILE1:      mm_body<false, 1>(op.u.mm, b, lds); break;
-        case B_MM_TILE1_F16:  mm_body<true, 1>(op.u.mm, b, lds); break;
+        case B_MM_SMALL:      mm_small_body<false>(op.u.mm, xcd_grouped(b, op.gy, op.gz), lds); break;
+        case B_MM_SMALL_F16:  mm_small_body<true>(op.u.mm, xcd_grouped(b, op.gy, op.gz), lds); break;
+        case B_MM_TILE1:      mm_body<false, 1>(op.u.mm, xcd_grouped(b, op.gy, op.gz), lds); break;
+        case B_MM_TILE1_F16:  mm_body<true, 1>(op.u.mm, xcd_grouped(b, op.gy, op.gz), lds); break;
         case B_COPY1:         copy_body<float>(op.u.copy, b); break;
         case B_COPY4:         copy_body<float4>(op.u.copy, b); break;
         case B_KVW_BF16:      kv_write_body<SRC_BF16, true, false>(op.u.kvw, b); break;
@@ -420,7 +421,7 @@ extern "C" int mla_front_batch_launch(const mla_front_op * ops, int32_t n_ops, v
                 continue;
             }
             const BatchOp & b = p.op[p.n];
-            p.first[p.n + 1] = p.first[p.n] + b.gx * b.gy * b.gz;
+            p.first[p.n + 1] = p.first[p.n] + ((b.gx * b.gy * b.gz + 7u) & ~7u);
             if (++p.n == MLA_FRONT_BATCH_MAX) {
                 const int e = flush();
                 if (e) return e;

@@ -17,6 +17,19 @@ namespace front {
 
 struct Blk { unsigned x, y, z, gx; };   // the body's block index, and its grid's x extent
 
+// Workgroups are handed to the 8 XCDs round-robin in dispatch order, and each XCD has its own L2.  The n tiles of a product that
+// share their activation rows (the same y, z; consecutive x) would land on different XCDs, each of which fetches those rows for
+// itself (the un-absorb product of a 128-head decode step: 50 MB fetched for 25 MB of operands).  With the grid's first block on
+// XCD 0 and a block count that is a multiple of 8, block l runs on XCD l % 8: it takes the tuple number (l % 8) * G / 8 + l / 8, so
+// that consecutive tuples -- the n tiles of one set of rows -- share an XCD.
+__device__ __forceinline__ Blk xcd_grouped(const Blk b, unsigned gy, unsigned gz) {
+    const unsigned G = b.gx * gy * gz;
+    if ((G & 7) != 0 || b.gx == 1) return b;
+    const unsigned l = (b.z * gy + b.y) * b.gx + b.x;
+    const unsigned v = (l & 7) * (G >> 3) + (l >> 3);
+    return Blk{ v % b.gx, (v / b.gx) % gy, v / (b.gx * gy), b.gx };
+}
+
 // ---------------------------------------------------------------- rotary embedding
 
 constexpr int ROPE_MAX_PAIRS = 256;
