@@ -31,12 +31,16 @@ MASK = "--mask" in ARGS                      # additive f16 mask rows (one per q
 KS = "--ks" in ARGS                          # at most 32 rows: the four waves split the 576 columns of K.Q^T (see ks_main)
 BIAS = "--bias" in ARGS                      # mask builds: ALiBi slope per head on the mask, tanh soft cap on the logits
 STREAM = "--stream" in ARGS                  # mask builds: the tile copies carry the non-temporal hint (see NT_HINT)
+HALF = "--half" in ARGS                      # 33 .. 64 rows: two row blocks; the waves without rows still copy tiles and take their columns of P.V
 assert not (MASK and CLK) and (MASK or not BIAS) and (MASK or not STREAM) and not (BIAS and STREAM)
+assert not (HALF and (MASK or KS or CLK))
+NHB = 2 if HALF else 4                       # row blocks of 32 rows
+NFRAG = 2 * NHB                              # P^T fragments of a tile
 MF_QK = "v_mfma_f32_32x32x16_f16" if F16KV else "v_mfma_f32_32x32x16_bf16"
 MF_PV = "v_mfma_f32_32x32x16_f16"
 
 
-CONV_P1 = 5                                  # V^T fragments converted in part 1; the rest in the first half of part 2
+CONV_P1 = 8 if HALF else 5                   # V^T fragments converted in part 1; the rest in the first half of part 2
 
 PITCH = 1168
 TILE_BYTES = 32 * PITCH
@@ -339,7 +343,7 @@ def v_conv_items(f, tmp):
 
 
 def p_read(f):
-    kk, hb = f // 4, f % 4
+    kk, hb = f // NHB, f % NHB
     lds.op("ds_read_b128 %s, %s offset:%d" % (v(PR + 4 * (f % PRING), 4), v(PADDR), (hb * 2 + kk) * 1024), ("p", f))
 
 
@@ -347,8 +351,8 @@ def pv_slots():
     """32 MFMA slots of O^T += V^T.P^T in the order [kk][hb][cb]: a P^T fragment serves four consecutive MFMAs, and
     MFMAs on the same accumulator block are 16 slots apart."""
     def mk(n):
-        kk, hb, cb = n // 16, (n // 4) % 4, n % 4
-        f = 4 * kk + hb
+        kk, hb, cb = n // (4 * NHB), (n // 4) % NHB, n % 4
+        f = NHB * kk + hb
         acc = 16 * (4 * cb + hb)
 
         def slot():
@@ -356,10 +360,10 @@ def pv_slots():
                 lds.need(("p", f))
             lds.need(("v", 4 * kk + cb, 1))          # f16 KV: the fragment is used as read; bf16: converted long before (no-op)
             e("%s %s, %s, %s, %s" % (MF_PV, a(acc, 16), v(VF + 4 * (4 * kk + cb), 4), v(PR + 4 * (f % PRING), 4), a(acc, 16)))
-            if cb == 0 and f + PRING - 1 < 8:
+            if cb == 0 and f + PRING - 1 < NFRAG:
                 p_read(f + PRING - 1)                # into the slot of fragment f - 1 (for f = 0: the tile before's last), whose last MFMA has been issued
         return slot
-    return [mk(n) for n in range(32)]
+    return [mk(n) for n in range(8 * NHB)]
 
 
 def softmax_lines(first_tile=False):
@@ -510,23 +514,25 @@ def mask_wait():
     e("%s:" % lab_md)
 
 
-def canon_tags():
+def canon_tags(rowless=False):
     """LDS reads in flight at the top of every iteration, in issue order (see handover)."""
-    return [("k", p) for p in range(KRING - 1)] + [("p", f) for f in range(PRING - 1)]
+    return ([] if rowless else [("k", p) for p in range(KRING - 1)]) + [("p", f) for f in range(PRING - 1)]
 
 
-def handover(tail, resc):
+def handover(tail, resc, rowless=False):
     """Behind the barrier that ends a tile (tile IT is the one whose P.V comes next): the flag words of the four waves, the
     first K fragments of the next K.Q^T (tile IT+1, buffer at s[OFF1]) and the first P^T fragments of tile IT, around the
     last four P.V MFMAs of the tile that ends (they still use ring slot 3, which fragment 3 takes afterwards), with the
     scalars of the coming iteration in their shadow; then the accumulators take the new row maxima if some wave's flag is
-    up (out of line, rare)."""
+    up (out of line, rare).  rowless (--half): a wave without rows multiplies no K.Q^T."""
     e("v_mov_b32 %s, 0x%x" % (v(T[4]), FOFF))
     lds.op("ds_read_b128 %s, %s" % (v(T[0], 4), v(T[4])), ("f",))
-    e("v_add_u32 %s, %s, %s" % (v(KADDR), s(OFF1), v(KADDR_LANE)))
-    k_warm()
-    # fragment 7, which the tail MFMAs still use, sits in ring slot 7 % PRING: a fragment that shares it is requested behind them
-    early = [f for f in range(PRING - 1) if not tail or f % PRING != 7 % PRING]
+    if not rowless:
+        e("v_add_u32 %s, %s, %s" % (v(KADDR), s(OFF1), v(KADDR_LANE)))
+        k_warm()
+    # the tile's last fragment, which the tail MFMAs still use, sits in ring slot (NFRAG - 1) % PRING: a fragment that shares it is
+    # requested behind them
+    early = [f for f in range(PRING - 1) if not tail or f % PRING != (NFRAG - 1) % PRING]
     for f in early:
         p_read(f)
     top = ["s_add_u32 %s, %s, 1" % (s(S0), s(IT)),
@@ -545,15 +551,18 @@ def handover(tail, resc):
             assert f > max(early)      # fragments return in order
             p_read(f)
     lds.need(("f",))
-    e("v_or3_b32 %s, %s, %s, %s" % (v(T[0]), v(T[0]), v(T[1]), v(T[2])))
-    e("v_or_b32 %s, %s, %s" % (v(T[0]), v(T[0]), v(T[3])))
+    if HALF:      # (the words of the waves without rows are never written)
+        e("v_or_b32 %s, %s, %s" % (v(T[0]), v(T[0]), v(T[1])))
+    else:
+        e("v_or3_b32 %s, %s, %s, %s" % (v(T[0]), v(T[0]), v(T[1]), v(T[2])))
+        e("v_or_b32 %s, %s, %s" % (v(T[0]), v(T[0]), v(T[3])))
     e("v_cmp_ne_u32 vcc, 0, %s" % v(T[0]))
     lab_resc, lab_back = label("resc"), label("back")
     e("s_cmp_lg_u64 vcc, 0")
     e("s_cbranch_scc1 %s" % lab_resc)
     e("%s:" % lab_back)
     resc.append((lab_resc, lab_back))
-    assert lds.pending == canon_tags(), (lds.pending, canon_tags())
+    assert lds.pending == canon_tags(rowless), (lds.pending, canon_tags(rowless))
 
 
 def rescale_block(ret_label):
@@ -564,7 +573,7 @@ def rescale_block(ret_label):
     e("ds_read_b128 %s, %s offset:%d" % (v(T[4], 4), v(PADDR), AOFF - PBUF))
     e("s_waitcnt lgkmcnt(0)")
     for cb in range(4):
-        for hb in range(4):
+        for hb in range(NHB):
             base = 16 * (4 * cb + hb)
             for i in range(0, 16, 4):
                 for j in range(4):
@@ -622,8 +631,98 @@ def clk_dump():
 # (a ring of four asks for fragment 7 at slot 16, a ring of three -- the mask builds -- at slot 20: with the barrier ahead of slot 20
 # the other waves' reads of fragment 7, wave 3's rows, raced with wave 3's write of the next tile's P), with an MFMA or two between
 # the request and the wait for it
-B2_AT = 22 if PRING == 3 else 20
-PW_AT = 24                        # P.V slot ahead of which P of the next tile is written (the softmax is done by then)
+B2_AT = 8 if HALF else 22 if PRING == 3 else 20
+PW_AT = 12 if HALF else 24        # P.V slot ahead of which P of the next tile is written (the softmax is done by then)
+TAIL_AT = 8 * NHB - 4             # the last four P.V MFMAs of a tile are issued behind the barrier that ends it (see handover)
+
+
+def v_stream(n_conv, tmp):
+    """Part 1: reads of all eight V^T fragments of tile IT (two fragments ahead of their conversion) and conversion of
+    the first n_conv, as one ordered stream: the conversions share two temporaries."""
+    items = v_read_items(0) + v_read_items(1)
+    for f in range(8):
+        if f < n_conv:
+            items += v_conv_items(f, tmp)
+        if f + 2 < 8:
+            items += v_read_items(f + 2)
+    return spread(items, 0, 35)
+
+
+def tile_end_wait():
+    """The loads of tile IT+2 have landed (those of tile IT+3, issued in this iteration, may still be in flight: loads complete in
+    order)."""
+    lab_w0, lab_wd = label("w0"), label("wd")
+    e("s_cmp_eq_u32 %s, 0" % s(VMW))
+    e("s_cbranch_scc1 %s" % lab_w0)
+    e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
+    e("s_branch %s" % lab_wd)
+    e("%s:" % lab_w0)
+    e("s_waitcnt vmcnt(0)")
+    e("%s:" % lab_wd)
+
+
+def rotate_buffers():
+    e("s_mov_b32 %s, %s" % (s(TMP), s(OFF0)))
+    e("s_mov_b32 %s, %s" % (s(OFF0), s(OFF1)))
+    e("s_mov_b32 %s, %s" % (s(OFF1), s(OFF2)))
+    e("s_mov_b32 %s, %s" % (s(OFF2), s(OFF3)))
+    e("s_mov_b32 %s, %s" % (s(OFF3), s(TMP)))
+    e("s_add_u32 %s, %s, 1" % (s(IT), s(IT)))
+
+
+def p_read_by_all():
+    # every P^T fragment of tile IT is in this wave's registers before any wave overwrites P
+    assert all(("p", f) in lds.issued for f in range(NFRAG)), "barrier ahead of the request for a P^T fragment"
+    lds.drain()
+    e("s_barrier")
+
+
+def iteration_rowless(resc, lab_loop):
+    """--half, a wave without rows: tile IT's share of the tile copies and the V^T fragments, then its 128 columns of P.V of the
+    two row blocks, through the same two barriers per tile as the waves with rows."""
+    e("; ---- iteration of a wave without rows")
+    e("s_mov_b32 %s, 0" % s(VMW))
+    lab_last, lab_nodma, lab_p2 = label("last"), label("nodma"), label("p2")
+    e("s_add_u32 %s, %s, 1" % (s(TMP), s(IT)))
+    e("s_cmp_ge_u32 %s, %s" % (s(TMP), s(NT)))
+    e("s_cbranch_scc1 %s" % lab_last)
+    e("s_add_u32 %s, %s, 3" % (s(TMP), s(IT)))
+    e("s_cmp_ge_u32 %s, %s" % (s(TMP), s(NT)))
+    e("s_cbranch_scc1 %s" % lab_nodma)
+
+    def part1(dma):
+        lds.reset(canon_tags(True))
+        run_slots([lambda: None] * 36, 0, [spread(dma, 0, 35), v_stream(8, (T[0], T[1]))])
+
+    e("s_mov_b32 %s, 1" % s(VMW))
+    dma = dma_tile_lines(TMP, OFF3)
+    part1(dma)
+    state_a = list(lds.pending)
+    e("s_branch %s" % lab_p2)
+    e("%s:" % lab_nodma)
+    part1([None] * len(dma))
+    assert lds.pending == state_a, (lds.pending, state_a)
+    e("%s:" % lab_p2)
+    pv = pv_slots()
+    left = run_slots(pv[:TAIL_AT], 36, [], {36 + B2_AT: [p_read_by_all]})
+    assert not left, left
+    lds.drain()
+    tile_end_wait()
+    e("s_barrier")
+    rotate_buffers()
+    handover(pv[TAIL_AT:], resc, True)
+    e("s_branch %s" % lab_loop)
+    e("%s:" % lab_last)
+    lds.reset(canon_tags(True))
+    for f in range(8):
+        for it_ in v_read_items(f):
+            emit_item(it_)
+    for f in range(8):
+        for it_ in v_conv_items(f, (T[0], T[1])):
+            emit_item(it_)
+    for sl in pv_slots():
+        sl()
+    lds.drain()
 
 
 def iteration(resc, lab_loop):
@@ -639,17 +738,6 @@ def iteration(resc, lab_loop):
     e("s_add_u32 %s, %s, 3" % (s(TMP), s(IT)))
     e("s_cmp_ge_u32 %s, %s" % (s(TMP), s(NT)))
     e("s_cbranch_scc1 %s" % lab_nodma)
-
-    def v_stream(n_conv, tmp):
-        """Part 1: reads of all eight V^T fragments of tile IT (two fragments ahead of their conversion) and conversion of
-        the first n_conv, as one ordered stream: the conversions share two temporaries."""
-        items = v_read_items(0) + v_read_items(1)
-        for f in range(8):
-            if f < n_conv:
-                items += v_conv_items(f, tmp)
-            if f + 2 < 8:
-                items += v_read_items(f + 2)
-        return spread(items, 0, 35)
 
     def part1(dma):
         lds.reset(canon_tags())
@@ -683,40 +771,22 @@ def iteration(resc, lab_loop):
         if MASK:
             mask_wait()
 
-    def p_read_by_all():
-        # every P^T fragment of tile IT is in this wave's registers before any wave overwrites P
-        assert all(("p", f) in lds.issued for f in range(8)), "barrier ahead of the request for a P^T fragment"
-        lds.drain()
-        e("s_barrier")
     sm = softmax_lines()
     streams = [conv2, spread(sm, 38, 36 + PW_AT - 1)]
     left = run_slots(pv[:PW_AT], 36, streams, {38: [qk_done], 36 + B2_AT: [p_read_by_all]})
     assert not left, left
     for it_ in p_write_items():
         emit_item(it_)
-    for sl in pv[PW_AT:28]:
+    for sl in pv[PW_AT:TAIL_AT]:
         sl()
     lds.drain()
-    # the loads of tile IT+2 have landed (those of tile IT+3, issued in this iteration, may still be in flight: loads
-    # complete in order); every wave is done with the buffers of tiles IT (V) and IT+1 (K), and P[IT+1] is written
-    lab_w0, lab_wd = label("w0"), label("wd")
-    e("s_cmp_eq_u32 %s, 0" % s(VMW))
-    e("s_cbranch_scc1 %s" % lab_w0)
-    e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
-    e("s_branch %s" % lab_wd)
-    e("%s:" % lab_w0)
-    e("s_waitcnt vmcnt(0)")
-    e("%s:" % lab_wd)
+    # the loads of tile IT+2 have landed; every wave is done with the buffers of tiles IT (V) and IT+1 (K), and P[IT+1] is written
+    tile_end_wait()
     if CLK:
         lap(1)
     e("s_barrier")
-    e("s_mov_b32 %s, %s" % (s(TMP), s(OFF0)))
-    e("s_mov_b32 %s, %s" % (s(OFF0), s(OFF1)))
-    e("s_mov_b32 %s, %s" % (s(OFF1), s(OFF2)))
-    e("s_mov_b32 %s, %s" % (s(OFF2), s(OFF3)))
-    e("s_mov_b32 %s, %s" % (s(OFF3), s(TMP)))
-    e("s_add_u32 %s, %s, 1" % (s(IT), s(IT)))
-    handover(pv[28:], resc)
+    rotate_buffers()
+    handover(pv[TAIL_AT:], resc)
     e("s_branch %s" % lab_loop)          # (tile IT exists: the iteration before was not the last)
     # ---- last tile: P.V only
     e("%s:" % lab_last)
@@ -857,9 +927,10 @@ def prologue_head(early=None):
 
 def q_image_issue():
     """The 36 coalesced 16-byte loads per lane of this wave's Q operands from the packed image, first thing in the program, so that
-    they are on their way while the prologue sets up its tables (not when FLG bit 6 says the operands wait in LDS)."""
+    they are on their way while the prologue sets up its tables (not when FLG bit 6 says the operands wait in LDS; --half: not
+    for a wave without rows, FLG bit 5)."""
     lab = label("qlds")
-    e("s_bitcmp1_b32 %s, 6" % s(FLG))
+    e("s_bitcmp1_b32 %s, %d" % (s(FLG), 5 if HALF else 6))
     e("s_cbranch_scc1 %s" % lab)
     e("v_lshlrev_b32 %s, 4, %s" % (v(X0), v(LANE)))
     e("s_mul_i32 %s, %s, %d" % (s(S0), s(WAVE), 36 * 1024))
@@ -881,19 +952,20 @@ def main():
     # the packed image since the top of the program (q_image_issue): tile 0.  Tiles 1 and 2 follow; go on as soon as tile 0 and Q
     # are there
     lab_img, lab_qd = label("qimg"), label("qdone")
-    e("s_bitcmp1_b32 %s, 6" % s(FLG))
-    e("s_cbranch_scc0 %s" % lab_img)
-    e("s_mul_i32 %s, %s, %d" % (s(S0), s(WAVE), TILE_BYTES))
-    e("v_add_u32 %s, %s, %s" % (v(X0), s(S0), v(KADDR_LANE)))
-    for ks in range(36):
-        e("ds_read_b128 %s, %s offset:%d" % (v(Q0 + 4 * ks, 4), v(X0), 32 * ks))
-    e("s_waitcnt lgkmcnt(0)")
-    e("s_barrier")
-    e("s_mov_b32 %s, 0" % s(TMP))
-    for ln in dma_tile_lines(TMP, OFF0, True):
-        e(ln)
-    e("s_branch %s" % lab_qd)
-    e("%s:" % lab_img)
+    if not HALF:          # (the launcher gives the two-row-block program an operand image)
+        e("s_bitcmp1_b32 %s, 6" % s(FLG))
+        e("s_cbranch_scc0 %s" % lab_img)
+        e("s_mul_i32 %s, %s, %d" % (s(S0), s(WAVE), TILE_BYTES))
+        e("v_add_u32 %s, %s, %s" % (v(X0), s(S0), v(KADDR_LANE)))
+        for ks in range(36):
+            e("ds_read_b128 %s, %s offset:%d" % (v(Q0 + 4 * ks, 4), v(X0), 32 * ks))
+        e("s_waitcnt lgkmcnt(0)")
+        e("s_barrier")
+        e("s_mov_b32 %s, 0" % s(TMP))
+        for ln in dma_tile_lines(TMP, OFF0, True):
+            e(ln)
+        e("s_branch %s" % lab_qd)
+        e("%s:" % lab_img)
     e("s_mov_b32 %s, 0" % s(TMP))
     for ln in dma_tile_lines(TMP, OFF0, True):
         e(ln)
@@ -952,6 +1024,10 @@ def main():
         e("v_mov_b32 %s, %s" % (v(SLOPE), v(DT[0])))
         e("v_readfirstlane_b32 %s, %s" % (s(K2), v(DT[1])))
     e("s_barrier")                      # tile 0 is complete; every wave has read its hand-off record
+    if HALF:
+        lab_rowless = label("rowless")
+        e("s_bitcmp1_b32 %s, 5" % s(FLG))
+        e("s_cbranch_scc1 %s" % lab_rowless)
     e("v_add_u32 %s, %s, %s" % (v(KADDR), s(OFF0), v(KADDR_LANE)))
     k_warm()
     for slot in qk_slots():
@@ -968,16 +1044,19 @@ def main():
     for it_ in p_write_items():
         emit_item(it_)
     lds.drain()
-    # tile 1 has landed (tile 2 may still be in flight)
-    lab_t1, lab_t1d = label("t1"), label("t1d")
-    e("s_cmp_lt_u32 %s, 3" % s(NT))
-    e("s_cbranch_scc1 %s" % lab_t1)
-    e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
-    e("s_branch %s" % lab_t1d)
-    e("%s:" % lab_t1)
-    e("s_waitcnt vmcnt(0)")
-    e("%s:" % lab_t1d)
-    e("s_barrier")
+
+    def tile1_wait():
+        # tile 1 has landed (tile 2 may still be in flight)
+        lab_t1, lab_t1d = label("t1"), label("t1d")
+        e("s_cmp_lt_u32 %s, 3" % s(NT))
+        e("s_cbranch_scc1 %s" % lab_t1)
+        e("s_waitcnt vmcnt(%d)" % DMA_PER_TILE)
+        e("s_branch %s" % lab_t1d)
+        e("%s:" % lab_t1)
+        e("s_waitcnt vmcnt(0)")
+        e("%s:" % lab_t1d)
+        e("s_barrier")
+    tile1_wait()
     resc = []
     handover([], resc)
     # ------------------------------------------------------------------ main loop
@@ -988,17 +1067,31 @@ def main():
     for lab, back in resc:
         e("%s:" % lab)
         rescale_block(back)
+    if HALF:
+        # ------------------------------------------------------------------ the waves without rows: the same barriers, no K.Q^T, no softmax
+        e("%s:" % lab_rowless)
+        lds.reset([])
+        tile1_wait()
+        resc = []
+        handover([], resc, True)
+        lab_loop = label("loop")
+        e("%s:" % lab_loop)
+        iteration_rowless(resc, lab_loop)
+        e("s_branch %s" % lab_end)
+        for lab, back in resc:
+            e("%s:" % lab)
+            rescale_block(back)
     e("%s:" % lab_end)
     clk_dump()
-    epilogue(4)
+    epilogue(NHB)
     emit()
 
 
 def epilogue(nhb):
-    """1 / l of the rows, then the stores: nhb = 4: the wave's 128 columns of all 128 rows, 1 / l exchanged through LDS; nhb = 1 (the
-    k-split program): 32 rows, every wave has l itself."""
+    """1 / l of the rows, then the stores: nhb = 4 (2: --half): the wave's 128 columns of all 128 (64) rows, 1 / l exchanged through
+    LDS; nhb = 1 (the k-split program): 32 rows, every wave has l itself."""
     # ------------------------------------------------------------------ epilogue
-    if nhb == 4:
+    if nhb > 1:
         e("s_barrier")                  # no wave is still reading rescale factors: their area carries 1 / l next
     e("s_nop 7")
     e("s_nop 7")
@@ -1018,8 +1111,8 @@ def epilogue(nhb):
     e("v_cmp_class_f32 vcc, %s, %s" % (v(T[3]), s(SCLS)))   # finite?
     e("s_nop 1")
     e("v_cndmask_b32 %s, %s, %s, vcc" % (v(T[2]), v(T[2]), v(T[3])))
-    if nhb == 4:
-        # every wave needs 1 / l of all 128 rows: through the rescale-factor area, [lane][hb]
+    if nhb > 1:
+        # every wave needs 1 / l of all 128 rows: through the rescale-factor area, [lane][hb] (a wave without rows leaves a word nobody reads)
         e("v_add_u32 %s, %s, %s" % (v(T[3]), s(W4), v(PADDR)))
         e("ds_write_b32 %s, %s offset:%d" % (v(T[3]), v(T[2]), AOFF - PBUF))
         e("s_waitcnt lgkmcnt(0)")
@@ -1459,7 +1552,7 @@ def ks_main():
 
 
 def emit():
-    print("// generated by gen_decode_cs_asm.py%s%s%s%s%s -- do not edit" % (" --ks" if KS else "", " --f16" if F16KV else "", " --mask" if MASK else "", " --bias" if BIAS else "", " --stream" if STREAM else ""))
+    print("// generated by gen_decode_cs_asm.py%s%s%s%s%s%s -- do not edit" % (" --ks" if KS else "", " --half" if HALF else "", " --f16" if F16KV else "", " --mask" if MASK else "", " --bias" if BIAS else "", " --stream" if STREAM else ""))
     for ln in out:
         print('"%s\\n\\t"' % ln)
     # and nothing of the program is in flight when the compiled code goes on (the mirror image of the wait at the top: an LDS read

@@ -36,7 +36,8 @@ enum { SRC_BF16 = 0, SRC_F16 = 1, SRC_Q8 = 2, SRC_BF16_CVT = 3,     // SRC_BF16_
        SRC_BF16_KS = 6, SRC_F16_KS = 7,                             // and its k-split programs for at most 32 rows (gen_decode_cs_asm.py --ks)
        SRC_BF16_CSQ = 8, SRC_F16_CSQ = 9,                           // column-split programs behind a prologue that rounds Q itself (no pre-pack pass)
        SRC_BF16_CSB = 10, SRC_F16_CSB = 11,                         // column-split programs with mask, ALiBi slope and soft cap (gen_decode_cs_asm.py --mask --bias)
-       SRC_BF16_KSB = 12, SRC_F16_KSB = 13 };                       // k-split programs with mask, ALiBi slope and soft cap (gen_decode_cs_asm.py --ks --mask --bias)
+       SRC_BF16_KSB = 12, SRC_F16_KSB = 13,                         // k-split programs with mask, ALiBi slope and soft cap (gen_decode_cs_asm.py --ks --mask --bias)
+       SRC_BF16_CSH = 14, SRC_F16_CSH = 15 };                       // column-split programs for 33 .. 64 rows: two of the four waves have rows (gen_decode_cs_asm.py --half)
 
 struct KParams {
     const char *    q;

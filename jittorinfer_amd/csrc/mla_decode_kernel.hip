@@ -24,7 +24,7 @@ namespace {
 // The column-split programs (SRC_*_CS) keep behind the four tiles: the P^T exchange buffer (8 KB; the hand-off records share it, they
 // are read before P is first written), the rescale factors (1 KB) and the waves' flag words (64 bytes).
 constexpr bool is_ks(int kvt) { return kvt == SRC_BF16_KS || kvt == SRC_F16_KS || kvt == SRC_BF16_KSB || kvt == SRC_F16_KSB; }
-constexpr bool is_cs(int kvt) { return kvt == SRC_BF16_CS || kvt == SRC_F16_CS || is_ks(kvt) || kvt == SRC_BF16_CSQ || kvt == SRC_F16_CSQ || kvt == SRC_BF16_CSB || kvt == SRC_F16_CSB; }
+constexpr bool is_cs(int kvt) { return kvt == SRC_BF16_CS || kvt == SRC_F16_CS || is_ks(kvt) || kvt == SRC_BF16_CSQ || kvt == SRC_F16_CSQ || kvt == SRC_BF16_CSB || kvt == SRC_F16_CSB || kvt == SRC_BF16_CSH || kvt == SRC_F16_CSH; }
 constexpr int handoff_off(int kvt) { return kvt == SRC_Q8 ? 3 * TILE_BYTES + 2 * Q8_TILE_RAW : 4 * TILE_BYTES; }
 constexpr int SCHED_MAX_SEQ = 256;                   // balanced schedule: sequences per launch
 constexpr int sched_off(int kvt) { return handoff_off(kvt) + (is_cs(kvt) ? 8192 + 1024 + 64 : NTHREADS * 32); }   // prefix sums of the sequences' tile counts
@@ -646,6 +646,16 @@ __device__ __forceinline__ void decode_body() {
         asm volatile(
 #include "mla_decode_ks_f16.inc"
             : : MLA_DECODE_CS_INPUTS : MLA_DECODE_CS_CLOBBERS);
+    } else if constexpr (KVT == SRC_BF16_CSH) {
+        static_assert(!MASK, "the programs for two row blocks have no mask build");
+        asm volatile(
+#include "mla_decode_csh_bf16.inc"
+            : : MLA_DECODE_CS_INPUTS : MLA_DECODE_CS_CLOBBERS);
+    } else if constexpr (KVT == SRC_F16_CSH) {
+        static_assert(!MASK, "the programs for two row blocks have no mask build");
+        asm volatile(
+#include "mla_decode_csh_f16.inc"
+            : : MLA_DECODE_CS_INPUTS : MLA_DECODE_CS_CLOBBERS);
     } else if constexpr (KVT == SRC_BF16_CS || KVT == SRC_BF16_CSQ) {
         asm volatile(
 #include "mla_decode_cs_bf16.inc"
@@ -1129,6 +1139,15 @@ static bool decode_cs_applicable(const KParams & kp, int kv_type) {
     return (tail == 0 || tail > 96) && kp.slot_rows < (1 << 22);
 }
 
+// 33 .. 64 rows per sequence (a decode step of a model with 48 or 64 heads per device), no mask: the column-split program for two row
+// blocks -- K.Q^T and the softmax on the two waves that have rows (36 MFMAs per tile each), P.V on all four (16 each), where the
+// row-split program puts all 68 on each of the two (gen_decode_cs_asm.py --half)
+static bool decode_csh_applicable(const KParams & kp, int kv_type) {
+    if (kv_type != MLA_TYPE_BF16 && kv_type != MLA_TYPE_F16) return false;
+    if (kp.bf16_direct || kp.q_as_q8 || kp.mask || kp.softcap != 0.0f || kp.max_bias > 0.0f) return false;
+    return kp.n_rows > 32 && kp.n_rows <= 64 && kp.slot_rows < (1 << 22);
+}
+
 // At most 32 rows per sequence (a decode step of a 16- or 32-head model): the four waves split the 576 columns of K.Q^T between
 // them instead of leaving it to the one wave that has rows (gen_decode_cs_asm.py --ks)
 static bool decode_ks_applicable(const KParams & kp, int kv_type) {
@@ -1158,7 +1177,8 @@ hipError_t launch_decode_fast(const KParams & kp_in, int kv_type, dim3 grid, hip
     // column-split programs (every wave computes S for its own 32 rows and P.V for its own 128 columns): blocks of 128 rows in
     // which all four waves have rows, not the Q8_0 expansion; bf16 K enters as bf16, so the Q image is the bf16 one
     const bool cs = decode_cs_applicable(kp_in, kv_type), ks = decode_ks_applicable(kp_in, kv_type);
-    const bool bf16_cvt = !cs && !kp_in.bf16_direct && kp_in.n_rows > 32;
+    const bool csh = !tok && decode_csh_applicable(kp_in, kv_type);
+    const bool bf16_cvt = !cs && !csh && !kp_in.bf16_direct && kp_in.n_rows > 32;
     // Q without the pre-pack pass: the k-split programs always round their quarter of Q themselves (144 columns of 32 rows per wave,
     // fetched behind the first tile loads); the column-split programs when every block of 128 rows is visited by one workgroup (one
     // split: a prefill chunk) -- the f32 rows are twice the bytes of the operand image, which pays when they are read once and not
@@ -1246,6 +1266,7 @@ hipError_t launch_decode_fast(const KParams & kp_in, int kv_type, dim3 grid, hip
         kp.softcap = kp.softcap != 0.0f ? -2.0f * kp.softcap : 0.0f;   // (not -0: the program tests the bits)
         return kv_type == MLA_TYPE_F16 ? launch_variant<SRC_F16_CSB, true>(kp, grid, st) : launch_variant<SRC_BF16_CSB, true>(kp, grid, st);
     }
+    if (csh) return kv_type == MLA_TYPE_F16 ? launch_variant<SRC_F16_CSH, false>(kp, grid, st) : launch_variant<SRC_BF16_CSH, false>(kp, grid, st);
     if (cs && q_in_kernel && kv_type == MLA_TYPE_F16) return m ? launch_variant<SRC_F16_CSQ, true>(kp, grid, st) : launch_variant<SRC_F16_CSQ, false>(kp, grid, st);
     if (cs && q_in_kernel)             return m ? launch_variant<SRC_BF16_CSQ, true>(kp, grid, st) : launch_variant<SRC_BF16_CSQ, false>(kp, grid, st);
     if (cs && m && stream) return kv_type == MLA_TYPE_F16 ? launch_variant<SRC_F16_CS, true, true>(kp, grid, st) : launch_variant<SRC_BF16_CS, true, true>(kp, grid, st);

@@ -195,7 +195,9 @@ def test_planner_schedules_without_gpu():
                                             ("gen_decode_cs_asm.py", ["--ks", "--mask", "--stream"], "mla_decode_ks_bf16_mask_nt.inc"),
                                             ("gen_decode_cs_asm.py", ["--ks", "--f16", "--mask", "--stream"], "mla_decode_ks_f16_mask_nt.inc"),
                                             ("gen_decode_cs_asm.py", ["--ks", "--mask", "--bias"], "mla_decode_ks_bf16_bias.inc"),
-                                            ("gen_decode_cs_asm.py", ["--ks", "--f16", "--mask", "--bias"], "mla_decode_ks_f16_bias.inc")])
+                                            ("gen_decode_cs_asm.py", ["--ks", "--f16", "--mask", "--bias"], "mla_decode_ks_f16_bias.inc"),
+                                            ("gen_decode_cs_asm.py", ["--half"], "mla_decode_csh_bf16.inc"),
+                                            ("gen_decode_cs_asm.py", ["--half", "--f16"], "mla_decode_csh_f16.inc")])
 def test_committed_wave_programs_are_what_the_generator_emits(gen, flags, name):
     """The instruction streams the decode kernel includes are generated files: each equals the generator's output.  None of
     them touches v252..v255: the asm block's clobber list ends at v251, and the compiler keeps there what lives across the

@@ -424,6 +424,34 @@ def test_few_rows_k_split_program(gpu, k_type):
     print(U.check(a, want, "few rows, V := K"))
 
 
+@pytest.mark.parametrize("k_type", [O.TYPE_BF16, O.TYPE_F16])
+def test_two_row_blocks_column_split_program(gpu, k_type):
+    """33 to 64 attention rows per sequence and no mask (a decode step of a model with 48 or 64 heads per device, a few query tokens
+    of 16 heads): the column-split program in which two of the four waves have rows -- they multiply K.Q^T and run the softmax, all
+    four take their 128 columns of P.V.  Paged with KV splits (f16 and f32 partials) and one piece per sequence (final rows), lengths
+    that end inside a tile, a contiguous cache, the 576-wide V in its two passes."""
+    rng = np.random.default_rng(101)
+    lens = [700, 129, 300, 1, 33, 2048]
+    pool, bt, seqs = U.make_paged(rng, lens, k_type)
+    f64 = k_type == O.TYPE_F16     # (ggml-cpu's f16 accumulator: the f32-accumulating kernels are held to the exact value)
+    ref = O.flash_attn_ext_f64 if f64 else O.flash_attn_ext
+    for n_head, n_tok in ((64, 1), (48, 1), (33, 1), (16, 4), (20, 2)):
+        q = rng.standard_normal((len(lens), n_head, n_tok, 576)).astype(np.float32)
+        want = np.stack([ref(q[b:b + 1], k[None], k_type, dv=512, scale=U.SCALE)[0] for b, k in enumerate(seqs)])
+        for n_splits in (0, 1, 3):
+            a = _run(gpu, q, pool, k_type, bt=bt, lens=lens, scale=U.SCALE, n_splits=n_splits)
+            print(n_head, n_tok, n_splits, U.check(a[..., :512], want, "two row blocks"))
+    q = rng.standard_normal((len(lens), 64, 1, 576)).astype(np.float32)
+    a = _run(gpu, q, pool, k_type, dv=576, bt=bt, lens=lens, scale=U.SCALE)
+    want = np.stack([ref(q[b:b + 1], k[None], k_type, dv=576, scale=U.SCALE)[0] for b, k in enumerate(seqs)])
+    print(U.check(a, want, "two row blocks, V := K"))
+    q = rng.standard_normal((3, 64, 1, 576)).astype(np.float32)
+    k = U.encode_kv(rng.standard_normal((3, 1000, 576)).astype(np.float32), k_type)
+    for n_splits in (0, 4):
+        a = _run(gpu, q, k, k_type, scale=U.SCALE, n_splits=n_splits)
+        print(n_splits, U.check(a[..., :512], ref(q, k, k_type, dv=512, scale=U.SCALE), "two row blocks, contiguous cache"))
+
+
 def test_q8_0_cache_with_arbitrary_block_scales(gpu):
     """A Q8_0 cache as the reference's quantizer leaves it -- every block its own scale d = amax / 127, not the power of two of
     BASELINE's config 5 -- through the paged decode path (128 heads, ragged lengths, KV splits) and through a masked launch:

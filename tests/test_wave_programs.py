@@ -57,10 +57,15 @@ class Coverage:
         """Branches that did not go both ways.  One cannot: the rescale test behind the first tile of the column-split programs (the
         first softmax clears its flag: the accumulators are still zero), the first branch to a label of that kind."""
         out = []
-        first_resc = next((pc for pc, ins in enumerate(wg.instrs) if ins[0] == "s_cbranch_scc1" and ins[1][0][1].startswith("Lresc")), None)
+        resc = [pc for pc, ins in enumerate(wg.instrs) if ins[0] == "s_cbranch_scc1" and ins[1][0][1].startswith("Lresc")]
+        first_resc = set(resc[:1])
+        # (the programs for two row blocks: the waves without rows run a loop of their own, with a first tile of its own)
+        rowless = next((at for lab, at in wg.labels.items() if lab.startswith("Lrowless")), None)
+        if rowless is not None:
+            first_resc |= set([pc for pc in resc if pc >= rowless][:1])
         for pc, ins in enumerate(wg.instrs):
             if ins[0].startswith("s_cbranch") and self.seen.get(pc, set()) != {True, False}:
-                if pc == first_resc and self.seen.get(pc) == {False} and "_cs_" in wg.name:
+                if pc in first_resc and self.seen.get(pc) == {False} and ("_cs_" in wg.name or "_csh_" in wg.name):
                     continue
                 out.append((pc, ins[3], sorted(self.seen.get(pc, set()))))
         return out
@@ -124,10 +129,11 @@ def run_cs(name, cov, f16, mask_build=False, bias_build=False, n_rows=128, kv=(0
     assert not findings, "%s: %s" % (name, findings[:5])
     want, m_want, l_want = piece.reference(scale=scale, softcap=softcap, slopes=slopes, v0=64 if v_col0 else 0)   # (V = columns 64 .. 575 in the second pass of a 576-wide V)
     if f32_rows:
-        got = piece.gmem.array("out").view(np.float32).reshape(128, 512)[:n_rows].astype(np.float64)
+        full = piece.gmem.array("out").view(np.float32).reshape(128, 512).astype(np.float64)
     else:   # f16 partials, [column / 8][row][8]
-        got = piece.gmem.array("out").view(np.float16).reshape(64, 128, 8).transpose(1, 0, 2).reshape(128, 512)[:n_rows].astype(np.float64)
-    _check(got, want, name)
+        full = piece.gmem.array("out").view(np.float16).reshape(64, 128, 8).transpose(1, 0, 2).reshape(128, 512).astype(np.float64)
+    _check(full[:n_rows], want, name)
+    assert not full[n_rows:].any(), "%s: rows that do not exist were stored" % name
     if not final:
         ml = piece.gmem.array("ml").view(np.float32).reshape(128, 2)[:n_rows].astype(np.float64)
         lse = ml[:, 0] + np.log2(ml[:, 1])
@@ -156,6 +162,30 @@ def test_column_split_programs(name, f16):
     cov = Coverage()
     for k, sc in enumerate(CS_SCENARIOS):
         wg = run_cs(name, cov, f16, seed=k, **sc)
+    assert not cov.missing(wg), cov.missing(wg)
+    _only_register_loads_ahead_of_tile_copies(cov)
+
+
+CSH_SCENARIOS = [
+    dict(kv=(0, 128)),                                                     # four tiles: one round of tile loads in the loop, then none
+    dict(kv=(0, 32), final=False, f32_rows=False),                         # one tile, f16 partial rows
+    dict(kv=(128, 128 + 64), seq_len=400, final=False, n_rows=48),         # two tiles inside a longer sequence, f32 partial rows; 48 heads
+    dict(kv=(96, 96 + 96 - 5), paged=True, n_rows=33),                     # a split that starts inside a page; ragged end; one row in the second block
+    dict(kv=(0, 7 * 32 + 1), paged=False),                                 # contiguous cache, eight tiles, one key in the last
+    dict(kv=(0, 160), boost=True),                                         # the running maxima move: accumulators rescaled, in both loops
+    dict(kv=(0, 96), n_rows=40, final=False, f32_rows=False),
+    dict(kv=(0, 96), v_col0=True),                                         # second pass of a 576-wide V
+    dict(kv=(256, 256 + 19), seq_len=256 + 19, n_rows=64),                 # one ragged tile
+]
+
+
+@pytest.mark.parametrize("name,f16", [("mla_decode_csh_bf16.inc", False), ("mla_decode_csh_f16.inc", True)])
+def test_column_split_programs_for_two_row_blocks(name, f16):
+    """33 .. 64 rows (a decode step of a model with 48 or 64 heads per device): waves 0 and 1 have rows, waves 2 and 3 copy their share
+    of the tiles and multiply their 128 columns of P.V, in a loop of their own with the same barriers."""
+    cov = Coverage()
+    for k, sc in enumerate(CSH_SCENARIOS):
+        wg = run_cs(name, cov, f16, seed=70 + k, **dict(dict(n_rows=64), **sc))
     assert not cov.missing(wg), cov.missing(wg)
     _only_register_loads_ahead_of_tile_copies(cov)
 
