@@ -26,6 +26,8 @@ F16 = "--f16" in sys.argv or Q8 or CVTB  # f16 KV: f16 MFMA, single P (no lo hal
 MF = "v_mfma_f32_32x32x16_f16" if F16 else "v_mfma_f32_32x32x16_bf16"
 CVT = "v_cvt_pk_f16_f32" if F16 else "v_cvt_pk_bf16_f32"
 SPLIT = not F16
+BIAS = "--bias" in sys.argv  # mask builds of the f16 kinds: ALiBi slope per head on the mask values, tanh soft cap on the logits (see bias_block)
+assert (MASK and not SPLIT and not CLK) or not BIAS
 
 PITCH = 1168
 TILE_BYTES = 32 * PITCH
@@ -68,7 +70,8 @@ KADDR_LANE, VADDR_LANE, MRUN, LRUN, NEGM = 236, 237, 238, 239, 240
 DROW, DCOL, VOFF, PAGES = 241, 242, 243, 244
 LANE, KADDR, VADDR, TMAX = 245, 246, 247, 248
 X0, X1, X2 = 249, 250, 251
-N_VGPR = 252
+SLOPE = 252         # bias builds: ALiBi slope of this lane's row (one register more than the other builds own)
+N_VGPR = 253 if BIAS else 252
 # ---- SGPR map (all inside the clobbered range s40..s79)
 KV, BT, KVB, KVE, CL2, NPP, NB1, FLG = 40, 42, 44, 45, 46, 47, 48, 49
 NT, IT, OFF0, OFF1, OFF2, WAVE, TB, TMP, NVM1 = 50, 51, 52, 53, 54, 55, 56, 58, 59
@@ -78,6 +81,8 @@ RAWB, DSTB, DZ = 197, 198, 199                    # Q8_0 builds: per-lane raw wi
 SCL, L2E, MSK = (82, 73, 80) if Q8 else (77, 73, 78)   # mask builds: scale, log2(e) (the register of SCLS until the epilogue), mask base (QP's registers once Q is loaded;
                                                         # Q8_0 builds keep the dequantizer's scalars there and take s80..s83)
 ONES = 83   # f16 builds: packed (1.0, 1.0)
+K1, K2 = CL2, NPP   # bias builds: 2 log2(e) scale / softcap (the input that carries c_log2 elsewhere) and -2 softcap, 0 = no soft cap
+                    # (NPP's register once the page ids are clamped; until then it waits in the upper half of RSC)
 EXS, S0, S1, S2, S3, DMAB, NVAL, THR, PG0, RSC, SPITCH, SCLS, OFF3, VMW, OSTR, QP = 60, 62, 63, 64, 65, 66, 67, 68, 69, 70, 72, 73, 74, 75, 76, 78
 
 out = []
@@ -529,6 +534,9 @@ def softmax_lines(sreg):
     if MASK:
         # u = s * scale + mask (ggml-cpu.c:12048-12057 order), element k = token 8(k/4) + 4g + k%4
         for k in range(16):
+            if BIAS:   # the logits were scaled (and capped) by bias_block(): u += slope * mask
+                L.append("v_fma_mix_f32 %s, %s, %s, %s op_sel:[%d,0,0] op_sel_hi:[1,0,0]" % (v(sreg + k), v(MKR[2 * (k // 4) + (k % 4) // 2]), v(SLOPE), v(sreg + k), k % 2))
+                continue
             t = T[5 + (k & 1)]
             L.append("v_cvt_f32_f16_sdwa %s, %s dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:WORD_%d" % (v(t), v(MKR[2 * (k // 4) + (k % 4) // 2]), k % 2))
             L.append("v_fma_f32 %s, %s, %s, %s" % (v(sreg + k), v(sreg + k), s(SCL), v(t)))
@@ -628,6 +636,33 @@ def rescale_block(ret_label):
     e("s_branch %s" % ret_label)
 
 
+def bias_block(sreg):
+    """Bias builds (ggml-cpu.c:12041-12057: u = softcap * tanh(s * scale / softcap) + slope(head) * mask), once the scores of a tile are
+    complete: s <- s * scale, or, with a soft cap, -2 softcap / (1 + 2^(s K1)) = softcap * tanh(s * scale / softcap) - softcap (a
+    constant added to every logit of a row changes neither the probabilities nor the split-K merge).  The launcher hands scale /
+    softcap, 2 log2(e) scale / softcap and -2 softcap where the plain builds find scale, scale log2(e) and nothing.  Ahead of
+    mask_tail(): the cap is bounded, so a key past the end of the sequence that was already at -inf would come back with a finite
+    logit."""
+    lab_plain, lab_done = label("nocap"), label("capd")
+    e("s_cmp_eq_u32 %s, 0" % s(K2))
+    e("s_cbranch_scc1 %s" % lab_plain)
+    for k in range(16):
+        e("v_mul_f32 %s, %s, %s" % (v(sreg + k), s(K1), v(sreg + k)))
+    for k in range(16):
+        e("v_exp_f32 %s, %s" % (v(sreg + k), v(sreg + k)))
+    for k in range(16):
+        e("v_add_f32 %s, 1.0, %s" % (v(sreg + k), v(sreg + k)))
+    for k in range(16):
+        e("v_rcp_f32 %s, %s" % (v(sreg + k), v(sreg + k)))
+    for k in range(16):
+        e("v_mul_f32 %s, %s, %s" % (v(sreg + k), s(K2), v(sreg + k)))
+    e("s_branch %s" % lab_done)
+    e("%s:" % lab_plain)
+    for k in range(16):
+        e("v_mul_f32 %s, %s, %s" % (v(sreg + k), s(SCL), v(sreg + k)))
+    e("%s:" % lab_done)
+
+
 def mask_tail(sreg):
     """Last tile only: tokens >= n_valid get score -inf.  element k is token 8*(k/4) + 4g + k%4."""
     lab = label("full")
@@ -711,6 +746,8 @@ def iteration(g_cur, g_next, tag):
     e("s_nop 7")                       # the last QK^T MFMA has written g_next
     if len(head) < 2:
         e("s_nop 7")
+    if BIAS:
+        bias_block(g_next)             # (ahead of mask_tail: the soft cap maps -inf to a finite value)
     mask_tail(g_next)
     if MASK:
         lab_m0, lab_md = label("m0"), label("md")
@@ -839,6 +876,10 @@ def main():
         e("v_mov_b32 %s, %s" % (v(MLPTR + 1), v(T[5])))
     if MASK:
         e("v_mov_b32 %s, %s" % (v(MOFF), v(T[0])))
+    if BIAS:
+        # the last 8 bytes of the record: the slope of this thread's row's head, and -2 softcap
+        e("v_mov_b32 %s, %s" % (v(SLOPE), v(T[6])))
+        e("v_readfirstlane_b32 %s, %s" % (s(RSC + 1), v(T[7])))
     # lane geometry
     e("v_and_b32 %s, 31, %s" % (v(X0), v(LANE)))                       # rl
     e("v_lshrrev_b32 %s, 5, %s" % (v(X1), v(LANE)))                    # g
@@ -954,6 +995,8 @@ def main():
         # that are never used; clamped so that no address leaves the pool
         e("v_max_i32 %s, 0, %s" % (v(PAGES), v(PAGES)))
         e("v_min_i32 %s, %s, %s" % (v(PAGES), s(NPP), v(PAGES)))
+        if BIAS:
+            e("s_mov_b32 %s, %s" % (s(K2), s(RSC + 1)))
     stamp(6)
     if Q8:
         # ------------------------------------------------------------------ Q8_0: per-lane offsets of the dequantizer
@@ -1185,6 +1228,8 @@ def main():
     e("s_min_u32 %s, %s, 32" % (s(NVAL), s(NVAL)))
     e("s_nop 7")
     e("s_nop 7")
+    if BIAS:
+        bias_block(SA)
     mask_tail(SA)
     for ln in softmax_lines(SA):
         e(ln)
@@ -1318,7 +1363,7 @@ def main():
 
     e("%s:" % LAB_EXIT)
 
-    print("// generated by gen_decode_asm.py%s%s -- do not edit" % (" --q8" if Q8 else " --f16" if "--f16" in sys.argv else "", " --mask" if MASK else ""))
+    print("// generated by gen_decode_asm.py%s%s%s -- do not edit" % (" --q8" if Q8 else " --f16" if "--f16" in sys.argv else "", " --mask" if MASK else "", " --bias" if BIAS else ""))
     for ln in out:
         print('"%s\\n\\t"' % ln)
     # and nothing of the program is in flight when the compiled code goes on (the mirror image of the wait at the top: an LDS read

@@ -123,6 +123,7 @@ constexpr int lds_total(int kvt) { return sched_off(kvt) + (2 * SCHED_MAX_SEQ + 
 #define MLA_DECODE_CS_BIAS_INPUTS MLA_DECODE_CS_INPUTS, [msk] "s"(mask_base), [scl] "s"(s_scale)
 #define MLA_DECODE_CS_BIAS_CLOBBERS MLA_DECODE_CS_CLOBBERS, "v252"
 #define MLA_DECODE_KS_BIAS_CLOBBERS MLA_DECODE_KS_CLOBBERS, "v252"
+#define MLA_DECODE_BIAS_CLOBBERS MLA_DECODE_CLOBBERS, "v252"
 
 #define MLA_DECODE_INPUTS                                                                                          \
     [kv] "s"(kv_base), [bt] "s"(bt_row), [kvb] "s"(s_kvb), [kve] "s"(s_kve), [cl2] "s"(c_log2_bits), [npp] "s"(s_npp), \
@@ -286,8 +287,10 @@ __device__ __forceinline__ void stage_q_rows(const KP & p, int b, int row0, int 
 // costs a piece 0.2 to 0.5 us of load latency, so only the kernels with two bodies ask for it.
 typedef const __attribute__((address_space(4))) KParams KParamsArg;
 // STREAM (masked column-split and k-split programs): the build whose tile copies carry the non-temporal hint
-template <int KVT, bool MASK, int KOFF, bool OPAQUE, bool STREAM = false>
+// RSBIAS (masked row-split programs of the f16 kinds: SRC_F16, SRC_BF16_CVT, SRC_Q8): the build with ALiBi slope and soft cap
+template <int KVT, bool MASK, int KOFF, bool OPAQUE, bool STREAM = false, bool RSBIAS = false>
 __device__ __forceinline__ void decode_body() {
+    static_assert(!RSBIAS || (MASK && (KVT == SRC_F16 || KVT == SRC_BF16_CVT || KVT == SRC_Q8)), "bias builds of the row-split programs");
     KParamsArg * p_ptr = (KParamsArg *) ((const __attribute__((address_space(4))) char *) __builtin_amdgcn_kernarg_segment_ptr() + KOFF);
     KParamsArg & p = *p_ptr;
     constexpr int HANDOFF_OFF = handoff_off(KVT);
@@ -526,7 +529,7 @@ __device__ __forceinline__ void decode_body() {
     // 2 log2(e) scale / softcap into p.c_log2_bits and -2 softcap (0: no soft cap) into p.softcap; the last 8 bytes of the hand-off
     // record are the slope of this thread's row's head (ggml-cpu.c:11985-11989, :12006-12008) and that -2 softcap; see
     // gen_decode_cs_asm.py
-    constexpr bool BIAS = KVT == SRC_BF16_CSB || KVT == SRC_F16_CSB || KVT == SRC_BF16_KSB || KVT == SRC_F16_KSB;
+    constexpr bool BIAS = RSBIAS || KVT == SRC_BF16_CSB || KVT == SRC_F16_CSB || KVT == SRC_BF16_KSB || KVT == SRC_F16_KSB;
     // (the k-split programs: every wave works on the same 32 rows, its lanes' rows do not depend on the wave)
     constexpr bool KS_ROWS = is_ks(KVT);
     float slope = 1.0f;
@@ -664,6 +667,18 @@ __device__ __forceinline__ void decode_body() {
         asm volatile(
 #include "mla_decode_cs_f16.inc"
             : : MLA_DECODE_CS_INPUTS : MLA_DECODE_CS_CLOBBERS);
+    } else if constexpr (KVT == SRC_Q8 && RSBIAS) {
+        asm volatile(
+#include "mla_decode_asm_q8_bias.inc"
+            : : MLA_DECODE_INPUTS : MLA_DECODE_BIAS_CLOBBERS);
+    } else if constexpr (KVT == SRC_BF16_CVT && RSBIAS) {
+        asm volatile(
+#include "mla_decode_asm_cvt_bias.inc"
+            : : MLA_DECODE_INPUTS : MLA_DECODE_BIAS_CLOBBERS);
+    } else if constexpr (KVT == SRC_F16 && RSBIAS) {
+        asm volatile(
+#include "mla_decode_asm_f16_bias.inc"
+            : : MLA_DECODE_INPUTS : MLA_DECODE_BIAS_CLOBBERS);
     } else if constexpr (KVT == SRC_Q8 && MASK) {
         asm volatile(
 #include "mla_decode_asm_q8_mask.inc"
@@ -701,8 +716,8 @@ __device__ __forceinline__ void decode_body() {
   }
 }
 
-template <int KVT, bool MASK, bool STREAM = false>
-__global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams) { decode_body<KVT, MASK, 0, false, STREAM>(); }   // (the body reads the argument segment)
+template <int KVT, bool MASK, bool STREAM = false, bool RSBIAS = false>
+__global__ void __launch_bounds__(NTHREADS) mla_decode_kernel(const KParams) { decode_body<KVT, MASK, 0, false, STREAM, RSBIAS>(); }   // (the body reads the argument segment)
 
 // A masked launch of few heads issued in two forms (the launcher's comment tells why): pb describes it as row blocks of 128 rows
 // (balanced == 2), pt token by token (balanced == 3: every query token a sequence of one token, its mask row that sequence's
@@ -1068,11 +1083,11 @@ bool decode_fast_applicable(const mla_attn_args * a) {
     const bool q8_copy = decode_fast_q8_copy_rows(a) > 0;
     if (a->kv_type == MLA_TYPE_Q8_0 && !q8_copy && !q8_raw_tiles_ok(a)) return false;
     if (a->logit_softcap != 0.0f || a->max_bias > 0.0f) {
-        // ALiBi / soft cap: the masked column-split programs (blocks of 128 rows in which every wave has rows) and the masked k-split
-        // programs (at most 32 rows) have a build for them, over 16-bit rows; everything else goes to the general kernel
-        const int64_t n_rows = (int64_t) a->n_tok * a->n_head, tail = n_rows % 128;
-        if (!a->mask || a->kv_type == MLA_TYPE_Q8_0 || (a->flags & MLA_FLAG_BF16_DIRECT)) return false;
-        if (!(n_rows <= 32 || tail == 0 || tail > 96) || n_rows >= (1 << 22)) return false;
+        // ALiBi / soft cap: every masked program but the hi + lo bf16 one has a build for them; a launch without a mask goes to the
+        // general kernel
+        const int64_t n_rows = (int64_t) a->n_tok * a->n_head;
+        if (!a->mask || (a->flags & MLA_FLAG_BF16_DIRECT)) return false;
+        if (n_rows >= (1 << 22)) return false;
         if (a->logit_softcap != 0.0f && !(a->logit_softcap > 0.0f && a->logit_softcap < INFINITY)) return false;
     }
     // 16-bit rows must be packed: the per-lane offsets of the tile copy are kept as 16-bit values (31 * 1152 + 1136 < 65536)
@@ -1121,12 +1136,12 @@ hipError_t launch_q8_to_f16(const char * src, int64_t src_nb1, int64_t src_nb3, 
     return hipGetLastError();
 }
 
-template <int KVT, bool MASK, bool STREAM = false>
+template <int KVT, bool MASK, bool STREAM = false, bool RSBIAS = false>
 static hipError_t launch_variant(const KParams & kp, dim3 grid, hipStream_t st) {
     static bool attr_done[MLA_MAX_DEVICES];
-    const hipError_t e = raise_lds_limit((const void *) mla_decode_kernel<KVT, MASK, STREAM>, attr_done);
+    const hipError_t e = raise_lds_limit((const void *) mla_decode_kernel<KVT, MASK, STREAM, RSBIAS>, attr_done);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((mla_decode_kernel<KVT, MASK, STREAM>), grid, dim3(NTHREADS), (size_t) lds_total(KVT), st, kp);
+    hipLaunchKernelGGL((mla_decode_kernel<KVT, MASK, STREAM, RSBIAS>), grid, dim3(NTHREADS), (size_t) lds_total(KVT), st, kp);
     return hipGetLastError();
 }
 
@@ -1184,7 +1199,7 @@ hipError_t launch_decode_fast(const KParams & kp_in, int kv_type, dim3 grid, hip
     // split: a prefill chunk) -- the f32 rows are twice the bytes of the operand image, which pays when they are read once and not
     // when the 8 splits of a decode step each read them.  Ahead of such a launch only the scan of the mask extents (masked launches)
     // is left, and nothing at all ahead of an unmasked one.
-    const bool bias = kp_in.softcap != 0.0f || kp_in.max_bias > 0.0f;   // (decode_fast_applicable let it through: masked, column-split)
+    const bool bias = kp_in.softcap != 0.0f || kp_in.max_bias > 0.0f;   // (decode_fast_applicable let it through: masked)
     const bool q_in_kernel = ks || (cs && !bias && kp_in.n_splits == 1 && !kp_in.balanced);
     KParams kp = kp_in;
     kp.q_in_kernel = q_in_kernel ? 1 : 0;
@@ -1244,28 +1259,25 @@ hipError_t launch_decode_fast(const KParams & kp_in, int kv_type, dim3 grid, hip
         if (cs) return tok_ks ? launch_dual<SRC_BF16_CS, SRC_BF16_KS>(kp, kt, grid, st) : launch_dual<SRC_BF16_CS, SRC_BF16_CVT>(kp, kt, grid, st);
         return tok_ks ? launch_dual<SRC_BF16_CVT, SRC_BF16_KS>(kp, kt, grid, st) : launch_dual<SRC_BF16_CVT, SRC_BF16_CVT>(kp, kt, grid, st);
     }
-    if (kv_type == MLA_TYPE_Q8_0) return m ? launch_variant<SRC_Q8, true>(kp, grid, st) : launch_variant<SRC_Q8, false>(kp, grid, st);
-    if (ks && bias) {
-        if (!m) return hipErrorInvalidValue;
+    if (bias) {
+        // ALiBi / soft cap (decode_fast_applicable let it through: masked): the bias build of whatever program the launch would run
+        // without them -- k-split, column-split, or the row-split program of an f16 kind (Q8_0 cells, a row block in which some
+        // waves have no rows)
+        if (!m || kp.bf16_direct) return hipErrorInvalidValue;
         // what the bias builds expect in place of scale, scale * log2(e) and softcap (see the kernel)
         if (kp.softcap != 0.0f) kp.scale = kp.scale / kp.softcap;
         const float k1 = 2.0f * 1.44269504088896340736f * kp.scale;
         kp.c_log2_bits = __builtin_bit_cast(int, k1);
         kp.softcap = kp.softcap != 0.0f ? -2.0f * kp.softcap : 0.0f;   // (not -0: the program tests the bits)
-        return kv_type == MLA_TYPE_F16 ? launch_variant<SRC_F16_KSB, true>(kp, grid, st) : launch_variant<SRC_BF16_KSB, true>(kp, grid, st);
+        if (kv_type == MLA_TYPE_Q8_0) return launch_variant<SRC_Q8, true, false, true>(kp, grid, st);
+        if (ks) return kv_type == MLA_TYPE_F16 ? launch_variant<SRC_F16_KSB, true>(kp, grid, st) : launch_variant<SRC_BF16_KSB, true>(kp, grid, st);
+        if (cs) return kv_type == MLA_TYPE_F16 ? launch_variant<SRC_F16_CSB, true>(kp, grid, st) : launch_variant<SRC_BF16_CSB, true>(kp, grid, st);
+        return kv_type == MLA_TYPE_F16 ? launch_variant<SRC_F16, true, false, true>(kp, grid, st) : launch_variant<SRC_BF16_CVT, true, false, true>(kp, grid, st);
     }
+    if (kv_type == MLA_TYPE_Q8_0) return m ? launch_variant<SRC_Q8, true>(kp, grid, st) : launch_variant<SRC_Q8, false>(kp, grid, st);
     if (ks && m && stream) return kv_type == MLA_TYPE_F16 ? launch_variant<SRC_F16_KS, true, true>(kp, grid, st) : launch_variant<SRC_BF16_KS, true, true>(kp, grid, st);
     if (ks && m) return kv_type == MLA_TYPE_F16 ? launch_variant<SRC_F16_KS, true>(kp, grid, st) : launch_variant<SRC_BF16_KS, true>(kp, grid, st);
     if (ks) return kv_type == MLA_TYPE_F16 ? launch_variant<SRC_F16_KS, false>(kp, grid, st) : launch_variant<SRC_BF16_KS, false>(kp, grid, st);
-    if (bias) {
-        if (!cs || !m) return hipErrorInvalidValue;
-        // what the bias builds expect in place of scale, scale * log2(e) and softcap (see the kernel)
-        if (kp.softcap != 0.0f) kp.scale = kp.scale / kp.softcap;
-        const float k1 = 2.0f * 1.44269504088896340736f * kp.scale;
-        kp.c_log2_bits = __builtin_bit_cast(int, k1);
-        kp.softcap = kp.softcap != 0.0f ? -2.0f * kp.softcap : 0.0f;   // (not -0: the program tests the bits)
-        return kv_type == MLA_TYPE_F16 ? launch_variant<SRC_F16_CSB, true>(kp, grid, st) : launch_variant<SRC_BF16_CSB, true>(kp, grid, st);
-    }
     if (csh) return kv_type == MLA_TYPE_F16 ? launch_variant<SRC_F16_CSH, false>(kp, grid, st) : launch_variant<SRC_BF16_CSH, false>(kp, grid, st);
     if (cs && q_in_kernel && kv_type == MLA_TYPE_F16) return m ? launch_variant<SRC_F16_CSQ, true>(kp, grid, st) : launch_variant<SRC_F16_CSQ, false>(kp, grid, st);
     if (cs && q_in_kernel)             return m ? launch_variant<SRC_BF16_CSQ, true>(kp, grid, st) : launch_variant<SRC_BF16_CSQ, false>(kp, grid, st);

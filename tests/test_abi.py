@@ -147,9 +147,11 @@ def test_planner_schedules_without_gpu():
     assert rc == 0 and info.variant == 2 and info.n_passes == 2 and info.balanced == 1
     rc, info, _ = _plan(dv=576, max_bias=8.0, mask=131072, mask_nb1=16384, mask_ne0=8192)   # ALiBi with a mask over 16-bit rows: the pipelined kernel has a build for it
     assert rc == 0 and info.variant == 2 and info.n_passes == 2
-    rc, info, _ = _plan(dv=576, max_bias=8.0, mask=131072, mask_nb1=16384, mask_ne0=8192, kv_type=J.MLA_TYPE_Q8_0, kv_nb1=612)   # not over Q8_0 rows: the general kernel, 2 x 288 columns
+    rc, info, _ = _plan(dv=576, max_bias=8.0, mask=131072, mask_nb1=16384, mask_ne0=8192, kv_type=J.MLA_TYPE_Q8_0, kv_nb1=612)   # and over Q8_0 rows
+    assert rc == 0 and info.variant == 2 and info.n_passes == 2
+    rc, info, _ = _plan(dv=576, max_bias=8.0, mask=131072, mask_nb1=16384, mask_ne0=8192, flags=J.MLA_FLAG_BF16_DIRECT)   # not for the hi + lo bf16 program: the general kernel, 2 x 288 columns
     assert rc == 0 and info.variant == 0 and info.n_passes == 2
-    rc, info, _ = _plan(logit_softcap=30.0)                      # softcap: general kernel, 64 rows per workgroup
+    rc, info, _ = _plan(logit_softcap=30.0)                      # softcap without a mask: general kernel, 64 rows per workgroup
     assert rc == 0 and info.variant == 0 and info.rows_per_wg == 64
     one = dict(n_seq=1, n_head=16, block_table=0, seq_lens=0, bt_stride=0, kv_nb3=0, kv_type=J.MLA_TYPE_F16)
     rc, info, _ = _plan(n_kv=1024, **one)                        # configs[0]: one short sequence, splits of one 32-key tile
@@ -196,6 +198,9 @@ def test_planner_schedules_without_gpu():
                                             ("gen_decode_cs_asm.py", ["--ks", "--f16", "--mask", "--stream"], "mla_decode_ks_f16_mask_nt.inc"),
                                             ("gen_decode_cs_asm.py", ["--ks", "--mask", "--bias"], "mla_decode_ks_bf16_bias.inc"),
                                             ("gen_decode_cs_asm.py", ["--ks", "--f16", "--mask", "--bias"], "mla_decode_ks_f16_bias.inc"),
+                                            ("gen_decode_asm.py", ["--cvt", "--mask", "--bias"], "mla_decode_asm_cvt_bias.inc"),
+                                            ("gen_decode_asm.py", ["--f16", "--mask", "--bias"], "mla_decode_asm_f16_bias.inc"),
+                                            ("gen_decode_asm.py", ["--q8", "--mask", "--bias"], "mla_decode_asm_q8_bias.inc"),
                                             ("gen_decode_cs_asm.py", ["--half"], "mla_decode_csh_bf16.inc"),
                                             ("gen_decode_cs_asm.py", ["--half", "--f16"], "mla_decode_csh_f16.inc")])
 def test_committed_wave_programs_are_what_the_generator_emits(gen, flags, name):

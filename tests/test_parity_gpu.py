@@ -582,3 +582,65 @@ def test_alibi_and_softcap_on_few_rows_and_past_the_end_of_a_paged_sequence(gpu,
             p /= p.sum(-1, keepdims=True)
             want = np.einsum("htk,kd->thd", p, kd[:, :512])
             print(U.check(got[b], want, "bias %g cap %g heads %d x %d tokens, sequence %d" % (max_bias, softcap, n_head, n_tok, b)))
+
+
+@pytest.mark.parametrize("k_type", [O.TYPE_BF16, O.TYPE_F16, O.TYPE_Q8_0])
+@pytest.mark.parametrize("max_bias,softcap", [(8.0, 0.0), (0.0, 30.0), (4.0, 1.5)])
+@pytest.mark.parametrize("paged", [False, True])
+def test_alibi_and_softcap_on_row_blocks_with_idle_waves_and_on_q8_0_cells(gpu, k_type, max_bias, softcap, paged):
+    """ALiBi slopes and the soft cap (ggml-cpu.c:11985-11989, :12041-12057) where the row-split programs run: masked launches whose row
+    blocks leave some waves without rows (48 heads; 20 heads x 3 tokens; 16 heads x 5 tokens; 11 heads x 16 tokens = a full block and
+    one of 48 rows) and Q8_0 cells at any row count (16 and 128 heads too).  Paged sequences end inside a tile while the mask is open
+    past their ends.  bf16 / f16: float64 numpy on the rounded operands; Q8_0: the oracle (ggml-cpu's arithmetic), held to the fast
+    path's documented 3e-3 where few keys carry a row."""
+    import torch
+    import jittorinfer_amd as J
+    rng = np.random.default_rng(int(max_bias * 10 + softcap * 4) + k_type + 1000)
+    q8 = k_type == O.TYPE_Q8_0
+    shapes = ((48, 1), (20, 3), (16, 5), (11, 16)) + (((16, 1), (128, 1)) if q8 else ())
+    for n_head, n_tok in shapes:
+        lens = [333, 70, 129] if paged else [320] * 3
+        n_seq = len(lens)
+        q = rng.standard_normal((n_seq, n_head, n_tok, 576)).astype(np.float32)
+        n_mask = 384      # whole tiles; with a table: every position the table can reach
+        m = (rng.standard_normal((n_tok, n_mask)) * 2.0).astype(np.float32)
+        m[rng.random((n_tok, n_mask)) < 0.3] = -np.inf
+        m[:, 0] = 0.0
+        mask = m.astype(np.float16)       # (open wherever the draw left it open, also past the end of a sequence)
+        if paged:
+            pool, bt, seqs = U.make_paged(rng, lens, k_type, sigma=0.7)
+            kw, k = dict(bt=bt, lens=lens), pool
+        else:
+            k = U.encode_kv((rng.standard_normal((n_seq, lens[0], 576)) * 0.7).astype(np.float32), k_type)
+            kw, seqs = {}, list(k)
+            mask = mask[:, :lens[0]].copy()
+        kt = {O.TYPE_BF16: J.MLA_TYPE_BF16, O.TYPE_F16: J.MLA_TYPE_F16, O.TYPE_Q8_0: J.MLA_TYPE_Q8_0}[k_type]
+        extra = dict(max_bias=max_bias, logit_softcap=softcap)
+        if paged:
+            extra.update(block_table=torch.from_numpy(bt).to(gpu), seq_lens=torch.tensor(lens, dtype=torch.int32, device=gpu))
+        tk = torch.from_numpy(k.view(np.int16) if k.dtype == np.uint16 else k).to(gpu)
+        info = J.plan(torch.from_numpy(q).to(gpu), tk, kt, dv=512, mask=torch.from_numpy(mask).to(gpu),
+                      scale=U.SCALE, out=torch.empty((n_seq, n_tok, n_head, 576), dtype=torch.float32, device=gpu), **extra)
+        assert info["variant"] == 2, info     # the pipelined kernel, not the general one
+        got = _run(gpu, q, k, k_type, mask=mask.view(np.uint16), scale=U.SCALE, max_bias=max_bias, logit_softcap=softcap, **kw)[..., :512]
+        what = "bias %g cap %g heads %d x %d tokens" % (max_bias, softcap, n_head, n_tok)
+        if q8:
+            for b in range(n_seq):
+                want = O.flash_attn_ext(q[b:b + 1], seqs[b][None], k_type, dv=512, mask=mask.view(np.uint16)[:, :len(seqs[b])], scale=U.SCALE,
+                                        max_bias=max_bias, softcap=softcap)[0]
+                print(U.check(got[b], want, "%s, Q8_0 sequence %d" % (what, b), max_abs=3e-3))
+            continue
+        n_log2 = 1 << int(np.floor(np.log2(n_head)))
+        m0, m1 = 2.0 ** (-max_bias / n_log2), 2.0 ** (-max_bias / 2 / n_log2)
+        slopes = np.array([1.0 if max_bias == 0 else (m0 ** (h + 1) if h < n_log2 else m1 ** (2 * (h - n_log2) + 1)) for h in range(n_head)])
+        qd = (O.bf16_to_f32(O.f32_to_bf16(q)) if k_type == O.TYPE_BF16 else O.f16_to_f32(O.f32_to_f16(q))).astype(np.float64)
+        for b in range(n_seq):
+            kd = (O.bf16_to_f32(seqs[b]) if k_type == O.TYPE_BF16 else O.f16_to_f32(seqs[b])).astype(np.float64)
+            s = np.einsum("htd,kd->htk", qd[b], kd) * U.SCALE
+            if softcap:
+                s = softcap * np.tanh(s / softcap)
+            s = s + slopes[:, None, None] * mask.astype(np.float64)[None, :, :kd.shape[0]]
+            p = np.exp(s - s.max(-1, keepdims=True))
+            p /= p.sum(-1, keepdims=True)
+            want = np.einsum("htk,kd->thd", p, kd[:, :512])
+            print(U.check(got[b], want, "%s, sequence %d" % (what, b)))

@@ -315,7 +315,7 @@ def test_bias_k_split_programs(name, f16):
 
 
 def run_rs(name, cov, kind, mask_build=False, n_rows=128, kv=(0, 128), seq_len=None, paged=None, f32_rows=True, final=True, boost=False, seed=0,
-           n_head=None, v_col0=False):
+           n_head=None, v_col0=False, bias_build=False, softcap=0.0, alibi=False, open_tail=False):
     rng = np.random.default_rng(seed)
     n_head = n_head or n_rows
     mask = None
@@ -324,14 +324,16 @@ def run_rs(name, cov, kind, mask_build=False, n_rows=128, kv=(0, 128), seq_len=N
     if mask_build:
         n_kv = (seq_len + 31) // 32 * 32
         n_tok = (n_rows + n_head - 1) // n_head
-        mask = np.where(rng.random((n_tok, n_kv)) < 0.25, -np.inf, 0.0)
-        mask[:, seq_len:] = -np.inf
+        mask = np.where(rng.random((n_tok, n_kv)) < 0.25, -np.inf, rng.standard_normal((n_tok, n_kv)) * (0.5 if alibi else 0.0))
+        if not open_tail:     # (open_tail: the caller's mask says nothing about the cells past the end of a paged sequence)
+            mask[:, seq_len:] = -np.inf
         mask[:, kv[0]] = 0.0
         if not paged:
             kv, seq_len = (kv[0], min(n_kv, (kv[1] + 31) // 32 * 32)), n_kv
     piece = S.PieceRS(rng, kind, n_rows=n_rows, kv_begin=kv[0], kv_end=kv[1], seq_len=seq_len, paged=paged, mask=mask, n_head=n_head,
                       k_boost=(lambda t: 4.0 ** ((t - kv[0]) // 32)) if boost else None)
-    inputs, lds_init = S.rs_setup(piece, f32_rows=f32_rows, final=final, v_col0=v_col0)
+    slopes = (2.0 ** (-8.0 * (np.arange(128) % n_head + 1) / n_head)).astype(np.float32) if alibi else None
+    inputs, lds_init = S.rs_setup(piece, f32_rows=f32_rows, final=final, v_col0=v_col0, bias_build=bias_build, slopes=slopes, softcap=softcap)
     wg = E.Workgroup(S.program_text(name), 4, piece.gmem, inputs, lds_init=lds_init)
     wg.name = name
     cov.install(wg)
@@ -343,7 +345,7 @@ def run_rs(name, cov, kind, mask_build=False, n_rows=128, kv=(0, 128), seq_len=N
         # of wave 3's share (an odd block) that word lies 4 bytes past the raw tile, in the buffer the next raw tile is being copied to.
         findings = [f for f in findings if not (f.kind == "lds-raw" and f.wave == 3 and re.fullmatch(r"ds_read_b32 v\d+, v\d+ offset:552", f.text))]
     assert not findings, "%s: %s" % (name, findings[:5])
-    want, m_want, l_want = piece.reference(v0=64 if v_col0 else 0)
+    want, m_want, l_want = piece.reference(v0=64 if v_col0 else 0, softcap=softcap, slopes=slopes)
     if f32_rows:
         got = piece.gmem.array("out").view(np.float32).reshape(128, 512)[:n_rows].astype(np.float64)
     else:
@@ -351,7 +353,10 @@ def run_rs(name, cov, kind, mask_build=False, n_rows=128, kv=(0, 128), seq_len=N
     _check(got, want, name)
     if not final:
         ml = piece.gmem.array("ml").view(np.float32).reshape(128, 2)[:n_rows].astype(np.float64)
-        assert np.abs(ml[:, 0] + np.log2(ml[:, 1]) - (m_want + np.log2(l_want))).max() < 1e-3, "%s: (m, l) of the piece" % name
+        lse = ml[:, 0] + np.log2(ml[:, 1])
+        if softcap:         # the capped logits are kept less the cap: a constant per row
+            lse = lse + softcap * np.log2(np.e)
+        assert np.abs(lse - (m_want + np.log2(l_want))).max() < 1e-3, "%s: (m, l) of the piece" % name
     return wg
 
 
@@ -383,6 +388,23 @@ def test_row_split_programs(name, kind, mask_build):
         wg = run_rs(name, cov, kind, mask_build=True, seed=120, kv=(0, 19), paged=True, n_head=8, n_rows=16)
         wg = run_rs(name, cov, kind, mask_build=True, seed=121, kv=(32, 128 + 7), paged=True, n_head=32)
         wg = run_rs(name, cov, kind, mask_build=True, seed=122, kv=(0, 64 + 7), paged=True, n_head=128)    # (the loop body exists twice)
+    assert not cov.missing(wg), cov.missing(wg)
+    _only_register_loads_ahead_of_tile_copies(cov)
+
+
+@pytest.mark.parametrize("name,kind", [("mla_decode_asm_cvt_bias.inc", "cvt"), ("mla_decode_asm_f16_bias.inc", "f16"), ("mla_decode_asm_q8_bias.inc", "q8")])
+def test_bias_row_split_programs(name, kind):
+    """ALiBi slopes and the soft cap on the row-split programs (row blocks in which some waves have no rows, Q8_0 cells): the scenarios
+    of the masked builds with a slope per head, a cap, both, neither; caps small enough that a key wrongly let in would show, under a
+    mask that is open past the end of a paged sequence."""
+    cov = Coverage()
+    for k, sc in enumerate(RS_SCENARIOS):
+        sc = {kk: vv for kk, vv in sc.items() if kk != "paged"}
+        wg = run_rs(name, cov, kind, mask_build=True, bias_build=True, seed=270 + k, n_head=16, alibi=k % 2 == 0,
+                    softcap=0.0 if sc.get("boost") else (30.0, 0.0, 2.0)[k % 3], **sc)   # (a cap keeps the running maxima from moving)
+    wg = run_rs(name, cov, kind, mask_build=True, bias_build=True, seed=290, kv=(0, 19), paged=True, n_head=8, n_rows=48, alibi=True, softcap=0.7, open_tail=True)
+    wg = run_rs(name, cov, kind, mask_build=True, bias_build=True, seed=291, kv=(32, 128 + 7), paged=True, n_head=32, n_rows=96, softcap=1.0, open_tail=True)
+    wg = run_rs(name, cov, kind, mask_build=True, bias_build=True, seed=292, kv=(0, 64 + 7), paged=True, n_head=128, alibi=True)    # (the loop body exists twice)
     assert not cov.missing(wg), cov.missing(wg)
     _only_register_loads_ahead_of_tile_copies(cov)
 

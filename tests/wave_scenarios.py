@@ -234,9 +234,10 @@ class PieceRS(Piece):
             self.qp_addr = self.gmem.add("q_image", img)
 
 
-def rs_setup(piece, f32_rows=True, final=True, scale=SCALE, v_col0=False):
+def rs_setup(piece, f32_rows=True, final=True, scale=SCALE, v_col0=False, bias_build=False, slopes=None, softcap=0.0):
     """Inputs (MLA_DECODE_INPUTS of mla_decode_kernel.hip) and hand-off records of the row-split programs: every thread finds the
-    address of its row's output (0: the row does not exist) and, lanes of the lower half, of its (m, l) pair in its record."""
+    address of its row's output (0: the row does not exist) and, lanes of the lower half, of its (m, l) pair in its record; bias
+    builds: in the last 8 bytes its row's slope and -2 softcap, and in the inputs what the launcher hands such a build."""
     q8 = piece.kind == "q8"
     hoff = (3 * TILE_BYTES + 2 * 32 * Q8_ROW) if q8 else 4 * TILE_BYTES
     out_rows = np.zeros((128, 512), np.float32) if f32_rows else np.zeros((64, 128, 8), np.float16)
@@ -253,10 +254,16 @@ def rs_setup(piece, f32_rows=True, final=True, scale=SCALE, v_col0=False):
             rec[t, 1] = ob + (row * 2048 + 16 * g if f32_rows else row * 16 + 8 * g)
             if not final and g == 0:
                 rec[t, 2] = ml + row * 8
+        if bias_build:
+            sl = np.array([1.0 if slopes is None else slopes[min(row, piece.n_rows - 1)], -2.0 * softcap if softcap else 0.0], np.float32)
+            rec[t, 3] = int(sl.view(np.uint32)[0]) | (int(sl.view(np.uint32)[1]) << 32)
     common = dict(kv=piece.kv_addr, bt=piece.bt_addr, kvb=piece.kv_begin, kve=piece.kv_end,
                   cl2=int(np.array([scale * np.log2(np.e)], np.float32).view(np.uint32)[0]), npp=piece.npp, nb1=Q8_ROW if q8 else 1152,
                   ntl=piece.n_tiles, ostr=128 * 16, qp=piece.qp_addr, pg0=piece.pg0, msk=getattr(piece, "mask_addr", 0),
                   scl=int(np.array([scale], np.float32).view(np.uint32)[0]))
+    if bias_build and softcap:
+        common["scl"] = int(np.array([scale / softcap], np.float32).view(np.uint32)[0])
+        common["cl2"] = int(np.array([2.0 * np.log2(np.e) * scale / softcap], np.float32).view(np.uint32)[0])
 
     def per_wave(w):
         d = dict(common)
