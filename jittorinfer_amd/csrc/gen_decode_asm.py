@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Generates mla_decode_asm*.inc: the hand-scheduled gfx950 instruction streams of the pipelined MLA decode kernel
-(one inline-asm block each inside mla_decode_kernel.hip).  Usage: python gen_decode_asm.py [--f16 | --q8 | --cvt] [--mask]
-> mla_decode_asm[_f16|_q8|_cvt][_mask].inc
+(one inline-asm block each inside mla_decode_kernel.hip).  Usage: python gen_decode_asm.py [--f16 | --q8 | --cvt] [--mask [--bias]]
+> mla_decode_asm[_f16|_q8|_cvt][_mask|_bias].inc
 
 Why a generator: the kernel keeps Q (144 VGPRs) and the O accumulator (256 AGPRs) resident, which leaves ~110
 registers for everything else; the instruction order (MFMA issue slots filled with LDS reads and softmax VALU work)
