@@ -23,7 +23,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 / fp16 MFMA rate
 KV_ROW_BYTES = 1152     # 576 bf16
 FLOP_PER_TOKEN_HEAD = 2 * 576 + 2 * 512
 # the commit and date at which profiles/mla_decode_kernel_c3_pmc.md's FETCH_SIZE / WRITE_SIZE readings (the `traffic` constants below) were taken
-TRAFFIC_PROFILE_COMMIT = ("300dc65", "2026-11-26")
+TRAFFIC_PROFILE_COMMIT = ("f539b15", "2026-11-26")
 
 
 def build_workload(dev, n_seq, n_head, ctx, n_pools, seed, kv="bf16"):
