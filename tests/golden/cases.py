@@ -15,6 +15,22 @@ CASES = {
     "config4_bf16_prefill_causal": (O.TYPE_BF16, 1, 16, 12, 76, "causal", 4),
     "config5_q8_0_h128_kv200": (O.TYPE_Q8_0, 1, 128, 1, 200, None, 5),
     "scattered_cells_mask": (O.TYPE_BF16, 1, 4, 3, 96, "random", 6),
+    # shapes that take the other wave programs of the HIP path: two row blocks (64 heads), row blocks with idle waves under a mask
+    "two_row_blocks_bf16_h64_kv300": (O.TYPE_BF16, 2, 64, 1, 300, None, 7),
+    "idle_waves_bf16_h20x3_mask": (O.TYPE_BF16, 1, 20, 3, 160, "biased", 8),
+    # ALiBi (max_bias) and the soft cap, BIAS below: on 48 heads (row-split), Q8_0 cells, 16 heads (k-split), 128 heads (column-split)
+    "alibi_softcap_bf16_h48_mask": (O.TYPE_BF16, 1, 48, 1, 160, "biased", 9),
+    "alibi_q8_0_h128x2_mask": (O.TYPE_Q8_0, 1, 128, 2, 160, "biased", 10),
+    "softcap_bf16_h16x2_mask": (O.TYPE_BF16, 1, 16, 2, 160, "biased", 11),
+    "alibi_softcap_bf16_h128_mask": (O.TYPE_BF16, 1, 128, 1, 160, "biased", 12),
+}
+
+# name: (max_bias, logit_softcap); absent: neither
+BIAS = {
+    "alibi_softcap_bf16_h48_mask": (8.0, 30.0),
+    "alibi_q8_0_h128x2_mask": (8.0, 0.0),
+    "softcap_bf16_h16x2_mask": (0.0, 20.0),
+    "alibi_softcap_bf16_h128_mask": (4.0, 10.0),
 }
 
 
@@ -33,12 +49,18 @@ def make_inputs(name):
         m = np.where(rng.random((n_tok, n_kv)) < 0.5, -np.inf, 0.0).astype(np.float16)
         m[:, 0] = 0
         mask = m.view(np.uint16)
+    elif mask_kind == "biased":     # finite biases (what an ALiBi slope multiplies) with holes
+        m = rng.standard_normal((n_tok, n_kv)).astype(np.float32)
+        m[rng.random((n_tok, n_kv)) < 0.3] = -np.inf
+        m[:, 0] = 0
+        mask = m.astype(np.float16).view(np.uint16)
+    max_bias, softcap = BIAS.get(name, (0.0, 0.0))
     h = hashlib.sha256()
     h.update(q.tobytes())
     h.update(k.tobytes())
     if mask is not None:
         h.update(mask.tobytes())
-    return dict(q=q, k=k, k_type=k_type, mask=mask, scale=U.SCALE, digest=h.hexdigest())
+    return dict(q=q, k=k, k_type=k_type, mask=mask, scale=U.SCALE, max_bias=max_bias, softcap=softcap, digest=h.hexdigest())
 
 
 # The nodes either side of the attention node: (kind, weight type, n_head, n_tok, rope mode, freq_scale, ext_factor, attn_factor, seed)

@@ -25,7 +25,8 @@ def main():
     out = {}
     for name in cases.CASES:
         inp = cases.make_inputs(name)
-        y = O.ref_flash_attn_ext(inp["q"], inp["k"], inp["k_type"], mask=inp["mask"], scale=inp["scale"], n_threads=4)
+        y = O.ref_flash_attn_ext(inp["q"], inp["k"], inp["k_type"], mask=inp["mask"], scale=inp["scale"], max_bias=inp["max_bias"],
+                                 softcap=inp["softcap"], n_threads=4)
         out[name] = y
         out[name + "/digest"] = np.frombuffer(inp["digest"].encode(), dtype=np.uint8)
         print(name, y.shape, float(np.abs(y).max()))

@@ -23,7 +23,7 @@ def _inputs(name):
 @pytest.mark.parametrize("name", list(cases.CASES))
 def test_oracle_matches_golden(name):
     inp = _inputs(name)
-    got = O.flash_attn_ext(inp["q"], inp["k"], inp["k_type"], dv=576, mask=inp["mask"], scale=inp["scale"])
+    got = O.flash_attn_ext(inp["q"], inp["k"], inp["k_type"], dv=576, mask=inp["mask"], scale=inp["scale"], max_bias=inp["max_bias"], softcap=inp["softcap"])
     ma, rl = O.errors(got, GOLD[name])
     if inp["k_type"] == O.TYPE_F16:
         assert ma < 2e-3 and rl < 3e-4, (ma, rl)  # f16 accumulator: rounding flips from 1e-7 differences in the dots
@@ -42,6 +42,7 @@ def test_gpu_matches_golden(gpu, name, dv):
     tk = torch.from_numpy(k.view(np.int16) if k.dtype == np.uint16 else k).to(gpu)
     tm = None if inp["mask"] is None else torch.from_numpy(inp["mask"].view(np.float16)).to(gpu)
     flags = J.MLA_FLAG_F16_ACC_STRICT if inp["k_type"] == O.TYPE_F16 else 0
-    out = J.ggml_flash_attn_ext(torch.from_numpy(inp["q"]).to(gpu), tk, inp["k_type"], dv=dv, mask=tm, scale=inp["scale"], flags=flags)
+    out = J.ggml_flash_attn_ext(torch.from_numpy(inp["q"]).to(gpu), tk, inp["k_type"], dv=dv, mask=tm, scale=inp["scale"], flags=flags,
+                                max_bias=inp["max_bias"], logit_softcap=inp["softcap"])
     torch.cuda.synchronize()
     U.check(out.cpu().numpy()[..., :dv], GOLD[name][..., :dv], name)
