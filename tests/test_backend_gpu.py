@@ -32,6 +32,26 @@ def test_node_as_ggml_cpu_accepts_it(gpu, k_type, use_sched):
     print(info, U.check(got, cpu, "plugin vs ggml-cpu"))
 
 
+@pytest.mark.parametrize("n_head,n_tok", [(48, 1), (16, 2), (128, 1)])
+@pytest.mark.parametrize("k_type", [O.TYPE_BF16, O.TYPE_Q8_0])
+def test_node_with_alibi_and_soft_cap(gpu, k_type, n_head, n_tok):
+    """max_bias and logit_softcap travel in the node's op_params (ggml.c:4024-4030): the same node, with a mask of finite biases, on
+    ggml-cpu and on the plugin -- 48 heads (a row block with idle waves), 16 heads x 2 tokens, 128 heads; bf16 and Q8_0 cells (block
+    scale 1/32: the f16 operands of the fast Q8_0 path are exact there)."""
+    rng = np.random.default_rng(23)
+    q = rng.standard_normal((2, n_head, n_tok, 576)).astype(np.float32)
+    k = U.encode_kv(rng.standard_normal((2, 224, 576)).astype(np.float32), k_type, q8_scale=1.0 / 32 if k_type == O.TYPE_Q8_0 else None)
+    m = rng.standard_normal((n_tok, 224)).astype(np.float32)
+    m[rng.random((n_tok, 224)) < 0.3] = -np.inf
+    m[:, 0] = 0
+    mask = m.astype(np.float16).view(np.uint16)
+    for max_bias, softcap in ((8.0, 0.0), (0.0, 30.0), (4.0, 12.0)):
+        got, info = O.ref_backend_flash_attn_ext(_so(), q, k, k_type, dv=576, mask=mask, scale=U.SCALE, max_bias=max_bias, softcap=softcap, use_sched=True)
+        assert "HIP-MLA" in info and "HIPMLA0" in info
+        cpu = O.ref_flash_attn_ext(q, k, k_type, mask=mask, scale=U.SCALE, max_bias=max_bias, softcap=softcap)
+        print(max_bias, softcap, U.check(got, cpu, "plugin vs ggml-cpu, max_bias %g softcap %g" % (max_bias, softcap)))
+
+
 def test_latent_prefix_view_and_block_table(gpu):
     """The MLA form: V is a 512-wide view of K, K is the page pool, src[4]/src[5] carry the block table and lengths."""
     rng = np.random.default_rng(22)
