@@ -120,15 +120,16 @@ def test_strided_q(gpu):
     print(U.check(out.cpu().numpy()[..., :512], want, "strided q"))
 
 
-def test_full_size_config3_properties(gpu):
-    """BASELINE configs[2] at full size (B=32, H=128, ctx 8192, bf16 pages): the output does not depend on where the
-    pages sit in the pool (bit-exact under a permutation of pages + table), nor on the number of KV splits (within the
-    f16-partial rounding), and one sequence equals the oracle."""
+@pytest.mark.parametrize("H", [128, 64])
+def test_full_size_config3_properties(gpu, H):
+    """BASELINE configs[2] at full size (B=32, H=128, ctx 8192, bf16 pages; and the same batch at 64 heads, which the two-row-block
+    program takes): the output does not depend on where the pages sit in the pool (bit-exact under a permutation of pages + table),
+    nor on the number of KV splits (within the f16-partial rounding), and one sequence equals the oracle."""
     import torch
     import jittorinfer_amd as J
     g = torch.Generator(device=gpu)
     g.manual_seed(5)
-    B, H, L = 32, 128, 8192
+    B, L = 32, 8192
     pages = B * L // 128
     pool = (torch.randn((pages * 128, 576), generator=g, device=gpu) * 0.5).to(torch.bfloat16).view(torch.int16)
     bt = torch.randperm(pages, generator=g, device=gpu).to(torch.int32).reshape(B, L // 128).contiguous()
@@ -686,9 +687,10 @@ def _run_flags(gpu, q, pool, k_type, bt, lens, flags):
     return out.cpu().numpy()[..., :512], info
 
 
+@pytest.mark.parametrize("n_head", [32, 64])
 @pytest.mark.parametrize("k_type", [O.TYPE_BF16, O.TYPE_Q8_0])
 @pytest.mark.parametrize("shape", ["many_short", "few_long_many_short", "one_sequence", "with_empties"])
-def test_balanced_schedule_of_ragged_decode_batches(gpu, k_type, shape):
+def test_balanced_schedule_of_ragged_decode_batches(gpu, k_type, shape, n_head):
     """The pipelined kernel's balanced schedule (equal runs of the batch's page list per workgroup, pieces of several
     sequences inside one workgroup, whole-sequence pieces written without the combine pass) against the oracle and
     against the uniform-split plan of the same call."""
@@ -709,7 +711,7 @@ def test_balanced_schedule_of_ragged_decode_batches(gpu, k_type, shape):
     if len(lens) * bt.shape[1] <= 256:
         # the schedule is planned when the table allows more than one page per workgroup: columns no sequence reaches
         bt = np.concatenate([bt, np.full((len(lens), 300 - bt.shape[1]), -5, np.int32)], axis=1)
-    q = rng.standard_normal((len(lens), 32, 1, 576)).astype(np.float32)
+    q = rng.standard_normal((len(lens), n_head, 1, 576)).astype(np.float32)
     got, info = _run_flags(gpu, q, pool, k_type, bt, lens, 0)
     assert info["variant"] == 2 and info["balanced"] == 1 and info["n_workgroups"] == 256
     uni, info_u = _run_flags(gpu, q, pool, k_type, bt, lens, J.MLA_FLAG_UNIFORM_SPLITS)
@@ -870,8 +872,9 @@ def test_prompt_chunk_behind_a_long_cache_without_a_table(gpu):
         assert worst < U.MAX_ABS_TOL, (n_tok, past, worst)
 
 
-def test_paged_decode_of_more_than_256_sequences_longest_first(gpu):
-    """A paged decode batch of more than 256 sequences of 128 heads is a workgroup per sequence, in rounds; the workgroups take the
+@pytest.mark.parametrize("n_head", [128, 64])
+def test_paged_decode_of_more_than_256_sequences_longest_first(gpu, n_head):
+    """A paged decode batch of more than 256 sequences of 128 (64) heads is a workgroup per sequence, in rounds; the workgroups take the
     sequences by falling length (an order the pre-pass writes into the workspace).  300 ragged sequences, some empty, some equal:
     against the oracle, and bit for bit against the same launch in batch order (MLA_FLAG_UNIFORM_SPLITS)."""
     import torch
@@ -882,7 +885,7 @@ def test_paged_decode_of_more_than_256_sequences_longest_first(gpu):
     lens[20:24] = [77, 77, 77, 77]
     pool, bt, seqs = U.make_paged(rng, np.maximum(lens, 1), O.TYPE_BF16)
     seqs = [s[:l] for s, l in zip(seqs, lens)]
-    q = rng.standard_normal((300, 128, 1, 576)).astype(np.float32)
+    q = rng.standard_normal((300, n_head, 1, 576)).astype(np.float32)
     tq, tk = torch.from_numpy(q).to(gpu), torch.from_numpy(pool.view(np.int16)).to(gpu)
     tb, tl = torch.from_numpy(bt).to(gpu), torch.from_numpy(np.asarray(lens, dtype=np.int32)).to(gpu)
     info = J.plan(tq, tk, O.TYPE_BF16, dv=512, scale=U.SCALE, block_table=tb, seq_lens=tl)
