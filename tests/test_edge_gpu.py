@@ -584,6 +584,49 @@ def test_repeated_launches_give_identical_results(gpu, k_type):
         assert bool(torch.isfinite(ref).all())
 
 
+def test_repeated_launches_of_the_programs_with_idle_waves(gpu):
+    """The same launches 100 times each, other launches in between, every result equal to the first bit for bit: a paged decode step
+    of 64 heads (the two-row-block program: two waves without rows in a loop of their own) and a masked one of 48 heads with ALiBi and
+    a soft cap over bf16 and over Q8_0 cells (the bias builds of the row-split programs)."""
+    import torch
+    import jittorinfer_amd as J
+    rng = np.random.default_rng(77)
+    lens = [1000, 333, 129, 2048, 77, 640]
+    pool, bt, _ = U.make_paged(rng, lens, O.TYPE_BF16)
+    q64 = torch.from_numpy(rng.standard_normal((len(lens), 64, 1, 576)).astype(np.float32)).to(gpu)
+    tp, tb = torch.from_numpy(pool.view(np.int16)).to(gpu), torch.from_numpy(bt).to(gpu)
+    tl = torch.tensor(lens, dtype=torch.int32, device=gpu)
+    n_kv = 640
+    q48 = torch.from_numpy(rng.standard_normal((2, 48, 1, 576)).astype(np.float32)).to(gpu)
+    kb = torch.from_numpy(U.encode_kv(rng.standard_normal((2, n_kv, 576)).astype(np.float32), O.TYPE_BF16).view(np.int16)).to(gpu)
+    kq = torch.from_numpy(U.encode_kv(rng.standard_normal((2, n_kv, 576)).astype(np.float32), O.TYPE_Q8_0)).to(gpu)
+    m = (rng.standard_normal((1, n_kv)) * 2).astype(np.float32)
+    m[rng.random((1, n_kv)) < 0.3] = -np.inf
+    m[:, 0] = 0
+    tm = torch.from_numpy(m.astype(np.float16)).to(gpu)
+    launches = [
+        ("64 heads, paged", lambda out: J.ggml_flash_attn_ext(q64, tp, O.TYPE_BF16, dv=512, scale=U.SCALE, block_table=tb, seq_lens=tl, out=out), (len(lens), 1, 64, 576)),
+        ("48 heads, bf16 cells, ALiBi + soft cap", lambda out: J.ggml_flash_attn_ext(q48, kb, O.TYPE_BF16, dv=512, scale=U.SCALE, mask=tm, out=out, max_bias=8.0, logit_softcap=20.0), (2, 1, 48, 576)),
+        ("48 heads, Q8_0 cells, ALiBi + soft cap", lambda out: J.ggml_flash_attn_ext(q48, kq, O.TYPE_Q8_0, dv=512, scale=U.SCALE, mask=tm, out=out, max_bias=8.0, logit_softcap=20.0), (2, 1, 48, 576)),
+    ]
+    for k, (what, f, shape) in enumerate(launches):
+        out = torch.empty(shape, dtype=torch.float32, device=gpu)
+        other = torch.empty(launches[(k + 1) % 3][2], dtype=torch.float32, device=gpu)
+        ref, differ = None, 0
+        for i in range(100):
+            if i % 3 == 0:
+                launches[(k + 1) % 3][1](other)
+            out.fill_(float("nan"))
+            f(out)
+            cur = out[..., :512].clone()
+            if ref is None:
+                ref = cur
+            elif not torch.equal(cur, ref):
+                differ += 1
+        assert differ == 0, "%s: %d of 99 launches differ from the first" % (what, differ)
+        assert bool(torch.isfinite(ref).all()), what
+
+
 @pytest.mark.parametrize("k_type", [O.TYPE_BF16, O.TYPE_Q8_0])
 @pytest.mark.parametrize("n_head,n_tok", [(128, 8), (16, 32), (16, 1), (48, 5)])
 def test_mask_extents_left_by_the_launch_before(gpu, k_type, n_head, n_tok):
