@@ -409,6 +409,66 @@ def test_bias_row_split_programs(name, kind):
     _only_register_loads_ahead_of_tile_copies(cov)
 
 
+RANDOM_PROGRAMS = [
+    # (runner, stream, its arguments, rows it is launched with, masked, bias build)
+    ("cs", "mla_decode_cs_bf16.inc", dict(f16=False), (97, 128), False, False),
+    ("cs", "mla_decode_cs_f16.inc", dict(f16=True), (97, 128), False, False),
+    ("cs", "mla_decode_cs_bf16_mask.inc", dict(f16=False, mask_build=True), (97, 128), True, False),
+    ("cs", "mla_decode_cs_f16_mask_nt.inc", dict(f16=True, mask_build=True), (97, 128), True, False),
+    ("cs", "mla_decode_cs_bf16_bias.inc", dict(f16=False, mask_build=True, bias_build=True), (97, 128), True, True),
+    ("cs", "mla_decode_cs_f16_bias.inc", dict(f16=True, mask_build=True, bias_build=True), (97, 128), True, True),
+    ("cs", "mla_decode_csh_bf16.inc", dict(f16=False), (33, 64), False, False),
+    ("cs", "mla_decode_csh_f16.inc", dict(f16=True), (33, 64), False, False),
+    ("ks", "mla_decode_ks_bf16.inc", dict(f16=False), (1, 32), False, False),
+    ("ks", "mla_decode_ks_f16_mask.inc", dict(f16=True, mask_build=True), (1, 32), True, False),
+    ("ks", "mla_decode_ks_bf16_mask_nt.inc", dict(f16=False, mask_build=True), (1, 32), True, False),
+    ("ks", "mla_decode_ks_bf16_bias.inc", dict(f16=False, mask_build=True, bias_build=True), (1, 32), True, True),
+    ("ks", "mla_decode_ks_f16_bias.inc", dict(f16=True, mask_build=True, bias_build=True), (1, 32), True, True),
+    ("rs", "mla_decode_asm.inc", dict(kind="bf16"), (1, 128), False, False),
+    ("rs", "mla_decode_asm_mask.inc", dict(kind="bf16", mask_build=True), (1, 128), True, False),
+    ("rs", "mla_decode_asm_f16.inc", dict(kind="f16"), (1, 128), False, False),
+    ("rs", "mla_decode_asm_f16_mask.inc", dict(kind="f16", mask_build=True), (1, 128), True, False),
+    ("rs", "mla_decode_asm_cvt.inc", dict(kind="cvt"), (1, 128), False, False),
+    ("rs", "mla_decode_asm_cvt_mask.inc", dict(kind="cvt", mask_build=True), (1, 128), True, False),
+    ("rs", "mla_decode_asm_q8.inc", dict(kind="q8"), (1, 128), False, False),
+    ("rs", "mla_decode_asm_q8_mask.inc", dict(kind="q8", mask_build=True), (1, 128), True, False),
+    ("rs", "mla_decode_asm_cvt_bias.inc", dict(kind="cvt", mask_build=True, bias_build=True), (1, 128), True, True),
+    ("rs", "mla_decode_asm_f16_bias.inc", dict(kind="f16", mask_build=True, bias_build=True), (1, 128), True, True),
+    ("rs", "mla_decode_asm_q8_bias.inc", dict(kind="q8", mask_build=True, bias_build=True), (1, 128), True, True),
+]
+
+
+def random_scenario(seed):
+    """A scenario nobody wrote down, drawn from the seed: the program, the rows of its block, a key range of 1 to 9 tiles that may
+    start inside a page and end inside a tile, behind which the sequence may go on; paged or contiguous; every kind of store; for the
+    masked builds the heads per query token, for the bias builds slopes, a cap, a mask open past the end of a paged sequence."""
+    rng = np.random.default_rng(seed)
+    runner, name, kw, (r0, r1), masked, bias = RANDOM_PROGRAMS[seed % len(RANDOM_PROGRAMS)]
+    n_tiles = int(rng.choice([1, 1, 2, 3, 4, 5, 6, 9]))
+    begin = int(rng.choice([0, 0, 32, 64, 96, 128, 160, 256]))
+    end = max(begin + n_tiles * 32 - (int(rng.integers(0, 32)) if rng.integers(2) else 0), begin + 1)
+    paged, f32_rows = bool(rng.integers(2)), bool(rng.integers(2))
+    args = dict(kw, n_rows=int(rng.integers(r0, r1 + 1)), kv=(begin, end), seq_len=end + (int(rng.integers(0, 200)) if rng.integers(2) else 0),
+                f32_rows=f32_rows, final=bool(rng.integers(2)) if f32_rows else False, seed=1000 + seed, paged=paged)
+    if masked:
+        args["n_head"] = int(rng.choice([1, 2, 4, 8, 16, 32, 64, 128]))
+    if bias:
+        args.update(alibi=bool(rng.integers(2)), softcap=float(rng.choice([0.0, 0.7, 5.0, 30.0])), open_tail=bool(rng.integers(2)) and paged)
+    if runner != "ks" and not masked and "csh" not in name and rng.integers(4) == 0:
+        args["v_col0"] = True
+    if rng.integers(5) == 0 and not (bias and args["softcap"]) and n_tiles <= 5:     # (the keys grow fourfold from tile to tile: within f16 for five)
+        args["boost"] = True
+    return runner, name, args
+
+
+@pytest.mark.parametrize("seed", range(2 * len(RANDOM_PROGRAMS)))
+def test_random_scenarios(seed):
+    """Two drawn scenarios per generated stream (600 more were run once on the streams as committed, without a finding): the result
+    against float64, and an empty hazard report."""
+    runner, name, args = random_scenario(3000 + seed)
+    {"cs": run_cs, "ks": run_ks, "rs": run_rs}[runner](name, Coverage(), **args)
+
+
 def test_the_report_names_a_barrier_ahead_of_the_last_fragment_request():
     """What the masked column-split programs once did: the barrier that frees the P^T buffer stood ahead of the request for the tile's
     last P^T fragment (wave 3's rows), whose read by the other waves then raced with wave 3's write of the next tile's P.  The same
