@@ -87,7 +87,7 @@ def run_cs(name, cov, f16, mask_build=False, bias_build=False, n_rows=128, kv=(0
         if not paged:         # (a masked launch over a cache without a table covers whole tiles; with a table the lengths may be ragged)
             kv, seq_len = (kv[0], min(n_kv, (kv[1] + 31) // 32 * 32)), n_kv
     piece = S.Piece(rng, f16, n_rows=n_rows, kv_begin=kv[0], kv_end=kv[1], seq_len=seq_len, paged=paged, mask=mask, n_head=n_head,
-                    k_boost=(lambda t: 4.0 ** ((t - kv[0]) // 32)) if boost else None)
+                    k_boost=(lambda t: 4.0 ** np.minimum((t - kv[0]) // 32, 6)) if boost else None)
     slopes = None
     if alibi:
         slopes = (2.0 ** (-8.0 * (np.arange(128) % n_head + 1) / n_head)).astype(np.float32)
@@ -237,7 +237,7 @@ def run_ks(name, cov, f16, mask_build=False, n_rows=32, kv=(0, 128), seq_len=Non
         if not paged:
             kv, seq_len = (kv[0], min(n_kv, (kv[1] + 31) // 32 * 32)), n_kv
     piece = S.Piece(rng, f16, n_rows=n_rows, kv_begin=kv[0], kv_end=kv[1], seq_len=seq_len, paged=paged, mask=mask, n_head=n_head,
-                    k_boost=(lambda t: 4.0 ** ((t - kv[0]) // 32)) if boost else None)
+                    k_boost=(lambda t: 4.0 ** np.minimum((t - kv[0]) // 32, 6)) if boost else None)
     slopes = (2.0 ** (-8.0 * (np.arange(128) % n_head + 1) / n_head)).astype(np.float32) if alibi else None
     lds_init = S.ks_lds_init(piece, bias_build, slopes, -2.0 * softcap if softcap else 0.0)
     inputs = S.ks_inputs(piece, piece.gmem, f32_rows=f32_rows, final=final, mask_build=mask_build)
@@ -331,7 +331,7 @@ def run_rs(name, cov, kind, mask_build=False, n_rows=128, kv=(0, 128), seq_len=N
         if not paged:
             kv, seq_len = (kv[0], min(n_kv, (kv[1] + 31) // 32 * 32)), n_kv
     piece = S.PieceRS(rng, kind, n_rows=n_rows, kv_begin=kv[0], kv_end=kv[1], seq_len=seq_len, paged=paged, mask=mask, n_head=n_head,
-                      k_boost=(lambda t: 4.0 ** ((t - kv[0]) // 32)) if boost else None)
+                      k_boost=(lambda t: 4.0 ** np.minimum((t - kv[0]) // 32, 6)) if boost else None)
     slopes = (2.0 ** (-8.0 * (np.arange(128) % n_head + 1) / n_head)).astype(np.float32) if alibi else None
     inputs, lds_init = S.rs_setup(piece, f32_rows=f32_rows, final=final, v_col0=v_col0, bias_build=bias_build, slopes=slopes, softcap=softcap)
     wg = E.Workgroup(S.program_text(name), 4, piece.gmem, inputs, lds_init=lds_init)
