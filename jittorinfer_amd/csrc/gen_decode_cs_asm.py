@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Generates mla_decode_cs_*.inc: the gfx950 instruction streams of the pipelined MLA decode kernel in its
 "column-split" form (one inline-asm block each inside mla_decode_kernel.hip).
-Usage: python gen_decode_cs_asm.py [--f16] [--mask] > mla_decode_cs_[bf16|f16][_mask].inc
+Usage: python gen_decode_cs_asm.py [--ks | --half] [--f16] [--mask [--bias | --stream]] > mla_decode_[cs|ks|csh]_[bf16|f16][_mask[_nt]|_bias].inc
 
 Work of one wave w of a 4-wave workgroup (128 attention rows x one KV split), per 32-token tile `it`:
     part 1   S = K[it+1].Q^T for the wave's own 32 rows (36 MFMA, Q resident in 144 VGPRs, K fragments from LDS);
@@ -21,6 +21,10 @@ eight registers they live in come out of the K and P^T fragment rings.
 (ggml-cpu.c:11985-11989, :12006-12008; 1 without ALiBi) is a per-lane input that stays in a register the program never writes; the
 soft cap runs as tanh(x) = 1 - 2 / (1 + 2^(2 x log2 e)) on v_exp_f32 / v_rcp_f32, and since a constant added to every logit of a
 row changes neither the probabilities nor the split-K merge, the program keeps -2 softcap / (1 + e^(2x)) and drops the "+ softcap".
+--half: 33 to 64 rows, i.e. two row blocks.  Waves 0 and 1 run the program above with two row blocks of P.V (16 MFMA); the waves
+without rows (FLG bit 5) leave it behind the barrier that completes tile 0 for a loop of their own (iteration_rowless): their share
+of the tile copies, the V^T fragments, their 128 columns of P.V, the same two barriers per tile -- no Q, no K.Q^T, no softmax.
+--ks: see ks_main.
 """
 import sys
 
